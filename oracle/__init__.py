@@ -1,0 +1,239 @@
+"""ctypes front-end of the CPU oracle (``oracle/zyx_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py``. The product package ``zyx_amd`` never imports it.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libzyx_oracle.so")
+
+# dtype codes, in the order of zyx/src/dtype.rs:20-47
+BF16, F16, F32, F64, U8, U16, U32, U64, I8, I16, I32, I64, BOOL = range(13)
+
+UNARY = dict(neg=0, exp=1, exp2=2, ln=3, log2=4, reciprocal=5, sqrt=6, sin=7, cos=8, floor=9, trunc=10, abs=11,
+             relu=32, tanh=33, gelu=34, sigmoid=35, rsqrt=36)
+BINARY = dict(add=0, sub=1, mul=2, div=3, pow=4, mod=5, cmplt=6, cmpgt=7, max=8, noteq=9, eq=10, cmpge=11)
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (a few seconds)."""
+    src = os.path.join(_HERE, "zyx_oracle.c")
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libzyx_oracle.so"], stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.zo_rng_next_u64.restype = C.c_uint64
+    return _lib
+
+
+def _p(a: np.ndarray | None):
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(C.c_void_p)
+
+
+_I64 = C.c_int64
+
+
+class Rng:
+    """zyx's xoshiro256++ generator (zyx/src/rng.rs); default seed 42069 (zyx/src/runtime.rs:178)."""
+
+    def __init__(self, seed: int = 42069):
+        self._s = (C.c_uint64 * 4)()
+        lib().zo_rng_seed(self._s, C.c_uint64(seed))
+
+    def next_u64(self) -> int:
+        return lib().zo_rng_next_u64(self._s)
+
+    def rand_u8(self, n: int) -> np.ndarray:
+        out = np.empty(n, np.uint8)
+        lib().zo_rand_u8(self._s, _p(out), _I64(n))
+        return out
+
+    def rand(self, shape) -> np.ndarray:
+        out = np.empty(shape, np.float32)
+        lib().zo_rand_f32(self._s, _p(out), _I64(out.size))
+        return out
+
+    def uniform(self, shape, lo: float, hi: float) -> np.ndarray:
+        out = np.empty(shape, np.float32)
+        lib().zo_uniform_f32(self._s, _p(out), _I64(out.size), C.c_float(lo), C.c_float(hi))
+        return out
+
+    def randn(self, shape, scale: float = 1.0) -> np.ndarray:
+        out = np.empty(shape, np.float32)
+        lib().zo_randn_f32(self._s, _p(out), _I64(out.size), C.c_float(scale))
+        return out
+
+    def randint(self, shape, lo: int, hi: int) -> np.ndarray:
+        out = np.empty(shape, np.int32)
+        lib().zo_randint_i32(self._s, _p(out), _I64(out.size), _I64(lo), _I64(hi))
+        return out
+
+
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.empty(x.shape, np.uint16)
+    lib().zo_f32_to_bf16(_p(x), _p(y), _I64(x.size))
+    return y
+
+
+def bf16_to_f32(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.uint16)
+    y = np.empty(x.shape, np.float32)
+    lib().zo_bf16_to_f32(_p(x), _p(y), _I64(x.size))
+    return y
+
+
+def f32_to_f16(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.empty(x.shape, np.uint16)
+    lib().zo_f32_to_f16(_p(x), _p(y), _I64(x.size))
+    return y
+
+
+def f16_to_f32(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.uint16)
+    y = np.empty(x.shape, np.float32)
+    lib().zo_f16_to_f32(_p(x), _p(y), _I64(x.size))
+    return y
+
+
+def _store_dtype(code: int):
+    return np.float32 if code == F32 else np.uint16
+
+
+def unary(op: str, x: np.ndarray, dtype: int = F32) -> np.ndarray:
+    x = np.ascontiguousarray(x, _store_dtype(dtype))
+    y = np.empty_like(x)
+    lib().zo_unary_map(UNARY[op], dtype, _p(x), _p(y), _I64(x.size))
+    return y
+
+
+def binary(op: str, x: np.ndarray, y: np.ndarray, dtype: int = F32) -> np.ndarray:
+    """x: [rows, cols] (or any shape, flattened to rows x last); y: same shape, [cols] or scalar."""
+    x = np.ascontiguousarray(x, _store_dtype(dtype))
+    y = np.ascontiguousarray(y, _store_dtype(dtype))
+    cols = x.shape[-1] if x.ndim else 1
+    rows = x.size // max(cols, 1)
+    if y.size == x.size:
+        bc = 0
+    elif y.size == 1:
+        bc = 2
+    else:
+        assert y.size == cols, "row-vector broadcast only"
+        bc = 1
+    z = np.empty_like(x)
+    lib().zo_binary_map(BINARY[op], dtype, _p(x), _p(y), _p(z), _I64(rows), _I64(cols), bc)
+    return z
+
+
+def reduce_rows(op: str, x: np.ndarray, dtype: int = F32) -> np.ndarray:
+    x = np.ascontiguousarray(x, _store_dtype(dtype))
+    rows, cols = x.shape
+    y = np.empty(rows, x.dtype)
+    lib().zo_reduce_rows(0 if op == "sum" else 1, dtype, _p(x), _p(y), _I64(rows), _I64(cols))
+    return y
+
+
+def reduce_cols(op: str, x: np.ndarray, dtype: int = F32) -> np.ndarray:
+    x = np.ascontiguousarray(x, _store_dtype(dtype))
+    rows, cols = x.shape
+    y = np.empty(cols, x.dtype)
+    lib().zo_reduce_cols(0 if op == "sum" else 1, dtype, _p(x), _p(y), _I64(rows), _I64(cols))
+    return y
+
+
+def reduce_rows_i32(op: str, x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.int32)
+    rows, cols = x.shape
+    y = np.empty(rows, np.int32)
+    lib().zo_reduce_rows_i32(0 if op == "sum" else 1, _p(x), _p(y), _I64(rows), _I64(cols))
+    return y
+
+
+def softmax_rows(x: np.ndarray, want_y=True, want_sum=True, want_arg=True):
+    """Returns (y, rowsum, argmax) of the reference's softmax -> sum / argmax_axis(-1) chain."""
+    x = np.ascontiguousarray(x, np.float32)
+    rows, cols = x.shape
+    y = np.empty_like(x) if want_y else None
+    s = np.empty(rows, np.float32) if want_sum else None
+    a = np.empty(rows, np.int32) if want_arg else None
+    lib().zo_softmax_rows_f32(_p(x), _p(y), _p(s), _p(a), _I64(rows), _I64(cols))
+    return y, s, a
+
+
+def softmax_rows_f64acc(x: np.ndarray):
+    x = np.ascontiguousarray(x, np.float32)
+    rows, cols = x.shape
+    y = np.empty_like(x)
+    s = np.empty(rows, np.float32)
+    lib().zo_softmax_rows_f64acc(_p(x), _p(y), _p(s), _I64(rows), _I64(cols))
+    return y, s
+
+
+def argmax_rows(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    rows, cols = x.shape
+    a = np.empty(rows, np.int32)
+    lib().zo_argmax_rows_f32(_p(x), _p(a), _I64(rows), _I64(cols))
+    return a
+
+
+def matmul(a: np.ndarray, b: np.ndarray, in_dtype: int = F32, out_dtype: int = F32, transb: bool = False) -> np.ndarray:
+    """dot / dot_dtype of zyx/src/tensor/mod.rs:1469-1518 on 2-D operands."""
+    a = np.ascontiguousarray(a)
+    b = np.ascontiguousarray(b)
+    m, k = a.shape
+    n = b.shape[0] if transb else b.shape[1]
+    assert (b.shape[1] if transb else b.shape[0]) == k
+    c = np.empty((m, n), _store_dtype(out_dtype))
+    lib().zo_matmul_float(in_dtype, out_dtype, _p(a), _p(b), _p(c), _I64(m), _I64(n), _I64(k), int(transb))
+    return c
+
+
+def matmul_f64acc(a: np.ndarray, b: np.ndarray, in_dtype: int = F32, transb: bool = False) -> np.ndarray:
+    a = np.ascontiguousarray(a)
+    b = np.ascontiguousarray(b)
+    m, k = a.shape
+    n = b.shape[0] if transb else b.shape[1]
+    c = np.empty((m, n), np.float64)
+    lib().zo_matmul_f64acc(in_dtype, _p(a), _p(b), _p(c), _I64(m), _I64(n), _I64(k), int(transb))
+    return c
+
+
+def matmul_int(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    a = np.ascontiguousarray(a)
+    b = np.ascontiguousarray(b)
+    m, k = a.shape
+    n = b.shape[1]
+    c = np.empty((m, n), a.dtype)
+    fn = lib().zo_matmul_i64 if a.dtype == np.int64 else lib().zo_matmul_i32
+    fn(_p(a), _p(b), _p(c), _I64(m), _I64(n), _I64(k))
+    return c
+
+
+def bias_act(c: np.ndarray, bias: np.ndarray | None, act: str = "none", bias_dtype: int = F32) -> np.ndarray:
+    c = np.array(c, np.float32, copy=True, order="C")
+    m, n = c.shape
+    lib().zo_bias_act_f32(_p(c), _p(None if bias is None else np.ascontiguousarray(bias)), bias_dtype, _I64(m), _I64(n),
+                          dict(none=0, relu=1, gelu=2)[act])
+    return c

@@ -1,0 +1,457 @@
+/*
+ * zyx_oracle.c -- CPU restatement of the arithmetic zyx's C/CPU backend performs
+ * for the ops that the MI355X HIP backend accelerates.
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE. It is the checker the HIP kernels are compared
+ * with, and the CPU baseline timed beside them. Nothing in the product library
+ * (zyx_amd/, include/) links, imports or calls it.
+ *
+ * The reference is Rust and generates its C kernels at run time, so no reference
+ * source can be compiled here; every function restates the cited reference code
+ * (paths relative to the reference checkout) and is pinned by the reference's own
+ * golden vectors in tests/test_oracle_*.py. Functions that no golden vector or
+ * closed form pins say "parity unpinned" in their comment.
+ *
+ * Conventions followed (zyx/src/codegen/c.rs):
+ *   - all float math runs in `float` registers, bf16/f16 are widened on load and
+ *     truncated on store (c.rs:135-140, 199-201, 456-497, 615-629);
+ *   - reductions keep one register accumulator, initialised to 0 / dtype.min,
+ *     and fold `acc = x (+) acc` serially over the reduce axis
+ *     (zyx/src/kernel/linearize.rs:920-952, zyx/src/dtype.rs:207-224);
+ *   - Max is fmax (c.rs:602), Mod is (int)x % (int)y (c.rs:598);
+ *   - the outermost output loop is `#pragma omp parallel for` (c.rs:89-91);
+ *   - built with -O3 -ffast-math -fno-associative-math (zyx/src/backend/c.rs:221-227).
+ */
+#include <float.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ZO_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------------- */
+/* RNG: zyx/src/rng.rs                                                        */
+/* ------------------------------------------------------------------------- */
+
+typedef struct {
+    uint64_t s[4];
+} zo_rng;
+
+static inline uint64_t rotl64(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+
+/* splitmix64 x4 seeding, rng.rs:15-57 */
+ZO_API void zo_rng_seed(zo_rng *r, uint64_t state) {
+    for (int i = 0; i < 4; i++) {
+        state += 0x9e3779b97f4a7c15ull;
+        uint64_t z = state;
+        z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+        z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+        r->s[i] = z ^ (z >> 31);
+    }
+}
+
+/* xoshiro256++, rng.rs:65-80 */
+ZO_API uint64_t zo_rng_next_u64(zo_rng *r) {
+    uint64_t *s = r->s;
+    uint64_t res = rotl64(s[0] + s[3], 23) + s[0];
+    uint64_t t = s[1] << 17;
+    s[2] ^= s[0];
+    s[3] ^= s[1];
+    s[1] ^= s[2];
+    s[0] ^= s[3];
+    s[2] ^= t;
+    s[3] = rotl64(s[3], 45);
+    return res;
+}
+
+/* next_f32, rng.rs:98-110: LCG step on the low 32 bits, modulo 2^32-1, divided by
+ * (float)(2^32-1) == 2^32. The value can be exactly 1.0f (v >= 2^32-128). */
+static inline float zo_next_f32(zo_rng *r) {
+    uint32_t seed = (uint32_t)zo_rng_next_u64(r);
+    uint32_t v = (uint32_t)(1664525u * seed + 1013904223u) % 0xffffffffu;
+    return (float)v / (float)0xffffffffu;
+}
+
+/* Tensor::rand for u8: one full 64-bit draw per element, low byte (rng.rs:92-95,131). */
+ZO_API void zo_rand_u8(zo_rng *r, uint8_t *out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = (uint8_t)zo_rng_next_u64(r);
+}
+ZO_API void zo_rand_u32(zo_rng *r, uint32_t *out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = (uint32_t)zo_rng_next_u64(r);
+}
+/* Tensor::rand for floats, row-major sequential draws (zyx/src/tensor/mod.rs:516-597). */
+ZO_API void zo_rand_f32(zo_rng *r, float *out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = zo_next_f32(r);
+}
+/* Tensor::uniform: rand * (hi - lo) + lo in f32 (tensor/mod.rs:637-648). */
+ZO_API void zo_uniform_f32(zo_rng *r, float *out, int64_t n, float lo, float hi) {
+    float span = hi - lo;
+    for (int64_t i = 0; i < n; i++) out[i] = zo_next_f32(r) * span + lo;
+}
+/* Tensor::randint for signed ints: next_u64 % range + lo (rng.rs:186-208). */
+ZO_API void zo_randint_i32(zo_rng *r, int32_t *out, int64_t n, int64_t lo, int64_t hi) {
+    uint64_t range = (uint64_t)(hi - lo);
+    for (int64_t i = 0; i < n; i++) out[i] = (int32_t)((int64_t)(zo_rng_next_u64(r) % range) + lo);
+}
+/* Tensor::randn (tensor/mod.rs:603-613): one rand([2, n]) draw, then
+ * cos(2*pi*u0[i]) * sqrt(-2*ln(1 - u1[i])). The reference evaluates cos/ln/sqrt as
+ * device kernels, so its bits depend on the backend; here host libm is used and the
+ * same buffer feeds both sides of every parity test. A draw u1 == 1.0f (possible,
+ * see zo_next_f32) would give ln(0) = -inf: it is clamped to the largest float
+ * below one, which changes that one sample and nothing after it. */
+ZO_API void zo_randn_f32(zo_rng *r, float *out, int64_t n, float scale) {
+    float *u0 = (float *)malloc(sizeof(float) * (size_t)n);
+    for (int64_t i = 0; i < n; i++) u0[i] = zo_next_f32(r);
+    const float two_pi = 2.0f * 3.14159265358979323846f;
+    for (int64_t i = 0; i < n; i++) {
+        float u1 = zo_next_f32(r);
+        if (u1 >= 1.0f) u1 = 0.99999994f;
+        float x1 = cosf(u0[i] * two_pi);
+        float x2 = sqrtf(logf(1.0f - u1) * -2.0f);
+        out[i] = x1 * x2 * scale;
+    }
+    free(u0);
+}
+
+/* ------------------------------------------------------------------------- */
+/* 16-bit float storage: zyx/src/codegen/c.rs:456-497, zyx/src/scalar.rs:33-45 */
+/* ------------------------------------------------------------------------- */
+
+static inline float bf16_load(uint16_t h) {
+    uint32_t b = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &b, 4);
+    return f;
+}
+static inline uint16_t bf16_store(float v) { /* truncation, not round-to-nearest */
+    uint32_t b;
+    memcpy(&b, &v, 4);
+    return (uint16_t)(b >> 16);
+}
+static inline float f16_load(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16, man = h & 0x3ffu, ex = (h >> 10) & 0x1fu, f;
+    if (ex == 0) { /* subnormal: man * 2^-24 exactly, as zyx/src/scalar.rs:155-165 */
+        float sub = ldexpf((float)man, -24);
+        return sign ? -sub : sub;
+    } else if (ex == 31) f = sign | 0x7f800000u | (man << 13);
+    else f = sign | ((ex + 112u) << 23) | (man << 13);
+    float r;
+    memcpy(&r, &f, 4);
+    return r;
+}
+static inline uint16_t f16_store(float v) { /* mantissa truncated, subnormals flushed */
+    uint32_t f;
+    memcpy(&f, &v, 4);
+    uint32_t sign = (f >> 16) & 0x8000u, ex = (f >> 23) & 0xffu, man = f & 0x7fffffu;
+    if (ex == 0) return (uint16_t)sign;
+    if (ex == 255) return (uint16_t)(sign | 0x7c00u | (man >> 13));
+    int ne = (int)ex - 127 + 15;
+    if (ne >= 31) return (uint16_t)(sign | 0x7c00u);
+    if (ne <= 0) return (uint16_t)sign;
+    return (uint16_t)(sign | ((uint32_t)ne << 10) | (man >> 13));
+}
+ZO_API void zo_f32_to_bf16(const float *x, uint16_t *y, int64_t n) {
+    for (int64_t i = 0; i < n; i++) y[i] = bf16_store(x[i]);
+}
+ZO_API void zo_bf16_to_f32(const uint16_t *x, float *y, int64_t n) {
+    for (int64_t i = 0; i < n; i++) y[i] = bf16_load(x[i]);
+}
+ZO_API void zo_f32_to_f16(const float *x, uint16_t *y, int64_t n) {
+    for (int64_t i = 0; i < n; i++) y[i] = f16_store(x[i]);
+}
+ZO_API void zo_f16_to_f32(const uint16_t *x, float *y, int64_t n) {
+    for (int64_t i = 0; i < n; i++) y[i] = f16_load(x[i]);
+}
+
+/* dtype codes follow zyx/src/dtype.rs:20-47 */
+enum { ZO_BF16 = 0, ZO_F16, ZO_F32, ZO_F64, ZO_U8, ZO_U16, ZO_U32, ZO_U64, ZO_I8, ZO_I16, ZO_I32, ZO_I64, ZO_BOOL };
+
+static inline float load_as_f32(const void *p, int dtype, int64_t i) {
+    switch (dtype) {
+    case ZO_BF16: return bf16_load(((const uint16_t *)p)[i]);
+    case ZO_F16: return f16_load(((const uint16_t *)p)[i]);
+    default: return ((const float *)p)[i];
+    }
+}
+static inline void store_from_f32(void *p, int dtype, int64_t i, float v) {
+    switch (dtype) {
+    case ZO_BF16: ((uint16_t *)p)[i] = bf16_store(v); break;
+    case ZO_F16: ((uint16_t *)p)[i] = f16_store(v); break;
+    default: ((float *)p)[i] = v; break;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Primitive unary / binary ops on float registers: zyx/src/kernel/ops.rs:187-261,
+ * zyx/src/codegen/c.rs:290-304, 593-611                                        */
+/* ------------------------------------------------------------------------- */
+
+enum { /* unary */
+    ZO_U_NEG = 0, ZO_U_EXP, ZO_U_EXP2, ZO_U_LN, ZO_U_LOG2, ZO_U_RECIPROCAL, ZO_U_SQRT, ZO_U_SIN, ZO_U_COS,
+    ZO_U_FLOOR, ZO_U_TRUNC, ZO_U_ABS,
+    /* composites from zyx/src/tensor/elementwise.rs */
+    ZO_U_RELU = 32, ZO_U_TANH, ZO_U_GELU, ZO_U_SIGMOID, ZO_U_RSQRT
+};
+enum { /* binary */
+    ZO_B_ADD = 0, ZO_B_SUB, ZO_B_MUL, ZO_B_DIV, ZO_B_POW, ZO_B_MOD, ZO_B_CMPLT, ZO_B_CMPGT, ZO_B_MAX,
+    ZO_B_NOTEQ, ZO_B_EQ, ZO_B_CMPGE
+};
+
+/* tanh = (exp(x+x) - 1) / (exp(x+x) + 1) (zyx/src/tensor/elementwise.rs:585-588);
+ * inf/inf = NaN once exp(2x) overflows (x > ~44.36). */
+static inline float zo_tanh(float z) {
+    float e = expf(z + z);
+    return (e - 1.0f) / (e + 1.0f);
+}
+/* gelu (elementwise.rs:168-170), in the reference's operation order:
+ * (x * 0.5) * (tanh((x + ((x*x)*x) * 0.044715) * sqrt(2/pi)) + 1) */
+static inline float zo_gelu(float x) {
+    float inner = (x + ((x * x) * x) * 0.044715f) * sqrtf(2.0f / 3.14159265358979323846f);
+    return (x * 0.5f) * (zo_tanh(inner) + 1.0f);
+}
+
+static inline float zo_unary(int op, float x) {
+    switch (op) {
+    case ZO_U_NEG: return -x;
+    case ZO_U_EXP: return expf(x);
+    case ZO_U_EXP2: return exp2f(x);
+    case ZO_U_LN: return logf(x);
+    case ZO_U_LOG2: return log2f(x);
+    case ZO_U_RECIPROCAL: return 1.0f / x;
+    case ZO_U_SQRT: return sqrtf(x);
+    case ZO_U_SIN: return sinf(x);
+    case ZO_U_COS: return cosf(x);
+    case ZO_U_FLOOR: return floorf(x);
+    case ZO_U_TRUNC: return truncf(x);
+    case ZO_U_ABS: return fabsf(x);
+    case ZO_U_RELU: return (float)(x > 0.0f) * x; /* (x>0).cast * x, elementwise.rs:289-293 */
+    case ZO_U_TANH: return zo_tanh(x);
+    case ZO_U_GELU: return zo_gelu(x);
+    case ZO_U_SIGMOID: { float e = expf(x); return e / (e + 1.0f); } /* elementwise.rs:457-460 */
+    case ZO_U_RSQRT: return sqrtf(1.0f / x);            /* elementwise.rs:305-307 */
+    default: return NAN;
+    }
+}
+static inline float zo_binary(int op, float x, float y) {
+    switch (op) {
+    case ZO_B_ADD: return x + y;
+    case ZO_B_SUB: return x - y;
+    case ZO_B_MUL: return x * y;
+    case ZO_B_DIV: return x / y;
+    case ZO_B_POW: return exp2f(log2f(x) * y); /* unfold_pows, kernel/fold_constants.rs:639-653 */
+    case ZO_B_MOD: return (float)((int)x % (int)y);
+    case ZO_B_CMPLT: return (float)(x < y);
+    case ZO_B_CMPGT: return (float)(x > y);
+    case ZO_B_CMPGE: return (float)(x >= y);
+    case ZO_B_MAX: return fmaxf(x, y);
+    case ZO_B_NOTEQ: return (float)(x != y);
+    case ZO_B_EQ: return (float)(x == y);
+    default: return NAN;
+    }
+}
+
+/* y[i] = op(x[i]) for a float dtype (f32/bf16/f16 storage). */
+ZO_API void zo_unary_map(int op, int dtype, const void *x, void *y, int64_t n) {
+#pragma omp parallel for
+    for (int64_t i = 0; i < n; i++) store_from_f32(y, dtype, i, zo_unary(op, load_as_f32(x, dtype, i)));
+}
+/* z[r,c] = op(x[r,c], y[...]) where y is same-shape (ybc=0), a row vector of
+ * length cols broadcast over rows (ybc=1) or one scalar (ybc=2). */
+ZO_API void zo_binary_map(int op, int dtype, const void *x, const void *y, void *z, int64_t rows, int64_t cols,
+                          int ybc) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t c = 0; c < cols; c++) {
+            int64_t i = r * cols + c;
+            int64_t j = ybc == 0 ? i : (ybc == 1 ? c : 0);
+            store_from_f32(z, dtype, i, zo_binary(op, load_as_f32(x, dtype, i), load_as_f32(y, dtype, j)));
+        }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Reductions: zyx/src/tensor/reduce_ops.rs:45-147, kernel/linearize.rs:920-952 */
+/* ------------------------------------------------------------------------- */
+
+/* Sum / max over the last axis of a [rows, cols] float tensor. Accumulates in f32
+ * (reduce_acc_dtype) and stores in `dtype`. op: 0 = sum, 1 = max. */
+ZO_API void zo_reduce_rows(int op, int dtype, const void *x, void *y, int64_t rows, int64_t cols) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++) {
+        float acc = op == 0 ? 0.0f : -FLT_MAX;
+        for (int64_t c = 0; c < cols; c++) {
+            float v = load_as_f32(x, dtype, r * cols + c);
+            acc = op == 0 ? v + acc : fmaxf(v, acc);
+        }
+        store_from_f32(y, dtype, r, acc);
+    }
+}
+/* Sum / max over axis 0 of [rows, cols]: one serial loop per output column. */
+ZO_API void zo_reduce_cols(int op, int dtype, const void *x, void *y, int64_t rows, int64_t cols) {
+#pragma omp parallel for
+    for (int64_t c = 0; c < cols; c++) {
+        float acc = op == 0 ? 0.0f : -FLT_MAX;
+        for (int64_t r = 0; r < rows; r++) {
+            float v = load_as_f32(x, dtype, r * cols + c);
+            acc = op == 0 ? v + acc : fmaxf(v, acc);
+        }
+        store_from_f32(y, dtype, c, acc);
+    }
+}
+/* Integer sums accumulate in i32 for narrower ints, i64 stays i64 (reduce_ops.rs:52-60). */
+ZO_API void zo_reduce_rows_i32(int op, const int32_t *x, int32_t *y, int64_t rows, int64_t cols) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++) {
+        int32_t acc = op == 0 ? 0 : INT32_MIN;
+        for (int64_t c = 0; c < cols; c++) {
+            int32_t v = x[r * cols + c];
+            acc = op == 0 ? (int32_t)((uint32_t)v + (uint32_t)acc) : (v > acc ? v : acc);
+        }
+        y[r] = acc;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* softmax (+ row sum, + row argmax): zyx/src/tensor/mod.rs:1457-1461, 2245-2269 */
+/* ------------------------------------------------------------------------- */
+
+/* For every row of x[rows, cols] (f32):
+ *   m = max_c x;  e = exp(x - m);  s = sum_c e;  y = e / s          (softmax)
+ *   rowsum = sum_c y                                                 (Tensor::sum)
+ *   arg = max_c( (y == max_c y) * c )  -> the LARGEST index among ties, i32
+ * Every reduce is the serial register accumulator of the C backend. y, rowsum and
+ * arg may each be NULL. */
+ZO_API void zo_softmax_rows_f32(const float *x, float *y, float *rowsum, int32_t *arg, int64_t rows, int64_t cols) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++) {
+        const float *xr = x + r * cols;
+        float *tmp = y ? y + r * cols : (float *)malloc(sizeof(float) * (size_t)cols);
+        float m = -FLT_MAX;
+        for (int64_t c = 0; c < cols; c++) m = fmaxf(xr[c], m);
+        float s = 0.0f;
+        for (int64_t c = 0; c < cols; c++) {
+            tmp[c] = expf(xr[c] - m);
+            s = tmp[c] + s;
+        }
+        float ys = 0.0f, ymax = -FLT_MAX;
+        for (int64_t c = 0; c < cols; c++) {
+            tmp[c] = tmp[c] / s;
+            ys = tmp[c] + ys;
+            ymax = fmaxf(tmp[c], ymax);
+        }
+        if (rowsum) rowsum[r] = ys;
+        if (arg) {
+            int32_t a = INT32_MIN;
+            for (int64_t c = 0; c < cols; c++) {
+                int32_t idx = (int32_t)(tmp[c] == ymax) * (int32_t)c;
+                a = idx > a ? idx : a;
+            }
+            arg[r] = a;
+        }
+        if (!y) free(tmp);
+    }
+}
+
+/* Same rows, but every accumulation in double: the "what the mathematics fixes"
+ * companion used to bound how far serial f32 summation itself is from the truth. */
+ZO_API void zo_softmax_rows_f64acc(const float *x, float *y, float *rowsum, int64_t rows, int64_t cols) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++) {
+        const float *xr = x + r * cols;
+        double m = -DBL_MAX, s = 0.0, ys = 0.0;
+        for (int64_t c = 0; c < cols; c++) m = xr[c] > m ? xr[c] : m;
+        for (int64_t c = 0; c < cols; c++) s += exp((double)xr[c] - m);
+        for (int64_t c = 0; c < cols; c++) {
+            double v = exp((double)xr[c] - m) / s;
+            if (y) y[r * cols + c] = (float)v;
+            ys += v;
+        }
+        if (rowsum) rowsum[r] = (float)ys;
+    }
+}
+
+/* argmax over the last axis for any f32 tensor (tensor/mod.rs:2245-2269). */
+ZO_API void zo_argmax_rows_f32(const float *x, int32_t *arg, int64_t rows, int64_t cols) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++) {
+        const float *xr = x + r * cols;
+        float m = -FLT_MAX;
+        for (int64_t c = 0; c < cols; c++) m = fmaxf(xr[c], m);
+        int32_t a = INT32_MIN;
+        for (int64_t c = 0; c < cols; c++) {
+            int32_t idx = (int32_t)(xr[c] == m) * (int32_t)c;
+            a = idx > a ? idx : a;
+        }
+        arg[r] = a;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* dot: zyx/src/tensor/mod.rs:1469-1518                                       */
+/* ------------------------------------------------------------------------- */
+
+/* C[m,n] = sum_k A[m,k] * B[k,n], the broadcast-multiply + serial k reduce the
+ * reference lowers to. in_dtype is the storage dtype of A and B; products and the
+ * accumulator live in float registers; the result is stored as out_dtype
+ * (`dot` on bf16 stores bf16, truncating; `dot_dtype(F32)` stores f32).
+ * transb != 0 reads B as [n,k] (Linear's W stored [out,in], linear.rs:38-44). */
+ZO_API void zo_matmul_float(int in_dtype, int out_dtype, const void *a, const void *b, void *c, int64_t m, int64_t n,
+                            int64_t k, int transb) {
+#pragma omp parallel for
+    for (int64_t i = 0; i < m; i++)
+        for (int64_t j = 0; j < n; j++) {
+            float acc = 0.0f;
+            for (int64_t p = 0; p < k; p++) {
+                float x = load_as_f32(a, in_dtype, i * k + p);
+                float y = load_as_f32(b, in_dtype, transb ? j * k + p : p * n + j);
+                acc = x * y + acc;
+            }
+            store_from_f32(c, out_dtype, i * n + j, acc);
+        }
+}
+/* The same product with a double accumulator: tolerance anchor for bf16/f32 GEMM. */
+ZO_API void zo_matmul_f64acc(int in_dtype, const void *a, const void *b, double *c, int64_t m, int64_t n, int64_t k,
+                             int transb) {
+#pragma omp parallel for
+    for (int64_t i = 0; i < m; i++)
+        for (int64_t j = 0; j < n; j++) {
+            double acc = 0.0;
+            for (int64_t p = 0; p < k; p++)
+                acc += (double)load_as_f32(a, in_dtype, i * k + p) *
+                       (double)load_as_f32(b, in_dtype, transb ? j * k + p : p * n + j);
+            c[i * n + j] = acc;
+        }
+}
+/* Integer dot is exact (wrapping) in the operand dtype. */
+ZO_API void zo_matmul_i64(const int64_t *a, const int64_t *b, int64_t *c, int64_t m, int64_t n, int64_t k) {
+#pragma omp parallel for
+    for (int64_t i = 0; i < m; i++)
+        for (int64_t j = 0; j < n; j++) {
+            uint64_t acc = 0;
+            for (int64_t p = 0; p < k; p++) acc += (uint64_t)a[i * k + p] * (uint64_t)b[p * n + j];
+            c[i * n + j] = (int64_t)acc;
+        }
+}
+ZO_API void zo_matmul_i32(const int32_t *a, const int32_t *b, int32_t *c, int64_t m, int64_t n, int64_t k) {
+#pragma omp parallel for
+    for (int64_t i = 0; i < m; i++)
+        for (int64_t j = 0; j < n; j++) {
+            uint32_t acc = 0;
+            for (int64_t p = 0; p < k; p++) acc += (uint32_t)a[i * k + p] * (uint32_t)b[p * n + j];
+            c[i * n + j] = (int32_t)acc;
+        }
+}
+
+/* Linear epilogue on an f32 [m,n] tensor: + bias[n] (bias stored as bias_dtype),
+ * then act: 0 none, 1 relu, 2 gelu (linear.rs:38-44, elementwise.rs:168-170,289-293). */
+ZO_API void zo_bias_act_f32(float *c, const void *bias, int bias_dtype, int64_t m, int64_t n, int act) {
+#pragma omp parallel for
+    for (int64_t i = 0; i < m; i++)
+        for (int64_t j = 0; j < n; j++) {
+            float v = c[i * n + j];
+            if (bias) v = v + load_as_f32(bias, bias_dtype, j);
+            if (act == 1) v = zo_unary(ZO_U_RELU, v);
+            else if (act == 2) v = zo_gelu(v);
+            c[i * n + j] = v;
+        }
+}
