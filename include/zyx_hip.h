@@ -1,0 +1,204 @@
+/*
+ * zyx_hip.h -- C ABI of the MI355X (gfx950) HIP backend for zyx.
+ *
+ * The entry points are what zyx's backend plugin slot for HIP dispatches to: one
+ * `zhip_ctx` stands for the `MemoryPool::HIP` + `Device::HIP` pair the reference
+ * creates per GPU (zyx/src/backend/hip.rs:122-339, zyx/src/backend/mod.rs:533-1028).
+ * Each declaration cites the reference method it replaces (paths relative to the
+ * reference checkout). Plain pointers and sizes only; no C++ or torch types.
+ *
+ * Conventions
+ *   - Every function returning int32_t returns a zhip_status: 0 = ok, 1..13 are the
+ *     reference's ErrorStatus variants in declaration order (zyx/src/error.rs:125-153).
+ *     The message of the last failure on a context is read with zhip_last_error().
+ *   - zhip_buf / zhip_prog are slab indices like PoolBufferId / DeviceProgramId
+ *     (zyx/src/backend/mod.rs:54-55,121-122; zyx/src/slab.rs): dense, reused after
+ *     free, ZHIP_NULL_ID (u32::MAX) = NULL.
+ *   - zhip_event is an opaque handle owned by the caller and consumed exactly once.
+ *     0 is the null event ("already signalled", the analogue of a null hipEvent_t,
+ *     hip.rs:375,396). Wait lists handed to zhip_h2d / zhip_d2h / zhip_launch /
+ *     zhip_free are CONSUMED by the call ("a removed event is consumed",
+ *     zyx/src/runtime.rs:13-15); the reference's HIP stub leaks them instead.
+ *   - Calls may come from any thread; a context serialises them internally (the
+ *     reference calls its backends under one global mutex, zyx/src/lib.rs:96).
+ *   - Launch argument order: read-only buffers first, then written buffers
+ *     (zyx/src/kernel/linearize.rs:138-155; AOT kernels: inputs then outputs,
+ *     zyx/src/backend/cblas.rs:260-263, zyx/src/graph/plan.rs:311-327).
+ *   - Callers over-allocate by one element / 8 bytes (zyx/src/backend/mod.rs:627,
+ *     zyx/src/graph/plan.rs:305); kernels never touch that slack.
+ */
+#ifndef ZYX_HIP_H
+#define ZYX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct zhip_ctx zhip_ctx;
+typedef uint32_t zhip_buf;
+typedef uint32_t zhip_prog;
+typedef uint64_t zhip_event;
+
+#define ZHIP_NULL_ID 0xffffffffu
+
+/* zyx/src/error.rs:125-153 (ErrorStatus), 0 added for success */
+enum zhip_status {
+    ZHIP_OK = 0,
+    ZHIP_DYLIB_NOT_FOUND = 1,
+    ZHIP_INITIALIZATION = 2,
+    ZHIP_DEINITIALIZATION = 3,
+    ZHIP_DEVICE_ENUMERATION = 4,
+    ZHIP_DEVICE_QUERY = 5,
+    ZHIP_MEMORY_ALLOCATION = 6,
+    ZHIP_MEMORY_DEALLOCATION = 7,
+    ZHIP_MEMORY_COPY_H2P = 8,
+    ZHIP_MEMORY_COPY_P2H = 9,
+    ZHIP_INCORRECT_KERNEL_ARG = 10,
+    ZHIP_KERNEL_COMPILATION = 11,
+    ZHIP_KERNEL_LAUNCH = 12,
+    ZHIP_KERNEL_SYNC = 13
+};
+
+/* zyx/src/dtype.rs:20-47 (DType discriminants) */
+enum zhip_dtype {
+    ZHIP_BF16 = 0, ZHIP_F16, ZHIP_F32, ZHIP_F64, ZHIP_U8, ZHIP_U16, ZHIP_U32, ZHIP_U64,
+    ZHIP_I8, ZHIP_I16, ZHIP_I32, ZHIP_I64, ZHIP_BOOL, ZHIP_N_DTYPES
+};
+
+/* HIPConfig (zyx/src/backend/hip.rs:27-32) + the runtime's debug mask
+ * (zyx/src/lib.rs:101-163): bit 0 devices, 5 kernel launches, 6 memory, 7 compile. */
+typedef struct zhip_config {
+    int32_t device_id;  /* HIP device ordinal; one context per device */
+    uint32_t debug;     /* ZYX_DEBUG bitmask */
+    uint64_t cache_bytes; /* freed blocks kept for reuse before going back to the driver; 0 = default (1 GiB) */
+} zhip_config;
+
+/* DeviceInfo (zyx/src/backend/mod.rs:506-531), filled from the device's properties. */
+typedef struct zhip_device_info {
+    uint64_t compute;                  /* peak f32 vector flop/s (u128 in the reference) */
+    uint64_t max_global_work_dims[3];
+    uint32_t max_local_threads;
+    uint32_t max_local_work_dims[3];
+    uint32_t preferred_vector_size;    /* bytes */
+    uint64_t local_mem_size;           /* LDS bytes a workgroup may use */
+    uint64_t max_register_bytes;
+    uint32_t tensor_cores;             /* MFMA present */
+    uint32_t warp_size;                /* 64 */
+    uint32_t dtype_capability[ZHIP_N_DTYPES]; /* DTypeCapability bits, mod.rs:440-471 */
+    uint32_t has_native_exp2;
+    uint32_t n_supported_vec_lens;
+    uint32_t supported_vec_lens[4];
+    /* not in the reference struct; for reports */
+    uint64_t total_bytes;
+    uint32_t compute_units;
+    uint32_t clock_khz;
+    char name[64];
+    char arch[32];
+} zhip_device_info;
+
+/* Hand-written kernels, registered as AOT programs (the slot cblas/cuDNN fill in the
+ * reference: zyx/src/backend/cblas.rs:213-238, zyx/src/backend/cuda.rs:1033-1074). */
+enum zhip_kernel_kind {
+    /* x[rows,cols] -> y = softmax(x, -1), rowsum = y.sum(-1), arg = y.argmax_axis(-1).
+     * dims = {rows, cols}; flags selects outputs (ZHIP_SOFTMAX_*); args: x, then the
+     * selected outputs in the order y, rowsum, arg.
+     * zyx/src/tensor/mod.rs:1457-1461, 2245-2269; zyx/src/tensor/reduce_ops.rs:197-199 */
+    ZHIP_K_SOFTMAX_ROWS = 1,
+    ZHIP_K_COUNT_
+};
+#define ZHIP_SOFTMAX_Y 1
+#define ZHIP_SOFTMAX_ROWSUM 2
+#define ZHIP_SOFTMAX_ARGMAX 4
+
+typedef struct zhip_kernel_desc {
+    int32_t kind;       /* zhip_kernel_kind */
+    int32_t dtype;      /* element dtype of the main operands */
+    int32_t out_dtype;  /* result dtype where it may differ */
+    int32_t flags;      /* kind specific */
+    int64_t dims[8];    /* kind specific sizes, fixed at registration like cblas m,n,k */
+    float fparams[4];   /* kind specific scalars */
+    int32_t iparams[8]; /* kind specific op codes */
+} zhip_kernel_desc;
+
+/* --- backend lifetime ------------------------------------------------------- */
+
+/* Number of usable GPUs (device enumeration of hip.rs:190-215). */
+int32_t zhip_device_count(int32_t *count);
+/* initialize_device (hip.rs:122-339): context, pool stream, 8 launch streams. */
+int32_t zhip_init(const zhip_config *cfg, zhip_ctx **out);
+/* HIPMemoryPool::deinitialize + HIPDevice::deinitialize (hip.rs:341-347, 489-493):
+ * drains streams, frees every buffer, program and event. */
+int32_t zhip_deinit(zhip_ctx *ctx);
+/* Message of the last failed call on ctx (ctx == NULL: last failed zhip_init /
+ * zhip_device_count on this thread). BackendError.context, zyx/src/error.rs:107-111. */
+const char *zhip_last_error(zhip_ctx *ctx);
+/* HIPDevice::info (hip.rs:495-497) */
+int32_t zhip_get_device_info(zhip_ctx *ctx, zhip_device_info *info);
+/* HIPMemoryPool::free_bytes (hip.rs:350): bookkeeping counter, not a driver query. */
+uint64_t zhip_free_bytes(zhip_ctx *ctx);
+/* HIPDevice::free_compute (hip.rs:726-728): device-selection weight. */
+uint64_t zhip_free_compute(zhip_ctx *ctx);
+
+/* --- memory pool ------------------------------------------------------------ */
+
+/* HIPMemoryPool::allocate (hip.rs:354-370). Fails with ZHIP_MEMORY_ALLOCATION when
+ * bytes > free_bytes. *ev is the event the first user must wait on (0 when the
+ * block is ready at once). */
+int32_t zhip_alloc(zhip_ctx *ctx, uint64_t bytes, zhip_buf *buf, zhip_event *ev);
+/* HIPMemoryPool::deallocate (hip.rs:373-385). Consumes evs. */
+int32_t zhip_free(zhip_ctx *ctx, zhip_buf buf, const zhip_event *evs, size_t n_evs);
+/* MemoryPool::store_variable / get_variable (backend/mod.rs:597-621): scalar kernel
+ * arguments live in the buffer id space; value = up to 8 little-endian bytes. */
+int32_t zhip_store_variable(zhip_ctx *ctx, int32_t dtype, const uint8_t value[8], zhip_buf *buf);
+int32_t zhip_get_variable(zhip_ctx *ctx, zhip_buf buf, int32_t *found, int32_t *dtype, uint8_t value[8]);
+/* HIPMemoryPool::host_to_pool (hip.rs:387-409): async; src must stay valid until
+ * *ev is synced. Consumes evs. */
+int32_t zhip_h2d(zhip_ctx *ctx, const void *src, uint64_t bytes, zhip_buf dst, const zhip_event *evs, size_t n_evs,
+                 zhip_event *ev);
+/* HIPMemoryPool::pool_to_host (hip.rs:411-434): blocks until the bytes are in dst.
+ * Consumes evs. */
+int32_t zhip_d2h(zhip_ctx *ctx, zhip_buf src, void *dst, uint64_t bytes, const zhip_event *evs, size_t n_evs);
+/* MemoryPool::pool_to_pool with a device source (backend/mod.rs:743-764, todo!() for
+ * HIP in the reference): device-to-device copy inside this pool. Consumes evs. */
+int32_t zhip_d2d(zhip_ctx *ctx, zhip_buf src, zhip_buf dst, uint64_t bytes, const zhip_event *evs, size_t n_evs,
+                 zhip_event *ev);
+/* HIPMemoryPool::sync_events (hip.rs:440-448): wait, then destroy. */
+int32_t zhip_sync_events(zhip_ctx *ctx, const zhip_event *evs, size_t n_evs);
+/* HIPMemoryPool::release_events (hip.rs:451-458): destroy without waiting. */
+int32_t zhip_release_events(zhip_ctx *ctx, const zhip_event *evs, size_t n_evs);
+/* Raw device address and size of a buffer (HIPBuffer{ptr,bytes}, hip.rs:85-88), for
+ * interop with other code on the same device. */
+int32_t zhip_buffer_ptr(zhip_ctx *ctx, zhip_buf buf, void **ptr, uint64_t *bytes);
+
+/* --- device ----------------------------------------------------------------- */
+
+/* AOT registration: validates desc and returns a program id, the role
+ * `self.programs.push(..)` plays in CblasDevice::match_graph (cblas.rs:225). */
+int32_t zhip_register_kernel(zhip_ctx *ctx, const zhip_kernel_desc *desc, zhip_prog *prog);
+/* Device::compile for generic kernel IR (backend/mod.rs:899-933). This backend is
+ * AOT-only (backend/mod.rs:892-894): always ZHIP_KERNEL_COMPILATION, the answer
+ * CblasDevice::compile gives (cblas.rs:203-208). */
+int32_t zhip_compile_ir(zhip_ctx *ctx, const void *ir, uint64_t ir_bytes, zhip_prog *prog);
+/* HIPDevice::launch (hip.rs:654-719). args = inputs then outputs; every argument is
+ * checked against the size the program needs before anything is enqueued. Consumes evs. */
+int32_t zhip_launch(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args, size_t n_args, const zhip_event *evs,
+                    size_t n_evs, zhip_event *ev);
+/* HIPDevice::release (hip.rs:721-724) */
+int32_t zhip_release_program(zhip_ctx *ctx, zhip_prog prog);
+/* launch_with_timings (zyx/src/kernel/autotune.rs:775-798): launch, sync, host
+ * wall-clock nanoseconds -- the value for Node::Kernel.time (graph/mod.rs:177-182). */
+int32_t zhip_time_kernel(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args, size_t n_args, uint64_t *ns);
+/* Device-side duration: `iters` back-to-back launches bracketed by HIP events on the
+ * stream they run on; *avg_us = mean microseconds per launch. arg_sets > 1 cycles
+ * through that many consecutive argument tuples (args holds arg_sets * n_args ids) so
+ * successive launches touch different memory. */
+int32_t zhip_profile_kernel(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args, size_t n_args, size_t arg_sets,
+                            int32_t iters, float *avg_us);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ZYX_HIP_H */

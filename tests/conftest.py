@@ -18,3 +18,13 @@ def oracle():
 
     _oracle.build()
     return _oracle
+
+
+@pytest.fixture(scope="session")
+def hip():
+    """(device, pool) on GPU 0 through the C ABI. No fallback: a missing library or GPU fails the test."""
+    import zyx_amd
+
+    pools, devices = zyx_amd.initialize_device(zyx_amd.HIPConfig(device_ids=[0]))
+    yield devices[0], pools[0]
+    pools[0].deinitialize()

@@ -1,0 +1,125 @@
+"""The pool / device calls of the HIP backend slot, exercised the way the reference's runtime
+drives them (zyx/src/runtime.rs:2075-2308, zyx/src/graph/plan.rs:271-361) on a real GPU."""
+import numpy as np
+import pytest
+
+from zyx_amd import BackendError, DType, ErrorStatus, Event, kernels
+
+pytestmark = pytest.mark.gpu
+
+
+def test_device_info(hip):
+    dev, pool = hip
+    info = dev.info()
+    assert info.arch.startswith("gfx950")
+    assert info.warp_size == 64 and info.tensor_cores and info.has_native_exp2
+    assert info.max_local_threads == 1024 and info.preferred_vector_size == 16
+    assert dev.aot_only() and dev.memory_pool_id() == 0
+    assert dev.free_compute() > 10 * 2**40  # must outrank the C backend's weight (c.rs:120)
+    assert pool.free_bytes() > 100 * 2**30
+
+
+def test_alloc_copy_roundtrip_and_accounting(hip):
+    dev, pool = hip
+    before = pool.free_bytes()
+    data = np.arange(100003, dtype=np.int32)
+    buf, ev = pool.allocate(data.nbytes + 8)
+    assert pool.free_bytes() == before - (data.nbytes + 8)
+    ev2 = pool.host_to_pool(data, buf, [ev])
+    out = np.empty_like(data)
+    pool.pool_to_host(buf, out, [ev2])
+    assert np.array_equal(out, data)
+    pool.deallocate(buf, [])
+    assert pool.free_bytes() == before
+
+
+def test_ids_are_reused_lowest_first(hip):
+    dev, pool = hip
+    ids = [pool.allocate(1024)[0] for _ in range(4)]
+    pool.deallocate(ids[1], [])
+    pool.deallocate(ids[2], [])
+    again = pool.allocate(64)[0]
+    assert again == ids[1]
+    for b in (ids[0], ids[3], again):
+        pool.deallocate(b, [])
+
+
+def test_oversized_allocation_fails(hip):
+    dev, pool = hip
+    with pytest.raises(BackendError) as ei:
+        pool.allocate(pool.free_bytes() + 1)
+    assert ei.value.status == ErrorStatus.MemoryAllocation and "Allocation failure" in ei.value.context
+
+
+def test_variables_live_in_buffer_id_space(hip):
+    dev, pool = hip
+    v = pool.store_variable(DType.I64, 42)
+    f = pool.store_variable(DType.F32, 0.5)
+    m, ev = pool.allocate(64)
+    assert pool.get_variable(v) == (DType.I64, 42)
+    assert pool.get_variable(f) == (DType.F32, 0.5)
+    assert pool.get_variable(m) is None
+    assert len({v, f, m}) == 3
+    prog = dev.register_kernel(kernels.softmax_rows_desc(1, 4, True, False, False))
+    with pytest.raises(BackendError) as ei:  # a scalar where memory is expected
+        dev.launch(prog, pool, [m, v], [ev])
+    assert ei.value.status == ErrorStatus.IncorrectKernelArg
+    dev.release(prog)
+    for b in (v, f, m):
+        pool.deallocate(b, [])
+
+
+def test_events_are_consumed_once(hip):
+    dev, pool = hip
+    data = np.ones(1024, np.float32)
+    buf, ev = pool.allocate(data.nbytes + 4)
+    e = pool.host_to_pool(data, buf, [ev])
+    pool.sync_events([e])
+    with pytest.raises(BackendError) as ei:
+        pool.sync_events([e])  # stale handle: an error, never a crash
+    assert ei.value.status == ErrorStatus.KernelSync
+    pool.sync_events([Event(0)])  # the null event is always signalled
+    e = pool.host_to_pool(data, buf, [])
+    pool.release_events([e])
+    pool.deallocate(buf, [])
+
+
+def test_generic_ir_is_refused(hip):
+    dev, pool = hip
+    with pytest.raises(BackendError) as ei:
+        dev.compile(b"\x00" * 16)
+    assert ei.value.status == ErrorStatus.KernelCompilation
+
+
+def test_dependent_launch_chain_and_block_reuse(hip, oracle):
+    """softmax(softmax(x)) through freed-and-reused blocks: the second launch must see the first's output."""
+    dev, pool = hip
+    x = oracle.Rng(1).randn((512, 1024), 3.0)
+    prog = dev.register_kernel(kernels.softmax_rows_desc(512, 1024, True, False, False))
+    want = oracle.softmax_rows(oracle.softmax_rows(x)[0])[0]
+    for _ in range(3):
+        xb, e0 = kernels.to_device(pool, x)
+        y1, e1 = pool.allocate(x.nbytes + 4)
+        l1 = dev.launch(prog, pool, [xb, y1], [e0, e1])
+        y2, e2 = pool.allocate(x.nbytes + 4)
+        l2 = dev.launch(prog, pool, [y1, y2], [l1, e2])
+        got = kernels.to_host(pool, y2, x.shape, np.float32, [l2])
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-37)
+        for b in (xb, y1, y2):
+            pool.deallocate(b, [])
+    dev.release(prog)
+
+
+def test_timer_and_profile(hip, oracle):
+    dev, pool = hip
+    x = oracle.Rng(2).randn((1024, 4096), 3.0)
+    prog = dev.register_kernel(kernels.softmax_rows_desc(1024, 4096))
+    xb, e0 = kernels.to_device(pool, x)
+    outs = [pool.allocate(n)[0] for n in (x.nbytes + 4, 1024 * 4 + 4, 1024 * 4 + 4)]
+    pool.sync_events([e0])
+    ns = dev.time_kernel(prog, [xb] + outs)
+    us = dev.profile_kernel(prog, [[xb] + outs], 10)
+    assert 0 < us < 1e4 and ns > 0
+    for b in [xb] + outs:
+        pool.deallocate(b, [])
+    dev.release(prog)

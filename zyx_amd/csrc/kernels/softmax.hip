@@ -1,0 +1,167 @@
+// Fused row softmax (+ row sum of the result, + row argmax of the result), f32.
+//
+// Computes what zyx evaluates as >= 5 kernels for
+//   y = x.softmax([-1]); s = y.sum([-1]); a = y.argmax_axis(-1)
+// (zyx/src/tensor/mod.rs:1457-1461, 2245-2269; zyx/src/tensor/reduce_ops.rs:45-147)
+// in one pass over HBM: x is read once, y written once.
+//
+// Register-resident variant: one 64-lane wave owns one row of up to 4096 columns,
+// each lane holding NV float4 (lane + 64*j addressing, so every load/store
+// instruction of a wave covers 1 KiB of consecutive bytes). The three row
+// reductions (max, sum of exp, sum/argmax of y) are DPP + readlane wave reductions:
+// no LDS, no barriers. Four waves per workgroup -> rows/4 workgroups.
+#include "kernels.hpp"
+#include "wave.hpp"
+
+namespace zk {
+
+// FULL: cols == 256*NV exactly, so no lane is ever masked.
+template <int NV, bool FULL, bool WY, bool WS, bool WA>
+__global__ __launch_bounds__(256) void softmax_rows_wave_k(const float *__restrict__ x, float *__restrict__ y,
+                                                           float *__restrict__ rowsum, int32_t *__restrict__ arg,
+                                                           int rows, int cols) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return; // whole wave leaves together; nothing below synchronises across waves
+    const int nvec = cols >> 2;
+    const f32x4 *xr = reinterpret_cast<const f32x4 *>(x + (size_t)row * cols);
+
+    f32x4 v[NV];
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        int i = lane + 64 * j;
+        if (FULL || i < nvec) v[j] = load_stream(xr + i);
+        else v[j] = f32x4{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+    }
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < NV; j++) m = fmaxf(fmaxf(fmaxf(v[j].x, v[j].y), fmaxf(v[j].z, v[j].w)), m);
+    m = wave_allreduce_f32(m, OpMaxF());
+
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        bool live = FULL || lane + 64 * j < nvec;
+        v[j].x = live ? exp_neg(v[j].x - m) : 0.0f;
+        v[j].y = live ? exp_neg(v[j].y - m) : 0.0f;
+        v[j].z = live ? exp_neg(v[j].z - m) : 0.0f;
+        v[j].w = live ? exp_neg(v[j].w - m) : 0.0f;
+        s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+    }
+    s = wave_allreduce_f32(s, OpAdd());
+    const float inv = 1.0f / s; // y of the row maximum (its exp is exactly 1), hence max(y)
+
+    float ys = 0.0f;
+    int best = 0;
+    f32x4 *yr = reinterpret_cast<f32x4 *>(y + (size_t)row * cols);
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        int i = lane + 64 * j;
+        f32x4 o = v[j] * inv;
+        if (WS) ys += (o.x + o.y) + (o.z + o.w);
+        if (WA) { // largest column whose y equals max(y): max_k((y == ymax) * k)
+            int c = i * 4;
+            best = o.x == inv ? max(best, c) : best;
+            best = o.y == inv ? max(best, c + 1) : best;
+            best = o.z == inv ? max(best, c + 2) : best;
+            best = o.w == inv ? max(best, c + 3) : best;
+        }
+        if (WY && (FULL || i < nvec)) store_stream(o, yr + i);
+    }
+    if (WS) {
+        ys = wave_allreduce_f32(ys, OpAdd());
+        if (lane == 0) rowsum[row] = ys;
+    }
+    if (WA) {
+        best = wave_allreduce_i32(best, OpMaxI());
+        if (lane == 0) arg[row] = best;
+    }
+}
+
+// Any cols / alignment: one 256-thread workgroup per row, three passes over the row
+// (rows of this size stay in L2 between passes), LDS only for the cross-wave folds.
+template <class Op> __device__ __forceinline__ float block_allreduce_f32(float v, Op op, float *lds) {
+    v = wave_allreduce_f32(v, op);
+    __syncthreads(); // lds may still be read from the previous reduction
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return op(op(lds[0], lds[1]), op(lds[2], lds[3]));
+}
+
+__global__ __launch_bounds__(256) void softmax_rows_generic_k(const float *__restrict__ x, float *__restrict__ y,
+                                                              float *__restrict__ rowsum, int32_t *__restrict__ arg,
+                                                              int rows, int64_t cols) {
+    __shared__ float lds[4];
+    __shared__ int ldsi[4];
+    const int64_t row = blockIdx.x; // grid == rows, every thread of the block reaches every barrier
+    const float *xr = x + row * cols;
+    float m = -FLT_MAX;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) m = fmaxf(xr[c], m);
+    m = block_allreduce_f32(m, OpMaxF(), lds);
+    float s = 0.0f;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) s += exp_neg(xr[c] - m);
+    s = block_allreduce_f32(s, OpAdd(), lds);
+    const float inv = 1.0f / s;
+    float ys = 0.0f;
+    int best = 0;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) {
+        float o = exp_neg(xr[c] - m) * inv;
+        ys += o;
+        best = o == inv ? max(best, (int)c) : best;
+        if (y) y[row * cols + c] = o;
+    }
+    if (rowsum) {
+        ys = block_allreduce_f32(ys, OpAdd(), lds);
+        if (threadIdx.x == 0) rowsum[row] = ys;
+    }
+    if (arg) {
+        best = wave_allreduce_i32(best, OpMaxI());
+        if ((threadIdx.x & 63) == 0) ldsi[threadIdx.x >> 6] = best;
+        __syncthreads();
+        if (threadIdx.x == 0) arg[row] = max(max(ldsi[0], ldsi[1]), max(ldsi[2], ldsi[3]));
+    }
+}
+
+template <int NV> static hipError_t launch_wave(const SoftmaxRows &p, hipStream_t st) {
+    dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
+    int rows = (int)p.rows, cols = (int)p.cols;
+    int sel = (p.y ? 1 : 0) | (p.rowsum ? 2 : 0) | (p.arg ? 4 : 0);
+    bool full = p.cols == 256 * NV;
+#define ZK_CASE(S, A, B, C)                                                                                           \
+    case S:                                                                                                           \
+        if (full)                                                                                                     \
+            hipLaunchKernelGGL((softmax_rows_wave_k<NV, true, A, B, C>), grid, block, 0, st, p.x, p.y, p.rowsum,     \
+                               p.arg, rows, cols);                                                                    \
+        else                                                                                                          \
+            hipLaunchKernelGGL((softmax_rows_wave_k<NV, false, A, B, C>), grid, block, 0, st, p.x, p.y, p.rowsum,    \
+                               p.arg, rows, cols);                                                                    \
+        break;
+    switch (sel) {
+        ZK_CASE(1, true, false, false) ZK_CASE(2, false, true, false) ZK_CASE(3, true, true, false)
+        ZK_CASE(4, false, false, true) ZK_CASE(5, true, false, true) ZK_CASE(6, false, true, true)
+        ZK_CASE(7, true, true, true)
+    default: return hipErrorInvalidValue;
+    }
+#undef ZK_CASE
+    return hipGetLastError();
+}
+
+hipError_t softmax_rows(const SoftmaxRows &p, hipStream_t st) {
+    if (p.rows <= 0 || p.cols <= 0) return hipSuccess; // empty tensor: nothing to write
+    bool vec_ok = (p.cols % 4 == 0) && p.cols <= 4096 && (reinterpret_cast<uintptr_t>(p.x) % 16 == 0) &&
+                  (p.y == nullptr || reinterpret_cast<uintptr_t>(p.y) % 16 == 0) && p.rows < (1ll << 31) - 4;
+    if (vec_ok) {
+        int64_t nvec = p.cols / 4;
+        if (nvec <= 64) return launch_wave<1>(p, st);
+        if (nvec <= 128) return launch_wave<2>(p, st);
+        if (nvec <= 256) return launch_wave<4>(p, st);
+        if (nvec <= 512) return launch_wave<8>(p, st);
+        return launch_wave<16>(p, st);
+    }
+    if (p.rows >= (1ll << 31) || p.cols >= (1ll << 31)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(softmax_rows_generic_k, dim3((unsigned)p.rows), dim3(256), 0, st, p.x, p.y, p.rowsum, p.arg,
+                       (int)p.rows, p.cols);
+    return hipGetLastError();
+}
+
+} // namespace zk

@@ -1,0 +1,733 @@
+// Host side of the MI355X HIP backend: the memory pool (caching allocator, async
+// copies, scalar variables), the event table, the stream scheduler and the program
+// registry behind the C ABI declared in include/zyx_hip.h.
+//
+// Design points that differ from the slot this fills (zyx/src/backend/hip.rs):
+//   * Events are pooled: hipEventCreate/Destroy happen once per slot, a handle is
+//     {slot, generation} so a stale or doubly consumed handle is an error, not a crash.
+//   * Launch streams are chosen by affinity: a launch goes to the stream that
+//     recorded the newest event of its wait list, so a dependency chain stays in one
+//     in-order stream and needs no cross-stream wait; independent work round-robins
+//     over the 8 launch streams.
+//   * Freed blocks are cached by size class together with the events of their last
+//     users; a reused block hands those events' completion to its next user through
+//     the event zhip_alloc returns. hipMalloc/hipFree (device-wide synchronising)
+//     leave the steady-state training step.
+#include "../../include/zyx_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "kernels/kernels.hpp"
+
+#define ZHIP_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+constexpr int kLaunchStreams = 8; // zyx/src/backend/hip.rs:242-274
+constexpr uint64_t kDefaultCacheBytes = 1ull << 30;
+constexpr uint64_t kAllocAlign = 256;
+
+thread_local std::string g_init_error;
+
+struct Buffer {
+    enum Kind : uint8_t { Free, Memory, Variable } kind = Free;
+    void *ptr = nullptr;
+    uint64_t bytes = 0;    // what the caller asked for (bookkeeping unit of free_bytes)
+    uint64_t capacity = 0; // size class actually backing it
+    int32_t var_dtype = 0;
+    uint8_t var_value[8] = {0};
+};
+
+struct EventSlot {
+    hipEvent_t ev = nullptr;
+    uint32_t gen = 1;
+    int16_t stream = -1; // launch stream index, -1 = pool stream
+    uint64_t seq = 0;    // position in that stream's record order
+    bool live = false;
+};
+
+struct CachedBlock {
+    void *ptr;
+    std::vector<zhip_event> pending; // last users; owned by the cache
+};
+
+struct Program {
+    bool live = false;
+    zhip_kernel_desc desc{};
+    int n_in = 0, n_out = 0;
+    uint64_t need[8] = {0}; // minimum bytes per argument
+};
+
+template <class T> struct Slab { // dense ids, lowest free id reused (zyx/src/slab.rs)
+    std::vector<T> items;
+    std::vector<uint32_t> free_ids;
+    uint32_t push(T v) {
+        if (!free_ids.empty()) {
+            // lowest id first keeps ids dense and deterministic
+            size_t best = 0;
+            for (size_t i = 1; i < free_ids.size(); i++)
+                if (free_ids[i] < free_ids[best]) best = i;
+            uint32_t id = free_ids[best];
+            free_ids.erase(free_ids.begin() + best);
+            items[id] = std::move(v);
+            return id;
+        }
+        items.push_back(std::move(v));
+        return (uint32_t)items.size() - 1;
+    }
+    void remove(uint32_t id) { free_ids.push_back(id); }
+};
+
+} // namespace
+
+struct zhip_ctx {
+    std::mutex mu;
+    int device = 0;
+    uint32_t debug = 0;
+    std::string last_error;
+    hipDeviceProp_t prop{};
+    zhip_device_info info{};
+
+    hipStream_t pool_stream = nullptr;
+    hipStream_t launch_streams[kLaunchStreams] = {nullptr};
+    uint64_t stream_seq[kLaunchStreams + 1] = {0}; // [kLaunchStreams] = pool stream
+    int rr = 0;
+
+    uint64_t free_bytes = 0;
+    uint64_t cache_limit = kDefaultCacheBytes, cached_bytes = 0;
+    Slab<Buffer> buffers;
+    std::map<uint64_t, std::vector<CachedBlock>> cache; // capacity -> blocks
+    std::vector<EventSlot> events;
+    std::vector<uint32_t> free_events;
+    Slab<Program> programs;
+    hipEvent_t prof_a = nullptr, prof_b = nullptr;
+
+    int32_t fail(int32_t status, const char *fmt, ...) __attribute__((format(printf, 3, 4))) {
+        char buf[512];
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(buf, sizeof buf, fmt, ap);
+        va_end(ap);
+        last_error = buf;
+        if (debug & 1) fprintf(stderr, "[zyx-hip] error %d: %s\n", status, buf);
+        return status;
+    }
+};
+
+#define HIPCHK(ctx, call, status)                                                                                     \
+    do {                                                                                                              \
+        hipError_t e_ = (call);                                                                                       \
+        if (e_ != hipSuccess) return (ctx)->fail((status), "%s failed: %s", #call, hipGetErrorString(e_));            \
+    } while (0)
+
+namespace {
+
+uint64_t size_class(uint64_t bytes) {
+    if (bytes < kAllocAlign) return kAllocAlign;
+    // 8 classes per power of two: at most 12.5% slack, few distinct sizes to cache
+    int msb = 63 - __builtin_clzll(bytes);
+    uint64_t step = 1ull << (msb > 3 ? msb - 3 : 0);
+    if (step < kAllocAlign) step = kAllocAlign;
+    return (bytes + step - 1) / step * step;
+}
+
+hipStream_t stream_of(zhip_ctx *c, int idx) { return idx < 0 ? c->pool_stream : c->launch_streams[idx]; }
+
+// --- events ---------------------------------------------------------------------
+EventSlot *event_lookup(zhip_ctx *c, zhip_event h) {
+    if (h == 0) return nullptr;
+    uint32_t idx = (uint32_t)(h & 0xffffffffu) - 1, gen = (uint32_t)(h >> 32);
+    if (idx >= c->events.size()) return nullptr;
+    EventSlot &s = c->events[idx];
+    return (s.live && s.gen == gen) ? &s : nullptr;
+}
+int32_t event_record(zhip_ctx *c, int stream_idx, int32_t status, zhip_event *out) {
+    uint32_t idx;
+    if (!c->free_events.empty()) {
+        idx = c->free_events.back();
+        c->free_events.pop_back();
+    } else {
+        EventSlot s;
+        HIPCHK(c, hipEventCreateWithFlags(&s.ev, hipEventDisableTiming), status);
+        c->events.push_back(s);
+        idx = (uint32_t)c->events.size() - 1;
+    }
+    EventSlot &s = c->events[idx];
+    hipError_t e = hipEventRecord(s.ev, stream_of(c, stream_idx));
+    if (e != hipSuccess) {
+        c->free_events.push_back(idx);
+        return c->fail(status, "hipEventRecord failed: %s", hipGetErrorString(e));
+    }
+    s.live = true;
+    s.stream = (int16_t)stream_idx;
+    s.seq = ++c->stream_seq[stream_idx < 0 ? kLaunchStreams : stream_idx];
+    *out = ((uint64_t)s.gen << 32) | (uint64_t)(idx + 1);
+    return ZHIP_OK;
+}
+void event_retire(zhip_ctx *c, EventSlot *s) {
+    s->live = false;
+    s->gen++;
+    if (s->gen == 0) s->gen = 1;
+    c->free_events.push_back((uint32_t)(s - c->events.data()));
+}
+// Makes `stream_idx` wait for every event of the list, then retires them (the call
+// consumes its wait list). Events recorded on the same in-order stream need no wait.
+int32_t wait_and_consume(zhip_ctx *c, int stream_idx, const zhip_event *evs, size_t n, int32_t status) {
+    int32_t rc = ZHIP_OK;
+    for (size_t i = 0; i < n; i++) {
+        if (evs[i] == 0) continue;
+        EventSlot *s = event_lookup(c, evs[i]);
+        if (!s) {
+            rc = c->fail(status, "wait list entry %zu is not a live event (stale or already consumed handle)", i);
+            continue;
+        }
+        if (s->stream != stream_idx) {
+            hipError_t e = hipStreamWaitEvent(stream_of(c, stream_idx), s->ev, 0);
+            if (e != hipSuccess) rc = c->fail(status, "hipStreamWaitEvent failed: %s", hipGetErrorString(e));
+        }
+        event_retire(c, s);
+    }
+    return rc;
+}
+
+// --- buffers --------------------------------------------------------------------
+Buffer *buffer_lookup(zhip_ctx *c, zhip_buf id) {
+    if (id >= c->buffers.items.size()) return nullptr;
+    Buffer &b = c->buffers.items[id];
+    return b.kind == Buffer::Free ? nullptr : &b;
+}
+
+void trim_cache(zhip_ctx *c, uint64_t limit) {
+    // Blocks go back to the driver largest first; their pending events are waited for
+    // by hipFree's own device synchronisation.
+    while (c->cached_bytes > limit && !c->cache.empty()) {
+        auto it = std::prev(c->cache.end());
+        CachedBlock blk = std::move(it->second.back());
+        it->second.pop_back();
+        uint64_t cap = it->first;
+        if (it->second.empty()) c->cache.erase(it);
+        for (zhip_event h : blk.pending)
+            if (EventSlot *s = event_lookup(c, h)) {
+                (void)hipEventSynchronize(s->ev);
+                event_retire(c, s);
+            }
+        (void)hipFree(blk.ptr);
+        c->cached_bytes -= cap;
+    }
+}
+
+// --- program registry -----------------------------------------------------------
+uint64_t dtype_bytes(int32_t dt) {
+    switch (dt) {
+    case ZHIP_BF16: case ZHIP_F16: case ZHIP_U16: case ZHIP_I16: return 2;
+    case ZHIP_F32: case ZHIP_U32: case ZHIP_I32: return 4;
+    case ZHIP_F64: case ZHIP_U64: case ZHIP_I64: return 8;
+    case ZHIP_U8: case ZHIP_I8: case ZHIP_BOOL: return 1;
+    default: return 0;
+    }
+}
+
+// Fills arity and per-argument byte requirements; rejects shapes/dtypes no kernel covers.
+int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
+    p.desc = d;
+    switch (d.kind) {
+    case ZHIP_K_SOFTMAX_ROWS: {
+        int64_t rows = d.dims[0], cols = d.dims[1];
+        if (d.dtype != ZHIP_F32) return c->fail(ZHIP_KERNEL_COMPILATION, "softmax_rows: only f32 is implemented");
+        if (rows < 0 || cols < 0 || rows >= (1ll << 31) || cols >= (1ll << 31))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "softmax_rows: rows/cols out of range");
+        if ((d.flags & 7) == 0 || (d.flags & ~7)) return c->fail(ZHIP_KERNEL_COMPILATION, "softmax_rows: bad output flags");
+        p.n_in = 1;
+        p.need[0] = (uint64_t)rows * cols * 4;
+        int o = 1;
+        if (d.flags & ZHIP_SOFTMAX_Y) p.need[o++] = (uint64_t)rows * cols * 4;
+        if (d.flags & ZHIP_SOFTMAX_ROWSUM) p.need[o++] = (uint64_t)rows * 4;
+        if (d.flags & ZHIP_SOFTMAX_ARGMAX) p.need[o++] = (uint64_t)rows * 4;
+        p.n_out = o - 1;
+        return ZHIP_OK;
+    }
+    default: return c->fail(ZHIP_KERNEL_COMPILATION, "unknown kernel kind %d", d.kind);
+    }
+}
+
+hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
+    const zhip_kernel_desc &d = p.desc;
+    switch (d.kind) {
+    case ZHIP_K_SOFTMAX_ROWS: {
+        zk::SoftmaxRows a{};
+        a.rows = d.dims[0];
+        a.cols = d.dims[1];
+        a.x = (const float *)ptr[0];
+        int o = 1;
+        if (d.flags & ZHIP_SOFTMAX_Y) a.y = (float *)ptr[o++];
+        if (d.flags & ZHIP_SOFTMAX_ROWSUM) a.rowsum = (float *)ptr[o++];
+        if (d.flags & ZHIP_SOFTMAX_ARGMAX) a.arg = (int32_t *)ptr[o++];
+        return zk::softmax_rows(a, st);
+    }
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// Resolves and checks launch arguments: arity, liveness, kind and size.
+int32_t resolve_args(zhip_ctx *c, zhip_prog prog, const zhip_buf *args, size_t n_args, Program **pp, void **ptr) {
+    if (prog >= c->programs.items.size() || !c->programs.items[prog].live)
+        return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "program %u does not exist", prog);
+    Program &p = c->programs.items[prog];
+    if (n_args != (size_t)(p.n_in + p.n_out))
+        return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "program %u takes %d inputs + %d outputs, got %zu arguments", prog,
+                       p.n_in, p.n_out, n_args);
+    for (size_t i = 0; i < n_args; i++) {
+        Buffer *b = buffer_lookup(c, args[i]);
+        if (!b) return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "argument %zu: buffer %u does not exist", i, args[i]);
+        if (b->kind != Buffer::Memory)
+            return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "argument %zu: buffer %u is a scalar variable, memory expected", i,
+                           args[i]);
+        if (b->bytes < p.need[i])
+            return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "argument %zu: buffer %u holds %llu bytes, kernel needs %llu", i,
+                           args[i], (unsigned long long)b->bytes, (unsigned long long)p.need[i]);
+        ptr[i] = b->ptr;
+    }
+    // an output must not alias an input or another output: the kernels assume restrict
+    for (size_t i = p.n_in; i < n_args; i++)
+        for (size_t j = 0; j < i; j++)
+            if (ptr[i] == ptr[j] && p.need[i] && p.need[j])
+                return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "arguments %zu and %zu are the same buffer", j, i);
+    *pp = &p;
+    return ZHIP_OK;
+}
+
+int pick_stream(zhip_ctx *c, const zhip_event *evs, size_t n) {
+    int best = -1;
+    uint64_t best_seq = 0;
+    for (size_t i = 0; i < n; i++)
+        if (EventSlot *s = event_lookup(c, evs[i]))
+            if (s->stream >= 0 && s->seq >= best_seq) {
+                best = s->stream;
+                best_seq = s->seq;
+            }
+    if (best >= 0) return best;
+    c->rr = (c->rr + 1) % kLaunchStreams;
+    return c->rr;
+}
+
+void fill_info(zhip_ctx *c) {
+    const hipDeviceProp_t &p = c->prop;
+    zhip_device_info &i = c->info;
+    memset(&i, 0, sizeof i);
+    i.compute_units = (uint32_t)p.multiProcessorCount;
+    i.clock_khz = (uint32_t)p.clockRate;
+    // 4 SIMDs x 16 lanes x 2 (fma) x 2 (dual-issue packed f32) per CU per clock
+    i.compute = (uint64_t)p.multiProcessorCount * 256ull * (uint64_t)p.clockRate * 1000ull;
+    for (int k = 0; k < 3; k++) {
+        i.max_global_work_dims[k] = (uint64_t)p.maxGridSize[k];
+        i.max_local_work_dims[k] = (uint32_t)p.maxThreadsDim[k];
+    }
+    i.max_local_threads = (uint32_t)p.maxThreadsPerBlock;
+    i.preferred_vector_size = 16; // 128-bit global loads/stores
+    i.local_mem_size = (uint64_t)p.sharedMemPerBlock;
+    i.max_register_bytes = 512 * 4; // 512 unified VGPRs per lane
+    i.tensor_cores = 1;
+    i.warp_size = (uint32_t)p.warpSize;
+    for (int d = 0; d < ZHIP_N_DTYPES; d++) i.dtype_capability[d] = 0;
+    i.dtype_capability[ZHIP_F32] = 0xffffffffu;
+    i.has_native_exp2 = 1;
+    i.n_supported_vec_lens = 2;
+    i.supported_vec_lens[0] = 2;
+    i.supported_vec_lens[1] = 4;
+    i.total_bytes = (uint64_t)p.totalGlobalMem;
+    snprintf(i.name, sizeof i.name, "%s", p.name[0] ? p.name : "AMD Instinct (name not reported)");
+    snprintf(i.arch, sizeof i.arch, "%s", p.gcnArchName);
+}
+
+} // namespace
+
+// =================================================================================
+// C ABI
+// =================================================================================
+
+ZHIP_EXPORT const char *zhip_last_error(zhip_ctx *ctx) { return ctx ? ctx->last_error.c_str() : g_init_error.c_str(); }
+
+ZHIP_EXPORT int32_t zhip_device_count(int32_t *count) {
+    if (!count) return ZHIP_DEVICE_ENUMERATION;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        *count = 0;
+        g_init_error = std::string("hipGetDeviceCount failed: ") + hipGetErrorString(e);
+        return ZHIP_DEVICE_ENUMERATION;
+    }
+    *count = n;
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_init(const zhip_config *cfg, zhip_ctx **out) {
+    if (!cfg || !out) {
+        g_init_error = "zhip_init: null argument";
+        return ZHIP_INITIALIZATION;
+    }
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0) {
+        g_init_error = std::string("no HIP device: ") + (e != hipSuccess ? hipGetErrorString(e) : "device count is 0");
+        return ZHIP_DEVICE_ENUMERATION;
+    }
+    if (cfg->device_id < 0 || cfg->device_id >= n) {
+        g_init_error = "device_id " + std::to_string(cfg->device_id) + " out of range, " + std::to_string(n) + " devices";
+        return ZHIP_DEVICE_ENUMERATION;
+    }
+    zhip_ctx *c = new zhip_ctx();
+    c->device = cfg->device_id;
+    c->debug = cfg->debug;
+    c->cache_limit = cfg->cache_bytes ? cfg->cache_bytes : kDefaultCacheBytes;
+    auto bail = [&](int32_t st, const char *what, hipError_t err) {
+        g_init_error = std::string(what) + ": " + hipGetErrorString(err);
+        delete c;
+        return st;
+    };
+    if ((e = hipSetDevice(c->device)) != hipSuccess) return bail(ZHIP_INITIALIZATION, "hipSetDevice", e);
+    if ((e = hipGetDeviceProperties(&c->prop, c->device)) != hipSuccess) return bail(ZHIP_DEVICE_QUERY, "hipGetDeviceProperties", e);
+    if (strncmp(c->prop.gcnArchName, "gfx950", 6) != 0) {
+        g_init_error = std::string("device is ") + c->prop.gcnArchName + ", this backend only carries gfx950 code";
+        delete c;
+        return ZHIP_INITIALIZATION;
+    }
+    size_t free_b = 0, total_b = 0;
+    if ((e = hipMemGetInfo(&free_b, &total_b)) != hipSuccess) return bail(ZHIP_DEVICE_QUERY, "hipMemGetInfo", e);
+    c->free_bytes = (uint64_t)free_b;
+    if ((e = hipStreamCreateWithFlags(&c->pool_stream, hipStreamNonBlocking)) != hipSuccess)
+        return bail(ZHIP_INITIALIZATION, "hipStreamCreate", e);
+    for (int i = 0; i < kLaunchStreams; i++)
+        if ((e = hipStreamCreateWithFlags(&c->launch_streams[i], hipStreamNonBlocking)) != hipSuccess)
+            return bail(ZHIP_INITIALIZATION, "hipStreamCreate", e);
+    if ((e = hipEventCreate(&c->prof_a)) != hipSuccess || (e = hipEventCreate(&c->prof_b)) != hipSuccess)
+        return bail(ZHIP_INITIALIZATION, "hipEventCreate", e);
+    fill_info(c);
+    if (c->debug & 1)
+        fprintf(stderr, "[zyx-hip] device %d: %s (%s), %u CUs, %.1f GiB free\n", c->device, c->info.name, c->info.arch,
+                c->info.compute_units, (double)c->free_bytes / (1 << 30));
+    *out = c;
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_deinit(zhip_ctx *c) {
+    if (!c) return ZHIP_DEINITIALIZATION;
+    {
+        std::lock_guard<std::mutex> lk(c->mu);
+        (void)hipSetDevice(c->device);
+        (void)hipStreamSynchronize(c->pool_stream);
+        for (auto s : c->launch_streams) (void)hipStreamSynchronize(s);
+        trim_cache(c, 0);
+        for (Buffer &b : c->buffers.items)
+            if (b.kind == Buffer::Memory) (void)hipFree(b.ptr);
+        for (EventSlot &s : c->events) (void)hipEventDestroy(s.ev);
+        (void)hipEventDestroy(c->prof_a);
+        (void)hipEventDestroy(c->prof_b);
+        (void)hipStreamDestroy(c->pool_stream);
+        for (auto s : c->launch_streams) (void)hipStreamDestroy(s);
+    }
+    delete c;
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_get_device_info(zhip_ctx *c, zhip_device_info *info) {
+    if (!c || !info) return ZHIP_DEVICE_QUERY;
+    *info = c->info;
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT uint64_t zhip_free_bytes(zhip_ctx *c) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    return c->free_bytes;
+}
+
+ZHIP_EXPORT uint64_t zhip_free_compute(zhip_ctx *c) { return c->info.compute; }
+
+ZHIP_EXPORT int32_t zhip_alloc(zhip_ctx *c, uint64_t bytes, zhip_buf *buf, zhip_event *ev) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!buf || !ev) return c->fail(ZHIP_MEMORY_ALLOCATION, "zhip_alloc: null out pointer");
+    *buf = ZHIP_NULL_ID;
+    *ev = 0;
+    if (bytes > c->free_bytes) return c->fail(ZHIP_MEMORY_ALLOCATION, "Allocation failure");
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_MEMORY_ALLOCATION);
+    uint64_t cap = size_class(bytes ? bytes : 1);
+    Buffer b;
+    b.kind = Buffer::Memory;
+    b.bytes = bytes;
+    b.capacity = cap;
+    auto it = c->cache.find(cap);
+    if (it != c->cache.end()) {
+        CachedBlock blk = std::move(it->second.back());
+        it->second.pop_back();
+        if (it->second.empty()) c->cache.erase(it);
+        c->cached_bytes -= cap;
+        b.ptr = blk.ptr;
+        if (!blk.pending.empty()) {
+            // the previous users' completion becomes the new owner's first dependency
+            int32_t rc = wait_and_consume(c, -1, blk.pending.data(), blk.pending.size(), ZHIP_MEMORY_ALLOCATION);
+            if (rc == ZHIP_OK) rc = event_record(c, -1, ZHIP_MEMORY_ALLOCATION, ev);
+            if (rc != ZHIP_OK) {
+                (void)hipStreamSynchronize(c->pool_stream);
+                *ev = 0;
+            }
+        }
+    } else {
+        hipError_t e = hipMalloc(&b.ptr, cap);
+        if (e != hipSuccess) { // give cached blocks back and retry once
+            (void)hipGetLastError();
+            trim_cache(c, 0);
+            e = hipMalloc(&b.ptr, cap);
+        }
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return c->fail(ZHIP_MEMORY_ALLOCATION, "hipMalloc(%llu) failed: %s", (unsigned long long)cap, hipGetErrorString(e));
+        }
+    }
+    c->free_bytes -= bytes;
+    *buf = c->buffers.push(b);
+    if (c->debug & 64) fprintf(stderr, "[zyx-hip] alloc %llu B -> buffer %u @%p\n", (unsigned long long)bytes, *buf, b.ptr);
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_free(zhip_ctx *c, zhip_buf id, const zhip_event *evs, size_t n) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    Buffer *b = buffer_lookup(c, id);
+    if (!b) return c->fail(ZHIP_MEMORY_DEALLOCATION, "buffer %u does not exist", id);
+    if (b->kind == Buffer::Variable) {
+        for (size_t i = 0; i < n; i++)
+            if (EventSlot *s = event_lookup(c, evs[i])) event_retire(c, s);
+        b->kind = Buffer::Free;
+        c->buffers.remove(id);
+        return ZHIP_OK;
+    }
+    (void)hipSetDevice(c->device);
+    CachedBlock blk{b->ptr, {}};
+    for (size_t i = 0; i < n; i++)
+        if (evs[i] != 0 && event_lookup(c, evs[i])) blk.pending.push_back(evs[i]);
+    c->free_bytes += b->bytes;
+    uint64_t cap = b->capacity;
+    b->kind = Buffer::Free;
+    b->ptr = nullptr;
+    c->buffers.remove(id);
+    c->cache[cap].push_back(std::move(blk));
+    c->cached_bytes += cap;
+    if (c->cached_bytes > c->cache_limit) trim_cache(c, c->cache_limit);
+    if (c->debug & 64) fprintf(stderr, "[zyx-hip] free buffer %u\n", id);
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_store_variable(zhip_ctx *c, int32_t dtype, const uint8_t value[8], zhip_buf *buf) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!buf || !value || dtype_bytes(dtype) == 0) return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "store_variable: bad argument");
+    Buffer b;
+    b.kind = Buffer::Variable;
+    b.var_dtype = dtype;
+    memcpy(b.var_value, value, 8);
+    *buf = c->buffers.push(b);
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_get_variable(zhip_ctx *c, zhip_buf id, int32_t *found, int32_t *dtype, uint8_t value[8]) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!found) return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "get_variable: null out pointer");
+    Buffer *b = buffer_lookup(c, id);
+    *found = (b && b->kind == Buffer::Variable) ? 1 : 0; // None for memory buffers (backend/mod.rs:609-621)
+    if (*found) {
+        if (dtype) *dtype = b->var_dtype;
+        if (value) memcpy(value, b->var_value, 8);
+    }
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_h2d(zhip_ctx *c, const void *src, uint64_t bytes, zhip_buf dst, const zhip_event *evs, size_t n,
+                             zhip_event *ev) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!ev) return c->fail(ZHIP_MEMORY_COPY_H2P, "zhip_h2d: null event out pointer");
+    *ev = 0;
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_MEMORY_COPY_H2P);
+    Buffer *b = buffer_lookup(c, dst);
+    int32_t rc = wait_and_consume(c, -1, evs, n, ZHIP_MEMORY_COPY_H2P);
+    if (rc != ZHIP_OK) return rc;
+    if (!b || b->kind != Buffer::Memory) return c->fail(ZHIP_MEMORY_COPY_H2P, "buffer %u is not device memory", dst);
+    if (bytes > b->bytes)
+        return c->fail(ZHIP_MEMORY_COPY_H2P, "copy of %llu bytes into buffer %u of %llu bytes", (unsigned long long)bytes,
+                       dst, (unsigned long long)b->bytes);
+    if (bytes) HIPCHK(c, hipMemcpyAsync(b->ptr, src, bytes, hipMemcpyHostToDevice, c->pool_stream), ZHIP_MEMORY_COPY_H2P);
+    return event_record(c, -1, ZHIP_MEMORY_COPY_H2P, ev);
+}
+
+ZHIP_EXPORT int32_t zhip_d2h(zhip_ctx *c, zhip_buf src, void *dst, uint64_t bytes, const zhip_event *evs, size_t n) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_MEMORY_COPY_P2H);
+    Buffer *b = buffer_lookup(c, src);
+    int32_t rc = wait_and_consume(c, -1, evs, n, ZHIP_MEMORY_COPY_P2H);
+    if (rc != ZHIP_OK) return rc;
+    if (!b || b->kind != Buffer::Memory) return c->fail(ZHIP_MEMORY_COPY_P2H, "buffer %u is not device memory", src);
+    if (bytes > b->bytes)
+        return c->fail(ZHIP_MEMORY_COPY_P2H, "copy of %llu bytes out of buffer %u of %llu bytes", (unsigned long long)bytes,
+                       src, (unsigned long long)b->bytes);
+    if (bytes) HIPCHK(c, hipMemcpyAsync(dst, b->ptr, bytes, hipMemcpyDeviceToHost, c->pool_stream), ZHIP_MEMORY_COPY_P2H);
+    HIPCHK(c, hipStreamSynchronize(c->pool_stream), ZHIP_MEMORY_COPY_P2H);
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_d2d(zhip_ctx *c, zhip_buf src, zhip_buf dst, uint64_t bytes, const zhip_event *evs, size_t n,
+                             zhip_event *ev) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!ev) return c->fail(ZHIP_MEMORY_COPY_H2P, "zhip_d2d: null event out pointer");
+    *ev = 0;
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_MEMORY_COPY_H2P);
+    Buffer *s = buffer_lookup(c, src), *d = buffer_lookup(c, dst);
+    int32_t rc = wait_and_consume(c, -1, evs, n, ZHIP_MEMORY_COPY_H2P);
+    if (rc != ZHIP_OK) return rc;
+    if (!s || !d || s->kind != Buffer::Memory || d->kind != Buffer::Memory)
+        return c->fail(ZHIP_MEMORY_COPY_H2P, "d2d: buffers %u -> %u are not both device memory", src, dst);
+    if (bytes > s->bytes || bytes > d->bytes) return c->fail(ZHIP_MEMORY_COPY_H2P, "d2d: %llu bytes exceed a buffer", (unsigned long long)bytes);
+    if (bytes) HIPCHK(c, hipMemcpyAsync(d->ptr, s->ptr, bytes, hipMemcpyDeviceToDevice, c->pool_stream), ZHIP_MEMORY_COPY_H2P);
+    return event_record(c, -1, ZHIP_MEMORY_COPY_H2P, ev);
+}
+
+ZHIP_EXPORT int32_t zhip_sync_events(zhip_ctx *c, const zhip_event *evs, size_t n) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    int32_t rc = ZHIP_OK;
+    for (size_t i = 0; i < n; i++) {
+        if (evs[i] == 0) continue;
+        EventSlot *s = event_lookup(c, evs[i]);
+        if (!s) {
+            rc = c->fail(ZHIP_KERNEL_SYNC, "event %zu is not live (stale or already consumed handle)", i);
+            continue;
+        }
+        hipError_t e = hipEventSynchronize(s->ev);
+        if (e != hipSuccess) rc = c->fail(ZHIP_KERNEL_SYNC, "hipEventSynchronize failed: %s", hipGetErrorString(e));
+        event_retire(c, s);
+    }
+    return rc;
+}
+
+ZHIP_EXPORT int32_t zhip_release_events(zhip_ctx *c, const zhip_event *evs, size_t n) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    int32_t rc = ZHIP_OK;
+    for (size_t i = 0; i < n; i++) {
+        if (evs[i] == 0) continue;
+        EventSlot *s = event_lookup(c, evs[i]);
+        if (!s) rc = c->fail(ZHIP_DEINITIALIZATION, "event %zu is not live (stale or already consumed handle)", i);
+        else event_retire(c, s);
+    }
+    return rc;
+}
+
+ZHIP_EXPORT int32_t zhip_buffer_ptr(zhip_ctx *c, zhip_buf id, void **ptr, uint64_t *bytes) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    Buffer *b = buffer_lookup(c, id);
+    if (!b || b->kind != Buffer::Memory) return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "buffer %u is not device memory", id);
+    if (ptr) *ptr = b->ptr;
+    if (bytes) *bytes = b->bytes;
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_register_kernel(zhip_ctx *c, const zhip_kernel_desc *desc, zhip_prog *prog) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!desc || !prog) return c->fail(ZHIP_KERNEL_COMPILATION, "register_kernel: null argument");
+    *prog = ZHIP_NULL_ID;
+    Program p;
+    int32_t rc = program_from_desc(c, *desc, p);
+    if (rc != ZHIP_OK) return rc;
+    p.live = true;
+    *prog = c->programs.push(p);
+    if (c->debug & 128) fprintf(stderr, "[zyx-hip] program %u = kind %d\n", *prog, desc->kind);
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_compile_ir(zhip_ctx *c, const void *, uint64_t, zhip_prog *prog) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (prog) *prog = ZHIP_NULL_ID;
+    return c->fail(ZHIP_KERNEL_COMPILATION,
+                   "HIP device only runs its registered AOT kernels, it does not compile generic kernels.");
+}
+
+ZHIP_EXPORT int32_t zhip_release_program(zhip_ctx *c, zhip_prog prog) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (prog >= c->programs.items.size() || !c->programs.items[prog].live)
+        return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "program %u does not exist", prog);
+    c->programs.items[prog].live = false;
+    c->programs.remove(prog);
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_launch(zhip_ctx *c, zhip_prog prog, const zhip_buf *args, size_t n_args, const zhip_event *evs,
+                                size_t n_evs, zhip_event *ev) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!ev) return c->fail(ZHIP_KERNEL_LAUNCH, "zhip_launch: null event out pointer");
+    *ev = 0;
+    Program *p = nullptr;
+    void *ptr[8] = {nullptr};
+    int32_t rc = resolve_args(c, prog, args, n_args, &p, ptr);
+    if (rc != ZHIP_OK) { // nothing enqueued; the wait list is still consumed so no event leaks
+        (void)hipSetDevice(c->device);
+        for (size_t i = 0; i < n_evs; i++)
+            if (EventSlot *s = event_lookup(c, evs[i])) event_retire(c, s);
+        return rc;
+    }
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
+    int si = pick_stream(c, evs, n_evs);
+    rc = wait_and_consume(c, si, evs, n_evs, ZHIP_KERNEL_LAUNCH);
+    if (rc != ZHIP_OK) return rc;
+    if (c->debug & 32) fprintf(stderr, "[zyx-hip] launch program %u (kind %d) on stream %d\n", prog, p->desc.kind, si);
+    hipError_t e = program_enqueue(*p, ptr, c->launch_streams[si]);
+    if (e != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "launch of program %u failed: %s", prog, hipGetErrorString(e));
+    return event_record(c, si, ZHIP_KERNEL_LAUNCH, ev);
+}
+
+ZHIP_EXPORT int32_t zhip_time_kernel(zhip_ctx *c, zhip_prog prog, const zhip_buf *args, size_t n_args, uint64_t *ns) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!ns) return c->fail(ZHIP_KERNEL_LAUNCH, "zhip_time_kernel: null out pointer");
+    Program *p = nullptr;
+    void *ptr[8] = {nullptr};
+    int32_t rc = resolve_args(c, prog, args, n_args, &p, ptr);
+    if (rc != ZHIP_OK) return rc;
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
+    hipStream_t st = c->launch_streams[0];
+    HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
+    auto t0 = std::chrono::steady_clock::now();
+    hipError_t e = program_enqueue(*p, ptr, st);
+    if (e != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "launch of program %u failed: %s", prog, hipGetErrorString(e));
+    HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
+    *ns = (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t0).count();
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_profile_kernel(zhip_ctx *c, zhip_prog prog, const zhip_buf *args, size_t n_args, size_t arg_sets,
+                                        int32_t iters, float *avg_us) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!avg_us || iters <= 0 || arg_sets == 0 || arg_sets > 64)
+        return c->fail(ZHIP_KERNEL_LAUNCH, "zhip_profile_kernel: bad argument");
+    std::vector<void *> ptrs(arg_sets * 8, nullptr);
+    Program *p = nullptr;
+    for (size_t s = 0; s < arg_sets; s++) {
+        int32_t rc = resolve_args(c, prog, args + s * n_args, n_args, &p, &ptrs[s * 8]);
+        if (rc != ZHIP_OK) return rc;
+    }
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
+    hipStream_t st = c->launch_streams[0];
+    HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
+    HIPCHK(c, hipEventRecord(c->prof_a, st), ZHIP_KERNEL_LAUNCH);
+    for (int32_t i = 0; i < iters; i++) {
+        hipError_t e = program_enqueue(*p, &ptrs[(i % arg_sets) * 8], st);
+        if (e != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "launch of program %u failed: %s", prog, hipGetErrorString(e));
+    }
+    HIPCHK(c, hipEventRecord(c->prof_b, st), ZHIP_KERNEL_LAUNCH);
+    HIPCHK(c, hipEventSynchronize(c->prof_b), ZHIP_KERNEL_SYNC);
+    float ms = 0.0f;
+    HIPCHK(c, hipEventElapsedTime(&ms, c->prof_a, c->prof_b), ZHIP_KERNEL_SYNC);
+    *avg_us = ms * 1000.0f / (float)iters;
+    return ZHIP_OK;
+}
