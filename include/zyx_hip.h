@@ -107,20 +107,68 @@ enum zhip_kernel_kind {
      * selected outputs in the order y, rowsum, arg.
      * zyx/src/tensor/mod.rs:1457-1461, 2245-2269; zyx/src/tensor/reduce_ops.rs:197-199 */
     ZHIP_K_SOFTMAX_ROWS = 1,
+    /* Fused elementwise chain over a [rows, cols] view (dims = {rows, cols}): up to 4
+     * inputs, each a full tensor, a [cols] row vector, a [rows] column vector or one
+     * scalar, combined by a short accumulator program (zhip_ew_op) whose op semantics are
+     * zyx's UOp/BOp tables (zyx/src/kernel/ops.rs:187-261, C meaning
+     * zyx/src/codegen/c.rs:290-304,593-611) plus the Tensor-level composites of
+     * zyx/src/tensor/elementwise.rs. Float dtypes compute in f32 registers and narrow only
+     * on store (bf16 truncates), as the C backend does; I32 computes in int32.
+     *   iparams[0] = n_inputs (1..4), iparams[1] = n_instr (1..18),
+     *   iparams[2+k] = input k: dtype | (zhip_ew_bcast << 8),
+     *   iparams[6+j] = instruction j: op | (src_a << 8) | (src_b << 16),
+     *   fparams[0..8] = constants, flags = 0. `dtype` is the register class (ZHIP_F32 or
+     *   ZHIP_I32), `out_dtype` the stored dtype. args: inputs in order, then the output. */
+    ZHIP_K_ELEMENTWISE = 2,
+    /* Reduce over the last axis (flags = 0: x[rows,cols] -> [rows]) or over axis 0
+     * (flags = 1: -> [cols]); iparams[0] = 0 sum, 1 max. Accumulates in f32 for float
+     * dtypes and i32 for ZHIP_I32, stores as `dtype` (zyx/src/tensor/reduce_ops.rs:45-147,
+     * accumulator init zyx/src/kernel/linearize.rs:920-952). args: x, out. */
+    ZHIP_K_REDUCE = 3,
     ZHIP_K_COUNT_
 };
 #define ZHIP_SOFTMAX_Y 1
 #define ZHIP_SOFTMAX_ROWSUM 2
 #define ZHIP_SOFTMAX_ARGMAX 4
 
+/* Accumulator program of ZHIP_K_ELEMENTWISE. One register `acc`, one saved register `t`.
+ * An operand (src_a / src_b) is: 0..3 = input k (read at that point), ZHIP_EW_SRC_T = t,
+ * ZHIP_EW_SRC_CONST + k = fparams[k] (converted to the register class). */
+enum zhip_ew_op {
+    ZHIP_EW_LOAD = 0, /* acc = a */
+    ZHIP_EW_SAVE,     /* t = acc */
+    /* UOp, acc = op(acc) */
+    ZHIP_EW_NEG, ZHIP_EW_BITNOT, ZHIP_EW_EXP, ZHIP_EW_EXP2, ZHIP_EW_LN, ZHIP_EW_LOG2, ZHIP_EW_RECIPROCAL,
+    ZHIP_EW_SQRT, ZHIP_EW_SIN, ZHIP_EW_COS, ZHIP_EW_FLOOR, ZHIP_EW_TRUNC, ZHIP_EW_ABS,
+    /* BOp, acc = acc op a */
+    ZHIP_EW_ADD, ZHIP_EW_SUB, ZHIP_EW_MUL, ZHIP_EW_DIV, ZHIP_EW_POW, ZHIP_EW_MOD, ZHIP_EW_CMPLT, ZHIP_EW_CMPGT,
+    ZHIP_EW_CMPGE, ZHIP_EW_MAX, ZHIP_EW_OR, ZHIP_EW_AND, ZHIP_EW_BITXOR, ZHIP_EW_BITOR, ZHIP_EW_BITAND,
+    ZHIP_EW_SHL, ZHIP_EW_SHR, ZHIP_EW_NOTEQ, ZHIP_EW_EQ,
+    /* operand first: acc = a op acc */
+    ZHIP_EW_RSUB, ZHIP_EW_RDIV,
+    /* acc = acc != 0 ? a : b   (Tensor::where_ with a true select) */
+    ZHIP_EW_WHERE,
+    /* acc = acc * a + b        (Op::Mad) */
+    ZHIP_EW_MAD,
+    /* Tensor-level composites, zyx/src/tensor/elementwise.rs:168-170,289-293,305-307,457-460,585-588 */
+    ZHIP_EW_RELU, ZHIP_EW_TANH, ZHIP_EW_GELU, ZHIP_EW_SIGMOID, ZHIP_EW_RSQRT,
+    /* Cast to an integer dtype inside a float chain: truncation toward zero (c.rs:243-261) */
+    ZHIP_EW_CAST_INT,
+    ZHIP_EW_OP_COUNT_
+};
+enum zhip_ew_bcast { ZHIP_EW_FULL = 0, ZHIP_EW_ROW = 1, ZHIP_EW_COL = 2, ZHIP_EW_SCALAR = 3 };
+#define ZHIP_EW_SRC_T 0x10
+#define ZHIP_EW_SRC_CONST 0x20
+#define ZHIP_EW_MAX_INSTR 18
+
 typedef struct zhip_kernel_desc {
-    int32_t kind;       /* zhip_kernel_kind */
-    int32_t dtype;      /* element dtype of the main operands */
-    int32_t out_dtype;  /* result dtype where it may differ */
-    int32_t flags;      /* kind specific */
-    int64_t dims[8];    /* kind specific sizes, fixed at registration like cblas m,n,k */
-    float fparams[4];   /* kind specific scalars */
-    int32_t iparams[8]; /* kind specific op codes */
+    int32_t kind;        /* zhip_kernel_kind */
+    int32_t dtype;       /* element dtype of the main operands */
+    int32_t out_dtype;   /* result dtype where it may differ */
+    int32_t flags;       /* kind specific */
+    int64_t dims[8];     /* kind specific sizes, fixed at registration like cblas m,n,k */
+    float fparams[8];    /* kind specific scalars */
+    int32_t iparams[24]; /* kind specific op codes */
 } zhip_kernel_desc;
 
 /* --- backend lifetime ------------------------------------------------------- */

@@ -237,3 +237,18 @@ def bias_act(c: np.ndarray, bias: np.ndarray | None, act: str = "none", bias_dty
     lib().zo_bias_act_f32(_p(c), _p(None if bias is None else np.ascontiguousarray(bias)), bias_dtype, _I64(m), _I64(n),
                           dict(none=0, relu=1, gelu=2)[act])
     return c
+
+
+def ew_chain(chain, arrays) -> np.ndarray:
+    """Evaluate a `zyx_amd.kernels.Chain` on the CPU with the reference's op semantics."""
+    np_store = {F32: np.float32, BF16: np.uint16, F16: np.uint16, I32: np.int32, U8: np.uint8, BOOL: np.uint8}
+    n_in = len(chain.inputs)
+    arrs = [np.ascontiguousarray(a, np_store[int(chain.inputs[k][0])]) for k, a in enumerate(arrays)]
+    in_desc = (C.c_int32 * 4)(*[int(dt) | (bc << 8) for dt, bc in chain.inputs])
+    ptrs = (C.c_void_p * 4)(*[a.ctypes.data for a in arrs])
+    code = (C.c_uint32 * 18)(*chain.code)
+    consts = (C.c_float * 8)(*chain.consts)
+    out = np.empty((chain.rows, chain.cols), np_store[int(chain.out_dtype)])
+    lib().zo_ew_chain(int(chain.reg), int(chain.out_dtype), n_in, in_desc, ptrs, len(chain.code), code, consts, _p(out),
+                      _I64(chain.rows), _I64(chain.cols))
+    return out

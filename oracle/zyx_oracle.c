@@ -455,3 +455,148 @@ ZO_API void zo_bias_act_f32(float *c, const void *bias, int bias_dtype, int64_t 
             c[i * n + j] = v;
         }
 }
+
+/* ------------------------------------------------------------------------- */
+/* Fused elementwise chains                                                   */
+/* ------------------------------------------------------------------------- */
+
+/* Evaluates an accumulator program (the encoding of ZHIP_K_ELEMENTWISE in
+ * include/zyx_hip.h; the encoding is this build's, each op's meaning is the reference's:
+ * UOp/BOp zyx/src/kernel/ops.rs:187-261 as emitted by zyx/src/codegen/c.rs:290-304,
+ * 593-611, composites zyx/src/tensor/elementwise.rs) element by element, the way the C
+ * backend's fused kernel would: float registers, narrowing only on the final store.
+ * in_desc[k] = dtype | bcast << 8 (bcast 0 full, 1 row vector, 2 column vector, 3 scalar). */
+static inline float ew_load(const void *p, int dtype, int64_t i) {
+    switch (dtype) {
+    case ZO_BF16: return bf16_load(((const uint16_t *)p)[i]);
+    case ZO_F16: return f16_load(((const uint16_t *)p)[i]);
+    case ZO_F32: return ((const float *)p)[i];
+    case ZO_I32: return (float)((const int32_t *)p)[i];
+    default: return (float)((const uint8_t *)p)[i];
+    }
+}
+static inline int32_t ew_load_i(const void *p, int dtype, int64_t i) {
+    return dtype == ZO_I32 ? ((const int32_t *)p)[i] : (int32_t)((const uint8_t *)p)[i];
+}
+enum { EW_LOAD = 0, EW_SAVE, EW_NEG, EW_BITNOT, EW_EXP, EW_EXP2, EW_LN, EW_LOG2, EW_RECIPROCAL, EW_SQRT, EW_SIN, EW_COS,
+       EW_FLOOR, EW_TRUNC, EW_ABS, EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_POW, EW_MOD, EW_CMPLT, EW_CMPGT, EW_CMPGE, EW_MAX,
+       EW_OR, EW_AND, EW_BITXOR, EW_BITOR, EW_BITAND, EW_SHL, EW_SHR, EW_NOTEQ, EW_EQ, EW_RSUB, EW_RDIV, EW_WHERE,
+       EW_MAD, EW_RELU, EW_TANH, EW_GELU, EW_SIGMOID, EW_RSQRT, EW_CAST_INT };
+
+static inline float ew_op_f(int op, float x, float a, float b) {
+    switch (op) {
+    case EW_LOAD: return a;
+    case EW_NEG: return zo_unary(ZO_U_NEG, x);
+    case EW_EXP: return zo_unary(ZO_U_EXP, x);
+    case EW_EXP2: return zo_unary(ZO_U_EXP2, x);
+    case EW_LN: return zo_unary(ZO_U_LN, x);
+    case EW_LOG2: return zo_unary(ZO_U_LOG2, x);
+    case EW_RECIPROCAL: return zo_unary(ZO_U_RECIPROCAL, x);
+    case EW_SQRT: return zo_unary(ZO_U_SQRT, x);
+    case EW_SIN: return zo_unary(ZO_U_SIN, x);
+    case EW_COS: return zo_unary(ZO_U_COS, x);
+    case EW_FLOOR: return zo_unary(ZO_U_FLOOR, x);
+    case EW_TRUNC: return zo_unary(ZO_U_TRUNC, x);
+    case EW_ABS: return zo_unary(ZO_U_ABS, x);
+    case EW_ADD: return zo_binary(ZO_B_ADD, x, a);
+    case EW_SUB: return zo_binary(ZO_B_SUB, x, a);
+    case EW_MUL: return zo_binary(ZO_B_MUL, x, a);
+    case EW_DIV: return zo_binary(ZO_B_DIV, x, a);
+    case EW_POW: return zo_binary(ZO_B_POW, x, a);
+    case EW_MOD: return zo_binary(ZO_B_MOD, x, a);
+    case EW_CMPLT: return zo_binary(ZO_B_CMPLT, x, a);
+    case EW_CMPGT: return zo_binary(ZO_B_CMPGT, x, a);
+    case EW_CMPGE: return zo_binary(ZO_B_CMPGE, x, a);
+    case EW_MAX: return zo_binary(ZO_B_MAX, x, a);
+    case EW_OR: return (float)(x != 0.0f || a != 0.0f);
+    case EW_AND: return (float)(x != 0.0f && a != 0.0f);
+    case EW_NOTEQ: return zo_binary(ZO_B_NOTEQ, x, a);
+    case EW_EQ: return zo_binary(ZO_B_EQ, x, a);
+    case EW_RSUB: return zo_binary(ZO_B_SUB, a, x);
+    case EW_RDIV: return zo_binary(ZO_B_DIV, a, x);
+    case EW_WHERE: return x != 0.0f ? a : b;
+    case EW_MAD: return x * a + b;
+    case EW_RELU: return zo_unary(ZO_U_RELU, x);
+    case EW_TANH: return zo_unary(ZO_U_TANH, x);
+    case EW_GELU: return zo_unary(ZO_U_GELU, x);
+    case EW_SIGMOID: return zo_unary(ZO_U_SIGMOID, x);
+    case EW_RSQRT: return zo_unary(ZO_U_RSQRT, x);
+    case EW_CAST_INT: return truncf(x);
+    default: return x;
+    }
+}
+static inline int32_t ew_op_i(int op, int32_t x, int32_t a, int32_t b) {
+    uint32_t ux = (uint32_t)x, ua = (uint32_t)a;
+    switch (op) {
+    case EW_LOAD: return a;
+    case EW_NEG: return (int32_t)(0u - ux);
+    case EW_BITNOT: return ~x;
+    case EW_ABS: return x < 0 ? (int32_t)(0u - ux) : x;
+    case EW_ADD: return (int32_t)(ux + ua);
+    case EW_SUB: return (int32_t)(ux - ua);
+    case EW_MUL: return (int32_t)(ux * ua);
+    case EW_DIV: return a == 0 ? 0 : (a == -1 ? (int32_t)(0u - ux) : x / a);
+    case EW_MOD: return (a == 0 || a == -1) ? 0 : x % a;
+    case EW_CMPLT: return x < a;
+    case EW_CMPGT: return x > a;
+    case EW_CMPGE: return x >= a;
+    case EW_MAX: return x > a ? x : a;
+    case EW_OR: return x || a;
+    case EW_AND: return x && a;
+    case EW_BITXOR: return x ^ a;
+    case EW_BITOR: return x | a;
+    case EW_BITAND: return x & a;
+    case EW_SHL: return (int32_t)(ux << (a & 31));
+    case EW_SHR: return x >> (a & 31);
+    case EW_NOTEQ: return x != a;
+    case EW_EQ: return x == a;
+    case EW_RSUB: return (int32_t)(ua - ux);
+    case EW_RDIV: return x == 0 ? 0 : (x == -1 ? (int32_t)(0u - ua) : a / x);
+    case EW_WHERE: return x != 0 ? a : b;
+    case EW_MAD: return (int32_t)(ux * ua + (uint32_t)b);
+    case EW_RELU: return x > 0 ? x : 0;
+    default: return x;
+    }
+}
+
+ZO_API void zo_ew_chain(int reg_class, int out_dtype, int n_in, const int32_t *in_desc, const void *const *in,
+                        int n_instr, const uint32_t *code, const float *consts, void *out, int64_t rows, int64_t cols) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t c = 0; c < cols; c++) {
+            int64_t i = r * cols + c;
+            float fa = 0, ft = 0;
+            int32_t ia = 0, it = 0;
+            for (int j = 0; j < n_instr; j++) {
+                int op = code[j] & 0xff, s[2] = {(int)((code[j] >> 8) & 0xff), (int)((code[j] >> 16) & 0xff)};
+                if (op == EW_SAVE) { ft = fa; it = ia; continue; }
+                float fv[2] = {0, 0};
+                int32_t iv[2] = {0, 0};
+                for (int q = 0; q < 2; q++) {
+                    int src = s[q];
+                    if (src < 4) {
+                        if (src >= n_in) continue;
+                        int dt = in_desc[src] & 0xff, bc = (in_desc[src] >> 8) & 0xff;
+                        int64_t idx = bc == 0 ? i : bc == 1 ? c : bc == 2 ? r : 0;
+                        if (reg_class == ZO_I32) iv[q] = ew_load_i(in[src], dt, idx);
+                        else fv[q] = ew_load(in[src], dt, idx);
+                    } else if (src == 0x10) { fv[q] = ft; iv[q] = it; }
+                    else if (src >= 0x20 && src < 0x28) { fv[q] = consts[src - 0x20]; iv[q] = (int32_t)consts[src - 0x20]; }
+                }
+                if (reg_class == ZO_I32) ia = ew_op_i(op, ia, iv[0], iv[1]);
+                else fa = ew_op_f(op, fa, fv[0], fv[1]);
+            }
+            if (reg_class == ZO_I32) {
+                if (out_dtype == ZO_I32) ((int32_t *)out)[i] = ia;
+                else ((uint8_t *)out)[i] = (uint8_t)ia;
+            } else {
+                switch (out_dtype) {
+                case ZO_BF16: ((uint16_t *)out)[i] = bf16_store(fa); break;
+                case ZO_F16: ((uint16_t *)out)[i] = f16_store(fa); break;
+                case ZO_F32: ((float *)out)[i] = fa; break;
+                case ZO_I32: ((int32_t *)out)[i] = (int32_t)fa; break; /* C cast: toward zero */
+                default: ((uint8_t *)out)[i] = (uint8_t)(int32_t)fa; break;
+                }
+            }
+        }
+}

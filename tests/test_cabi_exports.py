@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_struct_layouts_match_header():
-    assert ctypes.sizeof(backend.KernelDesc) == 4 * 4 + 8 * 8 + 4 * 4 + 8 * 4
+    assert ctypes.sizeof(backend.KernelDesc) == 4 * 4 + 8 * 8 + 8 * 4 + 24 * 4
     assert ctypes.sizeof(backend._Config) == 16
 
 

@@ -1,0 +1,70 @@
+"""Row / column sum and max on the GPU vs the CPU oracle; integer cases replay the
+reference's closed-form tests (zyx/tests/04_reduce.rs:7-175) bit-exactly.
+
+Float tolerance: the GPU folds in a tree, the reference serially; both are compared with
+the f64 sum at 1e-5 of sum(|x|) (the bound both orders satisfy), and max is exact.
+"""
+import numpy as np
+import pytest
+
+from zyx_amd import DType
+from zyx_amd.kernels import reduce
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(1, 1), (3, 5), (8, 4096), (1, 131072), (1, 1 << 22), (4096, 512), (100, 1000), (513, 257), (70000, 12),
+          (2, 100003), (64, 128), (64, 10), (8192, 4096)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("axis0", [False, True])
+def test_float_sum_max(hip, oracle, shape, axis0):
+    dev, pool = hip
+    x = oracle.Rng(shape[0] * 7 + shape[1]).randn(shape, 2.0)
+    xd = x.astype(np.float64)
+    ax = 0 if axis0 else 1
+    got = reduce(dev, pool, x, "sum", axis0)
+    want = xd.sum(ax)
+    bound = 1e-5 * np.abs(xd).sum(ax) + 1e-30
+    assert np.all(np.abs(got - want) <= bound), np.max(np.abs(got - want) / bound)
+    ref = (oracle.reduce_cols if axis0 else oracle.reduce_rows)("sum", x)
+    assert np.all(np.abs(ref - want) <= bound * 4)  # the serial reference order obeys the same kind of bound
+    assert np.array_equal(reduce(dev, pool, x, "max", axis0), x.max(ax))
+
+
+def test_reference_int_goldens(hip, oracle):
+    dev, pool = hip
+    assert reduce(dev, pool, np.ones((8, 4096), np.int32), "sum", False, DType.I32).tolist() == [4096] * 8
+    assert reduce(dev, pool, np.ones((1, 131072), np.int32), "sum", False, DType.I32).tolist() == [131072]
+    x = (np.arange(4 * 1024 * 512) % 10).astype(np.int32).reshape(4 * 1024, 512)
+    for axis0 in (False, True):
+        assert np.array_equal(reduce(dev, pool, x, "sum", axis0, DType.I32), x.sum(0 if axis0 else 1))
+        assert np.array_equal(reduce(dev, pool, x, "max", axis0, DType.I32), x.max(0 if axis0 else 1))
+    rng = np.random.default_rng(1)
+    big = rng.integers(-2**31, 2**31, size=(300, 999), dtype=np.int64).astype(np.int32)
+    assert np.array_equal(reduce(dev, pool, big, "sum", False, DType.I32), oracle.reduce_rows_i32("sum", big))  # wraps
+    assert np.array_equal(reduce(dev, pool, big, "max", True, DType.I32), big.max(0))
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16])
+def test_16bit_inputs_accumulate_in_f32(hip, oracle, dt):
+    dev, pool = hip
+    conv = oracle.f32_to_bf16 if dt == DType.BF16 else oracle.f32_to_f16
+    back = oracle.bf16_to_f32 if dt == DType.BF16 else oracle.f16_to_f32
+    code = oracle.BF16 if dt == DType.BF16 else oracle.F16
+    x = conv(oracle.Rng(5).randn((96, 2048)))
+    for axis0 in (False, True):
+        got = back(reduce(dev, pool, x, "sum", axis0, dt))
+        ref = back((oracle.reduce_cols if axis0 else oracle.reduce_rows)("sum", x, code))
+        # both truncate an f32 sum to 16 bits: results agree to one unit in the last 16-bit place
+        ulp = 2.0 ** (np.floor(np.log2(np.abs(ref) + 1e-30)) - (7 if dt == DType.BF16 else 10))
+        assert np.all(np.abs(got - ref) <= ulp + 1e-6)
+        assert np.array_equal(reduce(dev, pool, x, "max", axis0, dt),
+                              (oracle.reduce_cols if axis0 else oracle.reduce_rows)("max", x, code))
+
+
+def test_empty_axes(hip):
+    dev, pool = hip
+    assert reduce(dev, pool, np.zeros((4, 0), np.float32), "sum").tolist() == [0.0] * 4
+    assert reduce(dev, pool, np.zeros((0, 4), np.float32), "sum").shape == (0,)
+    assert np.all(reduce(dev, pool, np.zeros((4, 0), np.float32), "max") == np.float32(-3.4028235e38))

@@ -86,7 +86,7 @@ class _DeviceInfo(C.Structure):
 class KernelDesc(C.Structure):
     """zhip_kernel_desc"""
     _fields_ = [("kind", C.c_int32), ("dtype", C.c_int32), ("out_dtype", C.c_int32), ("flags", C.c_int32),
-                ("dims", C.c_int64 * 8), ("fparams", C.c_float * 4), ("iparams", C.c_int32 * 8)]
+                ("dims", C.c_int64 * 8), ("fparams", C.c_float * 8), ("iparams", C.c_int32 * 24)]
 
 
 @dataclass

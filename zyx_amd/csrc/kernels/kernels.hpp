@@ -16,4 +16,33 @@ struct SoftmaxRows {
 };
 hipError_t softmax_rows(const SoftmaxRows &p, hipStream_t stream);
 
+// Accumulator program over a [rows, cols] view; see zhip_ew_op in include/zyx_hip.h.
+struct Elementwise {
+    int64_t rows, cols;
+    int n_in, n_instr;
+    int reg_class;    // DT_F32 or DT_I32
+    int need_rowcol;  // some input is a row / column vector
+    int in_dtype[4], in_bcast[4];
+    int out_dtype;
+    uint32_t code[18];
+    float consts[8];
+    const void *in[4];
+    void *out;
+};
+hipError_t elementwise(const Elementwise &p, hipStream_t stream);
+
+// Sum / max over the last axis (axis0 == 0) or over axis 0 (axis0 == 1) of x[rows, cols].
+struct Reduce {
+    int64_t rows, cols;
+    int dtype;   // storage dtype of x and out: F32, BF16, F16 (f32 accumulate) or I32
+    int op;      // 0 sum, 1 max
+    int axis0;
+    const void *x;
+    void *out;
+    void *workspace;           // partial results of the two-stage variants
+    uint64_t workspace_bytes;
+};
+uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int axis0);
+hipError_t reduce(const Reduce &p, hipStream_t stream);
+
 } // namespace zk

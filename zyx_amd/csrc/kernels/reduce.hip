@@ -1,0 +1,305 @@
+// Row (last-axis) and column (axis-0) sum / max reductions.
+//
+// Semantics: zyx/src/tensor/reduce_ops.rs:45-147 -- floats accumulate in f32 and are cast
+// back to the input dtype on store, ints accumulate in i32; the accumulator starts at 0
+// for sum and at the dtype's lowest finite value for max (zyx/src/kernel/linearize.rs:
+// 920-952, zyx/src/dtype.rs:207-224). The reference folds serially; here each lane folds
+// a strided slice with 128-bit loads and lanes are combined by DPP wave reductions (rows)
+// or an LDS transpose-free fold over the four waves of a workgroup (columns). Long
+// single rows / tall thin matrices are split over several workgroups whose partials a
+// second, tiny launch folds.
+#include "dtypes.hpp"
+#include "kernels.hpp"
+#include "wave.hpp"
+
+namespace zk {
+
+namespace {
+
+template <int OP, typename A> struct Fold;
+template <> struct Fold<0, float> {
+    static __device__ __forceinline__ float init() { return 0.0f; }
+    static __device__ __forceinline__ float f(float a, float b) { return a + b; }
+};
+template <> struct Fold<1, float> {
+    static __device__ __forceinline__ float init() { return -FLT_MAX; }
+    static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); }
+};
+template <> struct Fold<0, int> {
+    static __device__ __forceinline__ int init() { return 0; }
+    static __device__ __forceinline__ int f(int a, int b) { return (int)((unsigned)a + (unsigned)b); }
+};
+template <> struct Fold<1, int> {
+    static __device__ __forceinline__ int init() { return INT32_MIN; }
+    static __device__ __forceinline__ int f(int a, int b) { return a > b ? a : b; }
+};
+
+// element access by dtype class: DT 0 = f32, 1 = bf16, 2 = f16, 3 = i32
+template <int DT> struct Elem;
+template <> struct Elem<0> {
+    typedef float S; typedef float A;
+    static __device__ __forceinline__ float ld(const float *p, int64_t i) { return p[i]; }
+    static __device__ __forceinline__ void ld4(const float *p, int64_t i, float (&v)[4]) {
+        f32x4 t = *(const f32x4 *)(p + i);
+        v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+    }
+    static __device__ __forceinline__ void st(float *p, int64_t i, float v) { p[i] = v; }
+};
+template <> struct Elem<1> {
+    typedef uint16_t S; typedef float A;
+    static __device__ __forceinline__ float ld(const uint16_t *p, int64_t i) { return bf16_to_f32(p[i]); }
+    static __device__ __forceinline__ void ld4(const uint16_t *p, int64_t i, float (&v)[4]) {
+        uint2 t = *(const uint2 *)(p + i);
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void st(uint16_t *p, int64_t i, float v) { p[i] = f32_to_bf16_trunc(v); }
+};
+template <> struct Elem<2> {
+    typedef uint16_t S; typedef float A;
+    static __device__ __forceinline__ float ld(const uint16_t *p, int64_t i) { return f16_to_f32(p[i]); }
+    static __device__ __forceinline__ void ld4(const uint16_t *p, int64_t i, float (&v)[4]) {
+        uint2 t = *(const uint2 *)(p + i);
+        v[0] = f16_to_f32((uint16_t)t.x); v[1] = f16_to_f32((uint16_t)(t.x >> 16));
+        v[2] = f16_to_f32((uint16_t)t.y); v[3] = f16_to_f32((uint16_t)(t.y >> 16));
+    }
+    static __device__ __forceinline__ void st(uint16_t *p, int64_t i, float v) { p[i] = f32_to_f16_trunc(v); }
+};
+template <> struct Elem<3> {
+    typedef int32_t S; typedef int A;
+    static __device__ __forceinline__ int ld(const int32_t *p, int64_t i) { return p[i]; }
+    static __device__ __forceinline__ void ld4(const int32_t *p, int64_t i, int (&v)[4]) {
+        i32x4 t = *(const i32x4 *)(p + i);
+        v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+    }
+    static __device__ __forceinline__ void st(int32_t *p, int64_t i, int v) { p[i] = v; }
+};
+
+template <int OP> __device__ __forceinline__ float wave_fold(float v) {
+    if (OP == 0) return wave_allreduce_f32(v, OpAdd());
+    return wave_allreduce_f32(v, OpMaxF());
+}
+template <int OP> __device__ __forceinline__ int wave_fold(int v) {
+    if (OP == 0) return wave_allreduce_i32(v, OpAdd());
+    return wave_allreduce_i32(v, OpMaxI());
+}
+
+// One wave folds columns [c0, c1) of one row. VEC: row start and c0 are 4-element aligned.
+template <int DT, int OP, bool VEC>
+__device__ __forceinline__ typename Elem<DT>::A fold_row_span(const typename Elem<DT>::S *__restrict__ xr, int64_t c0,
+                                                              int64_t c1, int lane, int nlanes) {
+    typedef typename Elem<DT>::A A;
+    typedef Fold<OP, A> F;
+    A acc = F::init();
+    if (VEC) {
+        int64_t nv = (c1 - c0) >> 2;
+        for (int64_t i = lane; i < nv; i += nlanes) {
+            A v[4];
+            Elem<DT>::ld4(xr, c0 + i * 4, v);
+            acc = F::f(acc, F::f(F::f(v[0], v[1]), F::f(v[2], v[3])));
+        }
+        for (int64_t c = c0 + nv * 4 + lane; c < c1; c += nlanes) acc = F::f(acc, Elem<DT>::ld(xr, c));
+    } else {
+        for (int64_t c = c0 + lane; c < c1; c += nlanes) acc = F::f(acc, Elem<DT>::ld(xr, c));
+    }
+    return acc;
+}
+
+// rows: one wave per (row, segment); 4 waves per workgroup. With segs == 1 the result is
+// stored as DT, otherwise the raw accumulator goes to partial[row * segs + seg].
+template <int DT, int OP, bool VEC>
+__global__ __launch_bounds__(256) void reduce_rows_wave_k(const typename Elem<DT>::S *__restrict__ x,
+                                                          typename Elem<DT>::S *__restrict__ out,
+                                                          typename Elem<DT>::A *__restrict__ partial, int64_t rows,
+                                                          int64_t cols, int segs, int64_t seg_len) {
+    const int lane = threadIdx.x & 63;
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= rows * segs) return; // whole wave; no cross-wave synchronisation below
+    const int64_t row = item / segs;
+    const int seg = (int)(item - row * segs);
+    const int64_t c0 = seg * seg_len, c1 = min(cols, c0 + seg_len);
+    typename Elem<DT>::A acc = fold_row_span<DT, OP, VEC>(x + row * cols, c0, c1, lane, 64);
+    acc = wave_fold<OP>(acc);
+    if (lane == 0) {
+        if (segs == 1) Elem<DT>::st(out, row, acc);
+        else partial[item] = acc;
+    }
+}
+
+// second stage: fold `segs` raw partials per row (accumulator type), store as DT.
+template <int DT, int OP>
+__global__ __launch_bounds__(256) void reduce_partials_k(const typename Elem<DT>::A *__restrict__ partial,
+                                                         typename Elem<DT>::S *__restrict__ out, int64_t rows, int segs) {
+    typedef typename Elem<DT>::A A;
+    typedef Fold<OP, A> F;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    A acc = F::init();
+    for (int s = lane; s < segs; s += 64) acc = F::f(acc, partial[row * segs + s]);
+    acc = wave_fold<OP>(acc);
+    if (lane == 0) Elem<DT>::st(out, row, acc);
+}
+
+// columns: a workgroup owns a strip of 256 columns (lane -> 4 adjacent columns when VEC,
+// else thread -> 1 column of a 64-wide strip per wave... kept simple: VEC strips are 256
+// wide, scalar strips 64 wide) and a chunk of rows split over its 4 waves.
+template <int DT, int OP, bool VEC>
+__global__ __launch_bounds__(256) void reduce_cols_k(const typename Elem<DT>::S *__restrict__ x,
+                                                     typename Elem<DT>::S *__restrict__ out,
+                                                     typename Elem<DT>::A *__restrict__ partial, int64_t rows,
+                                                     int64_t cols, int chunks, int64_t chunk_len) {
+    typedef typename Elem<DT>::A A;
+    typedef Fold<OP, A> F;
+    constexpr int W = VEC ? 4 : 1;
+    __shared__ A lds[4][64 * W];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t c = ((int64_t)blockIdx.x * 64 + lane) * W;
+    const int chunk = blockIdx.y;
+    const int64_t r0 = chunk * chunk_len, r1 = min(rows, r0 + chunk_len);
+    A acc[W];
+#pragma unroll
+    for (int k = 0; k < W; k++) acc[k] = F::init();
+    if (c < cols) {
+        for (int64_t r = r0 + wave; r < r1; r += 4) {
+            if (VEC) {
+                A v[4];
+                Elem<DT>::ld4(x, r * cols + c, v);
+#pragma unroll
+                for (int k = 0; k < W; k++) acc[k] = F::f(acc[k], v[k]);
+            } else {
+                acc[0] = F::f(acc[0], Elem<DT>::ld(x, r * cols + c));
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < W; k++) lds[wave][lane * W + k] = acc[k];
+    __syncthreads(); // every thread of the workgroup arrives: no early exit above
+    if (wave == 0 && c < cols) {
+#pragma unroll
+        for (int k = 0; k < W; k++) {
+            A v = F::f(F::f(lds[0][lane * W + k], lds[1][lane * W + k]), F::f(lds[2][lane * W + k], lds[3][lane * W + k]));
+            if (chunks == 1) Elem<DT>::st(out, c + k, v);
+            else partial[(int64_t)chunk * cols + c + k] = v;
+        }
+    }
+}
+// second stage for columns: partial[chunks, cols] (accumulator type) -> out[cols]
+template <int DT, int OP>
+__global__ __launch_bounds__(256) void reduce_col_partials_k(const typename Elem<DT>::A *__restrict__ partial,
+                                                             typename Elem<DT>::S *__restrict__ out, int64_t cols,
+                                                             int chunks) {
+    typedef typename Elem<DT>::A A;
+    typedef Fold<OP, A> F;
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= cols) return;
+    A acc = F::init();
+    for (int k = 0; k < chunks; k++) acc = F::f(acc, partial[(int64_t)k * cols + c]);
+    Elem<DT>::st(out, c, acc);
+}
+
+struct RowPlan { int segs; int64_t seg_len; };
+RowPlan plan_rows(int64_t rows, int64_t cols) {
+    // enough waves to fill 256 CUs (~8 per CU) when there are few long rows
+    int segs = 1;
+    if (rows < 2048 && cols >= 8192) {
+        int64_t want = (2048 + rows - 1) / rows;
+        int64_t max_by_len = cols / 4096; // a segment keeps >= 4096 elements
+        segs = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, max_by_len), 1024));
+    }
+    int64_t seg_len = (cols + segs - 1) / segs;
+    seg_len = (seg_len + 3) / 4 * 4; // keep segment starts 4-aligned
+    segs = (int)((cols + seg_len - 1) / seg_len);
+    return {segs, seg_len};
+}
+struct ColPlan { int chunks; int64_t chunk_len; };
+ColPlan plan_cols(int64_t rows, int64_t cols, bool vec) {
+    int64_t strips = (cols + (vec ? 255 : 63)) / (vec ? 256 : 64);
+    int chunks = 1;
+    if (strips < 1024 && rows >= 256) {
+        int64_t want = (1024 + strips - 1) / strips;
+        chunks = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, rows / 64), 4096));
+    }
+    int64_t chunk_len = (rows + chunks - 1) / chunks;
+    chunks = (int)((rows + chunk_len - 1) / chunk_len);
+    return {chunks, chunk_len};
+}
+
+template <int DT, int OP> hipError_t launch(const Reduce &p, hipStream_t st) {
+    typedef typename Elem<DT>::S S;
+    typedef typename Elem<DT>::A A;
+    const S *x = (const S *)p.x;
+    S *out = (S *)p.out;
+    A *ws = (A *)p.workspace;
+    const int esz = (int)sizeof(S);
+    if (!p.axis0) {
+        bool vec = (p.cols * esz) % (4 * esz) == 0 && p.cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+        RowPlan pl = plan_rows(p.rows, p.cols);
+        if (pl.segs > 1 && (uint64_t)p.rows * pl.segs * sizeof(A) > p.workspace_bytes) return hipErrorInvalidValue;
+        int64_t items = p.rows * pl.segs;
+        dim3 grid((unsigned)((items + 3) / 4)), block(256);
+        if (vec) hipLaunchKernelGGL((reduce_rows_wave_k<DT, OP, true>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.segs, pl.seg_len);
+        else hipLaunchKernelGGL((reduce_rows_wave_k<DT, OP, false>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.segs, pl.seg_len);
+        if (pl.segs > 1)
+            hipLaunchKernelGGL((reduce_partials_k<DT, OP>), dim3((unsigned)((p.rows + 3) / 4)), block, 0, st, ws, out, p.rows, pl.segs);
+    } else {
+        bool vec = p.cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+        ColPlan pl = plan_cols(p.rows, p.cols, vec);
+        if (pl.chunks > 1 && (uint64_t)pl.chunks * p.cols * sizeof(A) > p.workspace_bytes) return hipErrorInvalidValue;
+        int64_t strips = (p.cols + (vec ? 255 : 63)) / (vec ? 256 : 64);
+        dim3 grid((unsigned)strips, (unsigned)pl.chunks), block(256);
+        if (vec) hipLaunchKernelGGL((reduce_cols_k<DT, OP, true>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len);
+        else hipLaunchKernelGGL((reduce_cols_k<DT, OP, false>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len);
+        if (pl.chunks > 1)
+            hipLaunchKernelGGL((reduce_col_partials_k<DT, OP>), dim3((unsigned)((p.cols + 255) / 256)), block, 0, st, ws, out, p.cols, pl.chunks);
+    }
+    return hipGetLastError();
+}
+
+} // namespace
+
+uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int axis0) {
+    if (rows <= 0 || cols <= 0) return 0;
+    if (!axis0) {
+        RowPlan pl = plan_rows(rows, cols);
+        return pl.segs > 1 ? (uint64_t)rows * pl.segs * 4 : 0;
+    }
+    // the vectorised plan never needs more chunks than the scalar one for the same shape
+    ColPlan a = plan_cols(rows, cols, true), b = plan_cols(rows, cols, false);
+    int chunks = std::max(a.chunks, b.chunks);
+    return chunks > 1 ? (uint64_t)chunks * cols * 4 : 0;
+}
+
+hipError_t reduce(const Reduce &p, hipStream_t st) {
+    if (p.rows < 0 || p.cols < 0) return hipErrorInvalidValue;
+    int64_t n_out = p.axis0 ? p.cols : p.rows;
+    if (n_out == 0) return hipSuccess;
+    if ((p.axis0 ? p.rows : p.cols) == 0) {
+        // reducing an empty axis leaves the accumulator's initial value; one tiny fill via
+        // the partials kernel with zero segments
+        switch (p.dtype * 2 + p.op) {
+#define ZK_EMPTY(DTC, DT, OP)                                                                                        \
+    case DTC * 2 + OP:                                                                                                \
+        hipLaunchKernelGGL((reduce_partials_k<DT, OP>), dim3((unsigned)((n_out + 3) / 4)), dim3(256), 0, st,          \
+                           (const typename Elem<DT>::A *)nullptr, (typename Elem<DT>::S *)p.out, n_out, 0);           \
+        return hipGetLastError();
+            ZK_EMPTY(DT_F32, 0, 0) ZK_EMPTY(DT_F32, 0, 1) ZK_EMPTY(DT_BF16, 1, 0) ZK_EMPTY(DT_BF16, 1, 1)
+            ZK_EMPTY(DT_F16, 2, 0) ZK_EMPTY(DT_F16, 2, 1) ZK_EMPTY(DT_I32, 3, 0) ZK_EMPTY(DT_I32, 3, 1)
+#undef ZK_EMPTY
+        default: return hipErrorInvalidValue;
+        }
+    }
+    switch (p.dtype * 2 + p.op) {
+    case DT_F32 * 2 + 0: return launch<0, 0>(p, st);
+    case DT_F32 * 2 + 1: return launch<0, 1>(p, st);
+    case DT_BF16 * 2 + 0: return launch<1, 0>(p, st);
+    case DT_BF16 * 2 + 1: return launch<1, 1>(p, st);
+    case DT_F16 * 2 + 0: return launch<2, 0>(p, st);
+    case DT_F16 * 2 + 1: return launch<2, 1>(p, st);
+    case DT_I32 * 2 + 0: return launch<3, 0>(p, st);
+    case DT_I32 * 2 + 1: return launch<3, 1>(p, st);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+} // namespace zk

@@ -65,6 +65,8 @@ struct Program {
     zhip_kernel_desc desc{};
     int n_in = 0, n_out = 0;
     uint64_t need[8] = {0}; // minimum bytes per argument
+    void *workspace = nullptr; // device scratch owned by the program (two-stage reductions)
+    uint64_t workspace_bytes = 0;
 };
 
 template <class T> struct Slab { // dense ids, lowest free id reused (zyx/src/slab.rs)
@@ -255,6 +257,65 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.n_out = o - 1;
         return ZHIP_OK;
     }
+    case ZHIP_K_ELEMENTWISE: {
+        int64_t rows = d.dims[0], cols = d.dims[1];
+        int n_in = d.iparams[0], n_instr = d.iparams[1];
+        if (rows < 0 || cols < 0 || (cols && rows > (1ll << 40) / cols))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: rows/cols out of range");
+        if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_I32)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: register class must be F32 or I32");
+        if (n_in < 1 || n_in > 4 || n_instr < 1 || n_instr > ZHIP_EW_MAX_INSTR)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: %d inputs / %d instructions not supported", n_in, n_instr);
+        const bool ireg = d.dtype == ZHIP_I32;
+        auto dtype_ok = [&](int dt, bool out) {
+            if (ireg) return dt == ZHIP_I32 || dt == ZHIP_U8 || dt == ZHIP_BOOL;
+            (void)out;
+            return dt == ZHIP_F32 || dt == ZHIP_BF16 || dt == ZHIP_F16 || dt == ZHIP_I32 || dt == ZHIP_U8 || dt == ZHIP_BOOL;
+        };
+        for (int k = 0; k < n_in; k++) {
+            int dt = d.iparams[2 + k] & 0xff, bc = (d.iparams[2 + k] >> 8) & 0xff;
+            if (!dtype_ok(dt, false) || bc > ZHIP_EW_SCALAR)
+                return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: input %d has unsupported dtype %d / broadcast %d", k, dt, bc);
+            uint64_t elems = bc == ZHIP_EW_FULL ? (uint64_t)rows * cols : bc == ZHIP_EW_ROW ? (uint64_t)cols
+                             : bc == ZHIP_EW_COL ? (uint64_t)rows : 1;
+            p.need[k] = elems * dtype_bytes(dt);
+        }
+        if (!dtype_ok(d.out_dtype, true)) return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: unsupported output dtype %d", d.out_dtype);
+        auto src_ok = [&](int s) { return s < n_in || s == ZHIP_EW_SRC_T || (s >= ZHIP_EW_SRC_CONST && s < ZHIP_EW_SRC_CONST + 8); };
+        for (int j = 0; j < n_instr; j++) {
+            uint32_t ins = (uint32_t)d.iparams[6 + j];
+            int op = ins & 0xff, sa = (ins >> 8) & 0xff, sb = (ins >> 16) & 0xff;
+            if (op >= ZHIP_EW_OP_COUNT_) return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: instruction %d: unknown op %d", j, op);
+            bool unary = (op >= ZHIP_EW_NEG && op <= ZHIP_EW_ABS) || op >= ZHIP_EW_RELU || op == ZHIP_EW_SAVE;
+            if (!unary && !src_ok(sa)) return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: instruction %d: bad operand %d", j, sa);
+            if ((op == ZHIP_EW_WHERE || op == ZHIP_EW_MAD) && !src_ok(sb))
+                return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: instruction %d: bad second operand %d", j, sb);
+            bool float_only = (op >= ZHIP_EW_EXP && op <= ZHIP_EW_TRUNC) || op == ZHIP_EW_POW || op == ZHIP_EW_TANH ||
+                              op == ZHIP_EW_GELU || op == ZHIP_EW_SIGMOID || op == ZHIP_EW_RSQRT || op == ZHIP_EW_CAST_INT;
+            bool int_only = op == ZHIP_EW_BITNOT || (op >= ZHIP_EW_BITXOR && op <= ZHIP_EW_SHR);
+            if ((ireg && float_only) || (!ireg && int_only))
+                return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: instruction %d: op %d not defined for this register class", j, op);
+            if (j == 0 && op != ZHIP_EW_LOAD) return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: program must start with LOAD");
+        }
+        p.n_in = n_in;
+        p.n_out = 1;
+        p.need[n_in] = (uint64_t)rows * cols * dtype_bytes(d.out_dtype);
+        return ZHIP_OK;
+    }
+    case ZHIP_K_REDUCE: {
+        int64_t rows = d.dims[0], cols = d.dims[1];
+        if (rows < 0 || cols < 0 || (cols && rows > (1ll << 40) / cols))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "reduce: rows/cols out of range");
+        if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16 && d.dtype != ZHIP_F16 && d.dtype != ZHIP_I32)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "reduce: dtype %d not implemented", d.dtype);
+        if ((d.flags & ~1) || (d.iparams[0] != 0 && d.iparams[0] != 1)) return c->fail(ZHIP_KERNEL_COMPILATION, "reduce: bad flags/op");
+        p.n_in = 1;
+        p.n_out = 1;
+        p.need[0] = (uint64_t)rows * cols * dtype_bytes(d.dtype);
+        p.need[1] = (uint64_t)((d.flags & 1) ? cols : rows) * dtype_bytes(d.dtype);
+        p.workspace_bytes = zk::reduce_workspace_bytes(rows, cols, d.flags & 1);
+        return ZHIP_OK;
+    }
     default: return c->fail(ZHIP_KERNEL_COMPILATION, "unknown kernel kind %d", d.kind);
     }
 }
@@ -272,6 +333,38 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         if (d.flags & ZHIP_SOFTMAX_ROWSUM) a.rowsum = (float *)ptr[o++];
         if (d.flags & ZHIP_SOFTMAX_ARGMAX) a.arg = (int32_t *)ptr[o++];
         return zk::softmax_rows(a, st);
+    }
+    case ZHIP_K_ELEMENTWISE: {
+        zk::Elementwise a{};
+        a.rows = d.dims[0];
+        a.cols = d.dims[1];
+        a.n_in = d.iparams[0];
+        a.n_instr = d.iparams[1];
+        a.reg_class = d.dtype;
+        a.out_dtype = d.out_dtype;
+        for (int k = 0; k < a.n_in; k++) {
+            a.in_dtype[k] = d.iparams[2 + k] & 0xff;
+            a.in_bcast[k] = (d.iparams[2 + k] >> 8) & 0xff;
+            if (a.in_bcast[k] == ZHIP_EW_ROW || a.in_bcast[k] == ZHIP_EW_COL) a.need_rowcol = 1;
+            a.in[k] = ptr[k];
+        }
+        for (int j = 0; j < a.n_instr; j++) a.code[j] = (uint32_t)d.iparams[6 + j];
+        for (int k = 0; k < 8; k++) a.consts[k] = d.fparams[k];
+        a.out = ptr[a.n_in];
+        return zk::elementwise(a, st);
+    }
+    case ZHIP_K_REDUCE: {
+        zk::Reduce a{};
+        a.rows = d.dims[0];
+        a.cols = d.dims[1];
+        a.dtype = d.dtype;
+        a.op = d.iparams[0];
+        a.axis0 = d.flags & 1;
+        a.x = ptr[0];
+        a.out = ptr[1];
+        a.workspace = p.workspace;
+        a.workspace_bytes = p.workspace_bytes;
+        return zk::reduce(a, st);
     }
     default: return hipErrorInvalidValue;
     }
@@ -429,6 +522,8 @@ ZHIP_EXPORT int32_t zhip_deinit(zhip_ctx *c) {
         trim_cache(c, 0);
         for (Buffer &b : c->buffers.items)
             if (b.kind == Buffer::Memory) (void)hipFree(b.ptr);
+        for (Program &p : c->programs.items)
+            if (p.live && p.workspace) (void)hipFree(p.workspace);
         for (EventSlot &s : c->events) (void)hipEventDestroy(s.ev);
         (void)hipEventDestroy(c->prof_a);
         (void)hipEventDestroy(c->prof_b);
@@ -641,6 +736,10 @@ ZHIP_EXPORT int32_t zhip_register_kernel(zhip_ctx *c, const zhip_kernel_desc *de
     Program p;
     int32_t rc = program_from_desc(c, *desc, p);
     if (rc != ZHIP_OK) return rc;
+    if (p.workspace_bytes) {
+        HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_COMPILATION);
+        HIPCHK(c, hipMalloc(&p.workspace, p.workspace_bytes), ZHIP_KERNEL_COMPILATION);
+    }
     p.live = true;
     *prog = c->programs.push(p);
     if (c->debug & 128) fprintf(stderr, "[zyx-hip] program %u = kind %d\n", *prog, desc->kind);
@@ -658,7 +757,13 @@ ZHIP_EXPORT int32_t zhip_release_program(zhip_ctx *c, zhip_prog prog) {
     std::lock_guard<std::mutex> lk(c->mu);
     if (prog >= c->programs.items.size() || !c->programs.items[prog].live)
         return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "program %u does not exist", prog);
-    c->programs.items[prog].live = false;
+    Program &p = c->programs.items[prog];
+    if (p.workspace) { // hipFree waits for the device, so no launch still uses it
+        (void)hipSetDevice(c->device);
+        (void)hipFree(p.workspace);
+        p.workspace = nullptr;
+    }
+    p.live = false;
     c->programs.remove(prog);
     return ZHIP_OK;
 }

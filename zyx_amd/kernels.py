@@ -64,3 +64,120 @@ def softmax_rows(dev: HIPDevice, pool: HIPMemoryPool, x: np.ndarray, y=True, row
         pool.deallocate(b, [])
     dev.release(prog)
     return tuple(res)
+
+
+# ---- fused elementwise chains (ZHIP_K_ELEMENTWISE) ------------------------------------------
+K_ELEMENTWISE = 2
+K_REDUCE = 3
+
+EW_OPS = ["load", "save", "neg", "bitnot", "exp", "exp2", "ln", "log2", "reciprocal", "sqrt", "sin", "cos", "floor",
+          "trunc", "abs", "add", "sub", "mul", "div", "pow", "mod", "cmplt", "cmpgt", "cmpge", "max", "or", "and",
+          "bitxor", "bitor", "bitand", "shl", "shr", "noteq", "eq", "rsub", "rdiv", "where", "mad", "relu", "tanh",
+          "gelu", "sigmoid", "rsqrt", "cast_int"]
+EW_OP = {name: i for i, name in enumerate(EW_OPS)}
+EW_FULL, EW_ROW, EW_COL, EW_SCALAR = 0, 1, 2, 3
+EW_T = 0x10
+EW_CONST = 0x20
+
+
+class Chain:
+    """Builder of an accumulator program: `acc` is threaded through the ops, `t` is one saved
+    value. Operands are input indices (from `input()`), `Chain.T`, or constants (`const()`).
+
+        c = Chain(rows, cols)                      # gelu(x + bias)
+        x, b = c.input(DType.F32), c.input(DType.F32, EW_ROW)
+        c.load(x).add(b).gelu()
+    """
+    T = EW_T
+
+    def __init__(self, rows: int, cols: int, reg: DType = DType.F32, out_dtype: DType = DType.F32):
+        self.rows, self.cols, self.reg, self.out_dtype = rows, cols, DType(reg), DType(out_dtype)
+        self.inputs, self.code, self.consts = [], [], []
+
+    def input(self, dtype: DType = DType.F32, bcast: int = EW_FULL) -> int:
+        self.inputs.append((DType(dtype), bcast))
+        return len(self.inputs) - 1
+
+    def const(self, value: float) -> int:
+        value = float(np.float32(value))
+        if value not in self.consts:
+            self.consts.append(value)
+        return EW_CONST + self.consts.index(value)
+
+    def op(self, name: str, a: int = 0, b: int = 0) -> "Chain":
+        self.code.append(EW_OP[name] | (a << 8) | (b << 16))
+        return self
+
+    def __getattr__(self, name):
+        if name in EW_OP:
+            return lambda a=0, b=0: self.op(name, a, b)
+        raise AttributeError(name)
+
+    def input_elems(self, k: int) -> int:
+        bc = self.inputs[k][1]
+        return {EW_FULL: self.rows * self.cols, EW_ROW: self.cols, EW_COL: self.rows, EW_SCALAR: 1}[bc]
+
+    def desc(self) -> KernelDesc:
+        d = KernelDesc()
+        d.kind, d.dtype, d.out_dtype = K_ELEMENTWISE, self.reg, self.out_dtype
+        d.dims[0], d.dims[1] = self.rows, self.cols
+        d.iparams[0], d.iparams[1] = len(self.inputs), len(self.code)
+        for k, (dt, bc) in enumerate(self.inputs):
+            d.iparams[2 + k] = int(dt) | (bc << 8)
+        for j, ins in enumerate(self.code):
+            d.iparams[6 + j] = ins
+        for k, v in enumerate(self.consts):
+            d.fparams[k] = v
+        return d
+
+
+_NP_STORE = {DType.F32: np.float32, DType.BF16: np.uint16, DType.F16: np.uint16, DType.I32: np.int32,
+             DType.U8: np.uint8, DType.Bool: np.uint8}
+
+
+def run_chain(dev: HIPDevice, pool: HIPMemoryPool, chain: Chain, arrays) -> np.ndarray:
+    """Upload the inputs, launch the chain, read the [rows, cols] result back."""
+    prog = dev.register_kernel(chain.desc())
+    bufs, waits = [], []
+    keep = []
+    for k, a in enumerate(arrays):
+        a = np.ascontiguousarray(a, _NP_STORE[chain.inputs[k][0]])
+        assert a.size == chain.input_elems(k)
+        keep.append(a)
+        b, e = to_device(pool, a)
+        bufs.append(b)
+        waits.append(e)
+    out_np = _NP_STORE[chain.out_dtype]
+    ob, e = alloc_like(pool, chain.rows * chain.cols, np.dtype(out_np).itemsize)
+    waits.append(e)
+    done = dev.launch(prog, pool, bufs + [ob], waits)
+    res = to_host(pool, ob, (chain.rows, chain.cols), out_np, [done])
+    for b in bufs + [ob]:
+        pool.deallocate(b, [])
+    dev.release(prog)
+    return res
+
+
+def reduce_desc(rows: int, cols: int, op: str = "sum", axis0: bool = False, dtype: DType = DType.F32) -> KernelDesc:
+    d = KernelDesc()
+    d.kind, d.dtype, d.out_dtype = K_REDUCE, DType(dtype), DType(dtype)
+    d.flags = 1 if axis0 else 0
+    d.dims[0], d.dims[1] = rows, cols
+    d.iparams[0] = {"sum": 0, "max": 1}[op]
+    return d
+
+
+def reduce(dev: HIPDevice, pool: HIPMemoryPool, x: np.ndarray, op: str = "sum", axis0: bool = False,
+           dtype: DType = DType.F32) -> np.ndarray:
+    x = np.ascontiguousarray(x, _NP_STORE[DType(dtype)])
+    rows, cols = x.shape
+    prog = dev.register_kernel(reduce_desc(rows, cols, op, axis0, dtype))
+    xb, e0 = to_device(pool, x)
+    n_out = cols if axis0 else rows
+    ob, e1 = alloc_like(pool, n_out, x.itemsize)
+    done = dev.launch(prog, pool, [xb, ob], [e0, e1])
+    res = to_host(pool, ob, (n_out,), x.dtype, [done])
+    pool.deallocate(xb, [])
+    pool.deallocate(ob, [])
+    dev.release(prog)
+    return res
