@@ -125,11 +125,22 @@ enum zhip_kernel_kind {
      * dtypes and i32 for ZHIP_I32, stores as `dtype` (zyx/src/tensor/reduce_ops.rs:45-147,
      * accumulator init zyx/src/kernel/linearize.rs:920-952). args: x, out. */
     ZHIP_K_REDUCE = 3,
+    /* C[M,N] = op(A) . op(B) (+ bias[N]) (then ReLU / GELU): Tensor::dot / dot_dtype
+     * (zyx/src/tensor/mod.rs:1469-1518) and Linear::forward (zyx-nn/src/linear.rs:38-44),
+     * the pattern Graph::match_matmul recognises (zyx/src/vendor/matmul.rs:43-71).
+     * dims = {M, N, K}; dtype = operand dtype; out_dtype = dtype of C; flags bit 0: A is
+     * stored [K,M], bit 1: B is stored [N,K] (a Linear weight [out,in]);
+     * iparams[0] = epilogue: 0 none, 1 + bias, 2 + bias then ReLU, 3 + bias then GELU;
+     * iparams[1] = dtype of bias. Products and sums are f32 for float operands.
+     * args: A, B, (bias when iparams[0] != 0), then C. */
+    ZHIP_K_GEMM = 4,
     ZHIP_K_COUNT_
 };
 #define ZHIP_SOFTMAX_Y 1
 #define ZHIP_SOFTMAX_ROWSUM 2
 #define ZHIP_SOFTMAX_ARGMAX 4
+#define ZHIP_GEMM_TRANS_A 1
+#define ZHIP_GEMM_TRANS_B 2
 
 /* Accumulator program of ZHIP_K_ELEMENTWISE. One register `acc`, one saved register `t`.
  * An operand (src_a / src_b) is: 0..3 = input k (read at that point), ZHIP_EW_SRC_T = t,

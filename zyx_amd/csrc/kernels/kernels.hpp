@@ -45,4 +45,17 @@ struct Reduce {
 uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int axis0);
 hipError_t reduce(const Reduce &p, hipStream_t stream);
 
+// C[M,N] (f32) = op(A) . op(B) (+ bias[N], + activation), bf16 operands, f32 accumulate.
+// trans_a: A is stored [K,M]; trans_b: B is stored [N,K] (a Linear weight [out,in]).
+struct GemmBf16 {
+    int64_t M, N, K;
+    int trans_a, trans_b;
+    int epilogue;      // 0 none, 1 bias, 2 bias+relu, 3 bias+gelu
+    int bias_dtype;    // DT_BF16 or DT_F32
+    const void *A, *B, *bias;
+    void *C;
+};
+bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K);
+hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t stream);
+
 } // namespace zk

@@ -316,6 +316,27 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.workspace_bytes = zk::reduce_workspace_bytes(rows, cols, d.flags & 1);
         return ZHIP_OK;
     }
+    case ZHIP_K_GEMM: {
+        int64_t M = d.dims[0], N = d.dims[1], K = d.dims[2];
+        int epi = d.iparams[0];
+        if (M <= 0 || N <= 0 || K <= 0) return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: M, N, K must be positive");
+        if (epi < 0 || epi > 3 || (d.flags & ~3)) return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: bad epilogue/flags");
+        if (d.dtype == ZHIP_BF16 && d.out_dtype == ZHIP_F32 && zk::gemm_bf16_supported(M, N, K)) {
+            if (epi && d.iparams[1] != ZHIP_BF16 && d.iparams[1] != ZHIP_F32)
+                return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: bias must be bf16 or f32");
+        } else {
+            return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: no kernel for dtype %d -> %d with M=%lld N=%lld K=%lld", d.dtype,
+                           d.out_dtype, (long long)M, (long long)N, (long long)K);
+        }
+        int a = 0;
+        p.need[a++] = (uint64_t)M * K * dtype_bytes(d.dtype);
+        p.need[a++] = (uint64_t)K * N * dtype_bytes(d.dtype);
+        if (epi) p.need[a++] = (uint64_t)N * dtype_bytes(d.iparams[1]);
+        p.n_in = a;
+        p.need[a] = (uint64_t)M * N * dtype_bytes(d.out_dtype);
+        p.n_out = 1;
+        return ZHIP_OK;
+    }
     default: return c->fail(ZHIP_KERNEL_COMPILATION, "unknown kernel kind %d", d.kind);
     }
 }
@@ -365,6 +386,21 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         a.workspace = p.workspace;
         a.workspace_bytes = p.workspace_bytes;
         return zk::reduce(a, st);
+    }
+    case ZHIP_K_GEMM: {
+        zk::GemmBf16 a{};
+        a.M = d.dims[0];
+        a.N = d.dims[1];
+        a.K = d.dims[2];
+        a.trans_a = d.flags & ZHIP_GEMM_TRANS_A ? 1 : 0;
+        a.trans_b = d.flags & ZHIP_GEMM_TRANS_B ? 1 : 0;
+        a.epilogue = d.iparams[0];
+        a.bias_dtype = d.iparams[1];
+        a.A = ptr[0];
+        a.B = ptr[1];
+        a.bias = a.epilogue ? ptr[2] : nullptr;
+        a.C = ptr[p.n_in];
+        return zk::gemm_bf16(a, st);
     }
     default: return hipErrorInvalidValue;
     }
