@@ -6,18 +6,21 @@
 // exactly, products and sums are f32 (zyx/src/codegen/c.rs:491-496, 615-629).
 //
 // Shape of the kernel
-//   * workgroup tile 256 x 256, K step 64, 4 waves in a 2 x 2 grid, each wave owns a
-//     128 x 128 block of C = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulator registers;
-//   * operands go HBM/L2 -> LDS with 16-byte direct-to-LDS loads (no VGPR staging),
-//     two LDS stages of 64 KiB, the loads of K step t+1 are in flight while step t is
-//     multiplied;
-//   * LDS rows are XOR-swizzled at 16-byte granularity. Direct-to-LDS writes lane l of
-//     a wave at base + 16*l, so the swizzle is applied on the global side: each lane
-//     fetches the chunk that belongs in its LDS slot;
-//   * K-contiguous operands (A[M,K], B stored [N,K]) are read back with ds_read_b128;
-//     an operand stored with its M/N index contiguous (B[K,N]) is read with the
-//     transposing ds_read_b64_tr_b16, which hands each lane four consecutive k of one
-//     column;
+//   * workgroup tile 256 x 256, K step 64, 4 waves in a 2 x 2 grid (one per SIMD), each
+//     wave owns a 128 x 128 block of C = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulator
+//     registers (the AGPR half of the register file);
+//   * operands go L2 -> VGPR -> LDS: every thread keeps one K tile (16 x 16 bytes) in
+//     flight in registers; a chunk is written to LDS one tile time after its load was
+//     issued and its registers are immediately reused for the load of the tile after.
+//     Measured beside an MFMA stream on this part, a 1 KiB direct-to-LDS load costs the
+//     matrix pipe ~42 cycles, a register-staged load + ds_write_b128 pair ~16;
+//   * two LDS stages of 64 KiB; rows are XOR-swizzled at 16-byte granularity so that both
+//     the ds_write_b128 of the staging path and the fragment reads are conflict-free;
+//   * K-contiguous operands (A[M,K], B stored [N,K]) are read back with ds_read_b128; an
+//     operand stored with its M/N index contiguous (B[K,N]) is read with the transposing
+//     ds_read_b64_tr_b16, which hands each lane four consecutive k of one column;
+//   * per k step (16 MFMAs) a wave issues 8 fragment reads for the next step, 4 LDS
+//     writes and 4 global loads, slotted between the MFMAs;
 //   * workgroups are numbered so that the 32 that share an XCD (ids congruent mod 8)
 //     cover a compact 4 x 8 patch of tiles and re-use each other's panels in that
 //     XCD's L2.
@@ -41,54 +44,67 @@ constexpr int B_STAGE = BN * BK * 2;           // 32 KiB
 constexpr int STAGE = A_STAGE + B_STAGE;       // 64 KiB
 constexpr int GEMM_LDS = 2 * STAGE;            // 128 KiB
 
-__device__ __forceinline__ void g2lds16(const void *g, ZK_LDS void *l) {
-    __builtin_amdgcn_global_load_lds((const ZK_GLOBAL void *)g, l, 16, 0, 0);
-}
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-// K-contiguous operand tile: R = 256 rows x 64 k, LDS layout [row][chunk ^ (row & 7)],
-// 128-byte rows. One wave-load fills 8 rows; 8 loads per thread.
-__device__ __forceinline__ void load_tile_kc(const uint16_t *__restrict__ g, int64_t ld, int row0, int k0,
-                                             ZK_LDS uint8_t *lds, int wave, int lane) {
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int rbase = i * 32 + wave * 8;
-        const int row = rbase + (lane >> 3);
-        const int c = (lane & 7) ^ (row & 7);
-        g2lds16(g + (int64_t)(row0 + row) * ld + k0 + c * 8, lds + rbase * 128);
+// K-contiguous operand tile: 256 rows x 64 k, LDS layout [row][chunk ^ key(row)], 128-byte
+// rows, key(row) = (row >> 1) & 7: a 128-bit LDS access is served 16 lanes at a time over
+// 64 banks (256 bytes), and 16 consecutive rows at one logical chunk occupy 16 different
+// 16-byte slots modulo 256 bytes. Thread (wave w, lane l) moves, for i = 0..7, the chunk
+// that belongs at row i*32 + w*8 + l/8, physical slot l%8.
+__device__ __forceinline__ int swz_kc(int row) { return (row >> 1) & 7; }
+struct TileKC {
+    static __device__ __forceinline__ const uint16_t *src(const uint16_t *g, int64_t ld, int row0, int k0, int i, int wave,
+                                                         int lane) {
+        const int row = i * 32 + wave * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ swz_kc(row);
+        return g + (int64_t)(row0 + row) * ld + k0 + c * 8;
     }
-}
+    static constexpr __host__ __device__ __forceinline__ int dst(int i, int wave, int lane) { return (i * 32 + wave * 8) * 128 + lane * 16; }
+    static __device__ __forceinline__ int64_t k_advance(int64_t) { return BK; }
+};
 // MN-contiguous operand tile: 64 k rows x 256 columns, LDS layout [k][chunk ^ swz(k)],
-// 512-byte rows, swz(k) = (k & 3) << 1. One wave-load fills 2 k rows.
+// 512-byte rows, swz(k) = (k & 3) << 1. Thread (w, l) moves, for i = 0..7, the chunk at
+// k row i*8 + w*2 + l/32, physical slot l%32.
 __device__ __forceinline__ int swz_mn(int k) { return (k & 3) << 1; }
-__device__ __forceinline__ void load_tile_mn(const uint16_t *__restrict__ g, int64_t ld, int col0, int k0,
-                                             ZK_LDS uint8_t *lds, int wave, int lane) {
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int kbase = i * 8 + wave * 2;
-        const int k = kbase + (lane >> 5);
+struct TileMN {
+    static __device__ __forceinline__ const uint16_t *src(const uint16_t *g, int64_t ld, int col0, int k0, int i, int wave,
+                                                         int lane) {
+        const int k = i * 8 + wave * 2 + (lane >> 5);
         const int c = (lane & 31) ^ swz_mn(k);
-        g2lds16(g + (int64_t)(k0 + k) * ld + col0 + c * 8, lds + kbase * 512);
+        return g + (int64_t)(k0 + k) * ld + col0 + c * 8;
     }
-}
+    static constexpr __host__ __device__ __forceinline__ int dst(int i, int wave, int lane) { return (i * 8 + wave * 2) * 512 + lane * 16; }
+    static __device__ __forceinline__ int64_t k_advance(int64_t ld) { return BK * ld; }
+};
 
-// Fragment of a K-contiguous tile for MFMA 32x32x16: lane -> row (lane & 31),
-// k = ks*16 + (lane >> 5)*8 .. +7.
-__device__ __forceinline__ bf16x8 frag_kc(const ZK_LDS uint8_t *lds, int row, int ks, int lane) {
-    const int c = (ks * 2 + (lane >> 5)) ^ (row & 7);
-    return *(const ZK_LDS bf16x8 *)(lds + row * 128 + c * 16);
+// Fragment addressing. Everything that depends on the lane is folded into a few byte
+// offsets computed once before the K loop; stage, 32-row block and k step then only add
+// compile-time constants, which the LDS instructions take as immediate offsets.
+//
+// K-contiguous tile, MFMA 32x32x16 operand: lane -> row (lane & 31), k = ks*16 +
+// (lane >> 5)*8 .. +7, i.e. logical chunk ks*2 + (lane >> 5) at physical slot chunk ^ key.
+// key(row) is unchanged by adding multiples of 16 rows, so one offset per k step serves
+// every 32-row block: kc_off[ks] + block * 32 * 128.
+__device__ __forceinline__ int frag_kc_off(int row, int ks, int lane) {
+    return row * 128 + (((ks * 2 + (lane >> 5)) ^ swz_kc(row)) << 4);
 }
-// Same fragment out of an MN-contiguous tile through two transposing reads. In every
-// group of 16 lanes, lane r points at 4 consecutive columns of k row (r >> 2); the
-// hardware returns to lane i the column i of those 4 k rows.
-__device__ __forceinline__ bf16x8 frag_mn(const ZK_LDS uint8_t *lds, int col_base, int ks, int lane) {
+__device__ __forceinline__ bf16x8 frag_kc(const ZK_LDS uint8_t *lds, int off) {
+    return *(const ZK_LDS bf16x8 *)(lds + off);
+}
+// MN-contiguous tile through two transposing reads. In every group of 16 lanes, lane r
+// points at 4 consecutive columns of k row (r >> 2); the hardware returns to lane i the
+// column i of those 4 k rows. swz(k) only depends on k & 3 = (lane & 15) >> 2, so one
+// offset per 32-column block serves all k steps and both halves: mn_off[block] +
+// ks*16*512 (+ 4*512).
+__device__ __forceinline__ int frag_mn_off(int col_base, int lane) {
     const int g16 = lane >> 4, r = lane & 15;
     const int col = col_base + (g16 & 1) * 16 + (r & 3) * 4;
-    const int kk = ks * 16 + (g16 >> 1) * 8 + (r >> 2);
-    const int k0 = kk, k1 = kk + 4;
-    const ZK_LDS uint8_t *p0 = lds + k0 * 512 + (((col >> 3) ^ swz_mn(k0)) << 4) + (col & 4) * 2;
-    const ZK_LDS uint8_t *p1 = lds + k1 * 512 + (((col >> 3) ^ swz_mn(k1)) << 4) + (col & 4) * 2;
-    bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)p0);
-    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)p1);
+    const int k = (g16 >> 1) * 8 + (r >> 2);
+    return k * 512 + (((col >> 3) ^ swz_mn(k)) << 4) + (col & 4) * 2;
+}
+__device__ __forceinline__ bf16x8 frag_mn(const ZK_LDS uint8_t *lds, int off) {
+    bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(lds + off));
+    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(lds + off + 4 * 512));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
@@ -140,45 +156,132 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    auto issue_loads = [&](int kt, int stage) {
-        ZK_LDS uint8_t *sa = smem + stage * STAGE, *sb = sa + A_STAGE;
-        if (AT) load_tile_mn(A, M, m0, kt * BK, sa, wave, lane);
-        else load_tile_kc(A, K, m0, kt * BK, sa, wave, lane);
-        if (BT) load_tile_kc(B, K, n0, kt * BK, sb, wave, lane);
-        else load_tile_mn(B, N, n0, kt * BK, sb, wave, lane);
+    // Staging registers: ra[i] / rb[i] hold chunk i of the tile that is written to LDS
+    // during the current K tile and re-loaded (two tiles ahead) right after the write.
+    // Global addresses are a wave-uniform byte pointer that advances with the K tile plus a
+    // per-thread 32-bit offset fixed for the whole kernel; LDS addresses are one per-thread
+    // offset plus constants.
+    typedef typename std::conditional<AT, TileMN, TileKC>::type TA;
+    typedef typename std::conditional<BT, TileKC, TileMN>::type TB;
+    const int64_t lda = AT ? M : K, ldb = BT ? K : N;
+    uint32_t oa[8], ob[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        oa[i] = (uint32_t)((TA::src(A, lda, m0, 0, i, wave, lane) - A) * 2);
+        ob[i] = (uint32_t)((TB::src(B, ldb, n0, 0, i, wave, lane) - B) * 2);
+    }
+    const int da0 = TA::dst(0, wave, lane), db0 = A_STAGE + TB::dst(0, wave, lane);
+    constexpr int da_step = TA::dst(1, 0, 0) - TA::dst(0, 0, 0), db_step = TB::dst(1, 0, 0) - TB::dst(0, 0, 0);
+    const int64_t adv_a = TA::k_advance(lda) * 2, adv_b = TB::k_advance(ldb) * 2;
+    u32x4 ra[8], rb[8];
+    // staging unit u = 0..15: operand A (u even) or B (u odd), chunk u >> 1
+    auto gload = [&](int u, int kt) {
+        const int i = u >> 1;
+        if (u & 1) rb[i] = *(const u32x4 *)((const uint8_t *)B + kt * adv_b + ob[i]);
+        else ra[i] = *(const u32x4 *)((const uint8_t *)A + kt * adv_a + oa[i]);
     };
+    auto lwrite = [&](int u, int da_base, int db_base) {
+        const int i = u >> 1;
+        if (u & 1) *(ZK_LDS u32x4 *)(smem + db_base + i * db_step) = rb[i];
+        else *(ZK_LDS u32x4 *)(smem + da_base + i * da_step) = ra[i];
+    };
+    int fa_off[4], fb_off[4]; // per k step (K-contiguous) or per 32-wide block (MN-contiguous)
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        fa_off[q] = AT ? frag_mn_off(wm * 128 + q * 32, lane) : frag_kc_off(wm * 128 + (lane & 31), q, lane);
+        fb_off[q] = A_STAGE + (BT ? frag_kc_off(wn * 128 + (lane & 31), q, lane) : frag_mn_off(wn * 128 + q * 32, lane));
+    }
 
     const int KT = K / BK;
-    issue_loads(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0070); // vmcnt(0): the direct-to-LDS loads have landed
+#pragma unroll
+    for (int u = 0; u < 16; u++) gload(u, 0);
+#pragma unroll
+    for (int u = 0; u < 16; u++) {
+        lwrite(u, da0, db0);
+        gload(u, min(1, KT - 1));
+    }
     __syncthreads();
 
-    for (int kt = 0; kt < KT; kt++) {
-        const int stage = kt & 1;
-        if (kt + 1 < KT) issue_loads(kt + 1, stage ^ 1);
-        const ZK_LDS uint8_t *sa = smem + stage * STAGE, *sb = sa + A_STAGE;
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ks++) {
-            bf16x8 af[4], bfr[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                if (AT) af[i] = frag_mn(sa, wm * 128 + i * 32, ks, lane);
-                else af[i] = frag_kc(sa, wm * 128 + i * 32 + (lane & 31), ks, lane);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if (BT) bfr[j] = frag_kc(sb, wn * 128 + j * 32 + (lane & 31), ks, lane);
-                else bfr[j] = frag_mn(sb, wn * 128 + j * 32, ks, lane);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    // Fragments are double-buffered in registers: while the 16 MFMAs of k step s run, the
+    // 8 LDS reads of step s+1 are in flight. The step after the last one of a tile lives
+    // in the other stage, so the hand-over barrier sits before the last step's MFMAs.
+    bf16x8 af[2][4], bfr[2][4];
+    // fragment r = 0..3: A block r; r = 4..7: B block r - 4. fa/fb are the four per-lane
+    // offsets of each operand with the stage folded in.
+    auto load_frag = [&](const int (&fa)[4], const int (&fb)[4], int ks, int buf, int r) {
+        if (r < 4) {
+            if (AT) af[buf][r] = frag_mn(smem, fa[r] + ks * 16 * 512);
+            else af[buf][r] = frag_kc(smem, fa[ks] + r * 32 * 128);
+        } else {
+            const int j = r - 4;
+            if (BT) bfr[buf][j] = frag_kc(smem, fb[ks] + j * 32 * 128);
+            else bfr[buf][j] = frag_mn(smem, fb[j] + ks * 16 * 512);
         }
-        __builtin_amdgcn_s_waitcnt(0x0070);
-        __syncthreads(); // next stage is complete and everyone is done reading this one
+    };
+#pragma unroll
+    for (int r = 0; r < 8; r++) load_frag(fa_off, fb_off, 0, 0, r);
+
+    // One K tile = 4 k steps of 16 MFMAs. During tile c (stage c & 1) each step writes two
+    // staged chunk pairs of tile c+1 into the other stage and re-issues their loads for
+    // tile c+2. The body is branch-free so that it stays one basic block (the compiler's
+    // wait-count bookkeeping is exact only inside a block): tiles 0..KT-2 all hand over
+    // (loads past the end re-fetch the final tile and are never written), the final tile
+    // is peeled off below.
+    // Address registers of the tile being multiplied (c*) and of the other stage (n*) are
+    // formed once per tile: 18 adds, everything else in the loop is an immediate offset.
+    int cfa[4], cfb[4], nfa[4], nfb[4], nda, ndb;
+    auto set_stage = [&](int cur_off, int nxt_off) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            cfa[q] = fa_off[q] + cur_off;
+            cfb[q] = fb_off[q] + cur_off;
+            nfa[q] = fa_off[q] + nxt_off;
+            nfb[q] = fb_off[q] + nxt_off;
+        }
+        nda = da0 + nxt_off;
+        ndb = db0 + nxt_off;
+    };
+    // The instruction order of a k step is pinned by hand (a scheduling fence after every
+    // MFMA and every group of memory operations). Measured on an MFMA stream, a
+    // ds_write_b128 holds up the next MFMA of its SIMD for about the time its 1 KiB takes
+    // to leave the register file; writing a staged chunk and immediately re-issuing the
+    // load into its registers in one gap, and giving the neighbouring gaps one cheap
+    // fragment read each, costs the least. Steps 0 and 1 move 6 staging units, step 2 the
+    // last 4, step 3 only holds the hand-over barrier (after 4 MFMAs, so that the matrix
+    // pipe has work queued while the waves meet) and the first reads of the next tile.
+    auto k_step = [&](const int ks, int kt, const bool handover) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+        const bool last = ks == BK / 16 - 1;
+        const int u0 = ks * 6, nu = ks < 2 ? 6 : (ks == 2 ? 4 : 0);
+#pragma unroll
+        for (int m = 0; m < 16; m++) {
+            __builtin_amdgcn_sched_barrier(0);
+            acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][m >> 2], bfr[cur][m & 3], acc[m >> 2][m & 3], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (!last) {
+                if ((m & 1) == 0 && handover && (m >> 1) < nu) {
+                    lwrite(u0 + (m >> 1), nda, ndb);
+                    gload(u0 + (m >> 1), min(kt + 2, KT - 1));
+                }
+                if (m & 1) load_frag(cfa, cfb, ks + 1, nxt, m >> 1);
+            } else if (handover) {
+                if (m == 3) __syncthreads(); // tile kt+1 is complete in LDS; nobody reads this stage any more
+                if (m >= 3 && m < 11) load_frag(nfa, nfb, 0, nxt, m - 3);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    int cur_off = 0;
+    for (int kt = 0; kt < KT - 1; kt++) {
+        set_stage(cur_off, cur_off ^ STAGE);
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ks++) k_step(ks, kt, true);
+        cur_off ^= STAGE;
     }
+    set_stage(cur_off, cur_off ^ STAGE);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) k_step(ks, KT - 1, false);
+    __builtin_amdgcn_sched_barrier(0);
 
     // C tile of a 32x32 MFMA: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.
     const int col_in = lane & 31, row_in = (lane >> 5) * 4;
