@@ -128,10 +128,14 @@ enum zhip_kernel_kind {
     /* C[M,N] = op(A) . op(B) (+ bias[N]) (then ReLU / GELU): Tensor::dot / dot_dtype
      * (zyx/src/tensor/mod.rs:1469-1518) and Linear::forward (zyx-nn/src/linear.rs:38-44),
      * the pattern Graph::match_matmul recognises (zyx/src/vendor/matmul.rs:43-71).
-     * dims = {M, N, K}; dtype = operand dtype; out_dtype = dtype of C; flags bit 0: A is
-     * stored [K,M], bit 1: B is stored [N,K] (a Linear weight [out,in]);
+     * dims = {M, N, K, batch (0 = 1)}: `batch` independent dense products laid out back to
+     * back; dtype = operand dtype (F32, BF16, F16); out_dtype = dtype of C (F32 or dtype,
+     * narrowing stores truncate); flags bit 0: A is stored [K,M], bit 1: B is stored [N,K]
+     * (a Linear weight [out,in]);
      * iparams[0] = epilogue: 0 none, 1 + bias, 2 + bias then ReLU, 3 + bias then GELU;
-     * iparams[1] = dtype of bias. Products and sums are f32 for float operands.
+     * iparams[1] = dtype of bias; fparams[0] = alpha scaling the product (0 = 1).
+     * Products and sums are f32. bf16 -> f32 problems with M, N multiples of 256 and K a
+     * multiple of 64 run on the 256x256 LDS-tiled MFMA kernel, the rest on a 64x64 one.
      * args: A, B, (bias when iparams[0] != 0), then C. */
     ZHIP_K_GEMM = 4,
     ZHIP_K_COUNT_

@@ -68,3 +68,96 @@ def test_config3_full_size(hip, oracle):
     v = np.random.default_rng(1).standard_normal(4096)
     lhs, rhs = got.astype(np.float64) @ v, af @ (bf @ v)
     assert np.all(np.abs(lhs - rhs) <= 1e-4 * (np.abs(af) @ (np.abs(bf) @ np.abs(v))))
+
+
+# ---- general kernel: f32, ragged shapes, narrow outputs, batches -------------------------------------
+
+def test_reference_matmul_goldens(hip):
+    # zyx/tests/05_misc.rs:201-208 (matmul_2) on f32 registers, and 09_graph.rs:43-51
+    dev, pool = hip
+    x = np.array([[2, 4, 3], [1, 5, 1]], np.float32)
+    y = np.array([[2, 4], [3, 1], [5, 1]], np.float32)
+    assert gemm(dev, pool, x, y, dtype=DType.F32).tolist() == [[31, 15], [22, 10]]
+
+
+@pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("mnk", [(1, 1, 1), (64, 128, 784), (64, 10, 128), (128, 784, 64), (10, 128, 64), (56, 5, 12),
+                                 (315, 76, 243), (574, 97, 705), (1024, 1024, 1024)])
+def test_f32_gemm_any_shape(hip, oracle, mnk, trans_a, trans_b):
+    """f32: relative 1e-5 against the f64-accumulated product (measured against sum |a b|, the
+    scale rounding errors of any summation order are proportional to); sizes include the
+    reference's matmul_1 sweep corners (05_misc.rs:210-237) and the config-1 MLP products."""
+    dev, pool = hip
+    m, n, k = mnk
+    r = oracle.Rng(m * 31 + n * 7 + k)
+    a = r.uniform((k, m) if trans_a else (m, k), -1, 1)
+    b = r.uniform((n, k) if trans_b else (k, n), -1, 1)
+    got = gemm(dev, pool, a, b, dtype=DType.F32, trans_a=trans_a, trans_b=trans_b)
+    ad, bd = a.astype(np.float64), b.astype(np.float64)
+    ad, bd = (ad.T if trans_a else ad), (bd.T if trans_b else bd)
+    want, mag = ad @ bd, np.abs(ad) @ np.abs(bd)
+    assert np.all(np.abs(got - want) <= 1e-5 * mag + 1e-30), np.max(np.abs(got - want) / (mag + 1e-30))
+    if m * n * k <= 64 * 128 * 784 and not trans_a:
+        ser = oracle.matmul(a, b, oracle.F32, oracle.F32, transb=trans_b)  # the reference's serial order
+        assert np.all(np.abs(got - ser) <= 2e-5 * mag + 1e-30)
+
+
+def test_f32_integer_products_are_exact(hip):
+    """Integer-valued f32 operands (the reference's i+j / i-j matrices): every partial sum is
+    exact in f32, so any summation order must give the exact integer result."""
+    dev, pool = hip
+    m, k, n = 315, 243, 76
+    x = (np.arange(m)[:, None] + np.arange(k)[None, :]).astype(np.float32) % 16
+    y = (np.arange(k)[:, None] - np.arange(n)[None, :]).astype(np.float32) % 8
+    assert np.array_equal(gemm(dev, pool, x, y, dtype=DType.F32), x @ y)
+
+
+@pytest.mark.parametrize("epilogue", ["bias", "bias_relu", "bias_gelu"])
+def test_linear_epilogues(hip, oracle, epilogue):
+    dev, pool = hip
+    r = oracle.Rng(77)
+    x, w, b = r.randn((64, 784)), r.uniform((128, 784), -0.05, 0.05), r.uniform(128, -0.05, 0.05)
+    got = gemm(dev, pool, x, w, b, dtype=DType.F32, trans_b=True, epilogue=epilogue)  # Linear: x . W^T + b
+    lin = oracle.matmul(x, w, oracle.F32, oracle.F32, transb=True)
+    want = oracle.bias_act(lin, b, {"bias": "none", "bias_relu": "relu", "bias_gelu": "gelu"}[epilogue])
+    mag = np.abs(x) @ np.abs(w.T) + np.abs(b)
+    assert np.all(np.abs(got - want) <= 2e-5 * mag)
+    # bf16 operands, bf16 bias, big-tile kernel and general kernel give the same epilogue
+    xb, wb, bb = oracle.f32_to_bf16(r.randn((256, 128))), oracle.f32_to_bf16(r.uniform((256, 128), -0.1, 0.1)), \
+        oracle.f32_to_bf16(r.uniform(256, -1, 1))
+    got = gemm(dev, pool, xb, wb, bb, trans_b=True, epilogue=epilogue, bias_dtype=DType.BF16)
+    lin = oracle.matmul_f64acc(xb, wb, oracle.BF16, transb=True).astype(np.float32)
+    want = oracle.bias_act(lin, bb, {"bias": "none", "bias_relu": "relu", "bias_gelu": "gelu"}[epilogue], oracle.BF16)
+    assert np.all(np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-4)
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16])
+def test_16bit_ragged_and_narrow_store(hip, oracle, dt):
+    """`dot` on 16-bit tensors stores the f32 sum truncated to the operand dtype
+    (zyx/src/tensor/reduce_ops.rs:134-136, zyx/src/codegen/c.rs:494-496); includes the
+    reference's bf16_matmul_1 shape 17x2x19 (zyx/tests/10_bf16.rs:160-198)."""
+    dev, pool = hip
+    conv = oracle.f32_to_bf16 if dt == DType.BF16 else oracle.f32_to_f16
+    back = oracle.bf16_to_f32 if dt == DType.BF16 else oracle.f16_to_f32
+    code = oracle.BF16 if dt == DType.BF16 else oracle.F16
+    m, k, n = 17, 2, 19
+    xf = np.fromfunction(lambda i, j: np.fmod(i + j, 10.0), (m, k)).astype(np.float32)
+    yf = np.fromfunction(lambda i, j: np.fmod(i - j, 10.0), (k, n)).astype(np.float32)
+    got = gemm(dev, pool, conv(xf), conv(yf), dtype=dt, out_dtype=dt)
+    assert np.array_equal(got, oracle.matmul(conv(xf), conv(yf), code, code))  # small ints: exact, then truncated
+    r = oracle.Rng(5)
+    a, b = conv(r.uniform((100, 333), -1, 1)), conv(r.uniform((333, 77), -1, 1))
+    got = back(gemm(dev, pool, a, b, dtype=dt, out_dtype=dt))
+    want = oracle.matmul_f64acc(a, b, code)
+    assert np.all(np.abs(got - want) <= (2 ** -7 if dt == DType.BF16 else 2 ** -10) * np.abs(want) + 1e-4 * (np.abs(back(a)) @ np.abs(back(b))))
+
+
+def test_batched_and_scaled(hip, oracle):
+    """Batched product with alpha: the q . k^T * scale of attention (zyx-nn/src/causal_self_attention.rs:57-60)."""
+    dev, pool = hip
+    r = oracle.Rng(9)
+    q, k = r.randn((6, 40, 64)), r.randn((6, 50, 64))
+    got = gemm(dev, pool, q, k, dtype=DType.F32, trans_b=True, alpha=0.125)
+    want = np.einsum("bik,bjk->bij", q.astype(np.float64), k.astype(np.float64)) * 0.125
+    assert got.shape == (6, 40, 50)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-5)

@@ -1,0 +1,160 @@
+// General GEMM for every shape, layout and float dtype the fast bf16 kernel does not take:
+// f32 (v_mfma_f32_32x32x2_f32), and bf16 / f16 with ragged or small M, N, K
+// (v_mfma_f32_32x32x16_{bf16,f16}). C = op(A) . op(B) (+ bias) (ReLU | GELU), f32
+// accumulation, result stored as f32 or narrowed to the operand dtype with the C backend's
+// truncating stores (zyx/src/codegen/c.rs:456-497).
+//
+// This is the Linear / dot of the small configs (zyx-nn/src/linear.rs:38-44,
+// zyx/src/tensor/mod.rs:1469-1518), e.g. the 784 -> 128 -> 10 MLP, and of the backward
+// products dW = X^T . dY, dX = dY . W that autograd's Mul/Expand/Reduce rules collapse to
+// (zyx/src/graph/autograd.rs:120-125 and the rules kept in comments at :195-242, 269-295).
+//
+// 64 x 64 tile per 256-thread workgroup, 2 x 2 waves of one 32 x 32 MFMA tile each, K step
+// 32. Operands are read with bounds checks (zero fill) straight from their natural layout,
+// coalesced along whichever index is contiguous, and laid down K-contiguous in LDS with an
+// 8-element row pad, so fragment reads are the same for all four layouts.
+#include "dtypes.hpp"
+#include "kernels.hpp"
+#include "wave.hpp"
+
+namespace zk {
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int GM = 64, GN = 64, GK = 32, GPAD = 8;
+
+template <int DT> struct GT;
+template <> struct GT<DT_F32> {
+    typedef float S;
+    static __device__ __forceinline__ float zero() { return 0.0f; }
+};
+template <> struct GT<DT_BF16> {
+    typedef uint16_t S;
+    static __device__ __forceinline__ uint16_t zero() { return 0; }
+};
+template <> struct GT<DT_F16> {
+    typedef uint16_t S;
+    static __device__ __forceinline__ uint16_t zero() { return 0; }
+};
+
+__device__ __forceinline__ float gelu_ref(float x) { // zyx/src/tensor/elementwise.rs:168-170, saturating tanh
+    float inner = (x + ((x * x) * x) * 0.044715f) * 0.79788456080286535588f;
+    float e = expf(inner + inner);
+    float t = (inner + inner) > 88.0f ? 1.0f : (e - 1.0f) / (e + 1.0f);
+    return (x * 0.5f) * (t + 1.0f);
+}
+
+// Copies a [rows x GK] operand tile into LDS as dst[row][k]. `rs`/`ks` are the element
+// strides of the row index (m or n) and of k in global memory; one of them is 1.
+template <typename S>
+__device__ __forceinline__ void fill_tile(S *__restrict__ dst, const S *__restrict__ src, int64_t rs, int64_t ks,
+                                          int64_t row0, int64_t k0, int64_t rows, int64_t K, S zero) {
+    const int t = threadIdx.x;
+    if (ks == 1) { // K contiguous: consecutive threads walk along k
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int idx = e * 256 + t, r = idx >> 5, k = idx & 31;
+            const int64_t gr = row0 + r, gk = k0 + k;
+            dst[r * (GK + GPAD) + k] = (gr < rows && gk < K) ? src[gr * rs + gk] : zero;
+        }
+    } else { // row index contiguous: consecutive threads walk along the rows
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int idx = e * 256 + t, k = idx >> 6, r = idx & 63;
+            const int64_t gr = row0 + r, gk = k0 + k;
+            dst[r * (GK + GPAD) + k] = (gr < rows && gk < K) ? src[gr * rs + gk * ks] : zero;
+        }
+    }
+}
+
+template <int DT, int ODT>
+__global__ __launch_bounds__(256) void gemm_generic_k(const GemmGeneric p) {
+    typedef typename GT<DT>::S S;
+    __shared__ __attribute__((aligned(16))) S As[GM * (GK + GPAD)];
+    __shared__ __attribute__((aligned(16))) S Bs[GN * (GK + GPAD)];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int64_t m0 = (int64_t)blockIdx.y * GM, n0 = (int64_t)blockIdx.x * GN;
+    const S *A = (const S *)p.A + (int64_t)blockIdx.z * p.batch_a, *B = (const S *)p.B + (int64_t)blockIdx.z * p.batch_b;
+    const int64_t a_rs = p.trans_a ? 1 : p.K, a_ks = p.trans_a ? p.M : 1;
+    const int64_t b_rs = p.trans_b ? p.K : 1, b_ks = p.trans_b ? 1 : p.N;
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+    for (int64_t k0 = 0; k0 < p.K; k0 += GK) {
+        __syncthreads(); // previous step's fragment reads are done
+        fill_tile<S>(As, A, a_rs, a_ks, m0, k0, p.M, p.K, GT<DT>::zero());
+        fill_tile<S>(Bs, B, b_rs, b_ks, n0, k0, p.N, p.K, GT<DT>::zero());
+        __syncthreads();
+        const S *ar = As + (wm * 32 + (lane & 31)) * (GK + GPAD);
+        const S *br = Bs + (wn * 32 + (lane & 31)) * (GK + GPAD);
+        if (DT == DT_F32) {
+#pragma unroll
+            for (int ks = 0; ks < GK; ks += 2) {
+                float a = ((const float *)ar)[ks + (lane >> 5)], b = ((const float *)br)[ks + (lane >> 5)];
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < GK; ks += 16) {
+                const int off = ks + (lane >> 5) * 8;
+                if (DT == DT_BF16) {
+                    bf16x8 a = *(const bf16x8 *)((const uint16_t *)ar + off), b = *(const bf16x8 *)((const uint16_t *)br + off);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+                } else {
+                    f16x8 a = *(const f16x8 *)((const uint16_t *)ar + off), b = *(const f16x8 *)((const uint16_t *)br + off);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32 x 32 tile
+    const int64_t col = n0 + wn * 32 + (lane & 31);
+    if (col >= p.N) return; // no barrier follows
+    float bv = 0.0f;
+    if (p.epilogue >= 1) {
+        if (p.bias_dtype == DT_BF16) bv = bf16_to_f32(((const uint16_t *)p.bias)[col]);
+        else if (p.bias_dtype == DT_F16) bv = f16_to_f32(((const uint16_t *)p.bias)[col]);
+        else bv = ((const float *)p.bias)[col];
+    }
+    char *C = (char *)p.C + (int64_t)blockIdx.z * p.batch_c * (ODT == DT_F32 ? 4 : 2);
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int64_t row = m0 + wm * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (row >= p.M) continue;
+        float v = acc[r] * p.alpha;
+        if (p.epilogue >= 1) v += bv;
+        if (p.epilogue == 2) v = (v > 0.0f ? 1.0f : 0.0f) * v;
+        if (p.epilogue == 3) v = gelu_ref(v);
+        const int64_t o = row * p.N + col;
+        if (ODT == DT_F32) ((float *)C)[o] = v;
+        else if (ODT == DT_BF16) ((uint16_t *)C)[o] = f32_to_bf16_trunc(v);
+        else ((uint16_t *)C)[o] = f32_to_f16_trunc(v);
+    }
+}
+
+} // namespace
+
+hipError_t gemm_generic(const GemmGeneric &p, hipStream_t st) {
+    if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return hipSuccess;
+    if (p.K < 0 || (p.M + GM - 1) / GM > 65535 || p.batch > 65535) return hipErrorInvalidValue;
+    dim3 grid((unsigned)((p.N + GN - 1) / GN), (unsigned)((p.M + GM - 1) / GM), (unsigned)p.batch), block(256);
+#define ZK_G(D, O) hipLaunchKernelGGL((gemm_generic_k<D, O>), grid, block, 0, st, p)
+    if (p.dtype == DT_F32 && p.out_dtype == DT_F32) ZK_G(DT_F32, DT_F32);
+    else if (p.dtype == DT_BF16 && p.out_dtype == DT_F32) ZK_G(DT_BF16, DT_F32);
+    else if (p.dtype == DT_BF16 && p.out_dtype == DT_BF16) ZK_G(DT_BF16, DT_BF16);
+    else if (p.dtype == DT_F16 && p.out_dtype == DT_F32) ZK_G(DT_F16, DT_F32);
+    else if (p.dtype == DT_F16 && p.out_dtype == DT_F16) ZK_G(DT_F16, DT_F16);
+    else return hipErrorInvalidValue;
+#undef ZK_G
+    return hipGetLastError();
+}
+
+} // namespace zk

@@ -58,4 +58,19 @@ struct GemmBf16 {
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K);
 hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t stream);
 
+// Any-shape GEMM: dtype F32 / BF16 / F16 operands, f32 accumulate, C stored as F32 or as
+// the operand dtype (truncating). `batch` independent products at element strides
+// batch_a / batch_b / batch_c. C = alpha * op(A).op(B) (+ bias) (act).
+struct GemmGeneric {
+    int64_t M, N, K, batch;
+    int64_t batch_a, batch_b, batch_c;
+    int dtype, out_dtype;
+    int trans_a, trans_b;
+    int epilogue, bias_dtype;
+    float alpha;
+    const void *A, *B, *bias;
+    void *C;
+};
+hipError_t gemm_generic(const GemmGeneric &p, hipStream_t stream);
+
 } // namespace zk

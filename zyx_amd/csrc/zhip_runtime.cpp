@@ -317,23 +317,22 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         return ZHIP_OK;
     }
     case ZHIP_K_GEMM: {
-        int64_t M = d.dims[0], N = d.dims[1], K = d.dims[2];
+        int64_t M = d.dims[0], N = d.dims[1], K = d.dims[2], batch = d.dims[3] ? d.dims[3] : 1;
         int epi = d.iparams[0];
-        if (M <= 0 || N <= 0 || K <= 0) return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: M, N, K must be positive");
+        if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || batch > 65535) return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: M, N, K, batch out of range");
         if (epi < 0 || epi > 3 || (d.flags & ~3)) return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: bad epilogue/flags");
-        if (d.dtype == ZHIP_BF16 && d.out_dtype == ZHIP_F32 && zk::gemm_bf16_supported(M, N, K)) {
-            if (epi && d.iparams[1] != ZHIP_BF16 && d.iparams[1] != ZHIP_F32)
-                return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: bias must be bf16 or f32");
-        } else {
-            return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: no kernel for dtype %d -> %d with M=%lld N=%lld K=%lld", d.dtype,
-                           d.out_dtype, (long long)M, (long long)N, (long long)K);
-        }
+        bool float_in = d.dtype == ZHIP_F32 || d.dtype == ZHIP_BF16 || d.dtype == ZHIP_F16;
+        if (!float_in || (d.out_dtype != ZHIP_F32 && d.out_dtype != d.dtype))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: no kernel for dtype %d -> %d", d.dtype, d.out_dtype);
+        if (epi && d.iparams[1] != ZHIP_BF16 && d.iparams[1] != ZHIP_F32 && d.iparams[1] != ZHIP_F16)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: bias must be bf16, f16 or f32");
+        if ((M + 63) / 64 > 65535) return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: M too large for the general kernel");
         int a = 0;
-        p.need[a++] = (uint64_t)M * K * dtype_bytes(d.dtype);
-        p.need[a++] = (uint64_t)K * N * dtype_bytes(d.dtype);
+        p.need[a++] = (uint64_t)batch * M * K * dtype_bytes(d.dtype);
+        p.need[a++] = (uint64_t)batch * K * N * dtype_bytes(d.dtype);
         if (epi) p.need[a++] = (uint64_t)N * dtype_bytes(d.iparams[1]);
         p.n_in = a;
-        p.need[a] = (uint64_t)M * N * dtype_bytes(d.out_dtype);
+        p.need[a] = (uint64_t)batch * M * N * dtype_bytes(d.out_dtype);
         p.n_out = 1;
         return ZHIP_OK;
     }
@@ -388,19 +387,45 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         return zk::reduce(a, st);
     }
     case ZHIP_K_GEMM: {
-        zk::GemmBf16 a{};
-        a.M = d.dims[0];
-        a.N = d.dims[1];
-        a.K = d.dims[2];
-        a.trans_a = d.flags & ZHIP_GEMM_TRANS_A ? 1 : 0;
-        a.trans_b = d.flags & ZHIP_GEMM_TRANS_B ? 1 : 0;
-        a.epilogue = d.iparams[0];
-        a.bias_dtype = d.iparams[1];
-        a.A = ptr[0];
-        a.B = ptr[1];
-        a.bias = a.epilogue ? ptr[2] : nullptr;
-        a.C = ptr[p.n_in];
-        return zk::gemm_bf16(a, st);
+        const int64_t batch = d.dims[3] ? d.dims[3] : 1;
+        const float alpha = d.fparams[0] == 0.0f ? 1.0f : d.fparams[0];
+        const bool fast = d.dtype == ZHIP_BF16 && d.out_dtype == ZHIP_F32 && batch == 1 && alpha == 1.0f &&
+                          (d.iparams[0] == 0 || d.iparams[1] != ZHIP_F16) && zk::gemm_bf16_supported(d.dims[0], d.dims[1], d.dims[2]);
+        if (fast) {
+            zk::GemmBf16 a{};
+            a.M = d.dims[0];
+            a.N = d.dims[1];
+            a.K = d.dims[2];
+            a.trans_a = d.flags & ZHIP_GEMM_TRANS_A ? 1 : 0;
+            a.trans_b = d.flags & ZHIP_GEMM_TRANS_B ? 1 : 0;
+            a.epilogue = d.iparams[0];
+            a.bias_dtype = d.iparams[1];
+            a.A = ptr[0];
+            a.B = ptr[1];
+            a.bias = a.epilogue ? ptr[2] : nullptr;
+            a.C = ptr[p.n_in];
+            return zk::gemm_bf16(a, st);
+        }
+        zk::GemmGeneric g{};
+        g.M = d.dims[0];
+        g.N = d.dims[1];
+        g.K = d.dims[2];
+        g.batch = batch;
+        g.batch_a = g.M * g.K;
+        g.batch_b = g.K * g.N;
+        g.batch_c = g.M * g.N;
+        g.dtype = d.dtype;
+        g.out_dtype = d.out_dtype;
+        g.trans_a = d.flags & ZHIP_GEMM_TRANS_A ? 1 : 0;
+        g.trans_b = d.flags & ZHIP_GEMM_TRANS_B ? 1 : 0;
+        g.epilogue = d.iparams[0];
+        g.bias_dtype = d.iparams[1];
+        g.alpha = alpha;
+        g.A = ptr[0];
+        g.B = ptr[1];
+        g.bias = g.epilogue ? ptr[2] : nullptr;
+        g.C = ptr[p.n_in];
+        return zk::gemm_generic(g, st);
     }
     default: return hipErrorInvalidValue;
     }
