@@ -138,11 +138,31 @@ enum zhip_kernel_kind {
      * multiple of 64 run on the 256x256 LDS-tiled MFMA kernel, the rest on a 64x64 one.
      * args: A, B, (bias when iparams[0] != 0), then C. */
     ZHIP_K_GEMM = 4,
+    /* y = LayerNorm(x) or RMSNorm(x) over the last axis of x[rows, cols] (dims = {rows, cols},
+     * dtype F32 or BF16 for x, weight, bias and y, f32 arithmetic, one narrowing store).
+     * flags: ZHIP_NORM_RMS selects RMSNorm, ZHIP_NORM_WEIGHT / ZHIP_NORM_BIAS say which
+     * affine operands are passed; fparams[0] = eps. LayerNorm uses the unbiased (n-1)
+     * variance, as zyx-nn/src/layer_norm.rs:98-135 does through Tensor::var
+     * (zyx/src/tensor/reduce_ops.rs:795-805); RMSNorm is zyx-nn/src/rms_norm.rs:26-32.
+     * args: x, (weight[cols]), (bias[cols]), then y. */
+    ZHIP_K_NORM_ROWS = 5,
+    /* Tensor::cross_entropy of f32 logits[rows, cols] with I32 class indices[rows]
+     * (zyx/src/tensor/mod.rs:1639-1655; ln_softmax :1427-1431; one-hot by equal(arange)
+     * :1920-1946). flags: ZHIP_CE_LOSS writes the per-sample loss[rows] (ReduceOp::None),
+     * ZHIP_CE_GRAD writes d(fparams[0] * sum(loss))/d(logits) = (softmax - onehot) *
+     * fparams[0] into grad[rows, cols] (fparams[0] = 1/rows for the Mean reduction).
+     * args: logits, labels, (loss), (grad). */
+    ZHIP_K_CROSS_ENTROPY = 6,
     ZHIP_K_COUNT_
 };
 #define ZHIP_SOFTMAX_Y 1
 #define ZHIP_SOFTMAX_ROWSUM 2
 #define ZHIP_SOFTMAX_ARGMAX 4
+#define ZHIP_NORM_RMS 1
+#define ZHIP_NORM_WEIGHT 2
+#define ZHIP_NORM_BIAS 4
+#define ZHIP_CE_LOSS 1
+#define ZHIP_CE_GRAD 2
 #define ZHIP_GEMM_TRANS_A 1
 #define ZHIP_GEMM_TRANS_B 2
 
@@ -260,6 +280,22 @@ int32_t zhip_time_kernel(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args, si
  * successive launches touch different memory. */
 int32_t zhip_profile_kernel(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args, size_t n_args, size_t arg_sets,
                             int32_t iters, float *avg_us);
+
+/* --- cached execution plans ----------------------------------------------------- */
+
+/* The steady state of Tape::realize / FrozenTape::replay is a fixed list of Launch nodes on
+ * fixed buffers (ExecPlan, zyx/src/graph/plan.rs:58-237; replay loop :271-361; plan cache
+ * zyx/src/tape.rs:165-181, 299-318). zhip_plan_create records such a list once -- programs
+ * in execution order, each with its buffer ids (inputs then outputs), args_flat holding the
+ * lists back to back and n_args their lengths -- as a HIP graph on one in-order stream, so a
+ * later node sees the results of every earlier one. zhip_plan_launch replays it with one
+ * call: it waits for (and consumes) evs, and returns the event of the whole list. Buffers
+ * and programs named by a plan must stay alive until zhip_plan_destroy. */
+typedef uint32_t zhip_plan;
+int32_t zhip_plan_create(zhip_ctx *ctx, const zhip_prog *progs, const zhip_buf *args_flat, const uint32_t *n_args,
+                         size_t n_nodes, zhip_plan *plan);
+int32_t zhip_plan_launch(zhip_ctx *ctx, zhip_plan plan, const zhip_event *evs, size_t n_evs, zhip_event *ev);
+int32_t zhip_plan_destroy(zhip_ctx *ctx, zhip_plan plan);
 
 #ifdef __cplusplus
 }

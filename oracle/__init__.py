@@ -198,15 +198,17 @@ def argmax_rows(x: np.ndarray) -> np.ndarray:
     return a
 
 
-def matmul(a: np.ndarray, b: np.ndarray, in_dtype: int = F32, out_dtype: int = F32, transb: bool = False) -> np.ndarray:
-    """dot / dot_dtype of zyx/src/tensor/mod.rs:1469-1518 on 2-D operands."""
+def matmul(a: np.ndarray, b: np.ndarray, in_dtype: int = F32, out_dtype: int = F32, transb: bool = False,
+           transa: bool = False) -> np.ndarray:
+    """dot / dot_dtype of zyx/src/tensor/mod.rs:1469-1518 on 2-D operands (a stored [k,m] if transa,
+    b stored [n,k] if transb)."""
     a = np.ascontiguousarray(a)
     b = np.ascontiguousarray(b)
-    m, k = a.shape
+    m, k = (a.shape[1], a.shape[0]) if transa else a.shape
     n = b.shape[0] if transb else b.shape[1]
     assert (b.shape[1] if transb else b.shape[0]) == k
     c = np.empty((m, n), _store_dtype(out_dtype))
-    lib().zo_matmul_float(in_dtype, out_dtype, _p(a), _p(b), _p(c), _I64(m), _I64(n), _I64(k), int(transb))
+    lib().zo_matmul_float(in_dtype, out_dtype, _p(a), _p(b), _p(c), _I64(m), _I64(n), _I64(k), int(transb), int(transa))
     return c
 
 
@@ -252,3 +254,59 @@ def ew_chain(chain, arrays) -> np.ndarray:
     lib().zo_ew_chain(int(chain.reg), int(chain.out_dtype), n_in, in_desc, ptrs, len(chain.code), code, consts, _p(out),
                       _I64(chain.rows), _I64(chain.cols))
     return out
+
+
+def layer_norm(x, w=None, b=None, eps: float = 1e-5, dtype: int = F32) -> np.ndarray:
+    x = np.ascontiguousarray(x, _store_dtype(dtype))
+    rows, cols = x.shape
+    y = np.empty_like(x)
+    w = None if w is None else np.ascontiguousarray(w, x.dtype)
+    b = None if b is None else np.ascontiguousarray(b, x.dtype)
+    lib().zo_layer_norm(dtype, _p(x), _p(w), _p(b), _p(y), _I64(rows), _I64(cols), C.c_float(eps))
+    return y
+
+
+def rms_norm(x, w=None, eps: float = 1e-6, dtype: int = F32) -> np.ndarray:
+    x = np.ascontiguousarray(x, _store_dtype(dtype))
+    rows, cols = x.shape
+    y = np.empty_like(x)
+    w = None if w is None else np.ascontiguousarray(w, x.dtype)
+    lib().zo_rms_norm(dtype, _p(x), _p(w), _p(y), _I64(rows), _I64(cols), C.c_float(eps))
+    return y
+
+
+def cross_entropy(logits, labels, gscale: float | None = None):
+    """-> (per-sample loss [rows], grad of gscale*sum(loss) or None)."""
+    x = np.ascontiguousarray(logits, np.float32)
+    lab = np.ascontiguousarray(labels, np.int32)
+    rows, cols = x.shape
+    loss = np.empty(rows, np.float32)
+    grad = np.empty_like(x) if gscale is not None else None
+    lib().zo_cross_entropy(_p(x), _p(lab), _p(loss), _p(grad), _I64(rows), _I64(cols), C.c_float(gscale or 0.0))
+    return loss, grad
+
+
+def mlp_step(x, labels, w1, b1, w2, b2, lr: float):
+    """One SGD step of the 2-layer MLP of config 1 (Linear -> ReLU -> Linear -> cross_entropy mean),
+    composed from the oracle's primitives in the order zyx's Tape would evaluate them:
+      forward  zyx-nn/src/linear.rs:38-44 (x . W^T + b), relu = (x > 0) * x
+      backward zyx/src/graph/autograd.rs: Mul :120-125 (relu mask, dot products), Add :111-119 (bias:
+               gradient summed over the broadcast batch axis), dot = broadcast-mul + sum(-1)
+      update   zyx-optim/src/sgd.rs:77-81 p <- p - g * lr
+    Returns (mean loss, new w1, b1, w2, b2, dict of gradients)."""
+    n = x.shape[0]
+    pre = bias_act(matmul(x, w1, transb=True), b1, "none")
+    h = unary("relu", pre)
+    logits = bias_act(matmul(h, w2, transb=True), b2, "none")
+    loss, dlogits = cross_entropy(logits, labels, 1.0 / n)
+    dw2 = matmul(dlogits, h, transa=True)            # [out2, n] . [n, hidden]
+    db2 = reduce_cols("sum", dlogits)
+    dh = matmul(dlogits, w2)                           # [n, out2] . [out2, hidden]
+    dpre = binary("mul", binary("cmpgt", pre, np.float32(0.0)), dh)
+    dw1 = matmul(dpre, x, transa=True)
+    db1 = reduce_cols("sum", dpre)
+    lr32 = np.float32(lr)
+    upd = lambda p, g: binary("sub", p, binary("mul", g, lr32))
+    grads = dict(w1=dw1, b1=db1, w2=dw2, b2=db2, logits=dlogits)
+    mean_loss = np.float32(reduce_rows("sum", loss[None, :])[0] / np.float32(n))
+    return mean_loss, upd(w1, dw1), upd(b1[None, :], db1[None, :])[0], upd(w2, dw2), upd(b2[None, :], db2[None, :])[0], grads

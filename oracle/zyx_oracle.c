@@ -394,15 +394,16 @@ ZO_API void zo_argmax_rows_f32(const float *x, int32_t *arg, int64_t rows, int64
  * reference lowers to. in_dtype is the storage dtype of A and B; products and the
  * accumulator live in float registers; the result is stored as out_dtype
  * (`dot` on bf16 stores bf16, truncating; `dot_dtype(F32)` stores f32).
- * transb != 0 reads B as [n,k] (Linear's W stored [out,in], linear.rs:38-44). */
+ *  transb != 0 reads B as [n,k] (Linear's W stored [out,in], linear.rs:38-44), transa != 0
+ * reads A as [k,m] (the x.t() of a weight gradient). */
 ZO_API void zo_matmul_float(int in_dtype, int out_dtype, const void *a, const void *b, void *c, int64_t m, int64_t n,
-                            int64_t k, int transb) {
+                            int64_t k, int transb, int transa) {
 #pragma omp parallel for
     for (int64_t i = 0; i < m; i++)
         for (int64_t j = 0; j < n; j++) {
             float acc = 0.0f;
             for (int64_t p = 0; p < k; p++) {
-                float x = load_as_f32(a, in_dtype, i * k + p);
+                float x = load_as_f32(a, in_dtype, transa ? p * m + i : i * k + p);
                 float y = load_as_f32(b, in_dtype, transb ? j * k + p : p * n + j);
                 acc = x * y + acc;
             }
@@ -599,4 +600,75 @@ ZO_API void zo_ew_chain(int reg_class, int out_dtype, int n_in, const int32_t *i
                 }
             }
         }
+}
+
+
+/* ------------------------------------------------------------------------- */
+/* Normalisation layers and the classification loss                           */
+/* ------------------------------------------------------------------------- */
+
+/* LayerNorm over the last axis (zyx-nn/src/layer_norm.rs:98-135):
+ *   mean = sum(x) / n;  var = sum((x - mean)^2) / (n - 1)   (Tensor::var: correction 1,
+ *   zyx/src/tensor/reduce_ops.rs:795-805, 111-123)
+ *   y = (x - mean) / sqrt(var + eps) (* w) (+ b)
+ * evaluated as one fused float-register kernel; storage dtype f32 or bf16. */
+ZO_API void zo_layer_norm(int dtype, const void *x, const void *w, const void *b, void *y, int64_t rows, int64_t cols,
+                          float eps) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++) {
+        float s = 0.0f;
+        for (int64_t c = 0; c < cols; c++) s = load_as_f32(x, dtype, r * cols + c) + s;
+        float mean = s / (float)cols;
+        float v = 0.0f;
+        for (int64_t c = 0; c < cols; c++) {
+            float d = load_as_f32(x, dtype, r * cols + c) - mean;
+            v = d * d + v;
+        }
+        float den = sqrtf(v / (float)(cols - 1) + eps);
+        for (int64_t c = 0; c < cols; c++) {
+            float o = (load_as_f32(x, dtype, r * cols + c) - mean) / den;
+            if (w) o = o * load_as_f32(w, dtype, c);
+            if (b) o = o + load_as_f32(b, dtype, c);
+            store_from_f32(y, dtype, r * cols + c, o);
+        }
+    }
+}
+/* RMSNorm (zyx-nn/src/rms_norm.rs:26-32): x * sqrt(1 / (mean(x*x) + eps)) * scale */
+ZO_API void zo_rms_norm(int dtype, const void *x, const void *w, void *y, int64_t rows, int64_t cols, float eps) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++) {
+        float s = 0.0f;
+        for (int64_t c = 0; c < cols; c++) {
+            float v = load_as_f32(x, dtype, r * cols + c);
+            s = v * v + s;
+        }
+        float sc = sqrtf(1.0f / (s / (float)cols + eps));
+        for (int64_t c = 0; c < cols; c++) {
+            float o = load_as_f32(x, dtype, r * cols + c) * sc;
+            if (w) o = o * load_as_f32(w, dtype, c);
+            store_from_f32(y, dtype, r * cols + c, o);
+        }
+    }
+}
+/* Tensor::cross_entropy with class-index targets, reduction None (zyx/src/tensor/mod.rs:
+ * 1639-1655): m = x - max_c x; ls = m - ln(sum_c exp(m)); loss = sum_c (-ls[c]) * onehot[c]
+ * with onehot = (label == arange) (:1920-1946). grad (optional) is d(gscale * sum_r loss)/dx
+ * = (softmax - onehot) * gscale: what the reference's reverse rules for Sub/Exp/Ln/Sum/Max/Mul
+ * (zyx/src/graph/autograd.rs:87-134, 155-162) add up to; pinned by finite differences. */
+ZO_API void zo_cross_entropy(const float *x, const int32_t *labels, float *loss, float *grad, int64_t rows,
+                             int64_t cols, float gscale) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++) {
+        const float *xr = x + r * cols;
+        float mx = -FLT_MAX, s = 0.0f, l = 0.0f;
+        for (int64_t c = 0; c < cols; c++) mx = fmaxf(xr[c], mx);
+        for (int64_t c = 0; c < cols; c++) s = expf(xr[c] - mx) + s;
+        float lns = logf(s);
+        for (int64_t c = 0; c < cols; c++) {
+            float ls = (xr[c] - mx) - lns;
+            l = (-ls) * (float)(labels[r] == (int32_t)c) + l;
+            if (grad) grad[r * cols + c] = (expf(xr[c] - mx) / s - (float)(labels[r] == (int32_t)c)) * gscale;
+        }
+        if (loss) loss[r] = l;
+    }
 }

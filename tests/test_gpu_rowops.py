@@ -1,0 +1,76 @@
+"""LayerNorm / RMSNorm / cross entropy on the GPU vs the CPU oracle and the reference's goldens
+(zyx/tests/05_misc.rs:702-730 layer_norm, :1199-1214 cross_entropy). f32 tolerance 1e-5 relative
+to the row's scale (a normalised row has cancelling entries near zero, so the bound is
+rel 1e-5 * max(|want|, rms of the row))."""
+import numpy as np
+import pytest
+
+from zyx_amd import DType
+from zyx_amd.kernels import cross_entropy, norm_rows
+
+pytestmark = pytest.mark.gpu
+
+
+def close_rows(got, want, rtol=1e-5):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    scale = np.maximum(np.abs(want), np.sqrt((want**2).mean(-1, keepdims=True)))
+    assert np.all(np.abs(got - want) <= rtol * scale + 1e-30), np.max(np.abs(got - want) / (scale + 1e-30))
+
+
+def test_layer_norm_reference_golden(hip):
+    dev, pool = hip
+    x = np.array([[3, 5, 2, 1], [6, 1, 4, 2]], np.float32)
+    y = norm_rows(dev, pool, x, w=np.array([4, 5, 1, 2], np.float32), eps=0.00001)
+    np.testing.assert_allclose(y, [[0.585539, 6.587314, -0.439154, -2.049387], [4.960858, -5.073606, 0.338240, -1.127468]],
+                               rtol=2e-6)
+
+
+@pytest.mark.parametrize("shape", [(8192, 1024), (5, 7), (33, 1000), (4, 4096), (3, 5001), (1, 2)])
+@pytest.mark.parametrize("rms", [False, True])
+def test_norms_f32(hip, oracle, shape, rms):
+    dev, pool = hip
+    r = oracle.Rng(shape[1])
+    x, w, b = r.randn(shape, 2.0) + np.float32(0.5), r.randn(shape[1]), r.randn(shape[1])
+    if rms:
+        close_rows(norm_rows(dev, pool, x, w, rms=True, eps=1e-6), oracle.rms_norm(x, w, 1e-6))
+        close_rows(norm_rows(dev, pool, x, None, rms=True, eps=1e-6), oracle.rms_norm(x, None, 1e-6))
+    else:
+        close_rows(norm_rows(dev, pool, x, w, b), oracle.layer_norm(x, w, b))
+        close_rows(norm_rows(dev, pool, x, w, None), oracle.layer_norm(x, w, None))
+        close_rows(norm_rows(dev, pool, x), oracle.layer_norm(x))
+        xd = x.astype(np.float64)  # what the mathematics fixes: unbiased variance
+        want = (xd - xd.mean(1, keepdims=True)) / np.sqrt(xd.var(1, ddof=1, keepdims=True) + 1e-5)
+        close_rows(norm_rows(dev, pool, x), want)
+
+
+@pytest.mark.parametrize("rms", [False, True])
+def test_norms_bf16(hip, oracle, rms):
+    """bf16 storage: f32 arithmetic, one truncating store -> at most one bf16 unit from the oracle."""
+    dev, pool = hip
+    r = oracle.Rng(3)
+    x, w, b = (oracle.f32_to_bf16(a) for a in (r.randn((64, 1024)), r.randn(1024), r.randn(1024)))
+    if rms:
+        got, want = norm_rows(dev, pool, x, w, rms=True, eps=1e-6, dtype=DType.BF16), oracle.rms_norm(x, w, 1e-6, oracle.BF16)
+    else:
+        got, want = norm_rows(dev, pool, x, w, b, dtype=DType.BF16), oracle.layer_norm(x, w, b, 1e-5, oracle.BF16)
+    assert np.all(np.abs(got.astype(np.int32) - want.astype(np.int32)) <= 1)
+    assert np.mean(got == want) > 0.98
+
+
+def test_cross_entropy(hip, oracle):
+    dev, pool = hip
+    loss, _ = cross_entropy(dev, pool, np.array([[2, 3, 4], [5, 6, 7]], np.float32), np.array([1, 2], np.int32))
+    np.testing.assert_allclose(loss, [1.407606, 0.407606], rtol=2e-6)
+    r = oracle.Rng(8)
+    for rows, cols in ((64, 10), (1, 1), (300, 1000), (7, 65)):
+        x, lab = r.randn((rows, cols), 3.0), r.randint(rows, 0, cols)
+        loss, grad = cross_entropy(dev, pool, x, lab, 1.0 / rows)
+        wl, wg = oracle.cross_entropy(x, lab, 1.0 / rows)
+        np.testing.assert_allclose(loss, wl, rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(grad, wg, rtol=1e-5, atol=1e-9)
+        assert np.all(np.abs(grad.sum(1)) < 1e-6)  # softmax - onehot sums to zero in every row
+    # labels outside the class range match no class: zero loss, gradient = softmax * scale
+    x = r.randn((2, 5))
+    loss, grad = cross_entropy(dev, pool, x, np.array([-1, 5], np.int32), 1.0)
+    assert loss.tolist() == [0.0, 0.0]
+    np.testing.assert_allclose(grad.sum(1), [1.0, 1.0], rtol=1e-6)

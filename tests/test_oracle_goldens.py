@@ -232,3 +232,99 @@ def test_matmul_f32_vs_textbook(oracle):
     bias = r.uniform(64, -1, 1)
     c = oracle.matmul(a, b)
     assert close(oracle.bias_act(c, bias, "relu"), np.maximum(c + bias, 0), rel=1e-6)
+
+
+# ---- layer norm / variance: 05_misc.rs:702-730 (pins the n-1 variance) -----------------------
+def test_layer_norm_golden(oracle):
+    x = np.array([[3, 5, 2, 1], [6, 1, 4, 2]], np.float32)
+    y = oracle.layer_norm(x, w=np.array([4, 5, 1, 2], np.float32), eps=0.00001)
+    assert close(y, [[0.585539, 6.587314, -0.439154, -2.049387], [4.960858, -5.073606, 0.338240, -1.127468]], rel=2e-6)
+    r = oracle.Rng(2)
+    x, w, b = r.randn((7, 96)), r.randn(96), r.randn(96)
+    xd = x.astype(np.float64)
+    want = (xd - xd.mean(1, keepdims=True)) / np.sqrt(xd.var(1, ddof=1, keepdims=True) + 1e-5) * w + b
+    assert close(oracle.layer_norm(x, w, b), want, rel=1e-5, abs_=1e-5)
+    want = xd / np.sqrt((xd * xd).mean(1, keepdims=True) + 1e-6) * w
+    assert close(oracle.rms_norm(x, w), want, rel=1e-5, abs_=1e-6)
+
+
+# ---- cross entropy: 05_misc.rs:1199-1214 ------------------------------------------------------
+def test_cross_entropy_golden_and_gradient(oracle):
+    x = np.array([[2, 3, 4], [5, 6, 7]], np.float32)
+    loss, _ = oracle.cross_entropy(x, np.array([1, 2], np.int32))
+    assert close(loss, [1.407606, 0.407606], rel=2e-6)
+    # gradient against central finite differences of the oracle's own forward, in float64
+    r = oracle.Rng(4)
+    logits, labels = r.randn((5, 7)).astype(np.float64), np.array([0, 3, 6, 2, 2], np.int32)
+
+    def f(z):
+        m = z - z.max(1, keepdims=True)
+        ls = m - np.log(np.exp(m).sum(1, keepdims=True))
+        return -(ls[np.arange(5), labels]).sum() / 5
+
+    _, g = oracle.cross_entropy(logits.astype(np.float32), labels, 1.0 / 5)
+    num = np.zeros_like(logits)
+    for i in range(5):
+        for j in range(7):
+            d = np.zeros_like(logits)
+            d[i, j] = 1e-6
+            num[i, j] = (f(logits + d) - f(logits - d)) / 2e-6
+    assert np.allclose(g, num, rtol=1e-4, atol=1e-6)
+
+
+# ---- MLP backward: 11_autograd.rs:418-466 (grad_linear_2, exact integers) ----------------------
+def test_mlp_backward_golden(oracle):
+    """Same network shape as config 1 (Linear, ReLU, Linear) with a squared-error loss: the
+    reference's exact integer gradients pin the backward products (dW = x^T . dy, db = column sum,
+    relu mask, dX = dy . W) the oracle's mlp_step is composed of."""
+    x = np.array([[2, 3, 1]], np.float32)
+    y = np.array([[5, 4, 5, 2]], np.float32)
+    w1 = np.array([2, 3, 1, 4, 5, 1, 6, 2, 3, 1, 6, 2, 4, 1, 4], np.float32).reshape(3, 5)   # [in, out]
+    b1 = np.array([4, 1, 5, 7, 6], np.float32)
+    w2 = np.array([2, 3, 1, 4, 5, 1, 6, 2, 3, 1, 6, 2, 4, 1, 4, 5, 1, 2, 4, 1], np.float32).reshape(5, 4)
+    b2 = np.array([4, 1, 5, 7], np.float32)
+    pre = oracle.bias_act(oracle.matmul(x, w1), b1, "none")
+    h = oracle.unary("relu", pre)
+    out = oracle.bias_act(oracle.matmul(h, w2), b2, "none")
+    dout = 2 * (out - y)                       # d/dout of sum((out - y)^2)
+    dw2 = oracle.matmul(h, dout, transa=True)  # h^T . dout  -> [5, 4]
+    db2 = oracle.reduce_cols("sum", dout)
+    dh = oracle.matmul(dout, w2, transb=True)  # dout . w2^T -> [1, 5]
+    dpre = oracle.binary("mul", oracle.binary("cmpgt", pre, np.float32(0)), dh)
+    dw1 = oracle.matmul(x, dpre, transa=True)
+    db1 = oracle.reduce_cols("sum", dpre)
+    assert dw1.tolist() == [[11528, 21316, 18580, 19872, 11476], [17292, 31974, 27870, 29808, 17214],
+                            [5764, 10658, 9290, 9936, 5738]]
+    assert db1.tolist() == [5764, 10658, 9290, 9936, 5738]
+    assert dw2.tolist() == [[11628, 5542, 16082, 10506], [18468, 8802, 25542, 16686], [11628, 5542, 16082, 10506],
+                            [17100, 8150, 23650, 15450], [15732, 7498, 21758, 14214]]
+    assert db2.tolist() == [684, 326, 946, 618]
+
+
+def test_mlp_step_decreases_loss_and_matches_finite_differences(oracle):
+    r = oracle.Rng(42069)
+    w1, b1 = r.uniform((16, 24), -0.2, 0.2), r.uniform(16, -0.2, 0.2)
+    w2, b2 = r.uniform((5, 16), -0.25, 0.25), r.uniform(5, -0.25, 0.25)
+    x, labels = r.randn((8, 24)), r.randint(8, 0, 5)
+    loss0, nw1, nb1, nw2, nb2, g = oracle.mlp_step(x, labels, w1, b1, w2, b2, 0.1)
+
+    def f(w1_, b1_, w2_, b2_):
+        h = np.maximum(x.astype(np.float64) @ w1_.T + b1_, 0)
+        z = h @ w2_.T + b2_
+        m = z - z.max(1, keepdims=True)
+        ls = m - np.log(np.exp(m).sum(1, keepdims=True))
+        return -(ls[np.arange(8), labels]).mean()
+
+    assert abs(loss0 - f(w1, b1, w2, b2)) < 1e-5
+    base = [a.astype(np.float64) for a in (w1, b1, w2, b2)]
+    for idx, name in enumerate(["w1", "b1", "w2", "b2"]):
+        flat = base[idx].reshape(-1)
+        for pos in range(0, flat.size, max(1, flat.size // 7)):
+            args_p = [a.copy() for a in base]
+            args_m = [a.copy() for a in base]
+            args_p[idx].reshape(-1)[pos] += 1e-5
+            args_m[idx].reshape(-1)[pos] -= 1e-5
+            num = (f(*args_p) - f(*args_m)) / 2e-5
+            assert abs(g[name].reshape(-1)[pos] - num) < 1e-4 * max(1.0, abs(num)), (name, pos)
+    loss1 = oracle.mlp_step(x, labels, nw1, nb1, nw2, nb2, 0.1)[0]
+    assert loss1 < loss0

@@ -130,7 +130,7 @@ _EXPORTS = ["zhip_device_count", "zhip_init", "zhip_deinit", "zhip_last_error", 
             "zhip_free_bytes", "zhip_free_compute", "zhip_alloc", "zhip_free", "zhip_store_variable",
             "zhip_get_variable", "zhip_h2d", "zhip_d2h", "zhip_d2d", "zhip_sync_events", "zhip_release_events",
             "zhip_buffer_ptr", "zhip_register_kernel", "zhip_compile_ir", "zhip_launch", "zhip_release_program",
-            "zhip_time_kernel", "zhip_profile_kernel"]
+            "zhip_time_kernel", "zhip_profile_kernel", "zhip_plan_create", "zhip_plan_launch", "zhip_plan_destroy"]
 
 
 def load_library() -> C.CDLL:
@@ -344,6 +344,28 @@ class HIPDevice:
         self._ctx.check(self._ctx.lib.zhip_time_kernel(self._ctx.ptr, C.c_uint32(program_id), a, C.c_size_t(len(args)),
                                                        C.byref(ns)))
         return ns.value
+
+    def create_plan(self, nodes: Sequence) -> int:
+        """Record a fixed list of Launch nodes [(program_id, [buffer ids: loads then stores]), ...] as
+        one replayable unit: the cached ExecPlan of zyx/src/graph/plan.rs:58-237 kept as a HIP graph."""
+        progs = (C.c_uint32 * len(nodes))(*[n[0] for n in nodes])
+        flat = [b for n in nodes for b in n[1]]
+        args = (C.c_uint32 * max(len(flat), 1))(*flat)
+        counts = (C.c_uint32 * len(nodes))(*[len(n[1]) for n in nodes])
+        plan = C.c_uint32()
+        self._ctx.check(self._ctx.lib.zhip_plan_create(self._ctx.ptr, progs, args, counts, C.c_size_t(len(nodes)),
+                                                       C.byref(plan)))
+        return plan.value
+
+    def launch_plan(self, plan_id: int, event_wait_list: Sequence[Event] = ()) -> Event:
+        """execute_plan (zyx/src/graph/plan.rs:271-361) for a plan whose buffers are already allocated."""
+        arr, n = _events_array(event_wait_list)
+        ev = C.c_uint64()
+        self._ctx.check(self._ctx.lib.zhip_plan_launch(self._ctx.ptr, C.c_uint32(plan_id), arr, n, C.byref(ev)))
+        return Event(ev.value)
+
+    def destroy_plan(self, plan_id: int):
+        self._ctx.check(self._ctx.lib.zhip_plan_destroy(self._ctx.ptr, C.c_uint32(plan_id)))
 
     def profile_kernel(self, program_id: int, arg_sets: Sequence[Sequence[int]], iters: int) -> float:
         """Mean device microseconds per launch, HIP events on the launch stream."""

@@ -312,17 +312,8 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
 template <bool AT, bool BT> hipError_t launch_epi(const GemmBf16 &p, hipStream_t st) {
     dim3 grid((unsigned)((p.M / BM) * (p.N / BN))), block(256);
 #define ZK_GEMM(E)                                                                                                    \
-    {                                                                                                                 \
-        auto k = gemm_bf16_k<AT, BT, E>;                                                                              \
-        static bool attr_set = false;                                                                                 \
-        if (!attr_set) {                                                                                              \
-            hipError_t e = hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS); \
-            if (e != hipSuccess) return e;                                                                            \
-            attr_set = true;                                                                                          \
-        }                                                                                                             \
-        hipLaunchKernelGGL(k, grid, block, GEMM_LDS, st, (const uint16_t *)p.A, (const uint16_t *)p.B, (float *)p.C,  \
-                           p.bias, p.bias_dtype, (int)p.M, (int)p.N, (int)p.K);                                       \
-    }
+    hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E>), grid, block, GEMM_LDS, st, (const uint16_t *)p.A,                    \
+                       (const uint16_t *)p.B, (float *)p.C, p.bias, p.bias_dtype, (int)p.M, (int)p.N, (int)p.K);
     switch (p.epilogue) {
     case 0: ZK_GEMM(0) break;
     case 1: ZK_GEMM(1) break;
@@ -334,7 +325,28 @@ template <bool AT, bool BT> hipError_t launch_epi(const GemmBf16 &p, hipStream_t
     return hipGetLastError();
 }
 
+template <bool AT, bool BT, int E> hipError_t allow_lds() {
+    return hipFuncSetAttribute((const void *)gemm_bf16_k<AT, BT, E>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS);
+}
+template <bool AT, bool BT> hipError_t allow_lds_epi() {
+    hipError_t e;
+    if ((e = allow_lds<AT, BT, 0>()) != hipSuccess) return e;
+    if ((e = allow_lds<AT, BT, 1>()) != hipSuccess) return e;
+    if ((e = allow_lds<AT, BT, 2>()) != hipSuccess) return e;
+    return allow_lds<AT, BT, 3>();
+}
+
 } // namespace
+
+// The kernels use 128 KiB of dynamic LDS, above the default per-workgroup limit: raise it
+// once per device (the attribute lives with the device's copy of the code object).
+hipError_t gemm_bf16_init() {
+    hipError_t e;
+    if ((e = allow_lds_epi<false, false>()) != hipSuccess) return e;
+    if ((e = allow_lds_epi<false, true>()) != hipSuccess) return e;
+    if ((e = allow_lds_epi<true, false>()) != hipSuccess) return e;
+    return allow_lds_epi<true, true>();
+}
 
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K) {
     return M > 0 && N > 0 && K > 0 && M % BM == 0 && N % BN == 0 && K % BK == 0 && M < (1 << 30) && N < (1 << 30) &&

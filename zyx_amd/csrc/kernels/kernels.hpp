@@ -56,6 +56,7 @@ struct GemmBf16 {
     void *C;
 };
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K);
+hipError_t gemm_bf16_init(); // once per device, before the first launch
 hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t stream);
 
 // Any-shape GEMM: dtype F32 / BF16 / F16 operands, f32 accumulate, C stored as F32 or as
@@ -72,5 +73,26 @@ struct GemmGeneric {
     void *C;
 };
 hipError_t gemm_generic(const GemmGeneric &p, hipStream_t stream);
+
+// LayerNorm (rms == 0) / RMSNorm (rms == 1) over the last axis; w, b may be null.
+struct NormRows {
+    int64_t rows, cols;
+    int dtype; // DT_F32 or DT_BF16 storage of x, w, b, y
+    int rms;
+    float eps;
+    const void *x, *w, *b;
+    void *y;
+};
+hipError_t norm_rows(const NormRows &p, hipStream_t stream);
+
+// cross_entropy of f32 logits [rows, cols] with i32 class indices; loss / grad may be null.
+struct CrossEntropy {
+    int64_t rows, cols;
+    float gscale;
+    const float *x;
+    const int32_t *labels;
+    float *loss, *grad;
+};
+hipError_t cross_entropy(const CrossEntropy &p, hipStream_t stream);
 
 } // namespace zk

@@ -69,6 +69,13 @@ struct Program {
     uint64_t workspace_bytes = 0;
 };
 
+struct Plan {
+    bool live = false;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    size_t n_nodes = 0;
+};
+
 template <class T> struct Slab { // dense ids, lowest free id reused (zyx/src/slab.rs)
     std::vector<T> items;
     std::vector<uint32_t> free_ids;
@@ -101,7 +108,7 @@ struct zhip_ctx {
 
     hipStream_t pool_stream = nullptr;
     hipStream_t launch_streams[kLaunchStreams] = {nullptr};
-    uint64_t stream_seq[kLaunchStreams + 1] = {0}; // [kLaunchStreams] = pool stream
+    uint64_t stream_seq[kLaunchStreams + 2] = {0}; // [kLaunchStreams] = pool stream, [+1] = plan stream
     int rr = 0;
 
     uint64_t free_bytes = 0;
@@ -111,6 +118,8 @@ struct zhip_ctx {
     std::vector<EventSlot> events;
     std::vector<uint32_t> free_events;
     Slab<Program> programs;
+    Slab<Plan> plans;
+    hipStream_t plan_stream = nullptr; // plans are captured on and replayed into this stream
     hipEvent_t prof_a = nullptr, prof_b = nullptr;
 
     int32_t fail(int32_t status, const char *fmt, ...) __attribute__((format(printf, 3, 4))) {
@@ -142,7 +151,10 @@ uint64_t size_class(uint64_t bytes) {
     return (bytes + step - 1) / step * step;
 }
 
-hipStream_t stream_of(zhip_ctx *c, int idx) { return idx < 0 ? c->pool_stream : c->launch_streams[idx]; }
+// stream index: 0..7 launch streams, -1 pool stream, -2 plan stream
+hipStream_t stream_of(zhip_ctx *c, int idx) {
+    return idx == -1 ? c->pool_stream : idx == -2 ? c->plan_stream : c->launch_streams[idx];
+}
 
 // --- events ---------------------------------------------------------------------
 EventSlot *event_lookup(zhip_ctx *c, zhip_event h) {
@@ -171,7 +183,7 @@ int32_t event_record(zhip_ctx *c, int stream_idx, int32_t status, zhip_event *ou
     }
     s.live = true;
     s.stream = (int16_t)stream_idx;
-    s.seq = ++c->stream_seq[stream_idx < 0 ? kLaunchStreams : stream_idx];
+    s.seq = ++c->stream_seq[stream_idx == -1 ? kLaunchStreams : stream_idx == -2 ? kLaunchStreams + 1 : stream_idx];
     *out = ((uint64_t)s.gen << 32) | (uint64_t)(idx + 1);
     return ZHIP_OK;
 }
@@ -336,6 +348,37 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.n_out = 1;
         return ZHIP_OK;
     }
+    case ZHIP_K_NORM_ROWS: {
+        int64_t rows = d.dims[0], cols = d.dims[1];
+        if (rows < 0 || cols < 0 || cols >= (1ll << 31) || (cols && rows > (1ll << 40) / cols))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "norm_rows: rows/cols out of range");
+        if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16) return c->fail(ZHIP_KERNEL_COMPILATION, "norm_rows: dtype must be F32 or BF16");
+        if (d.flags & ~7) return c->fail(ZHIP_KERNEL_COMPILATION, "norm_rows: bad flags");
+        uint64_t e = dtype_bytes(d.dtype);
+        int a = 0;
+        p.need[a++] = (uint64_t)rows * cols * e;
+        if (d.flags & ZHIP_NORM_WEIGHT) p.need[a++] = (uint64_t)cols * e;
+        if (d.flags & ZHIP_NORM_BIAS) p.need[a++] = (uint64_t)cols * e;
+        p.n_in = a;
+        p.need[a] = (uint64_t)rows * cols * e;
+        p.n_out = 1;
+        return ZHIP_OK;
+    }
+    case ZHIP_K_CROSS_ENTROPY: {
+        int64_t rows = d.dims[0], cols = d.dims[1];
+        if (rows < 0 || cols < 0 || cols >= (1ll << 31) || (cols && rows > (1ll << 40) / cols))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "cross_entropy: rows/cols out of range");
+        if (d.dtype != ZHIP_F32) return c->fail(ZHIP_KERNEL_COMPILATION, "cross_entropy: logits must be F32");
+        if ((d.flags & 3) == 0 || (d.flags & ~3)) return c->fail(ZHIP_KERNEL_COMPILATION, "cross_entropy: bad output flags");
+        p.n_in = 2;
+        p.need[0] = (uint64_t)rows * cols * 4;
+        p.need[1] = (uint64_t)rows * 4;
+        int o = 2;
+        if (d.flags & ZHIP_CE_LOSS) p.need[o++] = (uint64_t)rows * 4;
+        if (d.flags & ZHIP_CE_GRAD) p.need[o++] = (uint64_t)rows * cols * 4;
+        p.n_out = o - 2;
+        return ZHIP_OK;
+    }
     default: return c->fail(ZHIP_KERNEL_COMPILATION, "unknown kernel kind %d", d.kind);
     }
 }
@@ -426,6 +469,32 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         g.bias = g.epilogue ? ptr[2] : nullptr;
         g.C = ptr[p.n_in];
         return zk::gemm_generic(g, st);
+    }
+    case ZHIP_K_NORM_ROWS: {
+        zk::NormRows a{};
+        a.rows = d.dims[0];
+        a.cols = d.dims[1];
+        a.dtype = d.dtype;
+        a.rms = d.flags & ZHIP_NORM_RMS ? 1 : 0;
+        a.eps = d.fparams[0];
+        int i = 0;
+        a.x = ptr[i++];
+        if (d.flags & ZHIP_NORM_WEIGHT) a.w = ptr[i++];
+        if (d.flags & ZHIP_NORM_BIAS) a.b = ptr[i++];
+        a.y = ptr[i];
+        return zk::norm_rows(a, st);
+    }
+    case ZHIP_K_CROSS_ENTROPY: {
+        zk::CrossEntropy a{};
+        a.rows = d.dims[0];
+        a.cols = d.dims[1];
+        a.gscale = d.fparams[0];
+        a.x = (const float *)ptr[0];
+        a.labels = (const int32_t *)ptr[1];
+        int o = 2;
+        if (d.flags & ZHIP_CE_LOSS) a.loss = (float *)ptr[o++];
+        if (d.flags & ZHIP_CE_GRAD) a.grad = (float *)ptr[o++];
+        return zk::cross_entropy(a, st);
     }
     default: return hipErrorInvalidValue;
     }
@@ -563,8 +632,11 @@ ZHIP_EXPORT int32_t zhip_init(const zhip_config *cfg, zhip_ctx **out) {
     for (int i = 0; i < kLaunchStreams; i++)
         if ((e = hipStreamCreateWithFlags(&c->launch_streams[i], hipStreamNonBlocking)) != hipSuccess)
             return bail(ZHIP_INITIALIZATION, "hipStreamCreate", e);
+    if ((e = hipStreamCreateWithFlags(&c->plan_stream, hipStreamNonBlocking)) != hipSuccess)
+        return bail(ZHIP_INITIALIZATION, "hipStreamCreate", e);
     if ((e = hipEventCreate(&c->prof_a)) != hipSuccess || (e = hipEventCreate(&c->prof_b)) != hipSuccess)
         return bail(ZHIP_INITIALIZATION, "hipEventCreate", e);
+    if ((e = zk::gemm_bf16_init()) != hipSuccess) return bail(ZHIP_INITIALIZATION, "raising the LDS limit of the GEMM kernels", e);
     fill_info(c);
     if (c->debug & 1)
         fprintf(stderr, "[zyx-hip] device %d: %s (%s), %u CUs, %.1f GiB free\n", c->device, c->info.name, c->info.arch,
@@ -580,6 +652,13 @@ ZHIP_EXPORT int32_t zhip_deinit(zhip_ctx *c) {
         (void)hipSetDevice(c->device);
         (void)hipStreamSynchronize(c->pool_stream);
         for (auto s : c->launch_streams) (void)hipStreamSynchronize(s);
+        (void)hipStreamSynchronize(c->plan_stream);
+        for (Plan &pl : c->plans.items)
+            if (pl.live) {
+                (void)hipGraphExecDestroy(pl.exec);
+                (void)hipGraphDestroy(pl.graph);
+            }
+        (void)hipStreamDestroy(c->plan_stream);
         trim_cache(c, 0);
         for (Buffer &b : c->buffers.items)
             if (b.kind == Buffer::Memory) (void)hipFree(b.ptr);
@@ -895,5 +974,71 @@ ZHIP_EXPORT int32_t zhip_profile_kernel(zhip_ctx *c, zhip_prog prog, const zhip_
     float ms = 0.0f;
     HIPCHK(c, hipEventElapsedTime(&ms, c->prof_a, c->prof_b), ZHIP_KERNEL_SYNC);
     *avg_us = ms * 1000.0f / (float)iters;
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_plan_create(zhip_ctx *c, const zhip_prog *progs, const zhip_buf *args_flat, const uint32_t *n_args,
+                                     size_t n_nodes, zhip_plan *plan) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!progs || !args_flat || !n_args || !plan || n_nodes == 0) return c->fail(ZHIP_KERNEL_COMPILATION, "plan_create: bad argument");
+    *plan = ZHIP_NULL_ID;
+    // resolve every node before anything is captured: a bad node must not leave a capture open
+    std::vector<Program *> ps(n_nodes);
+    std::vector<void *> ptrs(n_nodes * 8, nullptr);
+    size_t off = 0;
+    for (size_t i = 0; i < n_nodes; i++) {
+        int32_t rc = resolve_args(c, progs[i], args_flat + off, n_args[i], &ps[i], &ptrs[i * 8]);
+        if (rc != ZHIP_OK) return rc;
+        off += n_args[i];
+    }
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_COMPILATION);
+    HIPCHK(c, hipStreamSynchronize(c->plan_stream), ZHIP_KERNEL_SYNC);
+    HIPCHK(c, hipStreamBeginCapture(c->plan_stream, hipStreamCaptureModeThreadLocal), ZHIP_KERNEL_COMPILATION);
+    hipError_t bad = hipSuccess;
+    for (size_t i = 0; i < n_nodes && bad == hipSuccess; i++) bad = program_enqueue(*ps[i], &ptrs[i * 8], c->plan_stream);
+    Plan pl;
+    hipError_t e = hipStreamEndCapture(c->plan_stream, &pl.graph);
+    if (bad != hipSuccess || e != hipSuccess) {
+        if (pl.graph) (void)hipGraphDestroy(pl.graph);
+        (void)hipGetLastError();
+        return c->fail(ZHIP_KERNEL_COMPILATION, "plan capture failed: %s", hipGetErrorString(bad != hipSuccess ? bad : e));
+    }
+    e = hipGraphInstantiate(&pl.exec, pl.graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(pl.graph);
+        return c->fail(ZHIP_KERNEL_COMPILATION, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    }
+    pl.live = true;
+    pl.n_nodes = n_nodes;
+    *plan = c->plans.push(pl);
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_plan_launch(zhip_ctx *c, zhip_plan plan, const zhip_event *evs, size_t n_evs, zhip_event *ev) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!ev) return c->fail(ZHIP_KERNEL_LAUNCH, "plan_launch: null event out pointer");
+    *ev = 0;
+    if (plan >= c->plans.items.size() || !c->plans.items[plan].live) {
+        for (size_t i = 0; i < n_evs; i++)
+            if (EventSlot *s = event_lookup(c, evs[i])) event_retire(c, s);
+        return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "plan %u does not exist", plan);
+    }
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
+    int32_t rc = wait_and_consume(c, -2, evs, n_evs, ZHIP_KERNEL_LAUNCH);
+    if (rc != ZHIP_OK) return rc;
+    HIPCHK(c, hipGraphLaunch(c->plans.items[plan].exec, c->plan_stream), ZHIP_KERNEL_LAUNCH);
+    return event_record(c, -2, ZHIP_KERNEL_LAUNCH, ev);
+}
+
+ZHIP_EXPORT int32_t zhip_plan_destroy(zhip_ctx *c, zhip_plan plan) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (plan >= c->plans.items.size() || !c->plans.items[plan].live) return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "plan %u does not exist", plan);
+    Plan &pl = c->plans.items[plan];
+    (void)hipSetDevice(c->device);
+    (void)hipStreamSynchronize(c->plan_stream);
+    (void)hipGraphExecDestroy(pl.exec);
+    (void)hipGraphDestroy(pl.graph);
+    pl = Plan();
+    c->plans.remove(plan);
     return ZHIP_OK;
 }

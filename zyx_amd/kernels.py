@@ -224,3 +224,70 @@ def gemm(dev: HIPDevice, pool: HIPMemoryPool, a: np.ndarray, b: np.ndarray, bias
         pool.deallocate(bb, [])
     dev.release(prog)
     return res
+
+
+# ---- LayerNorm / RMSNorm (ZHIP_K_NORM_ROWS), cross entropy (ZHIP_K_CROSS_ENTROPY) --------------------
+K_NORM_ROWS, K_CROSS_ENTROPY = 5, 6
+NORM_RMS, NORM_WEIGHT, NORM_BIAS = 1, 2, 4
+CE_LOSS, CE_GRAD = 1, 2
+
+
+def norm_rows_desc(rows: int, cols: int, rms=False, weight=True, bias=True, eps=1e-5, dtype: DType = DType.F32) -> KernelDesc:
+    d = KernelDesc()
+    d.kind, d.dtype, d.out_dtype = K_NORM_ROWS, DType(dtype), DType(dtype)
+    d.flags = (NORM_RMS if rms else 0) | (NORM_WEIGHT if weight else 0) | (NORM_BIAS if bias and not rms else 0)
+    d.dims[0], d.dims[1] = rows, cols
+    d.fparams[0] = eps
+    return d
+
+
+def norm_rows(dev: HIPDevice, pool: HIPMemoryPool, x, w=None, b=None, rms=False, eps=1e-5, dtype: DType = DType.F32):
+    """LayerNorm::forward / RMSNorm::forward over the last axis of x[rows, cols]."""
+    st = _NP_STORE[DType(dtype)]
+    x = np.ascontiguousarray(x, st)
+    rows, cols = x.shape
+    prog = dev.register_kernel(norm_rows_desc(rows, cols, rms, w is not None, b is not None, eps, dtype))
+    bufs, waits = [], []
+    for arr in [x] + [np.ascontiguousarray(a, st) for a in (w, b) if a is not None]:
+        bb, e = to_device(pool, arr)
+        bufs.append(bb)
+        waits.append(e)
+    yb, e = alloc_like(pool, rows * cols, x.itemsize)
+    done = dev.launch(prog, pool, bufs + [yb], waits + [e])
+    y = to_host(pool, yb, (rows, cols), st, [done])
+    for bb in bufs + [yb]:
+        pool.deallocate(bb, [])
+    dev.release(prog)
+    return y
+
+
+def cross_entropy_desc(rows: int, cols: int, loss=True, grad=False, gscale: float = 1.0) -> KernelDesc:
+    d = KernelDesc()
+    d.kind, d.dtype, d.out_dtype = K_CROSS_ENTROPY, DType.F32, DType.F32
+    d.flags = (CE_LOSS if loss else 0) | (CE_GRAD if grad else 0)
+    d.dims[0], d.dims[1] = rows, cols
+    d.fparams[0] = gscale
+    return d
+
+
+def cross_entropy(dev: HIPDevice, pool: HIPMemoryPool, logits, labels, grad_scale=None):
+    """-> (per-sample loss, grad or None); grad = d(grad_scale * sum(loss)) / d(logits)."""
+    x = np.ascontiguousarray(logits, np.float32)
+    lab = np.ascontiguousarray(labels, np.int32)
+    rows, cols = x.shape
+    prog = dev.register_kernel(cross_entropy_desc(rows, cols, True, grad_scale is not None, grad_scale or 0.0))
+    xb, e0 = to_device(pool, x)
+    lb, e1 = to_device(pool, lab)
+    ob, e2 = alloc_like(pool, rows, 4)
+    outs, waits = [ob], [e0, e1, e2]
+    if grad_scale is not None:
+        gb, e3 = alloc_like(pool, rows * cols, 4)
+        outs.append(gb)
+        waits.append(e3)
+    done = dev.launch(prog, pool, [xb, lb] + outs, waits)
+    loss = to_host(pool, ob, (rows,), np.float32, [done])
+    grad = to_host(pool, outs[1], (rows, cols), np.float32) if grad_scale is not None else None
+    for bb in [xb, lb] + outs:
+        pool.deallocate(bb, [])
+    dev.release(prog)
+    return loss, grad
