@@ -26,6 +26,10 @@ ROWS, COLS = 8192, 4096
 ALGO_BYTES = ROWS * COLS * 4 * 2 + 2 * ROWS * 4
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 N_SETS = 4              # 4 x 268 MB working set > Infinity Cache
+# HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
+# by the same counter's reading for a plain copy kernel of known size in the same run
+# (profiles/softmax_rows_f32_8192x4096.md): 134,054,270 B fetched + 134,320,107 B written.
+TRAFFIC_BYTES = 268374377
 
 
 def cpu_baseline(x: np.ndarray, budget_s: float = 10.0):
@@ -50,12 +54,94 @@ def cpu_baseline(x: np.ndarray, budget_s: float = 10.0):
                       f"(serial per-row loops as zyx's C backend emits), {best * 1e3:.1f} ms/pass"}
 
 
+def extra_gemm(dev, pool, kernels, steps=100, warmup=200):
+    """Config 3: bf16 4096^3 GEMM (f32 accumulate), raw and with the fused bias+GELU epilogue."""
+    n = 4096
+    rng = np.random.default_rng(1)
+    trunc = lambda a: (a.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)  # bf16 by truncation, as zyx does
+    a, b = trunc(rng.uniform(-1, 1, (n, n))), trunc(rng.uniform(-1, 1, (n, n)))
+    bias = trunc(rng.uniform(-1 / 64, 1 / 64, n))
+    ab, e1 = kernels.to_device(pool, a)
+    bb, e2 = kernels.to_device(pool, b)
+    biasb, e3 = kernels.to_device(pool, bias)
+    cb, e4 = pool.allocate(n * n * 4 + 4)
+    pool.sync_events([e1, e2, e3, e4])
+    out = {}
+    for name, epi in (("nn", "none"), ("nn_bias_gelu", "bias_gelu")):
+        prog = dev.register_kernel(kernels.gemm_desc(n, n, n, epilogue=epi, bias_dtype=zyx_dtype_bf16()))
+        args = [ab, bb] + ([biasb] if epi != "none" else []) + [cb]
+        dev.profile_kernel(prog, [args], warmup)  # also lets the clocks settle
+        us = dev.profile_kernel(prog, [args], steps)
+        tf = 2.0 * n**3 / us / 1e6
+        out[name] = {"avg_launch_us": round(us, 2), "TFLOP/s": round(tf, 1), "frac_of_2.5PF_bf16_peak": round(tf / 2500.0, 4)}
+        dev.release(prog)
+    for b_ in (ab, bb, biasb, cb):
+        pool.deallocate(b_, [])
+    return out
+
+
+def zyx_dtype_bf16():
+    import zyx_amd
+    return zyx_amd.DType.BF16
+
+
+def extra_mlp(dev, pool, steps=100, cpu=True):
+    """Config 1: MLP 784->128->10, batch 64, SGD 0.01, 100 steps; steps 10..99 timed. GPU: per step two
+    device-to-device batch copies out of the resident dataset and one cached plan launch (15 kernels)."""
+    from zyx_amd.training import MLPTrainStep
+    B, NIN, H, NOUT, LR = 64, 784, 128, 10, 0.01
+    rng = np.random.default_rng(42069)
+    k1, k2 = 1 / np.sqrt(NIN), 1 / np.sqrt(H)
+    w1, b1 = rng.uniform(-k1, k1, (H, NIN)).astype(np.float32), rng.uniform(-k1, k1, H).astype(np.float32)
+    w2, b2 = rng.uniform(-k2, k2, (NOUT, H)).astype(np.float32), rng.uniform(-k2, k2, NOUT).astype(np.float32)
+    xs = rng.standard_normal((steps, B, NIN), dtype=np.float32)
+    ys = rng.integers(0, NOUT, (steps, B)).astype(np.int32)
+    m = MLPTrainStep(dev, pool, B, NIN, H, NOUT, LR)
+    m.set_params(w1, b1, w2, b2)
+    from zyx_amd import kernels as K
+    xb, e1 = K.to_device(pool, xs)  # the whole synthetic dataset is resident in HBM before timing
+    yb, e2 = K.to_device(pool, ys)
+    pool.sync_events([e1, e2])
+    t0 = None
+    for i in range(steps):
+        if i == 10:
+            pool.sync_events(m._pending)
+            m._pending = []
+            t0 = time.perf_counter()
+        m.set_batch_from_device(xb, yb, i)
+        m.step()
+    final = m.mean_loss()  # blocks until the last step is done
+    gpu_sps = (steps - 10) / (time.perf_counter() - t0)
+    m.close()
+    pool.deallocate(xb, [])
+    pool.deallocate(yb, [])
+    res = {"gpu_steps_per_s": round(gpu_sps, 1), "kernels_per_step": 15, "final_loss": round(final, 5)}
+    if cpu:
+        import oracle
+        p = (w1, b1, w2, b2)
+        for i in range(steps):
+            if i == 10:
+                t0 = time.perf_counter()
+            loss, *p, _ = oracle.mlp_step(xs[i], ys[i], *p, LR)
+            p = tuple(p)
+        res["cpu_oracle_steps_per_s"] = round((steps - 10) / (time.perf_counter() - t0), 1)
+        res["cpu_final_loss"] = round(float(loss), 5)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="only the headline workload (used for profiling)")
+    ap.add_argument("--gemm-only", action="store_true",
+                    help="run only the config-3 GEMM leg and print its numbers (used for profiling that kernel)")
+    ap.add_argument("--counters", action="store_true",
+                    help="short run for `rocprofv3 --pmc`: a few launches of the fused kernel and of a plain copy "
+                         "kernel over the same 8192x4096 f32 tensor (known traffic: 134217728 B read + written), "
+                         "then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend drives one GPU per context and this build measures one GPU only; "
@@ -67,6 +153,11 @@ def main():
     pools, devices = zyx_amd.initialize_device(zyx_amd.HIPConfig(device_ids=[0]))
     pool, dev = pools[0], devices[0]
     info = dev.info()
+
+    if args.gemm_only:
+        print(json.dumps({"config3_gemm_bf16_4096": extra_gemm(dev, pool, kernels, steps=args.steps, warmup=max(args.warmup, 100))}))
+        pool.deinitialize()
+        return
 
     rng = np.random.default_rng(42069)
     x = (rng.standard_normal((ROWS, COLS), dtype=np.float32) * 3.0).astype(np.float32)
@@ -85,12 +176,27 @@ def main():
     pool.sync_events(pending)
 
     def run(n):
-        last = {}
+        # each step waits on the previous one: the chain stays on one in-order launch stream, so
+        # a profiler sees back-to-back, non-overlapping dispatches
+        ev = []
         for i in range(n):
-            s = i % N_SETS
-            ev = dev.launch(prog, pool, sets[s], [last[s]] if s in last else [])
-            last[s] = ev
-        pool.sync_events(list(last.values()))
+            ev = [dev.launch(prog, pool, sets[i % N_SETS], ev)]
+        pool.sync_events(ev)
+
+    if args.counters:
+        copy = kernels.Chain(ROWS, COLS)
+        copy.load(copy.input())
+        cprog = dev.register_kernel(copy.desc())
+        ev = []
+        for i in range(5):
+            ev = [dev.launch(prog, pool, sets[i % N_SETS], ev)]
+        for i in range(5):
+            ev = [dev.launch(cprog, pool, [sets[i % N_SETS][0], sets[(i + 1) % N_SETS][1]], ev)]
+        pool.sync_events(ev)
+        print(json.dumps({"counters_run": True, "softmax_launches": 5, "copy_launches": 5,
+                          "copy_bytes_read": ROWS * COLS * 4, "copy_bytes_written": ROWS * COLS * 4}))
+        pool.deinitialize()
+        return
 
     run(args.warmup)
     t0 = time.perf_counter()
@@ -118,13 +224,17 @@ def main():
                    "algorithmic_bytes_per_step": ALGO_BYTES, "device": info.name, "arch": info.arch,
                    "compute_units": info.compute_units},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES,
                      "kernel": "softmax_rows_wave_k<16>", "avg_launch_us": round(us, 3)},
     }
     for s in sets:
         for b in s:
             pool.deallocate(b, [])
     dev.release(prog)
+    if not args.no_extra:
+        # other configs of the same backend, reported beside the headline (not part of `value`)
+        out["extra"] = {"config3_gemm_bf16_4096": extra_gemm(dev, pool, kernels),
+                        "config1_mlp_train": extra_mlp(dev, pool, cpu=not args.no_cpu)}
     pool.deinitialize()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(x)

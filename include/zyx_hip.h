@@ -245,9 +245,10 @@ int32_t zhip_h2d(zhip_ctx *ctx, const void *src, uint64_t bytes, zhip_buf dst, c
  * Consumes evs. */
 int32_t zhip_d2h(zhip_ctx *ctx, zhip_buf src, void *dst, uint64_t bytes, const zhip_event *evs, size_t n_evs);
 /* MemoryPool::pool_to_pool with a device source (backend/mod.rs:743-764, todo!() for
- * HIP in the reference): device-to-device copy inside this pool. Consumes evs. */
-int32_t zhip_d2d(zhip_ctx *ctx, zhip_buf src, zhip_buf dst, uint64_t bytes, const zhip_event *evs, size_t n_evs,
-                 zhip_event *ev);
+ * HIP in the reference): device-to-device copy of `bytes` from src + src_offset to
+ * dst + dst_offset inside this pool. Consumes evs. */
+int32_t zhip_d2d(zhip_ctx *ctx, zhip_buf src, uint64_t src_offset, zhip_buf dst, uint64_t dst_offset, uint64_t bytes,
+                 const zhip_event *evs, size_t n_evs, zhip_event *ev);
 /* HIPMemoryPool::sync_events (hip.rs:440-448): wait, then destroy. */
 int32_t zhip_sync_events(zhip_ctx *ctx, const zhip_event *evs, size_t n_evs);
 /* HIPMemoryPool::release_events (hip.rs:451-458): destroy without waiting. */

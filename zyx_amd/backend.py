@@ -256,10 +256,20 @@ class HIPMemoryPool:
             arr, n = _events_array(event_wait_list)
             ev = C.c_uint64()
             nbytes = min(self.buffer_bytes(src), self.buffer_bytes(dst))
-            self._ctx.check(self._ctx.lib.zhip_d2d(self._ctx.ptr, C.c_uint32(src), C.c_uint32(dst), C.c_uint64(nbytes),
-                                                   arr, n, C.byref(ev)))
+            self._ctx.check(self._ctx.lib.zhip_d2d(self._ctx.ptr, C.c_uint32(src), C.c_uint64(0), C.c_uint32(dst),
+                                                   C.c_uint64(0), C.c_uint64(nbytes), arr, n, C.byref(ev)))
             return Event(ev.value)
         return self.host_to_pool(src, dst, event_wait_list)
+
+    def copy_range(self, src: int, src_offset: int, dst: int, dst_offset: int, nbytes: int,
+                   event_wait_list: Sequence[Event] = ()) -> Event:
+        """Device-to-device copy of a byte range between two buffers of this pool (the data movement a
+        narrowed / sliced view needs; the reference has no HIP pool_to_pool yet)."""
+        arr, n = _events_array(event_wait_list)
+        ev = C.c_uint64()
+        self._ctx.check(self._ctx.lib.zhip_d2d(self._ctx.ptr, C.c_uint32(src), C.c_uint64(src_offset), C.c_uint32(dst),
+                                               C.c_uint64(dst_offset), C.c_uint64(nbytes), arr, n, C.byref(ev)))
+        return Event(ev.value)
 
     def sync_events(self, events: Sequence[Event]):
         arr, n = _events_array(events)

@@ -815,8 +815,8 @@ ZHIP_EXPORT int32_t zhip_d2h(zhip_ctx *c, zhip_buf src, void *dst, uint64_t byte
     return ZHIP_OK;
 }
 
-ZHIP_EXPORT int32_t zhip_d2d(zhip_ctx *c, zhip_buf src, zhip_buf dst, uint64_t bytes, const zhip_event *evs, size_t n,
-                             zhip_event *ev) {
+ZHIP_EXPORT int32_t zhip_d2d(zhip_ctx *c, zhip_buf src, uint64_t src_off, zhip_buf dst, uint64_t dst_off, uint64_t bytes,
+                             const zhip_event *evs, size_t n, zhip_event *ev) {
     std::lock_guard<std::mutex> lk(c->mu);
     if (!ev) return c->fail(ZHIP_MEMORY_COPY_H2P, "zhip_d2d: null event out pointer");
     *ev = 0;
@@ -826,8 +826,12 @@ ZHIP_EXPORT int32_t zhip_d2d(zhip_ctx *c, zhip_buf src, zhip_buf dst, uint64_t b
     if (rc != ZHIP_OK) return rc;
     if (!s || !d || s->kind != Buffer::Memory || d->kind != Buffer::Memory)
         return c->fail(ZHIP_MEMORY_COPY_H2P, "d2d: buffers %u -> %u are not both device memory", src, dst);
-    if (bytes > s->bytes || bytes > d->bytes) return c->fail(ZHIP_MEMORY_COPY_H2P, "d2d: %llu bytes exceed a buffer", (unsigned long long)bytes);
-    if (bytes) HIPCHK(c, hipMemcpyAsync(d->ptr, s->ptr, bytes, hipMemcpyDeviceToDevice, c->pool_stream), ZHIP_MEMORY_COPY_H2P);
+    if (src_off > s->bytes || bytes > s->bytes - src_off || dst_off > d->bytes || bytes > d->bytes - dst_off)
+        return c->fail(ZHIP_MEMORY_COPY_H2P, "d2d: %llu bytes at offsets %llu -> %llu exceed a buffer", (unsigned long long)bytes,
+                       (unsigned long long)src_off, (unsigned long long)dst_off);
+    if (bytes)
+        HIPCHK(c, hipMemcpyAsync((char *)d->ptr + dst_off, (const char *)s->ptr + src_off, bytes, hipMemcpyDeviceToDevice, c->pool_stream),
+               ZHIP_MEMORY_COPY_H2P);
     return event_record(c, -1, ZHIP_MEMORY_COPY_H2P, ev);
 }
 

@@ -105,6 +105,15 @@ class MLPTrainStep:
         e2 = self.pool.host_to_pool(self._y, self._bufs["labels"], [])
         self._pending = [e1, e2]
 
+    def set_batch_from_device(self, x_buf: int, y_buf: int, index: int):
+        """Batch `index` of a dataset already resident in the pool (x_buf f32 [n, batch, n_in], y_buf i32
+        [n, batch]): two device-to-device range copies, as Tensor::index_select feeds batches in
+        zyx-examples/examples/mnist.rs:62-64."""
+        b, n_in, _, _ = self.shape
+        e1 = self.pool.copy_range(x_buf, index * b * n_in * 4, self._bufs["x"], 0, b * n_in * 4, self._pending)
+        e2 = self.pool.copy_range(y_buf, index * b * 4, self._bufs["labels"], 0, b * 4, [])
+        self._pending = [e1, e2]
+
     def step(self):
         """One forward + backward + update: a single plan launch."""
         ev = self.dev.launch_plan(self._plans[self._cur], self._pending)
