@@ -153,6 +153,17 @@ enum zhip_kernel_kind {
      * fparams[0] into grad[rows, cols] (fparams[0] = 1/rows for the Mean reduction).
      * args: logits, labels, (loss), (grad). */
     ZHIP_K_CROSS_ENTROPY = 6,
+    /* Tensor::conv for 4-D NCHW input, groups = 1 (zyx/src/tensor/mod.rs:2583-2680; layer
+     * zyx-nn/src/conv2d.rs:60-70): y[N,Cout,OH,OW] = x[N,C,H,W] (*) w[Cout,C,KH,KW] (+ bias[Cout])
+     * (then ReLU), zero padding, OH = (H + 2*py - dy*(KH-1) - 1) / sy + 1 (OW likewise).
+     * dims = {N, C, H, W, Cout, KH, KW}; iparams = {sy, sx, py, px, dy, dx, has_bias, relu};
+     * dtype F32 or BF16 for x, w, bias; out_dtype = dtype, or F32 for BF16 operands. Products
+     * and sums are f32. args: x, w, (bias), y. */
+    ZHIP_K_CONV2D = 7,
+    /* Tensor::max_pool over the last two axes (zyx/src/tensor/mod.rs:2706-2741): padding counts
+     * as the dtype's lowest value. dims = {planes (product of the leading axes), H, W, KH, KW};
+     * iparams = {sy, sx, py, px, dy, dx}; dtype F32 or BF16. args: x, y[planes, OH, OW]. */
+    ZHIP_K_MAX_POOL2D = 8,
     ZHIP_K_COUNT_
 };
 #define ZHIP_SOFTMAX_Y 1

@@ -310,3 +310,32 @@ def mlp_step(x, labels, w1, b1, w2, b2, lr: float):
     grads = dict(w1=dw1, b1=db1, w2=dw2, b2=db2, logits=dlogits)
     mean_loss = np.float32(reduce_rows("sum", loss[None, :])[0] / np.float32(n))
     return mean_loss, upd(w1, dw1), upd(b1[None, :], db1[None, :])[0], upd(w2, dw2), upd(b2[None, :], db2[None, :])[0], grads
+
+
+def conv2d(x, w, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1), relu=False, dtype: int = F32,
+           out_dtype: int | None = None) -> np.ndarray:
+    """Tensor::conv on NCHW x and weight [Cout, C, KH, KW], groups = 1."""
+    out_dtype = dtype if out_dtype is None else out_dtype
+    x = np.ascontiguousarray(x, _store_dtype(dtype))
+    w = np.ascontiguousarray(w, _store_dtype(dtype))
+    b = None if bias is None else np.ascontiguousarray(bias, _store_dtype(dtype))
+    n, c, h, wd = x.shape
+    co, _, kh, kw = w.shape
+    oh = (h + 2 * padding[0] - dilation[0] * (kh - 1) - 1) // stride[0] + 1
+    ow = (wd + 2 * padding[1] - dilation[1] * (kw - 1) - 1) // stride[1] + 1
+    y = np.empty((n, co, oh, ow), _store_dtype(out_dtype))
+    lib().zo_conv2d(dtype, out_dtype, _p(x), _p(w), _p(b), _p(y), _I64(n), _I64(c), _I64(h), _I64(wd), _I64(co), _I64(kh),
+                    _I64(kw), stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1], int(relu))
+    return y
+
+
+def max_pool2d(x, kernel=(2, 2), stride=(2, 2), padding=(0, 0), dilation=(1, 1), dtype: int = F32) -> np.ndarray:
+    x = np.ascontiguousarray(x, _store_dtype(dtype))
+    h, wd = x.shape[-2:]
+    planes = x.size // (h * wd)
+    oh = (h + 2 * padding[0] - dilation[0] * (kernel[0] - 1) - 1) // stride[0] + 1
+    ow = (wd + 2 * padding[1] - dilation[1] * (kernel[1] - 1) - 1) // stride[1] + 1
+    y = np.empty(x.shape[:-2] + (oh, ow), x.dtype)
+    lib().zo_max_pool2d(dtype, _p(x), _p(y), _I64(planes), _I64(h), _I64(wd), _I64(kernel[0]), _I64(kernel[1]), stride[0],
+                        stride[1], padding[0], padding[1], dilation[0], dilation[1])
+    return y

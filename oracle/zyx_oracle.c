@@ -672,3 +672,64 @@ ZO_API void zo_cross_entropy(const float *x, const int32_t *labels, float *loss,
         if (loss) loss[r] = l;
     }
 }
+
+/* ------------------------------------------------------------------------- */
+/* conv2d and max-pool                                                        */
+/* ------------------------------------------------------------------------- */
+
+/* Tensor::conv (zyx/src/tensor/mod.rs:2583-2680), 4-D NCHW, groups = 1. The reference pads,
+ * takes the pool view [bs, 1, cin, 1, oy, ox, ky, kx], multiplies by the weight and sums over
+ * (cin, ky, kx) with one serial f32 register accumulator in that order, then adds the bias.
+ * Padding is a 0/1 mask multiplied onto a clamped load (zyx/src/kernel/linearize.rs:349-382):
+ * for finite inputs that is a zero tap. Restated here as the direct cross-correlation that
+ * view reduces to -- the config-4 shape itself is pinned only by this textbook form. */
+ZO_API void zo_conv2d(int dtype, int out_dtype, const void *x, const void *w, const void *bias, void *y, int64_t N,
+                      int64_t C, int64_t H, int64_t W, int64_t Co, int64_t KH, int64_t KW, int sy, int sx, int py, int px,
+                      int dy, int dx, int relu) {
+    int64_t OH = (H + 2 * py - dy * (KH - 1) - 1) / sy + 1, OW = (W + 2 * px - dx * (KW - 1) - 1) / sx + 1;
+#pragma omp parallel for collapse(2)
+    for (int64_t n = 0; n < N; n++)
+        for (int64_t co = 0; co < Co; co++)
+            for (int64_t oy = 0; oy < OH; oy++)
+                for (int64_t ox = 0; ox < OW; ox++) {
+                    float acc = 0.0f;
+                    for (int64_t c = 0; c < C; c++)
+                        for (int64_t ky = 0; ky < KH; ky++)
+                            for (int64_t kx = 0; kx < KW; kx++) {
+                                int64_t iy = oy * sy - py + ky * dy, ix = ox * sx - px + kx * dx;
+                                int ok = iy >= 0 && iy < H && ix >= 0 && ix < W;
+                                float xv = ok ? load_as_f32(x, dtype, ((n * C + c) * H + iy) * W + ix) : 0.0f;
+                                acc = xv * load_as_f32(w, dtype, ((co * C + c) * KH + ky) * KW + kx) + acc;
+                            }
+                    /* a 16-bit sum is stored (truncated) before the bias is added to it in a second kernel */
+                    if (bias) {
+                        if (dtype != ZO_F32 && out_dtype != ZO_F32) {
+                            uint16_t t = dtype == ZO_BF16 ? bf16_store(acc) : f16_store(acc);
+                            acc = dtype == ZO_BF16 ? bf16_load(t) : f16_load(t);
+                        }
+                        acc = acc + load_as_f32(bias, dtype, co);
+                    }
+                    if (relu) acc = (float)(acc > 0.0f) * acc;
+                    store_from_f32(y, out_dtype, ((n * Co + co) * OH + oy) * OW + ox, acc);
+                }
+}
+
+/* Tensor::max_pool (zyx/src/tensor/mod.rs:2706-2741): pad with dtype.min, window view, max. */
+ZO_API void zo_max_pool2d(int dtype, const void *x, void *y, int64_t planes, int64_t H, int64_t W, int64_t KH, int64_t KW,
+                          int sy, int sx, int py, int px, int dy, int dx) {
+    int64_t OH = (H + 2 * py - dy * (KH - 1) - 1) / sy + 1, OW = (W + 2 * px - dx * (KW - 1) - 1) / sx + 1;
+    float lowest = dtype == ZO_F32 ? -FLT_MAX : bf16_load(0xff7f);
+#pragma omp parallel for
+    for (int64_t pl = 0; pl < planes; pl++)
+        for (int64_t oy = 0; oy < OH; oy++)
+            for (int64_t ox = 0; ox < OW; ox++) {
+                float m = lowest;
+                for (int64_t ky = 0; ky < KH; ky++)
+                    for (int64_t kx = 0; kx < KW; kx++) {
+                        int64_t iy = oy * sy - py + ky * dy, ix = ox * sx - px + kx * dx;
+                        float v = (iy >= 0 && iy < H && ix >= 0 && ix < W) ? load_as_f32(x, dtype, (pl * H + iy) * W + ix) : lowest;
+                        m = fmaxf(v, m);
+                    }
+                store_from_f32(y, dtype, (pl * OH + oy) * OW + ox, m);
+            }
+}

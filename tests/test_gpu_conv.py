@@ -1,0 +1,98 @@
+"""conv2d (+bias, +ReLU) and max-pool on the GPU vs the CPU oracle. f32: 1e-5 relative to
+sum |x w| over the receptive field (the scale of any summation order's rounding); bf16: the
+f32 sum is truncated to bf16, so results agree to one bf16 unit (plus 1e-3 of that scale).
+Max-pool is exact. Goldens: zyx/tests/05_misc.rs:880-888 (conv1), :85-109 (test_max_pool)."""
+import numpy as np
+import pytest
+
+from zyx_amd import DType
+from zyx_amd.kernels import conv2d, max_pool2d
+
+pytestmark = pytest.mark.gpu
+
+
+def test_reference_goldens(hip):
+    dev, pool = hip
+    t = np.arange(9, dtype=np.float32).reshape(1, 1, 3, 3)
+    assert conv2d(dev, pool, t, np.ones((1, 1, 2, 2), np.float32)).tolist() == [[[[8.0, 12.0], [20.0, 24.0]]]]
+    x = np.arange(1, 17, dtype=np.float32).reshape(1, 1, 4, 4)
+    assert max_pool2d(dev, pool, x).tolist() == [[[[6.0, 8.0], [14.0, 16.0]]]]
+
+
+CASES = [
+    # n, c, h, w, cout, kh, kw, stride, pad, dil
+    (2, 3, 9, 11, 4, 3, 2, (1, 1), (1, 1), (1, 1)),
+    (2, 3, 9, 11, 4, 3, 2, (2, 1), (0, 2), (1, 1)),
+    (1, 5, 12, 10, 70, 3, 3, (1, 2), (2, 1), (2, 2)),
+    (3, 16, 14, 14, 33, 1, 1, (1, 1), (0, 0), (1, 1)),
+    (2, 64, 28, 28, 128, 3, 3, (1, 1), (1, 1), (1, 1)),
+    (1, 7, 5, 5, 3, 5, 5, (1, 1), (2, 2), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_conv_f32(hip, oracle, case):
+    dev, pool = hip
+    n, c, h, w, co, kh, kw, stride, pad, dil = case
+    r = oracle.Rng(c * 100 + co)
+    x, wt, b = r.randn((n, c, h, w)), r.randn((co, c, kh, kw), float(np.sqrt(2.0 / (c * kh * kw)))), r.randn(co, 0.1)
+    for bias, relu in ((None, False), (b, False), (b, True)):
+        got = conv2d(dev, pool, x, wt, bias, stride, pad, dil, relu)
+        want = oracle.conv2d(x, wt, bias, stride, pad, dil, relu)
+        mag = oracle.conv2d(np.abs(x), np.abs(wt), None if bias is None else np.abs(b), stride, pad, dil)
+        assert got.shape == want.shape
+        assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), np.max(np.abs(got - want) / (mag + 1e-30))
+
+
+def test_conv_relu_pool_config4_slice(hip, oracle):
+    """Config 4 geometry (C=64, 56x56, 3x3, 128 output channels, stride 1, pad 1, Kaiming-normal
+    weights, ReLU, 2x2 max-pool) on a batch of 2 -- the oracle needs ~0.5 s per image."""
+    dev, pool = hip
+    r = oracle.Rng(42069)
+    x, wt = r.randn((2, 64, 56, 56)), r.randn((128, 64, 3, 3), float(np.sqrt(2.0 / 576)))
+    y, pooled = conv2d(dev, pool, x, wt, None, (1, 1), (1, 1), (1, 1), relu=True, pool_kernel=(2, 2))
+    want = oracle.conv2d(x, wt, None, (1, 1), (1, 1), (1, 1), relu=True)
+    mag = oracle.conv2d(np.abs(x), np.abs(wt), None, (1, 1), (1, 1), (1, 1))
+    assert np.all(np.abs(y - want) <= 2e-5 * mag)
+    assert np.array_equal(pooled, oracle.max_pool2d(y))  # pooling the GPU's own conv output is exact
+    assert pooled.shape == (2, 128, 28, 28) and pooled.min() >= 0
+
+
+def test_conv_full_batch_linearity(hip, oracle):
+    """Full config-4 size (N=32): checked through properties instead of the CPU oracle --
+    conv(x, w1 + w2) == conv(x, w1) + conv(x, w2) and batch independence."""
+    dev, pool = hip
+    r = oracle.Rng(1)
+    x = r.randn((32, 64, 56, 56))
+    w1, w2 = r.randn((128, 64, 3, 3), 0.05), r.randn((128, 64, 3, 3), 0.05)
+    y1 = conv2d(dev, pool, x, w1, None, (1, 1), (1, 1))
+    y2 = conv2d(dev, pool, x, w2, None, (1, 1), (1, 1))
+    y12 = conv2d(dev, pool, x, w1 + w2, None, (1, 1), (1, 1))
+    assert y12.shape == (32, 128, 56, 56)
+    assert np.allclose(y12, y1 + y2, rtol=1e-4, atol=2e-4)
+    ysub = conv2d(dev, pool, x[5:7], w1, None, (1, 1), (1, 1))
+    assert np.array_equal(ysub, y1[5:7])
+
+
+def test_conv_bf16(hip, oracle):
+    dev, pool = hip
+    r = oracle.Rng(3)
+    x, wt, b = (oracle.f32_to_bf16(a) for a in (r.randn((2, 16, 20, 20)), r.randn((24, 16, 3, 3), 0.1), r.randn(24, 0.1)))
+    got = conv2d(dev, pool, x, wt, b, (1, 1), (1, 1), (1, 1), relu=True, dtype=DType.BF16)
+    want = oracle.conv2d(x, wt, b, (1, 1), (1, 1), (1, 1), True, oracle.BF16)
+    g, wv = oracle.bf16_to_f32(got), oracle.bf16_to_f32(want)
+    mag = oracle.conv2d(np.abs(oracle.bf16_to_f32(x)), np.abs(oracle.bf16_to_f32(wt)), np.abs(oracle.bf16_to_f32(b)), (1, 1), (1, 1))
+    assert np.all(np.abs(g - wv) <= 2.0 ** -7 * np.abs(wv) + 1e-3 * mag)
+    got32 = conv2d(dev, pool, x, wt, None, (1, 1), (1, 1), (1, 1), dtype=DType.BF16, out_dtype=DType.F32)
+    want32 = oracle.conv2d(x, wt, None, (1, 1), (1, 1), (1, 1), False, oracle.BF16, oracle.F32)
+    assert np.all(np.abs(got32 - want32) <= 1e-3 * np.abs(want32) + 2e-5 * mag)
+
+
+@pytest.mark.parametrize("args", [((2, 2), (2, 2), (0, 0), (1, 1)), ((3, 3), (2, 2), (1, 1), (1, 1)),
+                                  ((3, 2), (1, 2), (1, 0), (2, 1)), ((1, 1), (1, 1), (0, 0), (1, 1))])
+def test_max_pool(hip, oracle, args):
+    dev, pool = hip
+    x = oracle.Rng(2).randn((3, 5, 17, 23))
+    assert np.array_equal(max_pool2d(dev, pool, x, *args), oracle.max_pool2d(x, *args))
+    xb = oracle.f32_to_bf16(x)
+    assert np.array_equal(max_pool2d(dev, pool, xb, *args, dtype=DType.BF16), oracle.max_pool2d(xb, *args, dtype=oracle.BF16))

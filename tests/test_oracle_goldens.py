@@ -328,3 +328,28 @@ def test_mlp_step_decreases_loss_and_matches_finite_differences(oracle):
             assert abs(g[name].reshape(-1)[pos] - num) < 1e-4 * max(1.0, abs(num)), (name, pos)
     loss1 = oracle.mlp_step(x, labels, nw1, nb1, nw2, nb2, 0.1)[0]
     assert loss1 < loss0
+
+
+# ---- conv / max_pool: 05_misc.rs:880-888 (conv1), :85-109 (test_max_pool) -----------------------
+def test_conv_and_pool_goldens(oracle):
+    t = np.arange(9, dtype=np.float32).reshape(1, 1, 3, 3)
+    assert oracle.conv2d(t, np.ones((1, 1, 2, 2), np.float32)).tolist() == [[[[8.0, 12.0], [20.0, 24.0]]]]
+    x = np.arange(1, 17, dtype=np.float32).reshape(1, 1, 4, 4)
+    assert oracle.max_pool2d(x).tolist() == [[[[6.0, 8.0], [14.0, 16.0]]]]
+    # stride / padding / dilation against an independent scipy cross-correlation
+    from scipy.signal import correlate
+    r = oracle.Rng(6)
+    x, w, b = r.randn((2, 3, 9, 11)), r.randn((4, 3, 3, 2)), r.randn(4)
+    for stride, pad, dil in (((1, 1), (1, 1), (1, 1)), ((2, 1), (0, 2), (1, 1)), ((1, 2), (2, 1), (2, 2))):
+        got = oracle.conv2d(x, w, b, stride, pad, dil)
+        xp = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (pad[0], pad[0]), (pad[1], pad[1])))
+        wd = np.zeros((4, 3, (3 - 1) * dil[0] + 1, (2 - 1) * dil[1] + 1))
+        wd[:, :, ::dil[0], ::dil[1]] = w
+        want = np.stack([[sum(correlate(xp[n, c], wd[co, c], mode="valid") for c in range(3)) + b[co] for co in range(4)]
+                         for n in range(2)])[:, :, ::stride[0], ::stride[1]]
+        assert got.shape == want.shape and close(got, want, rel=1e-5, abs_=1e-5)
+    xp = oracle.max_pool2d(x, (3, 3), (2, 2), (1, 1))
+    padded = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1)), constant_values=-np.inf)
+    want = np.stack([[[[padded[n, c, 2 * i:2 * i + 3, 2 * j:2 * j + 3].max() for j in range(xp.shape[3])]
+                       for i in range(xp.shape[2])] for c in range(3)] for n in range(2)])
+    assert np.array_equal(xp, want.astype(np.float32))

@@ -1,0 +1,166 @@
+// conv2d forward as an implicit GEMM on the matrix cores, and max-pooling.
+//
+// zyx lowers Tensor::conv (zyx/src/tensor/mod.rs:2583-2680) to pad -> pool view -> broadcast
+// multiply with the weight -> sum over (cin, ky, kx) (+ bias), i.e. for NCHW input x and weight
+// w[cout, cin, kh, kw]:
+//   y[n, co, oy, ox] = sum_{c,ky,kx} x[n, c, oy*sy - py + ky*dy, ox*sx - px + kx*dx] * w[co, c, ky, kx]
+// with zero outside the image (the reference multiplies by a 0/1 mask, zyx/src/kernel/
+// linearize.rs:349-382; here out-of-image taps are simply not read). Products and sums are
+// f32; bf16 tensors store the result truncated (zyx/src/tensor/reduce_ops.rs:134-136).
+//
+// GEMM view: C'[co, p] = W[co, k] . X'[k, p], k = (c, ky, kx), p = (n, oy, ox). The weight is
+// the K-contiguous operand as stored; X' is gathered on the fly (im2col never exists in HBM).
+// Pixels are the MFMA column index, so a wave's stores run along ox: contiguous in NCHW.
+// 64 (cout) x 64 (pixels) per workgroup, K step 32, 2 x 2 waves of one 32 x 32 tile.
+// The k -> (input offset, dy, dx) table is built on the host at registration and read with
+// wave-uniform (scalar) loads.
+//
+// Tensor::max_pool (zyx/src/tensor/mod.rs:2706-2741): pad with the dtype's lowest value,
+// window view, max over the window: one thread per output element.
+#include "dtypes.hpp"
+#include "kernels.hpp"
+#include "wave.hpp"
+
+namespace zk {
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int CM = 64, CN = 64, CK = 32, CPAD = 8;
+
+template <int DT> struct CT;
+template <> struct CT<DT_F32> { typedef float S; };
+template <> struct CT<DT_BF16> { typedef uint16_t S; };
+
+template <int DT, int ODT>
+__global__ __launch_bounds__(256) void conv2d_k(const Conv2d p) {
+    typedef typename CT<DT>::S S;
+    __shared__ __attribute__((aligned(16))) S Ws[CM * (CK + CPAD)];
+    __shared__ __attribute__((aligned(16))) S Xs[CN * (CK + CPAD)];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int64_t co0 = (int64_t)blockIdx.y * CM, p0 = (int64_t)blockIdx.x * CN;
+    const int64_t K = (int64_t)p.C * p.KH * p.KW, OHW = (int64_t)p.OH * p.OW, P = (int64_t)p.N * OHW;
+    const S *W = (const S *)p.w, *X = (const S *)p.x;
+
+    // this thread gathers pixel p0 + (t & 63) for 8 values of k per K tile
+    const int64_t pix = p0 + (t & 63);
+    const bool pix_ok = pix < P;
+    const int64_t n = pix_ok ? pix / OHW : 0, rem = pix_ok ? pix - n * OHW : 0;
+    const int oy = (int)(rem / p.OW), ox = (int)(rem - (int64_t)oy * p.OW);
+    const int iy0 = oy * p.sy - p.py, ix0 = ox * p.sx - p.px;
+    const S *xn = X + n * (int64_t)p.C * p.H * p.W + (int64_t)iy0 * p.W + ix0;
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+    for (int64_t k0 = 0; k0 < K; k0 += CK) {
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < 8; e++) { // weight tile: K contiguous, consecutive threads along k
+            const int idx = e * 256 + t, r = idx >> 5, k = idx & 31;
+            const int64_t gr = co0 + r, gk = k0 + k;
+            Ws[r * (CK + CPAD) + k] = (gr < p.Cout && gk < K) ? W[gr * K + gk] : (S)0;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) { // gathered tile: k is uniform over a wave, lanes walk along the pixels
+            const int kl = __builtin_amdgcn_readfirstlane((t >> 6) + 4 * e);
+            const int64_t gk = k0 + kl;
+            S v = (S)0;
+            if (gk < K) {
+                const int32_t off = p.koff[gk];
+                const int32_t dyx = p.kdyx[gk];
+                const int iy = iy0 + (dyx >> 16), ix = ix0 + (dyx & 0xffff);
+                if (pix_ok && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W) v = xn[off];
+            }
+            Xs[(t & 63) * (CK + CPAD) + kl] = v;
+        }
+        __syncthreads();
+        const S *ar = Ws + (wm * 32 + (lane & 31)) * (CK + CPAD);
+        const S *br = Xs + (wn * 32 + (lane & 31)) * (CK + CPAD);
+        if (DT == DT_F32) {
+#pragma unroll
+            for (int ks = 0; ks < CK; ks += 2) {
+                float a = ((const float *)ar)[ks + (lane >> 5)], b = ((const float *)br)[ks + (lane >> 5)];
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < CK; ks += 16) {
+                const int off = ks + (lane >> 5) * 8;
+                bf16x8 a = *(const bf16x8 *)((const uint16_t *)ar + off), b = *(const bf16x8 *)((const uint16_t *)br + off);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+            }
+        }
+    }
+
+    // register r of lane l: row (cout) 8*(r/4) + 4*(l/32) + r%4, column (pixel) l%32
+    const int64_t opix = p0 + wn * 32 + (lane & 31);
+    if (opix >= P) return; // no barrier follows
+    const int64_t on = opix / OHW, orem = opix - on * OHW;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int64_t co = co0 + wm * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (co >= p.Cout) continue;
+        float v = acc[r];
+        if (p.bias) v += DT == DT_F32 ? ((const float *)p.bias)[co] : bf16_to_f32(((const uint16_t *)p.bias)[co]);
+        if (p.relu) v = (v > 0.0f ? 1.0f : 0.0f) * v;
+        const int64_t o = (on * p.Cout + co) * OHW + orem;
+        if (ODT == DT_F32) ((float *)p.y)[o] = v;
+        else ((uint16_t *)p.y)[o] = f32_to_bf16_trunc(v);
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void max_pool2d_k(const MaxPool2d p) {
+    typedef typename CT<DT>::S S;
+    const int64_t total = p.planes * p.OH * p.OW;
+    const S *X = (const S *)p.x;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t plane = i / ((int64_t)p.OH * p.OW), rem = i - plane * p.OH * p.OW;
+        const int oy = (int)(rem / p.OW), ox = (int)(rem - (int64_t)oy * p.OW);
+        const S *xp = X + plane * (int64_t)p.H * p.W;
+        float m = DT == DT_F32 ? -FLT_MAX : -3.3895313892515355e38f; // dtype.min: f32::MIN / bf16::MIN (0xff7f)
+        for (int ky = 0; ky < p.KH; ky++) {
+            const int iy = oy * p.sy - p.py + ky * p.dy;
+            if (iy < 0 || iy >= p.H) continue;
+            for (int kx = 0; kx < p.KW; kx++) {
+                const int ix = ox * p.sx - p.px + kx * p.dx;
+                if (ix < 0 || ix >= p.W) continue;
+                const float v = DT == DT_F32 ? ((const float *)xp)[(int64_t)iy * p.W + ix] : bf16_to_f32(((const uint16_t *)xp)[(int64_t)iy * p.W + ix]);
+                m = fmaxf(v, m);
+            }
+        }
+        if (DT == DT_F32) ((float *)p.y)[i] = m;
+        else ((uint16_t *)p.y)[i] = f32_to_bf16_trunc(m);
+    }
+}
+
+} // namespace
+
+hipError_t conv2d(const Conv2d &p, hipStream_t st) {
+    const int64_t P = (int64_t)p.N * p.OH * p.OW;
+    if (P <= 0 || p.Cout <= 0) return hipSuccess;
+    if ((p.Cout + CM - 1) / CM > 65535 || (P + CN - 1) / CN >= (1ll << 31)) return hipErrorInvalidValue;
+    dim3 grid((unsigned)((P + CN - 1) / CN), (unsigned)((p.Cout + CM - 1) / CM)), block(256);
+    if (p.dtype == DT_F32 && p.out_dtype == DT_F32) hipLaunchKernelGGL((conv2d_k<DT_F32, DT_F32>), grid, block, 0, st, p);
+    else if (p.dtype == DT_BF16 && p.out_dtype == DT_BF16) hipLaunchKernelGGL((conv2d_k<DT_BF16, DT_BF16>), grid, block, 0, st, p);
+    else if (p.dtype == DT_BF16 && p.out_dtype == DT_F32) hipLaunchKernelGGL((conv2d_k<DT_BF16, DT_F32>), grid, block, 0, st, p);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+hipError_t max_pool2d(const MaxPool2d &p, hipStream_t st) {
+    const int64_t total = p.planes * p.OH * p.OW;
+    if (total <= 0) return hipSuccess;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    if (p.dtype == DT_F32) hipLaunchKernelGGL((max_pool2d_k<DT_F32>), dim3((unsigned)blocks), dim3(256), 0, st, p);
+    else if (p.dtype == DT_BF16) hipLaunchKernelGGL((max_pool2d_k<DT_BF16>), dim3((unsigned)blocks), dim3(256), 0, st, p);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+} // namespace zk

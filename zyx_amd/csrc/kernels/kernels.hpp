@@ -85,6 +85,28 @@ struct NormRows {
 };
 hipError_t norm_rows(const NormRows &p, hipStream_t stream);
 
+// conv2d forward, NCHW input, weight [Cout, C, KH, KW], groups = 1. koff[k] / kdyx[k] (k = (c,ky,kx)):
+// input offset c*H*W + ky*dy*W + kx*dx and the tap displacement (ky*dy) << 16 | (kx*dx), device arrays.
+struct Conv2d {
+    int N, C, H, W, Cout, KH, KW, OH, OW;
+    int sy, sx, py, px, dy, dx;
+    int dtype, out_dtype, relu;
+    const void *x, *w, *bias;
+    void *y;
+    const int32_t *koff, *kdyx;
+};
+hipError_t conv2d(const Conv2d &p, hipStream_t stream);
+
+// max-pool over the last two axes of `planes` images [H, W] -> [OH, OW]
+struct MaxPool2d {
+    int64_t planes;
+    int H, W, OH, OW, KH, KW, sy, sx, py, px, dy, dx;
+    int dtype;
+    const void *x;
+    void *y;
+};
+hipError_t max_pool2d(const MaxPool2d &p, hipStream_t stream);
+
 // cross_entropy of f32 logits [rows, cols] with i32 class indices; loss / grad may be null.
 struct CrossEntropy {
     int64_t rows, cols;

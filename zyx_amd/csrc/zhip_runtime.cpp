@@ -379,8 +379,65 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.n_out = o - 2;
         return ZHIP_OK;
     }
+    case ZHIP_K_CONV2D: {
+        const int64_t N = d.dims[0], C = d.dims[1], H = d.dims[2], W = d.dims[3], Co = d.dims[4], KH = d.dims[5], KW = d.dims[6];
+        const int sy = d.iparams[0], sx = d.iparams[1], py = d.iparams[2], px = d.iparams[3], dy = d.iparams[4], dx = d.iparams[5];
+        if (N < 0 || C <= 0 || H <= 0 || W <= 0 || Co <= 0 || KH <= 0 || KW <= 0 || sy <= 0 || sx <= 0 || py < 0 || px < 0 || dy <= 0 || dx <= 0)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: bad shape or stride/padding/dilation");
+        if ((d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16) || (d.out_dtype != d.dtype && !(d.dtype == ZHIP_BF16 && d.out_dtype == ZHIP_F32)))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: dtype %d -> %d not implemented", d.dtype, d.out_dtype);
+        const int64_t eh = H + 2 * py - (int64_t)dy * (KH - 1) - 1, ew = W + 2 * px - (int64_t)dx * (KW - 1) - 1;
+        if (eh < 0 || ew < 0) return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: kernel larger than the padded input");
+        const int64_t OH = eh / sy + 1, OW = ew / sx + 1;
+        if (C * H * W >= (1ll << 31) || C * KH * KW >= (1ll << 31) || N * OH * OW >= (1ll << 37) || (KH - 1) * dy >= 32768 || (KW - 1) * dx >= 65536)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: shape out of range");
+        const uint64_t e = dtype_bytes(d.dtype);
+        int a = 0;
+        p.need[a++] = (uint64_t)N * C * H * W * e;
+        p.need[a++] = (uint64_t)Co * C * KH * KW * e;
+        if (d.iparams[6]) p.need[a++] = (uint64_t)Co * e;
+        p.n_in = a;
+        p.need[a] = (uint64_t)N * Co * OH * OW * dtype_bytes(d.out_dtype);
+        p.n_out = 1;
+        p.workspace_bytes = (uint64_t)C * KH * KW * 8; // two int32 tables, filled at registration
+        return ZHIP_OK;
+    }
+    case ZHIP_K_MAX_POOL2D: {
+        const int64_t planes = d.dims[0], H = d.dims[1], W = d.dims[2], KH = d.dims[3], KW = d.dims[4];
+        const int sy = d.iparams[0], sx = d.iparams[1], py = d.iparams[2], px = d.iparams[3], dy = d.iparams[4], dx = d.iparams[5];
+        if (planes < 0 || H <= 0 || W <= 0 || KH <= 0 || KW <= 0 || sy <= 0 || sx <= 0 || py < 0 || px < 0 || dy <= 0 || dx <= 0 ||
+            H >= (1 << 30) || W >= (1 << 30))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: bad shape or stride/padding/dilation");
+        if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16) return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: dtype must be F32 or BF16");
+        const int64_t eh = H + 2 * py - (int64_t)dy * (KH - 1) - 1, ew = W + 2 * px - (int64_t)dx * (KW - 1) - 1;
+        if (eh < 0 || ew < 0) return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: window larger than the padded input");
+        const uint64_t e = dtype_bytes(d.dtype);
+        p.n_in = 1;
+        p.n_out = 1;
+        p.need[0] = (uint64_t)planes * H * W * e;
+        p.need[1] = (uint64_t)planes * (eh / sy + 1) * (ew / sx + 1) * e;
+        return ZHIP_OK;
+    }
     default: return c->fail(ZHIP_KERNEL_COMPILATION, "unknown kernel kind %d", d.kind);
     }
+}
+
+// Kinds whose workspace holds constant tables fill them here, once, at registration.
+int32_t program_fill_workspace(zhip_ctx *c, Program &p) {
+    const zhip_kernel_desc &d = p.desc;
+    if (d.kind != ZHIP_K_CONV2D) return ZHIP_OK;
+    const int64_t C = d.dims[1], H = d.dims[2], W = d.dims[3], KH = d.dims[5], KW = d.dims[6], K = C * KH * KW;
+    const int dy = d.iparams[4], dx = d.iparams[5];
+    std::vector<int32_t> tab(2 * K);
+    for (int64_t ci = 0; ci < C; ci++)
+        for (int64_t ky = 0; ky < KH; ky++)
+            for (int64_t kx = 0; kx < KW; kx++) {
+                const int64_t k = (ci * KH + ky) * KW + kx;
+                tab[k] = (int32_t)(ci * H * W + ky * dy * W + kx * dx);
+                tab[K + k] = (int32_t)(((ky * dy) << 16) | (kx * dx));
+            }
+    HIPCHK(c, hipMemcpy(p.workspace, tab.data(), tab.size() * 4, hipMemcpyHostToDevice), ZHIP_KERNEL_COMPILATION);
+    return ZHIP_OK;
 }
 
 hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
@@ -495,6 +552,28 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         if (d.flags & ZHIP_CE_LOSS) a.loss = (float *)ptr[o++];
         if (d.flags & ZHIP_CE_GRAD) a.grad = (float *)ptr[o++];
         return zk::cross_entropy(a, st);
+    }
+    case ZHIP_K_CONV2D: {
+        zk::Conv2d a{};
+        a.N = (int)d.dims[0]; a.C = (int)d.dims[1]; a.H = (int)d.dims[2]; a.W = (int)d.dims[3];
+        a.Cout = (int)d.dims[4]; a.KH = (int)d.dims[5]; a.KW = (int)d.dims[6];
+        a.sy = d.iparams[0]; a.sx = d.iparams[1]; a.py = d.iparams[2]; a.px = d.iparams[3]; a.dy = d.iparams[4]; a.dx = d.iparams[5];
+        a.OH = (a.H + 2 * a.py - a.dy * (a.KH - 1) - 1) / a.sy + 1;
+        a.OW = (a.W + 2 * a.px - a.dx * (a.KW - 1) - 1) / a.sx + 1;
+        a.dtype = d.dtype; a.out_dtype = d.out_dtype; a.relu = d.iparams[7];
+        a.x = ptr[0]; a.w = ptr[1]; a.bias = d.iparams[6] ? ptr[2] : nullptr; a.y = ptr[p.n_in];
+        a.koff = (const int32_t *)p.workspace;
+        a.kdyx = a.koff + (int64_t)a.C * a.KH * a.KW;
+        return zk::conv2d(a, st);
+    }
+    case ZHIP_K_MAX_POOL2D: {
+        zk::MaxPool2d a{};
+        a.planes = d.dims[0]; a.H = (int)d.dims[1]; a.W = (int)d.dims[2]; a.KH = (int)d.dims[3]; a.KW = (int)d.dims[4];
+        a.sy = d.iparams[0]; a.sx = d.iparams[1]; a.py = d.iparams[2]; a.px = d.iparams[3]; a.dy = d.iparams[4]; a.dx = d.iparams[5];
+        a.OH = (a.H + 2 * a.py - a.dy * (a.KH - 1) - 1) / a.sy + 1;
+        a.OW = (a.W + 2 * a.px - a.dx * (a.KW - 1) - 1) / a.sx + 1;
+        a.dtype = d.dtype; a.x = ptr[0]; a.y = ptr[1];
+        return zk::max_pool2d(a, st);
     }
     default: return hipErrorInvalidValue;
     }
@@ -883,6 +962,11 @@ ZHIP_EXPORT int32_t zhip_register_kernel(zhip_ctx *c, const zhip_kernel_desc *de
     if (p.workspace_bytes) {
         HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_COMPILATION);
         HIPCHK(c, hipMalloc(&p.workspace, p.workspace_bytes), ZHIP_KERNEL_COMPILATION);
+        rc = program_fill_workspace(c, p);
+        if (rc != ZHIP_OK) {
+            (void)hipFree(p.workspace);
+            return rc;
+        }
     }
     p.live = true;
     *prog = c->programs.push(p);

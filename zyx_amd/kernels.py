@@ -291,3 +291,90 @@ def cross_entropy(dev: HIPDevice, pool: HIPMemoryPool, logits, labels, grad_scal
         pool.deallocate(bb, [])
     dev.release(prog)
     return loss, grad
+
+
+# ---- conv2d / max_pool2d (ZHIP_K_CONV2D, ZHIP_K_MAX_POOL2D) ---------------------------------------------
+K_CONV2D, K_MAX_POOL2D = 7, 8
+
+
+def conv_out(size: int, k: int, stride: int, pad: int, dil: int) -> int:
+    return (size + 2 * pad - dil * (k - 1) - 1) // stride + 1
+
+
+def conv2d_desc(n, c, h, w, cout, kh, kw, stride=(1, 1), padding=(0, 0), dilation=(1, 1), bias=False, relu=False,
+                dtype: DType = DType.F32, out_dtype: DType | None = None) -> KernelDesc:
+    d = KernelDesc()
+    d.kind, d.dtype, d.out_dtype = K_CONV2D, DType(dtype), DType(dtype if out_dtype is None else out_dtype)
+    for i, v in enumerate((n, c, h, w, cout, kh, kw)):
+        d.dims[i] = v
+    for i, v in enumerate((stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1], int(bias), int(relu))):
+        d.iparams[i] = v
+    return d
+
+
+def max_pool2d_desc(planes, h, w, kernel=(2, 2), stride=(2, 2), padding=(0, 0), dilation=(1, 1),
+                    dtype: DType = DType.F32) -> KernelDesc:
+    d = KernelDesc()
+    d.kind, d.dtype, d.out_dtype = K_MAX_POOL2D, DType(dtype), DType(dtype)
+    for i, v in enumerate((planes, h, w, kernel[0], kernel[1])):
+        d.dims[i] = v
+    for i, v in enumerate((stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1])):
+        d.iparams[i] = v
+    return d
+
+
+def conv2d(dev: HIPDevice, pool: HIPMemoryPool, x, w, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
+           relu=False, dtype: DType = DType.F32, out_dtype: DType | None = None, pool_kernel=None):
+    """Conv2d::forward (+ ReLU) and optionally max_pool(pool_kernel, stride = kernel) as two launches whose
+    second waits on the first's event. Returns y, or (y, pooled)."""
+    st = _NP_STORE[DType(dtype)]
+    out_dtype = DType(dtype if out_dtype is None else out_dtype)
+    x, w = np.ascontiguousarray(x, st), np.ascontiguousarray(w, st)
+    n, c, h, wd = x.shape
+    co, _, kh, kw = w.shape
+    oh, ow = conv_out(h, kh, stride[0], padding[0], dilation[0]), conv_out(wd, kw, stride[1], padding[1], dilation[1])
+    prog = dev.register_kernel(conv2d_desc(n, c, h, wd, co, kh, kw, stride, padding, dilation, bias is not None, relu,
+                                           dtype, out_dtype))
+    bufs, waits = [], []
+    for arr in (x, w) + ((np.ascontiguousarray(bias, st),) if bias is not None else ()):
+        bb, e = to_device(pool, arr)
+        bufs.append(bb)
+        waits.append(e)
+    out_np = _NP_STORE[out_dtype]
+    yb, e = alloc_like(pool, n * co * oh * ow, np.dtype(out_np).itemsize)
+    done = dev.launch(prog, pool, bufs + [yb], waits + [e])
+    progs, extra = [prog], []
+    if pool_kernel is not None:
+        ph, pw = conv_out(oh, pool_kernel[0], pool_kernel[0], 0, 1), conv_out(ow, pool_kernel[1], pool_kernel[1], 0, 1)
+        pprog = dev.register_kernel(max_pool2d_desc(n * co, oh, ow, pool_kernel, pool_kernel, dtype=out_dtype))
+        pb, e = alloc_like(pool, n * co * ph * pw, np.dtype(out_np).itemsize)
+        pdone = dev.launch(pprog, pool, [yb, pb], [done, e])
+        pooled = to_host(pool, pb, (n, co, ph, pw), out_np, [pdone])
+        y = to_host(pool, yb, (n, co, oh, ow), out_np)
+        progs.append(pprog)
+        extra.append(pb)
+    else:
+        y = to_host(pool, yb, (n, co, oh, ow), out_np, [done])
+    for bb in bufs + [yb] + extra:
+        pool.deallocate(bb, [])
+    for pr in progs:
+        dev.release(pr)
+    return (y, pooled) if pool_kernel is not None else y
+
+
+def max_pool2d(dev: HIPDevice, pool: HIPMemoryPool, x, kernel=(2, 2), stride=(2, 2), padding=(0, 0), dilation=(1, 1),
+               dtype: DType = DType.F32):
+    st = _NP_STORE[DType(dtype)]
+    x = np.ascontiguousarray(x, st)
+    h, wd = x.shape[-2:]
+    planes = x.size // (h * wd)
+    oh, ow = conv_out(h, kernel[0], stride[0], padding[0], dilation[0]), conv_out(wd, kernel[1], stride[1], padding[1], dilation[1])
+    prog = dev.register_kernel(max_pool2d_desc(planes, h, wd, kernel, stride, padding, dilation, dtype))
+    xb, e0 = to_device(pool, x)
+    yb, e1 = alloc_like(pool, planes * oh * ow, x.itemsize)
+    done = dev.launch(prog, pool, [xb, yb], [e0, e1])
+    y = to_host(pool, yb, x.shape[:-2] + (oh, ow), st, [done])
+    pool.deallocate(xb, [])
+    pool.deallocate(yb, [])
+    dev.release(prog)
+    return y
