@@ -164,6 +164,17 @@ enum zhip_kernel_kind {
      * as the dtype's lowest value. dims = {planes (product of the leading axes), H, W, KH, KW};
      * iparams = {sy, sx, py, px, dy, dx}; dtype F32 or BF16. args: x, y[planes, OH, OW]. */
     ZHIP_K_MAX_POOL2D = 8,
+    /* Tensor::gather / index_select / scatter along one axis, tensors of rank <= 4 given as
+     * 4-D shapes with leading 1s (zyx/src/tensor/index_ops.rs:321-445). Negative indices wrap
+     * once, indices still out of range read 0 (gather) or are dropped (scatter); scatter adds,
+     * duplicates sum in ascending position order, `self` is added last.
+     * dims[0..4] = shape of x / self, dims[4..8] = shape of the index tensor (for
+     * ZHIP_INDEX_SELECT: shape of the output, the index being 1-D of length dims[4+axis]);
+     * iparams[0] = axis (0..3 in the 4-D view), iparams[1] = index dtype (ZHIP_I32 / ZHIP_I64);
+     * flags = ZHIP_INDEX_GATHER | ZHIP_INDEX_SELECT | ZHIP_INDEX_SCATTER. dtype: gather and
+     * select copy any dtype bit for bit; scatter supports F32, F64, I32, U32, I64, U64.
+     * args: gather/select: x, index, out; scatter: self, index, src, out. */
+    ZHIP_K_INDEX = 9,
     ZHIP_K_COUNT_
 };
 #define ZHIP_SOFTMAX_Y 1
@@ -174,6 +185,9 @@ enum zhip_kernel_kind {
 #define ZHIP_NORM_BIAS 4
 #define ZHIP_CE_LOSS 1
 #define ZHIP_CE_GRAD 2
+#define ZHIP_INDEX_GATHER 0
+#define ZHIP_INDEX_SELECT 1
+#define ZHIP_INDEX_SCATTER 2
 #define ZHIP_GEMM_TRANS_A 1
 #define ZHIP_GEMM_TRANS_B 2
 

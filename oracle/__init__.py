@@ -339,3 +339,43 @@ def max_pool2d(x, kernel=(2, 2), stride=(2, 2), padding=(0, 0), dilation=(1, 1),
     lib().zo_max_pool2d(dtype, _p(x), _p(y), _I64(planes), _I64(h), _I64(wd), _I64(kernel[0]), _I64(kernel[1]), stride[0],
                         stride[1], padding[0], padding[1], dilation[0], dilation[1])
     return y
+
+
+# ---- gather / scatter / index_select: zyx/src/tensor/index_ops.rs:321-445 (numpy restatement) -------------
+def _wrap_index(idx: np.ndarray, dim: int):
+    idx = idx.astype(np.int64)
+    idx = idx + (idx < 0) * dim          # one wrap: idx + (idx < 0) * dim_size  (:342-343)
+    return idx, (idx >= 0) & (idx < dim)  # an index still out of range has an all-zero one-hot (:315-316)
+
+
+def gather(x: np.ndarray, axis: int, indices: np.ndarray) -> np.ndarray:
+    """out[i] = sum_k onehot(idx[i])[k] * x[.., k, ..] over x shrunk to the index tensor's extent."""
+    axis %= x.ndim
+    idx, ok = _wrap_index(np.asarray(indices), x.shape[axis])
+    sl = tuple(slice(None) if d == axis else slice(0, idx.shape[d]) for d in range(x.ndim))
+    vals = np.take_along_axis(x[sl], np.where(ok, idx, 0), axis)
+    return np.where(ok, vals, np.zeros((), x.dtype)).astype(x.dtype)
+
+
+def index_select(x: np.ndarray, axis: int, index: np.ndarray) -> np.ndarray:
+    axis %= x.ndim
+    shape = [1] * x.ndim
+    shape[axis] = len(index)
+    full = list(x.shape)
+    full[axis] = len(index)
+    return gather(x, axis, np.broadcast_to(np.asarray(index).reshape(shape), full))
+
+
+def scatter(x: np.ndarray, axis: int, indices: np.ndarray, src: np.ndarray) -> np.ndarray:
+    """self + sum over index positions j (ascending along `axis`) of onehot(idx[.., j, ..]) * src[.., j, ..]."""
+    axis %= x.ndim
+    idx, ok = _wrap_index(np.asarray(indices), x.shape[axis])
+    contrib = np.zeros_like(x)
+    grids = np.meshgrid(*[np.arange(n) for n in idx.shape], indexing="ij")
+    for j in range(idx.shape[axis]):
+        sel = tuple(slice(j, j + 1) if d == axis else slice(None) for d in range(x.ndim))
+        tgt = [g[sel] for g in grids]
+        tgt[axis] = idx[sel]
+        m = ok[sel]
+        np.add.at(contrib, tuple(t[m] for t in tgt), np.asarray(src, x.dtype)[sel][m])  # targets are distinct within one j
+    return (contrib + x).astype(x.dtype)

@@ -353,3 +353,35 @@ def test_conv_and_pool_goldens(oracle):
     want = np.stack([[[[padded[n, c, 2 * i:2 * i + 3, 2 * j:2 * j + 3].max() for j in range(xp.shape[3])]
                        for i in range(xp.shape[2])] for c in range(3)] for n in range(2)])
     assert np.array_equal(xp, want.astype(np.float32))
+
+
+# ---- gather / scatter / index_select: 08_indexing.rs:181-300, 303-435, 597-627; 05_misc.rs:778-798 ------
+def test_index_op_goldens(oracle):
+    g = oracle.gather
+    x = np.array([[10, 20, 30, 40, 50], [11, 21, 31, 41, 51], [12, 22, 32, 42, 52]], np.uint16)
+    assert g(x, 1, np.array([[0, 2, 4], [1, 3, 0], [4, 1, 2]])).tolist() == [[10, 30, 50], [21, 41, 11], [52, 22, 32]]
+    x = np.array([[1, 2, 3], [4, 5, 6], [7, 8, 9]], np.int32)
+    assert g(x, 0, np.array([[0, 1], [1, 2], [0, 2]])).tolist() == [[1, 5], [4, 8], [1, 8]]
+    assert g(np.array([[1, 2, 3], [4, 5, 6]], np.int32), 1, np.array([[-1, 0], [1, -2]])).tolist() == [[3, 1], [5, 5]]
+    x3 = np.array([[[1, 2], [3, 4]], [[5, 6], [7, 8]]], np.int32)
+    assert g(x3, 2, np.array([[[0], [1]], [[1], [0]]])).tolist() == [[[1], [4]], [[6], [7]]]
+    assert g(np.array([[1, 2], [3, 4], [5, 6]], np.int32), -2, np.array([[0], [0], [2]])).reshape(-1).tolist() == [1, 1, 5]
+    assert g(np.array([[1, 2], [3, 4]], np.int32), 1, np.array([[0, 0, 1], [1, 1, 0]])).tolist() == [[1, 1, 2], [4, 4, 3]]
+    assert g(np.array([1, 2, 3], np.int32), 0, np.array([0, 3, -4, 2])).tolist() == [1, 0, 0, 3]  # out of range -> 0
+    s = oracle.scatter
+    z = lambda *sh: np.zeros(sh, np.int32)
+    assert s(z(3, 3), 0, np.array([[0, 1, 2], [0, 1, 2]]), np.array([[1, 2, 3], [4, 5, 6]])).tolist() == [[5, 0, 0], [0, 7, 0], [0, 0, 9]]
+    assert s(z(3, 4), 1, np.array([[0, 3], [1, 2], [2, 1]]), np.array([[1, 2], [3, 4], [5, 6]])).tolist() == \
+        [[1, 0, 0, 2], [0, 3, 4, 0], [0, 6, 5, 0]]
+    assert s(z(5), 0, np.array([0, 0, 1, 1, 2, 4]), np.array([1, 2, 3, 4, 5, 6])).tolist() == [3, 7, 5, 0, 6]
+    assert s(np.full((2, 3), 10, np.int32), 1, np.array([[0, 1, 2]]), np.array([[1, 2, 3]])).tolist() == [[11, 12, 13], [10, 10, 10]]
+    assert s(z(3, 3), 1, np.array([[-1, -2], [0, 1]]), np.array([[1, 2], [3, 4]])).tolist() == [[0, 2, 1], [3, 4, 0], [0, 0, 0]]
+    assert s(z(2, 3, 4), 2, np.array([[[0, 3]], [[1, 2]]]), np.array([[[1, 2]], [[3, 4]]])).tolist() == \
+        [[[1, 0, 0, 2], [0, 0, 0, 0], [0, 0, 0, 0]], [[0, 3, 4, 0], [0, 0, 0, 0], [0, 0, 0, 0]]]
+    assert s(z(3, 3), 0, np.array([[0, 1, 2]]), np.array([[1, 2, 3]])).tolist() == [[1, 0, 0], [0, 2, 0], [0, 0, 3]]
+    x = np.array([[1, 2, 3], [4, 5, 6], [7, 8, 9]], np.int32)
+    sel = oracle.index_select
+    assert sel(x, 0, np.array([2, 0])).tolist() == [[7, 8, 9], [1, 2, 3]]
+    assert sel(x, 1, np.array([2, 0])).tolist() == [[3, 1], [6, 4], [9, 7]]
+    assert sel(x, 0, np.array([-1, -3])).tolist() == [[7, 8, 9], [1, 2, 3]]
+    assert sel(x, 1, np.array([-2, -1])).tolist() == [[2, 3], [5, 6], [8, 9]]

@@ -107,6 +107,17 @@ struct MaxPool2d {
 };
 hipError_t max_pool2d(const MaxPool2d &p, hipStream_t stream);
 
+// gather / index_select / scatter along `axis` of a rank-4 view (leading dims padded with 1).
+// gather: x has shape xs, idx (and out) shape os; select: idx is 1-D of length os[axis].
+// scatter: self (x) and out have shape xs, idx and src shape os.
+struct IndexOp {
+    int64_t xs[4], os[4];
+    int axis, dtype, idx64, select, scatter;
+    const void *x, *idx, *src;
+    void *out;
+};
+hipError_t index_op(const IndexOp &p, hipStream_t stream);
+
 // cross_entropy of f32 logits [rows, cols] with i32 class indices; loss / grad may be null.
 struct CrossEntropy {
     int64_t rows, cols;

@@ -418,6 +418,42 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.need[1] = (uint64_t)planes * (eh / sy + 1) * (ew / sx + 1) * e;
         return ZHIP_OK;
     }
+    case ZHIP_K_INDEX: {
+        const int axis = d.iparams[0], idt = d.iparams[1];
+        if (axis < 0 || axis > 3 || (idt != ZHIP_I32 && idt != ZHIP_I64) || d.flags < 0 || d.flags > 2)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "index: bad axis, index dtype or mode");
+        uint64_t nx = 1, no = 1;
+        for (int k = 0; k < 4; k++) {
+            if (d.dims[k] < 0 || d.dims[4 + k] < 0 || d.dims[k] >= (1ll << 31) || d.dims[4 + k] >= (1ll << 31))
+                return c->fail(ZHIP_KERNEL_COMPILATION, "index: dimension out of range");
+            if (k != axis && d.flags != ZHIP_INDEX_SELECT && d.dims[4 + k] > d.dims[k])
+                return c->fail(ZHIP_KERNEL_COMPILATION, "Shape mismatch at dimension %d: self.shape = %lld < indices.shape = %lld", k,
+                               (long long)d.dims[k], (long long)d.dims[4 + k]);
+            if (k != axis && d.flags == ZHIP_INDEX_SELECT && d.dims[4 + k] != d.dims[k])
+                return c->fail(ZHIP_KERNEL_COMPILATION, "index_select: output shape must equal the input's outside the axis");
+            nx *= (uint64_t)d.dims[k];
+            no *= (uint64_t)d.dims[4 + k];
+        }
+        if (nx >= (1ull << 40) || no >= (1ull << 40)) return c->fail(ZHIP_KERNEL_COMPILATION, "index: tensor too large");
+        const uint64_t e = dtype_bytes(d.dtype), ie = dtype_bytes(idt);
+        if (e == 0) return c->fail(ZHIP_KERNEL_COMPILATION, "index: bad dtype");
+        if (d.flags == ZHIP_INDEX_SCATTER) {
+            if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_F64 && d.dtype != ZHIP_I32 && d.dtype != ZHIP_U32 && d.dtype != ZHIP_I64 && d.dtype != ZHIP_U64)
+                return c->fail(ZHIP_KERNEL_COMPILATION, "scatter: dtype %d not implemented", d.dtype);
+            p.n_in = 3;
+            p.need[0] = nx * e;
+            p.need[1] = no * ie;
+            p.need[2] = no * e;
+            p.need[3] = nx * e;
+        } else {
+            p.n_in = 2;
+            p.need[0] = nx * e;
+            p.need[1] = (d.flags == ZHIP_INDEX_SELECT ? (uint64_t)d.dims[4 + axis] : no) * ie;
+            p.need[2] = no * e;
+        }
+        p.n_out = 1;
+        return ZHIP_OK;
+    }
     default: return c->fail(ZHIP_KERNEL_COMPILATION, "unknown kernel kind %d", d.kind);
     }
 }
@@ -574,6 +610,23 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         a.OW = (a.W + 2 * a.px - a.dx * (a.KW - 1) - 1) / a.sx + 1;
         a.dtype = d.dtype; a.x = ptr[0]; a.y = ptr[1];
         return zk::max_pool2d(a, st);
+    }
+    case ZHIP_K_INDEX: {
+        zk::IndexOp a{};
+        for (int k = 0; k < 4; k++) {
+            a.xs[k] = d.dims[k];
+            a.os[k] = d.dims[4 + k];
+        }
+        a.axis = d.iparams[0];
+        a.idx64 = d.iparams[1] == ZHIP_I64;
+        a.dtype = d.dtype;
+        a.select = d.flags == ZHIP_INDEX_SELECT;
+        a.scatter = d.flags == ZHIP_INDEX_SCATTER;
+        a.x = ptr[0];
+        a.idx = ptr[1];
+        a.src = a.scatter ? ptr[2] : nullptr;
+        a.out = ptr[p.n_in];
+        return zk::index_op(a, st);
     }
     default: return hipErrorInvalidValue;
     }

@@ -378,3 +378,84 @@ def max_pool2d(dev: HIPDevice, pool: HIPMemoryPool, x, kernel=(2, 2), stride=(2,
     pool.deallocate(yb, [])
     dev.release(prog)
     return y
+
+
+# ---- gather / index_select / scatter (ZHIP_K_INDEX) ----------------------------------------------------------
+K_INDEX = 9
+INDEX_GATHER, INDEX_SELECT, INDEX_SCATTER = 0, 1, 2
+_DT_OF_NP = {np.dtype(np.float32): DType.F32, np.dtype(np.float64): DType.F64, np.dtype(np.int32): DType.I32,
+             np.dtype(np.int64): DType.I64, np.dtype(np.uint8): DType.U8, np.dtype(np.uint16): DType.U16,
+             np.dtype(np.uint32): DType.U32, np.dtype(np.uint64): DType.U64, np.dtype(np.int8): DType.I8,
+             np.dtype(np.int16): DType.I16, np.dtype(np.bool_): DType.Bool}
+
+
+def _pad4(shape):
+    assert len(shape) <= 4, "rank <= 4"
+    return (1,) * (4 - len(shape)) + tuple(shape)
+
+
+def index_desc(mode: int, x_shape, idx_shape, axis: int, dtype: DType, idx_dtype: DType = DType.I32) -> KernelDesc:
+    d = KernelDesc()
+    d.kind, d.dtype, d.out_dtype, d.flags = K_INDEX, DType(dtype), DType(dtype), mode
+    rank = len(x_shape)
+    for i, v in enumerate(_pad4(x_shape) + _pad4(idx_shape)):
+        d.dims[i] = v
+    d.iparams[0], d.iparams[1] = (axis % rank) + (4 - rank), int(idx_dtype)
+    return d
+
+
+def _index_run(dev, pool, desc, arrays, out_shape, out_np):
+    prog = dev.register_kernel(desc)
+    bufs, waits = [], []
+    for a in arrays:
+        b, e = to_device(pool, a)
+        bufs.append(b)
+        waits.append(e)
+    n = int(np.prod(out_shape))
+    ob, e = alloc_like(pool, n, np.dtype(out_np).itemsize)
+    done = dev.launch(prog, pool, bufs + [ob], waits + [e])
+    out = to_host(pool, ob, out_shape, out_np, [done])
+    for b in bufs + [ob]:
+        pool.deallocate(b, [])
+    dev.release(prog)
+    return out
+
+
+def _as_index(indices):
+    idx = np.ascontiguousarray(indices)
+    if idx.dtype == np.int64:
+        return idx, DType.I64
+    return np.ascontiguousarray(idx, np.int32), DType.I32  # unsigned / narrow index dtypes widen losslessly
+
+
+def gather(dev: HIPDevice, pool: HIPMemoryPool, x, axis: int, indices):
+    """Tensor::gather (zyx/src/tensor/index_ops.rs:321-361)."""
+    x = np.ascontiguousarray(x)
+    idx, idt = _as_index(indices)
+    if x.ndim != idx.ndim:
+        raise ValueError(f"self.rank({x.ndim}) != indices.rank({idx.ndim})")
+    return _index_run(dev, pool, index_desc(INDEX_GATHER, x.shape, idx.shape, axis, _DT_OF_NP[x.dtype], idt), [x, idx],
+                      idx.shape, x.dtype)
+
+
+def index_select(dev: HIPDevice, pool: HIPMemoryPool, x, axis: int, index):
+    """Tensor::index_select (index_ops.rs:431-445): 1-D index along `axis`."""
+    x = np.ascontiguousarray(x)
+    idx, idt = _as_index(index)
+    out_shape = list(x.shape)
+    out_shape[axis % x.ndim] = idx.shape[0]
+    return _index_run(dev, pool, index_desc(INDEX_SELECT, x.shape, out_shape, axis, _DT_OF_NP[x.dtype], idt), [x, idx],
+                      tuple(out_shape), x.dtype)
+
+
+def scatter(dev: HIPDevice, pool: HIPMemoryPool, x, axis: int, indices, src):
+    """Tensor::scatter (index_ops.rs:376-425): adds src into self at the indexed positions."""
+    x = np.ascontiguousarray(x)
+    idx, idt = _as_index(indices)
+    src = np.ascontiguousarray(src, x.dtype)
+    if x.ndim != idx.ndim:
+        raise ValueError(f"self.rank({x.ndim}) != indices.rank({idx.ndim})")
+    if idx.shape != src.shape:
+        raise ValueError(f"indices shape {idx.shape} != src shape {src.shape}")
+    return _index_run(dev, pool, index_desc(INDEX_SCATTER, x.shape, idx.shape, axis, _DT_OF_NP[x.dtype], idt),
+                      [x, idx, src], x.shape, x.dtype)
