@@ -175,6 +175,15 @@ enum zhip_kernel_kind {
      * select copy any dtype bit for bit; scatter supports F32, F64, I32, U32, I64, U64.
      * args: gather/select: x, index, out; scatter: self, index, src, out. */
     ZHIP_K_INDEX = 9,
+    /* Attention core of CausalSelfAttention::forward (zyx-nn/src/causal_self_attention.rs:36-74) on the
+     * c_attn output qkv[B, T, 3*C], C = H*dh: split([c,c,c], 2), reshape [b,t,h,dh], transpose(1,2),
+     * att = q.dot(k.t()) * scale, softmax(-1), eval-mode dropout att / (1 - p)
+     * (zyx/src/tensor/mod.rs:822-828), att.dot(v), transpose(1,2).reshape([b,t,c]). The reference
+     * applies no mask, so none is applied. dims = {B, T, H, dh}; dtype BF16 or F32 (storage of qkv
+     * and y, f32 arithmetic); fparams[0] = scale (0 selects 1/sqrt(dh)), fparams[1] = dropout p;
+     * flags: ZHIP_ATTN_LSE also writes lse[B, H, T] (f32) = ln sum_j exp(scale q.k_j), which the
+     * backward needs. args: qkv, y[B, T, C], (lse). */
+    ZHIP_K_ATTENTION = 10,
     ZHIP_K_COUNT_
 };
 #define ZHIP_SOFTMAX_Y 1
@@ -188,6 +197,7 @@ enum zhip_kernel_kind {
 #define ZHIP_INDEX_GATHER 0
 #define ZHIP_INDEX_SELECT 1
 #define ZHIP_INDEX_SCATTER 2
+#define ZHIP_ATTN_LSE 1
 #define ZHIP_GEMM_TRANS_A 1
 #define ZHIP_GEMM_TRANS_B 2
 

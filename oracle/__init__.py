@@ -379,3 +379,56 @@ def scatter(x: np.ndarray, axis: int, indices: np.ndarray, src: np.ndarray) -> n
         m = ok[sel]
         np.add.at(contrib, tuple(t[m] for t in tgt), np.asarray(src, x.dtype)[sel][m])  # targets are distinct within one j
     return (contrib + x).astype(x.dtype)
+
+
+# ---- attention: zyx-nn/src/causal_self_attention.rs:36-74 ----------------------------------------------------
+def attention(qkv: np.ndarray, n_head: int, scale: float | None = None, dropout_p: float = 0.0, dtype: int = F32,
+              want_lse: bool = False):
+    """Core of CausalSelfAttention::forward on the c_attn output qkv[B,T,3C] -> y[B,T,C] (the reference applies
+    no mask). scale defaults to (1/sqrt(dh)) as f32; eval-mode dropout divides the probabilities by 1-p."""
+    qkv = np.ascontiguousarray(qkv, _store_dtype(dtype))
+    b, t, c3 = qkv.shape
+    c = c3 // 3
+    dh = c // n_head
+    scale = np.float32(1.0 / np.sqrt(float(dh))) if scale is None else np.float32(scale)
+    y = np.empty((b, t, c), qkv.dtype)
+    lse = np.empty((b, n_head, t), np.float32) if want_lse else None
+    lib().zo_attention(dtype, _p(qkv), _p(y), _p(lse), _I64(b), _I64(t), _I64(n_head), _I64(dh), C.c_float(scale),
+                       C.c_float(np.float32(1.0) - np.float32(dropout_p)))
+    return (y, lse) if want_lse else y
+
+
+def attention_bwd(qkv: np.ndarray, dy: np.ndarray, n_head: int, scale: float | None = None, dropout_p: float = 0.0,
+                  dtype: int = F32) -> np.ndarray:
+    """d(sum(y * dy)) / d(qkv) for `attention`, f64 arithmetic, stored in `dtype`."""
+    qkv = np.ascontiguousarray(qkv, _store_dtype(dtype))
+    dy = np.ascontiguousarray(dy, qkv.dtype)
+    b, t, c3 = qkv.shape
+    dh = c3 // 3 // n_head
+    scale = np.float32(1.0 / np.sqrt(float(dh))) if scale is None else np.float32(scale)
+    out = np.empty_like(qkv)
+    lib().zo_attention_bwd(dtype, _p(qkv), _p(dy), _p(out), _I64(b), _I64(t), _I64(n_head), _I64(dh), C.c_float(scale),
+                           C.c_float(np.float32(1.0) - np.float32(dropout_p)))
+    return out
+
+
+def linear(x: np.ndarray, w: np.ndarray, bias: np.ndarray | None = None, dtype: int = F32, act: str = "none") -> np.ndarray:
+    """Linear::forward (zyx-nn/src/linear.rs:38-44): x.dot(w^T) + b over the last axis, w stored [out, in]; f32
+    registers, one store in `dtype` after the optional activation."""
+    lead = x.shape[:-1]
+    c = matmul(x.reshape(-1, x.shape[-1]), w, dtype, F32, transb=True)
+    if bias is not None or act != "none":
+        c = bias_act(c, bias, act, dtype if bias is not None else F32)
+    if dtype == BF16:
+        c = f32_to_bf16(c)
+    elif dtype == F16:
+        c = f32_to_f16(c)
+    return c.reshape(*lead, w.shape[0])
+
+
+def causal_self_attention(x, w_attn, w_proj, n_head: int, b_attn=None, b_proj=None, dropout_p: float = 0.0,
+                          dtype: int = F32) -> np.ndarray:
+    """CausalSelfAttention::forward, tensors materialised (stored in `dtype`) after c_attn, att.dot(v), c_proj."""
+    qkv = linear(x, w_attn, b_attn, dtype)
+    y = attention(qkv, n_head, None, dropout_p, dtype)
+    return linear(y, w_proj, b_proj, dtype)

@@ -733,3 +733,100 @@ ZO_API void zo_max_pool2d(int dtype, const void *x, void *y, int64_t planes, int
                 store_from_f32(y, dtype, (pl * OH + oy) * OW + ox, m);
             }
 }
+
+/* ---- attention core of CausalSelfAttention::forward (zyx-nn/src/causal_self_attention.rs:36-74) ----------
+ * qkv[B,T,3C] is the c_attn output; split([c,c,c],2), reshape [b,t,h,c/h], transpose(1,2) address
+ * q/k/v of head h at column h*dh of the first/second/third C columns. att = q.dot(k.t()) * scale,
+ * softmax(-1) (max, sub, exp, sum, div: zyx/src/tensor/mod.rs:1457-1461), eval-mode dropout
+ * (att / (1-p), zyx/src/tensor/mod.rs:822-828), att.dot(v), transpose(1,2).reshape([b,t,c]).
+ * f32 registers, serial sums, one narrowing store for y. lse (optional) = max + ln(sum). */
+ZO_API void zo_attention(int dtype, const void *qkv, void *y, float *lse, int64_t B, int64_t T, int64_t H, int64_t dh,
+                         float scale, float keep) {
+    const int64_t Cc = H * dh, ld = 3 * Cc;
+#pragma omp parallel
+    {
+        float *s = (float *)malloc(sizeof(float) * (size_t)(T > 0 ? T : 1));
+#pragma omp for collapse(2)
+        for (int64_t bh = 0; bh < B * H; bh++)
+            for (int64_t t = 0; t < T; t++) {
+                const int64_t b = bh / H, h = bh % H;
+                const int64_t qo = (b * T + t) * ld + h * dh;
+                for (int64_t j = 0; j < T; j++) {
+                    const int64_t ko = (b * T + j) * ld + Cc + h * dh;
+                    float a = 0.0f;
+                    for (int64_t d = 0; d < dh; d++) a = load_as_f32(qkv, dtype, qo + d) * load_as_f32(qkv, dtype, ko + d) + a;
+                    s[j] = a * scale;
+                }
+                float m = s[0];
+                for (int64_t j = 1; j < T; j++) m = fmaxf(m, s[j]);
+                float sum = 0.0f;
+                for (int64_t j = 0; j < T; j++) {
+                    s[j] = expf(s[j] - m);
+                    sum = s[j] + sum;
+                }
+                for (int64_t j = 0; j < T; j++) s[j] = (s[j] / sum) / keep;
+                for (int64_t d = 0; d < dh; d++) {
+                    float a = 0.0f;
+                    for (int64_t j = 0; j < T; j++) a = s[j] * load_as_f32(qkv, dtype, (b * T + j) * ld + 2 * Cc + h * dh + d) + a;
+                    store_from_f32(y, dtype, (b * T + t) * Cc + h * dh + d, a);
+                }
+                if (lse) lse[bh * T + t] = m + logf(sum);
+            }
+        free(s);
+    }
+}
+
+/* Gradient of the above w.r.t. qkv given dy[B,T,C] (the chain of autograd rules Mul/Div/Exp/Sub/Sum,
+ * zyx/src/graph/autograd.rs:87-134, collapses to the softmax Jacobian; the max term cancels):
+ * P = softmax(scale q k^T) / keep; dV = P^T dO; dP = dO V^T / keep; dS = Ps o (dP - rowsum(Ps o dP)),
+ * Ps = softmax; dQ = scale dS K; dK = scale dS^T Q. Accumulated in f64, stored in `dtype`. */
+ZO_API void zo_attention_bwd(int dtype, const void *qkv, const void *dy, void *dqkv, int64_t B, int64_t T, int64_t H,
+                             int64_t dh, float scale, float keep) {
+    const int64_t Cc = H * dh, ld = 3 * Cc;
+#pragma omp parallel for
+    for (int64_t bh = 0; bh < B * H; bh++) {
+        const int64_t b = bh / H, h = bh % H;
+        double *P = (double *)malloc(sizeof(double) * (size_t)(T * T + 1));
+        double *dS = (double *)malloc(sizeof(double) * (size_t)(T * T + 1));
+        for (int64_t t = 0; t < T; t++) {
+            const int64_t qo = (b * T + t) * ld + h * dh;
+            double m = -INFINITY, sum = 0.0;
+            for (int64_t j = 0; j < T; j++) {
+                const int64_t ko = (b * T + j) * ld + Cc + h * dh;
+                double a = 0.0;
+                for (int64_t d = 0; d < dh; d++) a += (double)load_as_f32(qkv, dtype, qo + d) * (double)load_as_f32(qkv, dtype, ko + d);
+                P[t * T + j] = a * (double)scale;
+                if (P[t * T + j] > m) m = P[t * T + j];
+            }
+            for (int64_t j = 0; j < T; j++) {
+                P[t * T + j] = exp(P[t * T + j] - m);
+                sum += P[t * T + j];
+            }
+            double dot = 0.0;
+            for (int64_t j = 0; j < T; j++) {
+                P[t * T + j] /= sum;
+                double dp = 0.0;
+                for (int64_t d = 0; d < dh; d++)
+                    dp += (double)load_as_f32(dy, dtype, (b * T + t) * Cc + h * dh + d) *
+                          (double)load_as_f32(qkv, dtype, (b * T + j) * ld + 2 * Cc + h * dh + d);
+                dS[t * T + j] = dp / (double)keep;
+                dot += P[t * T + j] * dS[t * T + j];
+            }
+            for (int64_t j = 0; j < T; j++) dS[t * T + j] = P[t * T + j] * (dS[t * T + j] - dot);
+        }
+        for (int64_t t = 0; t < T; t++)
+            for (int64_t d = 0; d < dh; d++) {
+                double dq = 0.0, dk = 0.0, dv = 0.0;
+                for (int64_t j = 0; j < T; j++) {
+                    dq += dS[t * T + j] * (double)load_as_f32(qkv, dtype, (b * T + j) * ld + Cc + h * dh + d);
+                    dk += dS[j * T + t] * (double)load_as_f32(qkv, dtype, (b * T + j) * ld + h * dh + d);
+                    dv += P[j * T + t] / (double)keep * (double)load_as_f32(dy, dtype, (b * T + j) * Cc + h * dh + d);
+                }
+                store_from_f32(dqkv, dtype, (b * T + t) * ld + h * dh + d, (float)(dq * (double)scale));
+                store_from_f32(dqkv, dtype, (b * T + t) * ld + Cc + h * dh + d, (float)(dk * (double)scale));
+                store_from_f32(dqkv, dtype, (b * T + t) * ld + 2 * Cc + h * dh + d, (float)dv);
+            }
+        free(P);
+        free(dS);
+    }
+}

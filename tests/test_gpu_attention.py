@@ -1,0 +1,112 @@
+"""Attention core on the GPU against the oracle (zyx-nn/src/causal_self_attention.rs:36-74 restated) and the
+reference's goldens (zyx/tests/05_misc.rs:1073-1163, zyx-nn/src/causal_self_attention.rs:78-158).
+
+Tolerances: f32 storage 1e-5 relative to max(|y|, sum_j p_j |v_j|) =: mag. bf16 storage: 1e-3 * mag (north star
+for f32-accumulated bf16 matrix products) + 2^-9 * mag (the probabilities enter att.dot(v) as bf16 values, as the
+reference's bf16 `att` tensor does; round-to-nearest moves each by at most half a bf16 ulp) + 2^-7 * |y| (the
+truncating bf16 store of y)."""
+import numpy as np
+import pytest
+
+from zyx_amd import DType
+from zyx_amd.kernels import attention
+
+pytestmark = pytest.mark.gpu
+
+
+def sdpa64(qkv, n_head, scale=None, p=0.0):
+    b, t, c3 = qkv.shape
+    dh = c3 // 3 // n_head
+    q, k, v = [a.reshape(b, t, n_head, dh).transpose(0, 2, 1, 3) for a in np.split(qkv.astype(np.float64), 3, axis=2)]
+    s = np.einsum("bhtd,bhjd->bhtj", q, k) * float(np.float32(1 / np.sqrt(dh)) if scale is None else scale)
+    m = s.max(-1, keepdims=True)
+    e = np.exp(s - m)
+    pr = e / e.sum(-1, keepdims=True) / (1.0 - p)
+    y = np.einsum("bhtj,bhjd->bhtd", pr, v).transpose(0, 2, 1, 3).reshape(b, t, c3 // 3)
+    mag = np.einsum("bhtj,bhjd->bhtd", pr, np.abs(v)).transpose(0, 2, 1, 3).reshape(b, t, c3 // 3)
+    return y, mag, (m + np.log(e.sum(-1, keepdims=True)))[..., 0]
+
+
+def test_reference_goldens_f32(hip, oracle):
+    dev, pool = hip
+    w = np.array([[3, 1, 2, 3, 1, 2, 5, 4, 2, 3, 1, 3], [1, 1, 2, 3, 1, 2, 5, 4, 2, 3, 1, 3],
+                  [3, 1, 5, 3, 1, 2, 5, 4, 2, 3, 1, 3], [3, 1, 2, 3, 1, 2, 5, 8, 2, 3, 1, 3]], np.float32).T
+    x = np.array([[[1, 0, 4, 2], [2, 5, 0, 1], [0, 8, 1, 0], [5, 1, 0, 0]]], np.float32)
+    y = attention(dev, pool, oracle.linear(x, w), 4, DType.F32)
+    assert np.allclose(y, np.tile(np.array([18, 27, 9, 24], np.float32), (1, 4, 1)), rtol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(1, 3, 2, 2), (2, 7, 3, 5), (1, 64, 1, 64), (2, 65, 2, 80), (1, 200, 2, 130), (3, 129, 4, 16)])
+@pytest.mark.parametrize("p", [0.0, 0.25])
+def test_small_kernel_f32(hip, oracle, shape, p):
+    dev, pool = hip
+    b, t, h, dh = shape
+    qkv = oracle.Rng(t + dh).randn((b, t, 3 * h * dh))
+    y, lse = attention(dev, pool, qkv, h, DType.F32, dropout_p=p, want_lse=True)
+    want, mag, lse64 = sdpa64(qkv, h, p=p)
+    assert np.all(np.abs(y - want) <= 1e-5 * np.maximum(np.abs(want), mag) + 1e-7)
+    assert np.allclose(lse, lse64, rtol=1e-5, atol=1e-5)
+    ref, ref_lse = oracle.attention(qkv, h, dropout_p=p, want_lse=True)  # the reference's serial f32 order
+    assert np.all(np.abs(y - ref) <= 2e-5 * np.maximum(np.abs(want), mag) + 1e-7)
+
+
+def bf16_close(oracle, got_bits, want, mag):
+    got = oracle.bf16_to_f32(got_bits).astype(np.float64)
+    return np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + (1e-3 + 2.0 ** -9) * mag
+
+
+@pytest.mark.parametrize("shape", [(1, 128, 1, 64), (2, 256, 3, 64), (1, 1024, 2, 64), (8, 128, 8, 64)])
+def test_mfma_kernel_bf16(hip, oracle, shape):
+    dev, pool = hip
+    b, t, h, dh = shape
+    qkv = oracle.f32_to_bf16(oracle.Rng(t + b).randn((b, t, 3 * h * dh)))
+    y, lse = attention(dev, pool, qkv, h, DType.BF16, want_lse=True)
+    want, mag, lse64 = sdpa64(oracle.bf16_to_f32(qkv), h)
+    assert np.all(bf16_close(oracle, y, want, mag))
+    assert np.allclose(lse, lse64, rtol=1e-4, atol=1e-4)
+    ref = oracle.bf16_to_f32(oracle.attention(qkv, h, dtype=oracle.BF16)).astype(np.float64)  # serial f32, truncating store
+    assert np.all(np.abs(oracle.bf16_to_f32(y) - ref) <= 2.0 ** -6 * np.abs(want) + (1e-3 + 2.0 ** -9) * mag)
+
+
+def test_bf16_ragged_shapes_take_the_general_kernel(hip, oracle):
+    dev, pool = hip
+    for b, t, h, dh in [(2, 100, 2, 64), (1, 128, 2, 32)]:
+        qkv = oracle.f32_to_bf16(oracle.Rng(t).randn((b, t, 3 * h * dh)))
+        y = attention(dev, pool, qkv, h, DType.BF16, dropout_p=0.1)
+        want, mag, _ = sdpa64(oracle.bf16_to_f32(qkv), h, p=float(np.float32(1) - (np.float32(1) - np.float32(0.1))))
+        assert np.all(bf16_close(oracle, y, want, mag))
+
+
+def test_structured_inputs_bf16(hip, oracle):
+    """Cases with closed forms: identical keys give the mean of V; one dominant key selects its V row."""
+    dev, pool = hip
+    b, t, h, dh = 1, 256, 2, 64
+    rng = np.random.default_rng(3)
+    q = rng.standard_normal((b, t, h * dh)).astype(np.float32)
+    k = np.tile(rng.standard_normal((b, 1, h * dh)).astype(np.float32), (1, t, 1))
+    v = rng.integers(-8, 9, size=(b, t, h * dh)).astype(np.float32)
+    y = oracle.bf16_to_f32(attention(dev, pool, oracle.f32_to_bf16(np.concatenate([q, k, v], 2)), h))
+    assert np.allclose(y, np.broadcast_to(v.mean(1, keepdims=True), v.shape), rtol=2.0 ** -7, atol=1e-3)
+    k = np.zeros((b, t, h * dh), np.float32)
+    k[:, 77, :] = 16.0
+    q = np.full((b, t, h * dh), 2.0, np.float32)  # score of key 77: 64*32/8 = 256, others 0
+    y = oracle.bf16_to_f32(attention(dev, pool, oracle.f32_to_bf16(np.concatenate([q, k, v], 2)), h))
+    assert np.array_equal(y, np.broadcast_to(v[:, 77:78, :], v.shape))
+
+
+def test_config5_attention_full_size(hip, oracle):
+    """B=8, T=1024, 16 heads x 64, bf16: every element against the C oracle (f32 registers, serial sums) and
+    2 heads against the f64 textbook form."""
+    dev, pool = hip
+    r = oracle.Rng(42069)
+    qkv = oracle.f32_to_bf16(r.randn((8, 1024, 3072)))
+    y, lse = attention(dev, pool, qkv, 16, want_lse=True)
+    ref, ref_lse = oracle.attention(qkv, 16, dtype=oracle.BF16, want_lse=True)
+    yf, rf = oracle.bf16_to_f32(y), oracle.bf16_to_f32(ref)
+    # mag = sum_j p_j |v_j| stays near E|v| ~ 0.8 for these inputs, so (1e-3 + 2^-9) * mag < 3e-3
+    assert np.all(np.abs(yf - rf) <= 2.0 ** -6 * np.abs(rf) + 3e-3)
+    assert np.allclose(lse, ref_lse, rtol=1e-4, atol=1e-4)
+    sub = np.ascontiguousarray(qkv.reshape(8, 1024, 3, 16, 64)[:1, :, :, :2, :]).reshape(1, 1024, 3 * 128)
+    want, mag, _ = sdpa64(oracle.bf16_to_f32(sub), 2)
+    got = y.reshape(8, 1024, 16, 64)[:1, :, :2, :].reshape(1, 1024, 128)
+    assert np.all(bf16_close(oracle, got, want, mag))

@@ -385,3 +385,64 @@ def test_index_op_goldens(oracle):
     assert sel(x, 1, np.array([2, 0])).tolist() == [[3, 1], [6, 4], [9, 7]]
     assert sel(x, 0, np.array([-1, -3])).tolist() == [[7, 8, 9], [1, 2, 3]]
     assert sel(x, 1, np.array([-2, -1])).tolist() == [[2, 3], [5, 6], [8, 9]]
+
+
+# ---- attention ----------------------------------------------------------------------------------------------
+def test_attention_goldens(oracle):
+    # zyx/tests/05_misc.rs:1073-1163 and zyx/tests/09_graph.rs:64-111: 4 heads of width 1, integer data
+    w = np.array([[3, 1, 2, 3, 1, 2, 5, 4, 2, 3, 1, 3], [1, 1, 2, 3, 1, 2, 5, 4, 2, 3, 1, 3],
+                  [3, 1, 5, 3, 1, 2, 5, 4, 2, 3, 1, 3], [3, 1, 2, 3, 1, 2, 5, 8, 2, 3, 1, 3]], np.float32).T
+    x = np.array([[[1, 0, 4, 2], [2, 5, 0, 1], [0, 8, 1, 0], [5, 1, 0, 0]]], np.float32)
+    qkv = oracle.linear(x, w)  # x.dot(c_attn_weight.t()) with c_attn_weight = w
+    y = oracle.attention(qkv, 4)
+    assert np.allclose(y, np.tile(np.array([18, 27, 9, 24], np.float32), (1, 4, 1)), rtol=1e-5)
+    # zyx-nn/src/causal_self_attention.rs:78-158 (attention1): 2 heads, module applied 5 times
+    w_attn = np.array([[-0.495788, 0.119697, -0.139357, 0.059328], [0.407094, -0.065494, -0.129729, -0.074552],
+                       [0.324870, 0.155732, 0.297099, -0.412060], [0.020193, -0.336263, -0.009602, 0.116321],
+                       [-0.453359, -0.220178, 0.232500, 0.120824], [-0.457052, -0.312347, -0.267674, 0.344709],
+                       [-0.262033, -0.192330, -0.090726, -0.405672], [-0.472127, -0.110653, -0.040921, -0.487143],
+                       [-0.459970, 0.357617, 0.109131, 0.214290], [0.296274, 0.091488, 0.121792, -0.081484],
+                       [-0.097352, -0.116311, -0.033035, 0.236983], [0.078229, 0.294886, 0.363787, -0.383411]], np.float32)
+    w_proj = np.array([[-0.202461, -0.263050, -0.244990, 0.044416], [-0.398643, 0.219820, 0.253934, 0.204294],
+                       [-0.323065, 0.195841, -0.106940, 0.142828], [0.233007, -0.026790, -0.293228, 0.118043]], np.float32)
+    x = np.array([[[-1.363837, -0.801618, -1.304842, -1.664811], [-0.385430, -0.955608, -1.003842, 0.073811],
+                   [-0.785831, 1.030346, 0.593785, -0.214361]]], np.float32)
+    first = oracle.causal_self_attention(x, w_attn, w_proj, 2)
+    assert np.allclose(first, [[[0.04401812, -0.14199661, -0.11446018, 0.03237676],
+                                [0.05587596, -0.12779452, -0.10237779, 0.02773934],
+                                [0.03065444, -0.15511249, -0.12694199, 0.03479434]]], rtol=2e-5, atol=1e-7)
+    for _ in range(4):
+        first = oracle.causal_self_attention(first, w_attn, w_proj, 2)
+    want = np.tile(np.array([-1.34166388e-04, -3.10145377e-04, -3.39602208e-04, 2.14193460e-05], np.float32), (1, 3, 1))
+    assert np.allclose(first, want, rtol=1e-3)
+
+
+def test_attention_against_textbook_and_finite_differences(oracle):
+    """What the goldens leave open: lse, the eval-mode dropout divisor, and the backward. A dense f64 SDPA written
+    with einsum pins the forward; central differences of that f64 function pin the backward (a transposed operand,
+    a missing scale or a dropped softmax-Jacobian term each fail it)."""
+    rng = np.random.default_rng(0)
+    B, T, H, dh, p = 2, 7, 3, 5, 0.25
+    qkv = rng.standard_normal((B, T, 3 * H * dh)).astype(np.float32)
+
+    def f64(qkv64):
+        q, k, v = [a.reshape(B, T, H, dh).transpose(0, 2, 1, 3) for a in np.split(qkv64, 3, axis=2)]
+        s = np.einsum("bhtd,bhjd->bhtj", q, k) * float(np.float32(1 / np.sqrt(dh)))
+        m = s.max(-1, keepdims=True)
+        e = np.exp(s - m)
+        pr = e / e.sum(-1, keepdims=True) / float(np.float32(1) - np.float32(p))
+        return np.einsum("bhtj,bhjd->bhtd", pr, v).transpose(0, 2, 1, 3).reshape(B, T, H * dh), (m + np.log(e.sum(-1, keepdims=True)))[..., 0]
+
+    y, lse = oracle.attention(qkv, H, dropout_p=p, want_lse=True)
+    y64, lse64 = f64(qkv.astype(np.float64))
+    assert np.allclose(y, y64, rtol=1e-5, atol=1e-6) and np.allclose(lse, lse64, rtol=1e-6, atol=1e-6)
+    dy = rng.standard_normal(y.shape).astype(np.float32)
+    got = oracle.attention_bwd(qkv, dy, H, dropout_p=p)
+    num = np.empty(qkv.shape, np.float64)
+    base = qkv.astype(np.float64)
+    for i in np.ndindex(*qkv.shape):
+        hi, lo = base.copy(), base.copy()
+        hi[i] += 1e-5
+        lo[i] -= 1e-5
+        num[i] = ((f64(hi)[0] - f64(lo)[0]) * dy).sum() / 2e-5
+    assert np.allclose(got, num, rtol=1e-4, atol=1e-6)

@@ -1,0 +1,292 @@
+// Fused attention core of zyx-nn's CausalSelfAttention (zyx-nn/src/causal_self_attention.rs:36-74):
+// y = softmax(scale * q.k^T) / keep . v per head, no mask (the reference applies none), reading q, k, v
+// in place from the c_attn output qkv[B, T, 3, H, dh] and writing y[B, T, H*dh], i.e. split / reshape /
+// transpose(1,2) before and transpose(1,2) / reshape after are index arithmetic. The [T, T] score
+// tensors the reference materialises (q.dot(k.t()), softmax, dropout) never leave registers.
+//
+// attn_fwd_bf16_k (bf16, dh = 64, T % 128 == 0): one workgroup per (batch, head, 128 queries), 4 waves
+// of 32 queries. K and V tiles of 64 keys go L2 -> VGPR -> LDS, double buffered. Per tile a wave
+// computes S^T = K.Q^T (keys x queries) with v_mfma_f32_32x32x16_bf16, so that every lane owns one
+// query column: the running max / sum are per-lane scalars, and the exponentiated tile, packed to
+// bf16, already has the register layout of the B operand of O^T += V^T.P^T. V^T fragments come from
+// the row-major V tile through the transposing ds_read_b64_tr_b16. Keys are visited in a permuted
+// order inside each 32-key block (the order the S^T accumulator registers hold them); P and V use
+// the same permutation, and a sum over keys does not depend on it.
+//
+// attn_small_k: any dh <= 256 and T, f32 or bf16 storage, one wave per query, f32 arithmetic with
+// the accurate exponential. Serves the shapes the matrix-core kernel does not take.
+#include "dtypes.hpp"
+#include "kernels.hpp"
+#include "wave.hpp"
+
+namespace zk {
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+#define ZK_LDS __attribute__((address_space(3)))
+
+constexpr int QB = 128, KB = 64, DH = 64;
+constexpr int TILE = KB * DH * 2;   // one K or V tile: 8 KiB
+constexpr int STAGE = 2 * TILE;     // K tile then V tile
+constexpr float kLog2e = 1.44269504088896340736f, kLn2 = 0.69314718055994530942f;
+
+// K tile: [key][16-byte chunk ^ ((key >> 1) & 7)], 128-byte rows: ds_read_b128 of 16 consecutive keys
+// at one logical chunk touches 16 different slots modulo 256 bytes.
+__device__ __forceinline__ int k_slot(int key, int chunk) { return key * 128 + ((chunk ^ ((key >> 1) & 7)) << 4); }
+// V tile: [key][64-byte half ^ ((key >> 1) & 1)][...]: the transposing read of 4 consecutive keys x 32 columns
+// (four 64-byte pieces) covers all 64 banks once.
+__device__ __forceinline__ int v_slot(int key, int chunk) {
+    return key * 128 + (((chunk >> 2) ^ ((key >> 1) & 1)) << 6) + ((chunk & 3) << 4);
+}
+
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+template <bool LSE>
+__global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__restrict__ qkv, uint16_t *__restrict__ y,
+                                                          float *__restrict__ lse, int T, int H, float c, float out_scale) {
+    __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[2 * STAGE];
+    ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
+
+    // Workgroups whose ids are congruent mod 8 share an XCD (and its L2): give every XCD whole heads, so
+    // the K and V of a head are fetched into one L2 only.
+    const int QT = T / QB, BH = (int)gridDim.x / QT;
+    int bh, qt;
+    if (BH % 8 == 0) {
+        const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
+        bh = (i / QT) * 8 + x;
+        qt = i % QT;
+    } else {
+        bh = blockIdx.x / QT;
+        qt = blockIdx.x % QT;
+    }
+    const int bb = bh / H, h = bh % H;
+    const int64_t ld = 3 * (int64_t)H * DH;
+    const uint16_t *qp = qkv + (int64_t)bb * T * ld + h * DH, *kp = qp + H * DH, *vp = kp + H * DH;
+    const int tq = qt * QB + wave * 32 + (lane & 31);
+
+    bf16x8 qf[4]; // B operand of S^T: lane -> query lane % 32, dh = ks*16 + (lane / 32)*8 .. +7
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) qf[ks] = *(const bf16x8 *)(qp + (int64_t)tq * ld + ks * 16 + hh * 8);
+
+    // staging: thread moves chunks tid and tid + 256 of the 512 16-byte chunks of each tile
+    u32x4 rk[2], rv[2];
+    int sk[2], sv[2];
+    uint32_t go[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int ch = tid + 256 * i, key = ch >> 3, cc = ch & 7;
+        go[i] = (uint32_t)(key * ld + cc * 8) * 2;
+        sk[i] = k_slot(key, cc);
+        sv[i] = TILE + v_slot(key, cc);
+    }
+    auto gload = [&](int kt) {
+        const int64_t base = (int64_t)kt * KB * ld * 2;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            rk[i] = *(const u32x4 *)((const uint8_t *)kp + base + go[i]);
+            rv[i] = *(const u32x4 *)((const uint8_t *)vp + base + go[i]);
+        }
+    };
+    auto lwrite = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            *(ZK_LDS u32x4 *)(smem + stage + sk[i]) = rk[i];
+            *(ZK_LDS u32x4 *)(smem + stage + sv[i]) = rv[i];
+        }
+    };
+
+    // fragment offsets inside a stage
+    const int kf = (lane & 31) * 128; // + ((chunk ^ key7) << 4), key7 of row lane%32 (+32 leaves it unchanged)
+    const int key7 = ((lane & 31) >> 1) & 7;
+    int vf[2];
+    {
+        const int g16 = lane >> 4, r = lane & 15, kr = r >> 2;
+#pragma unroll
+        for (int db = 0; db < 2; db++)
+            vf[db] = TILE + (4 * (g16 >> 1) + kr) * 128 + ((db ^ ((kr >> 1) & 1)) << 6) + ((g16 & 1) * 16 + (r & 3) * 4) * 2;
+    }
+
+    f32x16 o[2];
+#pragma unroll
+    for (int db = 0; db < 2; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+
+    const int NT = T / KB;
+    gload(0);
+    lwrite(0);
+    __syncthreads();
+    int stage = 0;
+    for (int kt = 0; kt < NT; kt++) {
+        if (kt + 1 < NT) gload(kt + 1);
+
+        f32x16 s[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[kb][r] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                const bf16x8 a = *(const ZK_LDS bf16x8 *)(smem + stage + kb * 32 * 128 + kf + (((ks * 2 + hh) ^ key7) << 4));
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s[kb], 0, 0, 0);
+            }
+        }
+
+        float bm = s[0][0];
+#pragma unroll
+        for (int r = 1; r < 16; r++) bm = fmaxf(bm, s[0][r]);
+#pragma unroll
+        for (int r = 0; r < 16; r++) bm = fmaxf(bm, s[1][r]);
+        bm = fmaxf(bm, xor32(bm));
+        const float m_new = fmaxf(m, bm * c);
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        m = m_new;
+        float ps = 0.0f;
+        bf16x8 pf[2][2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                f32x8 p;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][8 * s2 + e], c, -m_new));
+                    ps += p[e];
+                }
+                pf[kb][s2] = __builtin_convertvector(p, bf16x8);
+            }
+        l = __builtin_fmaf(l, alpha, ps);
+#pragma unroll
+        for (int db = 0; db < 2; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+                for (int db = 0; db < 2; db++) {
+                    const int off = stage + vf[db] + (kb * 32 + 16 * s2) * 128;
+                    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(smem + off));
+                    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(smem + off + 8 * 128));
+                    const bf16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[kb][s2], o[db], 0, 0, 0);
+                }
+
+        if (kt + 1 < NT) lwrite(stage ^ STAGE);
+        __syncthreads();
+        stage ^= STAGE;
+    }
+
+    l += xor32(l);
+    const float inv = out_scale / l;
+    uint16_t *yp = y + ((int64_t)bb * T + tq) * ((int64_t)H * DH) + h * DH;
+#pragma unroll
+    for (int db = 0; db < 2; db++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            uint32_t w0 = (uint32_t)f32_to_bf16_trunc(o[db][4 * g + 0] * inv) | ((uint32_t)f32_to_bf16_trunc(o[db][4 * g + 1] * inv) << 16);
+            uint32_t w1 = (uint32_t)f32_to_bf16_trunc(o[db][4 * g + 2] * inv) | ((uint32_t)f32_to_bf16_trunc(o[db][4 * g + 3] * inv) << 16);
+            u32x2 w = {w0, w1};
+            *(u32x2 *)(yp + db * 32 + 8 * g + 4 * hh) = w;
+        }
+    if (LSE && hh == 0) lse[(int64_t)bh * T + tq] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+}
+
+// One wave per query. Keys are taken 64 at a time (lane = key) for the scores and the
+// exponentials, then lane = d for the weighted sum of V rows; p[] and q[] live in LDS.
+template <int DT>
+__global__ __launch_bounds__(64) void attn_small_k(const void *__restrict__ qkv_, void *__restrict__ y_, float *__restrict__ lse,
+                                                   int T, int H, int dh, float scale, float keep) {
+    __shared__ float qs[256], ps[64];
+    const int lane = threadIdx.x, t = blockIdx.x, bh = blockIdx.y, bb = bh / H, h = bh % H;
+    const int64_t C = (int64_t)H * dh, ld = 3 * C;
+    auto ldv = [&](int64_t i) -> float {
+        if (DT == DT_F32) return ((const float *)qkv_)[i];
+        return bf16_to_f32(((const uint16_t *)qkv_)[i]);
+    };
+    const int64_t qo = ((int64_t)bb * T + t) * ld + h * dh;
+    for (int d = lane; d < dh; d += 64) qs[d] = ldv(qo + d);
+    __syncthreads();
+    float o[4] = {0.0f, 0.0f, 0.0f, 0.0f}; // d = lane + 64*i
+    float m = -INFINITY, l = 0.0f;
+    for (int j0 = 0; j0 < T; j0 += 64) {
+        const int j = j0 + lane;
+        float s = -INFINITY;
+        if (j < T) {
+            const int64_t ko = ((int64_t)bb * T + j) * ld + C + h * dh;
+            float a = 0.0f;
+            for (int d = 0; d < dh; d++) a = __builtin_fmaf(qs[d], ldv(ko + d), a);
+            s = a * scale;
+        }
+        const float m_new = fmaxf(m, wave_allreduce_f32(s, OpMaxF()));
+        const float p = j < T ? exp_neg(s - m_new) : 0.0f;
+        const float alpha = m == -INFINITY ? 0.0f : exp_neg(m - m_new);
+        l = l * alpha + wave_allreduce_f32(p, OpAdd());
+        m = m_new;
+        __syncthreads(); // ps of the previous chunk has been consumed
+        ps[lane] = p;
+        __syncthreads();
+        const int nk = min(64, T - j0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int d = lane + 64 * i;
+            if (d < dh) {
+                float a = o[i] * alpha;
+                const int64_t vo = ((int64_t)bb * T + j0) * ld + 2 * C + h * dh + d;
+                for (int jj = 0; jj < nk; jj++) a = __builtin_fmaf(ps[jj], ldv(vo + jj * ld), a);
+                o[i] = a;
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int d = lane + 64 * i;
+        if (d < dh) {
+            const float v = (o[i] / l) / keep;
+            const int64_t yo = ((int64_t)bb * T + t) * C + h * dh + d;
+            if (DT == DT_F32) ((float *)y_)[yo] = v;
+            else ((uint16_t *)y_)[yo] = f32_to_bf16_trunc(v);
+        }
+    }
+    if (lse && lane == 0) lse[(int64_t)bh * T + t] = m + logf(l);
+}
+
+} // namespace
+
+bool attention_fast_path(const Attention &p) {
+    return p.dtype == DT_BF16 && p.dh == DH && p.T % QB == 0 && p.T > 0 && p.scale > 0.0f &&
+           (int64_t)p.B * p.H * (p.T / QB) < (1ll << 31) && (int64_t)p.T * 3 * p.H * DH * 2 < (1ll << 31);
+}
+
+hipError_t attention_fwd(const Attention &p, hipStream_t st) {
+    if (p.B <= 0 || p.T <= 0 || p.H <= 0 || p.dh <= 0) return hipSuccess;
+    if (attention_fast_path(p)) {
+        dim3 grid((unsigned)(p.B * p.H * (p.T / QB))), block(256);
+        if (p.lse)
+            hipLaunchKernelGGL(attn_fwd_bf16_k<true>, grid, block, 0, st, (const uint16_t *)p.qkv, (uint16_t *)p.y, p.lse, p.T, p.H,
+                               p.scale * kLog2e, 1.0f / p.keep);
+        else
+            hipLaunchKernelGGL(attn_fwd_bf16_k<false>, grid, block, 0, st, (const uint16_t *)p.qkv, (uint16_t *)p.y, p.lse, p.T, p.H,
+                               p.scale * kLog2e, 1.0f / p.keep);
+        return hipGetLastError();
+    }
+    if (p.dh > 256 || (int64_t)p.B * p.H > 65535 || (p.dtype != DT_F32 && p.dtype != DT_BF16)) return hipErrorInvalidValue;
+    dim3 grid((unsigned)p.T, (unsigned)(p.B * p.H)), block(64);
+    if (p.dtype == DT_F32)
+        hipLaunchKernelGGL(attn_small_k<DT_F32>, grid, block, 0, st, p.qkv, p.y, p.lse, p.T, p.H, p.dh, p.scale, p.keep);
+    else
+        hipLaunchKernelGGL(attn_small_k<DT_BF16>, grid, block, 0, st, p.qkv, p.y, p.lse, p.T, p.H, p.dh, p.scale, p.keep);
+    return hipGetLastError();
+}
+
+} // namespace zk

@@ -118,6 +118,19 @@ struct IndexOp {
 };
 hipError_t index_op(const IndexOp &p, hipStream_t stream);
 
+// Attention core over the packed c_attn output qkv[B, T, 3, H, dh] -> y[B, T, H*dh]:
+// y = softmax(scale q k^T) / keep . v per head, no mask. lse[B, H, T] (optional) = ln sum exp(scale q k^T).
+struct Attention {
+    int B, T, H, dh;
+    int dtype; // DT_BF16 or DT_F32 storage of qkv and y
+    float scale, keep;
+    const void *qkv;
+    void *y;
+    float *lse;
+};
+bool attention_fast_path(const Attention &p);
+hipError_t attention_fwd(const Attention &p, hipStream_t stream);
+
 // cross_entropy of f32 logits [rows, cols] with i32 class indices; loss / grad may be null.
 struct CrossEntropy {
     int64_t rows, cols;

@@ -20,6 +20,7 @@
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
+#include <cmath>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -454,6 +455,21 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.n_out = 1;
         return ZHIP_OK;
     }
+    case ZHIP_K_ATTENTION: {
+        const int64_t B = d.dims[0], T = d.dims[1], H = d.dims[2], dh = d.dims[3];
+        if (B < 0 || T < 0 || H <= 0 || dh <= 0 || dh > 256 || B * H > 65535 || T >= (1ll << 24) || B * T * 3 * H * dh >= (1ll << 40))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "attention: shape out of range (dh <= 256, B*H <= 65535)");
+        if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16) return c->fail(ZHIP_KERNEL_COMPILATION, "attention: dtype must be F32 or BF16");
+        if ((d.flags & ~ZHIP_ATTN_LSE) || d.fparams[0] < 0.0f || !(d.fparams[1] >= 0.0f && d.fparams[1] < 1.0f))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "attention: bad flags, scale or dropout probability");
+        const uint64_t e = dtype_bytes(d.dtype);
+        p.n_in = 1;
+        p.need[0] = (uint64_t)(B * T * 3 * H * dh) * e;
+        p.need[1] = (uint64_t)(B * T * H * dh) * e;
+        p.n_out = 1;
+        if (d.flags & ZHIP_ATTN_LSE) p.need[p.n_out++ + 1] = (uint64_t)(B * H * T) * 4;
+        return ZHIP_OK;
+    }
     default: return c->fail(ZHIP_KERNEL_COMPILATION, "unknown kernel kind %d", d.kind);
     }
 }
@@ -627,6 +643,17 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         a.src = a.scatter ? ptr[2] : nullptr;
         a.out = ptr[p.n_in];
         return zk::index_op(a, st);
+    }
+    case ZHIP_K_ATTENTION: {
+        zk::Attention a{};
+        a.B = (int)d.dims[0]; a.T = (int)d.dims[1]; a.H = (int)d.dims[2]; a.dh = (int)d.dims[3];
+        a.dtype = d.dtype;
+        a.scale = d.fparams[0] > 0.0f ? d.fparams[0] : (float)(1.0 / sqrt((double)a.dh));
+        a.keep = 1.0f - d.fparams[1];
+        a.qkv = ptr[0];
+        a.y = ptr[1];
+        a.lse = (d.flags & ZHIP_ATTN_LSE) ? (float *)ptr[2] : nullptr;
+        return zk::attention_fwd(a, st);
     }
     default: return hipErrorInvalidValue;
     }

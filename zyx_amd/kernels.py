@@ -459,3 +459,41 @@ def scatter(dev: HIPDevice, pool: HIPMemoryPool, x, axis: int, indices, src):
         raise ValueError(f"indices shape {idx.shape} != src shape {src.shape}")
     return _index_run(dev, pool, index_desc(INDEX_SCATTER, x.shape, idx.shape, axis, _DT_OF_NP[x.dtype], idt),
                       [x, idx, src], x.shape, x.dtype)
+
+
+# ---- attention core (ZHIP_K_ATTENTION) -----------------------------------------------------------------------
+K_ATTENTION = 10
+ATTN_LSE = 1
+
+
+def attention_desc(b: int, t: int, n_head: int, dh: int, dtype: DType = DType.BF16, scale: float = 0.0,
+                   dropout_p: float = 0.0, lse: bool = False) -> KernelDesc:
+    d = KernelDesc()
+    d.kind, d.dtype, d.out_dtype, d.flags = K_ATTENTION, DType(dtype), DType(dtype), ATTN_LSE if lse else 0
+    d.dims[0], d.dims[1], d.dims[2], d.dims[3] = b, t, n_head, dh
+    d.fparams[0], d.fparams[1] = scale, dropout_p
+    return d
+
+
+def attention(dev: HIPDevice, pool: HIPMemoryPool, qkv, n_head: int, dtype: DType = DType.BF16, scale: float = 0.0,
+              dropout_p: float = 0.0, want_lse: bool = False):
+    """Core of CausalSelfAttention::forward (zyx-nn/src/causal_self_attention.rs:36-74) on the c_attn output
+    qkv[B,T,3C] (bf16 bit patterns as uint16, or float32) -> y[B,T,C] (, lse[B,H,T])."""
+    qkv = np.ascontiguousarray(qkv)
+    b, t, c3 = qkv.shape
+    c = c3 // 3
+    prog = dev.register_kernel(attention_desc(b, t, n_head, c // n_head, dtype, scale, dropout_p, want_lse))
+    xb, e0 = to_device(pool, qkv)
+    yb, e1 = alloc_like(pool, b * t * c, qkv.dtype.itemsize)
+    bufs, waits = [xb, yb], [e0, e1]
+    if want_lse:
+        lb, e2 = alloc_like(pool, b * n_head * t, 4)
+        bufs.append(lb)
+        waits.append(e2)
+    done = dev.launch(prog, pool, bufs, waits)
+    y = to_host(pool, yb, (b, t, c), qkv.dtype, [done])
+    out = (y, to_host(pool, bufs[2], (b, n_head, t), np.float32, [])) if want_lse else y
+    for buf in bufs:
+        pool.deallocate(buf, [])
+    dev.release(prog)
+    return out
