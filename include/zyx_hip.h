@@ -184,6 +184,13 @@ enum zhip_kernel_kind {
      * flags: ZHIP_ATTN_LSE also writes lse[B, H, T] (f32) = ln sum_j exp(scale q.k_j), which the
      * backward needs. args: qkv, y[B, T, C], (lse). */
     ZHIP_K_ATTENTION = 10,
+    /* Gradient of ZHIP_K_ATTENTION with respect to qkv: what Runtime::gradient
+     * (zyx/src/graph/autograd.rs:14-424) builds from the reverse rules of the forward's ops (Mul :120-125,
+     * Div :126-134, Exp :87-95, Sub :111-119, the reduce rules :299-379), evaluated in one pass:
+     * dV = P^T.dy, dS = Ps o (dy.v^T / (1-p) - rowsum(dy o y)), dQ = scale dS.k, dK = scale dS^T.q, with the
+     * probabilities recomputed from lse. dims, dtype, fparams as for ZHIP_K_ATTENTION.
+     * args: qkv, y, dy[B, T, C], lse[B, H, T] (the forward's inputs and outputs), then dqkv[B, T, 3*C]. */
+    ZHIP_K_ATTENTION_BWD = 11,
     ZHIP_K_COUNT_
 };
 #define ZHIP_SOFTMAX_Y 1

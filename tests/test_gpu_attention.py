@@ -110,3 +110,83 @@ def test_config5_attention_full_size(hip, oracle):
     want, mag, _ = sdpa64(oracle.bf16_to_f32(sub), 2)
     got = y.reshape(8, 1024, 16, 64)[:1, :, :2, :].reshape(1, 1024, 128)
     assert np.all(bf16_close(oracle, got, want, mag))
+
+
+# ---- backward ---------------------------------------------------------------------------------------------------
+from zyx_amd.kernels import attention_bwd
+
+
+def grad64(qkv, dy, n_head, p=0.0):
+    """Textbook gradient in f64 (numpy), with the magnitude sums the tolerances are relative to."""
+    b, t, c3 = qkv.shape
+    dh = c3 // 3 // n_head
+    sc = float(np.float32(1 / np.sqrt(dh)))
+    q, k, v = [a.reshape(b, t, n_head, dh).transpose(0, 2, 1, 3) for a in np.split(qkv.astype(np.float64), 3, axis=2)]
+    do = dy.astype(np.float64).reshape(b, t, n_head, dh).transpose(0, 2, 1, 3)
+    s = np.einsum("bhtd,bhjd->bhtj", q, k) * sc
+    e = np.exp(s - s.max(-1, keepdims=True))
+    ps = e / e.sum(-1, keepdims=True)
+    dps = np.einsum("bhtd,bhjd->bhtj", do, v) / (1 - p)
+    ds = ps * (dps - (ps * dps).sum(-1, keepdims=True))
+    ads = ps * (np.abs(dps) + (ps * np.abs(dps)).sum(-1, keepdims=True))
+    back = lambda a: a.transpose(0, 2, 1, 3).reshape(b, t, n_head * dh)
+    g = np.concatenate([back(np.einsum("bhtj,bhjd->bhtd", ds, k) * sc), back(np.einsum("bhtj,bhtd->bhjd", ds, q) * sc),
+                        back(np.einsum("bhtj,bhtd->bhjd", ps, do) / (1 - p))], 2)
+    mag = np.concatenate([back(np.einsum("bhtj,bhjd->bhtd", ads, np.abs(k)) * sc), back(np.einsum("bhtj,bhtd->bhjd", ads, np.abs(q)) * sc),
+                          back(np.einsum("bhtj,bhtd->bhjd", ps, np.abs(do)) / (1 - p))], 2)
+    return g, mag
+
+
+@pytest.mark.parametrize("shape", [(1, 3, 2, 2), (2, 7, 3, 5), (2, 65, 2, 80), (1, 130, 2, 130)])
+@pytest.mark.parametrize("p", [0.0, 0.25])
+def test_backward_small_kernel_f32(hip, oracle, shape, p):
+    dev, pool = hip
+    b, t, h, dh = shape
+    qkv = oracle.Rng(t + dh).randn((b, t, 3 * h * dh))
+    dy = oracle.Rng(t).randn((b, t, h * dh))
+    y, lse = attention(dev, pool, qkv, h, DType.F32, dropout_p=p, want_lse=True)
+    got = attention_bwd(dev, pool, qkv, y, dy, lse, h, DType.F32, dropout_p=p)
+    keep = float(np.float32(1) - np.float32(p))
+    want, mag = grad64(qkv, dy, h, 1 - keep)
+    assert np.all(np.abs(got - want) <= 2e-5 * mag + 1e-7)
+    assert np.all(np.abs(got - oracle.attention_bwd(qkv, dy, h, dropout_p=p)) <= 2e-5 * mag + 1e-7)
+
+
+@pytest.mark.parametrize("shape", [(1, 128, 1, 64), (2, 256, 3, 64), (1, 512, 8, 64)])
+def test_backward_mfma_kernel_bf16(hip, oracle, shape):
+    """bf16 operands (P, dS, dy, q, k, v are bf16 matrix-core operands): 1e-3 of the magnitude sum for the f32
+    accumulation, 2^-8 of it for operand rounding of P / dS, one bf16 ulp for the truncating store."""
+    dev, pool = hip
+    b, t, h, dh = shape
+    qkv = oracle.f32_to_bf16(oracle.Rng(t + b).randn((b, t, 3 * h * dh)))
+    dy = oracle.f32_to_bf16(oracle.Rng(t).randn((b, t, h * dh)))
+    y, lse = attention(dev, pool, qkv, h, DType.BF16, want_lse=True)
+    got = oracle.bf16_to_f32(attention_bwd(dev, pool, qkv, y, dy, lse, h, DType.BF16)).astype(np.float64)
+    want, mag = grad64(oracle.bf16_to_f32(qkv), oracle.bf16_to_f32(dy), h)
+    assert np.all(np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + (1e-3 + 2.0 ** -8) * mag)
+    # the same through the general kernel (a shape the matrix-core path does not take) agrees as well
+    if t == 128:
+        y2, lse2 = attention(dev, pool, qkv[:, :100], h, DType.BF16, want_lse=True)
+        got2 = oracle.bf16_to_f32(attention_bwd(dev, pool, qkv[:, :100], y2, dy[:, :100], lse2, h, DType.BF16)).astype(np.float64)
+        want2, mag2 = grad64(oracle.bf16_to_f32(qkv[:, :100]), oracle.bf16_to_f32(dy[:, :100]), h)
+        assert np.all(np.abs(got2 - want2) <= 2.0 ** -7 * np.abs(want2) + 2e-3 * mag2)
+
+
+def test_config5_attention_backward_full_size(hip, oracle):
+    """B=8, T=1024, 16 x 64 bf16: two (batch, head) pairs against the f64 gradient; all of it through
+    d/dv linearity: sum_t dV[t] equals sum over queries of P^T dy, i.e. column sums of dV per head equal
+    column sums of dy per head (rows of P sum to one)."""
+    dev, pool = hip
+    qkv = oracle.f32_to_bf16(oracle.Rng(42069).randn((8, 1024, 3072)))
+    dy = oracle.f32_to_bf16(oracle.Rng(7).randn((8, 1024, 1024)))
+    y, lse = attention(dev, pool, qkv, 16, want_lse=True)
+    got = oracle.bf16_to_f32(attention_bwd(dev, pool, qkv, y, dy, lse, 16))
+    dv_sum = got[:, :, 2048:].astype(np.float64).sum(1)
+    dy_sum = oracle.bf16_to_f32(dy).astype(np.float64).sum(1)
+    assert np.all(np.abs(dv_sum - dy_sum) <= 2.0 ** -7 * np.abs(oracle.bf16_to_f32(dy)).astype(np.float64).sum(1))
+    for bsel, hsel in [(0, 0), (7, 15)]:
+        cols = np.concatenate([np.arange(64) + 1024 * i + 64 * hsel for i in range(3)])
+        sub, dsub = qkv[bsel:bsel + 1][:, :, cols], dy[bsel:bsel + 1, :, 64 * hsel:64 * hsel + 64]
+        want, mag = grad64(oracle.bf16_to_f32(sub), oracle.bf16_to_f32(dsub), 1)
+        g = got[bsel:bsel + 1][:, :, cols].astype(np.float64)
+        assert np.all(np.abs(g - want) <= 2.0 ** -7 * np.abs(want) + (1e-3 + 2.0 ** -8) * mag)

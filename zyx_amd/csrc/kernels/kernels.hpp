@@ -130,6 +130,16 @@ struct Attention {
 };
 bool attention_fast_path(const Attention &p);
 hipError_t attention_fwd(const Attention &p, hipStream_t stream);
+// d(sum(y o dy)) / d(qkv): fwd.y and fwd.lse are the forward's outputs (inputs here), dy[B, T, H*dh] the
+// incoming gradient, dqkv[B, T, 3, H, dh] the result. workspace: attention_bwd_workspace_bytes(fwd) bytes.
+struct AttentionBwd {
+    Attention fwd;
+    const void *dy;
+    void *dqkv;
+    void *workspace;
+};
+uint64_t attention_bwd_workspace_bytes(const Attention &p);
+hipError_t attention_bwd(const AttentionBwd &p, hipStream_t stream);
 
 // cross_entropy of f32 logits [rows, cols] with i32 class indices; loss / grad may be null.
 struct CrossEntropy {

@@ -252,6 +252,19 @@ uint64_t dtype_bytes(int32_t dt) {
 }
 
 // Fills arity and per-argument byte requirements; rejects shapes/dtypes no kernel covers.
+// Shape and scalar parameters of the two attention kinds.
+zk::Attention attention_args(const zhip_kernel_desc &d) {
+    zk::Attention a{};
+    a.B = (int)d.dims[0];
+    a.T = (int)d.dims[1];
+    a.H = (int)d.dims[2];
+    a.dh = (int)d.dims[3];
+    a.dtype = d.dtype;
+    a.scale = d.fparams[0] > 0.0f ? d.fparams[0] : (float)(1.0 / sqrt((double)a.dh));
+    a.keep = 1.0f - d.fparams[1];
+    return a;
+}
+
 int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
     p.desc = d;
     switch (d.kind) {
@@ -455,7 +468,8 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.n_out = 1;
         return ZHIP_OK;
     }
-    case ZHIP_K_ATTENTION: {
+    case ZHIP_K_ATTENTION:
+    case ZHIP_K_ATTENTION_BWD: {
         const int64_t B = d.dims[0], T = d.dims[1], H = d.dims[2], dh = d.dims[3];
         if (B < 0 || T < 0 || H <= 0 || dh <= 0 || dh > 256 || B * H > 65535 || T >= (1ll << 24) || B * T * 3 * H * dh >= (1ll << 40))
             return c->fail(ZHIP_KERNEL_COMPILATION, "attention: shape out of range (dh <= 256, B*H <= 65535)");
@@ -463,6 +477,17 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         if ((d.flags & ~ZHIP_ATTN_LSE) || d.fparams[0] < 0.0f || !(d.fparams[1] >= 0.0f && d.fparams[1] < 1.0f))
             return c->fail(ZHIP_KERNEL_COMPILATION, "attention: bad flags, scale or dropout probability");
         const uint64_t e = dtype_bytes(d.dtype);
+        if (d.kind == ZHIP_K_ATTENTION_BWD) {
+            if (d.flags) return c->fail(ZHIP_KERNEL_COMPILATION, "attention backward takes no flags");
+            p.n_in = 4;
+            p.need[0] = (uint64_t)(B * T * 3 * H * dh) * e;
+            p.need[1] = p.need[2] = (uint64_t)(B * T * H * dh) * e;
+            p.need[3] = (uint64_t)(B * H * T) * 4;
+            p.need[4] = p.need[0];
+            p.n_out = 1;
+            p.workspace_bytes = zk::attention_bwd_workspace_bytes(attention_args(d));
+            return ZHIP_OK;
+        }
         p.n_in = 1;
         p.need[0] = (uint64_t)(B * T * 3 * H * dh) * e;
         p.need[1] = (uint64_t)(B * T * H * dh) * e;
@@ -644,12 +669,19 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         a.out = ptr[p.n_in];
         return zk::index_op(a, st);
     }
+    case ZHIP_K_ATTENTION_BWD: {
+        zk::AttentionBwd a{};
+        a.fwd = attention_args(d);
+        a.fwd.qkv = ptr[0];
+        a.fwd.y = ptr[1];
+        a.dy = ptr[2];
+        a.fwd.lse = (float *)ptr[3];
+        a.dqkv = ptr[4];
+        a.workspace = p.workspace;
+        return zk::attention_bwd(a, st);
+    }
     case ZHIP_K_ATTENTION: {
-        zk::Attention a{};
-        a.B = (int)d.dims[0]; a.T = (int)d.dims[1]; a.H = (int)d.dims[2]; a.dh = (int)d.dims[3];
-        a.dtype = d.dtype;
-        a.scale = d.fparams[0] > 0.0f ? d.fparams[0] : (float)(1.0 / sqrt((double)a.dh));
-        a.keep = 1.0f - d.fparams[1];
+        zk::Attention a = attention_args(d);
         a.qkv = ptr[0];
         a.y = ptr[1];
         a.lse = (d.flags & ZHIP_ATTN_LSE) ? (float *)ptr[2] : nullptr;

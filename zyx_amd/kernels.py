@@ -497,3 +497,33 @@ def attention(dev: HIPDevice, pool: HIPMemoryPool, qkv, n_head: int, dtype: DTyp
         pool.deallocate(buf, [])
     dev.release(prog)
     return out
+
+
+K_ATTENTION_BWD = 11
+
+
+def attention_bwd_desc(b: int, t: int, n_head: int, dh: int, dtype: DType = DType.BF16, scale: float = 0.0,
+                       dropout_p: float = 0.0) -> KernelDesc:
+    d = attention_desc(b, t, n_head, dh, dtype, scale, dropout_p)
+    d.kind = K_ATTENTION_BWD
+    return d
+
+
+def attention_bwd(dev: HIPDevice, pool: HIPMemoryPool, qkv, y, dy, lse, n_head: int, dtype: DType = DType.BF16,
+                  scale: float = 0.0, dropout_p: float = 0.0):
+    """Gradient of `attention` with respect to qkv given dy; y and lse are the forward's outputs."""
+    qkv = np.ascontiguousarray(qkv)
+    b, t, c3 = qkv.shape
+    prog = dev.register_kernel(attention_bwd_desc(b, t, n_head, c3 // 3 // n_head, dtype, scale, dropout_p))
+    bufs, waits = [], []
+    for a in (qkv, np.ascontiguousarray(y, qkv.dtype), np.ascontiguousarray(dy, qkv.dtype), np.ascontiguousarray(lse, np.float32)):
+        buf, e = to_device(pool, a)
+        bufs.append(buf)
+        waits.append(e)
+    ob, e = alloc_like(pool, qkv.size, qkv.dtype.itemsize)
+    done = dev.launch(prog, pool, bufs + [ob], waits + [e])
+    out = to_host(pool, ob, qkv.shape, qkv.dtype, [done])
+    for buf in bufs + [ob]:
+        pool.deallocate(buf, [])
+    dev.release(prog)
+    return out
