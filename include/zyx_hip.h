@@ -133,10 +133,12 @@ enum zhip_kernel_kind {
      * narrowing stores truncate); flags bit 0: A is stored [K,M], bit 1: B is stored [N,K]
      * (a Linear weight [out,in]);
      * iparams[0] = epilogue: 0 none, 1 + bias, 2 + bias then ReLU, 3 + bias then GELU;
-     * iparams[1] = dtype of bias; fparams[0] = alpha scaling the product (0 = 1).
-     * Products and sums are f32. bf16 -> f32 problems with M, N multiples of 256 and K a
-     * multiple of 64 run on the 256x256 LDS-tiled MFMA kernel, the rest on a 64x64 one.
-     * args: A, B, (bias when iparams[0] != 0), then C. */
+     * iparams[1] = dtype of bias; iparams[2] != 0: a residual[batch, M, N] of dtype out_dtype is
+     * added last (the `x + module(x)` of a transformer block, zyx-examples/examples/nanogpt.rs:89-95);
+     * fparams[0] = alpha scaling the product (0 = 1).
+     * Products and sums are f32. bf16 problems with M, N multiples of 256 and K a multiple of
+     * 64 run on the 256x256 LDS-tiled MFMA kernel, the rest on a 64x64 one.
+     * args: A, B, (bias when iparams[0] != 0), (residual when iparams[2] != 0), then C. */
     ZHIP_K_GEMM = 4,
     /* y = LayerNorm(x) or RMSNorm(x) over the last axis of x[rows, cols] (dims = {rows, cols},
      * dtype F32 or BF16 for x, weight, bias and y, f32 arithmetic, one narrowing store).

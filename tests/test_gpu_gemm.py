@@ -161,3 +161,27 @@ def test_batched_and_scaled(hip, oracle):
     want = np.einsum("bik,bjk->bij", q.astype(np.float64), k.astype(np.float64)) * 0.125
     assert got.shape == (6, 40, 50)
     assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("mnk", [(256, 512, 128), (100, 70, 50)])
+@pytest.mark.parametrize("epilogue", ["none", "gelu"])
+def test_bf16_output_and_residual(hip, oracle, mnk, epilogue):
+    """bf16 C with the truncating store, and the fused residual add (x + Linear(x)): both kernels."""
+    dev, pool = hip
+    m, n, k = mnk
+    a, b = make(oracle, m, n, k, 11, trans_b=True)
+    r = oracle.Rng(5)
+    bias = oracle.f32_to_bf16(r.uniform((n,), -1, 1))
+    res = oracle.f32_to_bf16(r.randn((m, n)))
+    kw = dict(bias=bias, epilogue="bias" if epilogue == "none" else "bias_gelu", bias_dtype=DType.BF16, trans_b=True)
+    want, mag = reference(oracle, a, b, False, True)
+    want = want + oracle.bf16_to_f32(bias).astype(np.float64)
+    if epilogue == "gelu":
+        want = 0.5 * want * (1 + np.tanh(np.sqrt(2 / np.pi) * (want + 0.044715 * want ** 3)))
+    for residual in (None, res):
+        w = want + (oracle.bf16_to_f32(res).astype(np.float64) if residual is not None else 0.0)
+        got32 = gemm(dev, pool, a, b, out_dtype=DType.F32, residual=None if residual is None else oracle.bf16_to_f32(res), **kw)
+        assert np.all(np.abs(got32 - w) <= 1e-3 * np.abs(w) + 2e-5 * mag + 1e-6)
+        got16 = gemm(dev, pool, a, b, out_dtype=DType.BF16, residual=residual, **kw)
+        # the bf16 result is the truncation of the f32 one (identical arithmetic before the store)
+        assert np.array_equal(got16, oracle.f32_to_bf16(got32))

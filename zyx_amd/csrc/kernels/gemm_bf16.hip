@@ -120,8 +120,9 @@ __device__ __forceinline__ float gelu_fast(float x) {
 // instead of [K, N]. EPI: 0 none, 1 + bias, 2 + bias then ReLU, 3 + bias then GELU.
 template <bool AT, bool BT, int EPI>
 __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
-                                                      float *__restrict__ C, const void *__restrict__ bias,
-                                                      int bias_dtype, int M, int N, int K) {
+                                                      void *__restrict__ Cv, const void *__restrict__ bias,
+                                                      const void *__restrict__ residual, int bias_dtype, int out_bf16,
+                                                      int M, int N, int K) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -285,6 +286,12 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
 
     // C tile of a 32x32 MFMA: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.
     const int col_in = lane & 31, row_in = (lane >> 5) * 4;
+    auto finish = [&](float v, float bv) {
+        if (EPI >= 1) v += bv;
+        if (EPI == 2) v = (v > 0.0f ? 1.0f : 0.0f) * v;
+        if (EPI == 3) v = gelu_fast(v);
+        return v;
+    };
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int col = n0 + wn * 128 + j * 32 + col_in;
@@ -293,17 +300,42 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
             if (bias_dtype == DT_BF16) bv = bf16_to_f32(((const uint16_t *)bias)[col]);
             else bv = ((const float *)bias)[col];
         }
+        if (!out_bf16) {
+            float *C = (float *)Cv;
+            const float *R = (const float *)residual;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int rbase = m0 + wm * 128 + i * 32 + row_in;
+            for (int i = 0; i < 4; i++) {
+                const int rbase = m0 + wm * 128 + i * 32 + row_in;
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int row = rbase + (r >> 2) * 8 + (r & 3);
-                float v = acc[i][j][r];
-                if (EPI >= 1) v += bv;
-                if (EPI == 2) v = (v > 0.0f ? 1.0f : 0.0f) * v;
-                if (EPI == 3) v = gelu_fast(v);
-                C[(int64_t)row * N + col] = v;
+                for (int r = 0; r < 16; r++) {
+                    const int64_t o = (int64_t)(rbase + (r >> 2) * 8 + (r & 3)) * N + col;
+                    float v = finish(acc[i][j][r], bv);
+                    if (R) v += R[o];
+                    C[o] = v;
+                }
+            }
+        } else {
+            // bf16 result: neighbouring lanes trade one value of each register pair, so that the even lane
+            // holds columns (c, c+1) of row r and the odd lane columns (c-1, c) of row r+1: 4-byte stores.
+            uint16_t *C = (uint16_t *)Cv;
+            const uint16_t *R = (const uint16_t *)residual;
+            const int odd = lane & 1;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int rbase = m0 + wm * 128 + i * 32 + row_in;
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    const float v0 = finish(acc[i][j][r], bv), v1 = finish(acc[i][j][r + 1], bv);
+                    const float got = dpp_f32<kDppQuadXor1>(odd ? v0 : v1);
+                    float lo = odd ? got : v0, hi = odd ? v1 : got;
+                    const int64_t o = (int64_t)(rbase + (r >> 2) * 8 + (r & 3) + odd) * N + (col - odd);
+                    if (R) {
+                        const uint32_t rr = *(const uint32_t *)(R + o);
+                        lo += __uint_as_float(rr << 16);
+                        hi += __uint_as_float(rr & 0xffff0000u);
+                    }
+                    *(uint32_t *)(C + o) = (uint32_t)f32_to_bf16_trunc(lo) | ((uint32_t)f32_to_bf16_trunc(hi) << 16);
+                }
             }
         }
     }
@@ -313,7 +345,7 @@ template <bool AT, bool BT> hipError_t launch_epi(const GemmBf16 &p, hipStream_t
     dim3 grid((unsigned)((p.M / BM) * (p.N / BN))), block(256);
 #define ZK_GEMM(E)                                                                                                    \
     hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E>), grid, block, GEMM_LDS, st, (const uint16_t *)p.A,                    \
-                       (const uint16_t *)p.B, (float *)p.C, p.bias, p.bias_dtype, (int)p.M, (int)p.N, (int)p.K);
+                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K);
     switch (p.epilogue) {
     case 0: ZK_GEMM(0) break;
     case 1: ZK_GEMM(1) break;

@@ -134,6 +134,12 @@ __global__ __launch_bounds__(256) void gemm_generic_k(const GemmGeneric p) {
         if (p.epilogue == 2) v = (v > 0.0f ? 1.0f : 0.0f) * v;
         if (p.epilogue == 3) v = gelu_ref(v);
         const int64_t o = row * p.N + col;
+        if (p.residual) {
+            const char *R = (const char *)p.residual + (int64_t)blockIdx.z * p.batch_c * (ODT == DT_F32 ? 4 : 2);
+            if (ODT == DT_F32) v += ((const float *)R)[o];
+            else if (ODT == DT_BF16) v += bf16_to_f32(((const uint16_t *)R)[o]);
+            else v += f16_to_f32(((const uint16_t *)R)[o]);
+        }
         if (ODT == DT_F32) ((float *)C)[o] = v;
         else if (ODT == DT_BF16) ((uint16_t *)C)[o] = f32_to_bf16_trunc(v);
         else ((uint16_t *)C)[o] = f32_to_f16_trunc(v);

@@ -45,14 +45,16 @@ struct Reduce {
 uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int axis0);
 hipError_t reduce(const Reduce &p, hipStream_t stream);
 
-// C[M,N] (f32) = op(A) . op(B) (+ bias[N], + activation), bf16 operands, f32 accumulate.
+// C[M,N] = op(A) . op(B) (+ bias[N], + activation) (+ residual[M,N]), bf16 operands, f32 accumulate;
+// C and the residual are f32, or bf16 (truncating store) when out_bf16 is set.
 // trans_a: A is stored [K,M]; trans_b: B is stored [N,K] (a Linear weight [out,in]).
 struct GemmBf16 {
     int64_t M, N, K;
     int trans_a, trans_b;
     int epilogue;      // 0 none, 1 bias, 2 bias+relu, 3 bias+gelu
     int bias_dtype;    // DT_BF16 or DT_F32
-    const void *A, *B, *bias;
+    int out_bf16;
+    const void *A, *B, *bias, *residual; // residual may be null
     void *C;
 };
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K);
@@ -69,7 +71,7 @@ struct GemmGeneric {
     int trans_a, trans_b;
     int epilogue, bias_dtype;
     float alpha;
-    const void *A, *B, *bias;
+    const void *A, *B, *bias, *residual; // residual (dtype out_dtype, [batch, M, N]) may be null
     void *C;
 };
 hipError_t gemm_generic(const GemmGeneric &p, hipStream_t stream);

@@ -357,6 +357,7 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.need[a++] = (uint64_t)batch * M * K * dtype_bytes(d.dtype);
         p.need[a++] = (uint64_t)batch * K * N * dtype_bytes(d.dtype);
         if (epi) p.need[a++] = (uint64_t)N * dtype_bytes(d.iparams[1]);
+        if (d.iparams[2]) p.need[a++] = (uint64_t)batch * M * N * dtype_bytes(d.out_dtype);
         p.n_in = a;
         p.need[a] = (uint64_t)batch * M * N * dtype_bytes(d.out_dtype);
         p.n_out = 1;
@@ -566,7 +567,8 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
     case ZHIP_K_GEMM: {
         const int64_t batch = d.dims[3] ? d.dims[3] : 1;
         const float alpha = d.fparams[0] == 0.0f ? 1.0f : d.fparams[0];
-        const bool fast = d.dtype == ZHIP_BF16 && d.out_dtype == ZHIP_F32 && batch == 1 && alpha == 1.0f &&
+        const void *residual = d.iparams[2] ? ptr[p.n_in - 1] : nullptr;
+        const bool fast = d.dtype == ZHIP_BF16 && batch == 1 && alpha == 1.0f &&
                           (d.iparams[0] == 0 || d.iparams[1] != ZHIP_F16) && zk::gemm_bf16_supported(d.dims[0], d.dims[1], d.dims[2]);
         if (fast) {
             zk::GemmBf16 a{};
@@ -580,6 +582,8 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
             a.A = ptr[0];
             a.B = ptr[1];
             a.bias = a.epilogue ? ptr[2] : nullptr;
+            a.residual = residual;
+            a.out_bf16 = d.out_dtype == ZHIP_BF16;
             a.C = ptr[p.n_in];
             return zk::gemm_bf16(a, st);
         }
@@ -601,6 +605,7 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         g.A = ptr[0];
         g.B = ptr[1];
         g.bias = g.epilogue ? ptr[2] : nullptr;
+        g.residual = residual;
         g.C = ptr[p.n_in];
         return zk::gemm_generic(g, st);
     }
