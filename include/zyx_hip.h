@@ -193,6 +193,15 @@ enum zhip_kernel_kind {
      * probabilities recomputed from lse. dims, dtype, fparams as for ZHIP_K_ATTENTION.
      * args: qkv, y, dy[B, T, C], lse[B, H, T] (the forward's inputs and outputs), then dqkv[B, T, 3*C]. */
     ZHIP_K_ATTENTION_BWD = 11,
+    /* Gradients of ZHIP_K_NORM_ROWS (LayerNorm zyx-nn/src/layer_norm.rs:98-135, RMSNorm rms_norm.rs:26-32)
+     * as Runtime::gradient derives them (zyx/src/graph/autograd.rs:87-134, 299-379), one fused pass per row:
+     * LayerNorm dx = rstd (g - mean(g) - xh sum(g xh)/(n-1)), g = dy*w, xh = (x-mean) rstd (the n-1 is the
+     * unbiased variance of the forward); RMSNorm dx = r g - r^3 x sum(g x)/n; dw = sum_rows dy*xh,
+     * db = sum_rows dy. dims = {rows, cols}; dtype F32 or BF16; fparams[0] = eps; flags: ZHIP_NORM_RMS,
+     * ZHIP_NORM_WEIGHT (w is passed and dw is wanted), ZHIP_NORM_BIAS (db is wanted),
+     * ZHIP_NORM_ADD (a tensor [rows, cols] that is added to dx: the skip branch of x + f(norm(x))).
+     * args: x, (w), dy, (add), then dx, (dw), (db). */
+    ZHIP_K_NORM_ROWS_BWD = 12,
     ZHIP_K_COUNT_
 };
 #define ZHIP_SOFTMAX_Y 1
@@ -201,6 +210,7 @@ enum zhip_kernel_kind {
 #define ZHIP_NORM_RMS 1
 #define ZHIP_NORM_WEIGHT 2
 #define ZHIP_NORM_BIAS 4
+#define ZHIP_NORM_ADD 8
 #define ZHIP_CE_LOSS 1
 #define ZHIP_CE_GRAD 2
 #define ZHIP_INDEX_GATHER 0
@@ -233,6 +243,10 @@ enum zhip_ew_op {
     ZHIP_EW_RELU, ZHIP_EW_TANH, ZHIP_EW_GELU, ZHIP_EW_SIGMOID, ZHIP_EW_RSQRT,
     /* Cast to an integer dtype inside a float chain: truncation toward zero (c.rs:243-261) */
     ZHIP_EW_CAST_INT,
+    /* acc = d gelu(acc) / d acc: what the reverse rules of zyx/src/graph/autograd.rs:87-134 give for the
+     * ops gelu is written in (elementwise.rs:168-170): 0.5(1+t) + 0.5x(1-t^2)*sqrt(2/pi)(1+3*0.044715x^2),
+     * t = tanh(sqrt(2/pi)(x+0.044715x^3)) */
+    ZHIP_EW_GELU_GRAD,
     ZHIP_EW_OP_COUNT_
 };
 enum zhip_ew_bcast { ZHIP_EW_FULL = 0, ZHIP_EW_ROW = 1, ZHIP_EW_COL = 2, ZHIP_EW_SCALAR = 3 };

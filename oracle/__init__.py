@@ -432,3 +432,19 @@ def causal_self_attention(x, w_attn, w_proj, n_head: int, b_attn=None, b_proj=No
     qkv = linear(x, w_attn, b_attn, dtype)
     y = attention(qkv, n_head, None, dropout_p, dtype)
     return linear(y, w_proj, b_proj, dtype)
+
+
+def norm_bwd(x, dy, w=None, add=None, rms: bool = False, eps: float = 1e-5, dtype: int = F32, want_db: bool = True):
+    """Gradients of layer_norm / rms_norm: (dx (+ add), dw or None, db or None)."""
+    st = _store_dtype(dtype)
+    x = np.ascontiguousarray(x, st)
+    rows, cols = x.shape
+    dy = np.ascontiguousarray(dy, st)
+    w = None if w is None else np.ascontiguousarray(w, st)
+    add = None if add is None else np.ascontiguousarray(add, st)
+    dx = np.empty_like(x)
+    dw = np.empty(cols, st) if w is not None else None
+    db = np.empty(cols, st) if want_db and not rms else None
+    lib().zo_norm_bwd(dtype, int(rms), _p(x), _p(w), _p(dy), _p(add), _p(dx), _p(dw), _p(db), _I64(rows), _I64(cols),
+                      C.c_float(eps))
+    return dx, dw, db

@@ -211,6 +211,15 @@ static inline float zo_gelu(float x) {
     return (x * 0.5f) * (zo_tanh(inner) + 1.0f);
 }
 
+/* d gelu / dx, the product/chain rules (zyx/src/graph/autograd.rs:87-134) applied to the expression above;
+ * tanh saturates to 1 where exp(2z) overflows. */
+static inline float zo_gelu_grad(float x) {
+    const float k = sqrtf(2.0f / 3.14159265358979323846f), x2 = x * x;
+    const float z = (x + x2 * x * 0.044715f) * k;
+    const float t = (z + z) > 88.0f ? 1.0f : zo_tanh(z);
+    return 0.5f * (1.0f + t) + (0.5f * x) * ((1.0f - t * t) * (k * (1.0f + 0.134145f * x2)));
+}
+
 static inline float zo_unary(int op, float x) {
     switch (op) {
     case ZO_U_NEG: return -x;
@@ -482,7 +491,7 @@ static inline int32_t ew_load_i(const void *p, int dtype, int64_t i) {
 enum { EW_LOAD = 0, EW_SAVE, EW_NEG, EW_BITNOT, EW_EXP, EW_EXP2, EW_LN, EW_LOG2, EW_RECIPROCAL, EW_SQRT, EW_SIN, EW_COS,
        EW_FLOOR, EW_TRUNC, EW_ABS, EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_POW, EW_MOD, EW_CMPLT, EW_CMPGT, EW_CMPGE, EW_MAX,
        EW_OR, EW_AND, EW_BITXOR, EW_BITOR, EW_BITAND, EW_SHL, EW_SHR, EW_NOTEQ, EW_EQ, EW_RSUB, EW_RDIV, EW_WHERE,
-       EW_MAD, EW_RELU, EW_TANH, EW_GELU, EW_SIGMOID, EW_RSQRT, EW_CAST_INT };
+       EW_MAD, EW_RELU, EW_TANH, EW_GELU, EW_SIGMOID, EW_RSQRT, EW_CAST_INT, EW_GELU_GRAD };
 
 static inline float ew_op_f(int op, float x, float a, float b) {
     switch (op) {
@@ -523,6 +532,7 @@ static inline float ew_op_f(int op, float x, float a, float b) {
     case EW_SIGMOID: return zo_unary(ZO_U_SIGMOID, x);
     case EW_RSQRT: return zo_unary(ZO_U_RSQRT, x);
     case EW_CAST_INT: return truncf(x);
+    case EW_GELU_GRAD: return zo_gelu_grad(x);
     default: return x;
     }
 }
@@ -829,4 +839,44 @@ ZO_API void zo_attention_bwd(int dtype, const void *qkv, const void *dy, void *d
         free(P);
         free(dS);
     }
+}
+
+/* ---- gradients of LayerNorm / RMSNorm (zyx-nn/src/layer_norm.rs:98-135, rms_norm.rs:26-32) -----------------
+ * The reverse rules of zyx/src/graph/autograd.rs:87-134, 299-379 applied to the forward expressions; f64
+ * arithmetic, one store in `dtype`. LayerNorm's variance divides by n-1. w, add, dw, db may be null. */
+ZO_API void zo_norm_bwd(int dtype, int rms, const void *x, const void *w, const void *dy, const void *add, void *dx,
+                        void *dw, void *db, int64_t rows, int64_t cols, float eps) {
+    double *aw = (double *)calloc((size_t)cols + 1, sizeof(double)), *ab = (double *)calloc((size_t)cols + 1, sizeof(double));
+    for (int64_t r = 0; r < rows; r++) {
+        double mean = 0.0, ss = 0.0;
+        for (int64_t c = 0; c < cols; c++) mean += (double)load_as_f32(x, dtype, r * cols + c);
+        mean = rms ? 0.0 : mean / (double)cols;
+        for (int64_t c = 0; c < cols; c++) {
+            double d = (double)load_as_f32(x, dtype, r * cols + c) - mean;
+            ss += d * d;
+        }
+        const double rstd = rms ? sqrt(1.0 / (ss / (double)cols + (double)eps)) : 1.0 / sqrt(ss / (double)(cols - 1) + (double)eps);
+        double s1 = 0.0, s2 = 0.0;
+        for (int64_t c = 0; c < cols; c++) {
+            const double g = (double)load_as_f32(dy, dtype, r * cols + c) * (w ? (double)load_as_f32(w, dtype, c) : 1.0);
+            const double xh = ((double)load_as_f32(x, dtype, r * cols + c) - mean) * rstd;
+            s1 += g;
+            s2 += g * xh;
+            aw[c] += (double)load_as_f32(dy, dtype, r * cols + c) * xh;
+            ab[c] += (double)load_as_f32(dy, dtype, r * cols + c);
+        }
+        for (int64_t c = 0; c < cols; c++) {
+            const double g = (double)load_as_f32(dy, dtype, r * cols + c) * (w ? (double)load_as_f32(w, dtype, c) : 1.0);
+            const double xh = ((double)load_as_f32(x, dtype, r * cols + c) - mean) * rstd;
+            double o = rms ? rstd * (g - xh * s2 / (double)cols) : rstd * (g - s1 / (double)cols - xh * s2 / (double)(cols - 1));
+            if (add) o += (double)load_as_f32(add, dtype, r * cols + c);
+            store_from_f32(dx, dtype, r * cols + c, (float)o);
+        }
+    }
+    for (int64_t c = 0; c < cols; c++) {
+        if (dw) store_from_f32(dw, dtype, c, (float)aw[c]);
+        if (db) store_from_f32(db, dtype, c, (float)ab[c]);
+    }
+    free(aw);
+    free(ab);
 }

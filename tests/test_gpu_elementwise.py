@@ -187,3 +187,24 @@ def test_large_tensor_grid_stride(hip, oracle):
     c = Chain(4096, 8192)
     c.load(c.input()).mul(c.const(2.0)).add(c.const(1.0))
     assert np.array_equal(run_chain(dev, pool, c, [x]), x * np.float32(2) + np.float32(1))
+
+
+def test_gelu_grad_chain(hip, oracle):
+    """dh = dg * gelu'(h), the chain the MLP backward of a transformer block launches (bf16 storage)."""
+    from zyx_amd import DType
+    from zyx_amd.kernels import Chain, run_chain
+    dev, pool = hip
+    r = oracle.Rng(3)
+    h = r.randn((64, 512), 3.0)
+    dg = r.randn((64, 512))
+    c = Chain(64, 512)
+    hi, gi = c.input(DType.F32), c.input(DType.F32)
+    c.load(hi).gelu_grad().mul(gi)
+    got, want = run_chain(dev, pool, c, [h, dg]), oracle.ew_chain(c, [h, dg])
+    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-6 * np.abs(dg))
+    cb = Chain(64, 512, out_dtype=DType.BF16)
+    hi, gi = cb.input(DType.BF16), cb.input(DType.BF16)
+    cb.load(hi).gelu_grad().mul(gi)
+    hb, gb = oracle.f32_to_bf16(h), oracle.f32_to_bf16(dg)
+    got, want = run_chain(dev, pool, cb, [hb, gb]), oracle.ew_chain(cb, [hb, gb])
+    assert np.all(np.abs(oracle.bf16_to_f32(got) - oracle.bf16_to_f32(want)) <= 2.0 ** -7 * np.abs(oracle.bf16_to_f32(want)) + 1e-6)

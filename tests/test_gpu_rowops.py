@@ -74,3 +74,40 @@ def test_cross_entropy(hip, oracle):
     loss, grad = cross_entropy(dev, pool, x, np.array([-1, 5], np.int32), 1.0)
     assert loss.tolist() == [0.0, 0.0]
     np.testing.assert_allclose(grad.sum(1), [1.0, 1.0], rtol=1e-6)
+
+
+# ---- gradients of the norms ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(5, 9), (64, 128), (130, 1024), (3, 1000), (2100, 64)])
+@pytest.mark.parametrize("rms", [False, True])
+def test_norm_backward_f32(hip, oracle, shape, rms):
+    from zyx_amd.kernels import norm_rows_bwd
+    dev, pool = hip
+    rows, cols = shape
+    r = oracle.Rng(rows + cols)
+    x, dy, add, w = r.randn(shape), r.randn(shape), r.randn(shape), r.randn((cols,))
+    eps = 1e-6 if rms else 1e-5
+    for use_w, use_add in ((True, True), (False, False)):
+        got = norm_rows_bwd(dev, pool, x, dy, w if use_w else None, add if use_add else None, rms=rms, eps=eps)
+        want = oracle.norm_bwd(x, dy, w if use_w else None, add if use_add else None, rms=rms, eps=eps)
+        # dx: sums of `cols` terms of size |g|; dw/db: sums of `rows` terms
+        assert np.allclose(got[0], want[0], rtol=1e-5, atol=1e-5 * np.sqrt(cols))
+        for g, wv in zip(got[1:], want[1:]):
+            assert (g is None) == (wv is None)
+            if g is not None:
+                assert np.allclose(g, wv, rtol=1e-5, atol=2e-6 * rows)
+
+
+def test_norm_backward_bf16_config5_rows(hip, oracle):
+    """Rows of 1024 bf16 as in config 5 (8192 rows): f32 arithmetic, one truncating bf16 store."""
+    from zyx_amd.kernels import norm_rows_bwd
+    from zyx_amd import DType
+    dev, pool = hip
+    r = oracle.Rng(9)
+    shape = (8192, 1024)
+    x, dy, add = [oracle.f32_to_bf16(r.randn(shape)) for _ in range(3)]
+    w = oracle.f32_to_bf16(1.0 + 0.1 * r.randn((1024,)))
+    got = norm_rows_bwd(dev, pool, x, dy, w, add, dtype=DType.BF16)
+    want = oracle.norm_bwd(x, dy, w, add, dtype=oracle.BF16)
+    for g, wv, scale in zip(got, want, (1.0, 90.0, 90.0)):   # column sums of 8192 N(0,1) terms are ~90 in size
+        gf, wf = oracle.bf16_to_f32(g).astype(np.float64), oracle.bf16_to_f32(wv).astype(np.float64)
+        assert np.all(np.abs(gf - wf) <= 2.0 ** -7 * np.abs(wf) + 1e-4 * scale)

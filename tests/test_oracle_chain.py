@@ -63,3 +63,22 @@ def test_chain_int_registers_and_stores(oracle):
     c = Chain(1, 4, DType.F32, DType.I32)
     c.load(c.input())
     assert oracle.ew_chain(c, [x]).tolist() == [[1, -2, 3, 0]]
+
+
+def test_gelu_grad_matches_finite_differences(oracle):
+    """gelu_grad is the derivative of the oracle's own gelu: central differences in f64 of the reference's
+    expression (zyx/src/tensor/elementwise.rs:168-170) pin the formula; a wrong cubic coefficient (0.134145 =
+    3 * 0.044715) or a missing (1 - t^2) factor fails it."""
+    from zyx_amd.kernels import Chain
+    x = np.linspace(-6, 6, 1001).astype(np.float32).reshape(1, -1)
+    c = Chain(1, x.size)
+    c.load(c.input()).gelu_grad()
+    got = oracle.ew_chain(c, [x])
+    f = lambda v: 0.5 * v * (1 + np.tanh(np.sqrt(2 / np.pi) * (v + 0.044715 * v ** 3)))
+    x64 = x.astype(np.float64)
+    num = (f(x64 + 1e-6) - f(x64 - 1e-6)) / 2e-6
+    assert np.allclose(got, num, rtol=1e-5, atol=2e-6)
+    big = np.array([[50.0, -50.0, 1e4, -1e4]], np.float32)  # saturated tanh: slope 1 and 0
+    c2 = Chain(1, 4)
+    c2.load(c2.input()).gelu_grad()
+    assert oracle.ew_chain(c2, [big]).tolist() == [[1.0, 0.0, 1.0, 0.0]]

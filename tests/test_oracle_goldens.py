@@ -446,3 +446,42 @@ def test_attention_against_textbook_and_finite_differences(oracle):
         lo[i] -= 1e-5
         num[i] = ((f64(hi)[0] - f64(lo)[0]) * dy).sum() / 2e-5
     assert np.allclose(got, num, rtol=1e-4, atol=1e-6)
+
+
+def test_norm_backward_against_finite_differences(oracle):
+    """No reference test holds norm gradients. The forward is pinned by the goldens above; its f64 restatement
+    differentiated by central differences pins the backward (the n-1 of the unbiased variance, the mean(g) term
+    and the r^3 of RMSNorm each change the result by far more than the tolerance)."""
+    rng = np.random.default_rng(1)
+    rows, cols = 5, 9
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    w = rng.standard_normal(cols).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np.float32)
+    add = rng.standard_normal((rows, cols)).astype(np.float32)
+
+    def ln(xx, ww, bb):
+        m = xx.mean(1, keepdims=True)
+        v = ((xx - m) ** 2).sum(1, keepdims=True) / (cols - 1)
+        return (xx - m) / np.sqrt(v + 1e-5) * ww + bb
+
+    def rms(xx, ww, bb):
+        return xx * np.sqrt(1.0 / ((xx ** 2).mean(1, keepdims=True) + 1e-6)) * ww
+
+    for fwd, is_rms, eps in ((ln, False, 1e-5), (rms, True, 1e-6)):
+        assert np.allclose(fwd(x.astype(np.float64), w, b),
+                           oracle.rms_norm(x, w, eps) if is_rms else oracle.layer_norm(x, w, b, eps), rtol=1e-5, atol=1e-6)
+        dx, dw, db = oracle.norm_bwd(x, dy, w, add, rms=is_rms, eps=eps)
+
+        def num(arr, setter):
+            out = np.empty(arr.shape, np.float64)
+            for i in np.ndindex(*arr.shape):
+                hi, lo = arr.astype(np.float64), arr.astype(np.float64)
+                hi[i] += 1e-6
+                lo[i] -= 1e-6
+                out[i] = ((setter(hi) - setter(lo)) * dy).sum() / 2e-6
+            return out
+        assert np.allclose(dx, num(x, lambda a: fwd(a, w, b)) + add, rtol=1e-4, atol=1e-5)
+        assert np.allclose(dw, num(w, lambda a: fwd(x.astype(np.float64), a, b)), rtol=1e-4, atol=1e-5)
+        if not is_rms:
+            assert np.allclose(db, dy.sum(0), rtol=1e-5, atol=1e-6)

@@ -119,6 +119,12 @@ __device__ __forceinline__ float ref_gelu(float x) {
     return (x * 0.5f) * (ref_tanh(inner) + 1.0f);
 }
 
+__device__ __forceinline__ float ref_gelu_grad(float x) {
+    const float k = 0.79788456080286535588f, x2 = x * x;
+    const float t = ref_tanh((x + x2 * x * 0.044715f) * k);
+    return 0.5f * (1.0f + t) + (0.5f * x) * ((1.0f - t * t) * (k * (1.0f + 0.134145f * x2)));
+}
+
 __device__ __forceinline__ float op_f(int op, float x, float a, float b) {
     switch (op) {
     case 0: return a;                                  // LOAD
@@ -158,6 +164,7 @@ __device__ __forceinline__ float op_f(int op, float x, float a, float b) {
     case 41: { float e = expf(x); return e / (e + 1.0f); }
     case 42: return sqrtf(1.0f / x);                   // rsqrt = reciprocal().sqrt()
     case 43: return truncf(x);                         // CAST_INT inside a float chain
+    case 44: return ref_gelu_grad(x);
     default: return x;
     }
 }

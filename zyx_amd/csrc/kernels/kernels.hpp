@@ -87,6 +87,20 @@ struct NormRows {
 };
 hipError_t norm_rows(const NormRows &p, hipStream_t stream);
 
+// Gradients of the above: dx[rows, cols] (+ add, an optional tensor summed into dx: the other branch of a
+// residual connection), dw[cols] = sum_rows dy * xhat, db[cols] = sum_rows dy (each optional).
+struct NormRowsBwd {
+    int64_t rows, cols;
+    int dtype, rms;
+    float eps;
+    const void *x, *w, *dy, *add; // w, add may be null
+    void *dx, *dw, *db;           // dw, db may be null
+    void *workspace;              // norm_rows_bwd_workspace_bytes(rows, cols)
+    uint64_t workspace_bytes;
+};
+uint64_t norm_rows_bwd_workspace_bytes(int64_t rows, int64_t cols);
+hipError_t norm_rows_bwd(const NormRowsBwd &p, hipStream_t stream);
+
 // conv2d forward, NCHW input, weight [Cout, C, KH, KW], groups = 1. koff[k] / kdyx[k] (k = (c,ky,kx)):
 // input offset c*H*W + ky*dy*W + kx*dx and the tap displacement (ky*dy) << 16 | (kx*dx), device arrays.
 struct Conv2d {

@@ -8,6 +8,10 @@
 //              var = sum((x - mean)^2) / (n - 1)  (Tensor::var uses correction 1,
 //              zyx/src/tensor/reduce_ops.rs:795-805, 111-123)
 //   RMSNorm    zyx-nn/src/rms_norm.rs:26-32: x * sqrt(1 / (mean(x^2) + eps)) * scale
+//   their gradients: the reverse rules of zyx/src/graph/autograd.rs:87-134 (Sub, Mul, Div, the reduce
+//              rules :299-379) applied to the expressions above collapse, per row, to
+//              LayerNorm dx = rstd * (g - mean(g) - xh * sum(g*xh) / (n-1)), g = dy*w, xh = (x-mean)*rstd
+//              RMSNorm   dx = r * g - r^3 * x * sum(g*x) / n;  dw = sum_rows dy*xh, db = sum_rows dy
 //   cross_entropy zyx/src/tensor/mod.rs:1639-1655 with ln_softmax :1427-1431 and the class
 //              index target turned into a one-hot by equal(arange) :1920-1946.
 #include "dtypes.hpp"
@@ -136,6 +140,127 @@ __global__ __launch_bounds__(256) void cross_entropy_k(const float *__restrict__
     }
 }
 
+// dx of one row per wave; also leaves the row's mean and 1/sigma in stats[row*2 ..] for the parameter gradients.
+template <int DT, int MODE, bool VEC>
+__global__ __launch_bounds__(256) void norm_bwd_dx_k(const typename RowIO<DT>::S *__restrict__ x,
+                                                     const typename RowIO<DT>::S *__restrict__ w,
+                                                     const typename RowIO<DT>::S *__restrict__ dy,
+                                                     const typename RowIO<DT>::S *__restrict__ add,
+                                                     typename RowIO<DT>::S *__restrict__ dx, float *__restrict__ stats,
+                                                     int64_t rows, int cols, float eps) {
+    typedef RowIO<DT> IO;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const typename IO::S *xr = x + row * cols, *gr = dy + row * cols, *ar = add ? add + row * cols : nullptr;
+    typename IO::S *dr = dx + row * cols;
+    float mean = 0.0f, rstd;
+    if (MODE == 0) {
+        mean = row_sum<DT, VEC>(xr, cols, lane, [](float v) { return v; }) / (float)cols;
+        const float m = mean;
+        float var = row_sum<DT, VEC>(xr, cols, lane, [m](float v) { return (v - m) * (v - m); }) / (float)(cols - 1);
+        rstd = 1.0f / sqrtf(var + eps);
+    } else {
+        rstd = sqrtf(1.0f / (row_sum<DT, VEC>(xr, cols, lane, [](float v) { return v * v; }) / (float)cols + eps));
+    }
+    float s1 = 0.0f, s2 = 0.0f; // sum g, sum g * (xh | x)
+    auto accum = [&](float xv, float gv, int c) {
+        const float g = w ? gv * IO::ld(w, c) : gv;
+        s1 += g;
+        s2 += g * (MODE == 0 ? (xv - mean) * rstd : xv);
+    };
+    if (VEC) {
+        for (int c = lane * 4; c < cols; c += 256) {
+            float xv[4], gv[4];
+            IO::ld4(xr, c, xv);
+            IO::ld4(gr, c, gv);
+#pragma unroll
+            for (int k = 0; k < 4; k++) accum(xv[k], gv[k], c + k);
+        }
+    } else {
+        for (int c = lane; c < cols; c += 64) accum(IO::ld(xr, c), IO::ld(gr, c), c);
+    }
+    s1 = wave_allreduce_f32(s1, OpAdd());
+    s2 = wave_allreduce_f32(s2, OpAdd());
+    const float k1 = s1 / (float)cols, k2 = MODE == 0 ? s2 / (float)(cols - 1) : rstd * rstd * rstd * s2 / (float)cols;
+    auto apply = [&](float xv, float gv, float av, int c) {
+        const float g = w ? gv * IO::ld(w, c) : gv;
+        const float o = MODE == 0 ? rstd * ((g - k1) - ((xv - mean) * rstd) * k2) : rstd * g - xv * k2;
+        return o + av;
+    };
+    if (VEC) {
+        for (int c = lane * 4; c < cols; c += 256) {
+            float xv[4], gv[4], av[4] = {0.0f, 0.0f, 0.0f, 0.0f}, o[4];
+            IO::ld4(xr, c, xv);
+            IO::ld4(gr, c, gv);
+            if (ar) IO::ld4(ar, c, av);
+#pragma unroll
+            for (int k = 0; k < 4; k++) o[k] = apply(xv[k], gv[k], av[k], c + k);
+            IO::st4(dr, c, o);
+        }
+    } else {
+        for (int c = lane; c < cols; c += 64) IO::st(dr, c, apply(IO::ld(xr, c), IO::ld(gr, c), ar ? IO::ld(ar, c) : 0.0f, c));
+    }
+    if (lane == 0) {
+        stats[row * 2] = mean;
+        stats[row * 2 + 1] = rstd;
+    }
+}
+
+// Partial parameter gradients: thread = column, workgroup = 256 columns x one chunk of rows.
+// part[(chunk*2 + 0)*cols + c] = sum dy*xh, part[(chunk*2 + 1)*cols + c] = sum dy over the chunk.
+template <int DT>
+__global__ __launch_bounds__(256) void norm_bwd_param_k(const typename RowIO<DT>::S *__restrict__ x,
+                                                        const typename RowIO<DT>::S *__restrict__ dy,
+                                                        const float *__restrict__ stats, float *__restrict__ part,
+                                                        int64_t rows, int cols, int64_t rows_per_chunk) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_chunk, r1 = r0 + rows_per_chunk < rows ? r0 + rows_per_chunk : rows;
+    float pw = 0.0f, pb = 0.0f;
+    for (int64_t r = r0; r < r1; r++) {
+        const float g = RowIO<DT>::ld(dy, r * cols + c);
+        pw = __builtin_fmaf(g, (RowIO<DT>::ld(x, r * cols + c) - stats[r * 2]) * stats[r * 2 + 1], pw);
+        pb += g;
+    }
+    part[((int64_t)blockIdx.y * 2) * cols + c] = pw;
+    part[((int64_t)blockIdx.y * 2 + 1) * cols + c] = pb;
+}
+template <int DT>
+__global__ __launch_bounds__(256) void norm_bwd_param_sum_k(const float *__restrict__ part, typename RowIO<DT>::S *__restrict__ dw,
+                                                            typename RowIO<DT>::S *__restrict__ db, int cols, int chunks) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= cols) return;
+    float sw = 0.0f, sb = 0.0f;
+    for (int k = 0; k < chunks; k++) {
+        sw += part[((int64_t)k * 2) * cols + c];
+        sb += part[((int64_t)k * 2 + 1) * cols + c];
+    }
+    if (dw) RowIO<DT>::st(dw, c, sw);
+    if (db) RowIO<DT>::st(db, c, sb);
+}
+
+int norm_bwd_chunks(int64_t rows) { return (int)(rows < 64 * 32 ? (rows + 31) / 32 : 64); }
+
+template <int DT, int MODE> hipError_t launch_norm_bwd(const NormRowsBwd &p, hipStream_t st) {
+    typedef typename RowIO<DT>::S S;
+    const int esz = (int)sizeof(S);
+    auto al = [&](const void *q) { return reinterpret_cast<uintptr_t>(q) % (4 * esz) == 0; };
+    const bool vec = p.cols % 4 == 0 && al(p.x) && al(p.dy) && al(p.dx) && al(p.add);
+    float *stats = (float *)p.workspace, *part = stats + p.rows * 2;
+    dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
+    if (vec) hipLaunchKernelGGL((norm_bwd_dx_k<DT, MODE, true>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, (int)p.cols, p.eps);
+    else hipLaunchKernelGGL((norm_bwd_dx_k<DT, MODE, false>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, (int)p.cols, p.eps);
+    if (p.dw || p.db) {
+        const int chunks = norm_bwd_chunks(p.rows);
+        const int64_t rpc = (p.rows + chunks - 1) / chunks;
+        const unsigned cb = (unsigned)((p.cols + 255) / 256);
+        hipLaunchKernelGGL((norm_bwd_param_k<DT>), dim3(cb, (unsigned)chunks), block, 0, st, (const S *)p.x, (const S *)p.dy, stats, part, p.rows, (int)p.cols, rpc);
+        hipLaunchKernelGGL((norm_bwd_param_sum_k<DT>), dim3(cb), block, 0, st, part, (S *)p.dw, (S *)p.db, (int)p.cols, chunks);
+    }
+    return hipGetLastError();
+}
+
 template <int DT, int MODE> hipError_t launch_norm(const NormRows &p, hipStream_t st) {
     typedef typename RowIO<DT>::S S;
     dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
@@ -153,6 +278,20 @@ hipError_t norm_rows(const NormRows &p, hipStream_t st) {
     if (p.cols >= (1ll << 31) || (p.rows + 3) / 4 >= (1ll << 31)) return hipErrorInvalidValue;
     if (p.dtype == DT_F32) return p.rms ? launch_norm<0, 1>(p, st) : launch_norm<0, 0>(p, st);
     if (p.dtype == DT_BF16) return p.rms ? launch_norm<1, 1>(p, st) : launch_norm<1, 0>(p, st);
+    return hipErrorInvalidValue;
+}
+
+uint64_t norm_rows_bwd_workspace_bytes(int64_t rows, int64_t cols) {
+    return (uint64_t)rows * 8 + (uint64_t)norm_bwd_chunks(rows) * 2 * (uint64_t)cols * 4;
+}
+
+hipError_t norm_rows_bwd(const NormRowsBwd &p, hipStream_t st) {
+    if (p.rows <= 0 || p.cols <= 0) return hipSuccess;
+    if (p.cols >= (1ll << 31) || (p.rows + 3) / 4 >= (1ll << 31) || !p.workspace ||
+        p.workspace_bytes < norm_rows_bwd_workspace_bytes(p.rows, p.cols))
+        return hipErrorInvalidValue;
+    if (p.dtype == DT_F32) return p.rms ? launch_norm_bwd<0, 1>(p, st) : launch_norm_bwd<0, 0>(p, st);
+    if (p.dtype == DT_BF16) return p.rms ? launch_norm_bwd<1, 1>(p, st) : launch_norm_bwd<1, 0>(p, st);
     return hipErrorInvalidValue;
 }
 

@@ -317,7 +317,8 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
             if ((op == ZHIP_EW_WHERE || op == ZHIP_EW_MAD) && !src_ok(sb))
                 return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: instruction %d: bad second operand %d", j, sb);
             bool float_only = (op >= ZHIP_EW_EXP && op <= ZHIP_EW_TRUNC) || op == ZHIP_EW_POW || op == ZHIP_EW_TANH ||
-                              op == ZHIP_EW_GELU || op == ZHIP_EW_SIGMOID || op == ZHIP_EW_RSQRT || op == ZHIP_EW_CAST_INT;
+                              op == ZHIP_EW_GELU || op == ZHIP_EW_SIGMOID || op == ZHIP_EW_RSQRT || op == ZHIP_EW_CAST_INT ||
+                              op == ZHIP_EW_GELU_GRAD;
             bool int_only = op == ZHIP_EW_BITNOT || (op >= ZHIP_EW_BITXOR && op <= ZHIP_EW_SHR);
             if ((ireg && float_only) || (!ireg && int_only))
                 return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise: instruction %d: op %d not defined for this register class", j, op);
@@ -377,6 +378,27 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.n_in = a;
         p.need[a] = (uint64_t)rows * cols * e;
         p.n_out = 1;
+        return ZHIP_OK;
+    }
+    case ZHIP_K_NORM_ROWS_BWD: {
+        int64_t rows = d.dims[0], cols = d.dims[1];
+        if (rows < 0 || cols < 0 || cols >= (1ll << 31) || (cols && rows > (1ll << 40) / cols))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "norm_rows_bwd: rows/cols out of range");
+        if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16) return c->fail(ZHIP_KERNEL_COMPILATION, "norm_rows_bwd: dtype must be F32 or BF16");
+        if ((d.flags & ~15) || ((d.flags & ZHIP_NORM_RMS) && (d.flags & ZHIP_NORM_BIAS)))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "norm_rows_bwd: bad flags");
+        const uint64_t e = dtype_bytes(d.dtype), full = (uint64_t)rows * cols * e;
+        int a = 0;
+        p.need[a++] = full;
+        if (d.flags & ZHIP_NORM_WEIGHT) p.need[a++] = (uint64_t)cols * e;
+        p.need[a++] = full;
+        if (d.flags & ZHIP_NORM_ADD) p.need[a++] = full;
+        p.n_in = a;
+        p.need[a++] = full;
+        if (d.flags & ZHIP_NORM_WEIGHT) p.need[a++] = (uint64_t)cols * e;
+        if (d.flags & ZHIP_NORM_BIAS) p.need[a++] = (uint64_t)cols * e;
+        p.n_out = a - p.n_in;
+        p.workspace_bytes = zk::norm_rows_bwd_workspace_bytes(rows, cols);
         return ZHIP_OK;
     }
     case ZHIP_K_CROSS_ENTROPY: {
@@ -622,6 +644,25 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         if (d.flags & ZHIP_NORM_BIAS) a.b = ptr[i++];
         a.y = ptr[i];
         return zk::norm_rows(a, st);
+    }
+    case ZHIP_K_NORM_ROWS_BWD: {
+        zk::NormRowsBwd a{};
+        a.rows = d.dims[0];
+        a.cols = d.dims[1];
+        a.dtype = d.dtype;
+        a.rms = d.flags & ZHIP_NORM_RMS ? 1 : 0;
+        a.eps = d.fparams[0];
+        int i = 0;
+        a.x = ptr[i++];
+        if (d.flags & ZHIP_NORM_WEIGHT) a.w = ptr[i++];
+        a.dy = ptr[i++];
+        if (d.flags & ZHIP_NORM_ADD) a.add = ptr[i++];
+        a.dx = ptr[i++];
+        if (d.flags & ZHIP_NORM_WEIGHT) a.dw = ptr[i++];
+        if (d.flags & ZHIP_NORM_BIAS) a.db = ptr[i++];
+        a.workspace = p.workspace;
+        a.workspace_bytes = p.workspace_bytes;
+        return zk::norm_rows_bwd(a, st);
     }
     case ZHIP_K_CROSS_ENTROPY: {
         zk::CrossEntropy a{};

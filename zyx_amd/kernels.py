@@ -73,7 +73,7 @@ K_REDUCE = 3
 EW_OPS = ["load", "save", "neg", "bitnot", "exp", "exp2", "ln", "log2", "reciprocal", "sqrt", "sin", "cos", "floor",
           "trunc", "abs", "add", "sub", "mul", "div", "pow", "mod", "cmplt", "cmpgt", "cmpge", "max", "or", "and",
           "bitxor", "bitor", "bitand", "shl", "shr", "noteq", "eq", "rsub", "rdiv", "where", "mad", "relu", "tanh",
-          "gelu", "sigmoid", "rsqrt", "cast_int"]
+          "gelu", "sigmoid", "rsqrt", "cast_int", "gelu_grad"]
 EW_OP = {name: i for i, name in enumerate(EW_OPS)}
 EW_FULL, EW_ROW, EW_COL, EW_SCALAR = 0, 1, 2, 3
 EW_T = 0x10
@@ -531,3 +531,51 @@ def attention_bwd(dev: HIPDevice, pool: HIPMemoryPool, qkv, y, dy, lse, n_head: 
         pool.deallocate(buf, [])
     dev.release(prog)
     return out
+
+
+# ---- gradients of LayerNorm / RMSNorm (ZHIP_K_NORM_ROWS_BWD) -------------------------------------------------
+K_NORM_ROWS_BWD = 12
+NORM_ADD = 8
+
+
+def norm_rows_bwd_desc(rows: int, cols: int, rms=False, weight=True, bias=True, add=False, eps=1e-5,
+                       dtype: DType = DType.F32) -> KernelDesc:
+    d = KernelDesc()
+    d.kind, d.dtype, d.out_dtype = K_NORM_ROWS_BWD, DType(dtype), DType(dtype)
+    d.flags = (NORM_RMS if rms else 0) | (NORM_WEIGHT if weight else 0) | (NORM_BIAS if bias and not rms else 0) | \
+        (NORM_ADD if add else 0)
+    d.dims[0], d.dims[1] = rows, cols
+    d.fparams[0] = eps
+    return d
+
+
+def norm_rows_bwd(dev: HIPDevice, pool: HIPMemoryPool, x, dy, w=None, add=None, rms=False, want_db=True, eps=1e-5,
+                  dtype: DType = DType.F32):
+    """Gradients of LayerNorm / RMSNorm: returns (dx (+ add), dw or None, db or None)."""
+    st = _NP_STORE[DType(dtype)]
+    x = np.ascontiguousarray(x, st)
+    rows, cols = x.shape
+    want_db = want_db and not rms
+    prog = dev.register_kernel(norm_rows_bwd_desc(rows, cols, rms, w is not None, want_db, add is not None, eps, dtype))
+    ins = [x] + ([np.ascontiguousarray(w, st)] if w is not None else []) + [np.ascontiguousarray(dy, st)] + \
+        ([np.ascontiguousarray(add, st)] if add is not None else [])
+    bufs, waits = [], []
+    for arr in ins:
+        bb, e = to_device(pool, arr)
+        bufs.append(bb)
+        waits.append(e)
+    outs = [(rows, cols)] + ([(cols,)] if w is not None else []) + ([(cols,)] if want_db else [])
+    obufs = []
+    for shp in outs:
+        ob, e = alloc_like(pool, int(np.prod(shp)), x.itemsize)
+        obufs.append(ob)
+        waits.append(e)
+    done = dev.launch(prog, pool, bufs + obufs, waits)
+    res = [to_host(pool, ob, shp, st, [done] if i == 0 else []) for i, (ob, shp) in enumerate(zip(obufs, outs))]
+    for bb in bufs + obufs:
+        pool.deallocate(bb, [])
+    dev.release(prog)
+    dx = res[0]
+    dw = res[1] if w is not None else None
+    db = res[-1] if want_db else None
+    return dx, dw, db
