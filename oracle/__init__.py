@@ -448,3 +448,95 @@ def norm_bwd(x, dy, w=None, add=None, rms: bool = False, eps: float = 1e-5, dtyp
     lib().zo_norm_bwd(dtype, int(rms), _p(x), _p(w), _p(dy), _p(add), _p(dx), _p(dw), _p(db), _I64(rows), _I64(cols),
                       C.c_float(eps))
     return dx, dw, db
+
+
+# ---- pre-norm transformer block: zyx-examples/examples/nanogpt.rs:41-98 over zyx-nn modules --------------------
+def _gelu64(v):
+    return 0.5 * v * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (v + 0.044715 * v ** 3)))
+
+
+def block_forward_f64(p: dict, x: np.ndarray, n_head: int, eps: float = 1e-5) -> dict:
+    """x[B,T,d] -> every module output of `x + attn(ln_1(x)); x + mlp(ln_2(x))` in f64 (numpy). LayerNorm uses the
+    unbiased variance (zyx-nn/src/layer_norm.rs:98-135), attention applies no mask
+    (zyx-nn/src/causal_self_attention.rs:36-74), gelu is the tanh form (zyx/src/tensor/elementwise.rs:168-170)."""
+    B, T, d = x.shape
+    dh = d // n_head
+    f = {k: np.asarray(v, np.float64) for k, v in p.items()}
+
+    def ln(v, w, b):
+        mu = v.mean(-1, keepdims=True)
+        var = ((v - mu) ** 2).sum(-1, keepdims=True) / (d - 1)
+        return (v - mu) / np.sqrt(var + eps) * w + b
+
+    s = {"x": np.asarray(x, np.float64)}
+    s["n1"] = ln(s["x"], f["ln1_w"], f["ln1_b"])
+    s["qkv"] = s["n1"] @ f["attn_w"].T + f["attn_b"]
+    q, k, v = [a.reshape(B, T, n_head, dh).transpose(0, 2, 1, 3) for a in np.split(s["qkv"], 3, axis=2)]
+    sc = np.einsum("bhtd,bhjd->bhtj", q, k) * float(np.float32(1.0 / np.sqrt(float(dh))))
+    e = np.exp(sc - sc.max(-1, keepdims=True))
+    s["probs"] = e / e.sum(-1, keepdims=True)
+    s["att"] = np.einsum("bhtj,bhjd->bhtd", s["probs"], v).transpose(0, 2, 1, 3).reshape(B, T, d)
+    s["x2"] = s["x"] + s["att"] @ f["proj_w"].T + f["proj_b"]
+    s["n2"] = ln(s["x2"], f["ln2_w"], f["ln2_b"])
+    s["h"] = s["n2"] @ f["fc_w"].T + f["fc_b"]
+    s["g"] = _gelu64(s["h"])
+    s["out"] = s["x2"] + s["g"] @ f["proj2_w"].T + f["proj2_b"]
+    return s
+
+
+def block_backward_f64(p: dict, s: dict, dout: np.ndarray, n_head: int, eps: float = 1e-5) -> dict:
+    """Gradients of sum(out * dout) with respect to x and every parameter, given block_forward_f64's outputs `s`:
+    Runtime::gradient's reverse rules (zyx/src/graph/autograd.rs:14-424) composed per module."""
+    B, T, d = s["x"].shape
+    dh = d // n_head
+    f = {k: np.asarray(v, np.float64) for k, v in p.items()}
+    g = {}
+    r2 = lambda a: a.reshape(B * T, -1)
+
+    def ln_bwd(v, w, dy):
+        mu = v.mean(-1, keepdims=True)
+        rstd = 1.0 / np.sqrt(((v - mu) ** 2).sum(-1, keepdims=True) / (d - 1) + eps)
+        xh = (v - mu) * rstd
+        gg = dy * w
+        dx = rstd * (gg - gg.mean(-1, keepdims=True) - xh * (gg * xh).sum(-1, keepdims=True) / (d - 1))
+        return dx, r2(dy * xh).sum(0), r2(dy).sum(0)
+
+    def lin_bwd(name, inp, dy):
+        g[name + "_w"] = r2(dy).T @ r2(inp)
+        g[name + "_b"] = r2(dy).sum(0)
+        return dy @ f[name + "_w"]
+
+    dout = np.asarray(dout, np.float64)
+    g["dg"] = lin_bwd("proj2", s["g"], dout)
+    hv = s["h"]
+    k0 = np.sqrt(2.0 / np.pi)
+    t = np.tanh(k0 * (hv + 0.044715 * hv ** 3))
+    g["dh"] = g["dg"] * (0.5 * (1 + t) + 0.5 * hv * (1 - t * t) * k0 * (1 + 3 * 0.044715 * hv * hv))
+    g["dn2"] = lin_bwd("fc", s["n2"], g["dh"])
+    dx, g["ln2_w"], g["ln2_b"] = ln_bwd(s["x2"], f["ln2_w"], g["dn2"])
+    g["dx2"] = dout + dx
+    g["datt"] = lin_bwd("proj", s["att"], g["dx2"])
+    q, k, v = [a.reshape(B, T, n_head, dh).transpose(0, 2, 1, 3) for a in np.split(s["qkv"], 3, axis=2)]
+    do = g["datt"].reshape(B, T, n_head, dh).transpose(0, 2, 1, 3)
+    ps = s["probs"]
+    dps = np.einsum("bhtd,bhjd->bhtj", do, v)
+    ds = ps * (dps - (ps * dps).sum(-1, keepdims=True))
+    sc = float(np.float32(1.0 / np.sqrt(float(dh))))
+    back = lambda a: a.transpose(0, 2, 1, 3).reshape(B, T, d)
+    g["dqkv"] = np.concatenate([back(np.einsum("bhtj,bhjd->bhtd", ds, k) * sc), back(np.einsum("bhtj,bhtd->bhjd", ds, q) * sc),
+                                back(np.einsum("bhtj,bhtd->bhjd", ps, do))], 2)
+    g["dn1"] = lin_bwd("attn", s["n1"], g["dqkv"])
+    dx, g["ln1_w"], g["ln1_b"] = ln_bwd(s["x"], f["ln1_w"], g["dn1"])
+    g["dx"] = g["dx2"] + dx
+    return g
+
+
+def block_init(d_model: int, n_head: int, seed: int = 42069, std: float = 0.02, mlp_ratio: int = 4) -> dict:
+    """Parameters of config 5: Linear weights std * randn, Linear biases zero (nanogpt.rs:121-125), LayerNorm
+    weight 1 / bias 0 (zyx-nn/src/layer_norm.rs:52-62), drawn in PARAMS order from one seeded generator."""
+    r = Rng(seed)
+    d, f = d_model, mlp_ratio * d_model
+    z = lambda *s: np.zeros(s, np.float32)
+    return dict(ln1_w=np.ones(d, np.float32), ln1_b=z(d), attn_w=r.randn((3 * d, d), std), attn_b=z(3 * d),
+                proj_w=r.randn((d, d), std), proj_b=z(d), ln2_w=np.ones(d, np.float32), ln2_b=z(d),
+                fc_w=r.randn((f, d), std), fc_b=z(f), proj2_w=r.randn((d, f), std), proj2_b=z(d))

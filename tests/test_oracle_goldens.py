@@ -485,3 +485,33 @@ def test_norm_backward_against_finite_differences(oracle):
         assert np.allclose(dw, num(w, lambda a: fwd(x.astype(np.float64), a, b)), rtol=1e-4, atol=1e-5)
         if not is_rms:
             assert np.allclose(db, dy.sum(0), rtol=1e-5, atol=1e-6)
+
+
+def test_block_f64_forward_pieces_and_backward_finite_differences(oracle):
+    """The f64 block: its attention agrees with the golden-pinned `attention`, its LayerNorm with `layer_norm`,
+    its gelu with the chain op; the backward is pinned by central differences of the forward in every input."""
+    rng = np.random.default_rng(2)
+    B, T, d, H = 2, 4, 8, 2
+    p = {k: (rng.standard_normal(v.shape) * 0.3 + (1.0 if k.endswith("n1_w") or k.endswith("n2_w") else 0.0)).astype(np.float32)
+         for k, v in oracle.block_init(d, H).items()}
+    x = rng.standard_normal((B, T, d)).astype(np.float32)
+    s = oracle.block_forward_f64(p, x, H)
+    assert np.allclose(s["n1"].reshape(-1, d), oracle.layer_norm(x.reshape(-1, d), p["ln1_w"], p["ln1_b"]), rtol=1e-5, atol=1e-5)
+    assert np.allclose(s["att"], oracle.attention(s["qkv"].astype(np.float32), H), rtol=1e-4, atol=1e-5)
+    assert np.allclose(s["g"].reshape(-1, 4 * d), oracle.unary("gelu", s["h"].astype(np.float32).reshape(-1, 4 * d)), rtol=1e-4, atol=1e-5)
+    dout = rng.standard_normal((B, T, d))
+    g = oracle.block_backward_f64(p, s, dout, H)
+    loss = lambda pp, xx: (oracle.block_forward_f64(pp, xx, H)["out"] * dout).sum()
+    for name in list(p) + ["x"]:
+        base = (x if name == "x" else p[name]).astype(np.float64)
+        num = np.empty_like(base)
+        for i in np.ndindex(*base.shape):
+            hi, lo = base.copy(), base.copy()
+            hi[i] += 1e-6
+            lo[i] -= 1e-6
+            if name == "x":
+                num[i] = (loss(p, hi) - loss(p, lo)) / 2e-6
+            else:
+                num[i] = (loss({**p, name: hi}, x) - loss({**p, name: lo}, x)) / 2e-6
+        got = g["dx"] if name == "x" else g[name]
+        assert np.allclose(got, num, rtol=2e-5, atol=2e-6), name
