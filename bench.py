@@ -80,6 +80,85 @@ def extra_gemm(dev, pool, kernels, steps=100, warmup=200):
     return out
 
 
+def extra_conv(dev, pool, kernels, steps=50, warmup=50):
+    """Config 4: conv2d N=32 C=64 56x56, 3x3 -> 128 channels, stride 1 pad 1 (+ ReLU), then 2x2 max-pool."""
+    import zyx_amd
+    N, C, HW, CO = 32, 64, 56, 128
+    flop = 2.0 * N * CO * HW * HW * C * 9
+    rng = np.random.default_rng(4)
+    out = {}
+    for name, dt, isz in (("f32", zyx_amd.DType.F32, 4), ("bf16", zyx_amd.DType.BF16, 2)):
+        x = rng.standard_normal((N, C, HW, HW), dtype=np.float32)
+        w = (rng.standard_normal((CO, C, 3, 3), dtype=np.float32) * np.sqrt(2.0 / 576)).astype(np.float32)
+        if isz == 2:
+            x, w = [(a.view(np.uint32) >> 16).astype(np.uint16) for a in (x, w)]
+        xb, e1 = kernels.to_device(pool, x)
+        wb, e2 = kernels.to_device(pool, w)
+        yb, e3 = kernels.alloc_like(pool, N * CO * HW * HW, isz)
+        pb, e4 = kernels.alloc_like(pool, N * CO * (HW // 2) ** 2, isz)
+        pool.sync_events([e1, e2, e3, e4])
+        conv = dev.register_kernel(kernels.conv2d_desc(N, C, HW, HW, CO, 3, 3, padding=(1, 1), relu=True, dtype=dt))
+        mp = dev.register_kernel(kernels.max_pool2d_desc(N * CO, HW, HW, dtype=dt))
+        dev.profile_kernel(conv, [[xb, wb, yb]], warmup)
+        us = dev.profile_kernel(conv, [[xb, wb, yb]], steps)
+        us_p = dev.profile_kernel(mp, [[yb, pb]], steps)
+        pool_bytes = (N * CO * HW * HW + N * CO * (HW // 2) ** 2) * isz
+        peak = 157.3 if isz == 4 else 2500.0
+        out[name] = {"conv_relu_us": round(us, 2), "conv_TFLOP/s": round(flop / us / 1e6, 1),
+                     "conv_frac_of_peak": round(flop / us / 1e6 / peak, 4), "peak_TFLOP/s": peak,
+                     "max_pool_us": round(us_p, 2), "max_pool_GB/s": round(pool_bytes / us_p / 1e3, 1)}
+        dev.release(conv)
+        dev.release(mp)
+        for b_ in (xb, wb, yb, pb):
+            pool.deallocate(b_, [])
+    return out
+
+
+def extra_block(dev, pool, steps=20, warmup=5, cpu=True):
+    """Config 5: pre-norm transformer block B=8 T=1024 d=1024 16 heads, bf16, forward and forward + backward, each
+    one cached plan launch (8 and 24 kernels). FLOPs counted: the matrix products only (240.5 GFLOP forward)."""
+    import zyx_amd
+    import oracle
+    from zyx_amd.block import TransformerBlock
+    B, T, D, H = 8, 1024, 1024, 16
+    fwd_flop = 2.0 * B * T * (3 * D * D + D * D + 8 * D * D) + 4.0 * B * H * T * T * (D // H)
+    blk = TransformerBlock(dev, pool, B, T, D, H, zyx_amd.DType.BF16)
+    trunc = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    params = oracle.block_init(D, H)
+    blk.set_params({k: trunc(v) for k, v in params.items()})
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((B * T, D), dtype=np.float32)
+    blk.write("x", trunc(x))
+    blk.write("dout", trunc(np.ones((B * T, D), np.float32)))
+    res = {"kernels_forward": len(blk.forward_nodes), "kernels_forward_backward": len(blk.forward_nodes) + len(blk.backward_nodes)}
+    for name, fn, flop in (("forward", blk.forward, fwd_flop), ("forward_backward", blk.forward_backward, 3 * fwd_flop)):
+        for _ in range(warmup):
+            fn()
+        blk.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        blk.sync()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        res[name] = {"ms": round(ms, 3), "TFLOP/s": round(flop / ms / 1e9, 1), "frac_of_2.5PF_bf16_peak": round(flop / ms / 1e9 / 2500.0, 4)}
+    blk.close()
+    if cpu:
+        # one attention head pair and 64 rows of each Linear on the host cores, scaled to the whole forward
+        sub = trunc(rng.standard_normal((1, T, 3 * 128), dtype=np.float32))
+        t0 = time.perf_counter()
+        oracle.attention(sub, 2, dtype=oracle.BF16)
+        t_att = (time.perf_counter() - t0) * (B * H / 2)
+        rows = trunc(x[:64])
+        t0 = time.perf_counter()
+        for w in ("attn_w", "proj_w", "fc_w"):
+            oracle.linear(rows, trunc(params[w]), dtype=oracle.BF16)
+        oracle.linear(trunc(rng.standard_normal((64, 4 * D), dtype=np.float32)), trunc(params["proj2_w"]), dtype=oracle.BF16)
+        t_lin = (time.perf_counter() - t0) * (B * T / 64)
+        res["cpu_oracle_forward_s_extrapolated"] = round(t_att + t_lin, 2)
+        res["cpu_sample"] = "2 of 128 (batch, head) attention problems and 64 of 8192 rows of the four Linear layers"
+    return res
+
+
 def zyx_dtype_bf16():
     import zyx_amd
     return zyx_amd.DType.BF16
@@ -138,6 +217,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload (used for profiling)")
     ap.add_argument("--gemm-only", action="store_true",
                     help="run only the config-3 GEMM leg and print its numbers (used for profiling that kernel)")
+    ap.add_argument("--conv-only", action="store_true", help="run only the config-4 conv + max-pool leg")
+    ap.add_argument("--block-only", action="store_true", help="run only the config-5 transformer block leg")
     ap.add_argument("--counters", action="store_true",
                     help="short run for `rocprofv3 --pmc`: a few launches of the fused kernel and of a plain copy "
                          "kernel over the same 8192x4096 f32 tensor (known traffic: 134217728 B read + written), "
@@ -156,6 +237,13 @@ def main():
 
     if args.gemm_only:
         print(json.dumps({"config3_gemm_bf16_4096": extra_gemm(dev, pool, kernels, steps=args.steps, warmup=max(args.warmup, 100))}))
+        pool.deinitialize()
+        return
+
+    if args.conv_only or args.block_only:
+        res = {"config4_conv_relu_pool": extra_conv(dev, pool, kernels)} if args.conv_only else \
+            {"config5_transformer_block": extra_block(dev, pool, steps=args.steps if args.steps != 200 else 20, cpu=not args.no_cpu)}
+        print(json.dumps(res))
         pool.deinitialize()
         return
 
@@ -234,7 +322,9 @@ def main():
     if not args.no_extra:
         # other configs of the same backend, reported beside the headline (not part of `value`)
         out["extra"] = {"config3_gemm_bf16_4096": extra_gemm(dev, pool, kernels),
-                        "config1_mlp_train": extra_mlp(dev, pool, cpu=not args.no_cpu)}
+                        "config1_mlp_train": extra_mlp(dev, pool, cpu=not args.no_cpu),
+                        "config4_conv_relu_pool": extra_conv(dev, pool, kernels),
+                        "config5_transformer_block": extra_block(dev, pool, cpu=not args.no_cpu)}
     pool.deinitialize()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(x)
