@@ -163,7 +163,7 @@ def test_batched_and_scaled(hip, oracle):
     assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
 
 
-@pytest.mark.parametrize("mnk", [(256, 512, 128), (100, 70, 50)])
+@pytest.mark.parametrize("mnk", [(256, 512, 128), (100, 70, 50), (256, 256, 1024), (512, 256, 4096)])
 @pytest.mark.parametrize("epilogue", ["none", "gelu"])
 def test_bf16_output_and_residual(hip, oracle, mnk, epilogue):
     """bf16 C with the truncating store, and the fused residual add (x + Linear(x)): both kernels."""

@@ -122,7 +122,7 @@ template <bool AT, bool BT, int EPI>
 __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                       void *__restrict__ Cv, const void *__restrict__ bias,
                                                       const void *__restrict__ residual, int bias_dtype, int out_bf16,
-                                                      int M, int N, int K) {
+                                                      int M, int N, int K, int splits) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -131,9 +131,16 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
     // XCD-aware tile order: ids congruent mod 8 land on one XCD; give each XCD a patch
     // of 4 x 8 tiles (or the whole grid when it is smaller).
     const int tiles_m = M / BM, tiles_n = N / BN;
+    // split-K: workgroup z of a tile multiplies K range [z, z+1) * K/splits and stores its raw f32 partial
+    // tile into slice z of Cv (a [splits, M, N] workspace that a second kernel folds)
+    const int split = blockIdx.x / (tiles_m * tiles_n);
+    const int k_len = K / splits;
+    A += (int64_t)split * k_len * (AT ? M : 1);
+    B += (int64_t)split * k_len * (BT ? 1 : N);
+    if (splits > 1) Cv = (float *)Cv + (int64_t)split * M * N;
     int tm, tn;
     {
-        const int b = blockIdx.x, nb = tiles_m * tiles_n;
+        const int b = blockIdx.x % (tiles_m * tiles_n), nb = tiles_m * tiles_n;
         if (nb % 8 == 0 && tiles_m % 4 == 0 && tiles_n % 8 == 0 && (tiles_m / 4) * (tiles_n / 8) % 8 == 0) {
             const int xcd = b & 7, local = b >> 3;            // local: index among this XCD's tiles
             const int patches_n = tiles_n / 8;
@@ -193,7 +200,7 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
         fb_off[q] = A_STAGE + (BT ? frag_kc_off(wn * 128 + (lane & 31), q, lane) : frag_mn_off(wn * 128 + q * 32, lane));
     }
 
-    const int KT = K / BK;
+    const int KT = k_len / BK;
 #pragma unroll
     for (int u = 0; u < 16; u++) gload(u, 0);
 #pragma unroll
@@ -341,11 +348,55 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
     }
 }
 
+// Folds the [splits, M, N] f32 partials and applies the epilogue; one thread per 4 consecutive columns.
+__global__ __launch_bounds__(256) void gemm_splitk_fold_k(const float *__restrict__ ws, void *__restrict__ Cv,
+                                                          const void *__restrict__ bias, const void *__restrict__ residual,
+                                                          int epi, int bias_dtype, int out_bf16, int64_t MN, int N, int splits) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= MN) return;
+    f32x4 a = *(const f32x4 *)(ws + i);
+    for (int z = 1; z < splits; z++) a += *(const f32x4 *)(ws + (int64_t)z * MN + i);
+    const int col = (int)(i % N);
+    float v[4] = {a[0], a[1], a[2], a[3]};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        if (epi >= 1) v[k] += bias_dtype == DT_BF16 ? bf16_to_f32(((const uint16_t *)bias)[col + k]) : ((const float *)bias)[col + k];
+        if (epi == 2) v[k] = (v[k] > 0.0f ? 1.0f : 0.0f) * v[k];
+        if (epi == 3) v[k] = gelu_fast(v[k]);
+    }
+    if (!out_bf16) {
+        if (residual) {
+            const f32x4 r = *(const f32x4 *)((const float *)residual + i);
+#pragma unroll
+            for (int k = 0; k < 4; k++) v[k] += r[k];
+        }
+        *(f32x4 *)((float *)Cv + i) = f32x4{v[0], v[1], v[2], v[3]};
+    } else {
+        if (residual) {
+            const uint2 r = *(const uint2 *)((const uint16_t *)residual + i);
+            v[0] += __uint_as_float(r.x << 16); v[1] += __uint_as_float(r.x & 0xffff0000u);
+            v[2] += __uint_as_float(r.y << 16); v[3] += __uint_as_float(r.y & 0xffff0000u);
+        }
+        *(uint2 *)((uint16_t *)Cv + i) = make_uint2((__float_as_uint(v[0]) >> 16) | (__float_as_uint(v[1]) & 0xffff0000u),
+                                                    (__float_as_uint(v[2]) >> 16) | (__float_as_uint(v[3]) & 0xffff0000u));
+    }
+}
+
 template <bool AT, bool BT> hipError_t launch_epi(const GemmBf16 &p, hipStream_t st) {
-    dim3 grid((unsigned)((p.M / BM) * (p.N / BN))), block(256);
+    const int splits = gemm_bf16_splits(p.M, p.N, p.K);
+    dim3 grid((unsigned)((p.M / BM) * (p.N / BN) * splits)), block(256);
+    if (splits > 1) {
+        if (!p.workspace) return hipErrorInvalidValue;
+        hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0>), grid, block, GEMM_LDS, st, (const uint16_t *)p.A, (const uint16_t *)p.B,
+                           p.workspace, nullptr, nullptr, 0, 0, (int)p.M, (int)p.N, (int)p.K, splits);
+        const int64_t MN = p.M * p.N;
+        hipLaunchKernelGGL(gemm_splitk_fold_k, dim3((unsigned)((MN / 4 + 255) / 256)), block, 0, st, (const float *)p.workspace, p.C,
+                           p.bias, p.residual, p.epilogue, p.bias_dtype, p.out_bf16, MN, (int)p.N, splits);
+        return hipGetLastError();
+    }
 #define ZK_GEMM(E)                                                                                                    \
     hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E>), grid, block, GEMM_LDS, st, (const uint16_t *)p.A,                    \
-                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K);
+                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1);
     switch (p.epilogue) {
     case 0: ZK_GEMM(0) break;
     case 1: ZK_GEMM(1) break;
@@ -383,6 +434,19 @@ hipError_t gemm_bf16_init() {
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K) {
     return M > 0 && N > 0 && K > 0 && M % BM == 0 && N % BN == 0 && K % BK == 0 && M < (1 << 30) && N < (1 << 30) &&
            K < (1 << 30) && (M / BM) * (N / BN) < (1ll << 31);
+}
+
+// Split K when the output has too few 256x256 tiles to occupy the 256 CUs: the smallest power of two that
+// brings tiles * splits to 192 or more, while every split keeps at least 4 K tiles.
+int gemm_bf16_splits(int64_t M, int64_t N, int64_t K) {
+    const int64_t tiles = (M / BM) * (N / BN);
+    int s = 1;
+    while (tiles * s < 192 && s < 16 && K % (2 * s * BK) == 0 && K / (2 * s) >= 4 * BK) s *= 2;
+    return s;
+}
+uint64_t gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    const int s = gemm_bf16_splits(M, N, K);
+    return s > 1 ? (uint64_t)s * M * N * 4 : 0;
 }
 
 hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t st) {

@@ -56,7 +56,10 @@ struct GemmBf16 {
     int out_bf16;
     const void *A, *B, *bias, *residual; // residual may be null
     void *C;
+    void *workspace; // gemm_bf16_workspace_bytes(M, N, K) bytes (split-K partials), may be null when that is 0
 };
+int gemm_bf16_splits(int64_t M, int64_t N, int64_t K);
+uint64_t gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K);
 hipError_t gemm_bf16_init(); // once per device, before the first launch
 hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t stream);

@@ -252,6 +252,14 @@ uint64_t dtype_bytes(int32_t dt) {
 }
 
 // Fills arity and per-argument byte requirements; rejects shapes/dtypes no kernel covers.
+// bf16 problems of tile-multiple shape run on the 256x256 LDS-tiled kernel, everything else on the general one.
+bool gemm_takes_fast_path(const zhip_kernel_desc &d) {
+    const int64_t batch = d.dims[3] ? d.dims[3] : 1;
+    const float alpha = d.fparams[0] == 0.0f ? 1.0f : d.fparams[0];
+    return d.dtype == ZHIP_BF16 && batch == 1 && alpha == 1.0f && (d.iparams[0] == 0 || d.iparams[1] != ZHIP_F16) &&
+           zk::gemm_bf16_supported(d.dims[0], d.dims[1], d.dims[2]);
+}
+
 // Shape and scalar parameters of the two attention kinds.
 zk::Attention attention_args(const zhip_kernel_desc &d) {
     zk::Attention a{};
@@ -362,6 +370,7 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.n_in = a;
         p.need[a] = (uint64_t)batch * M * N * dtype_bytes(d.out_dtype);
         p.n_out = 1;
+        if (gemm_takes_fast_path(d)) p.workspace_bytes = zk::gemm_bf16_workspace_bytes(M, N, K);
         return ZHIP_OK;
     }
     case ZHIP_K_NORM_ROWS: {
@@ -590,9 +599,7 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         const int64_t batch = d.dims[3] ? d.dims[3] : 1;
         const float alpha = d.fparams[0] == 0.0f ? 1.0f : d.fparams[0];
         const void *residual = d.iparams[2] ? ptr[p.n_in - 1] : nullptr;
-        const bool fast = d.dtype == ZHIP_BF16 && batch == 1 && alpha == 1.0f &&
-                          (d.iparams[0] == 0 || d.iparams[1] != ZHIP_F16) && zk::gemm_bf16_supported(d.dims[0], d.dims[1], d.dims[2]);
-        if (fast) {
+        if (gemm_takes_fast_path(d)) {
             zk::GemmBf16 a{};
             a.M = d.dims[0];
             a.N = d.dims[1];
@@ -607,6 +614,7 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
             a.residual = residual;
             a.out_bf16 = d.out_dtype == ZHIP_BF16;
             a.C = ptr[p.n_in];
+            a.workspace = p.workspace;
             return zk::gemm_bf16(a, st);
         }
         zk::GemmGeneric g{};
