@@ -208,3 +208,69 @@ def test_gelu_grad_chain(hip, oracle):
     hb, gb = oracle.f32_to_bf16(h), oracle.f32_to_bf16(dg)
     got, want = run_chain(dev, pool, cb, [hb, gb]), oracle.ew_chain(cb, [hb, gb])
     assert np.all(np.abs(oracle.bf16_to_f32(got) - oracle.bf16_to_f32(want)) <= 2.0 ** -7 * np.abs(oracle.bf16_to_f32(want)) + 1e-6)
+
+
+# ---- chains above the size threshold run as code generated and compiled for that one program ----------------
+BIG = (1024, 2048)  # 2 Mi elements: above the default threshold of 1 Mi
+
+
+def _big_inputs(oracle, seed=0):
+    r = oracle.Rng(seed)
+    return r.randn(BIG, 2.0), r.randn(BIG), r.randn((BIG[1],)), r.randn((BIG[0],))
+
+
+def test_generated_chain_f32_all_operand_kinds(hip, oracle):
+    from zyx_amd import DType
+    from zyx_amd.kernels import Chain, EW_ROW, EW_COL, EW_SCALAR, run_chain
+    dev, pool = hip
+    x, y, rowv, colv = _big_inputs(oracle)
+    c = Chain(*BIG)
+    ix, iy, ir, ic = c.input(), c.input(), c.input(DType.F32, EW_ROW), c.input(DType.F32, EW_COL)
+    c.load(ix).mul(iy).save().add(ir).max(ic).mad(Chain.T, c.const(0.25)).relu().sub(c.const(1.5))
+    got, want = run_chain(dev, pool, c, [x, y, rowv, colv]), oracle.ew_chain(c, [x, y, rowv, colv])
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+    c = Chain(*BIG)
+    ix, isc = c.input(), c.input(DType.F32, EW_SCALAR)
+    c.load(ix).cmplt(isc).where(c.const(2.0), ix)
+    s = np.array([0.3], np.float32)
+    assert np.array_equal(run_chain(dev, pool, c, [x, s]), oracle.ew_chain(c, [x, s]))
+
+
+@pytest.mark.parametrize("op", ["gelu", "gelu_grad", "tanh", "sigmoid", "exp", "rsqrt", "neg", "abs"])
+def test_generated_unary_bf16(hip, oracle, op):
+    from zyx_amd import DType
+    from zyx_amd.kernels import Chain, run_chain
+    dev, pool = hip
+    x = oracle.f32_to_bf16(np.abs(_big_inputs(oracle, 1)[0]) + 0.01 if op == "rsqrt" else _big_inputs(oracle, 1)[0])
+    c = Chain(*BIG, out_dtype=DType.BF16)
+    getattr(c.load(c.input(DType.BF16)), op)()
+    got, want = oracle.bf16_to_f32(run_chain(dev, pool, c, [x])), oracle.bf16_to_f32(oracle.ew_chain(c, [x]))
+    ok = np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + 1e-6   # one truncating store apart at most
+    assert np.all(ok | (np.isnan(want) & (np.isnan(got) | np.isfinite(got))))
+
+
+def test_generated_mixed_dtypes_and_int_chain(hip, oracle):
+    from zyx_amd import DType
+    from zyx_amd.kernels import Chain, EW_ROW, run_chain
+    dev, pool = hip
+    x, y, rowv, _ = _big_inputs(oracle, 2)
+    # f32 master weights - lr * bf16 gradient -> f16 copy: three storage dtypes in one chain
+    c = Chain(*BIG, out_dtype=DType.F16)
+    ip, ig = c.input(DType.F32), c.input(DType.BF16)
+    c.load(ig).mul(c.const(0.01)).rsub(ip)
+    g = oracle.f32_to_bf16(y)
+    assert np.array_equal(run_chain(dev, pool, c, [x, g]), oracle.ew_chain(c, [x, g]))
+    # int32 registers, u8 and i32 operands, row-broadcast i32, u8 result
+    rng = np.random.default_rng(0)
+    a = rng.integers(0, 256, BIG).astype(np.uint8)
+    b = rng.integers(-1000, 1000, BIG).astype(np.int32)
+    r = rng.integers(1, 9, BIG[1]).astype(np.int32)
+    ci = Chain(*BIG, reg=DType.I32, out_dtype=DType.U8)
+    ia, ib, ir = ci.input(DType.U8), ci.input(DType.I32), ci.input(DType.I32, EW_ROW)
+    ci.load(ia).mul(ib).div(ir).bitxor(ib).shr(ci.const(3.0)).bitand(ci.const(255.0))
+    assert np.array_equal(run_chain(dev, pool, ci, [a, b, r]), oracle.ew_chain(ci, [a, b, r]))
+    ci = Chain(*BIG, reg=DType.I32, out_dtype=DType.I32)
+    ia, ib = ci.input(DType.I32), ci.input(DType.I32)
+    ci.load(ia).mod(ib).save().cmplt(ci.const(0.0)).where(ib, ci.const(0.0)).add(Chain.T)
+    b2 = rng.integers(-7, 8, BIG).astype(np.int32)
+    assert np.array_equal(run_chain(dev, pool, ci, [b, b2]), oracle.ew_chain(ci, [b, b2]))

@@ -4,6 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <string>
 
 namespace zk {
 
@@ -30,6 +31,13 @@ struct Elementwise {
     void *out;
 };
 hipError_t elementwise(const Elementwise &p, hipStream_t stream);
+// The same chain as code generated for this one program and compiled at run time (ew_jit.cpp).
+struct EwJit;
+bool ew_jit_eligible(const Elementwise &p, int *vector_width);
+EwJit *ew_jit_compile(const Elementwise &p, std::string &error);
+bool ew_jit_can_launch(const EwJit *j, const Elementwise &p);
+hipError_t ew_jit_launch(const EwJit *j, const Elementwise &p, hipStream_t stream);
+void ew_jit_destroy(EwJit *j);
 
 // Sum / max over the last axis (axis0 == 0) or over axis 0 (axis0 == 1) of x[rows, cols].
 struct Reduce {

@@ -21,6 +21,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -68,6 +69,7 @@ struct Program {
     uint64_t need[8] = {0}; // minimum bytes per argument
     void *workspace = nullptr; // device scratch owned by the program (two-stage reductions)
     uint64_t workspace_bytes = 0;
+    zk::EwJit *jit = nullptr;  // elementwise chains above the size threshold: code specialised at registration
 };
 
 struct Plan {
@@ -103,6 +105,7 @@ struct zhip_ctx {
     std::mutex mu;
     int device = 0;
     uint32_t debug = 0;
+    int64_t ew_jit_min = 1 << 20; // elementwise chains of at least this many elements are compiled at registration
     std::string last_error;
     hipDeviceProp_t prop{};
     zhip_device_info info{};
@@ -252,6 +255,25 @@ uint64_t dtype_bytes(int32_t dt) {
 }
 
 // Fills arity and per-argument byte requirements; rejects shapes/dtypes no kernel covers.
+// The chain program of a ZHIP_K_ELEMENTWISE descriptor, without pointers.
+zk::Elementwise elementwise_args(const zhip_kernel_desc &d) {
+    zk::Elementwise a{};
+    a.rows = d.dims[0];
+    a.cols = d.dims[1];
+    a.n_in = d.iparams[0];
+    a.n_instr = d.iparams[1];
+    a.reg_class = d.dtype;
+    a.out_dtype = d.out_dtype;
+    for (int k = 0; k < a.n_in; k++) {
+        a.in_dtype[k] = d.iparams[2 + k] & 0xff;
+        a.in_bcast[k] = (d.iparams[2 + k] >> 8) & 0xff;
+        if (a.in_bcast[k] == ZHIP_EW_ROW || a.in_bcast[k] == ZHIP_EW_COL) a.need_rowcol = 1;
+    }
+    for (int j = 0; j < a.n_instr; j++) a.code[j] = (uint32_t)d.iparams[6 + j];
+    for (int k = 0; k < 8; k++) a.consts[k] = d.fparams[k];
+    return a;
+}
+
 // bf16 problems of tile-multiple shape run on the 256x256 LDS-tiled kernel, everything else on the general one.
 bool gemm_takes_fast_path(const zhip_kernel_desc &d) {
     const int64_t batch = d.dims[3] ? d.dims[3] : 1;
@@ -564,22 +586,10 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         return zk::softmax_rows(a, st);
     }
     case ZHIP_K_ELEMENTWISE: {
-        zk::Elementwise a{};
-        a.rows = d.dims[0];
-        a.cols = d.dims[1];
-        a.n_in = d.iparams[0];
-        a.n_instr = d.iparams[1];
-        a.reg_class = d.dtype;
-        a.out_dtype = d.out_dtype;
-        for (int k = 0; k < a.n_in; k++) {
-            a.in_dtype[k] = d.iparams[2 + k] & 0xff;
-            a.in_bcast[k] = (d.iparams[2 + k] >> 8) & 0xff;
-            if (a.in_bcast[k] == ZHIP_EW_ROW || a.in_bcast[k] == ZHIP_EW_COL) a.need_rowcol = 1;
-            a.in[k] = ptr[k];
-        }
-        for (int j = 0; j < a.n_instr; j++) a.code[j] = (uint32_t)d.iparams[6 + j];
-        for (int k = 0; k < 8; k++) a.consts[k] = d.fparams[k];
+        zk::Elementwise a = elementwise_args(d);
+        for (int k = 0; k < a.n_in; k++) a.in[k] = ptr[k];
         a.out = ptr[a.n_in];
+        if (zk::ew_jit_can_launch(p.jit, a)) return zk::ew_jit_launch(p.jit, a, st);
         return zk::elementwise(a, st);
     }
     case ZHIP_K_REDUCE: {
@@ -856,6 +866,7 @@ ZHIP_EXPORT int32_t zhip_init(const zhip_config *cfg, zhip_ctx **out) {
     zhip_ctx *c = new zhip_ctx();
     c->device = cfg->device_id;
     c->debug = cfg->debug;
+    if (const char *e = getenv("ZYX_HIP_EW_JIT_MIN")) c->ew_jit_min = atoll(e);
     c->cache_limit = cfg->cache_bytes ? cfg->cache_bytes : kDefaultCacheBytes;
     auto bail = [&](int32_t st, const char *what, hipError_t err) {
         g_init_error = std::string(what) + ": " + hipGetErrorString(err);
@@ -907,8 +918,10 @@ ZHIP_EXPORT int32_t zhip_deinit(zhip_ctx *c) {
         trim_cache(c, 0);
         for (Buffer &b : c->buffers.items)
             if (b.kind == Buffer::Memory) (void)hipFree(b.ptr);
-        for (Program &p : c->programs.items)
+        for (Program &p : c->programs.items) {
             if (p.live && p.workspace) (void)hipFree(p.workspace);
+            if (p.live && p.jit) zk::ew_jit_destroy(p.jit);
+        }
         for (EventSlot &s : c->events) (void)hipEventDestroy(s.ev);
         (void)hipEventDestroy(c->prof_a);
         (void)hipEventDestroy(c->prof_b);
@@ -1134,6 +1147,19 @@ ZHIP_EXPORT int32_t zhip_register_kernel(zhip_ctx *c, const zhip_kernel_desc *de
             return rc;
         }
     }
+    // Large chains get code generated for exactly this program (zyx compiles every fused kernel at run time,
+    // zyx/src/backend/mod.rs:899-933); small ones run on the interpreting kernel, where the ~0.3 s compile
+    // would not pay. ZYX_HIP_EW_JIT_MIN overrides the element-count threshold (0 = always, -1 = never).
+    if (desc->kind == ZHIP_K_ELEMENTWISE) {
+        const zk::Elementwise a = elementwise_args(*desc);
+        int v;
+        if (c->ew_jit_min >= 0 && a.rows * a.cols >= c->ew_jit_min && zk::ew_jit_eligible(a, &v)) {
+            std::string err;
+            (void)hipSetDevice(c->device);
+            p.jit = zk::ew_jit_compile(a, err);
+            if (!p.jit) return c->fail(ZHIP_KERNEL_COMPILATION, "elementwise chain: %s", err.c_str());
+        }
+    }
     p.live = true;
     *prog = c->programs.push(p);
     if (c->debug & 128) fprintf(stderr, "[zyx-hip] program %u = kind %d\n", *prog, desc->kind);
@@ -1156,6 +1182,12 @@ ZHIP_EXPORT int32_t zhip_release_program(zhip_ctx *c, zhip_prog prog) {
         (void)hipSetDevice(c->device);
         (void)hipFree(p.workspace);
         p.workspace = nullptr;
+    }
+    if (p.jit) {
+        (void)hipSetDevice(c->device);
+        (void)hipDeviceSynchronize(); // a launch of the module may still be running
+        zk::ew_jit_destroy(p.jit);
+        p.jit = nullptr;
     }
     p.live = false;
     c->programs.remove(prog);
