@@ -161,7 +161,8 @@ __global__ __launch_bounds__(256) void reduce_cols_k(const typename Elem<DT>::S 
 #pragma unroll
     for (int k = 0; k < W; k++) acc[k] = F::init();
     if (c < cols) {
-        for (int64_t r = r0 + wave; r < r1; r += 4) {
+#pragma unroll 8
+        for (int64_t r = r0 + wave; r < r1; r += 4) { // unrolled: 8 independent row loads in flight per thread
             if (VEC) {
                 A v[4];
                 Elem<DT>::ld4(x, r * cols + c, v);
@@ -191,11 +192,18 @@ __global__ __launch_bounds__(256) void reduce_col_partials_k(const typename Elem
                                                              int chunks) {
     typedef typename Elem<DT>::A A;
     typedef Fold<OP, A> F;
-    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (c >= cols) return;
+    // a workgroup folds 64 columns: lane -> column, the 4 waves split the chunks, LDS joins them
+    __shared__ A lds[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t c = (int64_t)blockIdx.x * 64 + lane;
     A acc = F::init();
-    for (int k = 0; k < chunks; k++) acc = F::f(acc, partial[(int64_t)k * cols + c]);
-    Elem<DT>::st(out, c, acc);
+    if (c < cols) {
+#pragma unroll 8
+        for (int k = wave; k < chunks; k += 4) acc = F::f(acc, partial[(int64_t)k * cols + c]);
+    }
+    lds[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && c < cols) Elem<DT>::st(out, c, F::f(F::f(lds[0][lane], lds[1][lane]), F::f(lds[2][lane], lds[3][lane])));
 }
 
 struct RowPlan { int segs; int64_t seg_len; };
@@ -251,7 +259,7 @@ template <int DT, int OP> hipError_t launch(const Reduce &p, hipStream_t st) {
         if (vec) hipLaunchKernelGGL((reduce_cols_k<DT, OP, true>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len);
         else hipLaunchKernelGGL((reduce_cols_k<DT, OP, false>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len);
         if (pl.chunks > 1)
-            hipLaunchKernelGGL((reduce_col_partials_k<DT, OP>), dim3((unsigned)((p.cols + 255) / 256)), block, 0, st, ws, out, p.cols, pl.chunks);
+            hipLaunchKernelGGL((reduce_col_partials_k<DT, OP>), dim3((unsigned)((p.cols + 63) / 64)), block, 0, st, ws, out, p.cols, pl.chunks);
     }
     return hipGetLastError();
 }

@@ -207,40 +207,81 @@ __global__ __launch_bounds__(256) void norm_bwd_dx_k(const typename RowIO<DT>::S
     }
 }
 
-// Partial parameter gradients: thread = column, workgroup = 256 columns x one chunk of rows.
+// Partial parameter gradients. A workgroup owns a strip of 256 columns (lane -> 4 adjacent columns, 64 when the
+// row width is not a multiple of 4) and one chunk of rows, split over its 4 waves and joined through LDS.
 // part[(chunk*2 + 0)*cols + c] = sum dy*xh, part[(chunk*2 + 1)*cols + c] = sum dy over the chunk.
-template <int DT>
+template <int DT, bool VEC>
 __global__ __launch_bounds__(256) void norm_bwd_param_k(const typename RowIO<DT>::S *__restrict__ x,
                                                         const typename RowIO<DT>::S *__restrict__ dy,
                                                         const float *__restrict__ stats, float *__restrict__ part,
                                                         int64_t rows, int cols, int64_t rows_per_chunk) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= cols) return;
+    constexpr int W = VEC ? 4 : 1;
+    __shared__ float lds[4][2][64 * W];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = (blockIdx.x * 64 + lane) * W;
     const int64_t r0 = (int64_t)blockIdx.y * rows_per_chunk, r1 = r0 + rows_per_chunk < rows ? r0 + rows_per_chunk : rows;
-    float pw = 0.0f, pb = 0.0f;
-    for (int64_t r = r0; r < r1; r++) {
-        const float g = RowIO<DT>::ld(dy, r * cols + c);
-        pw = __builtin_fmaf(g, (RowIO<DT>::ld(x, r * cols + c) - stats[r * 2]) * stats[r * 2 + 1], pw);
-        pb += g;
+    float pw[W], pb[W];
+#pragma unroll
+    for (int k = 0; k < W; k++) pw[k] = pb[k] = 0.0f;
+    if (c < cols) {
+#pragma unroll 4
+        for (int64_t r = r0 + wave; r < r1; r += 4) {
+            const float mean = stats[r * 2], rstd = stats[r * 2 + 1];
+            float g[4], xv[4];
+            if (VEC) {
+                RowIO<DT>::ld4(dy, r * cols + c, g);
+                RowIO<DT>::ld4(x, r * cols + c, xv);
+            } else {
+                g[0] = RowIO<DT>::ld(dy, r * cols + c);
+                xv[0] = RowIO<DT>::ld(x, r * cols + c);
+            }
+#pragma unroll
+            for (int k = 0; k < W; k++) {
+                pw[k] = __builtin_fmaf(g[k], (xv[k] - mean) * rstd, pw[k]);
+                pb[k] += g[k];
+            }
+        }
     }
-    part[((int64_t)blockIdx.y * 2) * cols + c] = pw;
-    part[((int64_t)blockIdx.y * 2 + 1) * cols + c] = pb;
+#pragma unroll
+    for (int k = 0; k < W; k++) {
+        lds[wave][0][lane * W + k] = pw[k];
+        lds[wave][1][lane * W + k] = pb[k];
+    }
+    __syncthreads();
+    if (wave == 0 && c < cols) {
+#pragma unroll
+        for (int k = 0; k < W; k++) {
+            const int i = lane * W + k;
+            part[((int64_t)blockIdx.y * 2) * cols + c + k] = (lds[0][0][i] + lds[1][0][i]) + (lds[2][0][i] + lds[3][0][i]);
+            part[((int64_t)blockIdx.y * 2 + 1) * cols + c + k] = (lds[0][1][i] + lds[1][1][i]) + (lds[2][1][i] + lds[3][1][i]);
+        }
+    }
 }
+// lane -> column of a 64-column strip, the 4 waves split the chunks
 template <int DT>
 __global__ __launch_bounds__(256) void norm_bwd_param_sum_k(const float *__restrict__ part, typename RowIO<DT>::S *__restrict__ dw,
                                                             typename RowIO<DT>::S *__restrict__ db, int cols, int chunks) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= cols) return;
+    __shared__ float lds[4][2][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + lane;
     float sw = 0.0f, sb = 0.0f;
-    for (int k = 0; k < chunks; k++) {
-        sw += part[((int64_t)k * 2) * cols + c];
-        sb += part[((int64_t)k * 2 + 1) * cols + c];
+    if (c < cols) {
+#pragma unroll 8
+        for (int k = wave; k < chunks; k += 4) {
+            sw += part[((int64_t)k * 2) * cols + c];
+            sb += part[((int64_t)k * 2 + 1) * cols + c];
+        }
     }
-    if (dw) RowIO<DT>::st(dw, c, sw);
-    if (db) RowIO<DT>::st(db, c, sb);
+    lds[wave][0][lane] = sw;
+    lds[wave][1][lane] = sb;
+    __syncthreads();
+    if (wave == 0 && c < cols) {
+        if (dw) RowIO<DT>::st(dw, c, (lds[0][0][lane] + lds[1][0][lane]) + (lds[2][0][lane] + lds[3][0][lane]));
+        if (db) RowIO<DT>::st(db, c, (lds[0][1][lane] + lds[1][1][lane]) + (lds[2][1][lane] + lds[3][1][lane]));
+    }
 }
 
-int norm_bwd_chunks(int64_t rows) { return (int)(rows < 64 * 32 ? (rows + 31) / 32 : 64); }
+int norm_bwd_chunks(int64_t rows) { return (int)(rows < 256 * 32 ? (rows + 31) / 32 : 256); }
 
 template <int DT, int MODE> hipError_t launch_norm_bwd(const NormRowsBwd &p, hipStream_t st) {
     typedef typename RowIO<DT>::S S;
@@ -254,9 +295,9 @@ template <int DT, int MODE> hipError_t launch_norm_bwd(const NormRowsBwd &p, hip
     if (p.dw || p.db) {
         const int chunks = norm_bwd_chunks(p.rows);
         const int64_t rpc = (p.rows + chunks - 1) / chunks;
-        const unsigned cb = (unsigned)((p.cols + 255) / 256);
-        hipLaunchKernelGGL((norm_bwd_param_k<DT>), dim3(cb, (unsigned)chunks), block, 0, st, (const S *)p.x, (const S *)p.dy, stats, part, p.rows, (int)p.cols, rpc);
-        hipLaunchKernelGGL((norm_bwd_param_sum_k<DT>), dim3(cb), block, 0, st, part, (S *)p.dw, (S *)p.db, (int)p.cols, chunks);
+        if (vec) hipLaunchKernelGGL((norm_bwd_param_k<DT, true>), dim3((unsigned)((p.cols + 255) / 256), (unsigned)chunks), block, 0, st, (const S *)p.x, (const S *)p.dy, stats, part, p.rows, (int)p.cols, rpc);
+        else hipLaunchKernelGGL((norm_bwd_param_k<DT, false>), dim3((unsigned)((p.cols + 63) / 64), (unsigned)chunks), block, 0, st, (const S *)p.x, (const S *)p.dy, stats, part, p.rows, (int)p.cols, rpc);
+        hipLaunchKernelGGL((norm_bwd_param_sum_k<DT>), dim3((unsigned)((p.cols + 63) / 64)), block, 0, st, part, (S *)p.dw, (S *)p.db, (int)p.cols, chunks);
     }
     return hipGetLastError();
 }
