@@ -25,7 +25,7 @@ def reference(oracle, a, b, trans_a, trans_b):
 
 
 @pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("mnk", [(256, 256, 64), (256, 512, 128), (512, 256, 576), (1024, 2048, 512)])
+@pytest.mark.parametrize("mnk", [(256, 256, 64), (256, 512, 128), (512, 256, 576), (1024, 2048, 512), (256, 384, 256), (3072, 4096, 256)])
 def test_bf16_gemm_layouts(hip, oracle, mnk, trans_a, trans_b):
     dev, pool = hip
     m, n, k = mnk

@@ -38,11 +38,12 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define ZK_LDS __attribute__((address_space(3)))
 #define ZK_GLOBAL __attribute__((address_space(1)))
 
-constexpr int BM = 256, BN = 256, BK = 64;
+// Workgroup tile BM x BNV x BK with BNV = 256 (4 waves of 128 x 128) or 128 (4 waves of 128 x 64, for outputs
+// whose N is only a multiple of 128 or that have too few 256 x 256 tiles to occupy the chip).
+constexpr int BM = 256, BK = 64;
 constexpr int A_STAGE = BM * BK * 2;           // 32 KiB
-constexpr int B_STAGE = BN * BK * 2;           // 32 KiB
-constexpr int STAGE = A_STAGE + B_STAGE;       // 64 KiB
-constexpr int GEMM_LDS = 2 * STAGE;            // 128 KiB
+constexpr int stage_bytes(int bnv) { return A_STAGE + bnv * BK * 2; }   // 64 KiB / 48 KiB
+constexpr int lds_bytes(int bnv) { return 2 * stage_bytes(bnv); }       // 128 KiB / 96 KiB
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -52,7 +53,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // 16-byte slots modulo 256 bytes. Thread (wave w, lane l) moves, for i = 0..7, the chunk
 // that belongs at row i*32 + w*8 + l/8, physical slot l%8.
 __device__ __forceinline__ int swz_kc(int row) { return (row >> 1) & 7; }
-struct TileKC {
+struct TileKC { // NCHUNK chunks per thread = rows / 32
     static __device__ __forceinline__ const uint16_t *src(const uint16_t *g, int64_t ld, int row0, int k0, int i, int wave,
                                                          int lane) {
         const int row = i * 32 + wave * 8 + (lane >> 3);
@@ -65,15 +66,20 @@ struct TileKC {
 // MN-contiguous operand tile: 64 k rows x 256 columns, LDS layout [k][chunk ^ swz(k)],
 // 512-byte rows, swz(k) = (k & 3) << 1. Thread (w, l) moves, for i = 0..7, the chunk at
 // k row i*8 + w*2 + l/32, physical slot l%32.
-__device__ __forceinline__ int swz_mn(int k) { return (k & 3) << 1; }
-struct TileMN {
+// COLS = 128: 256-byte rows, swz(k) = (k & 3) << 2 (the four k rows of a transposing read then fall into four
+// different 64-byte bank windows); thread (w, l) moves, for i = 0..3, the chunk at k row i*16 + w*4 + l/16.
+template <int COLS> __device__ __forceinline__ int swz_mn(int k) { return COLS == 256 ? (k & 3) << 1 : (k & 3) << 2; }
+template <int COLS> struct TileMN {
+    static constexpr int CH = COLS / 8;          // 16-byte chunks per k row
+    static constexpr int KPW = 64 / CH;          // k rows one wave covers per pass
+    static constexpr int NCHUNK = COLS / 32;     // passes (chunks per thread)
     static __device__ __forceinline__ const uint16_t *src(const uint16_t *g, int64_t ld, int col0, int k0, int i, int wave,
                                                          int lane) {
-        const int k = i * 8 + wave * 2 + (lane >> 5);
-        const int c = (lane & 31) ^ swz_mn(k);
+        const int k = i * 4 * KPW + wave * KPW + lane / CH;
+        const int c = (lane % CH) ^ swz_mn<COLS>(k);
         return g + (int64_t)(k0 + k) * ld + col0 + c * 8;
     }
-    static constexpr __host__ __device__ __forceinline__ int dst(int i, int wave, int lane) { return (i * 8 + wave * 2) * 512 + lane * 16; }
+    static constexpr __host__ __device__ __forceinline__ int dst(int i, int wave, int lane) { return (i * 4 * KPW + wave * KPW) * COLS * 2 + lane * 16; }
     static __device__ __forceinline__ int64_t k_advance(int64_t ld) { return BK * ld; }
 };
 
@@ -96,15 +102,15 @@ __device__ __forceinline__ bf16x8 frag_kc(const ZK_LDS uint8_t *lds, int off) {
 // column i of those 4 k rows. swz(k) only depends on k & 3 = (lane & 15) >> 2, so one
 // offset per 32-column block serves all k steps and both halves: mn_off[block] +
 // ks*16*512 (+ 4*512).
-__device__ __forceinline__ int frag_mn_off(int col_base, int lane) {
+template <int COLS> __device__ __forceinline__ int frag_mn_off(int col_base, int lane) {
     const int g16 = lane >> 4, r = lane & 15;
     const int col = col_base + (g16 & 1) * 16 + (r & 3) * 4;
     const int k = (g16 >> 1) * 8 + (r >> 2);
-    return k * 512 + (((col >> 3) ^ swz_mn(k)) << 4) + (col & 4) * 2;
+    return k * COLS * 2 + (((col >> 3) ^ swz_mn<COLS>(k)) << 4) + (col & 4) * 2;
 }
-__device__ __forceinline__ bf16x8 frag_mn(const ZK_LDS uint8_t *lds, int off) {
+template <int COLS> __device__ __forceinline__ bf16x8 frag_mn(const ZK_LDS uint8_t *lds, int off) {
     bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(lds + off));
-    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(lds + off + 4 * 512));
+    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(lds + off + 4 * COLS * 2));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
@@ -118,19 +124,24 @@ __device__ __forceinline__ float gelu_fast(float x) {
 
 // AT: A stored [K, M] (M contiguous) instead of [M, K]; BT: B stored [N, K] (K contiguous)
 // instead of [K, N]. EPI: 0 none, 1 + bias, 2 + bias then ReLU, 3 + bias then GELU.
-template <bool AT, bool BT, int EPI>
+template <bool AT, bool BT, int EPI, int BNV>
 __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                       void *__restrict__ Cv, const void *__restrict__ bias,
                                                       const void *__restrict__ residual, int bias_dtype, int out_bf16,
                                                       int M, int N, int K, int splits) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
+    constexpr int NJ = BNV / 64;                 // 32-column MFMA blocks per wave
+    constexpr int NB = BNV / 32;                 // B staging chunks per thread
+    constexpr int NU = 8 + NB;                   // staging units per K tile
+    constexpr int WN = BNV / 2;                  // columns per wave
+    constexpr int STAGE = stage_bytes(BNV);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
 
     // XCD-aware tile order: ids congruent mod 8 land on one XCD; give each XCD a patch
     // of 4 x 8 tiles (or the whole grid when it is smaller).
-    const int tiles_m = M / BM, tiles_n = N / BN;
+    const int tiles_m = M / BM, tiles_n = N / BNV;
     // split-K: workgroup z of a tile multiplies K range [z, z+1) * K/splits and stores its raw f32 partial
     // tile into slice z of Cv (a [splits, M, N] workspace that a second kernel folds)
     const int split = blockIdx.x / (tiles_m * tiles_n);
@@ -154,13 +165,13 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
             tn = b % tiles_n;
         }
     }
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int m0 = tm * BM, n0 = tn * BNV;
 
-    f32x16 acc[4][4];
+    f32x16 acc[4][NJ];
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < NJ; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
@@ -169,42 +180,44 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
     // Global addresses are a wave-uniform byte pointer that advances with the K tile plus a
     // per-thread 32-bit offset fixed for the whole kernel; LDS addresses are one per-thread
     // offset plus constants.
-    typedef typename std::conditional<AT, TileMN, TileKC>::type TA;
-    typedef typename std::conditional<BT, TileKC, TileMN>::type TB;
+    typedef typename std::conditional<AT, TileMN<256>, TileKC>::type TA;
+    typedef typename std::conditional<BT, TileKC, TileMN<BNV>>::type TB;
     const int64_t lda = AT ? M : K, ldb = BT ? K : N;
-    uint32_t oa[8], ob[8];
+    uint32_t oa[8], ob[NB];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        oa[i] = (uint32_t)((TA::src(A, lda, m0, 0, i, wave, lane) - A) * 2);
-        ob[i] = (uint32_t)((TB::src(B, ldb, n0, 0, i, wave, lane) - B) * 2);
-    }
+    for (int i = 0; i < 8; i++) oa[i] = (uint32_t)((TA::src(A, lda, m0, 0, i, wave, lane) - A) * 2);
+#pragma unroll
+    for (int i = 0; i < NB; i++) ob[i] = (uint32_t)((TB::src(B, ldb, n0, 0, i, wave, lane) - B) * 2);
     const int da0 = TA::dst(0, wave, lane), db0 = A_STAGE + TB::dst(0, wave, lane);
     constexpr int da_step = TA::dst(1, 0, 0) - TA::dst(0, 0, 0), db_step = TB::dst(1, 0, 0) - TB::dst(0, 0, 0);
     const int64_t adv_a = TA::k_advance(lda) * 2, adv_b = TB::k_advance(ldb) * 2;
-    u32x4 ra[8], rb[8];
-    // staging unit u = 0..15: operand A (u even) or B (u odd), chunk u >> 1
+    u32x4 ra[8], rb[NB];
+    // staging unit u = 0..NU-1. BNV = 256: operand A (u even) or B (u odd), chunk u >> 1. BNV = 128: every
+    // third unit is a B chunk (u % 3 == 2 -> B chunk u / 3), the others A chunks 2*(u/3) + u%3.
+    auto unit_is_b = [](int u) { return NJ == 4 ? (u & 1) != 0 : u % 3 == 2; };
+    auto unit_chunk = [](int u) { return NJ == 4 ? u >> 1 : (u % 3 == 2 ? u / 3 : 2 * (u / 3) + u % 3); };
     auto gload = [&](int u, int kt) {
-        const int i = u >> 1;
-        if (u & 1) rb[i] = *(const u32x4 *)((const uint8_t *)B + kt * adv_b + ob[i]);
+        const int i = unit_chunk(u);
+        if (unit_is_b(u)) rb[i] = *(const u32x4 *)((const uint8_t *)B + kt * adv_b + ob[i]);
         else ra[i] = *(const u32x4 *)((const uint8_t *)A + kt * adv_a + oa[i]);
     };
     auto lwrite = [&](int u, int da_base, int db_base) {
-        const int i = u >> 1;
-        if (u & 1) *(ZK_LDS u32x4 *)(smem + db_base + i * db_step) = rb[i];
+        const int i = unit_chunk(u);
+        if (unit_is_b(u)) *(ZK_LDS u32x4 *)(smem + db_base + i * db_step) = rb[i];
         else *(ZK_LDS u32x4 *)(smem + da_base + i * da_step) = ra[i];
     };
     int fa_off[4], fb_off[4]; // per k step (K-contiguous) or per 32-wide block (MN-contiguous)
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        fa_off[q] = AT ? frag_mn_off(wm * 128 + q * 32, lane) : frag_kc_off(wm * 128 + (lane & 31), q, lane);
-        fb_off[q] = A_STAGE + (BT ? frag_kc_off(wn * 128 + (lane & 31), q, lane) : frag_mn_off(wn * 128 + q * 32, lane));
+        fa_off[q] = AT ? frag_mn_off<256>(wm * 128 + q * 32, lane) : frag_kc_off(wm * 128 + (lane & 31), q, lane);
+        fb_off[q] = A_STAGE + (BT ? frag_kc_off(wn * WN + (lane & 31), q, lane) : frag_mn_off<BNV>(wn * WN + (q % NJ) * 32, lane));
     }
 
     const int KT = k_len / BK;
 #pragma unroll
-    for (int u = 0; u < 16; u++) gload(u, 0);
+    for (int u = 0; u < NU; u++) gload(u, 0);
 #pragma unroll
-    for (int u = 0; u < 16; u++) {
+    for (int u = 0; u < NU; u++) {
         lwrite(u, da0, db0);
         gload(u, min(1, KT - 1));
     }
@@ -213,21 +226,22 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
     // Fragments are double-buffered in registers: while the 16 MFMAs of k step s run, the
     // 8 LDS reads of step s+1 are in flight. The step after the last one of a tile lives
     // in the other stage, so the hand-over barrier sits before the last step's MFMAs.
-    bf16x8 af[2][4], bfr[2][4];
-    // fragment r = 0..3: A block r; r = 4..7: B block r - 4. fa/fb are the four per-lane
+    bf16x8 af[2][4], bfr[2][NJ];
+    // fragment r = 0..3: A block r; r = 4..3+NJ: B block r - 4. fa/fb are the four per-lane
     // offsets of each operand with the stage folded in.
+    constexpr int NFRAG = 4 + NJ;
     auto load_frag = [&](const int (&fa)[4], const int (&fb)[4], int ks, int buf, int r) {
         if (r < 4) {
-            if (AT) af[buf][r] = frag_mn(smem, fa[r] + ks * 16 * 512);
+            if (AT) af[buf][r] = frag_mn<256>(smem, fa[r] + ks * 16 * 512);
             else af[buf][r] = frag_kc(smem, fa[ks] + r * 32 * 128);
         } else {
             const int j = r - 4;
             if (BT) bfr[buf][j] = frag_kc(smem, fb[ks] + j * 32 * 128);
-            else bfr[buf][j] = frag_mn(smem, fb[j] + ks * 16 * 512);
+            else bfr[buf][j] = frag_mn<BNV>(smem, fb[j] + ks * 16 * BNV * 2);
         }
     };
 #pragma unroll
-    for (int r = 0; r < 8; r++) load_frag(fa_off, fb_off, 0, 0, r);
+    for (int r = 0; r < NFRAG; r++) load_frag(fa_off, fb_off, 0, 0, r);
 
     // One K tile = 4 k steps of 16 MFMAs. During tile c (stage c & 1) each step writes two
     // staged chunk pairs of tile c+1 into the other stage and re-issues their loads for
@@ -260,21 +274,32 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
     auto k_step = [&](const int ks, int kt, const bool handover) {
         const int cur = ks & 1, nxt = cur ^ 1;
         const bool last = ks == BK / 16 - 1;
-        const int u0 = ks * 6, nu = ks < 2 ? 6 : (ks == 2 ? 4 : 0);
+        constexpr int MF = 4 * NJ; // MFMAs per k step
+        // BNV = 256: 6, 6, 4 staging units in steps 0..2 (after even MFMAs), one fragment read after every odd one.
+        // BNV = 128: 4, 4, 4 units; 6 fragment reads over the 4 odd slots (2, 1, 2, 1).
+        const int u0 = NJ == 4 ? ks * 6 : ks * 4, nu = NJ == 4 ? (ks < 2 ? 6 : (ks == 2 ? 4 : 0)) : (ks < 3 ? 4 : 0);
 #pragma unroll
-        for (int m = 0; m < 16; m++) {
+        for (int m = 0; m < MF; m++) {
             __builtin_amdgcn_sched_barrier(0);
-            acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][m >> 2], bfr[cur][m & 3], acc[m >> 2][m & 3], 0, 0, 0);
+            acc[m / NJ][m % NJ] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][m / NJ], bfr[cur][m % NJ], acc[m / NJ][m % NJ], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             if (!last) {
                 if ((m & 1) == 0 && handover && (m >> 1) < nu) {
                     lwrite(u0 + (m >> 1), nda, ndb);
                     gload(u0 + (m >> 1), min(kt + 2, KT - 1));
                 }
-                if (m & 1) load_frag(cfa, cfb, ks + 1, nxt, m >> 1);
+                if (m & 1) {
+                    if (NJ == 4) load_frag(cfa, cfb, ks + 1, nxt, m >> 1);
+                    else {
+                        const int s_ = m >> 1, r0 = s_ + (s_ + 1) / 2; // slots hold fragments {0,1}, {2}, {3,4}, {5}
+                        load_frag(cfa, cfb, ks + 1, nxt, r0);
+                        if ((s_ & 1) == 0) load_frag(cfa, cfb, ks + 1, nxt, r0 + 1);
+                    }
+                }
             } else if (handover) {
-                if (m == 3) __syncthreads(); // tile kt+1 is complete in LDS; nobody reads this stage any more
-                if (m >= 3 && m < 11) load_frag(nfa, nfb, 0, nxt, m - 3);
+                constexpr int SYNC_AT = NJ == 4 ? 3 : 1;
+                if (m == SYNC_AT) __syncthreads(); // tile kt+1 is complete in LDS; nobody reads this stage any more
+                if (m >= SYNC_AT && m < SYNC_AT + NFRAG) load_frag(nfa, nfb, 0, nxt, m - SYNC_AT);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -300,8 +325,8 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
         return v;
     };
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int col = n0 + wn * 128 + j * 32 + col_in;
+    for (int j = 0; j < NJ; j++) {
+        const int col = n0 + wn * WN + j * 32 + col_in;
         float bv = 0.0f;
         if (EPI >= 1) {
             if (bias_dtype == DT_BF16) bv = bf16_to_f32(((const uint16_t *)bias)[col]);
@@ -382,12 +407,12 @@ __global__ __launch_bounds__(256) void gemm_splitk_fold_k(const float *__restric
     }
 }
 
-template <bool AT, bool BT> hipError_t launch_epi(const GemmBf16 &p, hipStream_t st) {
+template <bool AT, bool BT, int BNV> hipError_t launch_epi(const GemmBf16 &p, hipStream_t st) {
     const int splits = gemm_bf16_splits(p.M, p.N, p.K);
-    dim3 grid((unsigned)((p.M / BM) * (p.N / BN) * splits)), block(256);
+    dim3 grid((unsigned)((p.M / BM) * (p.N / BNV) * splits)), block(256);
     if (splits > 1) {
         if (!p.workspace) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0>), grid, block, GEMM_LDS, st, (const uint16_t *)p.A, (const uint16_t *)p.B,
+        hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0, BNV>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, (const uint16_t *)p.B,
                            p.workspace, nullptr, nullptr, 0, 0, (int)p.M, (int)p.N, (int)p.K, splits);
         const int64_t MN = p.M * p.N;
         hipLaunchKernelGGL(gemm_splitk_fold_k, dim3((unsigned)((MN / 4 + 255) / 256)), block, 0, st, (const float *)p.workspace, p.C,
@@ -395,7 +420,7 @@ template <bool AT, bool BT> hipError_t launch_epi(const GemmBf16 &p, hipStream_t
         return hipGetLastError();
     }
 #define ZK_GEMM(E)                                                                                                    \
-    hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E>), grid, block, GEMM_LDS, st, (const uint16_t *)p.A,                    \
+    hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E, BNV>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A,         \
                        (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1);
     switch (p.epilogue) {
     case 0: ZK_GEMM(0) break;
@@ -407,16 +432,23 @@ template <bool AT, bool BT> hipError_t launch_epi(const GemmBf16 &p, hipStream_t
 #undef ZK_GEMM
     return hipGetLastError();
 }
+template <bool AT, bool BT> hipError_t launch_width(const GemmBf16 &p, hipStream_t st) {
+    return gemm_bf16_tile_n(p.M, p.N) == 128 ? launch_epi<AT, BT, 128>(p, st) : launch_epi<AT, BT, 256>(p, st);
+}
 
-template <bool AT, bool BT, int E> hipError_t allow_lds() {
-    return hipFuncSetAttribute((const void *)gemm_bf16_k<AT, BT, E>, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS);
+template <bool AT, bool BT, int E, int BNV> hipError_t allow_lds() {
+    return hipFuncSetAttribute((const void *)gemm_bf16_k<AT, BT, E, BNV>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
 }
 template <bool AT, bool BT> hipError_t allow_lds_epi() {
     hipError_t e;
-    if ((e = allow_lds<AT, BT, 0>()) != hipSuccess) return e;
-    if ((e = allow_lds<AT, BT, 1>()) != hipSuccess) return e;
-    if ((e = allow_lds<AT, BT, 2>()) != hipSuccess) return e;
-    return allow_lds<AT, BT, 3>();
+    if ((e = allow_lds<AT, BT, 0, 256>()) != hipSuccess) return e;
+    if ((e = allow_lds<AT, BT, 1, 256>()) != hipSuccess) return e;
+    if ((e = allow_lds<AT, BT, 2, 256>()) != hipSuccess) return e;
+    if ((e = allow_lds<AT, BT, 3, 256>()) != hipSuccess) return e;
+    if ((e = allow_lds<AT, BT, 0, 128>()) != hipSuccess) return e;
+    if ((e = allow_lds<AT, BT, 1, 128>()) != hipSuccess) return e;
+    if ((e = allow_lds<AT, BT, 2, 128>()) != hipSuccess) return e;
+    return allow_lds<AT, BT, 3, 128>();
 }
 
 } // namespace
@@ -432,14 +464,19 @@ hipError_t gemm_bf16_init() {
 }
 
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K) {
-    return M > 0 && N > 0 && K > 0 && M % BM == 0 && N % BN == 0 && K % BK == 0 && M < (1 << 30) && N < (1 << 30) &&
-           K < (1 << 30) && (M / BM) * (N / BN) < (1ll << 31);
+    return M > 0 && N > 0 && K > 0 && M % BM == 0 && N % 128 == 0 && K % BK == 0 && M < (1 << 30) && N < (1 << 30) &&
+           K < (1 << 30) && (M / BM) * (N / 128) < (1ll << 27);
 }
 
-// Split K when the output has too few 256x256 tiles to occupy the 256 CUs: the smallest power of two that
+// Tile width: 128 columns when N is not a multiple of 256 or when 256-wide tiles would leave CUs idle.
+int gemm_bf16_tile_n(int64_t M, int64_t N) {
+    return (N % 256 != 0 || (M / BM) * (N / 256) < 192) ? 128 : 256;
+}
+
+// Split K when the output still has too few tiles to occupy the 256 CUs: the smallest power of two that
 // brings tiles * splits to 192 or more, while every split keeps at least 4 K tiles.
 int gemm_bf16_splits(int64_t M, int64_t N, int64_t K) {
-    const int64_t tiles = (M / BM) * (N / BN);
+    const int64_t tiles = (M / BM) * (N / gemm_bf16_tile_n(M, N));
     int s = 1;
     while (tiles * s < 192 && s < 16 && K % (2 * s * BK) == 0 && K / (2 * s) >= 4 * BK) s *= 2;
     return s;
@@ -451,8 +488,8 @@ uint64_t gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 
 hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t st) {
     if (!gemm_bf16_supported(p.M, p.N, p.K)) return hipErrorInvalidValue;
-    if (p.trans_a) return p.trans_b ? launch_epi<true, true>(p, st) : launch_epi<true, false>(p, st);
-    return p.trans_b ? launch_epi<false, true>(p, st) : launch_epi<false, false>(p, st);
+    if (p.trans_a) return p.trans_b ? launch_width<true, true>(p, st) : launch_width<true, false>(p, st);
+    return p.trans_b ? launch_width<false, true>(p, st) : launch_width<false, false>(p, st);
 }
 
 } // namespace zk

@@ -66,6 +66,7 @@ struct GemmBf16 {
     void *C;
     void *workspace; // gemm_bf16_workspace_bytes(M, N, K) bytes (split-K partials), may be null when that is 0
 };
+int gemm_bf16_tile_n(int64_t M, int64_t N);
 int gemm_bf16_splits(int64_t M, int64_t N, int64_t K);
 uint64_t gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K);
