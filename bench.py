@@ -131,7 +131,8 @@ def extra_block(dev, pool, steps=20, warmup=5, cpu=True):
     blk.write("x", trunc(x))
     blk.write("dout", trunc(np.ones((B * T, D), np.float32)))
     res = {"kernels_forward": len(blk.forward_nodes), "kernels_forward_backward": len(blk.forward_nodes) + len(blk.backward_nodes)}
-    for name, fn, flop in (("forward", blk.forward, fwd_flop), ("forward_backward", blk.forward_backward, 3 * fwd_flop)):
+    for name, fn, flop in (("forward", blk.forward, fwd_flop), ("forward_backward", blk.forward_backward, 3 * fwd_flop),
+                           ("forward_backward_launch_by_launch", blk.forward_backward_unplanned, 3 * fwd_flop)):
         for _ in range(warmup):
             fn()
         blk.sync()

@@ -96,3 +96,54 @@ def test_max_pool(hip, oracle, args):
     assert np.array_equal(max_pool2d(dev, pool, x, *args), oracle.max_pool2d(x, *args))
     xb = oracle.f32_to_bf16(x)
     assert np.array_equal(max_pool2d(dev, pool, xb, *args, dtype=DType.BF16), oracle.max_pool2d(xb, *args, dtype=oracle.BF16))
+
+
+@pytest.mark.parametrize("case", [
+    # (N, C, H, W, Cout, k, stride, pad, dilation): pixels % 256 == 0, Cout % 128 == 0, C*k*k % 64 == 0 -> patches + tiled GEMM
+    (4, 64, 16, 16, 128, 3, 1, 1, 1), (2, 64, 32, 32, 256, 1, 1, 0, 1), (8, 16, 16, 16, 128, 2, 2, 0, 1), (1, 64, 34, 34, 128, 3, 2, 1, 2)])
+@pytest.mark.parametrize("bias,relu", [(True, True), (False, True), (True, False), (False, False)])
+def test_conv_bf16_on_the_tiled_gemm(hip, oracle, case, bias, relu):
+    dev, pool = hip
+    n, c, h, w, co, k, s, p, d = case
+    r = oracle.Rng(n + c + k)
+    x, wt = oracle.f32_to_bf16(r.randn((n, c, h, w))), oracle.f32_to_bf16(r.randn((co, c, k, k), 0.1))
+    b = oracle.f32_to_bf16(r.randn(co, 0.5)) if bias else None
+    args = ((s, s), (p, p), (d, d))
+    mag = oracle.conv2d(np.abs(oracle.bf16_to_f32(x)), np.abs(oracle.bf16_to_f32(wt)), None if b is None else np.abs(oracle.bf16_to_f32(b)), *args)
+    got = conv2d(dev, pool, x, wt, b, *args, relu=relu, dtype=DType.BF16)
+    want = oracle.conv2d(x, wt, b, *args, relu, oracle.BF16)
+    assert got.shape == want.shape and (got.shape[0] * got.shape[2] * got.shape[3]) % 256 == 0
+    g, wv = oracle.bf16_to_f32(got), oracle.bf16_to_f32(want)
+    # the oracle stores the 16-bit sum (truncating) before a second kernel adds the bias; the GPU adds the bias in
+    # the same kernel and stores once: they differ by up to one bf16 unit of the pre-bias value
+    pre = np.abs(wv) + (np.abs(oracle.bf16_to_f32(b)).reshape(1, -1, 1, 1) if bias else 0.0)
+    assert np.all(np.abs(g - wv) <= 2.0 ** -7 * pre + 1e-3 * mag)
+    got32 = conv2d(dev, pool, x, wt, b, *args, relu=relu, dtype=DType.BF16, out_dtype=DType.F32)
+    want32 = oracle.conv2d(x, wt, b, *args, relu, oracle.BF16, oracle.F32)
+    assert np.all(np.abs(got32 - want32) <= 1e-3 * np.abs(want32) + 2e-5 * mag)
+    # identical arithmetic before the store: the bf16 result is the truncation of the f32 one
+    assert np.array_equal(got, oracle.f32_to_bf16(got32))
+
+
+def test_config4_bf16_full_size(hip, oracle):
+    """N=32, C=64, 56x56, 3x3 -> 128, pad 1, ReLU, then 2x2 max-pool, bf16 storage: 4 images against the oracle,
+    all of it through linearity in the weights (ReLU off) and batch independence."""
+    dev, pool = hip
+    r = oracle.Rng(42069)
+    x = oracle.f32_to_bf16(r.randn((32, 64, 56, 56)))
+    w1 = oracle.f32_to_bf16(r.randn((128, 64, 3, 3), float(np.sqrt(2.0 / 576))))
+    y, pooled = conv2d(dev, pool, x, w1, None, (1, 1), (1, 1), relu=True, dtype=DType.BF16, pool_kernel=(2, 2))
+    assert y.shape == (32, 128, 56, 56) and pooled.shape == (32, 128, 28, 28)
+    sel = [0, 11, 31]
+    want = oracle.bf16_to_f32(oracle.conv2d(x[sel], w1, None, (1, 1), (1, 1), (1, 1), True, oracle.BF16))
+    mag = oracle.conv2d(np.abs(oracle.bf16_to_f32(x[sel])), np.abs(oracle.bf16_to_f32(w1)), None, (1, 1), (1, 1))
+    assert np.all(np.abs(oracle.bf16_to_f32(y[sel]) - want) <= 2.0 ** -7 * np.abs(want) + 1e-3 * mag)
+    assert np.array_equal(pooled, oracle.max_pool2d(y, dtype=oracle.BF16))
+    # f32 results of bf16 operands are linear in the weights up to f32 summation error
+    w2 = oracle.f32_to_bf16(r.randn((128, 64, 3, 3), 0.05))
+    w12 = oracle.f32_to_bf16(oracle.bf16_to_f32(w1) * 0.5)  # exact in bf16
+    ya = conv2d(dev, pool, x, w1, None, (1, 1), (1, 1), dtype=DType.BF16, out_dtype=DType.F32)
+    yb = conv2d(dev, pool, x, w12, None, (1, 1), (1, 1), dtype=DType.BF16, out_dtype=DType.F32)
+    assert np.array_equal(yb, ya * 0.5)  # scaling the weights by a power of two scales every product exactly
+    assert np.array_equal(conv2d(dev, pool, x[7:15], w2, None, (1, 1), (1, 1), dtype=DType.BF16, out_dtype=DType.F32),
+                          conv2d(dev, pool, x, w2, None, (1, 1), (1, 1), dtype=DType.BF16, out_dtype=DType.F32)[7:15])

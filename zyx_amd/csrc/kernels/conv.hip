@@ -138,11 +138,97 @@ __global__ __launch_bounds__(256) void max_pool2d_k(const MaxPool2d p) {
     }
 }
 
+// Patch matrix of the convolution, transposed: a[k][pixel] with k = (c*KH + ky)*KW + kx (the order of the
+// flattened weight [Cout, C*KH*KW]) and pixel = (n*OH + oy)*OW + ox; padding reads as 0. Rows of `a` run
+// along the image rows of x, so reads and the 16-byte writes are both coalesced. One thread = 8 pixels.
+__global__ __launch_bounds__(256) void im2col_t_bf16_k(const uint16_t *__restrict__ x, uint16_t *__restrict__ a, const Conv2d p,
+                                                      int64_t pixels) {
+    const int k = blockIdx.y;
+    const int kx = k % p.KW, ky = (k / p.KW) % p.KH, c = k / (p.KW * p.KH);
+    const int64_t pix0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (pix0 >= pixels) return;
+    const int plane = p.OH * p.OW;
+    int n = (int)(pix0 / plane), rem = (int)(pix0 - (int64_t)n * plane);
+    int oy = rem / p.OW, ox = rem - oy * p.OW;
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    const int iy0 = oy * p.sy - p.py + ky * p.dy, ix0 = ox * p.sx - p.px + kx * p.dx;
+    if (p.sx == 1 && ox + 8 <= p.OW) {
+        // the 8 pixels lie in one output row: one input row, 8 consecutive columns
+        if (iy0 >= 0 && iy0 < p.H) {
+            const uint16_t *row = x + (((int64_t)n * p.C + c) * p.H + iy0) * p.W;
+            if (ix0 >= 0 && ix0 + 8 <= p.W) {
+                typedef uint32_t u32x4a2 __attribute__((ext_vector_type(4), aligned(2)));
+                const u32x4a2 t = *(const u32x4a2 *)(row + ix0); // 2-byte aligned 128-bit load
+                w[0] = t[0]; w[1] = t[1]; w[2] = t[2]; w[3] = t[3];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int ix = ix0 + e;
+                    const uint32_t v = (ix >= 0 && ix < p.W) ? row[ix] : 0u;
+                    w[e >> 1] |= v << (16 * (e & 1));
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int iy = oy * p.sy - p.py + ky * p.dy, ix = ox * p.sx - p.px + kx * p.dx;
+            uint32_t v = 0;
+            if (iy >= 0 && iy < p.H && ix >= 0 && ix < p.W) v = x[(((int64_t)n * p.C + c) * p.H + iy) * p.W + ix];
+            w[e >> 1] |= v << (16 * (e & 1));
+            if (++ox == p.OW) {
+                ox = 0;
+                if (++oy == p.OH) {
+                    oy = 0;
+                    n++;
+                }
+            }
+        }
+    }
+    *(uint4 *)(a + (int64_t)k * pixels + pix0) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// bf16 convolutions whose lowered product fits the tiled MFMA GEMM exactly: patches . W^T with
+// M = pixels (multiple of 256), N = Cout (multiple of 128), K = C*KH*KW (multiple of 64), no K split.
+bool conv_uses_gemm(const Conv2d &p) {
+    const int64_t pixels = (int64_t)p.N * p.OH * p.OW, K = (int64_t)p.C * p.KH * p.KW;
+    return p.dtype == DT_BF16 && pixels > 0 && pixels % 256 == 0 && (p.OH * p.OW) % 4 == 0 && p.Cout % 128 == 0 && K % 64 == 0 &&
+           K <= 65535 && pixels < (1ll << 30) && gemm_bf16_supported(pixels, p.Cout, K) && gemm_bf16_splits(pixels, p.Cout, K) == 1;
+}
+constexpr uint64_t kZeroBiasBytes = 4096 * 4;
+
 } // namespace
+
+// scratch = [zero bias (for ReLU without bias)] [patch matrix K x pixels bf16]
+uint64_t conv2d_scratch_bytes(const Conv2d &p) {
+    if (!conv_uses_gemm(p) || p.Cout > 4096) return 0;
+    return kZeroBiasBytes + (uint64_t)p.C * p.KH * p.KW * (uint64_t)p.N * p.OH * p.OW * 2;
+}
 
 hipError_t conv2d(const Conv2d &p, hipStream_t st) {
     const int64_t P = (int64_t)p.N * p.OH * p.OW;
     if (P <= 0 || p.Cout <= 0) return hipSuccess;
+    if (p.scratch && conv2d_scratch_bytes(p)) {
+        // im2col (transposed) + GEMM: C[pixel, co] = sum_k a[k, pixel] * w[co, k], stored as NCHW by the epilogue
+        uint16_t *a = (uint16_t *)((char *)p.scratch + kZeroBiasBytes);
+        const int K = p.C * p.KH * p.KW;
+        hipLaunchKernelGGL(im2col_t_bf16_k, dim3((unsigned)((P / 8 + 255) / 256), (unsigned)K), dim3(256), 0, st, (const uint16_t *)p.x, a, p, P);
+        GemmBf16 g{};
+        g.M = P;
+        g.N = p.Cout;
+        g.K = K;
+        g.trans_a = 1;
+        g.trans_b = 1;
+        g.epilogue = p.relu ? 2 : (p.bias ? 1 : 0);
+        g.bias_dtype = DT_BF16;
+        g.out_bf16 = p.out_dtype == DT_BF16;
+        g.plane = p.OH * p.OW;
+        g.A = a;
+        g.B = p.w;
+        g.bias = p.bias ? p.bias : p.scratch; // the head of scratch is kept zero
+        g.C = p.y;
+        return gemm_bf16(g, st);
+    }
     if ((p.Cout + CM - 1) / CM > 65535 || (P + CN - 1) / CN >= (1ll << 31)) return hipErrorInvalidValue;
     dim3 grid((unsigned)((P + CN - 1) / CN), (unsigned)((p.Cout + CM - 1) / CM)), block(256);
     if (p.dtype == DT_F32 && p.out_dtype == DT_F32) hipLaunchKernelGGL((conv2d_k<DT_F32, DT_F32>), grid, block, 0, st, p);

@@ -128,7 +128,7 @@ template <bool AT, bool BT, int EPI, int BNV>
 __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                       void *__restrict__ Cv, const void *__restrict__ bias,
                                                       const void *__restrict__ residual, int bias_dtype, int out_bf16,
-                                                      int M, int N, int K, int splits) {
+                                                      int M, int N, int K, int splits, int plane) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
     constexpr int NJ = BNV / 64;                 // 32-column MFMA blocks per wave
@@ -332,7 +332,25 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
             if (bias_dtype == DT_BF16) bv = bf16_to_f32(((const uint16_t *)bias)[col]);
             else bv = ((const float *)bias)[col];
         }
-        if (!out_bf16) {
+        if (plane) {
+            // C is stored as [M / plane, N, plane] (the NCHW result of a convolution lowered to this product:
+            // row = image * plane + pixel, column = channel). The four consecutive rows a lane holds per
+            // register group are consecutive pixels of one image (plane % 4 == 0): one 16- or 8-byte store.
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int row = m0 + wm * 128 + i * 32 + row_in + g * 8;
+                    const int img = row / plane, pix = row - img * plane;
+                    const int64_t o = ((int64_t)img * N + col) * plane + pix;
+                    float v[4];
+#pragma unroll
+                    for (int k = 0; k < 4; k++) v[k] = finish(acc[i][j][4 * g + k], bv);
+                    if (out_bf16) *(uint2 *)((uint16_t *)Cv + o) = make_uint2((__float_as_uint(v[0]) >> 16) | (__float_as_uint(v[1]) & 0xffff0000u),
+                                                                                (__float_as_uint(v[2]) >> 16) | (__float_as_uint(v[3]) & 0xffff0000u));
+                    else *(f32x4 *)((float *)Cv + o) = f32x4{v[0], v[1], v[2], v[3]};
+                }
+        } else if (!out_bf16) {
             float *C = (float *)Cv;
             const float *R = (const float *)residual;
 #pragma unroll
@@ -409,11 +427,12 @@ __global__ __launch_bounds__(256) void gemm_splitk_fold_k(const float *__restric
 
 template <bool AT, bool BT, int BNV> hipError_t launch_epi(const GemmBf16 &p, hipStream_t st) {
     const int splits = gemm_bf16_splits(p.M, p.N, p.K);
+    if (p.plane && (splits > 1 || p.residual || p.plane % 4 || p.M % p.plane)) return hipErrorInvalidValue;
     dim3 grid((unsigned)((p.M / BM) * (p.N / BNV) * splits)), block(256);
     if (splits > 1) {
         if (!p.workspace) return hipErrorInvalidValue;
         hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0, BNV>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, (const uint16_t *)p.B,
-                           p.workspace, nullptr, nullptr, 0, 0, (int)p.M, (int)p.N, (int)p.K, splits);
+                           p.workspace, nullptr, nullptr, 0, 0, (int)p.M, (int)p.N, (int)p.K, splits, 0);
         const int64_t MN = p.M * p.N;
         hipLaunchKernelGGL(gemm_splitk_fold_k, dim3((unsigned)((MN / 4 + 255) / 256)), block, 0, st, (const float *)p.workspace, p.C,
                            p.bias, p.residual, p.epilogue, p.bias_dtype, p.out_bf16, MN, (int)p.N, splits);
@@ -421,7 +440,7 @@ template <bool AT, bool BT, int BNV> hipError_t launch_epi(const GemmBf16 &p, hi
     }
 #define ZK_GEMM(E)                                                                                                    \
     hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E, BNV>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A,         \
-                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1);
+                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, p.plane);
     switch (p.epilogue) {
     case 0: ZK_GEMM(0) break;
     case 1: ZK_GEMM(1) break;

@@ -62,6 +62,7 @@ struct GemmBf16 {
     int epilogue;      // 0 none, 1 bias, 2 bias+relu, 3 bias+gelu
     int bias_dtype;    // DT_BF16 or DT_F32
     int out_bf16;
+    int plane; // 0, or C is stored [M / plane, N, plane] (rows of one group of `plane` are contiguous per column)
     const void *A, *B, *bias, *residual; // residual may be null
     void *C;
     void *workspace; // gemm_bf16_workspace_bytes(M, N, K) bytes (split-K partials), may be null when that is 0
@@ -122,7 +123,9 @@ struct Conv2d {
     const void *x, *w, *bias;
     void *y;
     const int32_t *koff, *kdyx;
+    void *scratch; // conv2d_scratch_bytes(p) bytes when the product runs on the tiled MFMA GEMM, else unused
 };
+uint64_t conv2d_scratch_bytes(const Conv2d &p);
 hipError_t conv2d(const Conv2d &p, hipStream_t stream);
 
 // max-pool over the last two axes of `planes` images [H, W] -> [OH, OW]

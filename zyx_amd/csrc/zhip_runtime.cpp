@@ -255,6 +255,20 @@ uint64_t dtype_bytes(int32_t dt) {
 }
 
 // Fills arity and per-argument byte requirements; rejects shapes/dtypes no kernel covers.
+// Shape parameters of a ZHIP_K_CONV2D descriptor, without pointers.
+zk::Conv2d conv_args(const zhip_kernel_desc &d) {
+    zk::Conv2d a{};
+    a.N = (int)d.dims[0]; a.C = (int)d.dims[1]; a.H = (int)d.dims[2]; a.W = (int)d.dims[3];
+    a.Cout = (int)d.dims[4]; a.KH = (int)d.dims[5]; a.KW = (int)d.dims[6];
+    a.sy = d.iparams[0]; a.sx = d.iparams[1]; a.py = d.iparams[2]; a.px = d.iparams[3]; a.dy = d.iparams[4]; a.dx = d.iparams[5];
+    a.OH = (a.H + 2 * a.py - a.dy * (a.KH - 1) - 1) / a.sy + 1;
+    a.OW = (a.W + 2 * a.px - a.dx * (a.KW - 1) - 1) / a.sx + 1;
+    a.dtype = d.dtype; a.out_dtype = d.out_dtype; a.relu = d.iparams[7];
+    return a;
+}
+// the two int32 tap tables at the head of a conv program's workspace, rounded so what follows stays aligned
+uint64_t conv_table_bytes(const zhip_kernel_desc &d) { return ((uint64_t)d.dims[1] * d.dims[5] * d.dims[6] * 8 + 255) / 256 * 256; }
+
 // The chain program of a ZHIP_K_ELEMENTWISE descriptor, without pointers.
 zk::Elementwise elementwise_args(const zhip_kernel_desc &d) {
     zk::Elementwise a{};
@@ -467,7 +481,9 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.n_in = a;
         p.need[a] = (uint64_t)N * Co * OH * OW * dtype_bytes(d.out_dtype);
         p.n_out = 1;
-        p.workspace_bytes = (uint64_t)C * KH * KW * 8; // two int32 tables, filled at registration
+        // two int32 tables filled at registration, then (bf16 shapes that run on the tiled GEMM) a zero bias
+        // and the patch matrix
+        p.workspace_bytes = conv_table_bytes(d) + zk::conv2d_scratch_bytes(conv_args(d));
         return ZHIP_OK;
     }
     case ZHIP_K_MAX_POOL2D: {
@@ -568,6 +584,8 @@ int32_t program_fill_workspace(zhip_ctx *c, Program &p) {
                 tab[K + k] = (int32_t)(((ky * dy) << 16) | (kx * dx));
             }
     HIPCHK(c, hipMemcpy(p.workspace, tab.data(), tab.size() * 4, hipMemcpyHostToDevice), ZHIP_KERNEL_COMPILATION);
+    if (p.workspace_bytes > conv_table_bytes(d)) // head of the scratch part: the all-zero bias
+        HIPCHK(c, hipMemset((char *)p.workspace + conv_table_bytes(d), 0, 4096 * 4), ZHIP_KERNEL_COMPILATION);
     return ZHIP_OK;
 }
 
@@ -695,16 +713,11 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         return zk::cross_entropy(a, st);
     }
     case ZHIP_K_CONV2D: {
-        zk::Conv2d a{};
-        a.N = (int)d.dims[0]; a.C = (int)d.dims[1]; a.H = (int)d.dims[2]; a.W = (int)d.dims[3];
-        a.Cout = (int)d.dims[4]; a.KH = (int)d.dims[5]; a.KW = (int)d.dims[6];
-        a.sy = d.iparams[0]; a.sx = d.iparams[1]; a.py = d.iparams[2]; a.px = d.iparams[3]; a.dy = d.iparams[4]; a.dx = d.iparams[5];
-        a.OH = (a.H + 2 * a.py - a.dy * (a.KH - 1) - 1) / a.sy + 1;
-        a.OW = (a.W + 2 * a.px - a.dx * (a.KW - 1) - 1) / a.sx + 1;
-        a.dtype = d.dtype; a.out_dtype = d.out_dtype; a.relu = d.iparams[7];
+        zk::Conv2d a = conv_args(d);
         a.x = ptr[0]; a.w = ptr[1]; a.bias = d.iparams[6] ? ptr[2] : nullptr; a.y = ptr[p.n_in];
         a.koff = (const int32_t *)p.workspace;
         a.kdyx = a.koff + (int64_t)a.C * a.KH * a.KW;
+        if (zk::conv2d_scratch_bytes(a)) a.scratch = (char *)p.workspace + conv_table_bytes(d);
         return zk::conv2d(a, st);
     }
     case ZHIP_K_MAX_POOL2D: {
