@@ -114,6 +114,90 @@ def extra_conv(dev, pool, kernels, steps=50, warmup=50):
     return out
 
 
+def extra_streaming(dev, pool, kernels, steps=20, warmup=5):
+    """Memory-bound kernels at the transformer block's shapes: fused elementwise chains, column / row reductions,
+    LayerNorm forward and backward. GB/s = (bytes of every input + output tensor, each once) / kernel time."""
+    import zyx_amd
+    M, F, D = 8192, 4096, 1024
+    rng = np.random.default_rng(3)
+    out = {}
+
+    def dev_arr(shape, dt):
+        a = rng.standard_normal(shape, dtype=np.float32)
+        if dt == zyx_amd.DType.BF16:
+            a = (a.view(np.uint32) >> 16).astype(np.uint16)
+        b, e = kernels.to_device(pool, a)
+        pool.sync_events([e])
+        return b
+
+    def out_arr(n, isz):
+        b, e = kernels.alloc_like(pool, n, isz)
+        pool.sync_events([e])
+        return b
+
+    def timeit(name, desc, args, nbytes):
+        prog = dev.register_kernel(desc)
+        dev.profile_kernel(prog, [args], warmup)
+        us = dev.profile_kernel(prog, [args], steps)
+        out[name] = {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1), "frac_of_8TB/s": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        dev.release(prog)
+
+    for dt, isz, tag in ((zyx_amd.DType.BF16, 2, "bf16"), (zyx_amd.DType.F32, 4, "f32")):
+        h, g, o = dev_arr((M, F), dt), dev_arr((M, F), dt), out_arr(M * F, isz)
+        c = kernels.Chain(M, F, out_dtype=dt)
+        c.load(c.input(dt)).gelu()
+        timeit(f"gelu_{tag}_8192x4096", c.desc(), [h, o], 2 * M * F * isz)
+        c = kernels.Chain(M, F, out_dtype=dt)
+        a, b = c.input(dt), c.input(dt)
+        c.load(a).gelu_grad().mul(b)
+        timeit(f"gelu_grad_mul_{tag}_8192x4096", c.desc(), [h, g, o], 3 * M * F * isz)
+        c = kernels.Chain(M, F, out_dtype=dt)
+        a, b = c.input(dt), c.input(dt)
+        c.load(a).add(b)
+        timeit(f"add_{tag}_8192x4096", c.desc(), [h, g, o], 3 * M * F * isz)
+        timeit(f"colsum_{tag}_8192x4096", kernels.reduce_desc(M, F, "sum", axis0=True, dtype=dt), [h, out_arr(F, isz)], M * F * isz)
+        timeit(f"rowsum_{tag}_8192x4096", kernels.reduce_desc(M, F, "sum", dtype=dt), [h, out_arr(M, isz)], M * F * isz)
+        for b_ in (h, g, o):
+            pool.deallocate(b_, [])
+        x, w, bb, y = dev_arr((M, D), dt), dev_arr((D,), dt), dev_arr((D,), dt), out_arr(M * D, isz)
+        dy, ad = dev_arr((M, D), dt), dev_arr((M, D), dt)
+        timeit(f"layernorm_{tag}_8192x1024", kernels.norm_rows_desc(M, D, dtype=dt), [x, w, bb, y], 2 * M * D * isz)
+        timeit(f"layernorm_bwd_{tag}_8192x1024", kernels.norm_rows_bwd_desc(M, D, add=True, dtype=dt),
+               [x, w, dy, ad, y, out_arr(D, isz), out_arr(D, isz)], 4 * M * D * isz)
+        for b_ in (x, w, bb, y, dy, ad):
+            pool.deallocate(b_, [])
+    return out
+
+
+def extra_attention(dev, pool, kernels, steps=30, warmup=10):
+    """Config 5's attention core alone: B=8, T=1024, 16 heads x 64, bf16. FLOPs: 4*B*H*T*T*dh forward (QK^T, PV),
+    10*B*H*T*T*dh backward (5 products; the two-kernel backward recomputes QK^T and dy.V^T, not counted)."""
+    import zyx_amd
+    B, T, H, DH = 8, 1024, 16, 64
+    rng = np.random.default_rng(6)
+    trunc = lambda a: (a.view(np.uint32) >> 16).astype(np.uint16)
+    qkv = trunc(rng.standard_normal((B, T, 3 * H * DH), dtype=np.float32))
+    dy = trunc(rng.standard_normal((B, T, H * DH), dtype=np.float32))
+    xb, e0 = kernels.to_device(pool, qkv)
+    db, e1 = kernels.to_device(pool, dy)
+    yb, e2 = kernels.alloc_like(pool, B * T * H * DH, 2)
+    lb, e3 = kernels.alloc_like(pool, B * H * T, 4)
+    gb, e4 = kernels.alloc_like(pool, B * T * 3 * H * DH, 2)
+    pool.sync_events([e0, e1, e2, e3, e4])
+    fwd = dev.register_kernel(kernels.attention_desc(B, T, H, DH, zyx_amd.DType.BF16, lse=True))
+    bwd = dev.register_kernel(kernels.attention_bwd_desc(B, T, H, DH, zyx_amd.DType.BF16))
+    res = {}
+    for name, prog, args, flop in (("forward", fwd, [xb, yb, lb], 4.0 * B * H * T * T * DH), ("backward", bwd, [xb, yb, db, lb, gb], 10.0 * B * H * T * T * DH)):
+        dev.profile_kernel(prog, [args], warmup)
+        us = dev.profile_kernel(prog, [args], steps)
+        res[name] = {"us": round(us, 2), "TFLOP/s": round(flop / us / 1e6, 1), "frac_of_2.5PF_bf16_peak": round(flop / us / 1e6 / 2500.0, 4)}
+    dev.release(fwd)
+    dev.release(bwd)
+    for b_ in (xb, db, yb, lb, gb):
+        pool.deallocate(b_, [])
+    return res
+
+
 def extra_block(dev, pool, steps=20, warmup=5, cpu=True):
     """Config 5: pre-norm transformer block B=8 T=1024 d=1024 16 heads, bf16, forward and forward + backward, each
     one cached plan launch (8 and 24 kernels). FLOPs counted: the matrix products only (240.5 GFLOP forward)."""
@@ -220,6 +304,8 @@ def main():
                     help="run only the config-3 GEMM leg and print its numbers (used for profiling that kernel)")
     ap.add_argument("--conv-only", action="store_true", help="run only the config-4 conv + max-pool leg")
     ap.add_argument("--block-only", action="store_true", help="run only the config-5 transformer block leg")
+    ap.add_argument("--streaming-only", action="store_true", help="run only the memory-bound kernel leg")
+    ap.add_argument("--attention-only", action="store_true", help="run only the attention core leg")
     ap.add_argument("--counters", action="store_true",
                     help="short run for `rocprofv3 --pmc`: a few launches of the fused kernel and of a plain copy "
                          "kernel over the same 8192x4096 f32 tensor (known traffic: 134217728 B read + written), "
@@ -241,9 +327,15 @@ def main():
         pool.deinitialize()
         return
 
-    if args.conv_only or args.block_only:
-        res = {"config4_conv_relu_pool": extra_conv(dev, pool, kernels)} if args.conv_only else \
-            {"config5_transformer_block": extra_block(dev, pool, steps=args.steps if args.steps != 200 else 20, cpu=not args.no_cpu)}
+    if args.conv_only or args.block_only or args.streaming_only or args.attention_only:
+        if args.conv_only:
+            res = {"config4_conv_relu_pool": extra_conv(dev, pool, kernels)}
+        elif args.streaming_only:
+            res = {"memory_bound_kernels": extra_streaming(dev, pool, kernels)}
+        elif args.attention_only:
+            res = {"config5_attention_core": extra_attention(dev, pool, kernels)}
+        else:
+            res = {"config5_transformer_block": extra_block(dev, pool, steps=args.steps if args.steps != 200 else 20, cpu=not args.no_cpu)}
         print(json.dumps(res))
         pool.deinitialize()
         return
@@ -325,7 +417,9 @@ def main():
         out["extra"] = {"config3_gemm_bf16_4096": extra_gemm(dev, pool, kernels),
                         "config1_mlp_train": extra_mlp(dev, pool, cpu=not args.no_cpu),
                         "config4_conv_relu_pool": extra_conv(dev, pool, kernels),
-                        "config5_transformer_block": extra_block(dev, pool, cpu=not args.no_cpu)}
+                        "config5_attention_core": extra_attention(dev, pool, kernels),
+                        "config5_transformer_block": extra_block(dev, pool, cpu=not args.no_cpu),
+                        "memory_bound_kernels": extra_streaming(dev, pool, kernels)}
     pool.deinitialize()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(x)

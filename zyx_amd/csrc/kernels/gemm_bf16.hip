@@ -124,7 +124,7 @@ __device__ __forceinline__ float gelu_fast(float x) {
 
 // AT: A stored [K, M] (M contiguous) instead of [M, K]; BT: B stored [N, K] (K contiguous)
 // instead of [K, N]. EPI: 0 none, 1 + bias, 2 + bias then ReLU, 3 + bias then GELU.
-template <bool AT, bool BT, int EPI, int BNV>
+template <bool AT, bool BT, int EPI, int BNV, bool PLANE>
 __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                       void *__restrict__ Cv, const void *__restrict__ bias,
                                                       const void *__restrict__ residual, int bias_dtype, int out_bf16,
@@ -332,7 +332,7 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
             if (bias_dtype == DT_BF16) bv = bf16_to_f32(((const uint16_t *)bias)[col]);
             else bv = ((const float *)bias)[col];
         }
-        if (plane) {
+        if (PLANE) {
             // C is stored as [M / plane, N, plane] (the NCHW result of a convolution lowered to this product:
             // row = image * plane + pixel, column = channel). The four consecutive rows a lane holds per
             // register group are consecutive pixels of one image (plane % 4 == 0): one 16- or 8-byte store.
@@ -431,16 +431,30 @@ template <bool AT, bool BT, int BNV> hipError_t launch_epi(const GemmBf16 &p, hi
     dim3 grid((unsigned)((p.M / BM) * (p.N / BNV) * splits)), block(256);
     if (splits > 1) {
         if (!p.workspace) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0, BNV>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, (const uint16_t *)p.B,
+        hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0, BNV, false>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, (const uint16_t *)p.B,
                            p.workspace, nullptr, nullptr, 0, 0, (int)p.M, (int)p.N, (int)p.K, splits, 0);
         const int64_t MN = p.M * p.N;
         hipLaunchKernelGGL(gemm_splitk_fold_k, dim3((unsigned)((MN / 4 + 255) / 256)), block, 0, st, (const float *)p.workspace, p.C,
                            p.bias, p.residual, p.epilogue, p.bias_dtype, p.out_bf16, MN, (int)p.N, splits);
         return hipGetLastError();
     }
-#define ZK_GEMM(E)                                                                                                    \
-    hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E, BNV>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A,         \
+    if (p.plane) {
+        // only the product a convolution lowers to stores this way: A^T . B^T, epilogues none / bias / bias + ReLU
+        if (!(AT && BT) || p.epilogue > 2) return hipErrorInvalidValue;
+#define ZK_GEMM_PL(E)                                                                                                 \
+    hipLaunchKernelGGL((gemm_bf16_k<true, true, E, BNV, true>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, \
                        (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, p.plane);
+        switch (p.epilogue) {
+        case 0: ZK_GEMM_PL(0) break;
+        case 1: ZK_GEMM_PL(1) break;
+        default: ZK_GEMM_PL(2) break;
+        }
+#undef ZK_GEMM_PL
+        return hipGetLastError();
+    }
+#define ZK_GEMM(E)                                                                                                    \
+    hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E, BNV, false>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A,  \
+                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, 0);
     switch (p.epilogue) {
     case 0: ZK_GEMM(0) break;
     case 1: ZK_GEMM(1) break;
@@ -456,7 +470,11 @@ template <bool AT, bool BT> hipError_t launch_width(const GemmBf16 &p, hipStream
 }
 
 template <bool AT, bool BT, int E, int BNV> hipError_t allow_lds() {
-    return hipFuncSetAttribute((const void *)gemm_bf16_k<AT, BT, E, BNV>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
+    if (AT && BT && E <= 2) {
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_k<true, true, (E <= 2 ? E : 0), BNV, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
+        if (e != hipSuccess) return e;
+    }
+    return hipFuncSetAttribute((const void *)gemm_bf16_k<AT, BT, E, BNV, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
 }
 template <bool AT, bool BT> hipError_t allow_lds_epi() {
     hipError_t e;
