@@ -25,7 +25,7 @@ def test_layer_norm_reference_golden(hip):
                                rtol=2e-6)
 
 
-@pytest.mark.parametrize("shape", [(8192, 1024), (5, 7), (33, 1000), (4, 4096), (3, 5001), (1, 2)])
+@pytest.mark.parametrize("shape", [(8192, 1024), (5, 7), (33, 1000), (4, 4096), (3, 5001), (1, 2), (64, 256), (7, 512), (9, 2048)])
 @pytest.mark.parametrize("rms", [False, True])
 def test_norms_f32(hip, oracle, shape, rms):
     dev, pool = hip
@@ -77,7 +77,7 @@ def test_cross_entropy(hip, oracle):
 
 
 # ---- gradients of the norms ---------------------------------------------------------------------------------
-@pytest.mark.parametrize("shape", [(5, 9), (64, 128), (130, 1024), (3, 1000), (2100, 64)])
+@pytest.mark.parametrize("shape", [(5, 9), (64, 128), (130, 1024), (3, 1000), (2100, 64), (64, 256), (7, 512), (9, 2048)])
 @pytest.mark.parametrize("rms", [False, True])
 def test_norm_backward_f32(hip, oracle, shape, rms):
     from zyx_amd.kernels import norm_rows_bwd

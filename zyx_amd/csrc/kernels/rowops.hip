@@ -107,6 +107,134 @@ __global__ __launch_bounds__(256) void norm_rows_k(const typename RowIO<DT>::S *
     }
 }
 
+// Rows of 256*NV columns (NV = 1, 2, 4, 8, 16): the wave keeps its row in registers (4*NV values per lane,
+// vector j of a lane = columns (lane + 64*j)*4 .. +3, so every access of the wave covers consecutive bytes):
+// the row is read from memory once. Same arithmetic as norm_rows_k.
+template <int DT, int MODE, int NV>
+__global__ __launch_bounds__(256) void norm_rows_reg_k(const typename RowIO<DT>::S *__restrict__ x,
+                                                       const typename RowIO<DT>::S *__restrict__ w,
+                                                       const typename RowIO<DT>::S *__restrict__ b,
+                                                       typename RowIO<DT>::S *__restrict__ y, int64_t rows, float eps) {
+    typedef RowIO<DT> IO;
+    constexpr int cols = 256 * NV;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const typename IO::S *xr = x + row * cols;
+    typename IO::S *yr = y + row * cols;
+    float v[NV][4];
+#pragma unroll
+    for (int j = 0; j < NV; j++) IO::ld4(xr, (lane + 64 * j) * 4, v[j]);
+    float mean = 0.0f, scale;
+    if (MODE == 0) {
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++) s += (v[j][0] + v[j][1]) + (v[j][2] + v[j][3]);
+        mean = wave_allreduce_f32(s, OpAdd()) / (float)cols;
+        float q = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) q += (v[j][k] - mean) * (v[j][k] - mean);
+        scale = 1.0f / sqrtf(wave_allreduce_f32(q, OpAdd()) / (float)(cols - 1) + eps);
+    } else {
+        float q = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) q += v[j][k] * v[j][k];
+        scale = sqrtf(1.0f / (wave_allreduce_f32(q, OpAdd()) / (float)cols + eps));
+    }
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int c = (lane + 64 * j) * 4;
+        float wv[4] = {1.0f, 1.0f, 1.0f, 1.0f}, bv[4] = {0.0f, 0.0f, 0.0f, 0.0f}, o[4];
+        if (w) IO::ld4(w, c, wv);
+        if (b) IO::ld4(b, c, bv);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            o[k] = MODE == 0 ? (v[j][k] - mean) * scale : v[j][k] * scale;
+            if (w) o[k] *= wv[k];
+            if (b) o[k] += bv[k];
+        }
+        IO::st4(yr, c, o);
+    }
+}
+
+// dx for rows of 256*NV columns with x and dy held in registers (one read of each); otherwise as norm_bwd_dx_k.
+template <int DT, int MODE, int NV>
+__global__ __launch_bounds__(256) void norm_bwd_dx_reg_k(const typename RowIO<DT>::S *__restrict__ x,
+                                                         const typename RowIO<DT>::S *__restrict__ w,
+                                                         const typename RowIO<DT>::S *__restrict__ dy,
+                                                         const typename RowIO<DT>::S *__restrict__ add,
+                                                         typename RowIO<DT>::S *__restrict__ dx, float *__restrict__ stats,
+                                                         int64_t rows, float eps) {
+    typedef RowIO<DT> IO;
+    constexpr int cols = 256 * NV;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int64_t base = row * cols;
+    float xv[NV][4], g[NV][4];
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        IO::ld4(x + base, (lane + 64 * j) * 4, xv[j]);
+        IO::ld4(dy + base, (lane + 64 * j) * 4, g[j]);
+    }
+    float mean = 0.0f, rstd;
+    if (MODE == 0) {
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++) s += (xv[j][0] + xv[j][1]) + (xv[j][2] + xv[j][3]);
+        mean = wave_allreduce_f32(s, OpAdd()) / (float)cols;
+        float q = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) q += (xv[j][k] - mean) * (xv[j][k] - mean);
+        rstd = 1.0f / sqrtf(wave_allreduce_f32(q, OpAdd()) / (float)(cols - 1) + eps);
+    } else {
+        float q = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) q += xv[j][k] * xv[j][k];
+        rstd = sqrtf(1.0f / (wave_allreduce_f32(q, OpAdd()) / (float)cols + eps));
+    }
+    float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        if (w) {
+            float wv[4];
+            IO::ld4(w, (lane + 64 * j) * 4, wv);
+#pragma unroll
+            for (int k = 0; k < 4; k++) g[j][k] *= wv[k];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            s1 += g[j][k];
+            s2 += g[j][k] * (MODE == 0 ? (xv[j][k] - mean) * rstd : xv[j][k]);
+        }
+    }
+    s1 = wave_allreduce_f32(s1, OpAdd());
+    s2 = wave_allreduce_f32(s2, OpAdd());
+    const float k1 = s1 / (float)cols, k2 = MODE == 0 ? s2 / (float)(cols - 1) : rstd * rstd * rstd * s2 / (float)cols;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int c = (lane + 64 * j) * 4;
+        float av[4] = {0.0f, 0.0f, 0.0f, 0.0f}, o[4];
+        if (add) IO::ld4(add + base, c, av);
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            o[k] = (MODE == 0 ? rstd * ((g[j][k] - k1) - ((xv[j][k] - mean) * rstd) * k2) : rstd * g[j][k] - xv[j][k] * k2) + av[k];
+        IO::st4(dx + base, c, o);
+    }
+    if (lane == 0) {
+        stats[row * 2] = mean;
+        stats[row * 2 + 1] = rstd;
+    }
+}
+
 // Cross-entropy with class-index targets, one wave per sample. loss[r] = -(ln_softmax(x)[label])
 // computed as the reference does: m = x - max; ls = m - ln(sum exp(m)); loss = sum_c -ls[c] * onehot[c].
 // grad (optional) = (softmax(x) - onehot) * gscale, the gradient of gscale * sum_r loss[r].
@@ -290,7 +418,14 @@ template <int DT, int MODE> hipError_t launch_norm_bwd(const NormRowsBwd &p, hip
     const bool vec = p.cols % 4 == 0 && al(p.x) && al(p.dy) && al(p.dx) && al(p.add);
     float *stats = (float *)p.workspace, *part = stats + p.rows * 2;
     dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
-    if (vec) hipLaunchKernelGGL((norm_bwd_dx_k<DT, MODE, true>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, (int)p.cols, p.eps);
+#define ZK_BWD_REG(NV) hipLaunchKernelGGL((norm_bwd_dx_reg_k<DT, MODE, NV>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, p.eps)
+    const bool al16 = vec && (!p.w || reinterpret_cast<uintptr_t>(p.w) % (4 * esz) == 0);
+    if (al16 && p.cols == 256) ZK_BWD_REG(1);
+    else if (al16 && p.cols == 512) ZK_BWD_REG(2);
+    else if (al16 && p.cols == 1024) ZK_BWD_REG(4);
+    else if (al16 && p.cols == 2048) ZK_BWD_REG(8);
+#undef ZK_BWD_REG
+    else if (vec) hipLaunchKernelGGL((norm_bwd_dx_k<DT, MODE, true>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, (int)p.cols, p.eps);
     else hipLaunchKernelGGL((norm_bwd_dx_k<DT, MODE, false>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, (int)p.cols, p.eps);
     if (p.dw || p.db) {
         const int chunks = norm_bwd_chunks(p.rows);
@@ -307,7 +442,16 @@ template <int DT, int MODE> hipError_t launch_norm(const NormRows &p, hipStream_
     dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
     const int esz = (int)sizeof(S);
     bool vec = p.cols % 4 == 0 && reinterpret_cast<uintptr_t>(p.x) % (4 * esz) == 0 && reinterpret_cast<uintptr_t>(p.y) % (4 * esz) == 0;
-    if (vec) hipLaunchKernelGGL((norm_rows_k<DT, MODE, true>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.b, (S *)p.y, p.rows, (int)p.cols, p.eps);
+#define ZK_FWD_REG(NV) hipLaunchKernelGGL((norm_rows_reg_k<DT, MODE, NV>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.b, (S *)p.y, p.rows, p.eps)
+    auto al = [&](const void *q) { return reinterpret_cast<uintptr_t>(q) % (4 * esz) == 0; };
+    const bool al16 = vec && al(p.w) && al(p.b);
+    if (al16 && p.cols == 256) ZK_FWD_REG(1);
+    else if (al16 && p.cols == 512) ZK_FWD_REG(2);
+    else if (al16 && p.cols == 1024) ZK_FWD_REG(4);
+    else if (al16 && p.cols == 2048) ZK_FWD_REG(8);
+    else if (al16 && p.cols == 4096) ZK_FWD_REG(16);
+#undef ZK_FWD_REG
+    else if (vec) hipLaunchKernelGGL((norm_rows_k<DT, MODE, true>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.b, (S *)p.y, p.rows, (int)p.cols, p.eps);
     else hipLaunchKernelGGL((norm_rows_k<DT, MODE, false>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.b, (S *)p.y, p.rows, (int)p.cols, p.eps);
     return hipGetLastError();
 }
