@@ -5,7 +5,7 @@
 // tensors the reference materialises (q.dot(k.t()), softmax, dropout) never leave registers.
 //
 // attn_fwd_bf16_k (bf16, dh = 64, T % 128 == 0): one workgroup per (batch, head, 128 queries), 4 waves
-// of 32 queries. K and V tiles of 64 keys go L2 -> VGPR -> LDS, double buffered. Per tile a wave
+// of 32 queries. K and V tiles of 64 keys are loaded straight into LDS (global_load_lds), double buffered. Per tile a wave
 // computes S^T = K.Q^T (keys x queries) with v_mfma_f32_32x32x16_bf16, so that every lane owns one
 // query column: the running max / sum are per-lane scalars, and the exponentiated tile, packed to
 // bf16, already has the register layout of the B operand of O^T += V^T.P^T. V^T fragments come from
@@ -75,30 +75,27 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) qf[ks] = *(const bf16x8 *)(qp + (int64_t)tq * ld + ks * 16 + hh * 8);
 
-    // staging: thread moves chunks tid and tid + 256 of the 512 16-byte chunks of each tile
-    u32x4 rk[2], rv[2];
-    int sk[2], sv[2];
-    uint32_t go[2];
+    // staging: direct global -> LDS loads (a wave-load lays 64 x 16 bytes down contiguously: 8 tile rows). The
+    // swizzle is applied on the source side: lane l fetches the chunk that belongs at row l/8, physical slot l%8.
+    // Wave w issues loads i = 0, 1 of each tile: rows i*32 + w*8 .. +7. No staging registers, no ds_write.
+    uint32_t gk[2], gv[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        const int ch = tid + 256 * i, key = ch >> 3, cc = ch & 7;
-        go[i] = (uint32_t)(key * ld + cc * 8) * 2;
-        sk[i] = k_slot(key, cc);
-        sv[i] = TILE + v_slot(key, cc);
+        const int key = i * 32 + wave * 8 + (lane >> 3), slot = lane & 7;
+        const int ck = slot ^ ((key >> 1) & 7);                                   // inverse of k_slot
+        const int cv = ((((slot >> 2) ^ ((key >> 1) & 1)) << 2) | (slot & 3));   // inverse of v_slot
+        gk[i] = (uint32_t)(key * ld + ck * 8) * 2;
+        gv[i] = (uint32_t)(key * ld + cv * 8) * 2;
     }
-    auto gload = [&](int kt) {
+    auto stage_tile = [&](int kt, int stage) {
         const int64_t base = (int64_t)kt * KB * ld * 2;
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            rk[i] = *(const u32x4 *)((const uint8_t *)kp + base + go[i]);
-            rv[i] = *(const u32x4 *)((const uint8_t *)vp + base + go[i]);
-        }
-    };
-    auto lwrite = [&](int stage) {
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            *(ZK_LDS u32x4 *)(smem + stage + sk[i]) = rk[i];
-            *(ZK_LDS u32x4 *)(smem + stage + sv[i]) = rv[i];
+            const int rows = (i * 32 + wave * 8) * 128;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)((const uint8_t *)kp + base + gk[i]),
+                                             (ZK_LDS void *)(smem + stage + rows), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)((const uint8_t *)vp + base + gv[i]),
+                                             (ZK_LDS void *)(smem + stage + TILE + rows), 16, 0, 0);
         }
     };
 
@@ -121,12 +118,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
     float m = -INFINITY, l = 0.0f;
 
     const int NT = T / KB;
-    gload(0);
-    lwrite(0);
+    stage_tile(0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): this wave's part of tile 0 has landed in LDS
     __syncthreads();
     int stage = 0;
     for (int kt = 0; kt < NT; kt++) {
-        if (kt + 1 < NT) gload(kt + 1);
+        if (kt + 1 < NT) stage_tile(kt + 1, stage ^ STAGE); // the other stage was last read before the previous barrier
 
         f32x16 s[2];
 #pragma unroll
@@ -149,10 +146,17 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
         const float m_new = fmaxf(m, bm * c);
         const float alpha = __builtin_amdgcn_exp2f(m - m_new);
         m = m_new;
-        float ps = 0.0f;
-        bf16x8 pf[2][2];
+        // the accumulator needs rescaling only when some query's running maximum moved: rare after the first tiles
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+            for (int db = 0; db < 2; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+        }
+        float ps = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) { // exponentiate one 32-key block, feed it to the matrix pipe, then the next
+            bf16x8 pf[2];
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++) {
                 f32x8 p;
@@ -161,16 +165,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
                     p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][8 * s2 + e], c, -m_new));
                     ps += p[e];
                 }
-                pf[kb][s2] = __builtin_convertvector(p, bf16x8);
+                pf[s2] = __builtin_convertvector(p, bf16x8);
             }
-        l = __builtin_fmaf(l, alpha, ps);
-#pragma unroll
-        for (int db = 0; db < 2; db++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) o[db][r] *= alpha;
-
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++)
 #pragma unroll
@@ -179,10 +175,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
                     const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(smem + off));
                     const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(smem + off + 8 * 128));
                     const bf16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[kb][s2], o[db], 0, 0, 0);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[s2], o[db], 0, 0, 0);
                 }
+        }
+        l = __builtin_fmaf(l, alpha, ps);
 
-        if (kt + 1 < NT) lwrite(stage ^ STAGE);
+        __builtin_amdgcn_s_waitcnt(0x0f70); // this wave's loads of tile kt+1 have landed
         __syncthreads();
         stage ^= STAGE;
     }
