@@ -304,6 +304,7 @@ def main():
                     help="run only the config-3 GEMM leg and print its numbers (used for profiling that kernel)")
     ap.add_argument("--conv-only", action="store_true", help="run only the config-4 conv + max-pool leg")
     ap.add_argument("--block-only", action="store_true", help="run only the config-5 transformer block leg")
+    ap.add_argument("--mlp-only", action="store_true", help="run only the config-1 MLP training leg")
     ap.add_argument("--streaming-only", action="store_true", help="run only the memory-bound kernel leg")
     ap.add_argument("--attention-only", action="store_true", help="run only the attention core leg")
     ap.add_argument("--counters", action="store_true",
@@ -327,8 +328,10 @@ def main():
         pool.deinitialize()
         return
 
-    if args.conv_only or args.block_only or args.streaming_only or args.attention_only:
-        if args.conv_only:
+    if args.conv_only or args.block_only or args.streaming_only or args.attention_only or args.mlp_only:
+        if args.mlp_only:
+            res = {"config1_mlp_train": extra_mlp(dev, pool, cpu=not args.no_cpu)}
+        elif args.conv_only:
             res = {"config4_conv_relu_pool": extra_conv(dev, pool, kernels)}
         elif args.streaming_only:
             res = {"memory_bound_kernels": extra_streaming(dev, pool, kernels)}

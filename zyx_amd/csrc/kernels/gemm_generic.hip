@@ -13,6 +13,8 @@
 // 32. Operands are read with bounds checks (zero fill) straight from their natural layout,
 // coalesced along whichever index is contiguous, and laid down K-contiguous in LDS with an
 // 8-element row pad, so fragment reads are the same for all four layouts.
+#include <algorithm>
+
 #include "dtypes.hpp"
 #include "kernels.hpp"
 #include "wave.hpp"
@@ -79,7 +81,11 @@ __global__ __launch_bounds__(256) void gemm_generic_k(const GemmGeneric p) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int64_t m0 = (int64_t)blockIdx.y * GM, n0 = (int64_t)blockIdx.x * GN;
-    const S *A = (const S *)p.A + (int64_t)blockIdx.z * p.batch_a, *B = (const S *)p.B + (int64_t)blockIdx.z * p.batch_b;
+    // split-K: blockIdx.z = batch * splits + split; a split multiplies K range [k_lo, k_hi) and stores its raw
+    // f32 partial tile into slice (batch, split) of the workspace, which gemm_generic_fold_k sums
+    const int split = p.splits > 1 ? blockIdx.z % p.splits : 0, bz = p.splits > 1 ? blockIdx.z / p.splits : blockIdx.z;
+    const int64_t k_lo = (int64_t)split * p.k_len, k_hi = p.splits > 1 ? (k_lo + p.k_len < p.K ? k_lo + p.k_len : p.K) : p.K;
+    const S *A = (const S *)p.A + (int64_t)bz * p.batch_a, *B = (const S *)p.B + (int64_t)bz * p.batch_b;
     const int64_t a_rs = p.trans_a ? 1 : p.K, a_ks = p.trans_a ? p.M : 1;
     const int64_t b_rs = p.trans_b ? p.K : 1, b_ks = p.trans_b ? 1 : p.N;
 
@@ -87,10 +93,10 @@ __global__ __launch_bounds__(256) void gemm_generic_k(const GemmGeneric p) {
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.0f;
 
-    for (int64_t k0 = 0; k0 < p.K; k0 += GK) {
+    for (int64_t k0 = k_lo; k0 < k_hi; k0 += GK) {
         __syncthreads(); // previous step's fragment reads are done
-        fill_tile<S>(As, A, a_rs, a_ks, m0, k0, p.M, p.K, GT<DT>::zero());
-        fill_tile<S>(Bs, B, b_rs, b_ks, n0, k0, p.N, p.K, GT<DT>::zero());
+        fill_tile<S>(As, A, a_rs, a_ks, m0, k0, p.M, k_hi, GT<DT>::zero());
+        fill_tile<S>(Bs, B, b_rs, b_ks, n0, k0, p.N, k_hi, GT<DT>::zero());
         __syncthreads();
         const S *ar = As + (wm * 32 + (lane & 31)) * (GK + GPAD);
         const S *br = Bs + (wn * 32 + (lane & 31)) * (GK + GPAD);
@@ -118,6 +124,15 @@ __global__ __launch_bounds__(256) void gemm_generic_k(const GemmGeneric p) {
     // register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32 x 32 tile
     const int64_t col = n0 + wn * 32 + (lane & 31);
     if (col >= p.N) return; // no barrier follows
+    if (p.splits > 1) {
+        float *W = (float *)p.workspace + ((int64_t)bz * p.splits + split) * p.M * p.N;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int64_t row = m0 + wm * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            if (row < p.M) W[row * p.N + col] = acc[r];
+        }
+        return;
+    }
     float bv = 0.0f;
     if (p.epilogue >= 1) {
         if (p.bias_dtype == DT_BF16) bv = bf16_to_f32(((const uint16_t *)p.bias)[col]);
@@ -146,12 +161,59 @@ __global__ __launch_bounds__(256) void gemm_generic_k(const GemmGeneric p) {
     }
 }
 
+// Sums the split-K partials [batch, splits, M, N] and applies alpha, bias, activation, residual and the store dtype.
+template <int ODT> __global__ __launch_bounds__(256) void gemm_generic_fold_k(const GemmGeneric p) {
+    const int64_t MN = p.M * p.N, i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= MN * p.batch) return;
+    const int64_t bz = i / MN, o = i - bz * MN, col = o % p.N;
+    const float *W = (const float *)p.workspace + bz * p.splits * MN + o;
+    float a = W[0];
+    for (int z = 1; z < p.splits; z++) a += W[(int64_t)z * MN];
+    float v = a * p.alpha;
+    if (p.epilogue >= 1) {
+        if (p.bias_dtype == DT_BF16) v += bf16_to_f32(((const uint16_t *)p.bias)[col]);
+        else if (p.bias_dtype == DT_F16) v += f16_to_f32(((const uint16_t *)p.bias)[col]);
+        else v += ((const float *)p.bias)[col];
+    }
+    if (p.epilogue == 2) v = (v > 0.0f ? 1.0f : 0.0f) * v;
+    if (p.epilogue == 3) v = gelu_ref(v);
+    const int64_t oo = bz * p.batch_c + o;
+    if (p.residual) {
+        if (ODT == DT_F32) v += ((const float *)p.residual)[oo];
+        else if (ODT == DT_BF16) v += bf16_to_f32(((const uint16_t *)p.residual)[oo]);
+        else v += f16_to_f32(((const uint16_t *)p.residual)[oo]);
+    }
+    if (ODT == DT_F32) ((float *)p.C)[oo] = v;
+    else if (ODT == DT_BF16) ((uint16_t *)p.C)[oo] = f32_to_bf16_trunc(v);
+    else ((uint16_t *)p.C)[oo] = f32_to_f16_trunc(v);
+}
+
 } // namespace
 
-hipError_t gemm_generic(const GemmGeneric &p, hipStream_t st) {
+// Few output tiles and a long K (the weight-gradient and first-layer products of a small MLP): split K over
+// workgroups so the chip has work; each split keeps at least two 32-wide k steps.
+int gemm_generic_splits(int64_t M, int64_t N, int64_t K, int64_t batch, int64_t *k_len) {
+    const int64_t tiles = ((M + GM - 1) / GM) * ((N + GN - 1) / GN) * batch;
+    int64_t s = 1;
+    if (tiles < 128 && K >= 4 * GK) s = std::min<int64_t>(std::min<int64_t>(K / (2 * GK), 256 / tiles), 64);
+    if (s < 1) s = 1;
+    int64_t len = ((K + s - 1) / s + GK - 1) / GK * GK;
+    s = (K + len - 1) / len;
+    if (k_len) *k_len = len;
+    return (int)s;
+}
+uint64_t gemm_generic_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t batch) {
+    const int s = gemm_generic_splits(M, N, K, batch, nullptr);
+    return s > 1 ? (uint64_t)s * batch * M * N * 4 : 0;
+}
+
+hipError_t gemm_generic(const GemmGeneric &p0, hipStream_t st) {
+    GemmGeneric p = p0;
     if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return hipSuccess;
     if (p.K < 0 || (p.M + GM - 1) / GM > 65535 || p.batch > 65535) return hipErrorInvalidValue;
-    dim3 grid((unsigned)((p.N + GN - 1) / GN), (unsigned)((p.M + GM - 1) / GM), (unsigned)p.batch), block(256);
+    p.splits = gemm_generic_splits(p.M, p.N, p.K, p.batch, &p.k_len);
+    if (p.splits > 1 && (!p.workspace || (int64_t)p.batch * p.splits > 65535)) return hipErrorInvalidValue;
+    dim3 grid((unsigned)((p.N + GN - 1) / GN), (unsigned)((p.M + GM - 1) / GM), (unsigned)(p.batch * p.splits)), block(256);
 #define ZK_G(D, O) hipLaunchKernelGGL((gemm_generic_k<D, O>), grid, block, 0, st, p)
     if (p.dtype == DT_F32 && p.out_dtype == DT_F32) ZK_G(DT_F32, DT_F32);
     else if (p.dtype == DT_BF16 && p.out_dtype == DT_F32) ZK_G(DT_BF16, DT_F32);
@@ -160,6 +222,12 @@ hipError_t gemm_generic(const GemmGeneric &p, hipStream_t st) {
     else if (p.dtype == DT_F16 && p.out_dtype == DT_F16) ZK_G(DT_F16, DT_F16);
     else return hipErrorInvalidValue;
 #undef ZK_G
+    if (p.splits > 1) {
+        dim3 fg((unsigned)((p.M * p.N * p.batch + 255) / 256));
+        if (p.out_dtype == DT_F32) hipLaunchKernelGGL((gemm_generic_fold_k<DT_F32>), fg, block, 0, st, p);
+        else if (p.out_dtype == DT_BF16) hipLaunchKernelGGL((gemm_generic_fold_k<DT_BF16>), fg, block, 0, st, p);
+        else hipLaunchKernelGGL((gemm_generic_fold_k<DT_F16>), fg, block, 0, st, p);
+    }
     return hipGetLastError();
 }
 

@@ -86,7 +86,11 @@ struct GemmGeneric {
     float alpha;
     const void *A, *B, *bias, *residual; // residual (dtype out_dtype, [batch, M, N]) may be null
     void *C;
+    void *workspace;      // gemm_generic_workspace_bytes(M, N, K, batch) bytes, may be null when that is 0
+    int splits;           // set by the launcher
+    int64_t k_len;        // set by the launcher
 };
+uint64_t gemm_generic_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t batch);
 hipError_t gemm_generic(const GemmGeneric &p, hipStream_t stream);
 
 // LayerNorm (rms == 0) / RMSNorm (rms == 1) over the last axis; w, b may be null.

@@ -406,7 +406,7 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.n_in = a;
         p.need[a] = (uint64_t)batch * M * N * dtype_bytes(d.out_dtype);
         p.n_out = 1;
-        if (gemm_takes_fast_path(d)) p.workspace_bytes = zk::gemm_bf16_workspace_bytes(M, N, K);
+        p.workspace_bytes = gemm_takes_fast_path(d) ? zk::gemm_bf16_workspace_bytes(M, N, K) : zk::gemm_generic_workspace_bytes(M, N, K, batch);
         return ZHIP_OK;
     }
     case ZHIP_K_NORM_ROWS: {
@@ -664,6 +664,7 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         g.B = ptr[1];
         g.bias = g.epilogue ? ptr[2] : nullptr;
         g.residual = residual;
+        g.workspace = p.workspace;
         g.C = ptr[p.n_in];
         return zk::gemm_generic(g, st);
     }
