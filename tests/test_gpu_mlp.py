@@ -38,10 +38,12 @@ def test_single_step_gradients_and_update(hip, oracle):
     m.close()
 
 
-def test_100_steps_loss_curve(hip, oracle):
+@pytest.mark.parametrize("fused_update", [False, True])
+def test_100_steps_loss_curve(hip, oracle, fused_update):
+    """fused_update: w - lr * dW is formed in the weight-gradient GEMM's epilogue instead of a separate launch."""
     dev, pool = hip
     r, w1, b1, w2, b2 = init(oracle)
-    m = MLPTrainStep(dev, pool, B, NIN, H, NOUT, LR)
+    m = MLPTrainStep(dev, pool, B, NIN, H, NOUT, LR, fused_update=fused_update)
     m.set_params(w1, b1, w2, b2)
     gpu_losses, cpu_losses = [], []
     for step in range(100):

@@ -191,13 +191,13 @@ template <int ODT> __global__ __launch_bounds__(256) void gemm_generic_fold_k(co
 } // namespace
 
 // Few output tiles and a long K (the weight-gradient and first-layer products of a small MLP): split K over
-// workgroups so the chip has work; each split keeps at least two 32-wide k steps.
+// workgroups so the chip has work and every workgroup waits for few round trips to memory.
 int gemm_generic_splits(int64_t M, int64_t N, int64_t K, int64_t batch, int64_t *k_len) {
-    const int64_t tiles = ((M + GM - 1) / GM) * ((N + GN - 1) / GN) * batch;
+    const int64_t tiles = ((M + GM - 1) / GM) * ((N + GN - 1) / GN) * batch, steps = (K + GK - 1) / GK;
     int64_t s = 1;
-    if (tiles < 128 && K >= 4 * GK) s = std::min<int64_t>(std::min<int64_t>(K / (2 * GK), 256 / tiles), 64);
+    if (tiles < 128 && steps >= 2) s = std::min<int64_t>(std::min<int64_t>(steps, 256 / tiles), 64);
     if (s < 1) s = 1;
-    int64_t len = ((K + s - 1) / s + GK - 1) / GK * GK;
+    const int64_t len = (steps + s - 1) / s * GK;
     s = (K + len - 1) / len;
     if (k_len) *k_len = len;
     return (int)s;

@@ -26,7 +26,10 @@ from .backend import DType, HIPDevice, HIPMemoryPool
 
 
 class MLPTrainStep:
-    def __init__(self, dev: HIPDevice, pool: HIPMemoryPool, batch: int, n_in: int, hidden: int, n_out: int, lr: float):
+    def __init__(self, dev: HIPDevice, pool: HIPMemoryPool, batch: int, n_in: int, hidden: int, n_out: int, lr: float,
+                 fused_update: bool = False):
+        """fused_update: the weight-gradient GEMMs write `w - lr * dW` directly (alpha = -lr, the old weight as the
+        fused residual operand), so dW1 / dW2 are never materialised and two update launches disappear."""
         self.dev, self.pool = dev, pool
         self.shape = (batch, n_in, hidden, n_out)
         f32 = DType.F32
@@ -63,21 +66,26 @@ class MLPTrainStep:
             c.load(ig).mul(c.const(lr)).rsub(ip)
             return prog(c.desc())
 
+        if fused_update:
+            dw2_node = (prog(K.gemm_desc(n_out, hidden, batch, f32, f32, trans_a=True, alpha=-lr, residual=True)), [dlogits, h, w2, nw2])
+            dw1_node = (prog(K.gemm_desc(hidden, n_in, batch, f32, f32, trans_a=True, alpha=-lr, residual=True)), [dpre, x, w1, nw1])
+        else:
+            dw2_node = (prog(K.gemm_desc(n_out, hidden, batch, f32, f32, trans_a=True)), [dlogits, h, dw2])
+            dw1_node = (prog(K.gemm_desc(hidden, n_in, batch, f32, f32, trans_a=True)), [dpre, x, dw1])
         nodes = [
             (prog(K.gemm_desc(batch, hidden, n_in, f32, f32, trans_b=True, epilogue="bias_relu")), [x, w1, b1, h]),
             (prog(K.gemm_desc(batch, n_out, hidden, f32, f32, trans_b=True, epilogue="bias")), [h, w2, b2, logits]),
             (prog(K.cross_entropy_desc(batch, n_out, True, True, 1.0 / batch)), [logits, y, loss, dlogits]),
             (prog(K.reduce_desc(1, batch, "sum")), [loss, loss_sum]),
             (prog(scale.desc()), [loss_sum, mean_loss]),
-            (prog(K.gemm_desc(n_out, hidden, batch, f32, f32, trans_a=True)), [dlogits, h, dw2]),
+            dw2_node,
             (prog(K.reduce_desc(batch, n_out, "sum", axis0=True)), [dlogits, db2]),
             (prog(K.gemm_desc(batch, hidden, n_out, f32, f32)), [dlogits, w2, dh]),
             (prog(relu_bwd.desc()), [h, dh, dpre]),
-            (prog(K.gemm_desc(hidden, n_in, batch, f32, f32, trans_a=True)), [dpre, x, dw1]),
+            dw1_node,
             (prog(K.reduce_desc(batch, hidden, "sum", axis0=True)), [dpre, db1]),
-            (sgd(hidden, n_in), [w1, dw1, nw1]),
+        ] + ([] if fused_update else [(sgd(hidden, n_in), [w1, dw1, nw1]), (sgd(n_out, hidden), [w2, dw2, nw2])]) + [
             (sgd(1, hidden), [b1, db1, nb1]),
-            (sgd(n_out, hidden), [w2, dw2, nw2]),
             (sgd(1, n_out), [b2, db2, nb2]),
         ]
         # the updated parameters are written to fresh buffers (a kernel's outputs never alias its
