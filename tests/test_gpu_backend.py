@@ -123,3 +123,51 @@ def test_timer_and_profile(hip, oracle):
     for b in [xb] + outs:
         pool.deallocate(b, [])
     dev.release(prog)
+
+
+def test_plan_keeps_its_programs_alive(hip, oracle):
+    """A plan's graph holds its programs' kernels and scratch: releasing one while the plan lives is refused."""
+    from zyx_amd import BackendError, ErrorStatus
+    from zyx_amd.kernels import reduce_desc, to_device, alloc_like, to_host
+    dev, pool = hip
+    x = oracle.Rng(8).randn((4096, 512))
+    prog = dev.register_kernel(reduce_desc(4096, 512, "sum", axis0=True))  # two-stage: owns a workspace
+    xb, e0 = to_device(pool, x)
+    ob, e1 = alloc_like(pool, 512, 4)
+    pool.sync_events([e0, e1])
+    plan = dev.create_plan([(prog, [xb, ob])])
+    with pytest.raises(BackendError) as ei:
+        dev.release(prog)
+    assert ei.value.status == ErrorStatus.IncorrectKernelArg and "live plan" in ei.value.context
+    done = dev.launch_plan(plan, [])
+    got = to_host(pool, ob, (512,), np.float32, [done])
+    assert np.allclose(got, x.astype(np.float64).sum(0), rtol=1e-5, atol=1e-4)
+    dev.destroy_plan(plan)
+    dev.release(prog)
+    for b in (xb, ob):
+        pool.deallocate(b, [])
+
+
+def test_launches_of_one_program_do_not_overlap_on_its_workspace(hip, oracle):
+    """Independent wait lists send launches to different streams; a program with scratch memory (two-stage
+    column sum here) must still run them one after the other. Many rounds, every result checked."""
+    from zyx_amd.kernels import reduce_desc, to_device, alloc_like, to_host
+    dev, pool = hip
+    r = oracle.Rng(9)
+    xs = [r.randn((8192, 256)) for _ in range(4)]
+    want = [x.astype(np.float64).sum(0) for x in xs]
+    prog = dev.register_kernel(reduce_desc(8192, 256, "sum", axis0=True))
+    bufs = []
+    for x in xs:
+        xb, e = to_device(pool, x)
+        ob, e2 = alloc_like(pool, 256, 4)
+        pool.sync_events([e, e2])
+        bufs.append((xb, ob))
+    for _ in range(20):
+        evs = [dev.launch(prog, pool, [xb, ob], []) for xb, ob in bufs]  # empty wait lists: round-robin streams
+        for (xb, ob), ev, w in zip(bufs, evs, want):
+            assert np.allclose(to_host(pool, ob, (256,), np.float32, [ev]), w, rtol=1e-5, atol=2e-4)
+    dev.release(prog)
+    for xb, ob in bufs:
+        pool.deallocate(xb, [])
+        pool.deallocate(ob, [])

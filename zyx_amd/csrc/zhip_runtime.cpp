@@ -20,6 +20,7 @@
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -70,6 +71,10 @@ struct Program {
     void *workspace = nullptr; // device scratch owned by the program (two-stage reductions)
     uint64_t workspace_bytes = 0;
     zk::EwJit *jit = nullptr;  // elementwise chains above the size threshold: code specialised at registration
+    // A program's workspace is shared by all its launches: each launch waits for the previous one's event on
+    // whatever stream that ran, so two launches with unrelated wait lists never overlap on the scratch memory.
+    hipEvent_t ws_event = nullptr;
+    int plan_refs = 0;         // live plans whose graphs hold this program's kernels, workspace and code
 };
 
 struct Plan {
@@ -77,6 +82,7 @@ struct Plan {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     size_t n_nodes = 0;
+    std::vector<zhip_prog> progs; // distinct programs of the plan
 };
 
 template <class T> struct Slab { // dense ids, lowest free id reused (zyx/src/slab.rs)
@@ -935,6 +941,7 @@ ZHIP_EXPORT int32_t zhip_deinit(zhip_ctx *c) {
         for (Program &p : c->programs.items) {
             if (p.live && p.workspace) (void)hipFree(p.workspace);
             if (p.live && p.jit) zk::ew_jit_destroy(p.jit);
+            if (p.live && p.ws_event) (void)hipEventDestroy(p.ws_event);
         }
         for (EventSlot &s : c->events) (void)hipEventDestroy(s.ev);
         (void)hipEventDestroy(c->prof_a);
@@ -1160,6 +1167,10 @@ ZHIP_EXPORT int32_t zhip_register_kernel(zhip_ctx *c, const zhip_kernel_desc *de
             (void)hipFree(p.workspace);
             return rc;
         }
+        if (hipEventCreateWithFlags(&p.ws_event, hipEventDisableTiming) != hipSuccess) {
+            (void)hipFree(p.workspace);
+            return c->fail(ZHIP_KERNEL_COMPILATION, "register_kernel: cannot create the workspace event");
+        }
     }
     // Large chains get code generated for exactly this program (zyx compiles every fused kernel at run time,
     // zyx/src/backend/mod.rs:899-933); small ones run on the interpreting kernel, where the ~0.3 s compile
@@ -1192,6 +1203,11 @@ ZHIP_EXPORT int32_t zhip_release_program(zhip_ctx *c, zhip_prog prog) {
     if (prog >= c->programs.items.size() || !c->programs.items[prog].live)
         return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "program %u does not exist", prog);
     Program &p = c->programs.items[prog];
+    if (p.plan_refs > 0) return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "program %u is part of %d live plan(s): destroy them first", prog, p.plan_refs);
+    if (p.ws_event) {
+        (void)hipEventDestroy(p.ws_event);
+        p.ws_event = nullptr;
+    }
     if (p.workspace) { // hipFree waits for the device, so no launch still uses it
         (void)hipSetDevice(c->device);
         (void)hipFree(p.workspace);
@@ -1227,8 +1243,10 @@ ZHIP_EXPORT int32_t zhip_launch(zhip_ctx *c, zhip_prog prog, const zhip_buf *arg
     rc = wait_and_consume(c, si, evs, n_evs, ZHIP_KERNEL_LAUNCH);
     if (rc != ZHIP_OK) return rc;
     if (c->debug & 32) fprintf(stderr, "[zyx-hip] launch program %u (kind %d) on stream %d\n", prog, p->desc.kind, si);
+    if (p->ws_event) HIPCHK(c, hipStreamWaitEvent(c->launch_streams[si], p->ws_event, 0), ZHIP_KERNEL_LAUNCH);
     hipError_t e = program_enqueue(*p, ptr, c->launch_streams[si]);
     if (e != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "launch of program %u failed: %s", prog, hipGetErrorString(e));
+    if (p->ws_event) HIPCHK(c, hipEventRecord(p->ws_event, c->launch_streams[si]), ZHIP_KERNEL_LAUNCH);
     return event_record(c, si, ZHIP_KERNEL_LAUNCH, ev);
 }
 
@@ -1241,6 +1259,7 @@ ZHIP_EXPORT int32_t zhip_time_kernel(zhip_ctx *c, zhip_prog prog, const zhip_buf
     if (rc != ZHIP_OK) return rc;
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
     hipStream_t st = c->launch_streams[0];
+    if (p->ws_event) HIPCHK(c, hipEventSynchronize(p->ws_event), ZHIP_KERNEL_SYNC);
     HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
     auto t0 = std::chrono::steady_clock::now();
     hipError_t e = program_enqueue(*p, ptr, st);
@@ -1263,6 +1282,7 @@ ZHIP_EXPORT int32_t zhip_profile_kernel(zhip_ctx *c, zhip_prog prog, const zhip_
     }
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
     hipStream_t st = c->launch_streams[0];
+    if (p->ws_event) HIPCHK(c, hipEventSynchronize(p->ws_event), ZHIP_KERNEL_SYNC);
     HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
     HIPCHK(c, hipEventRecord(c->prof_a, st), ZHIP_KERNEL_LAUNCH);
     for (int32_t i = 0; i < iters; i++) {
@@ -1310,6 +1330,9 @@ ZHIP_EXPORT int32_t zhip_plan_create(zhip_ctx *c, const zhip_prog *progs, const 
     }
     pl.live = true;
     pl.n_nodes = n_nodes;
+    for (size_t i = 0; i < n_nodes; i++)
+        if (std::find(pl.progs.begin(), pl.progs.end(), progs[i]) == pl.progs.end()) pl.progs.push_back(progs[i]);
+    for (zhip_prog q : pl.progs) c->programs.items[q].plan_refs++;
     *plan = c->plans.push(pl);
     return ZHIP_OK;
 }
@@ -1326,7 +1349,12 @@ ZHIP_EXPORT int32_t zhip_plan_launch(zhip_ctx *c, zhip_plan plan, const zhip_eve
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
     int32_t rc = wait_and_consume(c, -2, evs, n_evs, ZHIP_KERNEL_LAUNCH);
     if (rc != ZHIP_OK) return rc;
-    HIPCHK(c, hipGraphLaunch(c->plans.items[plan].exec, c->plan_stream), ZHIP_KERNEL_LAUNCH);
+    Plan &pl = c->plans.items[plan];
+    for (zhip_prog q : pl.progs)
+        if (hipEvent_t we = c->programs.items[q].ws_event) HIPCHK(c, hipStreamWaitEvent(c->plan_stream, we, 0), ZHIP_KERNEL_LAUNCH);
+    HIPCHK(c, hipGraphLaunch(pl.exec, c->plan_stream), ZHIP_KERNEL_LAUNCH);
+    for (zhip_prog q : pl.progs)
+        if (hipEvent_t we = c->programs.items[q].ws_event) HIPCHK(c, hipEventRecord(we, c->plan_stream), ZHIP_KERNEL_LAUNCH);
     return event_record(c, -2, ZHIP_KERNEL_LAUNCH, ev);
 }
 
@@ -1338,6 +1366,8 @@ ZHIP_EXPORT int32_t zhip_plan_destroy(zhip_ctx *c, zhip_plan plan) {
     (void)hipStreamSynchronize(c->plan_stream);
     (void)hipGraphExecDestroy(pl.exec);
     (void)hipGraphDestroy(pl.graph);
+    for (zhip_prog q : pl.progs)
+        if (q < c->programs.items.size() && c->programs.items[q].plan_refs > 0) c->programs.items[q].plan_refs--;
     pl = Plan();
     c->plans.remove(plan);
     return ZHIP_OK;
