@@ -328,7 +328,9 @@ int32_t zhip_compile_ir(zhip_ctx *ctx, const void *ir, uint64_t ir_bytes, zhip_p
  * checked against the size the program needs before anything is enqueued. Consumes evs. */
 int32_t zhip_launch(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args, size_t n_args, const zhip_event *evs,
                     size_t n_evs, zhip_event *ev);
-/* HIPDevice::release (hip.rs:721-724) */
+/* HIPDevice::release (hip.rs:721-724). Refused (ZHIP_INCORRECT_KERNEL_ARG) while a live plan contains the
+ * program. Launches of one program that owns scratch memory are ordered among themselves even when their wait
+ * lists are unrelated. */
 int32_t zhip_release_program(zhip_ctx *ctx, zhip_prog prog);
 /* launch_with_timings (zyx/src/kernel/autotune.rs:775-798): launch, sync, host
  * wall-clock nanoseconds -- the value for Node::Kernel.time (graph/mod.rs:177-182). */
@@ -349,7 +351,7 @@ int32_t zhip_profile_kernel(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args,
  * lists back to back and n_args their lengths -- as a HIP graph on one in-order stream, so a
  * later node sees the results of every earlier one. zhip_plan_launch replays it with one
  * call: it waits for (and consumes) evs, and returns the event of the whole list. Buffers
- * and programs named by a plan must stay alive until zhip_plan_destroy. */
+ * named by a plan must stay alive until zhip_plan_destroy; its programs cannot be released before. */
 typedef uint32_t zhip_plan;
 int32_t zhip_plan_create(zhip_ctx *ctx, const zhip_prog *progs, const zhip_buf *args_flat, const uint32_t *n_args,
                          size_t n_nodes, zhip_plan *plan);
