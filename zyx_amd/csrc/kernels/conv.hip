@@ -11,7 +11,7 @@
 // GEMM view: C'[co, p] = W[co, k] . X'[k, p], k = (c, ky, kx), p = (n, oy, ox). The weight is
 // the K-contiguous operand as stored; X' is gathered on the fly (im2col never exists in HBM).
 // Pixels are the MFMA column index, so a wave's stores run along ox: contiguous in NCHW.
-// 64 (cout) x 64 (pixels) per workgroup, K step 32, 2 x 2 waves of one 32 x 32 tile.
+// 64 or 128 (cout) x 64 (pixels) per workgroup, K step 32, 2 x 2 waves.
 // The k -> (input offset, dy, dx) table is built on the host at registration and read with
 // wave-uniform (scalar) loads.
 //
@@ -27,20 +27,27 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-constexpr int CM = 64, CN = 64, CK = 32, CPAD = 8;
+constexpr int CM = 64, CN = 64, CK = 32;
+// LDS row padding: bf16 rows of 80 bytes keep the 128-bit fragment reads of 16 consecutive rows on distinct
+// banks; f32 rows of 33 words do the same for the one-word reads of 32 consecutive rows.
+template <int DT> constexpr int cpad() { return DT == DT_F32 ? 1 : 8; }
 
 template <int DT> struct CT;
 template <> struct CT<DT_F32> { typedef float S; };
 template <> struct CT<DT_BF16> { typedef uint16_t S; };
 
-template <int DT, int ODT>
+// MT = 1: 64 (cout) x 64 (pixels) per workgroup, 2 x 2 waves of one 32 x 32 tile. MT = 2: 128 x 64, 2 x 2 waves of
+// two stacked 32 x 32 tiles, so the gathered pixel tile is formed once for 128 output channels. The loads of K
+// step s+1 are issued into registers before the MFMAs of step s and written to LDS after them.
+template <int DT, int ODT, int MT>
 __global__ __launch_bounds__(256) void conv2d_k(const Conv2d p) {
     typedef typename CT<DT>::S S;
-    __shared__ __attribute__((aligned(16))) S Ws[CM * (CK + CPAD)];
+    constexpr int TM = CM * MT, CPAD = cpad<DT>();
+    __shared__ __attribute__((aligned(16))) S Ws[TM * (CK + CPAD)];
     __shared__ __attribute__((aligned(16))) S Xs[CN * (CK + CPAD)];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int64_t co0 = (int64_t)blockIdx.y * CM, p0 = (int64_t)blockIdx.x * CN;
+    const int64_t co0 = (int64_t)blockIdx.y * TM, p0 = (int64_t)blockIdx.x * CN;
     const int64_t K = (int64_t)p.C * p.KH * p.KW, OHW = (int64_t)p.OH * p.OW, P = (int64_t)p.N * OHW;
     const S *W = (const S *)p.w, *X = (const S *)p.x;
 
@@ -52,17 +59,19 @@ __global__ __launch_bounds__(256) void conv2d_k(const Conv2d p) {
     const int iy0 = oy * p.sy - p.py, ix0 = ox * p.sx - p.px;
     const S *xn = X + n * (int64_t)p.C * p.H * p.W + (int64_t)iy0 * p.W + ix0;
 
-    f32x16 acc;
+    f32x16 acc[MT];
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[m][r] = 0.0f;
 
-    for (int64_t k0 = 0; k0 < K; k0 += CK) {
-        __syncthreads();
+    S rw[8 * MT], rx[8];
+    auto fetch = [&](int64_t k0) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) { // weight tile: K contiguous, consecutive threads along k
+        for (int e = 0; e < 8 * MT; e++) { // weight tile: K contiguous, consecutive threads along k
             const int idx = e * 256 + t, r = idx >> 5, k = idx & 31;
             const int64_t gr = co0 + r, gk = k0 + k;
-            Ws[r * (CK + CPAD) + k] = (gr < p.Cout && gk < K) ? W[gr * K + gk] : (S)0;
+            rw[e] = (gr < p.Cout && gk < K) ? W[gr * K + gk] : (S)0;
         }
 #pragma unroll
         for (int e = 0; e < 8; e++) { // gathered tile: k is uniform over a wave, lanes walk along the pixels
@@ -75,23 +84,42 @@ __global__ __launch_bounds__(256) void conv2d_k(const Conv2d p) {
                 const int iy = iy0 + (dyx >> 16), ix = ix0 + (dyx & 0xffff);
                 if (pix_ok && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W) v = xn[off];
             }
-            Xs[(t & 63) * (CK + CPAD) + kl] = v;
+            rx[e] = v;
         }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int e = 0; e < 8 * MT; e++) {
+            const int idx = e * 256 + t;
+            Ws[(idx >> 5) * (CK + CPAD) + (idx & 31)] = rw[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) Xs[(t & 63) * (CK + CPAD) + (t >> 6) + 4 * e] = rx[e];
+    };
+
+    fetch(0);
+    for (int64_t k0 = 0; k0 < K; k0 += CK) {
+        __syncthreads(); // the previous step's fragment reads are done
+        stash();
         __syncthreads();
-        const S *ar = Ws + (wm * 32 + (lane & 31)) * (CK + CPAD);
+        if (k0 + CK < K) fetch(k0 + CK); // in flight while the matrix cores work on this step
         const S *br = Xs + (wn * 32 + (lane & 31)) * (CK + CPAD);
-        if (DT == DT_F32) {
 #pragma unroll
-            for (int ks = 0; ks < CK; ks += 2) {
-                float a = ((const float *)ar)[ks + (lane >> 5)], b = ((const float *)br)[ks + (lane >> 5)];
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
-            }
-        } else {
+        for (int m = 0; m < MT; m++) {
+            const S *ar = Ws + ((wm * MT + m) * 32 + (lane & 31)) * (CK + CPAD);
+            if (DT == DT_F32) {
 #pragma unroll
-            for (int ks = 0; ks < CK; ks += 16) {
-                const int off = ks + (lane >> 5) * 8;
-                bf16x8 a = *(const bf16x8 *)((const uint16_t *)ar + off), b = *(const bf16x8 *)((const uint16_t *)br + off);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+                for (int ks = 0; ks < CK; ks += 2) {
+                    float a = ((const float *)ar)[ks + (lane >> 5)], b = ((const float *)br)[ks + (lane >> 5)];
+                    acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[m], 0, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int ks = 0; ks < CK; ks += 16) {
+                    const int off = ks + (lane >> 5) * 8;
+                    bf16x8 a = *(const bf16x8 *)((const uint16_t *)ar + off), b = *(const bf16x8 *)((const uint16_t *)br + off);
+                    acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[m], 0, 0, 0);
+                }
             }
         }
     }
@@ -101,16 +129,18 @@ __global__ __launch_bounds__(256) void conv2d_k(const Conv2d p) {
     if (opix >= P) return; // no barrier follows
     const int64_t on = opix / OHW, orem = opix - on * OHW;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int64_t co = co0 + wm * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        if (co >= p.Cout) continue;
-        float v = acc[r];
-        if (p.bias) v += DT == DT_F32 ? ((const float *)p.bias)[co] : bf16_to_f32(((const uint16_t *)p.bias)[co]);
-        if (p.relu) v = (v > 0.0f ? 1.0f : 0.0f) * v;
-        const int64_t o = (on * p.Cout + co) * OHW + orem;
-        if (ODT == DT_F32) ((float *)p.y)[o] = v;
-        else ((uint16_t *)p.y)[o] = f32_to_bf16_trunc(v);
-    }
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int64_t co = co0 + (wm * MT + m) * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            if (co >= p.Cout) continue;
+            float v = acc[m][r];
+            if (p.bias) v += DT == DT_F32 ? ((const float *)p.bias)[co] : bf16_to_f32(((const uint16_t *)p.bias)[co]);
+            if (p.relu) v = (v > 0.0f ? 1.0f : 0.0f) * v;
+            const int64_t o = (on * p.Cout + co) * OHW + orem;
+            if (ODT == DT_F32) ((float *)p.y)[o] = v;
+            else ((uint16_t *)p.y)[o] = f32_to_bf16_trunc(v);
+        }
 }
 
 template <int DT>
@@ -229,12 +259,18 @@ hipError_t conv2d(const Conv2d &p, hipStream_t st) {
         g.C = p.y;
         return gemm_bf16(g, st);
     }
-    if ((p.Cout + CM - 1) / CM > 65535 || (P + CN - 1) / CN >= (1ll << 31)) return hipErrorInvalidValue;
-    dim3 grid((unsigned)((P + CN - 1) / CN), (unsigned)((p.Cout + CM - 1) / CM)), block(256);
-    if (p.dtype == DT_F32 && p.out_dtype == DT_F32) hipLaunchKernelGGL((conv2d_k<DT_F32, DT_F32>), grid, block, 0, st, p);
-    else if (p.dtype == DT_BF16 && p.out_dtype == DT_BF16) hipLaunchKernelGGL((conv2d_k<DT_BF16, DT_BF16>), grid, block, 0, st, p);
-    else if (p.dtype == DT_BF16 && p.out_dtype == DT_F32) hipLaunchKernelGGL((conv2d_k<DT_BF16, DT_F32>), grid, block, 0, st, p);
+    const int mt = p.Cout > CM ? 2 : 1;
+    const int64_t tm = CM * mt;
+    if ((p.Cout + tm - 1) / tm > 65535 || (P + CN - 1) / CN >= (1ll << 31)) return hipErrorInvalidValue;
+    dim3 grid((unsigned)((P + CN - 1) / CN), (unsigned)((p.Cout + tm - 1) / tm)), block(256);
+#define ZK_CONV(D, O)                                                                   \
+    if (mt == 2) hipLaunchKernelGGL((conv2d_k<D, O, 2>), grid, block, 0, st, p);        \
+    else hipLaunchKernelGGL((conv2d_k<D, O, 1>), grid, block, 0, st, p)
+    if (p.dtype == DT_F32 && p.out_dtype == DT_F32) { ZK_CONV(DT_F32, DT_F32); }
+    else if (p.dtype == DT_BF16 && p.out_dtype == DT_BF16) { ZK_CONV(DT_BF16, DT_BF16); }
+    else if (p.dtype == DT_BF16 && p.out_dtype == DT_F32) { ZK_CONV(DT_BF16, DT_F32); }
     else return hipErrorInvalidValue;
+#undef ZK_CONV
     return hipGetLastError();
 }
 

@@ -11,8 +11,8 @@
 //
 // 64 x 64 tile per 256-thread workgroup, 2 x 2 waves of one 32 x 32 MFMA tile each, K step
 // 32. Operands are read with bounds checks (zero fill) straight from their natural layout,
-// coalesced along whichever index is contiguous, and laid down K-contiguous in LDS with an
-// 8-element row pad, so fragment reads are the same for all four layouts.
+// coalesced along whichever index is contiguous, and laid down K-contiguous in LDS with a
+// row pad (8 elements for 16-bit types, 1 for f32), so fragment reads are the same for all four layouts.
 #include <algorithm>
 
 #include "dtypes.hpp"
@@ -27,7 +27,10 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int GM = 64, GN = 64, GK = 32, GPAD = 8;
+constexpr int GM = 64, GN = 64, GK = 32;
+// LDS row padding: 16-bit rows of 80 bytes keep 128-bit fragment reads of 16 consecutive rows on distinct banks;
+// f32 rows of 33 words do the same for the one-word reads of 32 consecutive rows.
+template <typename S> constexpr int gpad() { return sizeof(S) == 4 ? 1 : 8; }
 
 template <int DT> struct GT;
 template <> struct GT<DT_F32> {
@@ -55,6 +58,7 @@ __device__ __forceinline__ float gelu_ref(float x) { // zyx/src/tensor/elementwi
 template <typename S>
 __device__ __forceinline__ void fill_tile(S *__restrict__ dst, const S *__restrict__ src, int64_t rs, int64_t ks,
                                           int64_t row0, int64_t k0, int64_t rows, int64_t K, S zero) {
+    constexpr int GPAD = gpad<S>();
     const int t = threadIdx.x;
     if (ks == 1) { // K contiguous: consecutive threads walk along k
 #pragma unroll
@@ -76,6 +80,7 @@ __device__ __forceinline__ void fill_tile(S *__restrict__ dst, const S *__restri
 template <int DT, int ODT>
 __global__ __launch_bounds__(256) void gemm_generic_k(const GemmGeneric p) {
     typedef typename GT<DT>::S S;
+    constexpr int GPAD = gpad<S>();
     __shared__ __attribute__((aligned(16))) S As[GM * (GK + GPAD)];
     __shared__ __attribute__((aligned(16))) S Bs[GN * (GK + GPAD)];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
