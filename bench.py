@@ -145,6 +145,9 @@ def extra_streaming(dev, pool, kernels, steps=20, warmup=5):
     for dt, isz, tag in ((zyx_amd.DType.BF16, 2, "bf16"), (zyx_amd.DType.F32, 4, "f32")):
         h, g, o = dev_arr((M, F), dt), dev_arr((M, F), dt), out_arr(M * F, isz)
         c = kernels.Chain(M, F, out_dtype=dt)
+        c.load(c.input(dt))
+        timeit(f"copy_{tag}_8192x4096", c.desc(), [h, o], 2 * M * F * isz)  # the streaming ceiling of this part
+        c = kernels.Chain(M, F, out_dtype=dt)
         c.load(c.input(dt)).gelu()
         timeit(f"gelu_{tag}_8192x4096", c.desc(), [h, o], 2 * M * F * isz)
         c = kernels.Chain(M, F, out_dtype=dt)
