@@ -147,3 +147,21 @@ def test_config4_bf16_full_size(hip, oracle):
     assert np.array_equal(yb, ya * 0.5)  # scaling the weights by a power of two scales every product exactly
     assert np.array_equal(conv2d(dev, pool, x[7:15], w2, None, (1, 1), (1, 1), dtype=DType.BF16, out_dtype=DType.F32),
                           conv2d(dev, pool, x, w2, None, (1, 1), (1, 1), dtype=DType.BF16, out_dtype=DType.F32)[7:15])
+
+
+@pytest.mark.parametrize("geom", [
+    # (x shape, weight shape, stride, padding, dilation): shapes whose patch rows the GEMM gathers itself (unit
+    # column stride, output rows of 8k pixels); dilation, row stride, asymmetric padding, 1x1 and 5x5 windows
+    ((4, 64, 24, 24), (128, 64, 3, 3), (1, 1), (2, 2), (2, 2)), ((4, 64, 32, 16), (128, 64, 3, 3), (2, 1), (1, 1), (1, 1)),
+    ((2, 64, 8, 32), (256, 64, 1, 1), (1, 1), (0, 0), (1, 1)), ((1, 64, 16, 20), (128, 64, 5, 5), (1, 1), (2, 0), (1, 1)),
+    ((8, 32, 9, 16), (128, 32, 2, 1), (1, 1), (0, 0), (1, 1))])
+def test_conv_bf16_gathered_by_the_gemm(hip, oracle, geom):
+    dev, pool = hip
+    xs, ws, stride, pad, dil = geom
+    r = oracle.Rng(sum(xs))
+    x, wt, b = oracle.f32_to_bf16(r.randn(xs)), oracle.f32_to_bf16(r.randn(ws, 0.1)), oracle.f32_to_bf16(r.randn(ws[0], 0.5))
+    got32 = conv2d(dev, pool, x, wt, b, stride, pad, dil, relu=True, dtype=DType.BF16, out_dtype=DType.F32)
+    want32 = oracle.conv2d(x, wt, b, stride, pad, dil, True, oracle.BF16, oracle.F32)
+    mag = oracle.conv2d(np.abs(oracle.bf16_to_f32(x)), np.abs(oracle.bf16_to_f32(wt)), np.abs(oracle.bf16_to_f32(b)), stride, pad, dil)
+    assert got32.shape == want32.shape and got32.shape[3] % 8 == 0 and (got32.shape[0] * got32.shape[2] * got32.shape[3]) % 256 == 0
+    assert np.all(np.abs(got32 - want32) <= 1e-3 * np.abs(want32) + 2e-5 * mag)

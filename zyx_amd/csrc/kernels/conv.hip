@@ -218,6 +218,18 @@ __global__ __launch_bounds__(256) void im2col_t_bf16_k(const uint16_t *__restric
     *(uint4 *)(a + (int64_t)k * pixels + pix0) = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// Zero-padded copy of the input, xp[n, c, H + 2*py, W + 2*px]: with it every tap of every output pixel is an
+// in-bounds read, so the GEMM can gather its patch rows with plain 128-bit loads and no masks.
+__global__ __launch_bounds__(256) void pad_input_bf16_k(const uint16_t *__restrict__ x, uint16_t *__restrict__ xp, int H, int W,
+                                                        int py, int px, int64_t total) {
+    const int Hp = H + 2 * py, Wp = W + 2 * px;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t plane = i / (Hp * Wp);
+        const int rem = (int)(i - plane * (Hp * Wp)), yy = rem / Wp - py, xx = rem % Wp - px;
+        xp[i] = (yy >= 0 && yy < H && xx >= 0 && xx < W) ? x[(plane * H + yy) * W + xx] : (uint16_t)0;
+    }
+}
+
 // bf16 convolutions whose lowered product fits the tiled MFMA GEMM exactly: patches . W^T with
 // M = pixels (multiple of 256), N = Cout (multiple of 128), K = C*KH*KW (multiple of 64), no K split.
 bool conv_uses_gemm(const Conv2d &p) {
@@ -226,12 +238,20 @@ bool conv_uses_gemm(const Conv2d &p) {
            K <= 65535 && pixels < (1ll << 30) && gemm_bf16_supported(pixels, p.Cout, K) && gemm_bf16_splits(pixels, p.Cout, K) == 1;
 }
 constexpr uint64_t kZeroBiasBytes = 4096 * 4;
+// ... and whose patch rows are runs of 8 consecutive input columns (unit column stride, rows of 8k outputs): the
+// GEMM gathers them itself from a padded copy of the input and no patch matrix is written.
+bool conv_gathers_in_gemm(const Conv2d &p) {
+    return conv_uses_gemm(p) && p.sx == 1 && p.OW % 8 == 0 &&
+           (int64_t)p.N * p.C * (p.H + 2 * p.py) * (p.W + 2 * p.px) < (1ll << 30);
+}
 
 } // namespace
 
 // scratch = [zero bias (for ReLU without bias)] [patch matrix K x pixels bf16]
 uint64_t conv2d_scratch_bytes(const Conv2d &p) {
     if (!conv_uses_gemm(p) || p.Cout > 4096) return 0;
+    if (conv_gathers_in_gemm(p)) // padded input (+ 16 bytes: the last 128-bit load may start 7 elements before the end)
+        return kZeroBiasBytes + (uint64_t)p.N * p.C * (p.H + 2 * p.py) * (p.W + 2 * p.px) * 2 + 16;
     return kZeroBiasBytes + (uint64_t)p.C * p.KH * p.KW * (uint64_t)p.N * p.OH * p.OW * 2;
 }
 
@@ -242,8 +262,27 @@ hipError_t conv2d(const Conv2d &p, hipStream_t st) {
         // im2col (transposed) + GEMM: C[pixel, co] = sum_k a[k, pixel] * w[co, k], stored as NCHW by the epilogue
         uint16_t *a = (uint16_t *)((char *)p.scratch + kZeroBiasBytes);
         const int K = p.C * p.KH * p.KW;
-        hipLaunchKernelGGL(im2col_t_bf16_k, dim3((unsigned)((P / 8 + 255) / 256), (unsigned)K), dim3(256), 0, st, (const uint16_t *)p.x, a, p, P);
         GemmBf16 g{};
+        if (conv_gathers_in_gemm(p)) {
+            const int Hp = p.H + 2 * p.py, Wp = p.W + 2 * p.px;
+            const int64_t total = (int64_t)p.N * p.C * Hp * Wp;
+            int64_t blocks = (total + 255) / 256;
+            if (blocks > 256 * 64) blocks = 256 * 64;
+            hipLaunchKernelGGL(pad_input_bf16_k, dim3((unsigned)blocks), dim3(256), 0, st, (const uint16_t *)p.x, a, p.H, p.W, p.py, p.px, total);
+            ConvGather &c = g.gather;
+            c.ohw = p.OH * p.OW;
+            c.ow = p.OW;
+            c.img = p.C * Hp * Wp;
+            c.row = p.sy * Wp;
+            c.cs = Hp * Wp;
+            c.rs = p.dy * Wp;
+            c.dx = p.dx;
+            c.khw = (uint32_t)(p.KH * p.KW);
+            c.kw = (uint32_t)p.KW;
+            c.magic_khw = (uint32_t)(((1ull << 32) + c.khw - 1) / c.khw);
+            c.magic_kw = (uint32_t)(((1ull << 32) + c.kw - 1) / c.kw);
+        } else
+            hipLaunchKernelGGL(im2col_t_bf16_k, dim3((unsigned)((P / 8 + 255) / 256), (unsigned)K), dim3(256), 0, st, (const uint16_t *)p.x, a, p, P);
         g.M = P;
         g.N = p.Cout;
         g.K = K;

@@ -124,11 +124,14 @@ __device__ __forceinline__ float gelu_fast(float x) {
 
 // AT: A stored [K, M] (M contiguous) instead of [M, K]; BT: B stored [N, K] (K contiguous)
 // instead of [K, N]. EPI: 0 none, 1 + bias, 2 + bias then ReLU, 3 + bias then GELU.
-template <bool AT, bool BT, int EPI, int BNV, bool PLANE>
+// PLANE: 0 plain row-major C; 1 C stored [M / plane, N, plane] (NCHW result of a convolution whose patch matrix is
+// operand A); 2 the same store, and operand A is not a matrix in memory at all: its [K, M] tile rows are gathered
+// from a zero-padded NCHW input (`A` points at it, `g` describes it), 8 consecutive pixels per 128-bit load.
+template <bool AT, bool BT, int EPI, int BNV, int PLANE>
 __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                       void *__restrict__ Cv, const void *__restrict__ bias,
                                                       const void *__restrict__ residual, int bias_dtype, int out_bf16,
-                                                      int M, int N, int K, int splits, int plane) {
+                                                      int M, int N, int K, int splits, int plane, const ConvGather g) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
     constexpr int NJ = BNV / 64;                 // 32-column MFMA blocks per wave
@@ -185,7 +188,15 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
     const int64_t lda = AT ? M : K, ldb = BT ? K : N;
     uint32_t oa[8], ob[NB];
 #pragma unroll
-    for (int i = 0; i < 8; i++) oa[i] = (uint32_t)((TA::src(A, lda, m0, 0, i, wave, lane) - A) * 2);
+    for (int i = 0; i < 8; i++) {
+        if (PLANE == 2) {
+            // chunk i of this thread: k row i*8 + wave*2 + lane/32 of a K tile, pixels m0 + c*8 .. +7 (one output row)
+            const int kr = i * 8 + wave * 2 + (lane >> 5);
+            const int pix = m0 + (((lane & 31) ^ swz_mn<256>(kr)) << 3);
+            const int img = pix / g.ohw, rem = pix - img * g.ohw, oy = rem / g.ow, ox = rem - oy * g.ow;
+            oa[i] = (uint32_t)(img * g.img + oy * g.row + ox) * 2;
+        } else oa[i] = (uint32_t)((TA::src(A, lda, m0, 0, i, wave, lane) - A) * 2);
+    }
 #pragma unroll
     for (int i = 0; i < NB; i++) ob[i] = (uint32_t)((TB::src(B, ldb, n0, 0, i, wave, lane) - B) * 2);
     const int da0 = TA::dst(0, wave, lane), db0 = A_STAGE + TB::dst(0, wave, lane);
@@ -199,7 +210,14 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
     auto gload = [&](int u, int kt) {
         const int i = unit_chunk(u);
         if (unit_is_b(u)) rb[i] = *(const u32x4 *)((const uint8_t *)B + kt * adv_b + ob[i]);
-        else ra[i] = *(const u32x4 *)((const uint8_t *)A + kt * adv_a + oa[i]);
+        else if (PLANE == 2) {
+            // k = (c, ky, kx) of this chunk's row in K tile kt -> offset of that tap in the padded input
+            const uint32_t k = (uint32_t)(kt * BK + i * 8 + wave * 2 + (lane >> 5));
+            const uint32_t c = g.khw == 1 ? k : __umulhi(k, g.magic_khw), r = k - c * g.khw; // ceil(2^32 / 1) does not fit
+            const uint32_t ky = g.kw == 1 ? r : __umulhi(r, g.magic_kw), kx = r - ky * g.kw;
+            typedef uint32_t u32x4a2 __attribute__((ext_vector_type(4), aligned(2)));
+            ra[i] = *(const u32x4a2 *)((const uint8_t *)A + oa[i] + (c * g.cs + ky * g.rs + kx * g.dx) * 2);
+        } else ra[i] = *(const u32x4 *)((const uint8_t *)A + kt * adv_a + oa[i]);
     };
     auto lwrite = [&](int u, int da_base, int db_base) {
         const int i = unit_chunk(u);
@@ -332,7 +350,7 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
             if (bias_dtype == DT_BF16) bv = bf16_to_f32(((const uint16_t *)bias)[col]);
             else bv = ((const float *)bias)[col];
         }
-        if (PLANE) {
+        if (PLANE != 0) {
             // C is stored as [M / plane, N, plane] (the NCHW result of a convolution lowered to this product:
             // row = image * plane + pixel, column = channel). The four consecutive rows a lane holds per
             // register group are consecutive pixels of one image (plane % 4 == 0): one 16- or 8-byte store.
@@ -431,8 +449,8 @@ template <bool AT, bool BT, int BNV> hipError_t launch_epi(const GemmBf16 &p, hi
     dim3 grid((unsigned)((p.M / BM) * (p.N / BNV) * splits)), block(256);
     if (splits > 1) {
         if (!p.workspace) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0, BNV, false>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, (const uint16_t *)p.B,
-                           p.workspace, nullptr, nullptr, 0, 0, (int)p.M, (int)p.N, (int)p.K, splits, 0);
+        hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0, BNV, 0>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, (const uint16_t *)p.B,
+                           p.workspace, nullptr, nullptr, 0, 0, (int)p.M, (int)p.N, (int)p.K, splits, 0, ConvGather{});
         const int64_t MN = p.M * p.N;
         hipLaunchKernelGGL(gemm_splitk_fold_k, dim3((unsigned)((MN / 4 + 255) / 256)), block, 0, st, (const float *)p.workspace, p.C,
                            p.bias, p.residual, p.epilogue, p.bias_dtype, p.out_bf16, MN, (int)p.N, splits);
@@ -441,20 +459,28 @@ template <bool AT, bool BT, int BNV> hipError_t launch_epi(const GemmBf16 &p, hi
     if (p.plane) {
         // only the product a convolution lowers to stores this way: A^T . B^T, epilogues none / bias / bias + ReLU
         if (!(AT && BT) || p.epilogue > 2) return hipErrorInvalidValue;
-#define ZK_GEMM_PL(E)                                                                                                 \
-    hipLaunchKernelGGL((gemm_bf16_k<true, true, E, BNV, true>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, \
-                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, p.plane);
-        switch (p.epilogue) {
-        case 0: ZK_GEMM_PL(0) break;
-        case 1: ZK_GEMM_PL(1) break;
-        default: ZK_GEMM_PL(2) break;
+#define ZK_GEMM_PL(E, G)                                                                                              \
+    hipLaunchKernelGGL((gemm_bf16_k<true, true, E, BNV, G>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A,    \
+                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, p.plane, p.gather);
+        if (p.gather.khw) {
+            switch (p.epilogue) {
+            case 0: ZK_GEMM_PL(0, 2) break;
+            case 1: ZK_GEMM_PL(1, 2) break;
+            default: ZK_GEMM_PL(2, 2) break;
+            }
+        } else {
+            switch (p.epilogue) {
+            case 0: ZK_GEMM_PL(0, 1) break;
+            case 1: ZK_GEMM_PL(1, 1) break;
+            default: ZK_GEMM_PL(2, 1) break;
+            }
         }
 #undef ZK_GEMM_PL
         return hipGetLastError();
     }
 #define ZK_GEMM(E)                                                                                                    \
-    hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E, BNV, false>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A,  \
-                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, 0);
+    hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E, BNV, 0>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A,      \
+                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, 0, ConvGather{});
     switch (p.epilogue) {
     case 0: ZK_GEMM(0) break;
     case 1: ZK_GEMM(1) break;
@@ -471,10 +497,12 @@ template <bool AT, bool BT> hipError_t launch_width(const GemmBf16 &p, hipStream
 
 template <bool AT, bool BT, int E, int BNV> hipError_t allow_lds() {
     if (AT && BT && E <= 2) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_k<true, true, (E <= 2 ? E : 0), BNV, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_k<true, true, (E <= 2 ? E : 0), BNV, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute((const void *)gemm_bf16_k<true, true, (E <= 2 ? E : 0), BNV, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
         if (e != hipSuccess) return e;
     }
-    return hipFuncSetAttribute((const void *)gemm_bf16_k<AT, BT, E, BNV, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
+    return hipFuncSetAttribute((const void *)gemm_bf16_k<AT, BT, E, BNV, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
 }
 template <bool AT, bool BT> hipError_t allow_lds_epi() {
     hipError_t e;

@@ -53,6 +53,16 @@ struct Reduce {
 uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int axis0);
 hipError_t reduce(const Reduce &p, hipStream_t stream);
 
+// Geometry of a zero-padded NCHW input [images, C, Hp, Wp] from which gemm_bf16 gathers the patch matrix of a
+// convolution on the fly (khw == 0: not used). Offsets in elements; k = (c*KH + ky)*KW + kx.
+struct ConvGather {
+    int ohw, ow;        // output pixels per image, per row
+    int img, row;       // input elements per image; per output row step (sy * Wp)
+    int cs, rs, dx;     // per channel (Hp*Wp), per ky (dy*Wp), per kx (dx)
+    uint32_t khw, kw;   // KH*KW, KW
+    uint32_t magic_khw, magic_kw; // ceil(2^32 / khw), ceil(2^32 / kw): exact division of k < 2^16 by a multiply-high
+};
+
 // C[M,N] = op(A) . op(B) (+ bias[N], + activation) (+ residual[M,N]), bf16 operands, f32 accumulate;
 // C and the residual are f32, or bf16 (truncating store) when out_bf16 is set.
 // trans_a: A is stored [K,M]; trans_b: B is stored [N,K] (a Linear weight [out,in]).
@@ -63,6 +73,7 @@ struct GemmBf16 {
     int bias_dtype;    // DT_BF16 or DT_F32
     int out_bf16;
     int plane; // 0, or C is stored [M / plane, N, plane] (rows of one group of `plane` are contiguous per column)
+    ConvGather gather; // with plane != 0 and gather.khw != 0: A is the padded input, not a matrix
     const void *A, *B, *bias, *residual; // residual may be null
     void *C;
     void *workspace; // gemm_bf16_workspace_bytes(M, N, K) bytes (split-K partials), may be null when that is 0
