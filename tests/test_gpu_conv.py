@@ -154,7 +154,7 @@ def test_config4_bf16_full_size(hip, oracle):
     # column stride, output rows of 8k pixels); dilation, row stride, asymmetric padding, 1x1 and 5x5 windows
     ((4, 64, 24, 24), (128, 64, 3, 3), (1, 1), (2, 2), (2, 2)), ((4, 64, 32, 16), (128, 64, 3, 3), (2, 1), (1, 1), (1, 1)),
     ((2, 64, 8, 32), (256, 64, 1, 1), (1, 1), (0, 0), (1, 1)), ((1, 64, 16, 20), (128, 64, 5, 5), (1, 1), (2, 0), (1, 1)),
-    ((8, 32, 9, 16), (128, 32, 2, 1), (1, 1), (0, 0), (1, 1))])
+    ((8, 32, 9, 16), (128, 32, 2, 1), (1, 1), (0, 0), (1, 1)), ((2, 64, 17, 25), (128, 64, 2, 2), (1, 1), (0, 0), (1, 1))])
 def test_conv_bf16_gathered_by_the_gemm(hip, oracle, geom):
     dev, pool = hip
     xs, ws, stride, pad, dil = geom

@@ -221,12 +221,19 @@ __global__ __launch_bounds__(256) void im2col_t_bf16_k(const uint16_t *__restric
 // Zero-padded copy of the input, xp[n, c, H + 2*py, W + 2*px]: with it every tap of every output pixel is an
 // in-bounds read, so the GEMM can gather its patch rows with plain 128-bit loads and no masks.
 __global__ __launch_bounds__(256) void pad_input_bf16_k(const uint16_t *__restrict__ x, uint16_t *__restrict__ xp, int H, int W,
-                                                        int py, int px, int64_t total) {
-    const int Hp = H + 2 * py, Wp = W + 2 * px;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-        const int64_t plane = i / (Hp * Wp);
-        const int rem = (int)(i - plane * (Hp * Wp)), yy = rem / Wp - py, xx = rem % Wp - px;
-        xp[i] = (yy >= 0 && yy < H && xx >= 0 && xx < W) ? x[(plane * H + yy) * W + xx] : (uint16_t)0;
+                                                        int py, int px, int total) {
+    // 32-bit index arithmetic (total < 2^30); a thread writes two neighbouring elements as one word when rows are
+    // of even length (pairs then never straddle a row)
+    const int Hp = H + 2 * py, Wp = W + 2 * px, step = (Wp & 1) ? 1 : 2;
+    for (int i = (blockIdx.x * 256 + threadIdx.x) * step; i < total; i += gridDim.x * 256 * step) {
+        const int plane = i / (Hp * Wp), rem = i - plane * (Hp * Wp), yy = rem / Wp - py, xx = rem % Wp - px;
+        const uint16_t *row = x + ((int64_t)plane * H + yy) * W;
+        const bool rok = yy >= 0 && yy < H;
+        const uint32_t a = (rok && xx >= 0 && xx < W) ? row[xx] : 0u;
+        if (step == 2) {
+            const uint32_t b = (rok && xx + 1 >= 0 && xx + 1 < W) ? row[xx + 1] : 0u;
+            *(uint32_t *)(xp + i) = a | (b << 16);
+        } else xp[i] = (uint16_t)a;
     }
 }
 
@@ -265,8 +272,8 @@ hipError_t conv2d(const Conv2d &p, hipStream_t st) {
         GemmBf16 g{};
         if (conv_gathers_in_gemm(p)) {
             const int Hp = p.H + 2 * p.py, Wp = p.W + 2 * p.px;
-            const int64_t total = (int64_t)p.N * p.C * Hp * Wp;
-            int64_t blocks = (total + 255) / 256;
+            const int total = p.N * p.C * Hp * Wp; // < 2^30, checked by conv_gathers_in_gemm
+            int blocks = (total / ((Wp & 1) ? 1 : 2) + 255) / 256;
             if (blocks > 256 * 64) blocks = 256 * 64;
             hipLaunchKernelGGL(pad_input_bf16_k, dim3((unsigned)blocks), dim3(256), 0, st, (const uint16_t *)p.x, a, p.H, p.W, p.py, p.px, total);
             ConvGather &c = g.gather;
