@@ -185,3 +185,72 @@ def test_bf16_output_and_residual(hip, oracle, mnk, epilogue):
         got16 = gemm(dev, pool, a, b, out_dtype=DType.BF16, residual=residual, **kw)
         # the bf16 result is the truncation of the f32 one (identical arithmetic before the store)
         assert np.array_equal(got16, oracle.f32_to_bf16(got32))
+
+
+# ---- edge tiles of the big-tile kernel ------------------------------------------------------------------
+
+def _guarded_gemm(dev, pool, a, b, m, n, k, out_dtype, extra=(), **desc_kw):
+    """Runs one bf16 product into a result buffer followed by 4096 sentinel elements; returns (C, sentinels)."""
+    from zyx_amd.kernels import gemm_desc, to_device, to_host
+    prog = dev.register_kernel(gemm_desc(m, n, k, DType.BF16, out_dtype, **desc_kw))
+    np_out = np.uint16 if out_dtype == DType.BF16 else np.float32
+    bufs, waits = [], []
+    for arr in (a, b) + tuple(extra):
+        bb, e = to_device(pool, arr)
+        bufs.append(bb)
+        waits.append(e)
+    guard = np.full(m * n + 4096, 0x7fc1 if out_dtype == DType.BF16 else np.float32(-12345.5), np_out)
+    cb, e = to_device(pool, guard)
+    waits.append(e)
+    done = dev.launch(prog, pool, bufs + [cb], waits)
+    res = to_host(pool, cb, (m * n + 4096,), np_out, [done])
+    for bb in bufs + [cb]:
+        pool.deallocate(bb, [])
+    dev.release(prog)
+    return res[:m * n].reshape(m, n), (res[m * n:], guard[m * n:])
+
+
+@pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("mnk", [(264, 136, 64), (64, 64, 128), (200, 328, 192), (1000, 1000, 256), (520, 72, 1024),
+                                 (776, 2056, 128), (2048, 50264, 64)])
+def test_bf16_edge_tiles(hip, oracle, mnk, trans_a, trans_b):
+    """M and N that are not multiples of the tile: the edge tiles' clamped loads must not leak into stored
+    elements and their masked stores must not touch anything past row M - 1 or column N - 1 (the last shape
+    is a vocabulary projection; (520, 72, 1024) also takes the split-K path)."""
+    dev, pool = hip
+    m, n, k = mnk
+    a, b = make(oracle, m, n, k, m * 3 + n + k, trans_a, trans_b)
+    got, (tail, guard) = _guarded_gemm(dev, pool, a, b, m, n, k, DType.F32, trans_a=trans_a, trans_b=trans_b)
+    assert np.array_equal(tail, guard)
+    want, mag = reference(oracle, a, b, trans_a, trans_b)
+    assert np.all(np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-5 * mag), np.max(np.abs(got - want) / (mag + 1e-30))
+
+
+@pytest.mark.parametrize("mnk", [(300, 200, 128), (1000, 72, 64), (72, 1000, 256), (257, 258, 64), (130, 66, 2048)])
+@pytest.mark.parametrize("epilogue", ["bias", "bias_relu", "bias_gelu"])
+def test_bf16_edge_tiles_linear(hip, oracle, mnk, epilogue):
+    """Linear layers of ragged width (x . W^T + b, activation, + residual) with f32 and bf16 results; the bf16
+    result must be the truncation of the f32 one, edge tiles included (N here is even, not always a multiple of 8)."""
+    dev, pool = hip
+    m, n, k = mnk
+    a, b = make(oracle, m, n, k, 13, trans_b=True)
+    r = oracle.Rng(6)
+    bias = oracle.f32_to_bf16(r.uniform((n,), -1, 1))
+    res = oracle.f32_to_bf16(r.randn((m, n)))
+    want, mag = reference(oracle, a, b, False, True)
+    want = want + oracle.bf16_to_f32(bias).astype(np.float64)
+    if epilogue == "bias_relu":
+        want = np.maximum(want, 0.0)
+    if epilogue == "bias_gelu":
+        want = 0.5 * want * (1 + np.tanh(np.sqrt(2 / np.pi) * (want + 0.044715 * want ** 3)))
+    kw = dict(trans_b=True, epilogue=epilogue, bias_dtype=DType.BF16)
+    for residual in (False, True):
+        w = want + (oracle.bf16_to_f32(res).astype(np.float64) if residual else 0.0)
+        got32, (tail, guard) = _guarded_gemm(dev, pool, a, b, m, n, k, DType.F32,
+                                             (bias,) + ((oracle.bf16_to_f32(res),) if residual else ()), residual=residual, **kw)
+        assert np.array_equal(tail, guard)
+        assert np.all(np.abs(got32 - w) <= 1e-3 * np.abs(w) + 2e-5 * mag + 1e-6)
+        got16, (tail, guard) = _guarded_gemm(dev, pool, a, b, m, n, k, DType.BF16, (bias,) + ((res,) if residual else ()),
+                                             residual=residual, **kw)
+        assert np.array_equal(tail, guard)
+        assert np.array_equal(got16, oracle.f32_to_bf16(got32))

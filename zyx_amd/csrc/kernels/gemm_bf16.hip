@@ -55,10 +55,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ int swz_kc(int row) { return (row >> 1) & 7; }
 struct TileKC { // NCHUNK chunks per thread = rows / 32
     static __device__ __forceinline__ const uint16_t *src(const uint16_t *g, int64_t ld, int row0, int k0, int i, int wave,
-                                                         int lane) {
+                                                         int lane, int limit) {
         const int row = i * 32 + wave * 8 + (lane >> 3);
         const int c = (lane & 7) ^ swz_kc(row);
-        return g + (int64_t)(row0 + row) * ld + k0 + c * 8;
+        // rows past the operand's end (edge tiles) re-read its last row: in bounds, and never stored
+        return g + (int64_t)min(row0 + row, limit - 1) * ld + k0 + c * 8;
     }
     static constexpr __host__ __device__ __forceinline__ int dst(int i, int wave, int lane) { return (i * 32 + wave * 8) * 128 + lane * 16; }
     static __device__ __forceinline__ int64_t k_advance(int64_t) { return BK; }
@@ -74,10 +75,11 @@ template <int COLS> struct TileMN {
     static constexpr int KPW = 64 / CH;          // k rows one wave covers per pass
     static constexpr int NCHUNK = COLS / 32;     // passes (chunks per thread)
     static __device__ __forceinline__ const uint16_t *src(const uint16_t *g, int64_t ld, int col0, int k0, int i, int wave,
-                                                         int lane) {
+                                                         int lane, int limit) {
         const int k = i * 4 * KPW + wave * KPW + lane / CH;
         const int c = (lane % CH) ^ swz_mn<COLS>(k);
-        return g + (int64_t)(k0 + k) * ld + col0 + c * 8;
+        // chunks past the operand's end (edge tiles; the extent is a multiple of 8) re-read its last chunk
+        return g + (int64_t)(k0 + k) * ld + min(col0 + c * 8, limit - 8);
     }
     static constexpr __host__ __device__ __forceinline__ int dst(int i, int wave, int lane) { return (i * 4 * KPW + wave * KPW) * COLS * 2 + lane * 16; }
     static __device__ __forceinline__ int64_t k_advance(int64_t ld) { return BK * ld; }
@@ -127,7 +129,8 @@ __device__ __forceinline__ float gelu_fast(float x) {
 // PLANE: 0 plain row-major C; 1 C stored [M / plane, N, plane] (NCHW result of a convolution whose patch matrix is
 // operand A); 2 the same store, and operand A is not a matrix in memory at all: its [K, M] tile rows are gathered
 // from a zero-padded NCHW input (`A` points at it, `g` describes it), 8 consecutive pixels per 128-bit load.
-template <bool AT, bool BT, int EPI, int BNV, int PLANE>
+// TAIL: M and / or N are not multiples of the tile; edge tiles clamp their loads and mask their stores.
+template <bool AT, bool BT, int EPI, int BNV, int PLANE, bool TAIL>
 __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                       void *__restrict__ Cv, const void *__restrict__ bias,
                                                       const void *__restrict__ residual, int bias_dtype, int out_bf16,
@@ -144,7 +147,7 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
 
     // XCD-aware tile order: ids congruent mod 8 land on one XCD; give each XCD a patch
     // of 4 x 8 tiles (or the whole grid when it is smaller).
-    const int tiles_m = M / BM, tiles_n = N / BNV;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BNV - 1) / BNV;
     // split-K: workgroup z of a tile multiplies K range [z, z+1) * K/splits and stores its raw f32 partial
     // tile into slice z of Cv (a [splits, M, N] workspace that a second kernel folds)
     const int split = blockIdx.x / (tiles_m * tiles_n);
@@ -195,10 +198,10 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
             const int pix = m0 + (((lane & 31) ^ swz_mn<256>(kr)) << 3);
             const int img = pix / g.ohw, rem = pix - img * g.ohw, oy = rem / g.ow, ox = rem - oy * g.ow;
             oa[i] = (uint32_t)(img * g.img + oy * g.row + ox) * 2;
-        } else oa[i] = (uint32_t)((TA::src(A, lda, m0, 0, i, wave, lane) - A) * 2);
+        } else oa[i] = (uint32_t)((TA::src(A, lda, m0, 0, i, wave, lane, M) - A) * 2);
     }
 #pragma unroll
-    for (int i = 0; i < NB; i++) ob[i] = (uint32_t)((TB::src(B, ldb, n0, 0, i, wave, lane) - B) * 2);
+    for (int i = 0; i < NB; i++) ob[i] = (uint32_t)((TB::src(B, ldb, n0, 0, i, wave, lane, N) - B) * 2);
     const int da0 = TA::dst(0, wave, lane), db0 = A_STAGE + TB::dst(0, wave, lane);
     constexpr int da_step = TA::dst(1, 0, 0) - TA::dst(0, 0, 0), db_step = TB::dst(1, 0, 0) - TB::dst(0, 0, 0);
     const int64_t adv_a = TA::k_advance(lda) * 2, adv_b = TB::k_advance(ldb) * 2;
@@ -347,8 +350,9 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
         const int col = n0 + wn * WN + j * 32 + col_in;
         float bv = 0.0f;
         if (EPI >= 1) {
-            if (bias_dtype == DT_BF16) bv = bf16_to_f32(((const uint16_t *)bias)[col]);
-            else bv = ((const float *)bias)[col];
+            const int bc = TAIL ? min(col, N - 1) : col;
+            if (bias_dtype == DT_BF16) bv = bf16_to_f32(((const uint16_t *)bias)[bc]);
+            else bv = ((const float *)bias)[bc];
         }
         if (PLANE != 0) {
             // C is stored as [M / plane, N, plane] (the NCHW result of a convolution lowered to this product:
@@ -376,7 +380,9 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
                 const int rbase = m0 + wm * 128 + i * 32 + row_in;
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    const int64_t o = (int64_t)(rbase + (r >> 2) * 8 + (r & 3)) * N + col;
+                    const int row = rbase + (r >> 2) * 8 + (r & 3);
+                    if (TAIL && (row >= M || col >= N)) continue;
+                    const int64_t o = (int64_t)row * N + col;
                     float v = finish(acc[i][j][r], bv);
                     if (R) v += R[o];
                     C[o] = v;
@@ -396,6 +402,7 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
                     const float v0 = finish(acc[i][j][r], bv), v1 = finish(acc[i][j][r + 1], bv);
                     const float got = dpp_f32<kDppQuadXor1>(odd ? v0 : v1);
                     float lo = odd ? got : v0, hi = odd ? v1 : got;
+                    if (TAIL && (rbase + (r >> 2) * 8 + (r & 3) + odd >= M || col - odd + 1 >= N)) continue; // N is even
                     const int64_t o = (int64_t)(rbase + (r >> 2) * 8 + (r & 3) + odd) * N + (col - odd);
                     if (R) {
                         const uint32_t rr = *(const uint32_t *)(R + o);
@@ -443,13 +450,13 @@ __global__ __launch_bounds__(256) void gemm_splitk_fold_k(const float *__restric
     }
 }
 
-template <bool AT, bool BT, int BNV> hipError_t launch_epi(const GemmBf16 &p, hipStream_t st) {
+template <bool AT, bool BT, int BNV, bool TAIL> hipError_t launch_epi(const GemmBf16 &p, hipStream_t st) {
     const int splits = gemm_bf16_splits(p.M, p.N, p.K);
-    if (p.plane && (splits > 1 || p.residual || p.plane % 4 || p.M % p.plane)) return hipErrorInvalidValue;
-    dim3 grid((unsigned)((p.M / BM) * (p.N / BNV) * splits)), block(256);
+    if (p.plane && (TAIL || splits > 1 || p.residual || p.plane % 4 || p.M % p.plane)) return hipErrorInvalidValue;
+    dim3 grid((unsigned)(((p.M + BM - 1) / BM) * ((p.N + BNV - 1) / BNV) * splits)), block(256);
     if (splits > 1) {
         if (!p.workspace) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0, BNV, 0>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, (const uint16_t *)p.B,
+        hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0, BNV, 0, TAIL>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, (const uint16_t *)p.B,
                            p.workspace, nullptr, nullptr, 0, 0, (int)p.M, (int)p.N, (int)p.K, splits, 0, ConvGather{});
         const int64_t MN = p.M * p.N;
         hipLaunchKernelGGL(gemm_splitk_fold_k, dim3((unsigned)((MN / 4 + 255) / 256)), block, 0, st, (const float *)p.workspace, p.C,
@@ -460,7 +467,7 @@ template <bool AT, bool BT, int BNV> hipError_t launch_epi(const GemmBf16 &p, hi
         // only the product a convolution lowers to stores this way: A^T . B^T, epilogues none / bias / bias + ReLU
         if (!(AT && BT) || p.epilogue > 2) return hipErrorInvalidValue;
 #define ZK_GEMM_PL(E, G)                                                                                              \
-    hipLaunchKernelGGL((gemm_bf16_k<true, true, E, BNV, G>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A,    \
+    hipLaunchKernelGGL((gemm_bf16_k<true, true, E, BNV, G, false>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, \
                        (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, p.plane, p.gather);
         if (p.gather.khw) {
             switch (p.epilogue) {
@@ -479,7 +486,7 @@ template <bool AT, bool BT, int BNV> hipError_t launch_epi(const GemmBf16 &p, hi
         return hipGetLastError();
     }
 #define ZK_GEMM(E)                                                                                                    \
-    hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E, BNV, 0>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A,      \
+    hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E, BNV, 0, TAIL>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, \
                        (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, 0, ConvGather{});
     switch (p.epilogue) {
     case 0: ZK_GEMM(0) break;
@@ -492,17 +499,23 @@ template <bool AT, bool BT, int BNV> hipError_t launch_epi(const GemmBf16 &p, hi
     return hipGetLastError();
 }
 template <bool AT, bool BT> hipError_t launch_width(const GemmBf16 &p, hipStream_t st) {
-    return gemm_bf16_tile_n(p.M, p.N) == 128 ? launch_epi<AT, BT, 128>(p, st) : launch_epi<AT, BT, 256>(p, st);
+    const int bn = gemm_bf16_tile_n(p.M, p.N);
+    const bool tail = p.M % BM != 0 || p.N % bn != 0;
+    if (bn == 128) return tail ? launch_epi<AT, BT, 128, true>(p, st) : launch_epi<AT, BT, 128, false>(p, st);
+    return tail ? launch_epi<AT, BT, 256, true>(p, st) : launch_epi<AT, BT, 256, false>(p, st);
 }
 
 template <bool AT, bool BT, int E, int BNV> hipError_t allow_lds() {
+    hipError_t e;
     if (AT && BT && E <= 2) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemm_bf16_k<true, true, (E <= 2 ? E : 0), BNV, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
+        e = hipFuncSetAttribute((const void *)gemm_bf16_k<true, true, (E <= 2 ? E : 0), BNV, 1, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
         if (e != hipSuccess) return e;
-        e = hipFuncSetAttribute((const void *)gemm_bf16_k<true, true, (E <= 2 ? E : 0), BNV, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
+        e = hipFuncSetAttribute((const void *)gemm_bf16_k<true, true, (E <= 2 ? E : 0), BNV, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
         if (e != hipSuccess) return e;
     }
-    return hipFuncSetAttribute((const void *)gemm_bf16_k<AT, BT, E, BNV, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
+    e = hipFuncSetAttribute((const void *)gemm_bf16_k<AT, BT, E, BNV, 0, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute((const void *)gemm_bf16_k<AT, BT, E, BNV, 0, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(BNV));
 }
 template <bool AT, bool BT> hipError_t allow_lds_epi() {
     hipError_t e;
@@ -528,20 +541,34 @@ hipError_t gemm_bf16_init() {
     return allow_lds_epi<true, true>();
 }
 
+// Shapes whose every tile is whole (what the plane-store and gather variants need).
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K) {
     return M > 0 && N > 0 && K > 0 && M % BM == 0 && N % 128 == 0 && K % BK == 0 && M < (1 << 30) && N < (1 << 30) &&
-           K < (1 << 30) && (M / BM) * (N / 128) < (1ll << 27);
+           K < (1 << 30) && (M / BM) * (N / 128) < (1ll << 27) && M * K < (1ll << 31) && N * K < (1ll << 31); // 32-bit byte offsets
 }
 
-// Tile width: 128 columns when N is not a multiple of 256 or when 256-wide tiles would leave CUs idle.
+// The same kernel with edge tiles: any M and N of at least 64 whose 128-bit loads and paired stores stay
+// aligned, that is an extent that runs along memory in an operand ([K,M] A, [K,N] B) is a multiple of 8 and
+// N is even for a bf16 result. Loads of an edge tile clamp to the operand's last row / chunk, stores are masked.
+bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int out_bf16) {
+    if (gemm_bf16_supported(M, N, K)) return true;
+    return M >= 64 && N >= 64 && K > 0 && K % BK == 0 && M < (1 << 30) && N < (1 << 30) && K < (1 << 30) &&
+           ((M + BM - 1) / BM) * ((N + 127) / 128) < (1ll << 27) && (!trans_a || M % 8 == 0) && (trans_b || N % 8 == 0) &&
+           (!out_bf16 || N % 2 == 0) && M * K < (1ll << 31) && N * K < (1ll << 31);
+}
+
+// Tile width: 128 columns when that wastes fewer columns past N, or when 256-wide tiles would leave CUs idle.
 int gemm_bf16_tile_n(int64_t M, int64_t N) {
-    return (N % 256 != 0 || (M / BM) * (N / 256) < 192) ? 128 : 256;
+    const int64_t tm = (M + BM - 1) / BM;
+    return ((N + 127) / 128 * 128 != (N + 255) / 256 * 256 || tm * ((N + 255) / 256) < 192) ? 128 : 256;
 }
 
 // Split K when the output still has too few tiles to occupy the 256 CUs: the smallest power of two that
-// brings tiles * splits to 192 or more, while every split keeps at least 4 K tiles.
+// brings tiles * splits to 192 or more, while every split keeps at least 4 K tiles. The fold kernel works on
+// groups of 4 columns, so a ragged N that is not a multiple of 4 stays unsplit.
 int gemm_bf16_splits(int64_t M, int64_t N, int64_t K) {
-    const int64_t tiles = (M / BM) * (N / gemm_bf16_tile_n(M, N));
+    if (N % 4 != 0) return 1;
+    const int64_t tiles = ((M + BM - 1) / BM) * ((N + gemm_bf16_tile_n(M, N) - 1) / gemm_bf16_tile_n(M, N));
     int s = 1;
     while (tiles * s < 192 && s < 16 && K % (2 * s * BK) == 0 && K / (2 * s) >= 4 * BK) s *= 2;
     return s;
@@ -552,7 +579,7 @@ uint64_t gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 }
 
 hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t st) {
-    if (!gemm_bf16_supported(p.M, p.N, p.K)) return hipErrorInvalidValue;
+    if (!gemm_bf16_supported(p.M, p.N, p.K, p.trans_a, p.trans_b, p.out_bf16)) return hipErrorInvalidValue;
     if (p.trans_a) return p.trans_b ? launch_width<true, true>(p, st) : launch_width<true, false>(p, st);
     return p.trans_b ? launch_width<false, true>(p, st) : launch_width<false, false>(p, st);
 }

@@ -81,7 +81,8 @@ struct GemmBf16 {
 int gemm_bf16_tile_n(int64_t M, int64_t N);
 int gemm_bf16_splits(int64_t M, int64_t N, int64_t K);
 uint64_t gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K);
-bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K);
+bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K); // every tile whole
+bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int out_bf16); // edge tiles allowed
 hipError_t gemm_bf16_init(); // once per device, before the first launch
 hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t stream);
 

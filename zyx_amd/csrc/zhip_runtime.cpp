@@ -294,12 +294,14 @@ zk::Elementwise elementwise_args(const zhip_kernel_desc &d) {
     return a;
 }
 
-// bf16 problems of tile-multiple shape run on the 256x256 LDS-tiled kernel, everything else on the general one.
+// bf16 problems of K a multiple of 64 and M, N of at least 64 (aligned for 128-bit loads) run on the 256-row
+// LDS-tiled kernel, everything else on the general one.
 bool gemm_takes_fast_path(const zhip_kernel_desc &d) {
     const int64_t batch = d.dims[3] ? d.dims[3] : 1;
     const float alpha = d.fparams[0] == 0.0f ? 1.0f : d.fparams[0];
     return d.dtype == ZHIP_BF16 && batch == 1 && alpha == 1.0f && (d.iparams[0] == 0 || d.iparams[1] != ZHIP_F16) &&
-           zk::gemm_bf16_supported(d.dims[0], d.dims[1], d.dims[2]);
+           zk::gemm_bf16_supported(d.dims[0], d.dims[1], d.dims[2], d.flags & ZHIP_GEMM_TRANS_A ? 1 : 0,
+                                   d.flags & ZHIP_GEMM_TRANS_B ? 1 : 0, d.out_dtype == ZHIP_BF16);
 }
 
 // Shape and scalar parameters of the two attention kinds.
