@@ -264,6 +264,71 @@ typedef struct zhip_kernel_desc {
     int32_t iparams[24]; /* kind specific op codes */
 } zhip_kernel_desc;
 
+/* --- linearized kernel IR (what Device::compile receives) ---------------------- */
+
+/* A zyx `Kernel` after linearization is a linear SSA list of `OpNode`s walked from `head` through `next`
+ * (zyx/src/kernel/ops.rs:22-147, 353-358). Its image for zhip_compile_ir is
+ *     zhip_ir_header | zhip_ir_op[n_ops] in that order | uint32_t extra[n_extra]
+ * little endian. `id` is the op's OpId; operands name earlier ids. Ops that only exist before
+ * linearization (Move, Reduce) and the tile / tensor-core / assembly ops (Wmma, ReduceTile, MatmulTile,
+ * TransposeTile, Asm) have no code here: a kernel holding one is refused with ZHIP_KERNEL_COMPILATION,
+ * the answer a backend gives for what it cannot compile (zyx/src/codegen/cuda.rs:56-65).
+ *
+ *  opcode      dtype   a        b        c       aux                      imm
+ *  CONST       yes     -        -        -       -                        value bytes (Constant, dtype.rs)
+ *  PARAM       yes     -        -        -       zhip_ir_param_kind       elements the kernel may touch (0 = not checked)
+ *  STORAGE     yes     -        -        -       zhip_ir_scope            len
+ *  LOAD        -       src      index    -       0 scalar | vector len    -
+ *  STORE       -       dst      src      index   0 scalar | vector len    -
+ *  CAST        yes     x        -        -       -                        -
+ *  UNARY       -       x        -        -       zhip_ir_uop              -
+ *  BINARY      -       x        y        -       zhip_ir_bop              -
+ *  MAD         -       x        y        z       -                        -
+ *  STACK       -       first    count    -       -                        -      (operands = extra[first .. first+count))
+ *  DEVECTORIZE -       vec      -        -       lane                     -
+ *  INDEX       -       len op   -        -       axis | kind << 8         len for ZHIP_IR_IDX_LOCAL
+ *  LOOP        -       len op   -        -       -                        -
+ *  IF          -       cond     -        -       -                        -
+ *  ENDLOOP, ENDIF, BARRIER: no fields.
+ *
+ * Kernel arguments are the PARAM ops in list order (zyx/src/codegen/cuda.rs:24-37). Meaning of every op is
+ * the C backend's (zyx/src/codegen/c.rs:74-395, 583-612): bf16 / f16 values live in f32 registers, widen on
+ * load and truncate on store to global memory; register and local storage of those dtypes holds f32. */
+enum zhip_ir_opcode {
+    ZHIP_IR_CONST = 0, ZHIP_IR_PARAM, ZHIP_IR_STORAGE, ZHIP_IR_LOAD, ZHIP_IR_STORE, ZHIP_IR_CAST, ZHIP_IR_UNARY,
+    ZHIP_IR_BINARY, ZHIP_IR_MAD, ZHIP_IR_STACK, ZHIP_IR_DEVECTORIZE, ZHIP_IR_INDEX, ZHIP_IR_LOOP, ZHIP_IR_ENDLOOP,
+    ZHIP_IR_IF, ZHIP_IR_ENDIF, ZHIP_IR_BARRIER,
+    /* refused: */
+    ZHIP_IR_WMMA, ZHIP_IR_REDUCE_TILE, ZHIP_IR_MATMUL_TILE, ZHIP_IR_TRANSPOSE_TILE, ZHIP_IR_ASM, ZHIP_IR_MOVE, ZHIP_IR_REDUCE
+};
+/* ParamKind (ops.rs:11-19), MemScope (kernel/mod.rs:203-212), IdxKind (ops.rs:158-166) */
+enum zhip_ir_param_kind { ZHIP_IR_VARIABLE = 0, ZHIP_IR_GLOBAL = 1, ZHIP_IR_GLOBAL_MUT = 2 };
+enum zhip_ir_scope { ZHIP_IR_SCOPE_GLOBAL = 0, ZHIP_IR_SCOPE_LOCAL = 1, ZHIP_IR_SCOPE_REGISTER = 2, ZHIP_IR_SCOPE_CIRCULAR = 3 };
+enum zhip_ir_idx_kind { ZHIP_IR_IDX_GROUP = 0, ZHIP_IR_IDX_LOCAL = 1, ZHIP_IR_IDX_WARP = 2 };
+/* UOp (ops.rs:187-213) and BOp (ops.rs:221-260) discriminants */
+enum zhip_ir_uop {
+    ZHIP_IR_NEG = 0, ZHIP_IR_BITNOT, ZHIP_IR_EXP, ZHIP_IR_EXP2, ZHIP_IR_LN, ZHIP_IR_LOG2, ZHIP_IR_RECIPROCAL, ZHIP_IR_SQRT,
+    ZHIP_IR_SIN, ZHIP_IR_COS, ZHIP_IR_FLOOR, ZHIP_IR_TRUNC, ZHIP_IR_ABS
+};
+enum zhip_ir_bop {
+    ZHIP_IR_ADD = 0, ZHIP_IR_SUB, ZHIP_IR_MUL, ZHIP_IR_DIV, ZHIP_IR_POW, ZHIP_IR_MOD, ZHIP_IR_CMPLT, ZHIP_IR_CMPGT,
+    ZHIP_IR_CMPGE, ZHIP_IR_MAX, ZHIP_IR_OR, ZHIP_IR_AND, ZHIP_IR_BITXOR, ZHIP_IR_BITOR, ZHIP_IR_BITAND,
+    ZHIP_IR_SHL, ZHIP_IR_SHR, ZHIP_IR_NOTEQ, ZHIP_IR_EQ
+};
+#define ZHIP_IR_MAGIC 0x3152495au /* "ZIR1" */
+#define ZHIP_IR_NULL 0xffffffffu  /* OpId::NULL */
+#define ZHIP_IR_MAX_PARAMS 32
+typedef struct zhip_ir_header {
+    uint32_t magic, n_ops, n_extra, reserved;
+} zhip_ir_header;
+typedef struct zhip_ir_op {
+    uint32_t id;
+    uint16_t opcode; /* zhip_ir_opcode */
+    uint16_t dtype;  /* zhip_dtype where the table says so */
+    uint32_t a, b, c, aux;
+    uint64_t imm;
+} zhip_ir_op;
+
 /* --- backend lifetime ------------------------------------------------------- */
 
 /* Number of usable GPUs (device enumeration of hip.rs:190-215). */
@@ -320,10 +385,22 @@ int32_t zhip_buffer_ptr(zhip_ctx *ctx, zhip_buf buf, void **ptr, uint64_t *bytes
 /* AOT registration: validates desc and returns a program id, the role
  * `self.programs.push(..)` plays in CblasDevice::match_graph (cblas.rs:225). */
 int32_t zhip_register_kernel(zhip_ctx *ctx, const zhip_kernel_desc *desc, zhip_prog *prog);
-/* Device::compile for generic kernel IR (backend/mod.rs:899-933). This backend is
- * AOT-only (backend/mod.rs:892-894): always ZHIP_KERNEL_COMPILATION, the answer
- * CblasDevice::compile gives (cblas.rs:203-208). */
+/* Device::compile (backend/mod.rs:899-933; the HIP backend's own body is `todo!()`, hip.rs:598-646): turns a
+ * linearized kernel (image described above) into HIP source, the way generate_cuda does for CUDA
+ * (zyx/src/codegen/cuda.rs:18-396), and compiles it for this device with hiprtc. Grid = the Group index
+ * lengths (a constant, or a Variable parameter read at launch: GwsDim, backend/mod.rs:60-98), block = the
+ * Local index lengths. A launch takes one argument per PARAM, in order: a zhip_store_variable id for a
+ * Variable, a memory buffer otherwise. ZHIP_KERNEL_COMPILATION with the reason in zhip_last_error when the
+ * image is malformed, uses an op this backend has no code for, or does not compile. */
 int32_t zhip_compile_ir(zhip_ctx *ctx, const void *ir, uint64_t ir_bytes, zhip_prog *prog);
+/* Source generation alone, no device and no context needed: checks the image and writes the HIP source
+ * zhip_compile_ir would compile (ZHIP_OK), or the reason it is refused (ZHIP_KERNEL_COMPILATION), into buf
+ * (up to cap - 1 bytes plus a terminator; *len = full length). */
+int32_t zhip_ir_generate(const void *ir, uint64_t ir_bytes, char *buf, uint64_t cap, uint64_t *len);
+/* The HIP source zhip_compile_ir generated for `prog` (what ZYX_DEBUG=16 prints, hip.rs:560-580): copies up
+ * to cap - 1 bytes plus a terminator into buf, *len = full length. Programs registered with
+ * zhip_register_kernel have none (*len = 0). */
+int32_t zhip_program_source(zhip_ctx *ctx, zhip_prog prog, char *buf, uint64_t cap, uint64_t *len);
 /* HIPDevice::launch (hip.rs:654-719). args = inputs then outputs; every argument is
  * checked against the size the program needs before anything is enqueued. Consumes evs. */
 int32_t zhip_launch(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args, size_t n_args, const zhip_event *evs,

@@ -14,7 +14,7 @@ def test_device_info(hip):
     assert info.arch.startswith("gfx950")
     assert info.warp_size == 64 and info.tensor_cores and info.has_native_exp2
     assert info.max_local_threads == 1024 and info.preferred_vector_size == 16
-    assert dev.aot_only() and dev.memory_pool_id() == 0
+    assert not dev.aot_only() and dev.memory_pool_id() == 0
     assert dev.free_compute() > 10 * 2**40  # must outrank the C backend's weight (c.rs:120)
     assert pool.free_bytes() > 100 * 2**30
 
@@ -84,7 +84,7 @@ def test_events_are_consumed_once(hip):
     pool.deallocate(buf, [])
 
 
-def test_generic_ir_is_refused(hip):
+def test_malformed_ir_is_refused(hip):
     dev, pool = hip
     with pytest.raises(BackendError) as ei:
         dev.compile(b"\x00" * 16)

@@ -129,7 +129,8 @@ _lib = None
 _EXPORTS = ["zhip_device_count", "zhip_init", "zhip_deinit", "zhip_last_error", "zhip_get_device_info",
             "zhip_free_bytes", "zhip_free_compute", "zhip_alloc", "zhip_free", "zhip_store_variable",
             "zhip_get_variable", "zhip_h2d", "zhip_d2h", "zhip_d2d", "zhip_sync_events", "zhip_release_events",
-            "zhip_buffer_ptr", "zhip_register_kernel", "zhip_compile_ir", "zhip_launch", "zhip_release_program",
+            "zhip_buffer_ptr", "zhip_register_kernel", "zhip_compile_ir", "zhip_ir_generate", "zhip_program_source", "zhip_launch",
+            "zhip_release_program",
             "zhip_time_kernel", "zhip_profile_kernel", "zhip_plan_create", "zhip_plan_launch", "zhip_plan_destroy"]
 
 
@@ -318,14 +319,24 @@ class HIPDevice:
         return int(self._ctx.lib.zhip_free_compute(self._ctx.ptr))
 
     def aot_only(self) -> bool:
-        """backend/mod.rs:892-894"""
-        return True
+        """backend/mod.rs:892-894: false, the device also compiles linearized kernels."""
+        return False
 
     def compile(self, kernel_ir: bytes = b"", debug_asm: bool = False) -> int:
-        """Generic IR is refused with `KernelCompilation`, as CblasDevice::compile does (cblas.rs:203-208)."""
+        """Device::compile (backend/mod.rs:899-933) on the image of a linearized kernel (zyx_amd.ir.Kernel.to_bytes());
+        `KernelCompilation` when the image is malformed or holds an op the backend has no code for."""
         prog = C.c_uint32()
         self._ctx.check(self._ctx.lib.zhip_compile_ir(self._ctx.ptr, kernel_ir, C.c_uint64(len(kernel_ir)), C.byref(prog)))
+        if debug_asm:
+            print(self.program_source(prog.value))
         return prog.value
+
+    def program_source(self, program_id: int) -> str:
+        n = C.c_uint64()
+        self._ctx.check(self._ctx.lib.zhip_program_source(self._ctx.ptr, C.c_uint32(program_id), None, C.c_uint64(0), C.byref(n)))
+        buf = C.create_string_buffer(n.value + 1)
+        self._ctx.check(self._ctx.lib.zhip_program_source(self._ctx.ptr, C.c_uint32(program_id), buf, C.c_uint64(n.value + 1), C.byref(n)))
+        return buf.value.decode()
 
     def register_kernel(self, desc: KernelDesc) -> int:
         """AOT program registration: what `match_graph` does before pushing Node::Kernel (cblas.rs:225)."""
@@ -391,6 +402,19 @@ class HIPDevice:
 _NP_OF = {DType.BF16: np.uint16, DType.F16: np.float16, DType.F32: np.float32, DType.F64: np.float64,
           DType.U8: np.uint8, DType.U16: np.uint16, DType.U32: np.uint32, DType.U64: np.uint64, DType.I8: np.int8,
           DType.I16: np.int16, DType.I32: np.int32, DType.I64: np.int64, DType.Bool: np.bool_}
+
+
+def generate_source(kernel_ir: bytes) -> str:
+    """The HIP source `HIPDevice.compile` would build for this image; needs no GPU. `KernelCompilation` with the
+    reason when the image is refused."""
+    lib = load_library()
+    n = C.c_uint64()
+    lib.zhip_ir_generate(kernel_ir, C.c_uint64(len(kernel_ir)), None, C.c_uint64(0), C.byref(n))
+    buf = C.create_string_buffer(n.value + 1)
+    rc = lib.zhip_ir_generate(kernel_ir, C.c_uint64(len(kernel_ir)), buf, C.c_uint64(n.value + 1), C.byref(n))
+    if rc != 0:
+        raise BackendError(ErrorStatus(rc), buf.value.decode())
+    return buf.value.decode()
 
 
 def device_count() -> int:

@@ -29,6 +29,7 @@
 #include <string>
 #include <vector>
 
+#include "ir_compile.hpp"
 #include "kernels/kernels.hpp"
 
 #define ZHIP_EXPORT extern "C" __attribute__((visibility("default")))
@@ -36,6 +37,7 @@
 namespace {
 
 constexpr int kLaunchStreams = 8; // zyx/src/backend/hip.rs:242-274
+constexpr int kMaxArgs = ZHIP_IR_MAX_PARAMS; // arguments of one launch (hand-written kernels take at most 8)
 constexpr uint64_t kDefaultCacheBytes = 1ull << 30;
 constexpr uint64_t kAllocAlign = 256;
 
@@ -67,10 +69,11 @@ struct Program {
     bool live = false;
     zhip_kernel_desc desc{};
     int n_in = 0, n_out = 0;
-    uint64_t need[8] = {0}; // minimum bytes per argument
+    uint64_t need[kMaxArgs] = {0}; // minimum bytes per argument
     void *workspace = nullptr; // device scratch owned by the program (two-stage reductions)
     uint64_t workspace_bytes = 0;
     zk::EwJit *jit = nullptr;  // elementwise chains above the size threshold: code specialised at registration
+    zk::IrProgram *ir = nullptr; // compiled from a linearized kernel (zhip_compile_ir); desc.kind is 0 then
     // A program's workspace is shared by all its launches: each launch waits for the previous one's event on
     // whatever stream that ran, so two launches with unrelated wait lists never overlap on the scratch memory.
     hipEvent_t ws_event = nullptr;
@@ -599,6 +602,14 @@ int32_t program_fill_workspace(zhip_ctx *c, Program &p) {
 
 hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
     const zhip_kernel_desc &d = p.desc;
+    if (p.ir) {
+        // kernel parameters are passed by address: a buffer's is the slot holding its device pointer, a
+        // Variable's the bytes of its value (resolve_args left that address in the slot itself)
+        void *slots[kMaxArgs];
+        for (size_t i = 0; i < p.ir->params.size(); i++)
+            slots[i] = p.ir->params[i].kind == ZHIP_IR_VARIABLE ? ptr[i] : (void *)&ptr[i];
+        return zk::ir_launch(p.ir, slots, st, nullptr);
+    }
     switch (d.kind) {
     case ZHIP_K_SOFTMAX_ROWS: {
         zk::SoftmaxRows a{};
@@ -788,6 +799,15 @@ int32_t resolve_args(zhip_ctx *c, zhip_prog prog, const zhip_buf *args, size_t n
     for (size_t i = 0; i < n_args; i++) {
         Buffer *b = buffer_lookup(c, args[i]);
         if (!b) return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "argument %zu: buffer %u does not exist", i, args[i]);
+        if (p.ir && p.ir->params[i].kind == ZHIP_IR_VARIABLE) { // passed by value (cuda.rs:720-726)
+            if (b->kind != Buffer::Variable)
+                return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "argument %zu: buffer %u is memory, a scalar variable expected", i, args[i]);
+            if (b->var_dtype != p.ir->params[i].dtype)
+                return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "argument %zu: variable of dtype %d, the kernel takes dtype %d", i,
+                               b->var_dtype, p.ir->params[i].dtype);
+            ptr[i] = b->var_value;
+            continue;
+        }
         if (b->kind != Buffer::Memory)
             return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "argument %zu: buffer %u is a scalar variable, memory expected", i,
                            args[i]);
@@ -796,8 +816,9 @@ int32_t resolve_args(zhip_ctx *c, zhip_prog prog, const zhip_buf *args, size_t n
                            args[i], (unsigned long long)b->bytes, (unsigned long long)p.need[i]);
         ptr[i] = b->ptr;
     }
-    // an output must not alias an input or another output: the kernels assume restrict
-    for (size_t i = p.n_in; i < n_args; i++)
+    // an output must not alias an input or another output: the hand-written kernels assume restrict
+    // (generated kernels do not: zyx may hand one buffer to a kernel as source and destination)
+    for (size_t i = p.n_in; i < n_args && !p.ir; i++)
         for (size_t j = 0; j < i; j++)
             if (ptr[i] == ptr[j] && p.need[i] && p.need[j])
                 return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "arguments %zu and %zu are the same buffer", j, i);
@@ -943,6 +964,7 @@ ZHIP_EXPORT int32_t zhip_deinit(zhip_ctx *c) {
         for (Program &p : c->programs.items) {
             if (p.live && p.workspace) (void)hipFree(p.workspace);
             if (p.live && p.jit) zk::ew_jit_destroy(p.jit);
+            if (p.live && p.ir) zk::ir_destroy(p.ir);
             if (p.live && p.ws_event) (void)hipEventDestroy(p.ws_event);
         }
         for (EventSlot &s : c->events) (void)hipEventDestroy(s.ev);
@@ -1193,11 +1215,57 @@ ZHIP_EXPORT int32_t zhip_register_kernel(zhip_ctx *c, const zhip_kernel_desc *de
     return ZHIP_OK;
 }
 
-ZHIP_EXPORT int32_t zhip_compile_ir(zhip_ctx *c, const void *, uint64_t, zhip_prog *prog) {
+ZHIP_EXPORT int32_t zhip_compile_ir(zhip_ctx *c, const void *ir, uint64_t ir_bytes, zhip_prog *prog) {
     std::lock_guard<std::mutex> lk(c->mu);
-    if (prog) *prog = ZHIP_NULL_ID;
-    return c->fail(ZHIP_KERNEL_COMPILATION,
-                   "HIP device only runs its registered AOT kernels, it does not compile generic kernels.");
+    if (!prog) return c->fail(ZHIP_KERNEL_COMPILATION, "compile_ir: null out pointer");
+    *prog = ZHIP_NULL_ID;
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_COMPILATION);
+    std::string err;
+    zk::IrProgram *k = zk::ir_compile(ir, ir_bytes, err);
+    if (!k) return c->fail(ZHIP_KERNEL_COMPILATION, "%s", err.c_str());
+    if (c->debug & 16) fprintf(stderr, "[zyx-hip] generated kernel:\n%s\n", k->source.substr(k->source.find("extern \"C\"")).c_str());
+    Program p;
+    p.ir = k;
+    for (size_t i = 0; i < k->params.size(); i++) {
+        const zk::IrParam &q = k->params[i];
+        p.need[i] = q.kind == ZHIP_IR_VARIABLE ? 0 : q.elems * dtype_bytes(q.dtype);
+        if (q.kind == ZHIP_IR_GLOBAL_MUT) p.n_out++;
+        else p.n_in++;
+    }
+    p.live = true;
+    *prog = c->programs.push(p);
+    if (c->debug & 128) fprintf(stderr, "[zyx-hip] program %u = generated kernel, %zu parameters\n", *prog, k->params.size());
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_ir_generate(const void *ir, uint64_t ir_bytes, char *buf, uint64_t cap, uint64_t *len) {
+    zk::IrProgram k;
+    std::string err;
+    const bool ok = zk::ir_generate(ir, ir_bytes, k, err);
+    const std::string &text = ok ? k.source : err;
+    if (len) *len = text.size();
+    if (buf && cap) {
+        const size_t n = std::min<uint64_t>(cap - 1, text.size());
+        memcpy(buf, text.data(), n);
+        buf[n] = 0;
+    }
+    return ok ? ZHIP_OK : ZHIP_KERNEL_COMPILATION;
+}
+
+ZHIP_EXPORT int32_t zhip_program_source(zhip_ctx *c, zhip_prog prog, char *buf, uint64_t cap, uint64_t *len) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (prog >= c->programs.items.size() || !c->programs.items[prog].live)
+        return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "program %u does not exist", prog);
+    const Program &p = c->programs.items[prog];
+    const std::string empty;
+    const std::string &src = p.ir ? p.ir->source : empty;
+    if (len) *len = src.size();
+    if (buf && cap) {
+        const size_t n = std::min<uint64_t>(cap - 1, src.size());
+        memcpy(buf, src.data(), n);
+        buf[n] = 0;
+    }
+    return ZHIP_OK;
 }
 
 ZHIP_EXPORT int32_t zhip_release_program(zhip_ctx *c, zhip_prog prog) {
@@ -1214,6 +1282,12 @@ ZHIP_EXPORT int32_t zhip_release_program(zhip_ctx *c, zhip_prog prog) {
         (void)hipSetDevice(c->device);
         (void)hipFree(p.workspace);
         p.workspace = nullptr;
+    }
+    if (p.ir) {
+        (void)hipSetDevice(c->device);
+        (void)hipDeviceSynchronize(); // a launch of the module may still be running
+        zk::ir_destroy(p.ir);
+        p.ir = nullptr;
     }
     if (p.jit) {
         (void)hipSetDevice(c->device);
@@ -1232,7 +1306,7 @@ ZHIP_EXPORT int32_t zhip_launch(zhip_ctx *c, zhip_prog prog, const zhip_buf *arg
     if (!ev) return c->fail(ZHIP_KERNEL_LAUNCH, "zhip_launch: null event out pointer");
     *ev = 0;
     Program *p = nullptr;
-    void *ptr[8] = {nullptr};
+    void *ptr[kMaxArgs] = {nullptr};
     int32_t rc = resolve_args(c, prog, args, n_args, &p, ptr);
     if (rc != ZHIP_OK) { // nothing enqueued; the wait list is still consumed so no event leaks
         (void)hipSetDevice(c->device);
@@ -1256,7 +1330,7 @@ ZHIP_EXPORT int32_t zhip_time_kernel(zhip_ctx *c, zhip_prog prog, const zhip_buf
     std::lock_guard<std::mutex> lk(c->mu);
     if (!ns) return c->fail(ZHIP_KERNEL_LAUNCH, "zhip_time_kernel: null out pointer");
     Program *p = nullptr;
-    void *ptr[8] = {nullptr};
+    void *ptr[kMaxArgs] = {nullptr};
     int32_t rc = resolve_args(c, prog, args, n_args, &p, ptr);
     if (rc != ZHIP_OK) return rc;
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
@@ -1276,10 +1350,10 @@ ZHIP_EXPORT int32_t zhip_profile_kernel(zhip_ctx *c, zhip_prog prog, const zhip_
     std::lock_guard<std::mutex> lk(c->mu);
     if (!avg_us || iters <= 0 || arg_sets == 0 || arg_sets > 64)
         return c->fail(ZHIP_KERNEL_LAUNCH, "zhip_profile_kernel: bad argument");
-    std::vector<void *> ptrs(arg_sets * 8, nullptr);
+    std::vector<void *> ptrs(arg_sets * kMaxArgs, nullptr);
     Program *p = nullptr;
     for (size_t s = 0; s < arg_sets; s++) {
-        int32_t rc = resolve_args(c, prog, args + s * n_args, n_args, &p, &ptrs[s * 8]);
+        int32_t rc = resolve_args(c, prog, args + s * n_args, n_args, &p, &ptrs[s * kMaxArgs]);
         if (rc != ZHIP_OK) return rc;
     }
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
@@ -1288,7 +1362,7 @@ ZHIP_EXPORT int32_t zhip_profile_kernel(zhip_ctx *c, zhip_prog prog, const zhip_
     HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
     HIPCHK(c, hipEventRecord(c->prof_a, st), ZHIP_KERNEL_LAUNCH);
     for (int32_t i = 0; i < iters; i++) {
-        hipError_t e = program_enqueue(*p, &ptrs[(i % arg_sets) * 8], st);
+        hipError_t e = program_enqueue(*p, &ptrs[(i % arg_sets) * kMaxArgs], st);
         if (e != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "launch of program %u failed: %s", prog, hipGetErrorString(e));
     }
     HIPCHK(c, hipEventRecord(c->prof_b, st), ZHIP_KERNEL_LAUNCH);
@@ -1306,10 +1380,10 @@ ZHIP_EXPORT int32_t zhip_plan_create(zhip_ctx *c, const zhip_prog *progs, const 
     *plan = ZHIP_NULL_ID;
     // resolve every node before anything is captured: a bad node must not leave a capture open
     std::vector<Program *> ps(n_nodes);
-    std::vector<void *> ptrs(n_nodes * 8, nullptr);
+    std::vector<void *> ptrs(n_nodes * kMaxArgs, nullptr);
     size_t off = 0;
     for (size_t i = 0; i < n_nodes; i++) {
-        int32_t rc = resolve_args(c, progs[i], args_flat + off, n_args[i], &ps[i], &ptrs[i * 8]);
+        int32_t rc = resolve_args(c, progs[i], args_flat + off, n_args[i], &ps[i], &ptrs[i * kMaxArgs]);
         if (rc != ZHIP_OK) return rc;
         off += n_args[i];
     }
@@ -1317,7 +1391,7 @@ ZHIP_EXPORT int32_t zhip_plan_create(zhip_ctx *c, const zhip_prog *progs, const 
     HIPCHK(c, hipStreamSynchronize(c->plan_stream), ZHIP_KERNEL_SYNC);
     HIPCHK(c, hipStreamBeginCapture(c->plan_stream, hipStreamCaptureModeThreadLocal), ZHIP_KERNEL_COMPILATION);
     hipError_t bad = hipSuccess;
-    for (size_t i = 0; i < n_nodes && bad == hipSuccess; i++) bad = program_enqueue(*ps[i], &ptrs[i * 8], c->plan_stream);
+    for (size_t i = 0; i < n_nodes && bad == hipSuccess; i++) bad = program_enqueue(*ps[i], &ptrs[i * kMaxArgs], c->plan_stream);
     Plan pl;
     hipError_t e = hipStreamEndCapture(c->plan_stream, &pl.graph);
     if (bad != hipSuccess || e != hipSuccess) {
