@@ -172,6 +172,50 @@ def extra_streaming(dev, pool, kernels, steps=20, warmup=5):
     return out
 
 
+def extra_ir(dev, pool, kernels, steps=20, warmup=5):
+    """Kernels generated at run time from a linearized zyx kernel (Device::compile): the config-2 softmax rows written
+    as such a kernel (row in registers, local-memory reductions) beside the hand-written one, and an elementwise map."""
+    import zyx_amd
+    from zyx_amd import ir_examples
+    rng = np.random.default_rng(4)
+    out = {}
+    x = (rng.standard_normal((ROWS, COLS), dtype=np.float32) * 3.0).astype(np.float32)
+    sets, pending = [], []
+    for _ in range(N_SETS):  # rotating buffer sets, like the headline run: no launch finds its rows in the cache
+        xb, e1 = kernels.to_device(pool, x)
+        yb, e2 = kernels.alloc_like(pool, ROWS * COLS, 4)
+        sets.append([xb, yb])
+        pending += [e1, e2]
+    pool.sync_events(pending)
+
+    def timeit(name, prog, nbytes):
+        dev.profile_kernel(prog, sets, warmup)
+        us = dev.profile_kernel(prog, sets, steps)
+        out[name] = {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1), "frac_of_8TB/s": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+
+    import time
+    t0 = time.perf_counter()
+    prog = dev.compile(ir_examples.softmax_rows_local(ROWS, COLS).to_bytes())
+    out["compile_ms_softmax"] = round((time.perf_counter() - t0) * 1e3, 1)
+    timeit(f"generated_softmax_f32_{ROWS}x{COLS}", prog, 2 * ROWS * COLS * 4)
+    y = kernels.to_host(pool, sets[0][1], (ROWS, COLS), np.float32)
+    e = np.exp(x[:8].astype(np.float64) - x[:8].max(1, keepdims=True))
+    assert np.allclose(y[:8], e / e.sum(1, keepdims=True), rtol=1e-5, atol=1e-37), "generated softmax is wrong"
+    dev.release(prog)
+    hand = dev.register_kernel(kernels.softmax_rows_desc(ROWS, COLS, True, False, False))
+    timeit(f"handwritten_softmax_f32_{ROWS}x{COLS}", hand, 2 * ROWS * COLS * 4)
+    dev.release(hand)
+    for dt, isz, tag in ((zyx_amd.DType.F32, 4, "f32"), (zyx_amd.DType.BF16, 2, "bf16")):
+        n = ROWS * COLS
+        prog = dev.compile(ir_examples.scaled_exp2(n, dt, vlen=4 if isz == 4 else 8).to_bytes())
+        timeit(f"generated_exp2_scale_{tag}_{n}", prog, 2 * n * isz)
+        dev.release(prog)
+    for st in sets:
+        for b in st:
+            pool.deallocate(b, [])
+    return out
+
+
 def extra_attention(dev, pool, kernels, steps=30, warmup=10):
     """Config 5's attention core alone: B=8, T=1024, 16 heads x 64, bf16. FLOPs: 4*B*H*T*T*dh forward (QK^T, PV),
     10*B*H*T*T*dh backward (5 products; the two-kernel backward recomputes QK^T and dy.V^T, not counted)."""
@@ -312,6 +356,7 @@ def main():
     ap.add_argument("--mlp-only", action="store_true", help="run only the config-1 MLP training leg")
     ap.add_argument("--streaming-only", action="store_true", help="run only the memory-bound kernel leg")
     ap.add_argument("--attention-only", action="store_true", help="run only the attention core leg")
+    ap.add_argument("--ir-only", action="store_true", help="run only the generated-kernel leg")
     ap.add_argument("--counters", action="store_true",
                     help="short run for `rocprofv3 --pmc`: a few launches of the fused kernel and of a plain copy "
                          "kernel over the same 8192x4096 f32 tensor (known traffic: 134217728 B read + written), "
@@ -333,7 +378,7 @@ def main():
         pool.deinitialize()
         return
 
-    if args.conv_only or args.block_only or args.streaming_only or args.attention_only or args.mlp_only:
+    if args.conv_only or args.block_only or args.streaming_only or args.attention_only or args.mlp_only or args.ir_only:
         if args.mlp_only:
             res = {"config1_mlp_train": extra_mlp(dev, pool, cpu=not args.no_cpu)}
         elif args.conv_only:
@@ -342,6 +387,8 @@ def main():
             res = {"memory_bound_kernels": extra_streaming(dev, pool, kernels)}
         elif args.attention_only:
             res = {"config5_attention_core": extra_attention(dev, pool, kernels)}
+        elif args.ir_only:
+            res = {"generated_kernels": extra_ir(dev, pool, kernels)}
         else:
             res = {"config5_transformer_block": extra_block(dev, pool, steps=args.steps if args.steps != 200 else 20, cpu=not args.no_cpu)}
         print(json.dumps(res))
@@ -427,7 +474,8 @@ def main():
                         "config4_conv_relu_pool": extra_conv(dev, pool, kernels),
                         "config5_attention_core": extra_attention(dev, pool, kernels),
                         "config5_transformer_block": extra_block(dev, pool, cpu=not args.no_cpu),
-                        "memory_bound_kernels": extra_streaming(dev, pool, kernels)}
+                        "memory_bound_kernels": extra_streaming(dev, pool, kernels),
+                        "generated_kernels": extra_ir(dev, pool, kernels)}
     pool.deinitialize()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(x)

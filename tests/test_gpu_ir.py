@@ -260,3 +260,31 @@ def test_generated_kernels_in_plans_and_errors(hip, oracle):
     with pytest.raises(BackendError) as e:
         dev.compile(b"\x00" * 16)
     assert e.value.status == ErrorStatus.KernelCompilation
+
+
+def test_optimised_example_kernels(hip, oracle):
+    """The benchmark's generated kernels: parity with the interpreter at a small size, and at the benchmark's size
+    against the double-precision rows and the invariants (rows sum to 1, argmax preserved)."""
+    from zyx_amd import ir_examples
+    dev, pool = hip
+    x = (3 * oracle.Rng(21).randn((16, 1024))).astype(np.float32)
+    (g, c), = both(hip, ir_examples.softmax_rows_local(16, 1024, 64, 4), [x, np.zeros_like(x)])
+    assert np.allclose(g, c, rtol=1e-5, atol=1e-37)
+    x = (3 * oracle.Rng(22).randn((8192, 4096))).astype(np.float32)
+    prog = dev.compile(ir_examples.softmax_rows_local(8192, 4096).to_bytes())
+    xb, e1 = to_device(pool, x)
+    yb, e2 = pool.allocate(x.nbytes)
+    y = to_host(pool, yb, x.shape, np.float32, [dev.launch(prog, pool, [xb, yb], [e1, e2])])
+    y64, _ = oracle.softmax_rows_f64acc(x)
+    assert np.allclose(y, y64, rtol=1e-5, atol=1e-37)
+    assert np.allclose(y.sum(axis=1, dtype=np.float64), 1.0, atol=1e-5) and np.array_equal(y.argmax(1), x.argmax(1))
+    dev.release(prog)
+    for b in (xb, yb):
+        pool.deallocate(b, [])
+    for dt, vlen in ((DType.F32, 4), (DType.BF16, 8)):
+        n = 1 << 16
+        v = oracle.Rng(23).uniform(n, -4, 4)
+        arr = v if dt == DType.F32 else oracle.f32_to_bf16(v)
+        (g, c), = both(hip, ir_examples.scaled_exp2(n, dt, vlen=vlen), [arr, np.zeros_like(arr)])
+        gf, cf = (g, c) if dt == DType.F32 else (oracle.bf16_to_f32(g), oracle.bf16_to_f32(c))
+        assert np.all(np.abs(gf - cf) <= (1e-5 if dt == DType.F32 else 2.0 ** -7) * np.abs(cf))
