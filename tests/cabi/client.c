@@ -31,6 +31,11 @@ static int layout(void) {
     printf("kinds %d %d %d %d %d %d %d %d %d %d %d %d\n", ZHIP_K_SOFTMAX_ROWS, ZHIP_K_ELEMENTWISE, ZHIP_K_REDUCE, ZHIP_K_GEMM,
            ZHIP_K_NORM_ROWS, ZHIP_K_CROSS_ENTROPY, ZHIP_K_CONV2D, ZHIP_K_MAX_POOL2D, ZHIP_K_INDEX, ZHIP_K_ATTENTION,
            ZHIP_K_ATTENTION_BWD, ZHIP_K_NORM_ROWS_BWD);
+    printf("zhip_ir_op %zu id %zu opcode %zu dtype %zu a %zu b %zu c %zu aux %zu imm %zu\n", sizeof(zhip_ir_op), offsetof(zhip_ir_op, id),
+           offsetof(zhip_ir_op, opcode), offsetof(zhip_ir_op, dtype), offsetof(zhip_ir_op, a), offsetof(zhip_ir_op, b),
+           offsetof(zhip_ir_op, c), offsetof(zhip_ir_op, aux), offsetof(zhip_ir_op, imm));
+    printf("ir %zu %u %d %d %d %d %d %d\n", sizeof(zhip_ir_header), ZHIP_IR_MAGIC, ZHIP_IR_BARRIER, ZHIP_IR_REDUCE, ZHIP_IR_ABS, ZHIP_IR_EQ,
+           ZHIP_IR_GLOBAL_MUT, ZHIP_IR_SCOPE_REGISTER);
     return 0;
 }
 

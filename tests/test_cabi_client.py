@@ -35,6 +35,12 @@ def test_header_is_c_and_layouts_match_the_python_mirror(client):
     from zyx_amd import kernels as K
     assert [int(v) for v in out[3].split()[1:]] == [K.K_SOFTMAX_ROWS, K.K_ELEMENTWISE, K.K_REDUCE, K.K_GEMM, K.K_NORM_ROWS, K.K_CROSS_ENTROPY,
                                                     K.K_CONV2D, K.K_MAX_POOL2D, K.K_INDEX, K.K_ATTENTION, K.K_ATTENTION_BWD, K.K_NORM_ROWS_BWD]
+    from zyx_amd import ir
+    op = out[4].split()
+    assert op[0] == "zhip_ir_op" and int(op[1]) == ctypes.sizeof(ir.IrOp) == 32
+    assert {op[i]: int(op[i + 1]) for i in range(2, len(op), 2)} == {f[0]: getattr(ir.IrOp, f[0]).offset for f in ir.IrOp._fields_}
+    assert [int(v) for v in out[5].split()[1:]] == [ctypes.sizeof(ir.IrHeader), ir.MAGIC, ir.Opcode.BARRIER, ir.Opcode.REDUCE, ir.UOp.Abs,
+                                                    ir.BOp.Eq, ir.ParamKind.GlobalMut, ir.MemScope.Register]
 
 
 @pytest.mark.gpu
