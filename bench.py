@@ -231,15 +231,18 @@ def extra_attention(dev, pool, kernels, steps=30, warmup=10):
     lb, e3 = kernels.alloc_like(pool, B * H * T, 4)
     gb, e4 = kernels.alloc_like(pool, B * T * 3 * H * DH, 2)
     pool.sync_events([e0, e1, e2, e3, e4])
-    fwd = dev.register_kernel(kernels.attention_desc(B, T, H, DH, zyx_amd.DType.BF16, lse=True))
-    bwd = dev.register_kernel(kernels.attention_bwd_desc(B, T, H, DH, zyx_amd.DType.BF16))
     res = {}
-    for name, prog, args, flop in (("forward", fwd, [xb, yb, lb], 4.0 * B * H * T * T * DH), ("backward", bwd, [xb, yb, db, lb, gb], 10.0 * B * H * T * T * DH)):
-        dev.profile_kernel(prog, [args], warmup)
-        us = dev.profile_kernel(prog, [args], steps)
-        res[name] = {"us": round(us, 2), "TFLOP/s": round(flop / us / 1e6, 1), "frac_of_2.5PF_bf16_peak": round(flop / us / 1e6 / 2500.0, 4)}
-    dev.release(fwd)
-    dev.release(bwd)
+    # causal: the T(T+1)/2 visible (query, key) pairs are what is counted
+    for tag, causal, pairs in (("", False, float(T) * T), ("causal_", True, T * (T + 1) / 2.0)):
+        fwd = dev.register_kernel(kernels.attention_desc(B, T, H, DH, zyx_amd.DType.BF16, lse=True, causal=causal))
+        bwd = dev.register_kernel(kernels.attention_bwd_desc(B, T, H, DH, zyx_amd.DType.BF16, causal=causal))
+        for name, prog, args, flop in ((tag + "forward", fwd, [xb, yb, lb], 4.0 * B * H * pairs * DH),
+                                       (tag + "backward", bwd, [xb, yb, db, lb, gb], 10.0 * B * H * pairs * DH)):
+            dev.profile_kernel(prog, [args], warmup)
+            us = dev.profile_kernel(prog, [args], steps)
+            res[name] = {"us": round(us, 2), "TFLOP/s": round(flop / us / 1e6, 1), "frac_of_2.5PF_bf16_peak": round(flop / us / 1e6 / 2500.0, 4)}
+        dev.release(fwd)
+        dev.release(bwd)
     for b_ in (xb, db, yb, lb, gb):
         pool.deallocate(b_, [])
     return res

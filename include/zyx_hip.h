@@ -184,13 +184,16 @@ enum zhip_kernel_kind {
      * applies no mask, so none is applied. dims = {B, T, H, dh}; dtype BF16 or F32 (storage of qkv
      * and y, f32 arithmetic); fparams[0] = scale (0 selects 1/sqrt(dh)), fparams[1] = dropout p;
      * flags: ZHIP_ATTN_LSE also writes lse[B, H, T] (f32) = ln sum_j exp(scale q.k_j), which the
-     * backward needs. args: qkv, y[B, T, C], (lse). */
+     * backward needs; ZHIP_ATTN_CAUSAL: query t attends to keys 0..t only, what a lower-triangular
+     * mask filled with -inf before the softmax gives (the reference's module has no such mask; the
+     * flag serves models that add one). args: qkv, y[B, T, C], (lse). */
     ZHIP_K_ATTENTION = 10,
     /* Gradient of ZHIP_K_ATTENTION with respect to qkv: what Runtime::gradient
      * (zyx/src/graph/autograd.rs:14-424) builds from the reverse rules of the forward's ops (Mul :120-125,
      * Div :126-134, Exp :87-95, Sub :111-119, the reduce rules :299-379), evaluated in one pass:
      * dV = P^T.dy, dS = Ps o (dy.v^T / (1-p) - rowsum(dy o y)), dQ = scale dS.k, dK = scale dS^T.q, with the
-     * probabilities recomputed from lse. dims, dtype, fparams as for ZHIP_K_ATTENTION.
+     * probabilities recomputed from lse. dims, dtype, fparams as for ZHIP_K_ATTENTION; flags: ZHIP_ATTN_CAUSAL
+     * as in the forward (masked probabilities and their gradients are 0).
      * args: qkv, y, dy[B, T, C], lse[B, H, T] (the forward's inputs and outputs), then dqkv[B, T, 3*C]. */
     ZHIP_K_ATTENTION_BWD = 11,
     /* Gradients of ZHIP_K_NORM_ROWS (LayerNorm zyx-nn/src/layer_norm.rs:98-135, RMSNorm rms_norm.rs:26-32)
@@ -217,6 +220,7 @@ enum zhip_kernel_kind {
 #define ZHIP_INDEX_SELECT 1
 #define ZHIP_INDEX_SCATTER 2
 #define ZHIP_ATTN_LSE 1
+#define ZHIP_ATTN_CAUSAL 2
 #define ZHIP_GEMM_TRANS_A 1
 #define ZHIP_GEMM_TRANS_B 2
 

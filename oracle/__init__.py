@@ -383,9 +383,10 @@ def scatter(x: np.ndarray, axis: int, indices: np.ndarray, src: np.ndarray) -> n
 
 # ---- attention: zyx-nn/src/causal_self_attention.rs:36-74 ----------------------------------------------------
 def attention(qkv: np.ndarray, n_head: int, scale: float | None = None, dropout_p: float = 0.0, dtype: int = F32,
-              want_lse: bool = False):
+              want_lse: bool = False, causal: bool = False):
     """Core of CausalSelfAttention::forward on the c_attn output qkv[B,T,3C] -> y[B,T,C] (the reference applies
-    no mask). scale defaults to (1/sqrt(dh)) as f32; eval-mode dropout divides the probabilities by 1-p."""
+    no mask). scale defaults to (1/sqrt(dh)) as f32; eval-mode dropout divides the probabilities by 1-p.
+    causal: query t sees keys 0..t only (scores of later keys filled with -inf before the softmax)."""
     qkv = np.ascontiguousarray(qkv, _store_dtype(dtype))
     b, t, c3 = qkv.shape
     c = c3 // 3
@@ -394,12 +395,12 @@ def attention(qkv: np.ndarray, n_head: int, scale: float | None = None, dropout_
     y = np.empty((b, t, c), qkv.dtype)
     lse = np.empty((b, n_head, t), np.float32) if want_lse else None
     lib().zo_attention(dtype, _p(qkv), _p(y), _p(lse), _I64(b), _I64(t), _I64(n_head), _I64(dh), C.c_float(scale),
-                       C.c_float(np.float32(1.0) - np.float32(dropout_p)))
+                       C.c_float(np.float32(1.0) - np.float32(dropout_p)), C.c_int(int(causal)))
     return (y, lse) if want_lse else y
 
 
 def attention_bwd(qkv: np.ndarray, dy: np.ndarray, n_head: int, scale: float | None = None, dropout_p: float = 0.0,
-                  dtype: int = F32) -> np.ndarray:
+                  dtype: int = F32, causal: bool = False) -> np.ndarray:
     """d(sum(y * dy)) / d(qkv) for `attention`, f64 arithmetic, stored in `dtype`."""
     qkv = np.ascontiguousarray(qkv, _store_dtype(dtype))
     dy = np.ascontiguousarray(dy, qkv.dtype)
@@ -408,7 +409,7 @@ def attention_bwd(qkv: np.ndarray, dy: np.ndarray, n_head: int, scale: float | N
     scale = np.float32(1.0 / np.sqrt(float(dh))) if scale is None else np.float32(scale)
     out = np.empty_like(qkv)
     lib().zo_attention_bwd(dtype, _p(qkv), _p(dy), _p(out), _I64(b), _I64(t), _I64(n_head), _I64(dh), C.c_float(scale),
-                           C.c_float(np.float32(1.0) - np.float32(dropout_p)))
+                           C.c_float(np.float32(1.0) - np.float32(dropout_p)), C.c_int(int(causal)))
     return out
 
 
@@ -455,7 +456,7 @@ def _gelu64(v):
     return 0.5 * v * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (v + 0.044715 * v ** 3)))
 
 
-def block_forward_f64(p: dict, x: np.ndarray, n_head: int, eps: float = 1e-5) -> dict:
+def block_forward_f64(p: dict, x: np.ndarray, n_head: int, eps: float = 1e-5, causal: bool = False) -> dict:
     """x[B,T,d] -> every module output of `x + attn(ln_1(x)); x + mlp(ln_2(x))` in f64 (numpy). LayerNorm uses the
     unbiased variance (zyx-nn/src/layer_norm.rs:98-135), attention applies no mask
     (zyx-nn/src/causal_self_attention.rs:36-74), gelu is the tanh form (zyx/src/tensor/elementwise.rs:168-170)."""
@@ -473,6 +474,8 @@ def block_forward_f64(p: dict, x: np.ndarray, n_head: int, eps: float = 1e-5) ->
     s["qkv"] = s["n1"] @ f["attn_w"].T + f["attn_b"]
     q, k, v = [a.reshape(B, T, n_head, dh).transpose(0, 2, 1, 3) for a in np.split(s["qkv"], 3, axis=2)]
     sc = np.einsum("bhtd,bhjd->bhtj", q, k) * float(np.float32(1.0 / np.sqrt(float(dh))))
+    if causal:  # not part of the reference's module: scores of later keys filled with -inf (probability 0)
+        sc = np.where(np.tril(np.ones((T, T), bool)), sc, -np.inf)
     e = np.exp(sc - sc.max(-1, keepdims=True))
     s["probs"] = e / e.sum(-1, keepdims=True)
     s["att"] = np.einsum("bhtj,bhjd->bhtd", s["probs"], v).transpose(0, 2, 1, 3).reshape(B, T, d)

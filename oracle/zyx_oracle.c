@@ -751,7 +751,7 @@ ZO_API void zo_max_pool2d(int dtype, const void *x, void *y, int64_t planes, int
  * (att / (1-p), zyx/src/tensor/mod.rs:822-828), att.dot(v), transpose(1,2).reshape([b,t,c]).
  * f32 registers, serial sums, one narrowing store for y. lse (optional) = max + ln(sum). */
 ZO_API void zo_attention(int dtype, const void *qkv, void *y, float *lse, int64_t B, int64_t T, int64_t H, int64_t dh,
-                         float scale, float keep) {
+                         float scale, float keep, int causal) {
     const int64_t Cc = H * dh, ld = 3 * Cc;
 #pragma omp parallel
     {
@@ -761,23 +761,24 @@ ZO_API void zo_attention(int dtype, const void *qkv, void *y, float *lse, int64_
             for (int64_t t = 0; t < T; t++) {
                 const int64_t b = bh / H, h = bh % H;
                 const int64_t qo = (b * T + t) * ld + h * dh;
-                for (int64_t j = 0; j < T; j++) {
+                const int64_t n = causal ? t + 1 : T; /* a query sees keys 0..t: the rest are filled with -inf, exp gives 0 */
+                for (int64_t j = 0; j < n; j++) {
                     const int64_t ko = (b * T + j) * ld + Cc + h * dh;
                     float a = 0.0f;
                     for (int64_t d = 0; d < dh; d++) a = load_as_f32(qkv, dtype, qo + d) * load_as_f32(qkv, dtype, ko + d) + a;
                     s[j] = a * scale;
                 }
                 float m = s[0];
-                for (int64_t j = 1; j < T; j++) m = fmaxf(m, s[j]);
+                for (int64_t j = 1; j < n; j++) m = fmaxf(m, s[j]);
                 float sum = 0.0f;
-                for (int64_t j = 0; j < T; j++) {
+                for (int64_t j = 0; j < n; j++) {
                     s[j] = expf(s[j] - m);
                     sum = s[j] + sum;
                 }
-                for (int64_t j = 0; j < T; j++) s[j] = (s[j] / sum) / keep;
+                for (int64_t j = 0; j < n; j++) s[j] = (s[j] / sum) / keep;
                 for (int64_t d = 0; d < dh; d++) {
                     float a = 0.0f;
-                    for (int64_t j = 0; j < T; j++) a = s[j] * load_as_f32(qkv, dtype, (b * T + j) * ld + 2 * Cc + h * dh + d) + a;
+                    for (int64_t j = 0; j < n; j++) a = s[j] * load_as_f32(qkv, dtype, (b * T + j) * ld + 2 * Cc + h * dh + d) + a;
                     store_from_f32(y, dtype, (b * T + t) * Cc + h * dh + d, a);
                 }
                 if (lse) lse[bh * T + t] = m + logf(sum);
@@ -791,7 +792,7 @@ ZO_API void zo_attention(int dtype, const void *qkv, void *y, float *lse, int64_
  * P = softmax(scale q k^T) / keep; dV = P^T dO; dP = dO V^T / keep; dS = Ps o (dP - rowsum(Ps o dP)),
  * Ps = softmax; dQ = scale dS K; dK = scale dS^T Q. Accumulated in f64, stored in `dtype`. */
 ZO_API void zo_attention_bwd(int dtype, const void *qkv, const void *dy, void *dqkv, int64_t B, int64_t T, int64_t H,
-                             int64_t dh, float scale, float keep) {
+                             int64_t dh, float scale, float keep, int causal) {
     const int64_t Cc = H * dh, ld = 3 * Cc;
 #pragma omp parallel for
     for (int64_t bh = 0; bh < B * H; bh++) {
@@ -801,19 +802,21 @@ ZO_API void zo_attention_bwd(int dtype, const void *qkv, const void *dy, void *d
         for (int64_t t = 0; t < T; t++) {
             const int64_t qo = (b * T + t) * ld + h * dh;
             double m = -INFINITY, sum = 0.0;
-            for (int64_t j = 0; j < T; j++) {
+            const int64_t n = causal ? t + 1 : T;
+            for (int64_t j = n; j < T; j++) P[t * T + j] = dS[t * T + j] = 0.0; /* masked: probability and its gradient are 0 */
+            for (int64_t j = 0; j < n; j++) {
                 const int64_t ko = (b * T + j) * ld + Cc + h * dh;
                 double a = 0.0;
                 for (int64_t d = 0; d < dh; d++) a += (double)load_as_f32(qkv, dtype, qo + d) * (double)load_as_f32(qkv, dtype, ko + d);
                 P[t * T + j] = a * (double)scale;
                 if (P[t * T + j] > m) m = P[t * T + j];
             }
-            for (int64_t j = 0; j < T; j++) {
+            for (int64_t j = 0; j < n; j++) {
                 P[t * T + j] = exp(P[t * T + j] - m);
                 sum += P[t * T + j];
             }
             double dot = 0.0;
-            for (int64_t j = 0; j < T; j++) {
+            for (int64_t j = 0; j < n; j++) {
                 P[t * T + j] /= sum;
                 double dp = 0.0;
                 for (int64_t d = 0; d < dh; d++)
@@ -822,7 +825,7 @@ ZO_API void zo_attention_bwd(int dtype, const void *qkv, const void *dy, void *d
                 dS[t * T + j] = dp / (double)keep;
                 dot += P[t * T + j] * dS[t * T + j];
             }
-            for (int64_t j = 0; j < T; j++) dS[t * T + j] = P[t * T + j] * (dS[t * T + j] - dot);
+            for (int64_t j = 0; j < n; j++) dS[t * T + j] = P[t * T + j] * (dS[t * T + j] - dot);
         }
         for (int64_t t = 0; t < T; t++)
             for (int64_t d = 0; d < dh; d++) {

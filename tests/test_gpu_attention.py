@@ -14,11 +14,13 @@ from zyx_amd.kernels import attention
 pytestmark = pytest.mark.gpu
 
 
-def sdpa64(qkv, n_head, scale=None, p=0.0):
+def sdpa64(qkv, n_head, scale=None, p=0.0, causal=False):
     b, t, c3 = qkv.shape
     dh = c3 // 3 // n_head
     q, k, v = [a.reshape(b, t, n_head, dh).transpose(0, 2, 1, 3) for a in np.split(qkv.astype(np.float64), 3, axis=2)]
     s = np.einsum("bhtd,bhjd->bhtj", q, k) * float(np.float32(1 / np.sqrt(dh)) if scale is None else scale)
+    if causal:
+        s = np.where(np.tril(np.ones((t, t), bool)), s, -np.inf)  # masked_fill(-inf) above the diagonal
     m = s.max(-1, keepdims=True)
     e = np.exp(s - m)
     pr = e / e.sum(-1, keepdims=True) / (1.0 - p)
@@ -116,14 +118,18 @@ def test_config5_attention_full_size(hip, oracle):
 from zyx_amd.kernels import attention_bwd
 
 
-def grad64(qkv, dy, n_head, p=0.0):
-    """Textbook gradient in f64 (numpy), with the magnitude sums the tolerances are relative to."""
+def grad64(qkv, dy, n_head, p=0.0, causal=False, with_ymag=False):
+    """Textbook gradient in f64 (numpy), with the magnitude sums the tolerances are relative to. with_ymag also
+    returns how far one unit of relative error in every stored y element moves dq and dk: the backward reads y as
+    the forward stored it (D = rowsum(dy o y)), so a bf16 y brings 2^-7 of sum_d |dy_d y_d| into every dS of its row."""
     b, t, c3 = qkv.shape
     dh = c3 // 3 // n_head
     sc = float(np.float32(1 / np.sqrt(dh)))
     q, k, v = [a.reshape(b, t, n_head, dh).transpose(0, 2, 1, 3) for a in np.split(qkv.astype(np.float64), 3, axis=2)]
     do = dy.astype(np.float64).reshape(b, t, n_head, dh).transpose(0, 2, 1, 3)
     s = np.einsum("bhtd,bhjd->bhtj", q, k) * sc
+    if causal:
+        s = np.where(np.tril(np.ones((t, t), bool)), s, -np.inf)
     e = np.exp(s - s.max(-1, keepdims=True))
     ps = e / e.sum(-1, keepdims=True)
     dps = np.einsum("bhtd,bhjd->bhtj", do, v) / (1 - p)
@@ -134,6 +140,12 @@ def grad64(qkv, dy, n_head, p=0.0):
                         back(np.einsum("bhtj,bhtd->bhjd", ps, do) / (1 - p))], 2)
     mag = np.concatenate([back(np.einsum("bhtj,bhjd->bhtd", ads, np.abs(k)) * sc), back(np.einsum("bhtj,bhtd->bhjd", ads, np.abs(q)) * sc),
                           back(np.einsum("bhtj,bhtd->bhjd", ps, np.abs(do)) / (1 - p))], 2)
+    if with_ymag:
+        y = np.einsum("bhtj,bhjd->bhtd", ps, v) / (1 - p)
+        ey = ps * (np.abs(do) * np.abs(y)).sum(-1, keepdims=True)
+        zeros = np.zeros((b, t, n_head * dh))
+        ymag = np.concatenate([back(np.einsum("bhtj,bhjd->bhtd", ey, np.abs(k)) * sc), back(np.einsum("bhtj,bhtd->bhjd", ey, np.abs(q)) * sc), zeros], 2)
+        return g, mag, ymag
     return g, mag
 
 
@@ -190,3 +202,52 @@ def test_config5_attention_backward_full_size(hip, oracle):
         want, mag = grad64(oracle.bf16_to_f32(sub), oracle.bf16_to_f32(dsub), 1)
         g = got[bsel:bsel + 1][:, :, cols].astype(np.float64)
         assert np.all(np.abs(g - want) <= 2.0 ** -7 * np.abs(want) + (1e-3 + 2.0 ** -8) * mag)
+
+
+# ---- causal mask --------------------------------------------------------------------------------------------------
+# The reference's module applies no mask (zyx-nn/src/causal_self_attention.rs:57-62); the flag is checked against the
+# textbook masked softmax in f64 and against the oracle's serial loops over the keys 0..t.
+
+@pytest.mark.parametrize("shape", [(1, 3, 2, 2), (2, 7, 3, 5), (1, 64, 1, 64), (2, 65, 2, 80), (1, 200, 2, 130), (3, 129, 4, 16)])
+@pytest.mark.parametrize("p", [0.0, 0.25])
+def test_causal_small_kernel_f32(hip, oracle, shape, p):
+    dev, pool = hip
+    b, t, h, dh = shape
+    qkv = oracle.Rng(t + dh).randn((b, t, 3 * h * dh))
+    y, lse = attention(dev, pool, qkv, h, DType.F32, dropout_p=p, want_lse=True, causal=True)
+    want, mag, lse64 = sdpa64(qkv, h, p=p, causal=True)
+    assert np.all(np.abs(y - want) <= 1e-5 * np.maximum(np.abs(want), mag) + 1e-7)
+    assert np.allclose(lse, lse64, rtol=1e-5, atol=1e-5)
+    ref = oracle.attention(qkv, h, dropout_p=p, causal=True)
+    assert np.all(np.abs(y - ref) <= 2e-5 * np.maximum(np.abs(want), mag) + 1e-7)
+    # the first query sees one key: its row is v_0 / keep exactly
+    v0 = qkv[:, 0, 2 * h * dh:]
+    assert np.allclose(y[:, 0], v0 / (np.float32(1) - np.float32(p)), rtol=1e-6, atol=0)
+    dy = oracle.Rng(t).randn((b, t, h * dh))
+    got = attention_bwd(dev, pool, qkv, y, dy, lse, h, DType.F32, dropout_p=p, causal=True)
+    keep = float(np.float32(1) - np.float32(p))
+    gwant, gmag = grad64(qkv, dy, h, 1 - keep, causal=True)
+    assert np.all(np.abs(got - gwant) <= 2e-5 * gmag + 1e-7)
+    assert np.all(np.abs(got - oracle.attention_bwd(qkv, dy, h, dropout_p=p, causal=True)) <= 2e-5 * gmag + 1e-7)
+
+
+@pytest.mark.parametrize("shape", [(1, 128, 1, 64), (2, 256, 3, 64), (1, 1024, 2, 64), (8, 384, 8, 64)])
+def test_causal_mfma_kernels_bf16(hip, oracle, shape):
+    dev, pool = hip
+    b, t, h, dh = shape
+    qkv = oracle.f32_to_bf16(oracle.Rng(t + b).randn((b, t, 3 * h * dh)))
+    dy = oracle.f32_to_bf16(oracle.Rng(t).randn((b, t, h * dh)))
+    y, lse = attention(dev, pool, qkv, h, DType.BF16, want_lse=True, causal=True)
+    want, mag, lse64 = sdpa64(oracle.bf16_to_f32(qkv), h, causal=True)
+    assert np.all(bf16_close(oracle, y, want, mag))
+    assert np.allclose(lse, lse64, rtol=1e-4, atol=1e-4)
+    assert np.array_equal(y[:, 0], qkv[:, 0, 2 * h * dh:])         # one visible key: y_0 = v_0, bit for bit
+    y_nolse = attention(dev, pool, qkv, h, DType.BF16, causal=True)
+    assert np.array_equal(y_nolse, y)
+    got = oracle.bf16_to_f32(attention_bwd(dev, pool, qkv, y, dy, lse, h, DType.BF16, causal=True)).astype(np.float64)
+    # early queries see few keys: their y is as large as v, and its truncating bf16 store is felt in D = rowsum(dy o y)
+    gwant, gmag, ymag = grad64(oracle.bf16_to_f32(qkv), oracle.bf16_to_f32(dy), h, causal=True, with_ymag=True)
+    assert np.all(np.abs(got - gwant) <= 2.0 ** -7 * np.abs(gwant) + (1e-3 + 2.0 ** -8) * gmag + 2.0 ** -7 * ymag)
+    if t <= 256:
+        ref = oracle.bf16_to_f32(oracle.attention(qkv, h, dtype=oracle.BF16, causal=True)).astype(np.float64)
+        assert np.all(np.abs(oracle.bf16_to_f32(y) - ref) <= 2.0 ** -6 * np.abs(want) + (1e-3 + 2.0 ** -9) * mag)

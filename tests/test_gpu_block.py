@@ -17,6 +17,33 @@ from zyx_amd.block import PARAMS, TransformerBlock
 pytestmark = pytest.mark.gpu
 
 
+def test_block_with_causal_mask(hip, oracle):
+    """The mask the reference's module lacks (a flag of the attention launches): f32 on the general kernels and bf16
+    on the matrix-core kernels against the masked f64 block."""
+    B, T, d, H = 2, 5, 8, 2
+    blk, p, x, dout = make_block(hip, oracle, B, T, d, H, DType.F32, std=0.3, causal=True)
+    blk.forward_backward()
+    s = oracle.block_forward_f64(p, x.reshape(B, T, d), H, causal=True)
+    g = oracle.block_backward_f64(p, s, dout.reshape(B, T, d), H)
+    assert np.allclose(blk.read("out").reshape(B, T, d), s["out"], rtol=1e-4, atol=1e-5)
+    assert np.allclose(blk.read("dx").reshape(B, T, d), g["dx"], rtol=1e-4, atol=2e-5)
+    for n in PARAMS:
+        assert np.allclose(blk.read("d_" + n), g[n], rtol=1e-4, atol=2e-5), n
+    blk.close()
+    B, T, d, H = 2, 256, 256, 4
+    blk, p, x, dout = make_block(hip, oracle, B, T, d, H, DType.BF16, std=0.05, causal=True)
+    blk.forward_backward()
+    pf = {k: f64(oracle, v) for k, v in p.items()}
+    s = oracle.block_forward_f64(pf, f64(oracle, x).reshape(B, T, d), H, causal=True)
+    g = oracle.block_backward_f64(pf, s, f64(oracle, dout).reshape(B, T, d), H)
+    rel = lambda got, want: np.abs(f64(oracle, got).reshape(want.shape) - want).max() / np.abs(want).max()
+    assert rel(blk.read("att"), s["att"]) < 0.02 and rel(blk.read("out"), s["out"]) < 0.02
+    assert rel(blk.read("dx"), g["dx"]) < 0.03
+    for n in PARAMS:
+        assert rel(blk.read("d_" + n), g[n]) < 0.03, n
+    blk.close()
+
+
 def f64(oracle, a):
     return (oracle.bf16_to_f32(a) if a.dtype == np.uint16 else a).astype(np.float64)
 
@@ -25,9 +52,9 @@ def close_bf16(oracle, got, want, mag, extra=0.0):
     return np.abs(f64(oracle, got) - want) <= 2.0 ** -7 * np.abs(want) + (1e-3 + extra) * mag + 1e-30
 
 
-def make_block(hip, oracle, B, T, d, H, dtype, seed=1, std=0.02):
+def make_block(hip, oracle, B, T, d, H, dtype, seed=1, std=0.02, causal=False):
     dev, pool = hip
-    blk = TransformerBlock(dev, pool, B, T, d, H, dtype)
+    blk = TransformerBlock(dev, pool, B, T, d, H, dtype, causal=causal)
     p = oracle.block_init(d, H, seed, std)
     r = oracle.Rng(seed + 1)
     # non-trivial affine parts and biases so that every gradient path is exercised

@@ -448,6 +448,42 @@ def test_attention_against_textbook_and_finite_differences(oracle):
     assert np.allclose(got, num, rtol=1e-4, atol=1e-6)
 
 
+def test_causal_attention_against_textbook_and_finite_differences(oracle):
+    """The reference has no masked attention to take goldens from: the causal flag is pinned by the textbook
+    masked softmax in f64 (scores above the diagonal filled with -inf), central differences of it for the
+    backward, and two special cases (the first query copies v_0; with one key the mask changes nothing)."""
+    rng = np.random.default_rng(1)
+    B, T, H, dh, p = 2, 6, 2, 4, 0.25
+    qkv = rng.standard_normal((B, T, 3 * H * dh)).astype(np.float32)
+
+    def f64(qkv64):
+        q, k, v = [a.reshape(B, T, H, dh).transpose(0, 2, 1, 3) for a in np.split(qkv64, 3, axis=2)]
+        s = np.einsum("bhtd,bhjd->bhtj", q, k) * float(np.float32(1 / np.sqrt(dh)))
+        s = np.where(np.tril(np.ones((T, T), bool)), s, -np.inf)
+        m = s.max(-1, keepdims=True)
+        e = np.exp(s - m)
+        pr = e / e.sum(-1, keepdims=True) / float(np.float32(1) - np.float32(p))
+        return np.einsum("bhtj,bhjd->bhtd", pr, v).transpose(0, 2, 1, 3).reshape(B, T, H * dh), (m + np.log(e.sum(-1, keepdims=True)))[..., 0]
+
+    y, lse = oracle.attention(qkv, H, dropout_p=p, want_lse=True, causal=True)
+    y64, lse64 = f64(qkv.astype(np.float64))
+    assert np.allclose(y, y64, rtol=1e-5, atol=1e-6) and np.allclose(lse, lse64, rtol=1e-6, atol=1e-6)
+    assert not np.allclose(y, oracle.attention(qkv, H, dropout_p=p), rtol=1e-3)
+    assert np.allclose(y[:, 0], qkv[:, 0, 2 * H * dh:] / (np.float32(1) - np.float32(p)), rtol=1e-6)
+    one = qkv[:, :1]
+    assert np.array_equal(oracle.attention(one, H, causal=True), oracle.attention(one, H))
+    dy = rng.standard_normal(y.shape).astype(np.float32)
+    got = oracle.attention_bwd(qkv, dy, H, dropout_p=p, causal=True)
+    num = np.empty(qkv.shape, np.float64)
+    base = qkv.astype(np.float64)
+    for i in np.ndindex(*qkv.shape):
+        hi, lo = base.copy(), base.copy()
+        hi[i] += 1e-5
+        lo[i] -= 1e-5
+        num[i] = ((f64(hi)[0] - f64(lo)[0]) * dy).sum() / 2e-5
+    assert np.allclose(got, num, rtol=1e-4, atol=1e-6)
+
+
 def test_norm_backward_against_finite_differences(oracle):
     """No reference test holds norm gradients. The forward is pinned by the goldens above; its f64 restatement
     differentiated by central differences pins the backward (the n-1 of the unbiased variance, the mean(g) term
@@ -515,3 +551,18 @@ def test_block_f64_forward_pieces_and_backward_finite_differences(oracle):
                 num[i] = (loss({**p, name: hi}, x) - loss({**p, name: lo}, x)) / 2e-6
         got = g["dx"] if name == "x" else g[name]
         assert np.allclose(got, num, rtol=2e-5, atol=2e-6), name
+    # the optional causal mask: forward against the masked `attention`, backward by differences in x and c_attn
+    sc_ = oracle.block_forward_f64(p, x, H, causal=True)
+    assert np.allclose(sc_["att"], oracle.attention(sc_["qkv"].astype(np.float32), H, causal=True), rtol=1e-4, atol=1e-5)
+    assert np.all(np.triu(sc_["probs"], 1) == 0) and not np.allclose(sc_["out"], s["out"], rtol=1e-3)
+    gc = oracle.block_backward_f64(p, sc_, dout, H)
+    lossc = lambda pp, xx: (oracle.block_forward_f64(pp, xx, H, causal=True)["out"] * dout).sum()
+    for name in ("x", "attn_w"):
+        base = (x if name == "x" else p[name]).astype(np.float64)
+        num = np.empty_like(base)
+        for i in np.ndindex(*base.shape):
+            hi, lo = base.copy(), base.copy()
+            hi[i] += 1e-6
+            lo[i] -= 1e-6
+            num[i] = (lossc(p, hi) - lossc(p, lo)) / 2e-6 if name == "x" else (lossc({**p, name: hi}, x) - lossc({**p, name: lo}, x)) / 2e-6
+        assert np.allclose(gc["dx"] if name == "x" else gc[name], num, rtol=2e-5, atol=2e-6), name

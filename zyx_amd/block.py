@@ -4,7 +4,7 @@ the device once its plan is cached (zyx/src/tape.rs:141-202 -> zyx/src/graph/pla
 The block is `x = x + attn(ln_1(x)); x = x + mlp(ln_2(x))` of zyx-examples/examples/nanogpt.rs:68-98 built from
 zyx-nn modules: LayerNorm (zyx-nn/src/layer_norm.rs:98-135), CausalSelfAttention
 (zyx-nn/src/causal_self_attention.rs:36-74: c_attn Linear d -> 3d, per-head softmax(q k^T / sqrt(dh)) v with no
-mask, c_proj Linear d -> d), MLP = Linear d -> 4d, gelu, Linear 4d -> d (nanogpt.rs:41-66), Linear weights stored
+mask -- `causal=True` adds the lower-triangular one --, c_proj Linear d -> d), MLP = Linear d -> 4d, gelu, Linear 4d -> d (nanogpt.rs:41-66), Linear weights stored
 [out, in] (zyx-nn/src/linear.rs:24-44). Every tensor a module returns is stored once in `dtype` (bf16 stores
 truncate); arithmetic inside a kernel is f32.
 
@@ -34,7 +34,8 @@ PARAMS = ("ln1_w", "ln1_b", "attn_w", "attn_b", "proj_w", "proj_b", "ln2_w", "ln
 
 class TransformerBlock:
     def __init__(self, dev: HIPDevice, pool: HIPMemoryPool, batch: int, seq: int, d_model: int, n_head: int,
-                 dtype: DType = DType.BF16, eps: float = 1e-5, dropout_p: float = 0.0, mlp_ratio: int = 4):
+                 dtype: DType = DType.BF16, eps: float = 1e-5, dropout_p: float = 0.0, mlp_ratio: int = 4,
+                 causal: bool = False):
         self.dev, self.pool, self.dtype = dev, pool, DType(dtype)
         self.batch, self.seq, self.d, self.n_head, self.hidden = batch, seq, d_model, n_head, mlp_ratio * d_model
         self.np_dtype = np.uint16 if self.dtype == DType.BF16 else np.float32
@@ -80,7 +81,7 @@ class TransformerBlock:
         self.forward_nodes = [
             (ln, [x, P["ln1_w"], P["ln1_b"], n1]),
             (linear(m, 3 * d, d), [n1, P["attn_w"], P["attn_b"], qkv]),
-            (prog(K.attention_desc(batch, seq, n_head, dh_, dt, dropout_p=dropout_p, lse=True)), [qkv, att, lse]),
+            (prog(K.attention_desc(batch, seq, n_head, dh_, dt, dropout_p=dropout_p, lse=True, causal=causal)), [qkv, att, lse]),
             (linear(m, d, d, residual=True), [att, P["proj_w"], P["proj_b"], x, x2]),
             (ln, [x2, P["ln2_w"], P["ln2_b"], n2]),
             (linear(m, f, d), [n2, P["fc_w"], P["fc_b"], h]),
@@ -110,7 +111,7 @@ class TransformerBlock:
             (cs_d, [dx2, G["proj_b"]]),
             (dweight(d, d), [dx2, att, G["proj_w"]]),
             (dinput(d, d), [dx2, P["proj_w"], datt]),
-            (prog(K.attention_bwd_desc(batch, seq, n_head, dh_, dt, dropout_p=dropout_p)), [qkv, att, datt, lse, dqkv]),
+            (prog(K.attention_bwd_desc(batch, seq, n_head, dh_, dt, dropout_p=dropout_p, causal=causal)), [qkv, att, datt, lse, dqkv]),
             (colsum(3 * d), [dqkv, G["attn_b"]]),
             (dweight(3 * d, d), [dqkv, n1, G["attn_w"]]),
             (dinput(3 * d, d), [dqkv, P["attn_w"], dn1]),

@@ -1,5 +1,5 @@
 // Fused attention core of zyx-nn's CausalSelfAttention (zyx-nn/src/causal_self_attention.rs:36-74):
-// y = softmax(scale * q.k^T) / keep . v per head, no mask (the reference applies none), reading q, k, v
+// y = softmax(scale * q.k^T) / keep . v per head (the reference applies no mask; a causal one is optional), reading q, k, v
 // in place from the c_attn output qkv[B, T, 3, H, dh] and writing y[B, T, H*dh], i.e. split / reshape /
 // transpose(1,2) before and transpose(1,2) / reshape after are index arithmetic. The [T, T] score
 // tensors the reference materialises (q.dot(k.t()), softmax, dropout) never leave registers.
@@ -47,7 +47,9 @@ __device__ __forceinline__ int v_slot(int key, int chunk) {
 
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
-template <bool LSE>
+// CAUSAL: query t sees keys 0..t. A workgroup then stops at the key tile that holds its last query, a wave leaves out
+// tiles that lie wholly after its queries, and the tiles the diagonal crosses get -inf where key > query.
+template <bool LSE, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__restrict__ qkv, uint16_t *__restrict__ y,
                                                           float *__restrict__ lse, int T, int H, float c, float out_scale) {
     __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[2 * STAGE];
@@ -56,15 +58,24 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
 
     // Workgroups whose ids are congruent mod 8 share an XCD (and its L2): give every XCD whole heads, so
     // the K and V of a head are fetched into one L2 only.
-    const int QT = T / QB, BH = (int)gridDim.x / QT;
+    const int QT = T / QB, NB = CAUSAL ? (QT + 1) / 2 : QT, BH = (int)gridDim.x / NB; // NB blocks of the grid per head
     int bh, qt;
     if (BH % 8 == 0) {
         const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
-        bh = (i / QT) * 8 + x;
-        qt = i % QT;
+        bh = (i / NB) * 8 + x;
+        qt = i % NB;
     } else {
-        bh = blockIdx.x / QT;
-        qt = blockIdx.x % QT;
+        bh = blockIdx.x / NB;
+        qt = blockIdx.x % NB;
+    }
+    // Causal work grows with qt: a workgroup takes the query blocks qt and QT-1-qt one after the other, so every
+    // workgroup streams the same number of key tiles (2 QT + 2) whatever CU it lands on.
+    const int qt_first = qt;
+#pragma nounroll
+    for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
+    if (CAUSAL && pass) {
+        qt = QT - 1 - qt_first;
+        if (qt == qt_first) break; // odd QT: the middle block has no partner
     }
     const int bb = bh / H, h = bh % H;
     const int64_t ld = 3 * (int64_t)H * DH;
@@ -117,7 +128,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
         for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
     float m = -INFINITY, l = 0.0f;
 
-    const int NT = T / KB;
+    const int NT = CAUSAL ? 2 * qt + 2 : T / KB;
+    const int q0w = qt * QB + wave * 32; // first query of this wave
     stage_tile(0, 0);
     __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): this wave's part of tile 0 has landed in LDS
     __syncthreads();
@@ -125,6 +137,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
     for (int kt = 0; kt < NT; kt++) {
         if (kt + 1 < NT) stage_tile(kt + 1, stage ^ STAGE); // the other stage was last read before the previous barrier
 
+        if (!CAUSAL || kt * KB <= q0w + 31) {
         f32x16 s[2];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
@@ -137,6 +150,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
             }
         }
 
+        if (CAUSAL && kt * KB + KB - 1 > q0w) { // register r of block kb is key kb*32 + 8*(r/4) + 4*hh + r%4 of the tile
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if (kt * KB + kb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3) > tq) s[kb][r] = -INFINITY;
+        }
         float bm = s[0][0];
 #pragma unroll
         for (int r = 1; r < 16; r++) bm = fmaxf(bm, s[0][r]);
@@ -179,6 +199,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
                 }
         }
         l = __builtin_fmaf(l, alpha, ps);
+        }
 
         __builtin_amdgcn_s_waitcnt(0x0f70); // this wave's loads of tile kt+1 have landed
         __syncthreads();
@@ -198,13 +219,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
             *(u32x2 *)(yp + db * 32 + 8 * g + 4 * hh) = w;
         }
     if (LSE && hh == 0) lse[(int64_t)bh * T + tq] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+    }
 }
 
 // One wave per query. Keys are taken 64 at a time (lane = key) for the scores and the
 // exponentials, then lane = d for the weighted sum of V rows; p[] and q[] live in LDS.
 template <int DT>
 __global__ __launch_bounds__(64) void attn_small_k(const void *__restrict__ qkv_, void *__restrict__ y_, float *__restrict__ lse,
-                                                   int T, int H, int dh, float scale, float keep) {
+                                                   int T, int H, int dh, float scale, float keep, int causal) {
     __shared__ float qs[256], ps[64];
     const int lane = threadIdx.x, t = blockIdx.x, bh = blockIdx.y, bb = bh / H, h = bh % H;
     const int64_t C = (int64_t)H * dh, ld = 3 * C;
@@ -217,24 +239,25 @@ __global__ __launch_bounds__(64) void attn_small_k(const void *__restrict__ qkv_
     __syncthreads();
     float o[4] = {0.0f, 0.0f, 0.0f, 0.0f}; // d = lane + 64*i
     float m = -INFINITY, l = 0.0f;
-    for (int j0 = 0; j0 < T; j0 += 64) {
+    const int Tk = causal ? t + 1 : T; // keys this query sees
+    for (int j0 = 0; j0 < Tk; j0 += 64) {
         const int j = j0 + lane;
         float s = -INFINITY;
-        if (j < T) {
+        if (j < Tk) {
             const int64_t ko = ((int64_t)bb * T + j) * ld + C + h * dh;
             float a = 0.0f;
             for (int d = 0; d < dh; d++) a = __builtin_fmaf(qs[d], ldv(ko + d), a);
             s = a * scale;
         }
         const float m_new = fmaxf(m, wave_allreduce_f32(s, OpMaxF()));
-        const float p = j < T ? exp_neg(s - m_new) : 0.0f;
+        const float p = j < Tk ? exp_neg(s - m_new) : 0.0f;
         const float alpha = m == -INFINITY ? 0.0f : exp_neg(m - m_new);
         l = l * alpha + wave_allreduce_f32(p, OpAdd());
         m = m_new;
         __syncthreads(); // ps of the previous chunk has been consumed
         ps[lane] = p;
         __syncthreads();
-        const int nk = min(64, T - j0);
+        const int nk = min(64, Tk - j0);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int d = lane + 64 * i;
@@ -269,21 +292,27 @@ bool attention_fast_path(const Attention &p) {
 hipError_t attention_fwd(const Attention &p, hipStream_t st) {
     if (p.B <= 0 || p.T <= 0 || p.H <= 0 || p.dh <= 0) return hipSuccess;
     if (attention_fast_path(p)) {
-        dim3 grid((unsigned)(p.B * p.H * (p.T / QB))), block(256);
-        if (p.lse)
-            hipLaunchKernelGGL(attn_fwd_bf16_k<true>, grid, block, 0, st, (const uint16_t *)p.qkv, (uint16_t *)p.y, p.lse, p.T, p.H,
-                               p.scale * kLog2e, 1.0f / p.keep);
-        else
-            hipLaunchKernelGGL(attn_fwd_bf16_k<false>, grid, block, 0, st, (const uint16_t *)p.qkv, (uint16_t *)p.y, p.lse, p.T, p.H,
-                               p.scale * kLog2e, 1.0f / p.keep);
+        const int qblocks = p.T / QB;
+        dim3 grid((unsigned)(p.B * p.H * (p.causal ? (qblocks + 1) / 2 : qblocks))), block(256);
+#define ZK_ATTN(L, CA)                                                                                                \
+    hipLaunchKernelGGL((attn_fwd_bf16_k<L, CA>), grid, block, 0, st, (const uint16_t *)p.qkv, (uint16_t *)p.y, p.lse, p.T, p.H, \
+                       p.scale * kLog2e, 1.0f / p.keep)
+        if (p.lse) {
+            if (p.causal) ZK_ATTN(true, true);
+            else ZK_ATTN(true, false);
+        } else {
+            if (p.causal) ZK_ATTN(false, true);
+            else ZK_ATTN(false, false);
+        }
+#undef ZK_ATTN
         return hipGetLastError();
     }
     if (p.dh > 256 || (int64_t)p.B * p.H > 65535 || (p.dtype != DT_F32 && p.dtype != DT_BF16)) return hipErrorInvalidValue;
     dim3 grid((unsigned)p.T, (unsigned)(p.B * p.H)), block(64);
     if (p.dtype == DT_F32)
-        hipLaunchKernelGGL(attn_small_k<DT_F32>, grid, block, 0, st, p.qkv, p.y, p.lse, p.T, p.H, p.dh, p.scale, p.keep);
+        hipLaunchKernelGGL(attn_small_k<DT_F32>, grid, block, 0, st, p.qkv, p.y, p.lse, p.T, p.H, p.dh, p.scale, p.keep, p.causal);
     else
-        hipLaunchKernelGGL(attn_small_k<DT_BF16>, grid, block, 0, st, p.qkv, p.y, p.lse, p.T, p.H, p.dh, p.scale, p.keep);
+        hipLaunchKernelGGL(attn_small_k<DT_BF16>, grid, block, 0, st, p.qkv, p.y, p.lse, p.T, p.H, p.dh, p.scale, p.keep, p.causal);
     return hipGetLastError();
 }
 

@@ -53,6 +53,11 @@ __global__ __launch_bounds__(256) void attn_bwd_d_k(const uint16_t *__restrict__
     }
 }
 
+// CAUSAL (both kernels below): pairs with key > query carry probability 0. Tiles that hold only such pairs are not
+// visited (the workgroup's loop bounds) or not computed (a wave's own keys / queries), and the tiles the diagonal
+// crosses zero the masked probabilities, which zeroes dS too. The number of tiles then depends on the block, so a
+// workgroup takes blocks j and nblk-1-j one after the other: equal work for every workgroup, on whatever CU.
+template <bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ dy,
                                                          const float *__restrict__ lse, const float *__restrict__ D,
                                                          uint16_t *__restrict__ dqkv, int T, int H, float c, float scale,
@@ -61,7 +66,15 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restr
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
     int bh, kblk;
-    head_and_block(T / 128, bh, kblk);
+    const int nblk = T / 128;
+    head_and_block(CAUSAL ? (nblk + 1) / 2 : nblk, bh, kblk);
+    const int blk_first = kblk;
+#pragma nounroll
+    for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
+    if (CAUSAL && pass) {
+        kblk = nblk - 1 - blk_first;
+        if (kblk == blk_first) break;
+    }
     const int bb = bh / H, h = bh % H;
     const int64_t C = (int64_t)H * DH, ld = 3 * C;
     const uint16_t *qp = qkv + (int64_t)bb * T * ld + h * DH, *kp = qp + C, *vp = kp + C;
@@ -121,12 +134,16 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restr
         for (int r = 0; r < 16; r++) dkT[db][r] = dvT[db][r] = 0.0f;
 
     const int NT = T / TROWS;
-    gload(0);
+    const int QT0 = CAUSAL ? 2 * kblk : 0;        // first query tile that holds a query >= this block's first key
+    const int k0w = kblk * 128 + wave * 32;       // first key of this wave
+    gload(QT0);
     lwrite(0);
     __syncthreads();
     int stage = 0;
-    for (int qt = 0; qt < NT; qt++) {
+    for (int qt = QT0; qt < NT; qt++) {
         if (qt + 1 < NT) gload(qt + 1);
+        const bool diag = CAUSAL && qt * TROWS < k0w + 31; // some query of the tile is before some key of this wave
+        if (!CAUSAL || qt * TROWS + TROWS - 1 >= k0w) {
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) {
             f32x16 s, dp;
@@ -155,7 +172,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restr
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         const int r = 8 * s2 + 4 * g + j;
-                        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], c, -l2[j]));
+                        float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], c, -l2[j]));
+                        if (CAUSAL && diag && qt * TROWS + q0 + j < tk) pv = 0.0f;
                         p[4 * g + j] = pv;
                         ds[4 * g + j] = pv * __builtin_fmaf(dp[r], inv_keep, -dd[j]);
                     }
@@ -174,6 +192,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restr
                     dkT[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qT, dsb[s2], dkT[db], 0, 0, 0);
                 }
         }
+        }
         if (qt + 1 < NT) lwrite(stage ^ STAGE_BWD);
         __syncthreads();
         stage ^= STAGE_BWD;
@@ -189,8 +208,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restr
             *(u32x2 *)(dk + d) = pack4_trunc(dkT[db][4 * g] * scale, dkT[db][4 * g + 1] * scale, dkT[db][4 * g + 2] * scale, dkT[db][4 * g + 3] * scale);
             *(u32x2 *)(dv + d) = pack4_trunc(dvT[db][4 * g] * inv_keep, dvT[db][4 * g + 1] * inv_keep, dvT[db][4 * g + 2] * inv_keep, dvT[db][4 * g + 3] * inv_keep);
         }
+    }
 }
 
+template <bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ dy,
                                                         const float *__restrict__ lse, const float *__restrict__ D,
                                                         uint16_t *__restrict__ dqkv, int T, int H, float c, float scale,
@@ -199,7 +220,15 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restri
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
     int bh, qblk;
-    head_and_block(T / 128, bh, qblk);
+    const int nblk = T / 128;
+    head_and_block(CAUSAL ? (nblk + 1) / 2 : nblk, bh, qblk);
+    const int blk_first = qblk;
+#pragma nounroll
+    for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
+    if (CAUSAL && pass) {
+        qblk = nblk - 1 - blk_first;
+        if (qblk == blk_first) break;
+    }
     const int bb = bh / H, h = bh % H;
     const int64_t C = (int64_t)H * DH, ld = 3 * C;
     const uint16_t *qp = qkv + (int64_t)bb * T * ld + h * DH, *kp = qp + C, *vp = kp + C;
@@ -251,13 +280,16 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restri
 #pragma unroll
         for (int r = 0; r < 16; r++) dqT[db][r] = 0.0f;
 
-    const int NT = T / TROWS;
+    const int NT = CAUSAL ? 2 * qblk + 2 : T / TROWS;
+    const int q0w = qblk * 128 + wave * 32; // first query of this wave
     gload(0);
     lwrite(0);
     __syncthreads();
     int stage = 0;
     for (int kt = 0; kt < NT; kt++) {
         if (kt + 1 < NT) gload(kt + 1);
+        const bool diag = CAUSAL && kt * TROWS + TROWS - 1 > q0w;
+        if (!CAUSAL || kt * TROWS <= q0w + 31) {
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
             f32x16 s, dp;
@@ -279,7 +311,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restri
                 f32x8 ds;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * s2 + e], c, -l2));
+                    float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * s2 + e], c, -l2));
+                    // register r = 8*s2 + e is key kb*32 + 8*(r/4) + 4*hh + r%4 of the tile
+                    if (CAUSAL && diag && kt * TROWS + kb * 32 + 8 * (2 * s2 + (e >> 2)) + 4 * hh + (e & 3) > tq) pv = 0.0f;
                     ds[e] = pv * __builtin_fmaf(dp[8 * s2 + e], inv_keep, -dd);
                 }
                 dsb[s2] = __builtin_convertvector(ds, bf16x8);
@@ -293,6 +327,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restri
                     dqT[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kT, dsb[s2], dqT[db], 0, 0, 0);
                 }
         }
+        }
         if (kt + 1 < NT) lwrite(stage ^ (2 * TILE));
         __syncthreads();
         stage ^= 2 * TILE;
@@ -304,6 +339,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restri
         for (int g = 0; g < 4; g++)
             *(u32x2 *)(dq + db * 32 + 8 * g + 4 * hh) =
                 pack4_trunc(dqT[db][4 * g] * scale, dqT[db][4 * g + 1] * scale, dqT[db][4 * g + 2] * scale, dqT[db][4 * g + 3] * scale);
+    }
 }
 
 // ---- general path ---------------------------------------------------------------------------------------
@@ -322,7 +358,8 @@ template <int DT> __device__ __forceinline__ void stf(void *p, int64_t i, float 
 template <int DT, int ROLE>
 __global__ __launch_bounds__(64) void attn_bwd_small_k(const void *__restrict__ qkv, const void *__restrict__ y,
                                                        const void *__restrict__ dy, const float *__restrict__ lse,
-                                                       void *__restrict__ dqkv, int T, int H, int dh, float scale, float keep) {
+                                                       void *__restrict__ dqkv, int T, int H, int dh, float scale, float keep,
+                                                       int causal) {
     __shared__ float mine[2][256], w0[64], w1[64];
     const int lane = threadIdx.x, t = blockIdx.x, bh = blockIdx.y, bb = bh / H, h = bh % H;
     const int64_t C = (int64_t)H * dh, ld = 3 * C;
@@ -341,10 +378,12 @@ __global__ __launch_bounds__(64) void attn_bwd_small_k(const void *__restrict__ 
         lse_t = lse[(int64_t)bh * T + t];
     }
     float acc0[4] = {0, 0, 0, 0}, acc1[4] = {0, 0, 0, 0};
-    for (int j0 = 0; j0 < T; j0 += 64) {
+    // causal: a query's partners are the keys 0..t, a key's partners the queries t..T-1
+    const int jlo = (causal && ROLE == 1) ? t : 0, jhi = (causal && ROLE == 0) ? t + 1 : T;
+    for (int j0 = (jlo / 64) * 64; j0 < jhi; j0 += 64) {
         const int j = j0 + lane;
         float p = 0.0f, ds = 0.0f;
-        if (j < T) {
+        if (j >= jlo && j < jhi) {
             const int64_t rq = ((int64_t)bb * T + j) * ld + h * dh, ry = ((int64_t)bb * T + j) * C + h * dh;
             float s = 0.0f, dp = 0.0f, Dj = Dt;
             if (ROLE == 0) { // partner j is a key: s = q_t.k_j, dp = dy_t.v_j
@@ -416,19 +455,27 @@ hipError_t attention_bwd(const AttentionBwd &p, hipStream_t st) {
         float *D = (float *)p.workspace;
         hipLaunchKernelGGL(attn_bwd_d_k, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, st, (const uint16_t *)f.y,
                            (const uint16_t *)p.dy, D, rows, f.T, f.H);
-        dim3 grid((unsigned)(f.B * f.H * (f.T / 128))), block(256);
+        const int nblk = f.T / 128;
+        dim3 grid((unsigned)(f.B * f.H * (f.causal ? (nblk + 1) / 2 : nblk))), block(256);
         const float c = f.scale * kLog2e, ik = 1.0f / f.keep;
-        hipLaunchKernelGGL(attn_bwd_dkv_k, grid, block, 0, st, (const uint16_t *)f.qkv, (const uint16_t *)p.dy, f.lse, D,
-                           (uint16_t *)p.dqkv, f.T, f.H, c, f.scale, ik);
-        hipLaunchKernelGGL(attn_bwd_dq_k, grid, block, 0, st, (const uint16_t *)f.qkv, (const uint16_t *)p.dy, f.lse, D,
-                           (uint16_t *)p.dqkv, f.T, f.H, c, f.scale, ik);
+#define ZK_BWD(K)                                                                                                     \
+    hipLaunchKernelGGL(K, grid, block, 0, st, (const uint16_t *)f.qkv, (const uint16_t *)p.dy, f.lse, D, (uint16_t *)p.dqkv, \
+                       f.T, f.H, c, f.scale, ik)
+        if (f.causal) {
+            ZK_BWD(attn_bwd_dkv_k<true>);
+            ZK_BWD(attn_bwd_dq_k<true>);
+        } else {
+            ZK_BWD(attn_bwd_dkv_k<false>);
+            ZK_BWD(attn_bwd_dq_k<false>);
+        }
+#undef ZK_BWD
         return hipGetLastError();
     }
     if (f.dh > 256 || (int64_t)f.B * f.H > 65535 || (f.dtype != DT_F32 && f.dtype != DT_BF16)) return hipErrorInvalidValue;
     dim3 grid((unsigned)f.T, (unsigned)(f.B * f.H)), block(64);
 #define ZK_SMALL(DT, ROLE)                                                                                            \
     hipLaunchKernelGGL((attn_bwd_small_k<DT, ROLE>), grid, block, 0, st, f.qkv, f.y, p.dy, f.lse, p.dqkv, f.T, f.H, f.dh, \
-                       f.scale, f.keep)
+                       f.scale, f.keep, f.causal)
     if (f.dtype == DT_F32) {
         ZK_SMALL(DT_F32, 0);
         ZK_SMALL(DT_F32, 1);

@@ -171,6 +171,7 @@ struct Attention {
     int B, T, H, dh;
     int dtype; // DT_BF16 or DT_F32 storage of qkv and y
     float scale, keep;
+    int causal; // query t attends to keys 0..t only
     const void *qkv;
     void *y;
     float *lse;

@@ -317,6 +317,7 @@ zk::Attention attention_args(const zhip_kernel_desc &d) {
     a.dtype = d.dtype;
     a.scale = d.fparams[0] > 0.0f ? d.fparams[0] : (float)(1.0 / sqrt((double)a.dh));
     a.keep = 1.0f - d.fparams[1];
+    a.causal = d.flags & ZHIP_ATTN_CAUSAL ? 1 : 0;
     return a;
 }
 
@@ -555,11 +556,11 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         if (B < 0 || T < 0 || H <= 0 || dh <= 0 || dh > 256 || B * H > 65535 || T >= (1ll << 24) || B * T * 3 * H * dh >= (1ll << 40))
             return c->fail(ZHIP_KERNEL_COMPILATION, "attention: shape out of range (dh <= 256, B*H <= 65535)");
         if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16) return c->fail(ZHIP_KERNEL_COMPILATION, "attention: dtype must be F32 or BF16");
-        if ((d.flags & ~ZHIP_ATTN_LSE) || d.fparams[0] < 0.0f || !(d.fparams[1] >= 0.0f && d.fparams[1] < 1.0f))
+        if ((d.flags & ~(ZHIP_ATTN_LSE | ZHIP_ATTN_CAUSAL)) || d.fparams[0] < 0.0f || !(d.fparams[1] >= 0.0f && d.fparams[1] < 1.0f))
             return c->fail(ZHIP_KERNEL_COMPILATION, "attention: bad flags, scale or dropout probability");
         const uint64_t e = dtype_bytes(d.dtype);
         if (d.kind == ZHIP_K_ATTENTION_BWD) {
-            if (d.flags) return c->fail(ZHIP_KERNEL_COMPILATION, "attention backward takes no flags");
+            if (d.flags & ~ZHIP_ATTN_CAUSAL) return c->fail(ZHIP_KERNEL_COMPILATION, "attention backward takes no flag but ZHIP_ATTN_CAUSAL");
             p.n_in = 4;
             p.need[0] = (uint64_t)(B * T * 3 * H * dh) * e;
             p.need[1] = p.need[2] = (uint64_t)(B * T * H * dh) * e;

@@ -467,26 +467,27 @@ def scatter(dev: HIPDevice, pool: HIPMemoryPool, x, axis: int, indices, src):
 
 # ---- attention core (ZHIP_K_ATTENTION) -----------------------------------------------------------------------
 K_ATTENTION = 10
-ATTN_LSE = 1
+ATTN_LSE, ATTN_CAUSAL = 1, 2
 
 
 def attention_desc(b: int, t: int, n_head: int, dh: int, dtype: DType = DType.BF16, scale: float = 0.0,
-                   dropout_p: float = 0.0, lse: bool = False) -> KernelDesc:
+                   dropout_p: float = 0.0, lse: bool = False, causal: bool = False) -> KernelDesc:
     d = KernelDesc()
-    d.kind, d.dtype, d.out_dtype, d.flags = K_ATTENTION, DType(dtype), DType(dtype), ATTN_LSE if lse else 0
+    d.kind, d.dtype, d.out_dtype = K_ATTENTION, DType(dtype), DType(dtype)
+    d.flags = (ATTN_LSE if lse else 0) | (ATTN_CAUSAL if causal else 0)
     d.dims[0], d.dims[1], d.dims[2], d.dims[3] = b, t, n_head, dh
     d.fparams[0], d.fparams[1] = scale, dropout_p
     return d
 
 
 def attention(dev: HIPDevice, pool: HIPMemoryPool, qkv, n_head: int, dtype: DType = DType.BF16, scale: float = 0.0,
-              dropout_p: float = 0.0, want_lse: bool = False):
+              dropout_p: float = 0.0, want_lse: bool = False, causal: bool = False):
     """Core of CausalSelfAttention::forward (zyx-nn/src/causal_self_attention.rs:36-74) on the c_attn output
     qkv[B,T,3C] (bf16 bit patterns as uint16, or float32) -> y[B,T,C] (, lse[B,H,T])."""
     qkv = np.ascontiguousarray(qkv)
     b, t, c3 = qkv.shape
     c = c3 // 3
-    prog = dev.register_kernel(attention_desc(b, t, n_head, c // n_head, dtype, scale, dropout_p, want_lse))
+    prog = dev.register_kernel(attention_desc(b, t, n_head, c // n_head, dtype, scale, dropout_p, want_lse, causal))
     xb, e0 = to_device(pool, qkv)
     yb, e1 = alloc_like(pool, b * t * c, qkv.dtype.itemsize)
     bufs, waits = [xb, yb], [e0, e1]
@@ -507,18 +508,18 @@ K_ATTENTION_BWD = 11
 
 
 def attention_bwd_desc(b: int, t: int, n_head: int, dh: int, dtype: DType = DType.BF16, scale: float = 0.0,
-                       dropout_p: float = 0.0) -> KernelDesc:
-    d = attention_desc(b, t, n_head, dh, dtype, scale, dropout_p)
+                       dropout_p: float = 0.0, causal: bool = False) -> KernelDesc:
+    d = attention_desc(b, t, n_head, dh, dtype, scale, dropout_p, causal=causal)
     d.kind = K_ATTENTION_BWD
     return d
 
 
 def attention_bwd(dev: HIPDevice, pool: HIPMemoryPool, qkv, y, dy, lse, n_head: int, dtype: DType = DType.BF16,
-                  scale: float = 0.0, dropout_p: float = 0.0):
+                  scale: float = 0.0, dropout_p: float = 0.0, causal: bool = False):
     """Gradient of `attention` with respect to qkv given dy; y and lse are the forward's outputs."""
     qkv = np.ascontiguousarray(qkv)
     b, t, c3 = qkv.shape
-    prog = dev.register_kernel(attention_bwd_desc(b, t, n_head, c3 // 3 // n_head, dtype, scale, dropout_p))
+    prog = dev.register_kernel(attention_bwd_desc(b, t, n_head, c3 // 3 // n_head, dtype, scale, dropout_p, causal))
     bufs, waits = [], []
     for a in (qkv, np.ascontiguousarray(y, qkv.dtype), np.ascontiguousarray(dy, qkv.dtype), np.ascontiguousarray(lse, np.float32)):
         buf, e = to_device(pool, a)
