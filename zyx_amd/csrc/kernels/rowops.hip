@@ -161,77 +161,103 @@ __global__ __launch_bounds__(256) void norm_rows_reg_k(const typename RowIO<DT>:
     }
 }
 
-// dx for rows of 256*NV columns with x and dy held in registers (one read of each); otherwise as norm_bwd_dx_k.
-template <int DT, int MODE, int NV>
-__global__ __launch_bounds__(256) void norm_bwd_dx_reg_k(const typename RowIO<DT>::S *__restrict__ x,
-                                                         const typename RowIO<DT>::S *__restrict__ w,
-                                                         const typename RowIO<DT>::S *__restrict__ dy,
-                                                         const typename RowIO<DT>::S *__restrict__ add,
-                                                         typename RowIO<DT>::S *__restrict__ dx, float *__restrict__ stats,
-                                                         int64_t rows, float eps) {
+// dx for rows of 256*NV columns with x and dy held in registers (one read of each), and the parameter gradients in
+// the same pass: a workgroup of WAVES waves walks rows blockIdx*WAVES + wave, + gridDim*WAVES, ..., every lane keeps
+// running sums of dy*xh and dy for its 4*NV columns, the waves of a workgroup fold theirs through LDS in wave order
+// and the workgroup leaves one partial row pair in part[(blockIdx*2 + {0,1})*cols + c] for norm_bwd_param_sum_k.
+// The order of every sum is fixed by the launch shape: results are reproducible. part may be null (no dw / db).
+template <int DT, int MODE, int NV, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename RowIO<DT>::S *__restrict__ x,
+                                                                const typename RowIO<DT>::S *__restrict__ w,
+                                                                const typename RowIO<DT>::S *__restrict__ dy,
+                                                                const typename RowIO<DT>::S *__restrict__ add,
+                                                                typename RowIO<DT>::S *__restrict__ dx, float *__restrict__ part,
+                                                                int64_t rows, float eps) {
     typedef RowIO<DT> IO;
     constexpr int cols = 256 * NV;
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const int64_t base = row * cols;
-    float xv[NV][4], g[NV][4];
+    __shared__ float fold[2][cols];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float pw[NV][4], pb[NV][4];
 #pragma unroll
-    for (int j = 0; j < NV; j++) {
-        IO::ld4(x + base, (lane + 64 * j) * 4, xv[j]);
-        IO::ld4(dy + base, (lane + 64 * j) * 4, g[j]);
-    }
-    float mean = 0.0f, rstd;
-    if (MODE == 0) {
-        float s = 0.0f;
+    for (int j = 0; j < NV; j++)
 #pragma unroll
-        for (int j = 0; j < NV; j++) s += (xv[j][0] + xv[j][1]) + (xv[j][2] + xv[j][3]);
-        mean = wave_allreduce_f32(s, OpAdd()) / (float)cols;
-        float q = 0.0f;
+        for (int k = 0; k < 4; k++) pw[j][k] = pb[j][k] = 0.0f;
+    // (Fetching 16-bit rows one row ahead was tried: the 24 extra registers spill in a 16-wave workgroup and the
+    // kernel gets slower, 25.9 us against 18.7 us at 8192 x 1024.)
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < rows; row += (int64_t)gridDim.x * WAVES) {
+        const int64_t base = row * cols;
+        float xv[NV][4], g[NV][4];
 #pragma unroll
-        for (int j = 0; j < NV; j++)
-#pragma unroll
-            for (int k = 0; k < 4; k++) q += (xv[j][k] - mean) * (xv[j][k] - mean);
-        rstd = 1.0f / sqrtf(wave_allreduce_f32(q, OpAdd()) / (float)(cols - 1) + eps);
-    } else {
-        float q = 0.0f;
-#pragma unroll
-        for (int j = 0; j < NV; j++)
-#pragma unroll
-            for (int k = 0; k < 4; k++) q += xv[j][k] * xv[j][k];
-        rstd = sqrtf(1.0f / (wave_allreduce_f32(q, OpAdd()) / (float)cols + eps));
-    }
-    float s1 = 0.0f, s2 = 0.0f;
-#pragma unroll
-    for (int j = 0; j < NV; j++) {
-        if (w) {
-            float wv[4];
-            IO::ld4(w, (lane + 64 * j) * 4, wv);
-#pragma unroll
-            for (int k = 0; k < 4; k++) g[j][k] *= wv[k];
+        for (int j = 0; j < NV; j++) {
+            IO::ld4(x + base, (lane + 64 * j) * 4, xv[j]);
+            IO::ld4(dy + base, (lane + 64 * j) * 4, g[j]);
         }
+        float mean = 0.0f, rstd;
+        if (MODE == 0) {
+            float s = 0.0f;
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            s1 += g[j][k];
-            s2 += g[j][k] * (MODE == 0 ? (xv[j][k] - mean) * rstd : xv[j][k]);
+            for (int j = 0; j < NV; j++) s += (xv[j][0] + xv[j][1]) + (xv[j][2] + xv[j][3]);
+            mean = wave_allreduce_f32(s, OpAdd()) / (float)cols;
+            float q = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NV; j++)
+#pragma unroll
+                for (int k = 0; k < 4; k++) q += (xv[j][k] - mean) * (xv[j][k] - mean);
+            rstd = 1.0f / sqrtf(wave_allreduce_f32(q, OpAdd()) / (float)(cols - 1) + eps);
+        } else {
+            float q = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NV; j++)
+#pragma unroll
+                for (int k = 0; k < 4; k++) q += xv[j][k] * xv[j][k];
+            rstd = sqrtf(1.0f / (wave_allreduce_f32(q, OpAdd()) / (float)cols + eps));
+        }
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            float wv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+            if (w) IO::ld4(w, (lane + 64 * j) * 4, wv); // L1 / L2 hit: every row reads the same 4*NV values
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const float xh = (xv[j][k] - mean) * rstd; // mean is 0 for RMSNorm
+                pw[j][k] = __builtin_fmaf(g[j][k], xh, pw[j][k]);
+                pb[j][k] += g[j][k];
+                g[j][k] *= wv[k];
+                s1 += g[j][k];
+                s2 += g[j][k] * (MODE == 0 ? xh : xv[j][k]);
+            }
+        }
+        s1 = wave_allreduce_f32(s1, OpAdd());
+        s2 = wave_allreduce_f32(s2, OpAdd());
+        const float k1 = s1 / (float)cols, k2 = MODE == 0 ? s2 / (float)(cols - 1) : rstd * rstd * rstd * s2 / (float)cols;
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int c = (lane + 64 * j) * 4;
+            float o[4], av[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (add) IO::ld4(add + base, c, av);
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                o[k] = (MODE == 0 ? rstd * ((g[j][k] - k1) - ((xv[j][k] - mean) * rstd) * k2) : rstd * g[j][k] - xv[j][k] * k2) + av[k];
+            IO::st4(dx + base, c, o);
         }
     }
-    s1 = wave_allreduce_f32(s1, OpAdd());
-    s2 = wave_allreduce_f32(s2, OpAdd());
-    const float k1 = s1 / (float)cols, k2 = MODE == 0 ? s2 / (float)(cols - 1) : rstd * rstd * rstd * s2 / (float)cols;
+    if (!part) return; // uniform over the workgroup
+    for (int v = 0; v < WAVES; v++) {
+        if (wave == v) {
 #pragma unroll
-    for (int j = 0; j < NV; j++) {
-        const int c = (lane + 64 * j) * 4;
-        float av[4] = {0.0f, 0.0f, 0.0f, 0.0f}, o[4];
-        if (add) IO::ld4(add + base, c, av);
+            for (int j = 0; j < NV; j++)
 #pragma unroll
-        for (int k = 0; k < 4; k++)
-            o[k] = (MODE == 0 ? rstd * ((g[j][k] - k1) - ((xv[j][k] - mean) * rstd) * k2) : rstd * g[j][k] - xv[j][k] * k2) + av[k];
-        IO::st4(dx + base, c, o);
+                for (int k = 0; k < 4; k++) {
+                    const int c = (lane + 64 * j) * 4 + k;
+                    fold[0][c] = v == 0 ? pw[j][k] : fold[0][c] + pw[j][k];
+                    fold[1][c] = v == 0 ? pb[j][k] : fold[1][c] + pb[j][k];
+                }
+        }
+        __syncthreads();
     }
-    if (lane == 0) {
-        stats[row * 2] = mean;
-        stats[row * 2 + 1] = rstd;
+    for (int c = threadIdx.x; c < cols; c += WAVES * 64) {
+        part[((int64_t)blockIdx.x * 2) * cols + c] = fold[0][c];
+        part[((int64_t)blockIdx.x * 2 + 1) * cols + c] = fold[1][c];
     }
 }
 
@@ -385,17 +411,17 @@ __global__ __launch_bounds__(256) void norm_bwd_param_k(const typename RowIO<DT>
         }
     }
 }
-// lane -> column of a 64-column strip, the 4 waves split the chunks
+// lane -> column of a 64-column strip, the 16 waves split the chunks (independent loads, a few per wave)
 template <int DT>
-__global__ __launch_bounds__(256) void norm_bwd_param_sum_k(const float *__restrict__ part, typename RowIO<DT>::S *__restrict__ dw,
-                                                            typename RowIO<DT>::S *__restrict__ db, int cols, int chunks) {
-    __shared__ float lds[4][2][64];
+__global__ __launch_bounds__(1024) void norm_bwd_param_sum_k(const float *__restrict__ part, typename RowIO<DT>::S *__restrict__ dw,
+                                                             typename RowIO<DT>::S *__restrict__ db, int cols, int chunks) {
+    __shared__ float lds[16][2][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = blockIdx.x * 64 + lane;
     float sw = 0.0f, sb = 0.0f;
     if (c < cols) {
 #pragma unroll 8
-        for (int k = wave; k < chunks; k += 4) {
+        for (int k = wave; k < chunks; k += 16) {
             sw += part[((int64_t)k * 2) * cols + c];
             sb += part[((int64_t)k * 2 + 1) * cols + c];
         }
@@ -404,12 +430,29 @@ __global__ __launch_bounds__(256) void norm_bwd_param_sum_k(const float *__restr
     lds[wave][1][lane] = sb;
     __syncthreads();
     if (wave == 0 && c < cols) {
-        if (dw) RowIO<DT>::st(dw, c, (lds[0][0][lane] + lds[1][0][lane]) + (lds[2][0][lane] + lds[3][0][lane]));
-        if (db) RowIO<DT>::st(db, c, (lds[0][1][lane] + lds[1][1][lane]) + (lds[2][1][lane] + lds[3][1][lane]));
+        float tw = 0.0f, tb = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            tw += lds[v][0][lane];
+            tb += lds[v][1][lane];
+        }
+        if (dw) RowIO<DT>::st(dw, c, tw);
+        if (db) RowIO<DT>::st(db, c, tb);
     }
 }
 
 int norm_bwd_chunks(int64_t rows) { return (int)(rows < 256 * 32 ? (rows + 31) / 32 : 256); }
+// the fused register kernel: one workgroup per CU's worth of waves, at most 256 partial row pairs
+constexpr int kFusedBlocks = 256;
+template <int NV> constexpr int fused_waves() { return NV <= 4 ? 16 : 8; }
+
+template <int DT, int MODE, int NV> void launch_norm_bwd_reg(const NormRowsBwd &p, float *part, int &chunks, hipStream_t st) {
+    typedef typename RowIO<DT>::S S;
+    constexpr int WAVES = fused_waves<NV>();
+    chunks = (int)((p.rows + WAVES - 1) / WAVES < kFusedBlocks ? (p.rows + WAVES - 1) / WAVES : kFusedBlocks);
+    hipLaunchKernelGGL((norm_bwd_dx_reg_k<DT, MODE, NV, WAVES>), dim3((unsigned)chunks), dim3(WAVES * 64), 0, st, (const S *)p.x,
+                       (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, (p.dw || p.db) ? part : nullptr, p.rows, p.eps);
+}
 
 template <int DT, int MODE> hipError_t launch_norm_bwd(const NormRowsBwd &p, hipStream_t st) {
     typedef typename RowIO<DT>::S S;
@@ -418,21 +461,22 @@ template <int DT, int MODE> hipError_t launch_norm_bwd(const NormRowsBwd &p, hip
     const bool vec = p.cols % 4 == 0 && al(p.x) && al(p.dy) && al(p.dx) && al(p.add);
     float *stats = (float *)p.workspace, *part = stats + p.rows * 2;
     dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
-#define ZK_BWD_REG(NV) hipLaunchKernelGGL((norm_bwd_dx_reg_k<DT, MODE, NV>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, p.eps)
     const bool al16 = vec && (!p.w || reinterpret_cast<uintptr_t>(p.w) % (4 * esz) == 0);
-    if (al16 && p.cols == 256) ZK_BWD_REG(1);
-    else if (al16 && p.cols == 512) ZK_BWD_REG(2);
-    else if (al16 && p.cols == 1024) ZK_BWD_REG(4);
-    else if (al16 && p.cols == 2048) ZK_BWD_REG(8);
-#undef ZK_BWD_REG
+    int chunks = 0; // > 0: the dx kernel has left this many partial row pairs in part
+    if (al16 && p.cols == 256) launch_norm_bwd_reg<DT, MODE, 1>(p, part, chunks, st);
+    else if (al16 && p.cols == 512) launch_norm_bwd_reg<DT, MODE, 2>(p, part, chunks, st);
+    else if (al16 && p.cols == 1024) launch_norm_bwd_reg<DT, MODE, 4>(p, part, chunks, st);
+    else if (al16 && p.cols == 2048) launch_norm_bwd_reg<DT, MODE, 8>(p, part, chunks, st);
     else if (vec) hipLaunchKernelGGL((norm_bwd_dx_k<DT, MODE, true>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, (int)p.cols, p.eps);
     else hipLaunchKernelGGL((norm_bwd_dx_k<DT, MODE, false>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, (int)p.cols, p.eps);
     if (p.dw || p.db) {
-        const int chunks = norm_bwd_chunks(p.rows);
-        const int64_t rpc = (p.rows + chunks - 1) / chunks;
-        if (vec) hipLaunchKernelGGL((norm_bwd_param_k<DT, true>), dim3((unsigned)((p.cols + 255) / 256), (unsigned)chunks), block, 0, st, (const S *)p.x, (const S *)p.dy, stats, part, p.rows, (int)p.cols, rpc);
-        else hipLaunchKernelGGL((norm_bwd_param_k<DT, false>), dim3((unsigned)((p.cols + 63) / 64), (unsigned)chunks), block, 0, st, (const S *)p.x, (const S *)p.dy, stats, part, p.rows, (int)p.cols, rpc);
-        hipLaunchKernelGGL((norm_bwd_param_sum_k<DT>), dim3((unsigned)((p.cols + 63) / 64)), block, 0, st, part, (S *)p.dw, (S *)p.db, (int)p.cols, chunks);
+        if (chunks == 0) {
+            chunks = norm_bwd_chunks(p.rows);
+            const int64_t rpc = (p.rows + chunks - 1) / chunks;
+            if (vec) hipLaunchKernelGGL((norm_bwd_param_k<DT, true>), dim3((unsigned)((p.cols + 255) / 256), (unsigned)chunks), block, 0, st, (const S *)p.x, (const S *)p.dy, stats, part, p.rows, (int)p.cols, rpc);
+            else hipLaunchKernelGGL((norm_bwd_param_k<DT, false>), dim3((unsigned)((p.cols + 63) / 64), (unsigned)chunks), block, 0, st, (const S *)p.x, (const S *)p.dy, stats, part, p.rows, (int)p.cols, rpc);
+        }
+        hipLaunchKernelGGL((norm_bwd_param_sum_k<DT>), dim3((unsigned)((p.cols + 63) / 64)), dim3(1024), 0, st, part, (S *)p.dw, (S *)p.db, (int)p.cols, chunks);
     }
     return hipGetLastError();
 }
@@ -466,8 +510,8 @@ hipError_t norm_rows(const NormRows &p, hipStream_t st) {
     return hipErrorInvalidValue;
 }
 
-uint64_t norm_rows_bwd_workspace_bytes(int64_t rows, int64_t cols) {
-    return (uint64_t)rows * 8 + (uint64_t)norm_bwd_chunks(rows) * 2 * (uint64_t)cols * 4;
+uint64_t norm_rows_bwd_workspace_bytes(int64_t rows, int64_t cols) { // row statistics, then up to 256 partial row pairs
+    return (uint64_t)rows * 8 + 256ull * 2 * (uint64_t)cols * 4;
 }
 
 hipError_t norm_rows_bwd(const NormRowsBwd &p, hipStream_t st) {
