@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HIP backend's hot path on one MI355X.
 
-Workload (BASELINE config 2): fused row softmax + row-sum + row-argmax over an f32
+Workload (benchmark configuration 2): fused row softmax + row-sum + row-argmax over an f32
 8192x4096 tensor, inputs resident in HBM. A "step" is one launch of the fused kernel
 through the C ABI (zhip_launch) on one buffer set; buffer sets rotate so no step finds
 its input in the 256 MB Infinity Cache left by the previous one.

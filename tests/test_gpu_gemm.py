@@ -54,7 +54,7 @@ def test_identity_and_exactness(hip, oracle):
 
 
 def test_config3_full_size(hip, oracle):
-    """BASELINE config 3: A, B uniform(-1,1) truncated to bf16, 4096^3, f32 out. The full
+    """Benchmark configuration 3: A, B uniform(-1,1) truncated to bf16, 4096^3, f32 out. The full
     oracle product takes minutes on the CPU, so 64 rows x 4096 columns are checked against
     the f64-accumulated oracle and the rest through linearity: C . v == A . (B . v)."""
     dev, pool = hip

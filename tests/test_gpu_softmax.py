@@ -54,7 +54,7 @@ def test_reference_goldens(hip, oracle):
 
 
 def test_config2_full_size(hip, oracle):
-    """BASELINE config: f32 8192x4096 drawn N(0, 3^2), seeded with zyx's generator."""
+    """The headline benchmark shape: f32 8192x4096 drawn N(0, 3^2), seeded with zyx's generator."""
     x = oracle.Rng(42069).randn((8192, 4096), 3.0)
     y, s, a = run_and_check(hip, oracle, x)
     yo, _, _ = oracle.softmax_rows(x)
