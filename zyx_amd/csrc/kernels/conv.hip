@@ -222,18 +222,34 @@ __global__ __launch_bounds__(256) void im2col_t_bf16_k(const uint16_t *__restric
 // in-bounds read, so the GEMM can gather its patch rows with plain 128-bit loads and no masks.
 __global__ __launch_bounds__(256) void pad_input_bf16_k(const uint16_t *__restrict__ x, uint16_t *__restrict__ xp, int H, int W,
                                                         int py, int px, int total) {
-    // 32-bit index arithmetic (total < 2^30); a thread writes two neighbouring elements as one word when rows are
-    // of even length (pairs then never straddle a row)
-    const int Hp = H + 2 * py, Wp = W + 2 * px, step = (Wp & 1) ? 1 : 2;
-    for (int i = (blockIdx.x * 256 + threadIdx.x) * step; i < total; i += gridDim.x * 256 * step) {
-        const int plane = i / (Hp * Wp), rem = i - plane * (Hp * Wp), yy = rem / Wp - py, xx = rem % Wp - px;
-        const uint16_t *row = x + ((int64_t)plane * H + yy) * W;
-        const bool rok = yy >= 0 && yy < H;
-        const uint32_t a = (rok && xx >= 0 && xx < W) ? row[xx] : 0u;
-        if (step == 2) {
-            const uint32_t b = (rok && xx + 1 >= 0 && xx + 1 < W) ? row[xx + 1] : 0u;
-            *(uint32_t *)(xp + i) = a | (b << 16);
-        } else xp[i] = (uint16_t)a;
+    // 32-bit index arithmetic (total < 2^30). A thread fills 8 consecutive elements of the padded array (one 128-bit
+    // store; xp is 16-byte aligned): the position is decoded once by division and then stepped across row and
+    // plane ends, the 8 source elements are neighbouring 2-byte loads.
+    const int Hp = H + 2 * py, Wp = W + 2 * px;
+    for (int i = (blockIdx.x * 256 + threadIdx.x) * 8; i < total; i += gridDim.x * 256 * 8) {
+        int plane = i / (Hp * Wp);
+        const int rem = i - plane * (Hp * Wp);
+        int yy = rem / Wp, xx = rem - yy * Wp;
+        uint32_t v[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int sy = yy - py, sx = xx - px;
+            v[e] = (i + e < total && sy >= 0 && sy < H && sx >= 0 && sx < W) ? x[((int64_t)plane * H + sy) * W + sx] : 0u;
+            if (++xx == Wp) {
+                xx = 0;
+                if (++yy == Hp) {
+                    yy = 0;
+                    ++plane;
+                }
+            }
+        }
+        if (i + 8 <= total) {
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            u32x4 w = {v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16)};
+            *(u32x4 *)(xp + i) = w;
+        } else {
+            for (int e = 0; i + e < total; e++) xp[i + e] = (uint16_t)v[e];
+        }
     }
 }
 
@@ -273,7 +289,7 @@ hipError_t conv2d(const Conv2d &p, hipStream_t st) {
         if (conv_gathers_in_gemm(p)) {
             const int Hp = p.H + 2 * p.py, Wp = p.W + 2 * p.px;
             const int total = p.N * p.C * Hp * Wp; // < 2^30, checked by conv_gathers_in_gemm
-            int blocks = (total / ((Wp & 1) ? 1 : 2) + 255) / 256;
+            int blocks = ((total + 7) / 8 + 255) / 256;
             if (blocks > 256 * 64) blocks = 256 * 64;
             hipLaunchKernelGGL(pad_input_bf16_k, dim3((unsigned)blocks), dim3(256), 0, st, (const uint16_t *)p.x, a, p.H, p.W, p.py, p.px, total);
             ConvGather &c = g.gather;
