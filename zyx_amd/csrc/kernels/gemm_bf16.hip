@@ -347,6 +347,9 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
     };
 #pragma unroll
     for (int j = 0; j < NJ; j++) {
+        // the residual is added to the finished value as written, never fused into the activation's last multiply:
+        // f32 and bf16 results of one product then differ by the store's truncation only, whatever the code shape
+#pragma clang fp contract(off)
         const int col = n0 + wn * WN + j * 32 + col_in;
         float bv = 0.0f;
         if (EPI >= 1) {
@@ -378,13 +381,23 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int rbase = m0 + wm * 128 + i * 32 + row_in;
+                // 128-wide tiles: the residual values of the block are requested together, one memory latency per 16
+                // loads (the 256-wide tile has no registers to spare for that: it would spill)
+                float rv[BNV == 128 ? 16 : 1];
+                if (BNV == 128 && R) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int row = rbase + (r >> 2) * 8 + (r & 3);
+                        rv[BNV == 128 ? r : 0] = (TAIL && (row >= M || col >= N)) ? 0.0f : R[(int64_t)row * N + col];
+                    }
+                }
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int row = rbase + (r >> 2) * 8 + (r & 3);
                     if (TAIL && (row >= M || col >= N)) continue;
                     const int64_t o = (int64_t)row * N + col;
                     float v = finish(acc[i][j][r], bv);
-                    if (R) v += R[o];
+                    if (R) v += BNV == 128 ? rv[BNV == 128 ? r : 0] : R[o];
                     C[o] = v;
                 }
             }
@@ -394,6 +407,21 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
             uint16_t *C = (uint16_t *)Cv;
             const uint16_t *R = (const uint16_t *)residual;
             const int odd = lane & 1;
+            // 128-wide tiles: the residual words of the whole column block are requested before the first is used,
+            // one memory latency per 32 loads instead of one per load (the accumulators leave the compiler too few
+            // registers to do this by itself; the 256-wide tile has none to spare at all and keeps load-then-use)
+            constexpr bool BATCH = BNV == 128;
+            uint32_t rr[BATCH ? 4 : 1][BATCH ? 8 : 1];
+            if (BATCH && R) {
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r += 2) {
+                        const int row = m0 + wm * 128 + i * 32 + row_in + (r >> 2) * 8 + (r & 3) + odd;
+                        rr[BATCH ? i : 0][BATCH ? r >> 1 : 0] =
+                            (TAIL && (row >= M || col - odd + 1 >= N)) ? 0u : *(const uint32_t *)(R + (int64_t)row * N + (col - odd));
+                    }
+            }
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int rbase = m0 + wm * 128 + i * 32 + row_in;
@@ -405,9 +433,9 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
                     if (TAIL && (rbase + (r >> 2) * 8 + (r & 3) + odd >= M || col - odd + 1 >= N)) continue; // N is even
                     const int64_t o = (int64_t)(rbase + (r >> 2) * 8 + (r & 3) + odd) * N + (col - odd);
                     if (R) {
-                        const uint32_t rr = *(const uint32_t *)(R + o);
-                        lo += __uint_as_float(rr << 16);
-                        hi += __uint_as_float(rr & 0xffff0000u);
+                        const uint32_t w = BATCH ? rr[BATCH ? i : 0][BATCH ? r >> 1 : 0] : *(const uint32_t *)(R + o);
+                        lo += __uint_as_float(w << 16);
+                        hi += __uint_as_float(w & 0xffff0000u);
                     }
                     *(uint32_t *)(C + o) = (uint32_t)f32_to_bf16_trunc(lo) | ((uint32_t)f32_to_bf16_trunc(hi) << 16);
                 }
