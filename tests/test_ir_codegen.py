@@ -155,3 +155,38 @@ def test_refusals():
     k._next = 0
     k.const_idx(2)
     refused(k, "defined twice")
+
+
+def test_mutated_images_are_refused_or_compiled_never_crash():
+    """The image comes from outside the library: random corruptions of valid images (opcodes, operand ids, dtypes,
+    lengths, the header) must each end in source text or a KernelCompilation reason."""
+    import random
+    rnd = random.Random(1234)
+    bases = [k.to_bytes() for k in kernels().values()]
+    outcomes = {"ok": 0, "refused": 0}
+    for trial in range(3000):
+        img = bytearray(rnd.choice(bases))
+        for _ in range(rnd.randint(1, 4)):
+            kind = rnd.random()
+            if len(img) < 48:
+                break
+            if kind < 0.6:      # one field of one op
+                n_ops = (len(img) - 16) // 32
+                op = rnd.randrange(max(n_ops, 1))
+                off = 16 + 32 * op + rnd.choice([0, 4, 6, 8, 12, 16, 20, 24])
+                val = rnd.choice([0, 1, 2, 3, 7, 16, 0xFFFF, 0xFFFFFFFF, rnd.getrandbits(32)])
+                img[off:off + 2] = (val & 0xFFFF).to_bytes(2, "little")
+            elif kind < 0.8:    # any byte
+                img[rnd.randrange(len(img))] = rnd.getrandbits(8)
+            elif kind < 0.9:    # truncation
+                del img[rnd.randrange(len(img)):]
+            else:               # header counts
+                img[4:12] = rnd.getrandbits(64).to_bytes(8, "little")
+        try:
+            src = generate_source(bytes(img))
+            assert "zir_kernel" in src
+            outcomes["ok"] += 1
+        except BackendError as e:
+            assert e.status == ErrorStatus.KernelCompilation and str(e)
+            outcomes["refused"] += 1
+    assert outcomes["ok"] > 50 and outcomes["refused"] > 500, outcomes

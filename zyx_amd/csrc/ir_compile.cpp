@@ -347,7 +347,10 @@ bool ir_generate(const void *image, uint64_t bytes, IrProgram &out, std::string 
             if (!reg_type(o.dtype)) return g.fail(i, "storage of unknown dtype");
             if (o.aux != ZHIP_IR_SCOPE_LOCAL && o.aux != ZHIP_IR_SCOPE_REGISTER)
                 return g.fail(i, "storage must be local or register scoped");
-            if (o.imm == 0 || o.imm > (1u << 24)) return g.fail(i, "storage length out of range");
+            // local memory: what one workgroup can have on this part (160 KiB); register arrays: a bound that keeps
+            // a corrupt length from asking the compiler for gigabytes of scratch
+            if (o.imm == 0 || (o.aux == ZHIP_IR_SCOPE_LOCAL ? o.imm * (uint64_t)(is_f16ish(o.dtype) ? 4 : mem_bytes(o.dtype)) > 160u * 1024 : o.imm > 16384))
+                return g.fail(i, "storage length out of range");
             if (o.aux == ZHIP_IR_SCOPE_LOCAL && depth) return g.fail(i, "local storage must be declared outside loops and branches");
             v.cls = Val::Storage;
             v.dtype = o.dtype;
