@@ -171,3 +171,29 @@ def test_launches_of_one_program_do_not_overlap_on_its_workspace(hip, oracle):
     for xb, ob in bufs:
         pool.deallocate(xb, [])
         pool.deallocate(ob, [])
+
+
+def test_calls_from_several_threads(hip, oracle):
+    """zyx calls its backends from whichever user thread holds the runtime mutex (zyx/src/lib.rs:96): the library is
+    not thread-affine. Four threads each upload, launch a softmax of their own data and read it back, 20 times."""
+    import threading
+    from zyx_amd.kernels import softmax_rows
+    dev, pool = hip
+    errors = []
+
+    def work(seed):
+        try:
+            x = (3 * oracle.Rng(seed).randn((64, 512))).astype(np.float32)
+            want, _, want_arg = oracle.softmax_rows(x)
+            for _ in range(20):
+                y, s, a = softmax_rows(dev, pool, x)
+                assert np.allclose(y, want, rtol=1e-5, atol=1e-37) and np.array_equal(a, want_arg)
+        except Exception as e:  # surfaced in the main thread below
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=work, args=(100 + i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
