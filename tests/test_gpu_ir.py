@@ -288,3 +288,25 @@ def test_optimised_example_kernels(hip, oracle):
         (g, c), = both(hip, ir_examples.scaled_exp2(n, dt, vlen=vlen), [arr, np.zeros_like(arr)])
         gf, cf = (g, c) if dt == DType.F32 else (oracle.bf16_to_f32(g), oracle.bf16_to_f32(c))
         assert np.all(np.abs(gf - cf) <= (1e-5 if dt == DType.F32 else 2.0 ** -7) * np.abs(cf))
+
+
+def test_autotune_call_sequence(hip):
+    """What zyx's autotuner does with a candidate kernel (zyx/src/kernel/autotune.rs:358-430, 775-798): buffers of
+    ones plus one spare element, dynamic dimensions stored as 42, compile, a timed launch, release."""
+    dev, pool = hip
+    k = K.dynamic_rows(64)
+    rows = pool.store_variable(DType.I64, 42)
+    x, e1 = to_device(pool, np.ones(42 * 64 + 1, np.float32))
+    y, e2 = to_device(pool, np.ones(42 * 64 + 1, np.float32))
+    pool.sync_events([e1, e2])
+    prog = dev.compile(k.to_bytes())
+    ns = dev.time_kernel(prog, [rows, x, y])
+    assert 0 < ns < 1e9
+    got = to_host(pool, y, (42 * 64 + 1,), np.float32, [])
+    assert np.array_equal(got[:-1].reshape(42, 64), 1.0 + np.arange(42, dtype=np.float32)[:, None] * np.ones((1, 64), np.float32))
+    assert got[-1] == 1.0          # the spare element is not touched
+    us = dev.profile_kernel(prog, [[rows, x, y]], 5)
+    assert us > 0
+    dev.release(prog)
+    for b in (rows, x, y):
+        pool.deallocate(b, [])
