@@ -254,3 +254,25 @@ def test_bf16_edge_tiles_linear(hip, oracle, mnk, epilogue):
                                              residual=residual, **kw)
         assert np.array_equal(tail, guard)
         assert np.array_equal(got16, oracle.f32_to_bf16(got32))
+
+
+@pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
+def test_bf16_column_blocks(hip, oracle, trans_a, trans_b):
+    """4096 x 6144: 384 wide tiles would fill one and a half rounds of the 256 CUs, so the product is launched as two
+    blocks of columns (4096 of wide tiles, 2048 of narrow ones) that share A and write one C: every layout, with
+    bias + residual, f32 and bf16 results."""
+    dev, pool = hip
+    m, n, k = 4096, 6144, 64
+    a, b = make(oracle, m, n, k, 77, trans_a, trans_b)
+    r = oracle.Rng(78)
+    bias = oracle.f32_to_bf16(r.uniform((n,), -1, 1))
+    res = oracle.f32_to_bf16(r.randn((m, n)))
+    want, mag = reference(oracle, a, b, trans_a, trans_b)
+    got = gemm(dev, pool, a, b, trans_a=trans_a, trans_b=trans_b)
+    assert np.all(np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-5 * mag)
+    w = want + oracle.bf16_to_f32(bias).astype(np.float64) + oracle.bf16_to_f32(res).astype(np.float64)
+    kw = dict(bias=bias, epilogue="bias", bias_dtype=DType.BF16, trans_a=trans_a, trans_b=trans_b)
+    got32 = gemm(dev, pool, a, b, out_dtype=DType.F32, residual=oracle.bf16_to_f32(res), **kw)
+    assert np.all(np.abs(got32 - w) <= 1e-3 * np.abs(w) + 2e-5 * mag + 1e-6)
+    got16 = gemm(dev, pool, a, b, out_dtype=DType.BF16, residual=res, **kw)
+    assert np.array_equal(got16, oracle.f32_to_bf16(got32))

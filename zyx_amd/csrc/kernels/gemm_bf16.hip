@@ -134,7 +134,9 @@ template <bool AT, bool BT, int EPI, int BNV, int PLANE, bool TAIL>
 __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                       void *__restrict__ Cv, const void *__restrict__ bias,
                                                       const void *__restrict__ residual, int bias_dtype, int out_bf16,
-                                                      int M, int N, int K, int splits, int plane, const ConvGather g) {
+                                                      int M, int N, int K, int ldn, int splits, int plane, const ConvGather g) {
+    // ldn: elements between rows of C, of the residual and of a [K, N] operand B: N, or the full width when this
+    // launch computes a block of columns of a wider product
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
     constexpr int NJ = BNV / 64;                 // 32-column MFMA blocks per wave
@@ -153,7 +155,7 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
     const int split = blockIdx.x / (tiles_m * tiles_n);
     const int k_len = K / splits;
     A += (int64_t)split * k_len * (AT ? M : 1);
-    B += (int64_t)split * k_len * (BT ? 1 : N);
+    B += (int64_t)split * k_len * (BT ? 1 : ldn);
     if (splits > 1) Cv = (float *)Cv + (int64_t)split * M * N;
     int tm, tn;
     {
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
     // offset plus constants.
     typedef typename std::conditional<AT, TileMN<256>, TileKC>::type TA;
     typedef typename std::conditional<BT, TileKC, TileMN<BNV>>::type TB;
-    const int64_t lda = AT ? M : K, ldb = BT ? K : N;
+    const int64_t lda = AT ? M : K, ldb = BT ? K : ldn;
     uint32_t oa[8], ob[NB];
 #pragma unroll
     for (int i = 0; i < 8; i++) {
@@ -388,14 +390,14 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const int row = rbase + (r >> 2) * 8 + (r & 3);
-                        rv[BNV == 128 ? r : 0] = (TAIL && (row >= M || col >= N)) ? 0.0f : R[(int64_t)row * N + col];
+                        rv[BNV == 128 ? r : 0] = (TAIL && (row >= M || col >= N)) ? 0.0f : R[(int64_t)row * ldn + col];
                     }
                 }
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int row = rbase + (r >> 2) * 8 + (r & 3);
                     if (TAIL && (row >= M || col >= N)) continue;
-                    const int64_t o = (int64_t)row * N + col;
+                    const int64_t o = (int64_t)row * ldn + col;
                     float v = finish(acc[i][j][r], bv);
                     if (R) v += BNV == 128 ? rv[BNV == 128 ? r : 0] : R[o];
                     C[o] = v;
@@ -419,7 +421,7 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
                     for (int r = 0; r < 16; r += 2) {
                         const int row = m0 + wm * 128 + i * 32 + row_in + (r >> 2) * 8 + (r & 3) + odd;
                         rr[BATCH ? i : 0][BATCH ? r >> 1 : 0] =
-                            (TAIL && (row >= M || col - odd + 1 >= N)) ? 0u : *(const uint32_t *)(R + (int64_t)row * N + (col - odd));
+                            (TAIL && (row >= M || col - odd + 1 >= N)) ? 0u : *(const uint32_t *)(R + (int64_t)row * ldn + (col - odd));
                     }
             }
 #pragma unroll
@@ -431,7 +433,7 @@ __global__ __launch_bounds__(256, 1) void gemm_bf16_k(const uint16_t *__restrict
                     const float got = dpp_f32<kDppQuadXor1>(odd ? v0 : v1);
                     float lo = odd ? got : v0, hi = odd ? v1 : got;
                     if (TAIL && (rbase + (r >> 2) * 8 + (r & 3) + odd >= M || col - odd + 1 >= N)) continue; // N is even
-                    const int64_t o = (int64_t)(rbase + (r >> 2) * 8 + (r & 3) + odd) * N + (col - odd);
+                    const int64_t o = (int64_t)(rbase + (r >> 2) * 8 + (r & 3) + odd) * ldn + (col - odd);
                     if (R) {
                         const uint32_t w = BATCH ? rr[BATCH ? i : 0][BATCH ? r >> 1 : 0] : *(const uint32_t *)(R + o);
                         lo += __uint_as_float(w << 16);
@@ -479,13 +481,13 @@ __global__ __launch_bounds__(256) void gemm_splitk_fold_k(const float *__restric
 }
 
 template <bool AT, bool BT, int BNV, bool TAIL> hipError_t launch_epi(const GemmBf16 &p, hipStream_t st) {
-    const int splits = gemm_bf16_splits(p.M, p.N, p.K);
+    const int splits = p.ldn ? 1 : gemm_bf16_splits(p.M, p.N, p.K); // a column block of a wider product is never K-split
     if (p.plane && (TAIL || splits > 1 || p.residual || p.plane % 4 || p.M % p.plane)) return hipErrorInvalidValue;
     dim3 grid((unsigned)(((p.M + BM - 1) / BM) * ((p.N + BNV - 1) / BNV) * splits)), block(256);
     if (splits > 1) {
         if (!p.workspace) return hipErrorInvalidValue;
         hipLaunchKernelGGL((gemm_bf16_k<AT, BT, 0, BNV, 0, TAIL>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, (const uint16_t *)p.B,
-                           p.workspace, nullptr, nullptr, 0, 0, (int)p.M, (int)p.N, (int)p.K, splits, 0, ConvGather{});
+                           p.workspace, nullptr, nullptr, 0, 0, (int)p.M, (int)p.N, (int)p.K, (int)p.N, splits, 0, ConvGather{});
         const int64_t MN = p.M * p.N;
         hipLaunchKernelGGL(gemm_splitk_fold_k, dim3((unsigned)((MN / 4 + 255) / 256)), block, 0, st, (const float *)p.workspace, p.C,
                            p.bias, p.residual, p.epilogue, p.bias_dtype, p.out_bf16, MN, (int)p.N, splits);
@@ -496,7 +498,7 @@ template <bool AT, bool BT, int BNV, bool TAIL> hipError_t launch_epi(const Gemm
         if (!(AT && BT) || p.epilogue > 2) return hipErrorInvalidValue;
 #define ZK_GEMM_PL(E, G)                                                                                              \
     hipLaunchKernelGGL((gemm_bf16_k<true, true, E, BNV, G, false>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, \
-                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, p.plane, p.gather);
+                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, (int)p.N, 1, p.plane, p.gather);
         if (p.gather.khw) {
             switch (p.epilogue) {
             case 0: ZK_GEMM_PL(0, 2) break;
@@ -515,7 +517,7 @@ template <bool AT, bool BT, int BNV, bool TAIL> hipError_t launch_epi(const Gemm
     }
 #define ZK_GEMM(E)                                                                                                    \
     hipLaunchKernelGGL((gemm_bf16_k<AT, BT, E, BNV, 0, TAIL>), grid, block, lds_bytes(BNV), st, (const uint16_t *)p.A, \
-                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, 1, 0, ConvGather{});
+                       (const uint16_t *)p.B, p.C, p.bias, p.residual, p.bias_dtype, p.out_bf16, (int)p.M, (int)p.N, (int)p.K, (int)(p.ldn ? p.ldn : p.N), 1, 0, ConvGather{});
     switch (p.epilogue) {
     case 0: ZK_GEMM(0) break;
     case 1: ZK_GEMM(1) break;
@@ -606,10 +608,42 @@ uint64_t gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     return s > 1 ? (uint64_t)s * M * N * 4 : 0;
 }
 
-hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t st) {
-    if (!gemm_bf16_supported(p.M, p.N, p.K, p.trans_a, p.trans_b, p.out_bf16)) return hipErrorInvalidValue;
+namespace {
+hipError_t launch_layout(const GemmBf16 &p, hipStream_t st) {
     if (p.trans_a) return p.trans_b ? launch_width<true, true>(p, st) : launch_width<true, false>(p, st);
     return p.trans_b ? launch_width<false, true>(p, st) : launch_width<false, false>(p, st);
+}
+} // namespace
+
+// Columns of a tile-aligned product whose 256-wide tiles fill whole rounds of the 256 CUs, when the rest would leave
+// a second round mostly idle and fits one round of 128-wide tiles (e.g. 8192 x 3072: 384 tiles = 1.5 rounds become
+// 2048 columns = 256 tiles and 1024 columns = 256 narrower, cheaper tiles). 0: compute the product in one launch.
+int64_t gemm_bf16_column_split(int64_t M, int64_t N, int64_t K) {
+    if (M % BM || N % 256 || gemm_bf16_tile_n(M, N) != 256 || gemm_bf16_splits(M, N, K) != 1) return 0;
+    const int64_t tm = M / BM, tiles = tm * (N / 256);
+    if (tiles <= 256 || tiles % 256 == 0 || ((tiles / 256) * 256) % tm) return 0;
+    const int64_t n1 = (tiles / 256) * 256 / tm * 256, n2 = N - n1;
+    if (n2 <= 0 || tm * (n2 / 128) > 256 || gemm_bf16_tile_n(M, n2) != 128 || gemm_bf16_splits(M, n2, K) != 1) return 0;
+    return n1;
+}
+
+hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t st) {
+    if (!gemm_bf16_supported(p.M, p.N, p.K, p.trans_a, p.trans_b, p.out_bf16)) return hipErrorInvalidValue;
+    const int64_t n1 = (p.plane || p.ldn) ? 0 : gemm_bf16_column_split(p.M, p.N, p.K);
+    if (n1) {
+        GemmBf16 a = p, b = p;
+        a.N = n1;
+        a.ldn = b.ldn = p.N;
+        b.N = p.N - n1;
+        const int64_t csz = p.out_bf16 ? 2 : 4, bsz = p.bias_dtype == DT_BF16 ? 2 : 4;
+        b.B = (const uint16_t *)p.B + (p.trans_b ? n1 * p.K : n1);
+        b.C = (char *)p.C + n1 * csz;
+        if (p.bias) b.bias = (const char *)p.bias + n1 * bsz;
+        if (p.residual) b.residual = (const char *)p.residual + n1 * csz;
+        hipError_t e = launch_layout(a, st);
+        return e != hipSuccess ? e : launch_layout(b, st);
+    }
+    return launch_layout(p, st);
 }
 
 } // namespace zk

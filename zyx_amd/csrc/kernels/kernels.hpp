@@ -73,6 +73,7 @@ struct GemmBf16 {
     int bias_dtype;    // DT_BF16 or DT_F32
     int out_bf16;
     int plane; // 0, or C is stored [M / plane, N, plane] (rows of one group of `plane` are contiguous per column)
+    int64_t ldn; // 0, or the launch computes N columns of a product ldn columns wide (row stride of C, residual, [K,N] B)
     ConvGather gather; // with plane != 0 and gather.khw != 0: A is the padded input, not a matrix
     const void *A, *B, *bias, *residual; // residual may be null
     void *C;
