@@ -47,6 +47,7 @@ class MLPTrainStep:
             return p
 
         x, y = buf("x", batch * n_in), buf("labels", batch)
+        x2, y2 = buf("x2", batch * n_in), buf("labels2", batch)  # the batch of the other plan (see below)
         w1, b1, w2, b2 = buf("w1", hidden * n_in), buf("b1", hidden), buf("w2", n_out * hidden), buf("b2", n_out)
         h, logits = buf("h", batch * hidden), buf("logits", batch * n_out)
         loss, mean_loss, dlogits = buf("loss", batch), buf("mean_loss", 1), buf("dlogits", batch * n_out)
@@ -89,14 +90,33 @@ class MLPTrainStep:
             (sgd(1, n_out), [b2, db2, nb2]),
         ]
         # the updated parameters are written to fresh buffers (a kernel's outputs never alias its
-        # inputs); the two parameter sets swap roles every step, so two plans alternate
-        swap = {w1: nw1, b1: nb1, w2: nw2, b2: nb2, nw1: w1, nb1: b1, nw2: w2, nb2: b2}
+        # inputs); the two parameter sets swap roles every step, so two plans alternate. Each plan also reads its
+        # own batch buffers: the next batch is copied in while the current step still runs.
+        swap = {w1: nw1, b1: nb1, w2: nw2, b2: nb2, nw1: w1, nb1: b1, nw2: w2, nb2: b2, x: x2, y: y2}
         nodes_b = [(p, [swap.get(b, b) for b in bufs]) for p, bufs in nodes]
         self.nodes = nodes
         self._plans = [dev.create_plan(nodes), dev.create_plan(nodes_b)]
         self._param_sets = [dict(w1=w1, b1=b1, w2=w2, b2=b2), dict(w1=nw1, b1=nb1, w2=nw2, b2=nb2)]
+        self._batch_bufs = [(x, y), (x2, y2)]
         self._cur = 0
-        self._pending = []
+        self._plan_ev = [None, None]  # event of the last launch of each plan, until something waits for it
+        self._copy_ev = []            # uploads of the batch the next step reads
+        self._batch_no = 0            # batches set so far, and which of them each pair of batch buffers holds
+        self._holds = [0, 0]
+
+    @property
+    def _pending(self):
+        """Every event the host has to wait for before it touches a buffer of the step."""
+        return self._copy_ev + [e for e in self._plan_ev if e is not None]
+
+    @_pending.setter
+    def _pending(self, events):
+        assert not events, "outstanding events are tracked per plan; only clearing is supported"
+        self._copy_ev, self._plan_ev = [], [None, None]
+
+    def _take_plan_event(self, parity: int):
+        ev, self._plan_ev[parity] = self._plan_ev[parity], None
+        return [ev] if ev is not None else []
 
     # -- host <-> device ------------------------------------------------------------------------
     def set_params(self, w1, b1, w2, b2):
@@ -106,45 +126,74 @@ class MLPTrainStep:
         self.pool.sync_events(evs)
 
     def set_batch(self, x, labels):
-        """Uploads wait for the previous step: it may still be reading x / labels."""
+        """Uploads wait for the step before the previous one: it read the same pair of batch buffers."""
         self._x = np.ascontiguousarray(x, np.float32)
         self._y = np.ascontiguousarray(labels, np.int32)
-        e1 = self.pool.host_to_pool(self._x, self._bufs["x"], self._pending)
-        e2 = self.pool.host_to_pool(self._y, self._bufs["labels"], [])
-        self._pending = [e1, e2]
+        xb, yb = self._batch_bufs[self._cur]
+        if self._copy_ev:  # a batch that no step consumed
+            self.pool.sync_events(self._copy_ev)
+        e1 = self.pool.host_to_pool(self._x, xb, self._take_plan_event(self._cur))
+        e2 = self.pool.host_to_pool(self._y, yb, [])
+        self._copy_ev = [e1, e2]
+        self._batch_no += 1
+        self._holds[self._cur] = self._batch_no
 
     def set_batch_from_device(self, x_buf: int, y_buf: int, index: int):
         """Batch `index` of a dataset already resident in the pool (x_buf f32 [n, batch, n_in], y_buf i32
         [n, batch]): two device-to-device range copies, as Tensor::index_select feeds batches in
         zyx-examples/examples/mnist.rs:62-64."""
         b, n_in, _, _ = self.shape
-        e1 = self.pool.copy_range(x_buf, index * b * n_in * 4, self._bufs["x"], 0, b * n_in * 4, self._pending)
-        e2 = self.pool.copy_range(y_buf, index * b * 4, self._bufs["labels"], 0, b * 4, [])
-        self._pending = [e1, e2]
+        xb, yb = self._batch_bufs[self._cur]
+        if self._copy_ev:
+            self.pool.sync_events(self._copy_ev)
+        e1 = self.pool.copy_range(x_buf, index * b * n_in * 4, xb, 0, b * n_in * 4, self._take_plan_event(self._cur))
+        e2 = self.pool.copy_range(y_buf, index * b * 4, yb, 0, b * 4, [])
+        self._copy_ev = [e1, e2]
+        self._batch_no += 1
+        self._holds[self._cur] = self._batch_no
+
+    def _same_batch_again(self):
+        """A step without a new batch reads the last one: it is copied over from the other plan's buffers."""
+        if self._holds[self._cur] == self._batch_no:
+            return
+        b, n_in, _, _ = self.shape
+        (sx, sy), (dx, dy) = self._batch_bufs[self._cur ^ 1], self._batch_bufs[self._cur]
+        e1 = self.pool.copy_range(sx, 0, dx, 0, b * n_in * 4, self._copy_ev + self._take_plan_event(self._cur))
+        e2 = self.pool.copy_range(sy, 0, dy, 0, b * 4, [])  # the pool's copies run in order
+        self._copy_ev = [e1, e2]
+        self._holds[self._cur] = self._batch_no
 
     def step(self):
         """One forward + backward + update: a single plan launch."""
-        ev = self.dev.launch_plan(self._plans[self._cur], self._pending)
-        self._pending = [ev]
+        self._same_batch_again()
+        old = self._take_plan_event(self._cur)  # only there when the batch buffers were not written since
+        ev = self.dev.launch_plan(self._plans[self._cur], self._copy_ev + old)
+        self._copy_ev = []
+        self._plan_ev[self._cur] = ev
         self._cur ^= 1
 
     def step_unplanned(self):
         """The same list issued node by node through HIPDevice::launch (no cached plan)."""
+        self._same_batch_again()
         nodes = self.nodes if self._cur == 0 else None
         if nodes is None:
             cur, oth = self._param_sets[1], self._param_sets[0]
             swap = {**{oth[k]: cur[k] for k in cur}, **{cur[k]: oth[k] for k in cur}}
+            swap.update(zip(self._batch_bufs[0], self._batch_bufs[1]))
             nodes = [(p, [swap.get(b, b) for b in bufs]) for p, bufs in self.nodes]
-        ev = self._pending
+        ev = self._pending  # launch by launch: simply after everything outstanding
+        self._pending = []
         for p, bufs in nodes:
             ev = [self.dev.launch(p, self.pool, bufs, ev)]
-        self._pending = ev
+        self._plan_ev[self._cur] = ev[0]
         self._cur ^= 1
 
     def read(self, name: str, shape) -> np.ndarray:
         params = self._param_sets[self._cur]
         out = np.empty(shape, np.int32 if name == "labels" else np.float32)
-        self.pool.pool_to_host(params.get(name, self._bufs.get(name)), out, self._pending)
+        last = self._batch_bufs[self._cur ^ 1]  # the batch the most recent step read
+        src = params.get(name, {"x": last[0], "labels": last[1]}.get(name, self._bufs.get(name)))
+        self.pool.pool_to_host(src, out, self._pending)
         self._pending = []
         return out
 
