@@ -1,0 +1,150 @@
+"""zyx_amd.graph on the GPU: graphs and their gradients realised by `Tape` (lowered kernels compiled and launched
+through the C ABI) against the CPU evaluation of the same graph (oracle/graph_eval.py) and the gradients
+zyx/tests/11_autograd.rs asserts. Bar: bit-exact for integer graphs and for float graphs made of + - * / max,
+comparisons, casts and movement ops (same serial order, no contraction); within 1e-5 relative (f32) / 1e-12 (f64)
+where exp / log / sin / cos / pow / sqrt are involved."""
+import numpy as np
+import pytest
+
+from graph_cases import CASES, mixed_graph, mlp_graph
+from oracle import graph_eval
+from zyx_amd import DType
+from zyx_amd.graph import Tape, storage_dtype
+from zyx_amd.ir import BOp, UOp
+
+pytestmark = pytest.mark.gpu
+
+_EXACT_UOPS = (UOp.Neg, UOp.Reciprocal, UOp.Floor, UOp.Trunc, UOp.Abs, UOp.BitNot)
+
+
+def on_device(hip, build, *args, **kw):
+    dev, pool = hip
+    tape, leaves = Tape(dev, pool), {}
+
+    def leaf(array, dtype):
+        a = np.ascontiguousarray(np.asarray(array).astype(storage_dtype(dtype)))
+        nid = tape.tensor(a, dtype)
+        leaves[nid] = a
+        return nid
+
+    return tape, leaves, build(tape.graph, leaf, *args, **kw)
+
+
+def is_exact(g, nodes):
+    """No transcendental op anywhere below these nodes."""
+    seen, stack = set(), list(nodes)
+    while stack:
+        i = stack.pop()
+        if i in seen:
+            continue
+        seen.add(i)
+        n = g[i]
+        if (n.kind == "unary" and n.op not in _EXACT_UOPS) or (n.kind == "binary" and n.op == BOp.Pow):
+            return False
+        stack.extend(n.src)
+    return True
+
+
+def compare(tape, leaves, nodes, rtol):
+    g = tape.graph
+    want = graph_eval.evaluate(g.nodes, leaves, nodes)
+    tape.realize(nodes)
+    for nid in nodes:
+        got = tape.numpy(nid)
+        assert got.dtype == want[nid].dtype and got.shape == want[nid].shape
+        if is_exact(g, [nid]):
+            assert np.array_equal(got, want[nid], equal_nan=True), nid
+        else:
+            np.testing.assert_allclose(got, want[nid], rtol=rtol, atol=0)
+    return want
+
+
+@pytest.mark.parametrize("name,build", CASES, ids=[c[0] for c in CASES])
+def test_reference_gradients(hip, name, build):
+    tape, leaves, (target, sources, expected) = on_device(hip, build)
+    try:
+        grads = tape.gradient(target, sources)
+        f64 = any(tape.graph[s].dtype == DType.F64 for s in sources)
+        compare(tape, leaves, grads + [target], 1e-12 if f64 else 1e-5)
+        for gid, src, exp in zip(grads, sources, expected):
+            if exp is None:
+                continue
+            got = tape.numpy(gid)
+            if tape.graph[src].dtype in (DType.F32, DType.F64):
+                np.testing.assert_allclose(got, exp, rtol=1e-12 if f64 else 1e-5, atol=0)
+            else:
+                assert got.tolist() == np.asarray(exp).tolist()
+    finally:
+        tape.close()
+
+
+@pytest.mark.parametrize("dtype,rtol", [(DType.F64, 1e-11), (DType.F32, 2e-4)])
+def test_every_rule(hip, dtype, rtol):
+    """f32: the loss sums exponentials of sines of products, so a few ulp in one function move the result by more
+    than 1e-5 of some gradient entries that cancel; the f64 run holds the tight bar."""
+    tape, leaves, (loss, sources) = on_device(hip, mixed_graph, dtype=dtype)
+    try:
+        grads = tape.gradient(loss, sources)
+        compare(tape, leaves, grads + [loss], rtol)
+    finally:
+        tape.close()
+
+
+@pytest.mark.parametrize("shape", [dict(batch=8, n_in=12, hidden=16, n_out=5), dict(batch=64, n_in=784, hidden=128, n_out=10)])
+def test_mlp_gradients(hip, shape):
+    """zz_bw_relu_matmul (11_autograd.rs:908-927), at a small size and at the size of the MNIST network: gradients
+    of sum(logits) and one SGD step `w - g * lr` realised on the device, against the evaluation of the same graph
+    (exact: only + * and comparisons) and the closed-form backward products in f64."""
+    tape, leaves, (loss, sources, (x, w1, b1, w2, b2)) = on_device(hip, mlp_graph, **shape)
+    try:
+        g = tape.graph
+        grads = tape.gradient(loss, sources)
+        lr = g.const(0.01, DType.F32)
+        new = [g.binary(s, g.binary(gr, lr, BOp.Mul), BOp.Sub) for s, gr in zip(sources, grads)]
+        want = compare(tape, leaves, grads + new + [loss], 1e-5)
+        X, W1, B1, W2 = (leaves[i].astype(np.float64) for i in (x, w1, b1, w2))
+        pre = X @ W1.T + B1
+        dh = (np.ones((X.shape[0], W2.shape[0])) @ W2) * (pre > 0)
+        ref = [dh.T @ X, dh.sum(0), np.ones((W2.shape[0], X.shape[0])) @ np.maximum(pre, 0), np.full(W2.shape[0], X.shape[0])]
+        for gid, r in zip(grads, ref):
+            np.testing.assert_allclose(tape.numpy(gid), r, rtol=1e-4, atol=1e-4 * np.abs(r).max())
+    finally:
+        tape.close()
+
+
+def test_movement_and_reduce_at_size(hip):
+    """Index arithmetic of every movement op and both reduces on tensors of a few hundred thousand elements."""
+    dev, pool = hip
+    tape = Tape(dev, pool)
+    try:
+        r = np.random.default_rng(5)
+        g = tape.graph
+        xa = r.integers(-100, 100, (37, 129, 65)).astype(np.int32)
+        x = tape.tensor(xa, DType.I32)
+        a = g.flip(g.permute(x, [2, 0, 1]), [0, 2])                       # [65, 37, 129]
+        b = g.reduce(a, BOp.Add, [1])                                     # [65, 129]
+        c = g.reduce(g.binary(a, g.expand(g.reshape(b, [65, 1, 129]), [65, 37, 129]), BOp.Mul), BOp.Max, [0, 2])  # [37]
+        d = g.expand(g.reshape(c, [37, 1]), [3, 37, 5])
+        tape.realize([a, b, c, d])
+        A = np.flip(np.transpose(xa, (2, 0, 1)), (0, 2))
+        B = A.sum(1, dtype=np.int32)
+        Cc = (A * B[:, None, :]).max((0, 2))
+        assert np.array_equal(tape.numpy(a), A) and np.array_equal(tape.numpy(b), B)
+        assert np.array_equal(tape.numpy(c), Cc)
+        assert np.array_equal(tape.numpy(d), np.broadcast_to(Cc.reshape(37, 1), (3, 37, 5)))
+    finally:
+        tape.close()
+
+
+def test_programs_are_compiled_once(hip):
+    dev, pool = hip
+    tape = Tape(dev, pool)
+    try:
+        g = tape.graph
+        xs = [tape.tensor(np.full(100, i, np.float32), DType.F32) for i in range(4)]
+        outs = [g.binary(x, g.const(2.0, DType.F32), BOp.Mul) for x in xs]
+        tape.realize(outs)
+        assert len(tape._programs) == 1
+        assert [tape.numpy(o)[0] for o in outs] == [0.0, 2.0, 4.0, 6.0]
+    finally:
+        tape.close()

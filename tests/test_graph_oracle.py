@@ -1,0 +1,198 @@
+"""zyx_amd.graph on the CPU: the reverse rules against the gradients zyx/tests/11_autograd.rs asserts, finite
+differences and closed forms (evaluated by oracle/graph_eval.py), and the lowered kernels executed by the kernel
+interpreter (oracle/ir_interp.py) against that evaluation, bit for bit."""
+import numpy as np
+import pytest
+
+from graph_cases import CASES, mixed_graph, mlp_graph
+from oracle import graph_eval, ir_interp
+from zyx_amd import DType
+from zyx_amd.graph import Graph, lower, storage_dtype
+from zyx_amd.ir import BOp, UOp
+
+_FLOAT = (DType.F32, DType.F64)
+
+
+def _build(build, *args, **kw):
+    g, leaves = Graph(), {}
+
+    def leaf(array, dtype):
+        a = np.ascontiguousarray(np.asarray(array).astype(storage_dtype(dtype)))
+        nid = g.leaf(a.shape, dtype)
+        leaves[nid] = a
+        return nid
+
+    return g, leaves, build(g, leaf, *args, **kw)
+
+
+def run_lowered(g, leaves, outputs):
+    """Executes the schedule with the kernel interpreter; buffers are flat arrays in storage format."""
+    bufs = {i: a.reshape(-1).copy() for i, a in leaves.items()}
+    for kern in lower(g, outputs):
+        out = np.zeros(kern.elements, storage_dtype(g[kern.output].dtype))
+        ir_interp.run(kern.image, [bufs[i] for i in kern.inputs] + [out])
+        bufs[kern.output] = out
+    return {o: bufs[o].reshape(g[o].shape) for o in outputs}
+
+
+@pytest.mark.parametrize("name,build", CASES, ids=[c[0] for c in CASES])
+def test_reference_gradients(name, build):
+    g, leaves, (target, sources, expected) = _build(build)
+    grads = g.gradient(target, sources)
+    want = graph_eval.evaluate(g.nodes, leaves, grads + [target])
+    for gid, src, exp in zip(grads, sources, expected):
+        assert g[gid].shape == g[src].shape and g[gid].dtype == g[src].dtype
+        if exp is None:
+            continue
+        if g[src].dtype in _FLOAT:
+            np.testing.assert_allclose(want[gid], exp, rtol=2e-7 if g[src].dtype == DType.F32 else 1e-12, atol=0)
+        else:
+            assert want[gid].tolist() == np.asarray(exp).tolist()
+    got = run_lowered(g, leaves, grads + [target])
+    for gid in grads + [target]:
+        assert got[gid].dtype == want[gid].dtype
+        assert np.array_equal(got[gid], want[gid], equal_nan=True), (name, gid)
+
+
+def _loss(build, leaves_override, **kw):
+    g, leaves, out = _build(build, **kw)
+    leaves.update(leaves_override)
+    return float(graph_eval.evaluate(g.nodes, leaves, [out[0]])[out[0]].reshape(-1)[0])
+
+
+def test_every_rule_against_finite_differences():
+    g, leaves, (loss, sources) = _build(mixed_graph)
+    grads = g.gradient(loss, sources)
+    got = graph_eval.evaluate(g.nodes, leaves, grads)
+    low = run_lowered(g, leaves, grads)
+    for gid, src in zip(grads, sources):
+        assert np.array_equal(low[gid], got[gid])
+        base = leaves[src]
+        num = np.zeros_like(base)
+        for i in np.ndindex(base.shape):
+            h = 1e-6
+            up, dn = base.copy(), base.copy()
+            up[i] += h
+            dn[i] -= h
+            num[i] = (_loss(mixed_graph, {src: up}) - _loss(mixed_graph, {src: dn})) / (2 * h)
+        np.testing.assert_allclose(got[gid], num, rtol=2e-6, atol=1e-8)
+
+
+def test_max_ties():
+    """Reduce max: every tied maximum receives the full gradient (mask 1 - (x < max), autograd.rs:330-352); binary
+    Max: strict comparisons on both sides, so a tie passes nothing (:155-162)."""
+    g = Graph()
+    x = g.leaf((2, 3), DType.F32)
+    y = g.leaf((2, 3), DType.F32)
+    leaves = {x: np.array([[1, 5, 5], [7, 7, 7]], np.float32), y: np.array([[1, 9, 5], [0, 7, 8]], np.float32)}
+    r = g.reduce(x, BOp.Max, [1])
+    (gr,) = g.gradient(r, [x])
+    m = g.binary(x, y, BOp.Max)
+    gx, gy = g.gradient(m, [x, y])
+    got = run_lowered(g, leaves, [gr, gx, gy, r])
+    assert got[r].tolist() == [5, 7]
+    assert got[gr].tolist() == [[0, 1, 1], [1, 1, 1]]
+    assert got[gx].tolist() == [[0, 0, 0], [1, 0, 0]]
+    assert got[gy].tolist() == [[0, 1, 0], [0, 0, 1]]
+
+
+def test_mlp_gradients_closed_form():
+    g, leaves, (loss, sources, (x, w1, b1, w2, b2)) = _build(mlp_graph)
+    grads = g.gradient(loss, sources)
+    got = run_lowered(g, leaves, grads + [loss])
+    X, W1, B1, W2 = (leaves[i].astype(np.float64) for i in (x, w1, b1, w2))
+    pre = X @ W1.T + B1
+    h = np.maximum(pre, 0)
+    dlogits = np.ones((X.shape[0], W2.shape[0]))
+    dh = (dlogits @ W2) * (pre > 0)
+    want = [dh.T @ X, dh.sum(0), dlogits.T @ h, dlogits.sum(0)]
+    for gid, w in zip(grads, want):
+        np.testing.assert_allclose(got[gid], w, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(got[loss], [(h @ W2.T + leaves[b2]).sum()], rtol=1e-5)
+
+
+def test_unrelated_source_and_dtype_of_gradient():
+    g = Graph()
+    x, y = g.leaf((3,), DType.F32), g.leaf((2, 2), DType.I32)
+    z = g.unary(x, UOp.Exp)
+    gx, gy = g.gradient(z, [x, y])
+    got = run_lowered(g, {x: np.zeros(3, np.float32), y: np.zeros((2, 2), np.int32)}, [gx, gy])
+    assert got[gy].dtype == np.int32 and got[gy].tolist() == [[0, 0], [0, 0]]
+    assert got[gx].tolist() == [1, 1, 1]
+    # a cast on the way: the gradient returns in the source's dtype
+    c = g.cast(y, DType.F32)
+    s = g.sum_all(g.binary(c, c, BOp.Mul))
+    (gc,) = g.gradient(s, [y])
+    got = run_lowered(g, {y: np.array([[1, 2], [3, 4]], np.int32)}, [gc])
+    assert got[gc].dtype == np.int32 and got[gc].tolist() == [[2, 4], [6, 8]]
+
+
+@pytest.mark.parametrize("n", [1, 63, 64, 65, 130, 4097])
+def test_lowered_sizes_and_movement(n):
+    """Thread guard for sizes that are not a multiple of the workgroup, and the index arithmetic of every movement op."""
+    r = np.random.default_rng(n)
+    g = Graph()
+    x = g.leaf((n, 3), DType.I32)
+    leaves = {x: r.integers(-50, 50, (n, 3)).astype(np.int32)}
+    a = g.flip(g.permute(x, [1, 0]), [1])                       # [3, n]
+    b = g.expand(g.reshape(a, [3, 1, n]), [3, 2, n])            # [3, 2, n]
+    c = g.reduce(b, BOp.Add, [1])                               # [3, n]
+    d = g.reduce(g.binary(c, a, BOp.Mul), BOp.Max, [0])         # [n]
+    e = g.reduce(b, BOp.Add, [0, 2])                            # [2]
+    got = run_lowered(g, leaves, [a, b, c, d, e])
+    A = np.flip(leaves[x].T, 1)
+    B = np.broadcast_to(A.reshape(3, 1, n), (3, 2, n))
+    assert np.array_equal(got[a], A) and np.array_equal(got[b], B)
+    assert np.array_equal(got[c], B.sum(1)) and np.array_equal(got[d], (B.sum(1) * A).max(0))
+    assert np.array_equal(got[e], B.sum((0, 2)))
+
+
+def test_schedule_shape():
+    """One kernel per requested output and per reduce; read-only parameters come first, in first-use order."""
+    g = Graph()
+    x, y = g.leaf((4, 4), DType.F32), g.leaf((4, 4), DType.F32)
+    s = g.reduce(g.binary(y, x, BOp.Mul), BOp.Add, [1])
+    out = g.binary_b(g.unary(x, UOp.Exp), g.reshape(s, [4, 1]), BOp.Div)
+    ks = lower(g, [out])
+    assert [k.output for k in ks] == [s, out]
+    assert ks[0].inputs == [y, x] and ks[1].inputs == [x, s]
+    ops, _ = ir_interp.parse(ks[1].image)
+    params = [o for o in ops if o[1] == ir_interp.PARAM]
+    assert [p[6] for p in params] == [ir_interp.GLOBAL, ir_interp.GLOBAL, ir_interp.GLOBAL_MUT]
+    # nodes that already have a buffer are not computed again
+    assert [k.output for k in lower(g, [out], stored=[s])] == [out]
+
+
+def test_shape_errors():
+    g = Graph()
+    x = g.leaf((2, 3), DType.F32)
+    for bad in (lambda: g.reshape(x, [4]), lambda: g.expand(x, [2, 4]), lambda: g.permute(x, [0, 0]),
+                lambda: g.binary(x, g.leaf((3, 2), DType.F32), BOp.Add), lambda: g.reduce(x, BOp.Mul, [0]),
+                lambda: g.dot(x, g.leaf((2, 3), DType.F32))):
+        with pytest.raises(ValueError):
+            bad()
+
+
+def test_lowered_kernels_are_accepted_by_the_source_generator():
+    """Every image the lowering produces for the reference's cases turns into HIP source (no GPU needed); the
+    largest one is also compiled for gfx950 when hipcc is present."""
+    import os, shutil, subprocess, tempfile
+    from zyx_amd.backend import generate_source
+    biggest = ""
+    for name, build in CASES + [("mixed", lambda g, leaf: mixed_graph(g, leaf) + ([None] * 3,))]:
+        g, leaves, (target, sources, _) = _build(build)
+        for kern in lower(g, g.gradient(target, sources) + [target]):
+            src = generate_source(kern.image)
+            assert "zir_kernel" in src
+            biggest = max(biggest, src, key=len)
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "k.hip")
+        open(path, "w").write(biggest)
+        r = subprocess.run([hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fwrapv", "-Xclang",
+                            "-target-feature", "-Xclang", "-packed-fp32-ops", "--cuda-device-only", "-include",
+                            "hip/hip_runtime.h", "-c", path, "-o", os.path.join(d, "k.o")],
+                           capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, r.stderr[-2000:]

@@ -19,6 +19,7 @@ from .backend import (  # noqa: F401
 from . import kernels  # noqa: F401
 from . import safetensors_io  # noqa: F401
 from . import ir  # noqa: F401
+from . import graph  # noqa: F401
 
 __all__ = ["BackendError", "DType", "DeviceInfo", "ErrorStatus", "Event", "HIPConfig", "HIPDevice", "HIPMemoryPool",
            "KernelDesc", "initialize_device", "library_path", "kernels"]

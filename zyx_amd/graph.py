@@ -1,0 +1,601 @@
+"""Graph nodes, reverse-mode differentiation and lowering to generated kernels.
+
+The node kinds are the ones `Runtime::gradient` differentiates (zyx/src/graph/autograd.rs:14-424; `Node` in
+zyx/src/graph/mod.rs): Leaf, Const, Unary, Binary, Cast, Reshape, Expand, Permute, Flip, Reduce. `Graph.gradient`
+applies that function's rules node by node, including the rules the reference keeps as comments beside a `todo!()`
+(Reshape :183-194, Expand :195-242, Reduce sum :269-295, Reduce max :299-379: every tied maximum receives the
+full gradient). `lower` turns the nodes to compute into kernels in the linearized-kernel image `Device::compile`
+takes: one thread per output element, movement ops folded into the index arithmetic of the loads, a reduce as one
+serial loop per output element with its accumulator in a register (zyx/src/kernel/linearize.rs:920-952) -- the kernel
+the reference generates before any optimisation pass. `Tape` runs them on a HIP device.
+
+Conventions where the graph leaves the dtype open (`Graph::dtype` returns x's dtype for every Binary, graph/mod.rs:
+1113-1134, and scalars broadcast implicitly, :1759-1769): a comparison or logical op yields Bool; when the operands
+of a Binary differ in dtype, a Const or Bool operand is converted to the other operand's dtype, otherwise y to x's.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Sequence
+
+import numpy as np
+
+from .backend import DType
+from .ir import BOp, Kernel, MemScope, ParamKind, UOp
+
+_BOOL_OPS = (BOp.Cmplt, BOp.Cmpgt, BOp.Cmpge, BOp.NotEq, BOp.Eq, BOp.Or, BOp.And)
+_NO_GRAD_BOPS = _BOOL_OPS + (BOp.BitXor, BOp.BitOr, BOp.BitAnd, BOp.BitShiftLeft, BOp.BitShiftRight)
+_FLOATS = (DType.BF16, DType.F16, DType.F32, DType.F64)
+_NP = {DType.BF16: np.uint16, DType.F16: np.float16, DType.F32: np.float32, DType.F64: np.float64, DType.U8: np.uint8,
+       DType.U16: np.uint16, DType.U32: np.uint32, DType.U64: np.uint64, DType.I8: np.int8, DType.I16: np.int16,
+       DType.I32: np.int32, DType.I64: np.int64, DType.Bool: np.uint8}
+
+
+def storage_dtype(dtype: DType):
+    """numpy type of a buffer of this dtype (bf16 travels as its 16 bits)."""
+    return _NP[DType(dtype)]
+
+
+def min_constant(dtype: DType):
+    """Neutral element of a max reduce: the lowest finite value (zyx/src/dtype.rs:207-224), not -inf."""
+    dtype = DType(dtype)
+    if dtype in (DType.BF16, DType.F32):
+        return -3.4028234663852886e38 if dtype == DType.F32 else -3.3895313892515355e38
+    if dtype == DType.F16:
+        return -65504.0
+    if dtype == DType.F64:
+        return -1.7976931348623157e308
+    if dtype == DType.Bool:
+        return 0
+    return int(np.iinfo(_NP[dtype]).min)
+
+
+@dataclasses.dataclass(frozen=True)
+class Node:
+    kind: str                 # leaf const unary binary cast reshape expand permute flip reduce
+    dtype: DType
+    shape: tuple
+    src: tuple = ()           # operand node ids
+    op: int | None = None     # UOp / BOp (reduce: BOp.Add or BOp.Max)
+    arg: object = None        # const value / axes
+
+
+def _numel(shape) -> int:
+    n = 1
+    for d in shape:
+        n *= int(d)
+    return n
+
+
+class Graph:
+    def __init__(self):
+        self.nodes: list[Node] = []
+
+    def _push(self, node: Node) -> int:
+        self.nodes.append(node)
+        return len(self.nodes) - 1
+
+    def __getitem__(self, i: int) -> Node:
+        return self.nodes[i]
+
+    # -- nodes --------------------------------------------------------------------------------------------------
+    def leaf(self, shape, dtype: DType) -> int:
+        return self._push(Node("leaf", DType(dtype), tuple(int(d) for d in shape)))
+
+    def const(self, value, dtype: DType) -> int:
+        return self._push(Node("const", DType(dtype), (), arg=value))
+
+    def unary(self, x: int, uop: UOp) -> int:
+        n = self[x]
+        return self._push(Node("unary", n.dtype, n.shape, (x,), UOp(uop)))
+
+    def binary(self, x: int, y: int, bop: BOp) -> int:
+        bop = BOp(bop)
+        nx, ny = self[x], self[y]
+        if nx.shape != ny.shape and nx.shape != () and ny.shape != ():
+            raise ValueError(f"binary operands have shapes {nx.shape} and {ny.shape}: only scalars broadcast implicitly")
+        shape = nx.shape if nx.shape != () else ny.shape
+        return self._push(Node("binary", DType.Bool if bop in _BOOL_OPS else self.operand_dtype(x, y), shape, (x, y), bop))
+
+    def operand_dtype(self, x: int, y: int) -> DType:
+        """The dtype both operands of a Binary are brought to (module docstring)."""
+        nx, ny = self[x], self[y]
+
+        def yields(n: Node) -> int:
+            return 2 if n.dtype == DType.Bool else (1 if n.kind == "const" else 0)
+
+        return ny.dtype if yields(ny) < yields(nx) else nx.dtype
+
+    def cast(self, x: int, dtype: DType) -> int:
+        return self._push(Node("cast", DType(dtype), self[x].shape, (x,)))
+
+    def reshape(self, x: int, shape) -> int:
+        shape = tuple(int(d) for d in shape)
+        if _numel(shape) != _numel(self[x].shape):
+            raise ValueError(f"cannot reshape {self[x].shape} to {shape}")
+        return x if shape == self[x].shape else self._push(Node("reshape", self[x].dtype, shape, (x,)))
+
+    def expand(self, x: int, shape) -> int:
+        """Right-aligned broadcast: dims of size 1 stretch, missing leading dims are added."""
+        shape, xs = tuple(int(d) for d in shape), self[x].shape
+        pad = len(shape) - len(xs)
+        if pad < 0 or any(d != 1 and d != shape[pad + i] for i, d in enumerate(xs)):
+            raise ValueError(f"cannot expand {xs} to {shape}")
+        return x if shape == xs else self._push(Node("expand", self[x].dtype, shape, (x,)))
+
+    def permute(self, x: int, axes) -> int:
+        xs = self[x].shape
+        axes = tuple(int(a) % len(xs) for a in axes)
+        if sorted(axes) != list(range(len(xs))):
+            raise ValueError(f"{axes} is not a permutation of the axes of {xs}")
+        return self._push(Node("permute", self[x].dtype, tuple(xs[a] for a in axes), (x,), arg=axes))
+
+    def flip(self, x: int, axes) -> int:
+        xs = self[x].shape
+        return self._push(Node("flip", self[x].dtype, xs, (x,), arg=tuple(sorted({int(a) % len(xs) for a in axes}))))
+
+    def reduce(self, x: int, rop: BOp, axes) -> int:
+        """Reduced dims are dropped; reducing every axis leaves shape [1]."""
+        rop, xs = BOp(rop), self[x].shape
+        if rop not in (BOp.Add, BOp.Max):
+            raise ValueError("reduce ops are Add and Max")
+        axes = tuple(sorted({int(a) % len(xs) for a in axes}))
+        shape = tuple(d for i, d in enumerate(xs) if i not in axes) or (1,)
+        return self._push(Node("reduce", self[x].dtype, shape, (x,), rop, axes))
+
+    # -- tensor-level compositions the reference builds from those nodes -------------------------------------------
+    def broadcast(self, x: int, shape) -> int:
+        """`Tensor::broadcast` for one side: pad the shape with leading 1s, then expand."""
+        xs = self[x].shape
+        if xs == ():
+            return self.expand(x, shape)
+        return self.expand(self.reshape(x, (1,) * (len(shape) - len(xs)) + xs), shape)
+
+    def binary_b(self, x: int, y: int, bop: BOp) -> int:
+        """Binary after numpy-style broadcasting of both operands."""
+        xs, ys = self[x].shape, self[y].shape
+        if xs != ys and xs != () and ys != ():
+            shape = tuple(np.broadcast_shapes(xs, ys))
+            x, y = self.broadcast(x, shape), self.broadcast(y, shape)
+        return self.binary(x, y, bop)
+
+    def relu(self, x: int) -> int:
+        """`self.cmpgt(0) * self` (zyx/src/tensor/elementwise.rs:289-293)."""
+        return self.binary(self.binary(x, self.const(0, self[x].dtype), BOp.Cmpgt), x, BOp.Mul)
+
+    def t(self, x: int) -> int:
+        r = len(self[x].shape)
+        return x if r < 2 else self.permute(x, tuple(range(r - 2)) + (r - 1, r - 2))
+
+    def dot(self, x: int, y: int) -> int:
+        """`Tensor::dot` (zyx/src/tensor/mod.rs:1469-1490): x[.., m, 1, k] * y^T[.., 1, n, k], summed over k."""
+        yt = self.t(y)
+        xs, ys = self[x].shape, self[yt].shape
+        if xs[-1] != ys[-1]:
+            raise ValueError(f"cannot dot tensors with shapes {xs} and {self[y].shape}")
+        x3 = self.reshape(x, xs[:-1] + (1, xs[-1]))
+        y3 = self.reshape(yt, ys[:-2] + (1,) + ys[max(len(ys) - 2, 0):])
+        prod = self.binary_b(x3, y3, BOp.Mul)
+        s = self.reduce(prod, BOp.Add, [-1])
+        return self.reshape(s, xs[:-1] + (ys[-2] if len(ys) > 1 else 1,))
+
+    def sum_all(self, x: int) -> int:
+        return self.reduce(x, BOp.Add, range(len(self[x].shape)))
+
+    def max_all(self, x: int) -> int:
+        return self.reduce(x, BOp.Max, range(len(self[x].shape)))
+
+    # -- reverse mode ---------------------------------------------------------------------------------------------
+    def _grad_order(self, target: int, sources: set) -> list:
+        """Nodes between the sources and the target, target first (`Graph::build_topo`, autograd.rs:427-493):
+        operands of comparison, logical and bit ops are not followed."""
+        needs: dict[int, bool] = {}
+
+        def visit(i: int) -> bool:
+            if i in needs:
+                return needs[i]
+            n = self[i]
+            blocked = n.kind == "binary" and n.op in _NO_GRAD_BOPS
+            dep = False
+            if not blocked:
+                for s in n.src:
+                    dep = (visit(s) or s in sources) or dep
+            needs[i] = dep
+            return dep
+
+        import sys
+        old = sys.getrecursionlimit()
+        sys.setrecursionlimit(max(old, 10000 + 4 * len(self.nodes)))
+        try:
+            visit(target)
+        finally:
+            sys.setrecursionlimit(old)
+        # node ids are topological (operands are created before their users): descending id = reverse topological
+        return sorted((i for i, d in needs.items() if d), reverse=True)
+
+    def gradient(self, target: int, sources: Sequence[int]) -> list:
+        """d target / d source for every source, as new nodes (`Runtime::gradient`, autograd.rs:14-424). The seed is
+        1 in the target's dtype; a source the target does not depend on gets zeros of its shape and dtype."""
+        src_set = set(sources)
+        grads: dict[int, int] = {target: self.expand(self.const(1, self[target].dtype), self[target].shape)}
+        order = self._grad_order(target, src_set)
+        wanted = set(order) | src_set
+
+        def acc(x: int, g: int):
+            if x in wanted:
+                grads[x] = self.binary(grads[x], g, BOp.Add) if x in grads else g
+
+        for cid in order:
+            if cid not in grads:
+                continue
+            grad, n = grads[cid], self[cid]
+            if n.kind == "unary":
+                (x,) = n.src
+                u = n.op
+                if u == UOp.Neg:
+                    acc(x, self.unary(grad, UOp.Neg))
+                elif u == UOp.Reciprocal:  # -z^2 * grad
+                    acc(x, self.binary(grad, self.unary(self.binary(cid, cid, BOp.Mul), UOp.Neg), BOp.Mul))
+                elif u == UOp.Exp2:
+                    acc(x, self.binary(grad, self.binary(cid, self.const(np.log(2.0), DType.F64), BOp.Mul), BOp.Mul))
+                elif u == UOp.Log2:
+                    acc(x, self.binary(grad, self.binary(x, self.const(np.log(2.0), DType.F64), BOp.Mul), BOp.Div))
+                elif u == UOp.Sqrt:
+                    acc(x, self.binary(grad, self.binary(cid, self.const(2, DType.I32), BOp.Mul), BOp.Div))
+                elif u == UOp.Sin:
+                    acc(x, self.binary(grad, self.unary(x, UOp.Cos), BOp.Mul))
+                elif u == UOp.Cos:
+                    acc(x, self.binary(grad, self.unary(self.unary(x, UOp.Sin), UOp.Neg), BOp.Mul))
+                elif u == UOp.Exp:
+                    acc(x, self.binary(grad, self.unary(x, UOp.Exp), BOp.Mul))
+                elif u == UOp.Ln:
+                    acc(x, self.binary(grad, x, BOp.Div))
+                elif u == UOp.Abs:  # grad * ((x > 0) * 1 + (x < 0) * -1); the constants take x's dtype so the sign survives
+                    zero, one, neg = (self.const(c, n.dtype) for c in (0, 1, -1))
+                    pos = self.binary(self.binary(x, zero, BOp.Cmpgt), one, BOp.Mul)
+                    ngt = self.binary(self.binary(x, zero, BOp.Cmplt), neg, BOp.Mul)
+                    acc(x, self.binary(grad, self.binary(pos, ngt, BOp.Add), BOp.Mul))
+                # Floor, Trunc, BitNot: no gradient
+            elif n.kind == "binary":
+                x, y = n.src
+                b = n.op
+                if b == BOp.Add:
+                    acc(x, grad)
+                    acc(y, grad)
+                elif b == BOp.Sub:
+                    acc(x, grad)
+                    acc(y, self.unary(grad, UOp.Neg))
+                elif b == BOp.Mul:
+                    acc(x, self.binary(grad, y, BOp.Mul))
+                    acc(y, self.binary(grad, x, BOp.Mul))
+                elif b == BOp.Div:
+                    acc(x, self.binary(grad, y, BOp.Div))
+                    x_mul = self.binary(self.unary(grad, UOp.Neg), x, BOp.Mul)
+                    acc(y, self.binary(x_mul, self.binary(y, y, BOp.Mul), BOp.Div))
+                elif b == BOp.Pow:
+                    y_1 = self.binary(y, self.const(1, DType.U8), BOp.Sub)
+                    y_mul = self.binary(y, self.binary(x, y_1, BOp.Pow), BOp.Mul)
+                    acc(x, self.binary(grad, y_mul, BOp.Mul))
+                    acc(y, self.binary(grad, self.binary(cid, self.unary(x, UOp.Ln), BOp.Mul), BOp.Mul))
+                elif b == BOp.Mod:
+                    acc(x, grad)
+                    floored = self.unary(self.binary(x, y, BOp.Div), UOp.Floor)
+                    acc(y, self.binary(self.unary(floored, UOp.Neg), grad, BOp.Mul))
+                elif b == BOp.Max:  # strict comparisons: neither side of a tie receives anything
+                    acc(x, self.binary(grad, self.binary(x, y, BOp.Cmpgt), BOp.Mul))
+                    acc(y, self.binary(grad, self.binary(x, y, BOp.Cmplt), BOp.Mul))
+            elif n.kind == "cast":
+                acc(n.src[0], self.cast(grad, self[n.src[0]].dtype))
+            elif n.kind == "reshape":
+                acc(n.src[0], self.reshape(grad, self[n.src[0]].shape))
+            elif n.kind == "expand":
+                x = n.src[0]
+                xs = self[x].shape
+                pad = len(n.shape) - len(xs)
+                axes = list(range(pad)) + [pad + i for i, d in enumerate(xs) if d == 1 and n.shape[pad + i] > 1]
+                g = grad if not axes else self.reshape(self.reduce(grad, BOp.Add, axes), xs)
+                acc(x, g)
+            elif n.kind == "permute":
+                inv = [0] * len(n.arg)
+                for i, a in enumerate(n.arg):
+                    inv[a] = i
+                acc(n.src[0], self.permute(grad, inv))
+            elif n.kind == "flip":
+                acc(n.src[0], self.flip(grad, n.arg))
+            elif n.kind == "reduce":
+                x = n.src[0]
+                xs = self[x].shape
+                keep = tuple(1 if i in n.arg else d for i, d in enumerate(xs))
+                grad_e = self.expand(self.reshape(grad, keep), xs)
+                if n.op == BOp.Add:
+                    acc(x, grad_e)
+                else:  # (1 - (x < max)) * grad
+                    z_b = self.expand(self.reshape(cid, keep), xs)
+                    cmp_f = self.cast(self.binary(x, z_b, BOp.Cmplt), self[x].dtype)
+                    one_e = self.expand(self.const(1, self[x].dtype), xs)
+                    acc(x, self.binary(self.binary(one_e, cmp_f, BOp.Sub), grad_e, BOp.Mul))
+        out = []
+        for s in sources:
+            if s in grads:
+                g = grads[s]
+                if self[g].dtype != self[s].dtype:
+                    g = self.cast(g, self[s].dtype)
+                out.append(g)
+            else:
+                out.append(self.expand(self.const(0, self[s].dtype), self[s].shape))
+        return out
+
+
+# ---- lowering ---------------------------------------------------------------------------------------------------------
+
+@dataclasses.dataclass
+class LoweredKernel:
+    image: bytes
+    inputs: list      # node ids of the buffers read, in parameter order
+    output: int       # node id of the buffer written
+    elements: int
+
+
+class _V:
+    """An index value that lives in an IR op (Python ints stand for constants and are folded)."""
+    __slots__ = ("id",)
+
+    def __init__(self, op_id: int):
+        self.id = op_id
+
+
+class _Emitter:
+    LOCAL = 64
+
+    def __init__(self, graph: Graph, stored: set):
+        self.g, self.stored = graph, stored
+
+    # index arithmetic with constant folding
+    def _ix(self, v):
+        if isinstance(v, _V):
+            return v.id
+        if v not in self.consts:
+            self.consts[v] = self.k.const_idx(v)
+        return self.consts[v]
+
+    def _op(self, a, b, bop, fold):
+        if not isinstance(a, _V) and not isinstance(b, _V):
+            return fold(a, b)
+        return _V(self.k.binary(self._ix(a), self._ix(b), bop))
+
+    def add(self, a, b):
+        if not isinstance(a, _V) and a == 0: return b
+        if not isinstance(b, _V) and b == 0: return a
+        return self._op(a, b, BOp.Add, lambda p, q: p + q)
+
+    def mul(self, a, c: int):
+        if c == 1: return a
+        if c == 0: return 0
+        return self._op(a, c, BOp.Mul, lambda p, q: p * q)
+
+    def div(self, a, c: int):
+        return a if c == 1 else self._op(a, c, BOp.Div, lambda p, q: p // q)
+
+    def mod(self, a, c: int):
+        return 0 if c == 1 else self._op(a, c, BOp.Mod, lambda p, q: p % q)
+
+    def ravel(self, idx, shape):
+        lin, stride = 0, 1
+        for i, d in zip(reversed(idx), reversed(shape)):
+            lin = self.add(lin, self.mul(i, stride))
+            stride *= d
+        return lin
+
+    def unravel(self, lin, shape):
+        """lin < numel(shape) for every caller, so the first component of extent > 1 needs no remainder."""
+        idx, total = [], _numel(shape)
+        remaining = total
+        for d in shape:
+            stride = remaining // d
+            if d == 1:
+                idx.append(0)
+            else:
+                q = self.div(lin, stride)
+                idx.append(q if remaining == total else self.mod(q, d))
+            remaining = stride
+        return idx
+
+    # expression emission -----------------------------------------------------------------------------------------
+    def value(self, nid: int, idx: list, root: bool = False):
+        """IR op holding element `idx` of node `nid`."""
+        key = (nid, tuple(i.id if isinstance(i, _V) else ("c", i) for i in idx))
+        if key in self.memo:
+            return self.memo[key]
+        n, k = self.g[nid], self.k
+        if (n.kind == "leaf" or nid in self.stored) and not root:
+            v = k.load(self.params[nid], self._ix(self.ravel(idx, n.shape)))
+        elif n.kind == "const":
+            v = k.const(n.arg, n.dtype)
+        elif n.kind == "unary":
+            v = k.unary(self.value(n.src[0], idx), n.op)
+        elif n.kind == "binary":
+            x, y = n.src
+            dt = self.g.operand_dtype(x, y)
+            v = k.binary(self.operand(x, idx, dt), self.operand(y, idx, dt), n.op)
+        elif n.kind == "cast":
+            v = k.cast(self.value(n.src[0], idx), n.dtype)
+        elif n.kind == "reshape":
+            v = self.value(n.src[0], self.unravel(self.ravel(idx, n.shape), self.g[n.src[0]].shape))
+        elif n.kind == "expand":
+            xs = self.g[n.src[0]].shape
+            pad = len(n.shape) - len(xs)
+            v = self.value(n.src[0], [0 if d == 1 else idx[pad + i] for i, d in enumerate(xs)])
+        elif n.kind == "permute":
+            x_idx = [0] * len(idx)
+            for i, a in enumerate(n.arg):
+                x_idx[a] = idx[i]
+            v = self.value(n.src[0], x_idx)
+        elif n.kind == "flip":
+            x_idx = list(idx)
+            for a in n.arg:
+                i = idx[a]
+                x_idx[a] = n.shape[a] - 1 - i if not isinstance(i, _V) else _V(k.sub(self._ix(n.shape[a] - 1), i.id))
+            v = self.value(n.src[0], x_idx)
+        else:
+            raise ValueError(f"node kind {n.kind} cannot be computed inside an expression")
+        self.memo[key] = v
+        return v
+
+    def operand(self, nid: int, idx: list, dtype: DType):
+        n = self.g[nid]
+        if n.dtype == dtype:
+            return self.value(nid, idx if n.shape != () else [])
+        if n.kind == "const":
+            return self.k.const(n.arg, dtype)
+        return self.k.cast(self.value(nid, idx if n.shape != () else []), dtype)
+
+    def _inputs(self, nid: int, root: bool, seen: set, order: list):
+        n = self.g[nid]
+        if (n.kind == "leaf" or nid in self.stored) and not root:
+            if nid not in seen:
+                seen.add(nid)
+                order.append(nid)
+            return
+        for s in n.src:
+            self._inputs(s, False, seen, order)
+
+    def kernel(self, nid: int) -> LoweredKernel:
+        n = self.g[nid]
+        self.k = k = Kernel()
+        self.consts, self.memo = {}, {}
+        inputs: list = []
+        self._inputs(nid, True, set(), inputs)
+        self.params = {i: k.param(self.g[i].dtype, ParamKind.Global, max(_numel(self.g[i].shape), 1)) for i in inputs}
+        total = max(_numel(n.shape), 1)
+        out = k.param(n.dtype, ParamKind.GlobalMut, total)
+        local = self.LOCAL if total >= self.LOCAL else 1
+        groups = (total + local - 1) // local
+        gid = _V(k.group_index(0, k.const_idx(groups)))
+        lin = gid if local == 1 else self.add(self.mul(gid, local), _V(k.local_index(0, local)))
+        guarded = groups * local != total
+        if guarded:
+            k.if_(k.cmplt(self._ix(lin), self._ix(total)))
+            self.consts = {}  # constants created from here on live inside the If
+        idx = self.unravel(lin, n.shape) if n.shape else []
+        if n.kind == "reduce":
+            x = n.src[0]
+            xs = self.g[x].shape
+            red = [xs[a] for a in n.arg]
+            zero = self._ix(0)
+            accu = k.storage(n.dtype, MemScope.Register, 1)
+            k.store(accu, k.const(0 if n.op == BOp.Add else min_constant(n.dtype), n.dtype), zero)
+            r = _V(k.loop(self._ix(_numel(red))))
+            outer, self.consts = dict(self.consts), dict(self.consts)
+            r_idx = self.unravel(r, red)
+            kept = iter(idx if len(n.arg) < len(xs) else [])
+            x_idx = [r_idx[n.arg.index(i)] if i in n.arg else next(kept) for i in range(len(xs))]
+            v = self.value(x, x_idx)
+            k.store(accu, k.binary(v, k.load(accu, zero), n.op), zero)  # x (op) acc, linearize.rs:943-946
+            k.end_loop()
+            self.consts = outer
+            v = k.load(accu, zero)
+        else:
+            v = self.value(nid, idx, root=True)
+        k.store(out, v, self._ix(lin))
+        if guarded:
+            k.end_if()
+        return LoweredKernel(k.to_bytes(), inputs, nid, total)
+
+
+def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = ()) -> list:
+    """Kernels that compute `outputs`, in execution order. Leaves and the nodes in `stored` already have buffers;
+    every Reduce on the way and every output gets one (and is appended to the schedule once)."""
+    have = set(stored)
+    emitter = _Emitter(graph, have)
+    schedule: list = []
+
+    def need(nid: int, root: bool):
+        n = graph[nid]
+        if n.kind == "leaf" or nid in have:
+            return
+        for s in n.src:
+            need(s, False)
+        if root or n.kind == "reduce":
+            schedule.append(emitter.kernel(nid))
+            have.add(nid)
+
+    import sys
+    old = sys.getrecursionlimit()
+    sys.setrecursionlimit(max(old, 10000 + 4 * len(graph.nodes)))
+    try:
+        for o in outputs:
+            need(o, True)
+    finally:
+        sys.setrecursionlimit(old)
+    return schedule
+
+
+# ---- device -----------------------------------------------------------------------------------------------------------
+
+class Tape:
+    """Tensors of one graph on a HIP device: leaves are uploaded, `realize` lowers, compiles (once per distinct
+    kernel) and launches, `numpy` downloads. The analogue of `Tape::new` / `gradient` / `realize`
+    (zyx/tests/11_autograd.rs uses them throughout)."""
+
+    def __init__(self, device, pool):
+        self.dev, self.pool, self.graph = device, pool, Graph()
+        self._buf: dict[int, int] = {}
+        self._ev: dict[int, object] = {}
+        self._programs: dict[bytes, int] = {}
+        self._keep: list = []
+        self._last = None  # event of the most recent launch: launches form one chain
+
+    def tensor(self, array, dtype: DType) -> int:
+        a = np.ascontiguousarray(array, storage_dtype(dtype))
+        nid = self.graph.leaf(a.shape, dtype)
+        self._alloc(nid)
+        self._keep.append(a)  # the source of an upload stays valid until its event is synced
+        self._ev[nid] = self.pool.host_to_pool(a, self._buf[nid], [self._ev.pop(nid)])
+        return nid
+
+    def _alloc(self, nid: int):
+        n = self.graph[nid]
+        buf, ev = self.pool.allocate(max(_numel(n.shape), 1) * np.dtype(storage_dtype(n.dtype)).itemsize)
+        self._buf[nid], self._ev[nid] = buf, ev
+
+    def gradient(self, target: int, sources: Sequence[int]) -> list:
+        return self.graph.gradient(target, sources)
+
+    def realize(self, nodes: Sequence[int]):
+        for kern in lower(self.graph, [n for n in nodes if n not in self._buf], stored=list(self._buf)):
+            prog = self._programs.get(kern.image)
+            if prog is None:
+                prog = self._programs[kern.image] = self.dev.compile(kern.image)
+            self._alloc(kern.output)
+            # A launch consumes the events it waits for. Every launch waits for the one before it, so a buffer whose
+            # event an earlier launch consumed is ready for all later ones too.
+            waits = [self._ev.pop(i) for i in kern.inputs + [kern.output] if i in self._ev]
+            if self._last is not None:
+                waits.append(self._last)
+            self._last = self.dev.launch(prog, self.pool, [self._buf[i] for i in kern.inputs] + [self._buf[kern.output]], waits)
+
+    def numpy(self, nid: int) -> np.ndarray:
+        if nid not in self._buf:
+            self.realize([nid])
+        n = self.graph[nid]
+        out = np.empty(n.shape if n.shape else (1,), storage_dtype(n.dtype))
+        self.sync()
+        self.pool.pool_to_host(self._buf[nid], out, [])
+        return out.reshape(n.shape)
+
+    def sync(self):
+        evs = list(self._ev.values()) + ([self._last] if self._last is not None else [])
+        self._ev.clear()
+        self._last = None
+        if evs:
+            self.pool.sync_events(evs)
+        self._keep.clear()
+
+    def close(self):
+        self.sync()
+        for prog in self._programs.values():
+            self.dev.release(prog)
+        for buf in self._buf.values():
+            self.pool.deallocate(buf, [])
+        self._programs.clear()
+        self._buf.clear()
