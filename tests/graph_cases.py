@@ -196,3 +196,26 @@ def mlp_graph(g, leaf, batch=8, n_in=12, hidden=16, n_out=5, seed=1, dtype=F32):
     l1 = g.relu(g.binary_b(g.dot(x, g.t(w1)), b1, BOp.Add))
     logits = g.binary_b(g.dot(l1, g.t(w2)), b2, BOp.Add)
     return g.sum_all(logits), [w1, b1, w2, b2], (x, w1, b1, w2, b2)
+
+
+def attention_graph(g, leaf, b=2, h=2, t=24, dh=8, seed=3, causal=False, p=0.0, training=False, dtype=F32):
+    """Core of CausalSelfAttention::forward (zyx-nn/src/causal_self_attention.rs:50-70) as graph nodes: scores
+    q.k^T * scale, optional additive mask (0 / -inf above the diagonal), softmax over keys, dropout (evaluation
+    scale, or the training mask from a uniform tensor), . v. Loss = sum(y * dy) so that d loss / d(q, k, v) is the
+    backward of the fused kernel for the upstream gradient dy. Returns (loss, [q, k, v], (y, arrays))."""
+    r = np.random.default_rng(seed)
+    arrs = {n: r.standard_normal((b, h, t, dh)) for n in ("q", "k", "v", "dy")}
+    q, k, v, dy = (leaf(arrs[n], dtype) for n in ("q", "k", "v", "dy"))
+    att = g.binary(g.dot(q, g.t(k)), g.const(float(np.float32(1.0 / np.sqrt(dh))), dtype), BOp.Mul)
+    if causal:
+        mask = leaf(np.where(np.tril(np.ones((t, t), bool)), 0.0, -np.inf), dtype)
+        att = g.binary_b(att, mask, BOp.Add)
+    att = g.softmax(att, [-1])
+    if training:
+        arrs["u"] = r.uniform(0, 1, (b, h, t, t))
+        att = g.dropout(att, p, leaf(arrs["u"], dtype))
+    elif p:
+        att = g.dropout(att, p)
+    y = g.dot(att, v)
+    loss = g.sum_all(g.binary(y, dy, BOp.Mul))
+    return loss, [q, k, v], (y, arrs)

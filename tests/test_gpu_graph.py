@@ -148,3 +148,46 @@ def test_programs_are_compiled_once(hip):
         assert [tape.numpy(o)[0] for o in outs] == [0.0, 2.0, 4.0, 6.0]
     finally:
         tape.close()
+
+
+@pytest.mark.parametrize("causal,p", [(False, 0.0), (True, 0.25)])
+def test_fused_attention_against_the_graph_path(hip, causal, p):
+    """Two independent routes on the device: the fused attention kernels (forward + backward) and the same maths
+    as graph nodes differentiated by the reverse rules and run as generated kernels. f32 both; they sum in
+    different orders, so the bar is 1e-5 of the largest magnitude of each tensor."""
+    from graph_cases import attention_graph
+    from zyx_amd import kernels as K
+    dev, pool = hip
+    tape, leaves, (loss, sources, (y, arrs)) = on_device(hip, attention_graph, causal=causal, p=p)
+    try:
+        grads = tape.gradient(loss, sources)
+        tape.realize(grads + [y])
+        b, h, t, dh = arrs["q"].shape
+        pack = lambda a: np.ascontiguousarray(a.transpose(0, 2, 1, 3).reshape(b, t, h * dh))  # [B,H,T,dh] -> [B,T,C]
+        qkv = np.concatenate([pack(arrs[n]) for n in ("q", "k", "v")], 2).astype(np.float32)
+        y_f, lse = K.attention(dev, pool, qkv, h, DType.F32, dropout_p=p, want_lse=True, causal=causal)
+        dqkv = K.attention_bwd(dev, pool, qkv, y_f, pack(arrs["dy"]).astype(np.float32), lse, h, DType.F32, dropout_p=p, causal=causal)
+        y_g = pack(tape.numpy(y))
+        np.testing.assert_allclose(y_f, y_g, rtol=0, atol=1e-5 * np.abs(y_g).max())
+        for i, gid in enumerate(grads):
+            g_g = pack(tape.numpy(gid))
+            np.testing.assert_allclose(dqkv[:, :, i * h * dh:(i + 1) * h * dh], g_g, rtol=0, atol=2e-5 * np.abs(g_g).max())
+    finally:
+        tape.close()
+
+
+@pytest.mark.parametrize("dtype,rtol", [(DType.F64, 1e-10), (DType.F32, 1e-4)])
+def test_attention_with_training_dropout(hip, dtype, rtol):
+    """Training-mode dropout inside attention (`probability.cmplt(rand) * att`, tensor/mod.rs:822-828) through the
+    graph path, forward and gradients, against the CPU evaluation of the same graph."""
+    from graph_cases import attention_graph
+    tape, leaves, (loss, sources, (y, arrs)) = on_device(hip, attention_graph, causal=True, p=0.3, training=True, dtype=dtype)
+    try:
+        grads = tape.gradient(loss, sources)
+        nodes = grads + [y]
+        want = graph_eval.evaluate(tape.graph.nodes, leaves, nodes)
+        tape.realize(nodes)
+        for nid in nodes:
+            np.testing.assert_allclose(tape.numpy(nid), want[nid], rtol=0, atol=rtol * np.abs(want[nid]).max())
+    finally:
+        tape.close()

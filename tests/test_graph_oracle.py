@@ -196,3 +196,45 @@ def test_lowered_kernels_are_accepted_by_the_source_generator():
                             "hip/hip_runtime.h", "-c", path, "-o", os.path.join(d, "k.o")],
                            capture_output=True, text=True, timeout=120)
         assert r.returncode == 0, r.stderr[-2000:]
+
+
+def test_softmax_and_dropout_compositions():
+    """softmax golden of zyx/tests/05_misc.rs:664-683 through the graph; training-mode dropout keeps x where
+    p < u without rescaling, evaluation divides by 1 - p (tensor/mod.rs:822-828)."""
+    g = Graph()
+    x = g.leaf((1, 3), DType.F32)
+    u = g.leaf((1, 3), DType.F32)
+    leaves = {x: np.array([[2, 4, 3]], np.float32), u: np.array([[0.1, 0.25, 0.9]], np.float32)}
+    sm, ls = g.softmax(x, [-1]), g.ln_softmax(x, [-1])
+    tr, evl = g.dropout(x, 0.25, u), g.dropout(x, 0.25)
+    got = run_lowered(g, leaves, [sm, ls, tr, evl])
+    np.testing.assert_allclose(got[sm], [[0.090030566, 0.6652409, 0.24472846]], rtol=1e-6)
+    np.testing.assert_allclose(np.exp(got[ls]), got[sm], rtol=1e-6)
+    assert got[tr].tolist() == [[0, 0, 3]]
+    assert np.array_equal(got[evl], np.array([[2, 4, 3]], np.float32) / np.float32(0.75))
+
+
+@pytest.mark.parametrize("causal,p,training", [(False, 0.0, False), (True, 0.25, False), (True, 0.3, True)])
+def test_attention_graph_gradients(causal, p, training):
+    """The attention core built from graph nodes and differentiated by the reverse rules, against the textbook
+    forward and backward in f64 (with the dropout mask applied after the softmax, as the reference orders them)."""
+    from graph_cases import attention_graph
+    g, leaves, (loss, sources, (y, arrs)) = _build(attention_graph, causal=causal, p=p, training=training, dtype=DType.F64)
+    grads = g.gradient(loss, sources)
+    got = graph_eval.evaluate(g.nodes, leaves, grads + [y])
+    q, k, v, dy = (arrs[n] for n in ("q", "k", "v", "dy"))
+    t, dh = q.shape[2], q.shape[3]
+    sc = float(np.float32(1 / np.sqrt(dh)))
+    s = np.einsum("bhtd,bhjd->bhtj", q, k) * sc
+    if causal:
+        s = np.where(np.tril(np.ones((t, t), bool)), s, -np.inf)
+    e = np.exp(s - s.max(-1, keepdims=True))
+    ps = e / e.sum(-1, keepdims=True)
+    keep = (p < arrs["u"]).astype(np.float64) if training else np.full_like(ps, 1 / (1 - p))
+    pd = ps * keep
+    np.testing.assert_allclose(got[y], np.einsum("bhtj,bhjd->bhtd", pd, v), rtol=1e-11, atol=1e-13)
+    dpd = np.einsum("bhtd,bhjd->bhtj", dy, v) * keep
+    ds = ps * (dpd - (ps * dpd).sum(-1, keepdims=True))
+    want = [np.einsum("bhtj,bhjd->bhtd", ds, k) * sc, np.einsum("bhtj,bhtd->bhjd", ds, q) * sc, np.einsum("bhtj,bhtd->bhjd", pd, dy)]
+    for gid, w in zip(grads, want):
+        np.testing.assert_allclose(got[gid], w, rtol=1e-9, atol=1e-12)

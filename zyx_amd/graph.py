@@ -179,6 +179,30 @@ class Graph:
         s = self.reduce(prod, BOp.Add, [-1])
         return self.reshape(s, xs[:-1] + (ys[-2] if len(ys) > 1 else 1,))
 
+    def reduce_keepdim(self, x: int, rop: BOp, axes) -> int:
+        xs = self[x].shape
+        axes = [int(a) % len(xs) for a in axes] or list(range(len(xs)))
+        return self.reshape(self.reduce(x, rop, axes), tuple(1 if i in axes else d for i, d in enumerate(xs)))
+
+    def softmax(self, x: int, axes) -> int:
+        """`e = (x - max_keepdim).exp(); e / e.sum_keepdim` (zyx/src/tensor/mod.rs:1457-1461)."""
+        e = self.unary(self.binary_b(x, self.reduce_keepdim(x, BOp.Max, axes), BOp.Sub), UOp.Exp)
+        return self.binary_b(e, self.reduce_keepdim(e, BOp.Add, axes), BOp.Div)
+
+    def ln_softmax(self, x: int, axes) -> int:
+        """`m = x - max_keepdim; m - m.exp().sum_keepdim.ln()` (zyx/src/tensor/mod.rs:1427-1431)."""
+        m = self.binary_b(x, self.reduce_keepdim(x, BOp.Max, axes), BOp.Sub)
+        return self.binary_b(m, self.unary(self.reduce_keepdim(self.unary(m, UOp.Exp), BOp.Add, axes), UOp.Ln), BOp.Sub)
+
+    def dropout(self, x: int, probability: float, uniform: int | None = None) -> int:
+        """`Tensor::dropout` (zyx/src/tensor/mod.rs:822-828). Training (`uniform` = the tensor `Tensor::rand` would
+        draw, same shape and dtype as x): `probability.cmplt(uniform) * x`, without rescaling; evaluation:
+        `x / (1 - probability)`."""
+        dt = self[x].dtype
+        if uniform is None:
+            return self.binary(x, self.const(1.0 - probability, dt), BOp.Div)
+        return self.binary(self.binary(self.const(probability, dt), uniform, BOp.Cmplt), x, BOp.Mul)
+
     def sum_all(self, x: int) -> int:
         return self.reduce(x, BOp.Add, range(len(self[x].shape)))
 
