@@ -191,3 +191,76 @@ def test_attention_with_training_dropout(hip, dtype, rtol):
             np.testing.assert_allclose(tape.numpy(nid), want[nid], rtol=0, atol=rtol * np.abs(want[nid]).max())
     finally:
         tape.close()
+
+
+# ---- products matched to the hand-written GEMM ---------------------------------------------------------------------------
+
+def _dense_mlp(g, leaf, **shape):
+    loss, sources, leaves5 = mlp_graph(g, leaf, **shape)
+    logits = g[loss].src[0]
+    return g.sum_all(g.binary(logits, logits, BOp.Mul)), sources, leaves5
+
+
+def matched_tape(hip, build, match=True, **kw):
+    dev, pool = hip
+    tape, leaves = Tape(dev, pool, match=match), {}
+
+    def leaf(array, dtype):
+        a = np.ascontiguousarray(np.asarray(array).astype(storage_dtype(dtype)))
+        nid = tape.tensor(a, dtype)
+        leaves[nid] = a
+        return nid
+
+    return tape, leaves, build(tape.graph, leaf, **kw)
+
+
+def test_mlp_products_run_on_the_gemm_kernel(hip):
+    """The MNIST-size network with a dense upstream gradient: the two forward and the three backward products are
+    launched as GEMMs reading the operands in place (weights [out, in], x and dY through trans_a); f32, bar 1e-5 of
+    each tensor's magnitude against the CPU evaluation of the graph (the GEMM sums in another order)."""
+    tape, leaves, (loss, sources, _) = matched_tape(hip, _dense_mlp, batch=64, n_in=784, hidden=128, n_out=10)
+    try:
+        grads = tape.gradient(loss, sources)
+        want = graph_eval.evaluate(tape.graph.nodes, leaves, grads + [loss])
+        tape.realize(grads + [loss])
+        assert tape.matched == 5
+        for nid in grads + [loss]:
+            np.testing.assert_allclose(tape.numpy(nid), want[nid], rtol=0, atol=1e-5 * np.abs(want[nid]).max())
+    finally:
+        tape.close()
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_products_run_on_the_batched_gemm(hip, causal):
+    from graph_cases import attention_graph
+    tape, leaves, (loss, sources, (y, _)) = matched_tape(hip, attention_graph, causal=causal, p=0.1, t=40, dh=16)
+    try:
+        grads = tape.gradient(loss, sources)
+        want = graph_eval.evaluate(tape.graph.nodes, leaves, grads + [y])
+        tape.realize(grads + [y])
+        assert tape.matched == 6
+        for nid in grads + [y]:
+            np.testing.assert_allclose(tape.numpy(nid), want[nid], rtol=0, atol=3e-5 * np.abs(want[nid]).max())
+    finally:
+        tape.close()
+
+
+def test_gemm_and_generated_kernel_compete_on_time(hip):
+    """A 512^3 product: both candidates are timed with the autotuner's clock and the GEMM wins by a wide margin (the
+    generated kernel is one serial loop per output element)."""
+    def build(g, leaf):
+        r = np.random.default_rng(9)
+        a, b = leaf(r.standard_normal((512, 512)), DType.F32), leaf(r.standard_normal((512, 512)), DType.F32)
+        return g.dot(a, b), (a, b)
+
+    tape, leaves, (out, (a, b)) = matched_tape(hip, build, match="time")
+    try:
+        tape.realize([out])
+        (c, t_gemm, t_gen), = tape.timings
+        assert (c.m, c.n, c.k, c.trans_a, c.trans_b) == (512, 512, 512, False, False)
+        assert t_gemm < t_gen and tape.matched == 1
+        ref = leaves[a].astype(np.float64) @ leaves[b].astype(np.float64)
+        np.testing.assert_allclose(tape.numpy(out), ref, rtol=0, atol=1e-5 * np.abs(ref).max())
+        print(f"512^3 f32: GEMM {t_gemm / 1e3:.1f} us, generated kernel {t_gen / 1e3:.1f} us")
+    finally:
+        tape.close()

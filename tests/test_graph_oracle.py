@@ -7,7 +7,7 @@ import pytest
 from graph_cases import CASES, mixed_graph, mlp_graph
 from oracle import graph_eval, ir_interp
 from zyx_amd import DType
-from zyx_amd.graph import Graph, lower, storage_dtype
+from zyx_amd.graph import Contraction, Graph, lower, match_contraction, storage_dtype, view_of
 from zyx_amd.ir import BOp, UOp
 
 _FLOAT = (DType.F32, DType.F64)
@@ -25,10 +25,21 @@ def _build(build, *args, **kw):
     return g, leaves, build(g, leaf, *args, **kw)
 
 
-def run_lowered(g, leaves, outputs):
-    """Executes the schedule with the kernel interpreter; buffers are flat arrays in storage format."""
+def run_lowered(g, leaves, outputs, match=False, seen=None):
+    """Executes the schedule with the kernel interpreter; buffers are flat arrays in storage format. A matched
+    product is computed the way the GEMM kernel reads its operands: in place, [batch, m, k] or [batch, k, m]
+    (trans_a) times [batch, k, n] or [batch, n, k] (trans_b), written as [batch, m, n]."""
     bufs = {i: a.reshape(-1).copy() for i, a in leaves.items()}
-    for kern in lower(g, outputs):
+    for kern in lower(g, outputs, match=match):
+        if isinstance(kern, Contraction):
+            A = bufs[kern.a].reshape((kern.batch, kern.k, kern.m) if kern.trans_a else (kern.batch, kern.m, kern.k))
+            B = bufs[kern.b].reshape((kern.batch, kern.n, kern.k) if kern.trans_b else (kern.batch, kern.k, kern.n))
+            A = A.transpose(0, 2, 1) if kern.trans_a else A
+            B = B.transpose(0, 2, 1) if kern.trans_b else B
+            bufs[kern.out] = np.matmul(A.astype(np.float64), B.astype(np.float64)).astype(A.dtype).reshape(-1)
+            if seen is not None:
+                seen.append(kern)
+            continue
         out = np.zeros(kern.elements, storage_dtype(g[kern.output].dtype))
         ir_interp.run(kern.image, [bufs[i] for i in kern.inputs] + [out])
         bufs[kern.output] = out
@@ -238,3 +249,68 @@ def test_attention_graph_gradients(causal, p, training):
     want = [np.einsum("bhtj,bhjd->bhtd", ds, k) * sc, np.einsum("bhtj,bhtd->bhjd", ds, q) * sc, np.einsum("bhtj,bhtd->bhjd", pd, dy)]
     for gid, w in zip(grads, want):
         np.testing.assert_allclose(got[gid], w, rtol=1e-9, atol=1e-12)
+
+
+# ---- products matched to the GEMM kernel -----------------------------------------------------------------------------
+
+def test_views_and_reshape_strides():
+    g = Graph()
+    x = g.leaf((4, 6, 5), DType.F32)
+    assert view_of(g, g.permute(x, [2, 0, 1])) == (x, [1, 30, 5])
+    assert view_of(g, g.reshape(x, [24, 5])) == (x, [5, 1])
+    assert view_of(g, g.reshape(x, [2, 2, 3, 2, 5])) == (x, [60, 30, 10, 5, 1])
+    assert view_of(g, g.expand(g.reshape(x, [4, 1, 6, 5]), [4, 7, 6, 5])) == (x, [30, 0, 5, 1])
+    assert view_of(g, g.reshape(g.permute(x, [1, 0, 2]), [6, 20]))[0] != x      # merging permuted dims needs a copy
+    t = g.reshape(g.permute(x, [1, 0, 2]), [6, 4, 1, 5])
+    assert view_of(g, t) == (x, [5, 30, 0, 1])                                  # inserting a 1 into permuted dims does not
+    assert view_of(g, g.flip(x, [0]))[0] != x
+
+
+def _mlp_sq(g, leaf):
+    loss, sources, leaves5 = mlp_graph(g, leaf)
+    logits = g[loss].src[0]
+    return g.sum_all(g.binary(logits, logits, BOp.Mul)), sources, leaves5
+
+
+def test_matched_products_of_an_mlp():
+    """Forward products x.W^T, and with a loss that gives a dense upstream gradient all three backward products
+    (dY^T.X read through trans_a, dY.W) are recognised; results agree with the unmatched schedule."""
+    g, leaves, (loss, sources, _) = _build(_mlp_sq)
+    grads = g.gradient(loss, sources)
+    seen = []
+    got = run_lowered(g, leaves, grads + [loss], match=True, seen=seen)
+    want = run_lowered(g, leaves, grads + [loss])
+    shapes = sorted((c.m, c.n, c.k, c.trans_a, c.trans_b) for c in seen)
+    assert shapes == sorted([(8, 16, 12, False, True), (8, 5, 16, False, True),      # x.W1^T, h.W2^T
+                             (8, 16, 5, False, False),                               # dh = dlogits.W2
+                             (5, 16, 8, True, False), (16, 12, 8, True, False)])     # dW2 = dlogits^T.h, dW1 = dpre^T.x
+    for nid in grads + [loss]:
+        np.testing.assert_allclose(got[nid], want[nid], rtol=2e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_matched_products_of_attention(causal):
+    from graph_cases import attention_graph
+    g, leaves, (loss, sources, (y, _)) = _build(attention_graph, causal=causal, p=0.1)
+    grads = g.gradient(loss, sources)
+    seen = []
+    got = run_lowered(g, leaves, grads + [y], match=True, seen=seen)
+    want = run_lowered(g, leaves, grads + [y])
+    assert len(seen) == 6 and all(c.batch == 4 for c in seen)   # q.k^T, att.v and the four backward products
+    for nid in grads + [y]:
+        np.testing.assert_allclose(got[nid], want[nid], rtol=0, atol=2e-5 * np.abs(want[nid]).max())
+
+
+def test_products_that_are_not_matched():
+    g = Graph()
+    xi, yi = g.leaf((4, 3), DType.I32), g.leaf((3, 5), DType.I32)
+    assert match_contraction(g, g[g.dot(xi, yi)].src[0] if g[g.dot(xi, yi)].kind == "reshape" else g.dot(xi, yi)) is None  # integers
+    x, y = g.leaf((4, 3), DType.F32), g.leaf((3, 5), DType.F32)
+    prod = g.binary(g.expand(g.reshape(x, [4, 1, 3]), [4, 5, 3]), g.expand(g.reshape(g.t(y), [1, 5, 3]), [4, 5, 3]), BOp.Mul)
+    assert match_contraction(g, g.reduce(prod, BOp.Add, [2])) is not None
+    assert match_contraction(g, g.reduce(prod, BOp.Max, [2])) is None               # not a sum
+    assert match_contraction(g, g.reduce(prod, BOp.Add, [1])) is None               # sums an axis only one side has
+    assert match_contraction(g, g.reduce(g.binary(prod, prod, BOp.Add), BOp.Add, [2])) is None
+    fl = g.binary(g.expand(g.reshape(g.flip(x, [1]), [4, 1, 3]), [4, 5, 3]), g.expand(g.reshape(g.t(y), [1, 5, 3]), [4, 5, 3]), BOp.Mul)
+    c = match_contraction(g, g.reduce(fl, BOp.Add, [2]))
+    assert c is not None and g[c.a].kind == "flip"                                  # the flipped operand is copied first

@@ -350,6 +350,158 @@ class Graph:
         return out
 
 
+# ---- matching: products summed over shared axes -> the hand-written GEMM -------------------------------------------------
+
+@dataclasses.dataclass
+class Contraction:
+    """`out[batch, m, n] = sum_k a . b` found in the graph: `a` and `b` are the nodes whose buffers the GEMM reads in
+    place (`[batch, m, k]`, or `[batch, k, m]` with trans_a; `[batch, k, n]`, or `[batch, n, k]` with trans_b)."""
+    a: int
+    b: int
+    out: int
+    m: int
+    n: int
+    k: int
+    batch: int
+    trans_a: bool
+    trans_b: bool
+    dtype: DType
+    fallback: object = None   # the generated kernel for the same node, reading the same operand buffers (set by `lower`)
+
+
+def _reshape_strides(old_shape, old_strides, new_shape):
+    """Strides of `new_shape` over the same elements, or None when the reshape needs a copy. Dims of extent 1 carry
+    stride 0; a group of old dims can be split or merged only where it is contiguous in itself."""
+    old = [(d, st) for d, st in zip(old_shape, old_strides) if d != 1]
+    new_strides = [0] * len(new_shape)
+    oi = ni = 0
+    while ni < len(new_shape):
+        if new_shape[ni] == 1:
+            ni += 1
+            continue
+        if oi >= len(old):
+            return None
+        np_, op_, nj, oj = new_shape[ni], old[oi][0], ni + 1, oi + 1
+        while np_ != op_:
+            if np_ < op_:
+                if nj >= len(new_shape):
+                    return None
+                np_ *= new_shape[nj]
+                nj += 1
+            else:
+                if oj >= len(old):
+                    return None
+                op_ *= old[oj][0]
+                oj += 1
+        if any(old[t][1] != old[t + 1][1] * old[t + 1][0] for t in range(oi, oj - 1)):
+            return None
+        st = old[oj - 1][1]
+        for t in range(nj - 1, ni - 1, -1):
+            if new_shape[t] != 1:
+                new_strides[t] = st
+                st *= new_shape[t]
+        ni, oi = nj, oj
+    return new_strides if oi == len(old) else None
+
+
+def _contiguous(shape):
+    st, out = 1, []
+    for d in reversed(shape):
+        out.append(0 if d == 1 else st)
+        st *= d
+    return out[::-1]
+
+
+def view_of(graph: Graph, nid: int):
+    """(base node, element strides of every dim of `nid` in the base's row-major buffer): looks through Permute,
+    Expand and every Reshape that needs no copy. Anything else -- including a Flip -- is a base itself."""
+    n = graph[nid]
+    if n.kind == "permute":
+        base, st = view_of(graph, n.src[0])
+        return base, [st[a] for a in n.arg]
+    if n.kind == "expand":
+        base, st = view_of(graph, n.src[0])
+        pad = len(n.shape) - len(st)
+        return base, [0] * pad + [0 if graph[n.src[0]].shape[i] == 1 else v for i, v in enumerate(st)]
+    if n.kind == "reshape":
+        base, st = view_of(graph, n.src[0])
+        new = _reshape_strides(graph[n.src[0]].shape, st, n.shape)
+        if new is not None:
+            return base, new
+    return nid, _contiguous(n.shape)
+
+
+def match_contraction(graph: Graph, nid: int):
+    """`Graph::match_matmul` (zyx/src/vendor/matmul.rs:41-71) generalised from the canonical `dot` form to every
+    Reduce(Add) over a Mul of two views: the forward product, both backward products (which autograd leaves as
+    sums over the m or the n axis of the same broadcast product) and batched products. Returns None when the node is
+    not such a product or its operands would need a copy first."""
+    r = graph[nid]
+    if r.kind != "reduce" or r.op != BOp.Add or r.dtype not in (DType.F32, DType.BF16, DType.F16):
+        return None
+    p = graph[r.src[0]]
+    if p.kind != "binary" or p.op != BOp.Mul or any(graph[s].dtype != r.dtype for s in p.src):
+        return None
+    (xa, sa), (xb, sb) = view_of(graph, p.src[0]), view_of(graph, p.src[1])
+    if graph[p.src[0]].shape != p.shape or graph[p.src[1]].shape != p.shape:
+        return None  # a scalar operand
+    groups = {"batch": [], "m": [], "n": [], "k": []}
+    order = []
+    for d, ext in enumerate(p.shape):
+        if ext == 1:
+            continue
+        ina, inb, red = sa[d] != 0, sb[d] != 0, d in r.arg
+        kind = "k" if (red and ina and inb) else None if red else "batch" if (ina and inb) else "m" if ina else "n" if inb else None
+        if kind is None:
+            return None
+        groups[kind].append(d)
+        if not red and (not order or order[-1] != kind):
+            order.append(kind)
+    if not groups["k"] or order not in (["batch", "m", "n"], ["batch", "n", "m"], ["m", "n"], ["n", "m"], ["batch", "m"], ["batch", "n"],
+                                        ["m"], ["n"], ["batch"], []):
+        return None
+    if order and order[-1] == "m" and "n" in order:  # out is [.., n, m]: compute the transposed product
+        xa, sa, xb, sb = xb, sb, xa, sa
+        groups["m"], groups["n"] = groups["n"], groups["m"]
+
+    def merged(dims, strides):
+        """(extent, stride) of a group of dims seen as one, or None."""
+        if not dims:
+            return 1, 0
+        if any(strides[dims[i]] != strides[dims[i + 1]] * p.shape[dims[i + 1]] for i in range(len(dims) - 1)):
+            return None
+        return _numel([p.shape[d] for d in dims]), strides[dims[-1]]
+
+    parts = {}
+    for name in ("batch", "m", "n", "k"):
+        for tag, st in (("a", sa), ("b", sb)):
+            if (name, tag) in (("n", "a"), ("m", "b")):
+                continue
+            got = merged(groups[name], st)
+            if got is None:
+                return None
+            parts[name, tag] = got
+    batch, m, n, k = parts["batch", "a"][0], parts["m", "a"][0], parts["n", "b"][0], parts["k", "a"][0]
+    if batch * m * n == 1:
+        return None  # an inner product of two vectors: one output element is a reduce, not a GEMM
+
+    def layout(rows, row_st, cols, col_st, batch_st, base):
+        """False: [rows, cols] row-major; True: [cols, rows]; None: neither."""
+        if _numel(graph[base].shape) != batch * rows * cols or (batch > 1 and batch_st != rows * cols):
+            return None
+        if (cols == 1 or col_st == 1) and (rows == 1 or row_st == cols):
+            return False
+        if (rows == 1 or row_st == 1) and (cols == 1 or col_st == rows):
+            return True
+        return None
+
+    ta = layout(m, parts["m", "a"][1], k, parts["k", "a"][1], parts["batch", "a"][1], xa)
+    tb = layout(k, parts["k", "b"][1], n, parts["n", "b"][1], parts["batch", "b"][1], xb)
+    if ta is None or tb is None:
+        return None
+    return Contraction(xa, xb, nid, m, n, k, batch, ta, tb, r.dtype)
+
+
 # ---- lowering ---------------------------------------------------------------------------------------------------------
 
 @dataclasses.dataclass
@@ -526,9 +678,12 @@ class _Emitter:
         return LoweredKernel(k.to_bytes(), inputs, nid, total)
 
 
-def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = ()) -> list:
+def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), match: bool = False) -> list:
     """Kernels that compute `outputs`, in execution order. Leaves and the nodes in `stored` already have buffers;
-    every Reduce on the way and every output gets one (and is appended to the schedule once)."""
+    every Reduce on the way and every output gets one (and is appended to the schedule once). With `match`, a Reduce
+    that `match_contraction` recognises is scheduled as a `Contraction` (its operands get buffers first) with the
+    generated kernel kept beside it as `.fallback`, so the caller can let the two compete on measured time the way
+    kernel nodes compete in the reference's graph (zyx/src/backend/cblas.rs:227-236)."""
     have = set(stored)
     emitter = _Emitter(graph, have)
     schedule: list = []
@@ -536,6 +691,14 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = ()) -> l
     def need(nid: int, root: bool):
         n = graph[nid]
         if n.kind == "leaf" or nid in have:
+            return
+        c = match_contraction(graph, nid) if match else None
+        if c is not None:
+            for s in (c.a, c.b):
+                need(s, True)
+            c.fallback = emitter.kernel(nid)
+            schedule.append(c)
+            have.add(nid)
             return
         for s in n.src:
             need(s, False)
@@ -561,8 +724,15 @@ class Tape:
     kernel) and launches, `numpy` downloads. The analogue of `Tape::new` / `gradient` / `realize`
     (zyx/tests/11_autograd.rs uses them throughout)."""
 
-    def __init__(self, device, pool):
-        self.dev, self.pool, self.graph = device, pool, Graph()
+    def __init__(self, device, pool, match=False):
+        """match: True -- products summed over shared axes run on the hand-written GEMM instead of a generated
+        kernel; "time" -- both are timed once per distinct product (`zhip_time_kernel`, the clock the reference's
+        autotuner uses, zyx/src/kernel/autotune.rs:775-798) and the faster one runs, as kernel nodes compete on
+        `time` in the reference's graph."""
+        self.dev, self.pool, self.graph, self.match = device, pool, Graph(), match
+        self.matched = 0
+        self.timings: list = []   # (Contraction, ns of the GEMM, ns of the generated kernel)
+        self._choice: dict = {}
         self._buf: dict[int, int] = {}
         self._ev: dict[int, object] = {}
         self._programs: dict[bytes, int] = {}
@@ -586,17 +756,45 @@ class Tape:
         return self.graph.gradient(target, sources)
 
     def realize(self, nodes: Sequence[int]):
-        for kern in lower(self.graph, [n for n in nodes if n not in self._buf], stored=list(self._buf)):
+        for kern in lower(self.graph, [n for n in nodes if n not in self._buf], stored=list(self._buf), match=self.match):
+            if isinstance(kern, Contraction):
+                kern = self._gemm_or_generated(kern)
             prog = self._programs.get(kern.image)
             if prog is None:
                 prog = self._programs[kern.image] = self.dev.compile(kern.image)
-            self._alloc(kern.output)
+            if kern.output not in self._buf:
+                self._alloc(kern.output)
             # A launch consumes the events it waits for. Every launch waits for the one before it, so a buffer whose
             # event an earlier launch consumed is ready for all later ones too.
             waits = [self._ev.pop(i) for i in kern.inputs + [kern.output] if i in self._ev]
             if self._last is not None:
                 waits.append(self._last)
             self._last = self.dev.launch(prog, self.pool, [self._buf[i] for i in kern.inputs] + [self._buf[kern.output]], waits)
+
+    def _gemm_or_generated(self, c: Contraction) -> LoweredKernel:
+        from .kernels import gemm_desc
+        desc = gemm_desc(c.m, c.n, c.k, c.dtype, c.dtype, c.trans_a, c.trans_b, batch=c.batch)
+        key = bytes(desc)
+        if key not in self._programs:
+            self._programs[key] = self.dev.register_kernel(desc)
+        gemm = LoweredKernel(key, [c.a, c.b], c.out, c.batch * c.m * c.n)
+        if self.match == "time":
+            pair = (key, c.fallback.image)
+            if pair not in self._choice:
+                if c.fallback.image not in self._programs:
+                    self._programs[c.fallback.image] = self.dev.compile(c.fallback.image)
+                self._alloc(c.out)
+                self.sync()  # the operands are complete and the new buffer exists
+                ns = []
+                for k in (gemm, c.fallback):
+                    args = [self._buf[i] for i in k.inputs] + [self._buf[c.out]]
+                    ns.append(min(self.dev.time_kernel(self._programs[k.image], args) for _ in range(3)))
+                self.timings.append((c, ns[0], ns[1]))
+                self._choice[pair] = ns[0] <= ns[1]
+            if not self._choice[pair]:
+                return c.fallback
+        self.matched += 1
+        return gemm
 
     def numpy(self, nid: int) -> np.ndarray:
         if nid not in self._buf:
