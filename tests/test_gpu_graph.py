@@ -238,7 +238,7 @@ def test_attention_products_run_on_the_batched_gemm(hip, causal):
         grads = tape.gradient(loss, sources)
         want = graph_eval.evaluate(tape.graph.nodes, leaves, grads + [y])
         tape.realize(grads + [y])
-        assert tape.matched == 6
+        assert tape.matched == 7   # six batched products and the softmax over keys
         for nid in grads + [y]:
             np.testing.assert_allclose(tape.numpy(nid), want[nid], rtol=0, atol=3e-5 * np.abs(want[nid]).max())
     finally:
@@ -262,5 +262,24 @@ def test_gemm_and_generated_kernel_compete_on_time(hip):
         ref = leaves[a].astype(np.float64) @ leaves[b].astype(np.float64)
         np.testing.assert_allclose(tape.numpy(out), ref, rtol=0, atol=1e-5 * np.abs(ref).max())
         print(f"512^3 f32: GEMM {t_gemm / 1e3:.1f} us, generated kernel {t_gen / 1e3:.1f} us")
+    finally:
+        tape.close()
+
+
+def test_softmax_runs_on_the_fused_kernel(hip):
+    """`Tensor::softmax` over the last axis of a graph tensor is launched as the fused row-softmax kernel (one pass)
+    in place of two reduces and a map; f32 within 2e-6 relative of the CPU evaluation (exp and summation order)."""
+    def build(g, leaf):
+        x = leaf(3 * np.random.default_rng(4).standard_normal((4, 128, 4096)), DType.F32)
+        return g.softmax(x, [-1]), x
+
+    tape, leaves, (sm, x) = matched_tape(hip, build)
+    try:
+        tape.realize([sm])
+        assert tape.matched == 1 and len(tape._programs) == 1
+        got = tape.numpy(sm)
+        xv = leaves[x].astype(np.float64)
+        e = np.exp(xv - xv.max(-1, keepdims=True))
+        np.testing.assert_allclose(got, e / e.sum(-1, keepdims=True), rtol=2e-6, atol=1e-12)
     finally:
         tape.close()

@@ -104,6 +104,32 @@ def test_large_magnitudes(hip, oracle):
     run_and_check(hip, oracle, x)
 
 
+@pytest.mark.parametrize("cols", [4096, 1000, 333, 8192])
+def test_masked_entries(hip, oracle, cols):
+    """-inf entries (a masked_fill before the softmax) give exactly 0 and take no part in the sum, as exp(-inf) = 0
+    does in the C backend; the extremes of the finite range behave the same way; a NaN poisons its own row only;
+    a row that is -inf throughout is 0 / 0 = NaN on both sides (the max reduce starts from the lowest finite value)."""
+    r = oracle.Rng(11)
+    x = r.randn((12, cols), 2.0)
+    x[0, ::3] = -np.inf
+    x[1, 1:] = -np.inf                       # a single live entry
+    x[2, : cols // 2] = -3.0e38              # x - max overflows to -inf
+    x[3, 5] = 3.0e38
+    x[3, 7] = -3.0e38
+    x[4, :] = -np.inf
+    x[5, 9] = np.nan
+    dev, pool = hip
+    y, s, a = kernels.softmax_rows(dev, pool, x)
+    yo, so, ao = oracle.softmax_rows(x)
+    fin = [0, 1, 2, 3] + list(range(6, 12))
+    assert not np.isnan(y[fin]).any() and (y[0, ::3] == 0).all() and y[1, 0] == 1.0 and (y[1, 1:] == 0).all()
+    assert (y[2, : cols // 2] == 0).all() and y[3, 5] == 1.0 and y[3, 7] == 0
+    assert_close(y[fin], yo[fin], slack=1e-6 * np.abs(yo[fin]))
+    assert_close(s[fin], so[fin], slack=2e-6)
+    assert np.array_equal(a[fin], ao[fin])
+    assert np.isnan(y[4]).all() and np.isnan(yo[4]).all() and np.isnan(y[5]).all() and np.isnan(yo[5]).all()
+
+
 @pytest.mark.parametrize("flags", [(True, False, False), (False, True, False), (False, False, True),
                                    (True, True, False), (True, False, True), (False, True, True)])
 @pytest.mark.parametrize("shape", [(37, 4096), (5, 333)])

@@ -7,7 +7,7 @@ import pytest
 from graph_cases import CASES, mixed_graph, mlp_graph
 from oracle import graph_eval, ir_interp
 from zyx_amd import DType
-from zyx_amd.graph import Contraction, Graph, lower, match_contraction, storage_dtype, view_of
+from zyx_amd.graph import Contraction, Graph, SoftmaxRows, lower, match_softmax, match_contraction, storage_dtype, view_of
 from zyx_amd.ir import BOp, UOp
 
 _FLOAT = (DType.F32, DType.F64)
@@ -37,6 +37,13 @@ def run_lowered(g, leaves, outputs, match=False, seen=None):
             A = A.transpose(0, 2, 1) if kern.trans_a else A
             B = B.transpose(0, 2, 1) if kern.trans_b else B
             bufs[kern.out] = np.matmul(A.astype(np.float64), B.astype(np.float64)).astype(A.dtype).reshape(-1)
+            if seen is not None:
+                seen.append(kern)
+            continue
+        if isinstance(kern, SoftmaxRows):
+            x = bufs[kern.x].reshape(kern.rows, kern.cols).astype(np.float64)
+            e = np.exp(x - x.max(1, keepdims=True))
+            bufs[kern.out] = (e / e.sum(1, keepdims=True)).astype(np.float32).reshape(-1)
             if seen is not None:
                 seen.append(kern)
             continue
@@ -296,7 +303,10 @@ def test_matched_products_of_attention(causal):
     seen = []
     got = run_lowered(g, leaves, grads + [y], match=True, seen=seen)
     want = run_lowered(g, leaves, grads + [y])
-    assert len(seen) == 6 and all(c.batch == 4 for c in seen)   # q.k^T, att.v and the four backward products
+    gemms = [c for c in seen if isinstance(c, Contraction)]
+    assert len(gemms) == 6 and all(c.batch == 4 for c in gemms)   # q.k^T, att.v and the four backward products
+    (sm,) = [c for c in seen if isinstance(c, SoftmaxRows)]
+    assert (sm.rows, sm.cols) == (2 * 2 * 24, 24)
     for nid in grads + [y]:
         np.testing.assert_allclose(got[nid], want[nid], rtol=0, atol=2e-5 * np.abs(want[nid]).max())
 
@@ -314,3 +324,29 @@ def test_products_that_are_not_matched():
     fl = g.binary(g.expand(g.reshape(g.flip(x, [1]), [4, 1, 3]), [4, 5, 3]), g.expand(g.reshape(g.t(y), [1, 5, 3]), [4, 5, 3]), BOp.Mul)
     c = match_contraction(g, g.reduce(fl, BOp.Add, [2]))
     assert c is not None and g[c.a].kind == "flip"                                  # the flipped operand is copied first
+
+
+def test_softmax_match():
+    g = Graph()
+    x = g.leaf((3, 5, 7), DType.F32)
+    sm = g.softmax(x, [-1])
+    m = match_softmax(g, sm)
+    assert (m.x, m.rows, m.cols) == (x, 15, 7)
+    assert match_softmax(g, g.softmax(x, [1])) is None                       # not the last axis
+    assert match_softmax(g, g.softmax(x, [1, 2])) is None                    # two axes
+    assert match_softmax(g, g.ln_softmax(x, [-1])) is None
+    h = g.leaf((3, 5, 7), DType.F64)
+    assert match_softmax(g, g.softmax(h, [-1])) is None                      # f32 only
+    y = g.unary(g.permute(x, [1, 0, 2]), UOp.Neg)                            # an expression: gets its own buffer
+    m = match_softmax(g, g.softmax(y, [-1]))
+    assert m.x == y and (m.rows, m.cols) == (15, 7)
+    p = g.permute(x, [1, 0, 2])                                              # a permuted view is not row-contiguous
+    assert match_softmax(g, g.softmax(p, [-1])).x == p
+    # e / sum(e) where e is not exp(x - max): no match
+    e = g.unary(x, UOp.Exp)
+    assert match_softmax(g, g.binary_b(e, g.reduce_keepdim(e, BOp.Add, [-1]), BOp.Div)) is None
+    leaves = {x: np.random.default_rng(2).standard_normal((3, 5, 7)).astype(np.float32)}
+    seen = []
+    got = run_lowered(g, leaves, [sm], match=True, seen=seen)
+    assert len(seen) == 1
+    np.testing.assert_allclose(got[sm], run_lowered(g, leaves, [sm])[sm], rtol=1e-6)

@@ -502,6 +502,45 @@ def match_contraction(graph: Graph, nid: int):
     return Contraction(xa, xb, nid, m, n, k, batch, ta, tb, r.dtype)
 
 
+@dataclasses.dataclass
+class SoftmaxRows:
+    """`out[rows, cols] = softmax(x, last axis)` found in the graph; `x` is the node whose buffer the fused kernel reads."""
+    x: int
+    out: int
+    rows: int
+    cols: int
+
+
+def _keepdim_reduce_of(graph: Graph, nid: int, rop: BOp, src: int):
+    """True when `nid` is `src` reduced with `rop` over its last axis and broadcast back to src's shape."""
+    base, st = view_of(graph, nid)
+    b, shape = graph[base], graph[src].shape
+    return (b.kind == "reduce" and b.op == rop and b.src[0] == src and b.arg == (len(shape) - 1,)
+            and graph[nid].shape == shape and st == _contiguous(shape[:-1]) + [0])
+
+
+def match_softmax(graph: Graph, nid: int):
+    """`e = exp(x - max_keepdim(x)); e / sum_keepdim(e)` over the last axis (`Tensor::softmax`,
+    zyx/src/tensor/mod.rs:1457-1461) in f32: the shape the fused row-softmax kernel computes in one pass."""
+    n = graph[nid]
+    if n.kind != "binary" or n.op != BOp.Div or n.dtype != DType.F32 or len(n.shape) < 1 or n.shape[-1] < 2:
+        return None
+    e, den = n.src
+    ne = graph[e]
+    if ne.kind != "unary" or ne.op != UOp.Exp or ne.dtype != DType.F32 or not _keepdim_reduce_of(graph, den, BOp.Add, e):
+        return None
+    d = graph[ne.src[0]]
+    if d.kind != "binary" or d.op != BOp.Sub or graph[d.src[0]].dtype != DType.F32:
+        return None
+    x, mx = d.src
+    if graph[x].shape != n.shape or not _keepdim_reduce_of(graph, mx, BOp.Max, x):
+        return None
+    base, st = view_of(graph, x)
+    if st != _contiguous(n.shape) or _numel(graph[base].shape) != _numel(n.shape):
+        base = x  # not a plain view of a whole buffer: x gets its own
+    return SoftmaxRows(base, nid, _numel(n.shape[:-1]), n.shape[-1])
+
+
 # ---- lowering ---------------------------------------------------------------------------------------------------------
 
 @dataclasses.dataclass
@@ -683,7 +722,8 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
     every Reduce on the way and every output gets one (and is appended to the schedule once). With `match`, a Reduce
     that `match_contraction` recognises is scheduled as a `Contraction` (its operands get buffers first) with the
     generated kernel kept beside it as `.fallback`, so the caller can let the two compete on measured time the way
-    kernel nodes compete in the reference's graph (zyx/src/backend/cblas.rs:227-236)."""
+    kernel nodes compete in the reference's graph (zyx/src/backend/cblas.rs:227-236); a softmax over the last axis is
+    scheduled as a `SoftmaxRows` (one fused pass in place of two reduces and a map: no competition needed)."""
     have = set(stored)
     emitter = _Emitter(graph, have)
     schedule: list = []
@@ -692,11 +732,12 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
         n = graph[nid]
         if n.kind == "leaf" or nid in have:
             return
-        c = match_contraction(graph, nid) if match else None
+        c = (match_contraction(graph, nid) or match_softmax(graph, nid)) if match else None
         if c is not None:
-            for s in (c.a, c.b):
+            for s in ((c.a, c.b) if isinstance(c, Contraction) else (c.x,)):
                 need(s, True)
-            c.fallback = emitter.kernel(nid)
+            if isinstance(c, Contraction):
+                c.fallback = emitter.kernel(nid)
             schedule.append(c)
             have.add(nid)
             return
@@ -730,8 +771,8 @@ class Tape:
         autotuner uses, zyx/src/kernel/autotune.rs:775-798) and the faster one runs, as kernel nodes compete on
         `time` in the reference's graph."""
         self.dev, self.pool, self.graph, self.match = device, pool, Graph(), match
-        self.matched = 0
-        self.timings: list = []   # (Contraction, ns of the GEMM, ns of the generated kernel)
+        self.matched = 0          # launches that went to a hand-written kernel
+        self.timings: list = []   # (match, ns of the hand-written kernel, ns of the generated kernel)
         self._choice: dict = {}
         self._buf: dict[int, int] = {}
         self._ev: dict[int, object] = {}
@@ -757,8 +798,8 @@ class Tape:
 
     def realize(self, nodes: Sequence[int]):
         for kern in lower(self.graph, [n for n in nodes if n not in self._buf], stored=list(self._buf), match=self.match):
-            if isinstance(kern, Contraction):
-                kern = self._gemm_or_generated(kern)
+            if isinstance(kern, (Contraction, SoftmaxRows)):
+                kern = self._matched_or_generated(kern)
             prog = self._programs.get(kern.image)
             if prog is None:
                 prog = self._programs[kern.image] = self.dev.compile(kern.image)
@@ -771,14 +812,19 @@ class Tape:
                 waits.append(self._last)
             self._last = self.dev.launch(prog, self.pool, [self._buf[i] for i in kern.inputs] + [self._buf[kern.output]], waits)
 
-    def _gemm_or_generated(self, c: Contraction) -> LoweredKernel:
-        from .kernels import gemm_desc
-        desc = gemm_desc(c.m, c.n, c.k, c.dtype, c.dtype, c.trans_a, c.trans_b, batch=c.batch)
+    def _matched_or_generated(self, c) -> LoweredKernel:
+        from .kernels import gemm_desc, softmax_rows_desc
+        if isinstance(c, Contraction):
+            desc = gemm_desc(c.m, c.n, c.k, c.dtype, c.dtype, c.trans_a, c.trans_b, batch=c.batch)
+            inputs, elements = [c.a, c.b], c.batch * c.m * c.n
+        else:
+            desc = softmax_rows_desc(c.rows, c.cols, y=True, rowsum=False, argmax=False)
+            inputs, elements = [c.x], c.rows * c.cols
         key = bytes(desc)
         if key not in self._programs:
             self._programs[key] = self.dev.register_kernel(desc)
-        gemm = LoweredKernel(key, [c.a, c.b], c.out, c.batch * c.m * c.n)
-        if self.match == "time":
+        gemm = LoweredKernel(key, inputs, c.out, elements)
+        if self.match == "time" and isinstance(c, Contraction):
             pair = (key, c.fallback.image)
             if pair not in self._choice:
                 if c.fallback.image not in self._programs:
