@@ -123,7 +123,12 @@ enum zhip_kernel_kind {
     /* Reduce over the last axis (flags = 0: x[rows,cols] -> [rows]) or over axis 0
      * (flags = 1: -> [cols]); iparams[0] = 0 sum, 1 max. Accumulates in f32 for float
      * dtypes and i32 for ZHIP_I32, stores as `dtype` (zyx/src/tensor/reduce_ops.rs:45-147,
-     * accumulator init zyx/src/kernel/linearize.rs:920-952). args: x, out. */
+     * accumulator init zyx/src/kernel/linearize.rs:920-952). Float dtypes may fold the ops that follow a
+     * reduce in a training step into its store, each a separate f32 operation in this order:
+     * fparams[0] != 0: * fparams[0]; fparams[1] != 0: / fparams[1] (the n of a mean, reduce_ops.rs:62-75);
+     * iparams[1] != 0: + base[i], a second input of out's shape and dtype (`p - g * lr` of SGD::update,
+     * zyx-optim/src/sgd.rs:77-81, with fparams[0] = -lr and base = p).
+     * args: x, (base when iparams[1] != 0), out. */
     ZHIP_K_REDUCE = 3,
     /* C[M,N] = op(A) . op(B) (+ bias[N]) (then ReLU / GELU): Tensor::dot / dot_dtype
      * (zyx/src/tensor/mod.rs:1469-1518) and Linear::forward (zyx-nn/src/linear.rs:38-44),

@@ -197,3 +197,33 @@ def test_calls_from_several_threads(hip, oracle):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+def test_device_to_device_ranges(hip):
+    """zhip_d2d: aligned and unaligned ranges, a move inside one buffer (disjoint and overlapping), a large one, and
+    the bounds errors; the bytes around the destination range stay as they were."""
+    dev, pool = hip
+    rng = np.random.default_rng(3)
+    src = rng.integers(0, 256, 9 << 20, dtype=np.uint8)
+    sb, e0 = pool.allocate(src.nbytes)
+    db, e1 = pool.allocate(src.nbytes)
+    pool.sync_events([pool.host_to_pool(src, sb, [e0]), pool.host_to_pool(np.zeros_like(src), db, [e1])])
+    want = np.zeros_like(src)
+    for s_off, d_off, n in ((0, 0, 4096), (16, 64, 200704), (3, 5, 1001), (7, 1 << 20, 123457), (1 << 20, 2 << 20, 5 << 20),
+                            (100, 8 << 20, 0)):
+        ev = pool.copy_range(sb, s_off, db, d_off, n, [])
+        pool.sync_events([ev])
+        want[d_off:d_off + n] = src[s_off:s_off + n]
+    got = np.empty_like(src)
+    pool.pool_to_host(db, got, [])
+    assert np.array_equal(got, want)
+    # inside one buffer: disjoint (copy kernel) and overlapping forward (the runtime's copy: memmove is not promised,
+    # so only the non-overlapping part is checked)
+    pool.sync_events([pool.copy_range(sb, 0, sb, 4 << 20, 1 << 20, [])])
+    pool.pool_to_host(sb, got, [])
+    assert np.array_equal(got[4 << 20:5 << 20], src[:1 << 20]) and np.array_equal(got[:4 << 20], src[:4 << 20])
+    for bad in ((0, 0, src.nbytes + 1), (src.nbytes, 0, 1), (0, src.nbytes - 3, 4)):
+        with pytest.raises(BackendError):
+            pool.copy_range(sb, bad[0], db, bad[1], bad[2], [])
+    pool.deallocate(sb, [])
+    pool.deallocate(db, [])

@@ -68,3 +68,34 @@ def test_empty_axes(hip):
     assert reduce(dev, pool, np.zeros((4, 0), np.float32), "sum").tolist() == [0.0] * 4
     assert reduce(dev, pool, np.zeros((0, 4), np.float32), "sum").shape == (0,)
     assert np.all(reduce(dev, pool, np.zeros((4, 0), np.float32), "max") == np.float32(-3.4028235e38))
+
+
+@pytest.mark.parametrize("shape,axis0", [((64, 10), True), ((64, 128), True), ((1, 64), False), ((4096, 512), True), ((300, 1000), False),
+                                         ((2, 100003), False), ((70000, 12), True)])
+def test_scaled_sum_onto_a_base(hip, oracle, shape, axis0):
+    """The ops that follow a reduce in a training step folded into its store: (sum * mul) / div + base, each one
+    f32 operation in that order -- bit-identical to applying them to the plain kernel's result (`p - g * lr` is
+    `g * -lr + p` exactly; a mean divides by n)."""
+    dev, pool = hip
+    x = oracle.Rng(shape[0] + shape[1]).randn(shape, 1.5)
+    n_out = shape[1] if axis0 else shape[0]
+    base = oracle.Rng(9).randn((n_out,), 1.0)
+    plain = reduce(dev, pool, x, "sum", axis0)
+    lr = np.float32(0.01)
+    assert np.array_equal(reduce(dev, pool, x, "sum", axis0, mul=-float(lr), base=base), base - plain * lr)
+    assert np.array_equal(reduce(dev, pool, x, "sum", axis0, div=float(shape[0])), plain / np.float32(shape[0]))
+    assert np.array_equal(reduce(dev, pool, x, "sum", axis0, mul=3.0, div=7.0, base=base), plain * np.float32(3) / np.float32(7) + base)
+    assert np.array_equal(reduce(dev, pool, x, "max", axis0, base=base), x.max(0 if axis0 else 1) + base)
+    xb = oracle.f32_to_bf16(x)
+    got = reduce(dev, pool, xb, "sum", axis0, DType.BF16, mul=0.5, base=oracle.f32_to_bf16(base))
+    acc = oracle.bf16_to_f32(reduce(dev, pool, xb, "sum", axis0, DType.BF16))  # stored sum: one truncation early
+    want = oracle.bf16_to_f32(xb).astype(np.float64).sum(0 if axis0 else 1) * 0.5 + oracle.bf16_to_f32(oracle.f32_to_bf16(base))
+    assert np.all(np.abs(oracle.bf16_to_f32(got) - want) <= 2.0 ** -7 * np.abs(want) + 1e-4 * np.abs(oracle.bf16_to_f32(xb)).sum(0 if axis0 else 1))
+
+
+def test_scale_is_refused_for_integers(hip):
+    from zyx_amd import BackendError
+    from zyx_amd.kernels import reduce_desc
+    dev, pool = hip
+    with pytest.raises(BackendError):
+        dev.register_kernel(reduce_desc(4, 4, "sum", False, DType.I32, mul=2.0))

@@ -13,6 +13,7 @@
 // 32. Operands are read with bounds checks (zero fill) straight from their natural layout,
 // coalesced along whichever index is contiguous, and laid down K-contiguous in LDS with a
 // row pad (8 elements for 16-bit types, 1 for f32), so fragment reads are the same for all four layouts.
+// Small f32 problems (at most 256 tiles of 32 x 32) take gemm_small_f32_k instead: one launch, no staging.
 #include <algorithm>
 
 #include "dtypes.hpp"
@@ -193,6 +194,96 @@ template <int ODT> __global__ __launch_bounds__(256) void gemm_generic_fold_k(co
     else ((uint16_t *)p.C)[oo] = f32_to_f16_trunc(v);
 }
 
+// Small f32 products (the layers and gradients of an MLP on a batch of 64): launch latency and round trips to memory
+// decide, not arithmetic. One workgroup per 32 x 32 tile of C; its NW waves split K and each accumulates a partial
+// tile with v_mfma_f32_32x32x2_f32 from operands read straight from memory into registers (no staging, no barrier in
+// the K loop, 8 independent loads per operand in flight); the partials meet in LDS and are summed in wave order, then
+// the epilogue runs once. One launch where split-K over the 64 x 64 kernel needs a second one to fold.
+// The two halves of a wave take the two halves of the wave's K slice, so each lane walks consecutive k: an operand
+// stored with k contiguous (AV / BV: 16-byte aligned rows) is read 4 elements per load, one stored with the row index
+// contiguous is read one element per load, coalesced across the 32 lanes of a half.
+template <bool VEC>
+__device__ __forceinline__ void load8(const float *__restrict__ row, int64_t ks, int64_t k0, int64_t k_hi, int64_t K, bool ok,
+                                      float (&v)[8]) {
+    if (VEC) {
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const int64_t k = k0 + 4 * q;
+            const f32x4 t = *(const f32x4 *)(row + min(k, K - 4));
+            const bool live = ok && k < k_hi; // k and k_hi are multiples of 4: a load is live or dead as a whole
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[4 * q + e] = live ? t[e] : 0.0f;
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int64_t k = k0 + u;
+            const float t = row[min(k, K - 1) * ks];
+            v[u] = ok && k < k_hi ? t : 0.0f;
+        }
+    }
+}
+
+template <int NW, bool AV, bool BV> __global__ __launch_bounds__(64 * NW) void gemm_small_f32_k(const GemmGeneric p) {
+    __shared__ float part[NW][32 * 33];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5, l32 = lane & 31;
+    const int64_t m0 = (int64_t)blockIdx.y * 32, n0 = (int64_t)blockIdx.x * 32, bz = blockIdx.z;
+    const float *A = (const float *)p.A + bz * p.batch_a, *B = (const float *)p.B + bz * p.batch_b;
+    const int64_t a_rs = p.trans_a ? 1 : p.K, a_ks = p.trans_a ? p.M : 1;
+    const int64_t b_rs = p.trans_b ? p.K : 1, b_ks = p.trans_b ? 1 : p.N;
+    int64_t half = ((p.K + NW - 1) / NW + 1) / 2;                    // k per lane half
+    if (AV || BV) half = (half + 3) / 4 * 4;
+    const int64_t k_lo = min(p.K, (2 * wave + h) * half), k_hi = min(p.K, k_lo + half);
+    const int64_t row = m0 + l32, col = n0 + l32;
+    const bool row_ok = row < p.M, col_ok = col < p.N;
+    const float *ap = A + min(row, p.M - 1) * a_rs, *bp = B + min(col, p.N - 1) * b_rs;
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+    for (int64_t s0 = 0; s0 < half; s0 += 8) { // both halves run the same number of steps: the MFMA needs the whole wave
+        float a[8], b[8];
+        load8<AV>(ap, a_ks, k_lo + s0, k_hi, p.K, row_ok, a);
+        load8<BV>(bp, b_ks, k_lo + s0, k_hi, p.K, col_ok, b);
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+    }
+    // register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the tile
+#pragma unroll
+    for (int r = 0; r < 16; r++) part[wave][((r >> 2) * 8 + h * 4 + (r & 3)) * 33 + l32] = acc[r];
+    __syncthreads();
+    for (int e = threadIdx.x; e < 1024; e += 64 * NW) {
+        const int rr = e >> 5, cc = e & 31;
+        const int64_t orow = m0 + rr, ocol = n0 + cc;
+        if (orow >= p.M || ocol >= p.N) continue;
+        float sum = part[0][rr * 33 + cc];
+#pragma unroll
+        for (int w = 1; w < NW; w++) sum += part[w][rr * 33 + cc];
+        float v = sum * p.alpha;
+        if (p.epilogue >= 1) {
+            if (p.bias_dtype == DT_BF16) v += bf16_to_f32(((const uint16_t *)p.bias)[ocol]);
+            else if (p.bias_dtype == DT_F16) v += f16_to_f32(((const uint16_t *)p.bias)[ocol]);
+            else v += ((const float *)p.bias)[ocol];
+        }
+        if (p.epilogue == 2) v = (v > 0.0f ? 1.0f : 0.0f) * v;
+        if (p.epilogue == 3) v = gelu_ref(v);
+        const int64_t o = bz * p.batch_c + orow * p.N + ocol;
+        if (p.residual) v += ((const float *)p.residual)[o];
+        ((float *)p.C)[o] = v;
+    }
+}
+
+// waves per tile of the small kernel: about 16 k per wave, at most 8 waves; 0: the shape goes to the 64 x 64 kernel
+int gemm_small_waves(const GemmGeneric &p) {
+    if (p.dtype != DT_F32 || p.out_dtype != DT_F32 || p.K < 1) return 0;
+    const int64_t tiles = ((p.M + 31) / 32) * ((p.N + 31) / 32) * p.batch;
+    if (tiles > 256 || (p.N + 31) / 32 > 65535 || (p.M + 31) / 32 > 65535) return 0;
+    int nw = 1;
+    while (nw < 8 && p.K > 16 * nw) nw *= 2;
+    return nw;
+}
+
 } // namespace
 
 // Few output tiles and a long K (the weight-gradient and first-layer products of a small MLP): split K over
@@ -216,6 +307,28 @@ hipError_t gemm_generic(const GemmGeneric &p0, hipStream_t st) {
     GemmGeneric p = p0;
     if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return hipSuccess;
     if (p.K < 0 || (p.M + GM - 1) / GM > 65535 || p.batch > 65535) return hipErrorInvalidValue;
+    if (const int nw = gemm_small_waves(p)) {
+        dim3 grid((unsigned)((p.N + 31) / 32), (unsigned)((p.M + 31) / 32), (unsigned)p.batch);
+        // k-contiguous operands whose rows start 16-byte aligned take 4 elements per load
+        const bool k4 = p.K % 4 == 0 && p.K >= 4;
+        const bool av = k4 && !p.trans_a && (uintptr_t)p.A % 16 == 0 && p.batch_a % 4 == 0;
+        const bool bv = k4 && p.trans_b && (uintptr_t)p.B % 16 == 0 && p.batch_b % 4 == 0;
+#define ZK_S(NW) \
+    do { \
+        if (av && bv) hipLaunchKernelGGL((gemm_small_f32_k<NW, true, true>), grid, dim3(64 * NW), 0, st, p); \
+        else if (av) hipLaunchKernelGGL((gemm_small_f32_k<NW, true, false>), grid, dim3(64 * NW), 0, st, p); \
+        else if (bv) hipLaunchKernelGGL((gemm_small_f32_k<NW, false, true>), grid, dim3(64 * NW), 0, st, p); \
+        else hipLaunchKernelGGL((gemm_small_f32_k<NW, false, false>), grid, dim3(64 * NW), 0, st, p); \
+    } while (0)
+        switch (nw) {
+        case 1: ZK_S(1); break;
+        case 2: ZK_S(2); break;
+        case 4: ZK_S(4); break;
+        default: ZK_S(8); break;
+        }
+#undef ZK_S
+        return hipGetLastError();
+    }
     p.splits = gemm_generic_splits(p.M, p.N, p.K, p.batch, &p.k_len);
     if (p.splits > 1 && (!p.workspace || (int64_t)p.batch * p.splits > 65535)) return hipErrorInvalidValue;
     dim3 grid((unsigned)((p.N + GN - 1) / GN), (unsigned)((p.M + GM - 1) / GM), (unsigned)(p.batch * p.splits)), block(256);

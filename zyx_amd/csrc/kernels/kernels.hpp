@@ -49,6 +49,8 @@ struct Reduce {
     void *out;
     void *workspace;           // partial results of the two-stage variants
     uint64_t workspace_bytes;
+    float mul = 0.0f, div = 0.0f;   // float dtypes: out = (reduce * mul) / div + base, a 0 / null step is left out
+    const void *base = nullptr;     // [len(out)] of the same dtype
 };
 uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int axis0);
 hipError_t reduce(const Reduce &p, hipStream_t stream);
@@ -165,6 +167,8 @@ struct IndexOp {
     void *out;
 };
 hipError_t index_op(const IndexOp &p, hipStream_t stream);
+// dst[0, bytes) = src[0, bytes) (ranges must not overlap), as one kernel launch
+hipError_t copy_range(void *dst, const void *src, uint64_t bytes, hipStream_t stream);
 
 // Attention core over the packed c_attn output qkv[B, T, 3, H, dh] -> y[B, T, H*dh]:
 // y = softmax(scale q k^T) / keep . v per head, no mask. lse[B, H, T] (optional) = ln sum exp(scale q k^T).

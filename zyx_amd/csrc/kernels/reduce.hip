@@ -84,6 +84,26 @@ template <int OP> __device__ __forceinline__ int wave_fold(int v) {
     return wave_allreduce_i32(v, OpMaxI());
 }
 
+// Final store of result i: for the float dtypes optionally (acc * mul) / div + base[i], each step a separate f32
+// operation in that order (`p - g * lr` with mul = -lr and base = p; a mean with div = n); integers store acc as is.
+struct Epilogue {
+    float mul, div;     // 0 = step absent
+    const void *base;   // nullptr = absent; same dtype and length as out
+};
+template <int DT> __device__ __forceinline__ void store_result(typename Elem<DT>::S *out, int64_t i, typename Elem<DT>::A acc,
+                                                               const Epilogue &e) {
+    if constexpr (std::is_same<typename Elem<DT>::A, float>::value) {
+#pragma clang fp contract(off)
+        float v = acc;
+        if (e.mul != 0.0f) v = v * e.mul;
+        if (e.div != 0.0f) v = v / e.div;
+        if (e.base) v = v + Elem<DT>::ld((const typename Elem<DT>::S *)e.base, i);
+        Elem<DT>::st(out, i, v);
+    } else {
+        Elem<DT>::st(out, i, acc);
+    }
+}
+
 // One wave folds columns [c0, c1) of one row. VEC: row start and c0 are 4-element aligned.
 template <int DT, int OP, bool VEC>
 __device__ __forceinline__ typename Elem<DT>::A fold_row_span(const typename Elem<DT>::S *__restrict__ xr, int64_t c0,
@@ -111,7 +131,7 @@ template <int DT, int OP, bool VEC>
 __global__ __launch_bounds__(256) void reduce_rows_wave_k(const typename Elem<DT>::S *__restrict__ x,
                                                           typename Elem<DT>::S *__restrict__ out,
                                                           typename Elem<DT>::A *__restrict__ partial, int64_t rows,
-                                                          int64_t cols, int segs, int64_t seg_len) {
+                                                          int64_t cols, int segs, int64_t seg_len, const Epilogue epi) {
     const int lane = threadIdx.x & 63;
     const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (item >= rows * segs) return; // whole wave; no cross-wave synchronisation below
@@ -121,7 +141,7 @@ __global__ __launch_bounds__(256) void reduce_rows_wave_k(const typename Elem<DT
     typename Elem<DT>::A acc = fold_row_span<DT, OP, VEC>(x + row * cols, c0, c1, lane, 64);
     acc = wave_fold<OP>(acc);
     if (lane == 0) {
-        if (segs == 1) Elem<DT>::st(out, row, acc);
+        if (segs == 1) store_result<DT>(out, row, acc, epi);
         else partial[item] = acc;
     }
 }
@@ -129,7 +149,8 @@ __global__ __launch_bounds__(256) void reduce_rows_wave_k(const typename Elem<DT
 // second stage: fold `segs` raw partials per row (accumulator type), store as DT.
 template <int DT, int OP>
 __global__ __launch_bounds__(256) void reduce_partials_k(const typename Elem<DT>::A *__restrict__ partial,
-                                                         typename Elem<DT>::S *__restrict__ out, int64_t rows, int segs) {
+                                                         typename Elem<DT>::S *__restrict__ out, int64_t rows, int segs,
+                                                         const Epilogue epi) {
     typedef typename Elem<DT>::A A;
     typedef Fold<OP, A> F;
     const int lane = threadIdx.x & 63;
@@ -138,7 +159,7 @@ __global__ __launch_bounds__(256) void reduce_partials_k(const typename Elem<DT>
     A acc = F::init();
     for (int s = lane; s < segs; s += 64) acc = F::f(acc, partial[row * segs + s]);
     acc = wave_fold<OP>(acc);
-    if (lane == 0) Elem<DT>::st(out, row, acc);
+    if (lane == 0) store_result<DT>(out, row, acc, epi);
 }
 
 // columns: a workgroup owns a strip of 256 columns (lane -> 4 adjacent columns when VEC,
@@ -148,7 +169,7 @@ template <int DT, int OP, bool VEC>
 __global__ __launch_bounds__(256) void reduce_cols_k(const typename Elem<DT>::S *__restrict__ x,
                                                      typename Elem<DT>::S *__restrict__ out,
                                                      typename Elem<DT>::A *__restrict__ partial, int64_t rows,
-                                                     int64_t cols, int chunks, int64_t chunk_len) {
+                                                     int64_t cols, int chunks, int64_t chunk_len, const Epilogue epi) {
     typedef typename Elem<DT>::A A;
     typedef Fold<OP, A> F;
     constexpr int W = VEC ? 4 : 1;
@@ -180,7 +201,7 @@ __global__ __launch_bounds__(256) void reduce_cols_k(const typename Elem<DT>::S 
 #pragma unroll
         for (int k = 0; k < W; k++) {
             A v = F::f(F::f(lds[0][lane * W + k], lds[1][lane * W + k]), F::f(lds[2][lane * W + k], lds[3][lane * W + k]));
-            if (chunks == 1) Elem<DT>::st(out, c + k, v);
+            if (chunks == 1) store_result<DT>(out, c + k, v, epi);
             else partial[(int64_t)chunk * cols + c + k] = v;
         }
     }
@@ -189,7 +210,7 @@ __global__ __launch_bounds__(256) void reduce_cols_k(const typename Elem<DT>::S 
 template <int DT, int OP>
 __global__ __launch_bounds__(256) void reduce_col_partials_k(const typename Elem<DT>::A *__restrict__ partial,
                                                              typename Elem<DT>::S *__restrict__ out, int64_t cols,
-                                                             int chunks) {
+                                                             int chunks, const Epilogue epi) {
     typedef typename Elem<DT>::A A;
     typedef Fold<OP, A> F;
     // a workgroup folds 64 columns: lane -> column, the 4 waves split the chunks, LDS joins them
@@ -203,7 +224,7 @@ __global__ __launch_bounds__(256) void reduce_col_partials_k(const typename Elem
     }
     lds[wave][lane] = acc;
     __syncthreads();
-    if (wave == 0 && c < cols) Elem<DT>::st(out, c, F::f(F::f(lds[0][lane], lds[1][lane]), F::f(lds[2][lane], lds[3][lane])));
+    if (wave == 0 && c < cols) store_result<DT>(out, c, F::f(F::f(lds[0][lane], lds[1][lane]), F::f(lds[2][lane], lds[3][lane])), epi);
 }
 
 struct RowPlan { int segs; int64_t seg_len; };
@@ -240,26 +261,27 @@ template <int DT, int OP> hipError_t launch(const Reduce &p, hipStream_t st) {
     S *out = (S *)p.out;
     A *ws = (A *)p.workspace;
     const int esz = (int)sizeof(S);
+    const Epilogue epi{p.mul, p.div, p.base};
     if (!p.axis0) {
         bool vec = (p.cols * esz) % (4 * esz) == 0 && p.cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
         RowPlan pl = plan_rows(p.rows, p.cols);
         if (pl.segs > 1 && (uint64_t)p.rows * pl.segs * sizeof(A) > p.workspace_bytes) return hipErrorInvalidValue;
         int64_t items = p.rows * pl.segs;
         dim3 grid((unsigned)((items + 3) / 4)), block(256);
-        if (vec) hipLaunchKernelGGL((reduce_rows_wave_k<DT, OP, true>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.segs, pl.seg_len);
-        else hipLaunchKernelGGL((reduce_rows_wave_k<DT, OP, false>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.segs, pl.seg_len);
+        if (vec) hipLaunchKernelGGL((reduce_rows_wave_k<DT, OP, true>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.segs, pl.seg_len, epi);
+        else hipLaunchKernelGGL((reduce_rows_wave_k<DT, OP, false>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.segs, pl.seg_len, epi);
         if (pl.segs > 1)
-            hipLaunchKernelGGL((reduce_partials_k<DT, OP>), dim3((unsigned)((p.rows + 3) / 4)), block, 0, st, ws, out, p.rows, pl.segs);
+            hipLaunchKernelGGL((reduce_partials_k<DT, OP>), dim3((unsigned)((p.rows + 3) / 4)), block, 0, st, ws, out, p.rows, pl.segs, epi);
     } else {
         bool vec = p.cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
         ColPlan pl = plan_cols(p.rows, p.cols, vec);
         if (pl.chunks > 1 && (uint64_t)pl.chunks * p.cols * sizeof(A) > p.workspace_bytes) return hipErrorInvalidValue;
         int64_t strips = (p.cols + (vec ? 255 : 63)) / (vec ? 256 : 64);
         dim3 grid((unsigned)strips, (unsigned)pl.chunks), block(256);
-        if (vec) hipLaunchKernelGGL((reduce_cols_k<DT, OP, true>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len);
-        else hipLaunchKernelGGL((reduce_cols_k<DT, OP, false>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len);
+        if (vec) hipLaunchKernelGGL((reduce_cols_k<DT, OP, true>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len, epi);
+        else hipLaunchKernelGGL((reduce_cols_k<DT, OP, false>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len, epi);
         if (pl.chunks > 1)
-            hipLaunchKernelGGL((reduce_col_partials_k<DT, OP>), dim3((unsigned)((p.cols + 63) / 64)), block, 0, st, ws, out, p.cols, pl.chunks);
+            hipLaunchKernelGGL((reduce_col_partials_k<DT, OP>), dim3((unsigned)((p.cols + 63) / 64)), block, 0, st, ws, out, p.cols, pl.chunks, epi);
     }
     return hipGetLastError();
 }
@@ -289,7 +311,8 @@ hipError_t reduce(const Reduce &p, hipStream_t st) {
 #define ZK_EMPTY(DTC, DT, OP)                                                                                        \
     case DTC * 2 + OP:                                                                                                \
         hipLaunchKernelGGL((reduce_partials_k<DT, OP>), dim3((unsigned)((n_out + 3) / 4)), dim3(256), 0, st,          \
-                           (const typename Elem<DT>::A *)nullptr, (typename Elem<DT>::S *)p.out, n_out, 0);           \
+                           (const typename Elem<DT>::A *)nullptr, (typename Elem<DT>::S *)p.out, n_out, 0,            \
+                           Epilogue{p.mul, p.div, p.base});                                                            \
         return hipGetLastError();
             ZK_EMPTY(DT_F32, 0, 0) ZK_EMPTY(DT_F32, 0, 1) ZK_EMPTY(DT_BF16, 1, 0) ZK_EMPTY(DT_BF16, 1, 1)
             ZK_EMPTY(DT_F16, 2, 0) ZK_EMPTY(DT_F16, 2, 1) ZK_EMPTY(DT_I32, 3, 0) ZK_EMPTY(DT_I32, 3, 1)

@@ -210,6 +210,9 @@ void event_retire(zhip_ctx *c, EventSlot *s) {
 // consumes its wait list). Events recorded on the same in-order stream need no wait.
 int32_t wait_and_consume(zhip_ctx *c, int stream_idx, const zhip_event *evs, size_t n, int32_t status) {
     int32_t rc = ZHIP_OK;
+    // Streams run in order: of several events recorded on one stream only the latest needs a wait (a cross-stream
+    // wait is the expensive part of a launch on the host). Slot -1 / -2 are the pool and plan streams.
+    EventSlot *latest[kLaunchStreams + 2] = {nullptr};
     for (size_t i = 0; i < n; i++) {
         if (evs[i] == 0) continue;
         EventSlot *s = event_lookup(c, evs[i]);
@@ -218,11 +221,18 @@ int32_t wait_and_consume(zhip_ctx *c, int stream_idx, const zhip_event *evs, siz
             continue;
         }
         if (s->stream != stream_idx) {
+            EventSlot *&l = latest[s->stream == -1 ? kLaunchStreams : s->stream == -2 ? kLaunchStreams + 1 : s->stream];
+            if (!l || s->seq > l->seq) l = s;
+        }
+    }
+    for (EventSlot *s : latest)
+        if (s) {
             hipError_t e = hipStreamWaitEvent(stream_of(c, stream_idx), s->ev, 0);
             if (e != hipSuccess) rc = c->fail(status, "hipStreamWaitEvent failed: %s", hipGetErrorString(e));
         }
-        event_retire(c, s);
-    }
+    for (size_t i = 0; i < n; i++)
+        if (evs[i] != 0)
+            if (EventSlot *s = event_lookup(c, evs[i])) event_retire(c, s);
     return rc;
 }
 
@@ -392,10 +402,15 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16 && d.dtype != ZHIP_F16 && d.dtype != ZHIP_I32)
             return c->fail(ZHIP_KERNEL_COMPILATION, "reduce: dtype %d not implemented", d.dtype);
         if ((d.flags & ~1) || (d.iparams[0] != 0 && d.iparams[0] != 1)) return c->fail(ZHIP_KERNEL_COMPILATION, "reduce: bad flags/op");
-        p.n_in = 1;
+        const bool base = d.iparams[1] != 0;
+        if ((base || d.fparams[0] != 0.0f || d.fparams[1] != 0.0f) && d.dtype == ZHIP_I32)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "reduce: scale / base apply to float dtypes only");
+        if (!std::isfinite(d.fparams[0]) || !std::isfinite(d.fparams[1])) return c->fail(ZHIP_KERNEL_COMPILATION, "reduce: scale is not finite");
+        p.n_in = base ? 2 : 1;
         p.n_out = 1;
         p.need[0] = (uint64_t)rows * cols * dtype_bytes(d.dtype);
         p.need[1] = (uint64_t)((d.flags & 1) ? cols : rows) * dtype_bytes(d.dtype);
+        p.need[2] = p.need[1];
         p.workspace_bytes = zk::reduce_workspace_bytes(rows, cols, d.flags & 1);
         return ZHIP_OK;
     }
@@ -638,7 +653,10 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         a.op = d.iparams[0];
         a.axis0 = d.flags & 1;
         a.x = ptr[0];
-        a.out = ptr[1];
+        a.base = d.iparams[1] != 0 ? ptr[1] : nullptr;
+        a.out = ptr[p.n_in];
+        a.mul = d.fparams[0];
+        a.div = d.fparams[1];
         a.workspace = p.workspace;
         a.workspace_bytes = p.workspace_bytes;
         return zk::reduce(a, st);
@@ -1133,9 +1151,15 @@ ZHIP_EXPORT int32_t zhip_d2d(zhip_ctx *c, zhip_buf src, uint64_t src_off, zhip_b
     if (src_off > s->bytes || bytes > s->bytes - src_off || dst_off > d->bytes || bytes > d->bytes - dst_off)
         return c->fail(ZHIP_MEMORY_COPY_H2P, "d2d: %llu bytes at offsets %llu -> %llu exceed a buffer", (unsigned long long)bytes,
                        (unsigned long long)src_off, (unsigned long long)dst_off);
-    if (bytes)
-        HIPCHK(c, hipMemcpyAsync((char *)d->ptr + dst_off, (const char *)s->ptr + src_off, bytes, hipMemcpyDeviceToDevice, c->pool_stream),
-               ZHIP_MEMORY_COPY_H2P);
+    if (bytes) {
+        char *to = (char *)d->ptr + dst_off;
+        const char *from = (const char *)s->ptr + src_off;
+        // small moves go through a copy kernel (cheaper to issue); overlapping ranges of one buffer and large moves
+        // through the runtime's copy
+        const bool overlap = s == d && src_off < dst_off + bytes && dst_off < src_off + bytes;
+        if (bytes <= (4u << 20) && !overlap) HIPCHK(c, zk::copy_range(to, from, bytes, c->pool_stream), ZHIP_MEMORY_COPY_H2P);
+        else HIPCHK(c, hipMemcpyAsync(to, from, bytes, hipMemcpyDeviceToDevice, c->pool_stream), ZHIP_MEMORY_COPY_H2P);
+    }
     return event_record(c, -1, ZHIP_MEMORY_COPY_H2P, ev);
 }
 

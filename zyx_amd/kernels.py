@@ -158,27 +158,36 @@ def run_chain(dev: HIPDevice, pool: HIPMemoryPool, chain: Chain, arrays) -> np.n
     return res
 
 
-def reduce_desc(rows: int, cols: int, op: str = "sum", axis0: bool = False, dtype: DType = DType.F32) -> KernelDesc:
+def reduce_desc(rows: int, cols: int, op: str = "sum", axis0: bool = False, dtype: DType = DType.F32, mul: float = 0.0,
+                div: float = 0.0, base: bool = False) -> KernelDesc:
+    """out = reduce (* mul) (/ div) (+ base); args: x, (base), out."""
     d = KernelDesc()
     d.kind, d.dtype, d.out_dtype = K_REDUCE, DType(dtype), DType(dtype)
     d.flags = 1 if axis0 else 0
     d.dims[0], d.dims[1] = rows, cols
     d.iparams[0] = {"sum": 0, "max": 1}[op]
+    d.iparams[1] = int(bool(base))
+    d.fparams[0], d.fparams[1] = mul, div
     return d
 
 
 def reduce(dev: HIPDevice, pool: HIPMemoryPool, x: np.ndarray, op: str = "sum", axis0: bool = False,
-           dtype: DType = DType.F32) -> np.ndarray:
+           dtype: DType = DType.F32, mul: float = 0.0, div: float = 0.0, base: np.ndarray | None = None) -> np.ndarray:
     x = np.ascontiguousarray(x, _NP_STORE[DType(dtype)])
     rows, cols = x.shape
-    prog = dev.register_kernel(reduce_desc(rows, cols, op, axis0, dtype))
+    prog = dev.register_kernel(reduce_desc(rows, cols, op, axis0, dtype, mul, div, base is not None))
     xb, e0 = to_device(pool, x)
     n_out = cols if axis0 else rows
+    bufs, waits = [xb], [e0]
+    if base is not None:
+        bb, eb = to_device(pool, np.ascontiguousarray(base, x.dtype))
+        bufs.append(bb)
+        waits.append(eb)
     ob, e1 = alloc_like(pool, n_out, x.itemsize)
-    done = dev.launch(prog, pool, [xb, ob], [e0, e1])
+    done = dev.launch(prog, pool, bufs + [ob], waits + [e1])
     res = to_host(pool, ob, (n_out,), x.dtype, [done])
-    pool.deallocate(xb, [])
-    pool.deallocate(ob, [])
+    for buf in bufs + [ob]:
+        pool.deallocate(buf, [])
     dev.release(prog)
     return res
 

@@ -77,18 +77,19 @@ class MLPTrainStep:
             (prog(K.gemm_desc(batch, hidden, n_in, f32, f32, trans_b=True, epilogue="bias_relu")), [x, w1, b1, h]),
             (prog(K.gemm_desc(batch, n_out, hidden, f32, f32, trans_b=True, epilogue="bias")), [h, w2, b2, logits]),
             (prog(K.cross_entropy_desc(batch, n_out, True, True, 1.0 / batch)), [logits, y, loss, dlogits]),
-            (prog(K.reduce_desc(1, batch, "sum")), [loss, loss_sum]),
-            (prog(scale.desc()), [loss_sum, mean_loss]),
+        ] + ([(prog(K.reduce_desc(1, batch, "sum", div=float(batch))), [loss, mean_loss])] if fused_update else
+             [(prog(K.reduce_desc(1, batch, "sum")), [loss, loss_sum]), (prog(scale.desc()), [loss_sum, mean_loss])]) + [
             dw2_node,
+            # bias gradients are column sums; the fused form stores b - lr * sum straight into the new bias
+            (prog(K.reduce_desc(batch, n_out, "sum", axis0=True, mul=-lr, base=True)), [dlogits, b2, nb2]) if fused_update else
             (prog(K.reduce_desc(batch, n_out, "sum", axis0=True)), [dlogits, db2]),
             (prog(K.gemm_desc(batch, hidden, n_out, f32, f32)), [dlogits, w2, dh]),
             (prog(relu_bwd.desc()), [h, dh, dpre]),
             dw1_node,
+            (prog(K.reduce_desc(batch, hidden, "sum", axis0=True, mul=-lr, base=True)), [dpre, b1, nb1]) if fused_update else
             (prog(K.reduce_desc(batch, hidden, "sum", axis0=True)), [dpre, db1]),
-        ] + ([] if fused_update else [(sgd(hidden, n_in), [w1, dw1, nw1]), (sgd(n_out, hidden), [w2, dw2, nw2])]) + [
-            (sgd(1, hidden), [b1, db1, nb1]),
-            (sgd(1, n_out), [b2, db2, nb2]),
-        ]
+        ] + ([] if fused_update else [(sgd(hidden, n_in), [w1, dw1, nw1]), (sgd(n_out, hidden), [w2, dw2, nw2]),
+                                      (sgd(1, hidden), [b1, db1, nb1]), (sgd(1, n_out), [b2, db2, nb2])])
         # the updated parameters are written to fresh buffers (a kernel's outputs never alias its
         # inputs); the two parameter sets swap roles every step, so two plans alternate. Each plan also reads its
         # own batch buffers: the next batch is copied in while the current step still runs.
