@@ -138,8 +138,11 @@ enum zhip_kernel_kind {
      * narrowing stores truncate); flags bit 0: A is stored [K,M], bit 1: B is stored [N,K]
      * (a Linear weight [out,in]);
      * iparams[0] = epilogue: 0 none, 1 + bias, 2 + bias then ReLU, 3 + bias then GELU;
-     * iparams[1] = dtype of bias; iparams[2] != 0: a residual[batch, M, N] of dtype out_dtype is
+     * iparams[1] = dtype of bias; iparams[2] = 1: a residual[batch, M, N] of dtype out_dtype is
      * added last (the `x + module(x)` of a transformer block, zyx-examples/examples/nanogpt.rs:89-95);
+     * iparams[2] = 2: that tensor is a mask instead, the result is multiplied by (mask > 0) last: the
+     * gradient of relu = cmpgt(0) * x applied to a product dY . W (zyx/src/tensor/elementwise.rs:289-293,
+     * zyx/src/graph/autograd.rs:120-125), with the forward's activations as the mask;
      * fparams[0] = alpha scaling the product (0 = 1).
      * Products and sums are f32. bf16 problems with M, N multiples of 256 and K a multiple of
      * 64 run on the 256x256 LDS-tiled MFMA kernel, the rest on a 64x64 one.

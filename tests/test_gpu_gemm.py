@@ -276,3 +276,27 @@ def test_bf16_column_blocks(hip, oracle, trans_a, trans_b):
     assert np.all(np.abs(got32 - w) <= 1e-3 * np.abs(w) + 2e-5 * mag + 1e-6)
     got16 = gemm(dev, pool, a, b, out_dtype=DType.BF16, residual=res, **kw)
     assert np.array_equal(got16, oracle.f32_to_bf16(got32))
+
+
+@pytest.mark.parametrize("dtype", [DType.F32, DType.BF16])
+@pytest.mark.parametrize("mnk", [(64, 128, 10), (70, 33, 45), (256, 512, 64), (1000, 300, 96)])
+def test_relu_mask_epilogue(hip, oracle, dtype, mnk):
+    """C = (mask > 0) * (A . B): the gradient of relu folded into the product that feeds it; equal, bit for bit, to
+    masking the plain product afterwards (small, general and split-K paths)."""
+    dev, pool = hip
+    m, n, k = mnk
+    r = oracle.Rng(m + n)
+    a, b, mask = r.randn((m, k)), r.randn((k, n)), r.randn((m, n))
+    mask[0, :] = 0.0
+    mask[1, 0] = -0.0
+    if dtype == DType.BF16:
+        a, b = oracle.f32_to_bf16(a), oracle.f32_to_bf16(b)
+    plain = gemm(dev, pool, a, b, dtype=dtype, out_dtype=DType.F32)
+    got = gemm(dev, pool, a, b, dtype=dtype, out_dtype=DType.F32, residual=mask, relu_mask=True)
+    want = (mask > 0).astype(np.float32) * plain
+    if dtype == DType.F32:
+        assert np.array_equal(got, want)
+    else:  # the unmasked bf16 product may run on the LDS-tiled kernel, which sums in another order
+        np.testing.assert_allclose(got, want, rtol=0, atol=2e-6 * np.abs(plain).max() * np.sqrt(k))
+        assert np.array_equal(got == 0, want == 0)
+    assert (got[0] == 0).all() and got[1, 0] == 0

@@ -157,9 +157,8 @@ __global__ __launch_bounds__(256) void gemm_generic_k(const GemmGeneric p) {
         const int64_t o = row * p.N + col;
         if (p.residual) {
             const char *R = (const char *)p.residual + (int64_t)blockIdx.z * p.batch_c * (ODT == DT_F32 ? 4 : 2);
-            if (ODT == DT_F32) v += ((const float *)R)[o];
-            else if (ODT == DT_BF16) v += bf16_to_f32(((const uint16_t *)R)[o]);
-            else v += f16_to_f32(((const uint16_t *)R)[o]);
+            const float r = ODT == DT_F32 ? ((const float *)R)[o] : ODT == DT_BF16 ? bf16_to_f32(((const uint16_t *)R)[o]) : f16_to_f32(((const uint16_t *)R)[o]);
+            v = p.residual_is_mask ? (r > 0.0f ? 1.0f : 0.0f) * v : v + r;
         }
         if (ODT == DT_F32) ((float *)C)[o] = v;
         else if (ODT == DT_BF16) ((uint16_t *)C)[o] = f32_to_bf16_trunc(v);
@@ -185,9 +184,8 @@ template <int ODT> __global__ __launch_bounds__(256) void gemm_generic_fold_k(co
     if (p.epilogue == 3) v = gelu_ref(v);
     const int64_t oo = bz * p.batch_c + o;
     if (p.residual) {
-        if (ODT == DT_F32) v += ((const float *)p.residual)[oo];
-        else if (ODT == DT_BF16) v += bf16_to_f32(((const uint16_t *)p.residual)[oo]);
-        else v += f16_to_f32(((const uint16_t *)p.residual)[oo]);
+        const float r = ODT == DT_F32 ? ((const float *)p.residual)[oo] : ODT == DT_BF16 ? bf16_to_f32(((const uint16_t *)p.residual)[oo]) : f16_to_f32(((const uint16_t *)p.residual)[oo]);
+        v = p.residual_is_mask ? (r > 0.0f ? 1.0f : 0.0f) * v : v + r;
     }
     if (ODT == DT_F32) ((float *)p.C)[oo] = v;
     else if (ODT == DT_BF16) ((uint16_t *)p.C)[oo] = f32_to_bf16_trunc(v);
@@ -269,7 +267,10 @@ template <int NW, bool AV, bool BV> __global__ __launch_bounds__(64 * NW) void g
         if (p.epilogue == 2) v = (v > 0.0f ? 1.0f : 0.0f) * v;
         if (p.epilogue == 3) v = gelu_ref(v);
         const int64_t o = bz * p.batch_c + orow * p.N + ocol;
-        if (p.residual) v += ((const float *)p.residual)[o];
+        if (p.residual) {
+            const float r = ((const float *)p.residual)[o];
+            v = p.residual_is_mask ? (r > 0.0f ? 1.0f : 0.0f) * v : v + r;
+        }
         ((float *)p.C)[o] = v;
     }
 }

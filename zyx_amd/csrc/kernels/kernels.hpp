@@ -100,6 +100,7 @@ struct GemmGeneric {
     int epilogue, bias_dtype;
     float alpha;
     const void *A, *B, *bias, *residual; // residual (dtype out_dtype, [batch, M, N]) may be null
+    int residual_is_mask = 0;            // the residual is not added: the result is multiplied by (residual > 0)
     void *C;
     void *workspace;      // gemm_generic_workspace_bytes(M, N, K, batch) bytes, may be null when that is 0
     int splits;           // set by the launcher

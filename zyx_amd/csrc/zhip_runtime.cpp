@@ -312,7 +312,7 @@ zk::Elementwise elementwise_args(const zhip_kernel_desc &d) {
 bool gemm_takes_fast_path(const zhip_kernel_desc &d) {
     const int64_t batch = d.dims[3] ? d.dims[3] : 1;
     const float alpha = d.fparams[0] == 0.0f ? 1.0f : d.fparams[0];
-    return d.dtype == ZHIP_BF16 && batch == 1 && alpha == 1.0f && (d.iparams[0] == 0 || d.iparams[1] != ZHIP_F16) &&
+    return d.dtype == ZHIP_BF16 && batch == 1 && alpha == 1.0f && (d.iparams[0] == 0 || d.iparams[1] != ZHIP_F16) && d.iparams[2] != 2 &&
            zk::gemm_bf16_supported(d.dims[0], d.dims[1], d.dims[2], d.flags & ZHIP_GEMM_TRANS_A ? 1 : 0,
                                    d.flags & ZHIP_GEMM_TRANS_B ? 1 : 0, d.out_dtype == ZHIP_BF16);
 }
@@ -418,7 +418,8 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         int64_t M = d.dims[0], N = d.dims[1], K = d.dims[2], batch = d.dims[3] ? d.dims[3] : 1;
         int epi = d.iparams[0];
         if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || batch > 65535) return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: M, N, K, batch out of range");
-        if (epi < 0 || epi > 3 || (d.flags & ~3)) return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: bad epilogue/flags");
+        if (epi < 0 || epi > 3 || (d.flags & ~3) || d.iparams[2] < 0 || d.iparams[2] > 2)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: bad epilogue/flags");
         bool float_in = d.dtype == ZHIP_F32 || d.dtype == ZHIP_BF16 || d.dtype == ZHIP_F16;
         if (!float_in || (d.out_dtype != ZHIP_F32 && d.out_dtype != d.dtype))
             return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: no kernel for dtype %d -> %d", d.dtype, d.out_dtype);
@@ -702,6 +703,7 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         g.B = ptr[1];
         g.bias = g.epilogue ? ptr[2] : nullptr;
         g.residual = residual;
+        g.residual_is_mask = d.iparams[2] == 2;
         g.workspace = p.workspace;
         g.C = ptr[p.n_in];
         return zk::gemm_generic(g, st);

@@ -205,22 +205,23 @@ def gemm_desc(m: int, n: int, k: int, dtype: DType = DType.BF16, out_dtype: DTyp
     d.kind, d.dtype, d.out_dtype = K_GEMM, DType(dtype), DType(out_dtype)
     d.flags = (GEMM_TRANS_A if trans_a else 0) | (GEMM_TRANS_B if trans_b else 0)
     d.dims[0], d.dims[1], d.dims[2], d.dims[3] = m, n, k, batch
-    d.iparams[0], d.iparams[1], d.iparams[2] = EPILOGUE[epilogue], int(bias_dtype), int(bool(residual))
+    d.iparams[0], d.iparams[1], d.iparams[2] = EPILOGUE[epilogue], int(bias_dtype), 2 if residual == "relu_mask" else int(bool(residual))
     d.fparams[0] = alpha
     return d
 
 
 def gemm(dev: HIPDevice, pool: HIPMemoryPool, a: np.ndarray, b: np.ndarray, bias: np.ndarray | None = None,
          dtype: DType = DType.BF16, out_dtype: DType = DType.F32, trans_a=False, trans_b=False, epilogue: str = "none",
-         bias_dtype: DType = DType.F32, alpha: float = 1.0, residual: np.ndarray | None = None) -> np.ndarray:
+         bias_dtype: DType = DType.F32, alpha: float = 1.0, residual: np.ndarray | None = None,
+         relu_mask: bool = False) -> np.ndarray:
     """a: [M,K] ([K,M] if trans_a), b: [K,N] ([N,K] if trans_b) in their storage dtype; returns C[M,N]
-    (+ residual[M,N], stored like C)."""
+    (+ residual[M,N], stored like C; with relu_mask the result is multiplied by (residual > 0) instead)."""
     a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
     batch = a.shape[0] if a.ndim == 3 else 1
     m, k = (a.shape[-1], a.shape[-2]) if trans_a else a.shape[-2:]
     n = b.shape[-2] if trans_b else b.shape[-1]
     prog = dev.register_kernel(gemm_desc(m, n, k, dtype, out_dtype, trans_a, trans_b, epilogue, bias_dtype, batch, alpha,
-                                         residual is not None))
+                                         "relu_mask" if relu_mask else residual is not None))
     bufs, waits = [], []
     extra = ((np.ascontiguousarray(bias),) if epilogue != "none" else ()) + \
         ((np.ascontiguousarray(residual, _NP_STORE[DType(out_dtype)]),) if residual is not None else ())

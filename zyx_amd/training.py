@@ -83,8 +83,8 @@ class MLPTrainStep:
             # bias gradients are column sums; the fused form stores b - lr * sum straight into the new bias
             (prog(K.reduce_desc(batch, n_out, "sum", axis0=True, mul=-lr, base=True)), [dlogits, b2, nb2]) if fused_update else
             (prog(K.reduce_desc(batch, n_out, "sum", axis0=True)), [dlogits, db2]),
-            (prog(K.gemm_desc(batch, hidden, n_out, f32, f32)), [dlogits, w2, dh]),
-            (prog(relu_bwd.desc()), [h, dh, dpre]),
+        ] + ([(prog(K.gemm_desc(batch, hidden, n_out, f32, f32, residual="relu_mask")), [dlogits, w2, h, dpre])] if fused_update else
+             [(prog(K.gemm_desc(batch, hidden, n_out, f32, f32)), [dlogits, w2, dh]), (prog(relu_bwd.desc()), [h, dh, dpre])]) + [
             dw1_node,
             (prog(K.reduce_desc(batch, hidden, "sum", axis0=True, mul=-lr, base=True)), [dpre, b1, nb1]) if fused_update else
             (prog(K.reduce_desc(batch, hidden, "sum", axis0=True)), [dpre, db1]),
