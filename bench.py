@@ -28,8 +28,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 N_SETS = 4              # 4 x 268 MB working set > Infinity Cache
 # HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
 # by the same counter's reading for a plain copy kernel of known size in the same run
-# (profiles/softmax_rows_f32_8192x4096.md): 134,054,270 B fetched + 134,320,107 B written.
-TRAFFIC_BYTES = 268374377
+# (profiles/softmax_rows_f32_8192x4096.md): 134,352,818 B fetched + 134,461,653 B written.
+TRAFFIC_BYTES = 268814470
 
 
 def cpu_baseline(x: np.ndarray, budget_s: float = 10.0):

@@ -61,15 +61,18 @@ template <class Op> __device__ __forceinline__ int wave_allreduce_i32(int v, Op 
 // split so its rounding error does not grow with |d|: hi = fl(d*L), lo = the exact
 // remainder of that product plus d times the tail of L; exp2(hi) is then corrected
 // by (1 + lo*ln2). Relative error stays ~2 ulp for the whole range. Where exp2 underflows to 0 the
-// result is 0 whatever the correction term holds: for d = -inf (a masked score) and for products that
-// overflow, `lo` is inf - inf or inf, and 0 * lo would be NaN. A NaN d still gives NaN (r is NaN).
+// result must be 0 whatever the correction term holds: for d = -inf (a masked score) and for products that
+// overflow, `lo` is inf - inf or inf. The correction is therefore formed with v_mul_legacy_f32, whose
+// product is 0 whenever a factor is 0 (0 * NaN = 0 * inf = 0); a NaN d still gives NaN (r is NaN).
 __device__ __forceinline__ float exp_neg(float d) {
     const float L_hi = 1.44269502162933349609375f; // fl(log2 e)
     const float L_lo = 1.925963033500011e-08f;     // log2 e - L_hi
     float hi = d * L_hi;
     float lo = __builtin_fmaf(d, L_hi, -hi) + d * L_lo;
     float r = __builtin_amdgcn_exp2f(hi);
-    return r == 0.0f ? 0.0f : __builtin_fmaf(r, lo * 0.693147182464599609375f, r);
+    float corr;
+    asm("v_mul_legacy_f32 %0, %1, %2" : "=v"(corr) : "v"(r), "v"(lo * 0.693147182464599609375f));
+    return r + corr;
 }
 
 } // namespace zk
