@@ -165,3 +165,23 @@ def test_conv_bf16_gathered_by_the_gemm(hip, oracle, geom):
     mag = oracle.conv2d(np.abs(oracle.bf16_to_f32(x)), np.abs(oracle.bf16_to_f32(wt)), np.abs(oracle.bf16_to_f32(b)), stride, pad, dil)
     assert got32.shape == want32.shape and got32.shape[3] % 8 == 0 and (got32.shape[0] * got32.shape[2] * got32.shape[3]) % 256 == 0
     assert np.all(np.abs(got32 - want32) <= 1e-3 * np.abs(want32) + 2e-5 * mag)
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 8, 8), (32, 128, 56, 56), (1, 5, 17, 24), (3, 2, 2, 16), (1, 1, 9, 40)])
+def test_max_pool_2x2_fast_path(hip, oracle, shape):
+    """2 x 2 / stride 2 windows over rows of a multiple of 8 elements take the vectorised kernel: exact against the
+    oracle, including odd heights, a NaN beside numbers (ignored by fmax) and -inf (the running maximum starts at the
+    lowest finite value, which a window of -inf therefore returns). A window of NaN only is left out: the reference
+    compiles its kernels with -ffast-math, under which fmax of two NaN-free-by-assumption operands is whatever the
+    compiler picked."""
+    dev, pool = hip
+    x = oracle.Rng(shape[2] * shape[3]).randn(shape, 3.0)
+    x[0, 0, 0, 0] = np.nan
+    x[0, 0, 0, 4:6] = -np.inf
+    x[0, 0, 1, 4:6] = -np.inf                # a window of -inf only
+    x[-1, -1, 1, -1] = np.inf
+    args = ((2, 2), (2, 2), (0, 0), (1, 1))
+    got, want = max_pool2d(dev, pool, x, *args), oracle.max_pool2d(x, *args)
+    assert np.array_equal(got, want) and got[0, 0, 0, 2] == np.float32(-3.4028234663852886e38)
+    xb = oracle.f32_to_bf16(x)
+    assert np.array_equal(max_pool2d(dev, pool, xb, *args, dtype=DType.BF16), oracle.max_pool2d(xb, *args, dtype=oracle.BF16))

@@ -168,6 +168,61 @@ __global__ __launch_bounds__(256) void max_pool2d_k(const MaxPool2d p) {
     }
 }
 
+// 2 x 2 windows, stride 2, no padding or dilation, rows of a multiple of 8 elements (the pool after a convolution
+// block): a thread owns 4 neighbouring outputs = 2 input rows x 8 elements, read with 128-bit loads. The running
+// maximum starts at the dtype's lowest finite value like the general kernel's, so NaN and -inf inputs come out alike.
+template <int DT> __global__ __launch_bounds__(256) void max_pool2x2_k(const MaxPool2d p) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const int ow4 = p.OW >> 2;
+    const int64_t total = p.planes * p.OH * ow4;
+    const float lowest = DT == DT_F32 ? -FLT_MAX : -3.3895313892515355e38f;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t prow = i / ow4; // plane * OH + oy
+        const int q = (int)(i - prow * ow4);
+        const int64_t plane = prow / p.OH;
+        const int oy = (int)(prow - plane * p.OH);
+        const int64_t in0 = (plane * p.H + 2 * oy) * (int64_t)p.W + 8 * q;
+        float r[2][8];
+        if (DT == DT_F32) {
+            const float *x = (const float *)p.x;
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const f32x4 t = __builtin_nontemporal_load((const f32x4 *)(x + in0 + (int64_t)a * p.W + 4 * h));
+#pragma unroll
+                    for (int e = 0; e < 4; e++) r[a][4 * h + e] = t[e];
+                }
+        } else {
+            const uint16_t *x = (const uint16_t *)p.x;
+#pragma unroll
+            for (int a = 0; a < 2; a++) {
+                const u32x4 t = __builtin_nontemporal_load((const u32x4 *)(x + in0 + (int64_t)a * p.W));
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    r[a][2 * e] = __uint_as_float(t[e] << 16);
+                    r[a][2 * e + 1] = __uint_as_float(t[e] & 0xffff0000u);
+                }
+            }
+        }
+        float m[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            m[j] = fmaxf(r[1][2 * j + 1], fmaxf(r[1][2 * j], fmaxf(r[0][2 * j + 1], fmaxf(r[0][2 * j], lowest)))); // window order
+        const int64_t o = prow * p.OW + 4 * q;
+        if (DT == DT_F32) {
+            const f32x4 v = {m[0], m[1], m[2], m[3]};
+            __builtin_nontemporal_store(v, (f32x4 *)((float *)p.y + o));
+        } else {
+            const u32x2 v = {(uint32_t)f32_to_bf16_trunc(m[0]) | ((uint32_t)f32_to_bf16_trunc(m[1]) << 16),
+                             (uint32_t)f32_to_bf16_trunc(m[2]) | ((uint32_t)f32_to_bf16_trunc(m[3]) << 16)};
+            __builtin_nontemporal_store(v, (u32x2 *)((uint16_t *)p.y + o));
+        }
+    }
+}
+
 // Patch matrix of the convolution, transposed: a[k][pixel] with k = (c*KH + ky)*KW + kx (the order of the
 // flattened weight [Cout, C*KH*KW]) and pixel = (n*OH + oy)*OW + ox; padding reads as 0. Rows of `a` run
 // along the image rows of x, so reads and the 16-byte writes are both coalesced. One thread = 8 pixels.
@@ -339,6 +394,14 @@ hipError_t conv2d(const Conv2d &p, hipStream_t st) {
 hipError_t max_pool2d(const MaxPool2d &p, hipStream_t st) {
     const int64_t total = p.planes * p.OH * p.OW;
     if (total <= 0) return hipSuccess;
+    if (p.KH == 2 && p.KW == 2 && p.sy == 2 && p.sx == 2 && p.py == 0 && p.px == 0 && p.dy == 1 && p.dx == 1 && p.W % 8 == 0 &&
+        p.H >= 2 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 16 == 0 && (p.dtype == DT_F32 || p.dtype == DT_BF16)) {
+        const int64_t quads = p.planes * p.OH * (p.OW / 4);
+        const unsigned grid = (unsigned)std::min<int64_t>((quads + 255) / 256, 256 * 32);
+        if (p.dtype == DT_F32) hipLaunchKernelGGL((max_pool2x2_k<DT_F32>), dim3(grid), dim3(256), 0, st, p);
+        else hipLaunchKernelGGL((max_pool2x2_k<DT_BF16>), dim3(grid), dim3(256), 0, st, p);
+        return hipGetLastError();
+    }
     int64_t blocks = (total + 255) / 256;
     if (blocks > 256 * 32) blocks = 256 * 32;
     if (p.dtype == DT_F32) hipLaunchKernelGGL((max_pool2d_k<DT_F32>), dim3((unsigned)blocks), dim3(256), 0, st, p);
