@@ -78,3 +78,39 @@ def test_ragged_shapes_next_to_the_fast_paths(hip, oracle):
     got = oracle.bf16_to_f32(K.attention(dev, pool, qkv, 1))
     ref = oracle.bf16_to_f32(oracle.attention(qkv, 1, dtype=oracle.BF16))
     assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 3e-3)
+
+
+def test_shapes_whose_byte_counts_would_overflow_are_refused(hip):
+    """Every tensor of a kernel stays below 2^40 elements: a descriptor whose sizes would wrap the 64-bit byte counts
+    (and so pass the buffer-size check of a launch) is refused at registration."""
+    from zyx_amd import BackendError, ErrorStatus, KernelDesc
+    from zyx_amd import kernels as K
+    dev, pool = hip
+    big = 1 << 62
+
+    def refused(d):
+        with pytest.raises(BackendError) as e:
+            dev.release(dev.register_kernel(d))
+        assert e.value.status == ErrorStatus.KernelCompilation
+
+    for m, n, k in ((64, big, 64), (64, 64, big), (1 << 21, 1 << 21, 64), (64, (1 << 31), 64)):
+        refused(K.gemm_desc(m, n, k, DType.F32, DType.F32))
+    d = K.gemm_desc(64, 64, 64, DType.F32, DType.F32)
+    d.dims[3] = 1 << 20
+    refused(d)
+    d = K.conv2d_desc(1, 3, 8, 8, 4, 3, 3) if hasattr(K, "conv2d_desc") else None
+    if d is not None:
+        for idx, val in ((0, big), (4, big), (4, 1 << 33), (5, 1 << 40), (1, 1 << 30)):
+            e = KernelDesc.from_buffer_copy(bytes(d))
+            e.dims[idx] = val
+            refused(e)
+    d = K.max_pool2d_desc(4, 8, 8) if hasattr(K, "max_pool2d_desc") else None
+    if d is not None:
+        e = KernelDesc.from_buffer_copy(bytes(d))
+        e.dims[0] = big
+        refused(e)
+    d = K.attention_desc(1, 16, 2, 8, DType.F32)
+    for idx, val in ((2, big), (0, 1 << 40), (2, 70000)):
+        e = KernelDesc.from_buffer_copy(bytes(d))
+        e.dims[idx] = val
+        refused(e)

@@ -24,6 +24,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <initializer_list>
 #include <map>
 #include <mutex>
 #include <string>
@@ -331,6 +332,19 @@ zk::Attention attention_args(const zhip_kernel_desc &d) {
     return a;
 }
 
+// True when the product of the non-negative factors stays below 2^40 (elements; checked without overflowing), the
+// bound every tensor of a kernel has to respect so that byte counts and indices fit their types.
+bool elems_fit(std::initializer_list<int64_t> factors) {
+    uint64_t n = 1;
+    for (int64_t f : factors) {
+        if (f < 0) return false;
+        if (f == 0) return true;
+        if ((uint64_t)f >= (1ull << 40) || n > (1ull << 40) / (uint64_t)f) return false;
+        n *= (uint64_t)f;
+    }
+    return n < (1ull << 40);
+}
+
 int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
     p.desc = d;
     switch (d.kind) {
@@ -417,7 +431,9 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
     case ZHIP_K_GEMM: {
         int64_t M = d.dims[0], N = d.dims[1], K = d.dims[2], batch = d.dims[3] ? d.dims[3] : 1;
         int epi = d.iparams[0];
-        if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || batch > 65535) return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: M, N, K, batch out of range");
+        if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || batch > 65535 || M >= (1ll << 31) || N >= (1ll << 31) || K >= (1ll << 31) ||
+            !elems_fit({batch, M, K}) || !elems_fit({batch, K, N}) || !elems_fit({batch, M, N}))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: M, N, K, batch out of range");
         if (epi < 0 || epi > 3 || (d.flags & ~3) || d.iparams[2] < 0 || d.iparams[2] > 2)
             return c->fail(ZHIP_KERNEL_COMPILATION, "gemm: bad epilogue/flags");
         bool float_in = d.dtype == ZHIP_F32 || d.dtype == ZHIP_BF16 || d.dtype == ZHIP_F16;
@@ -499,7 +515,10 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         const int64_t eh = H + 2 * py - (int64_t)dy * (KH - 1) - 1, ew = W + 2 * px - (int64_t)dx * (KW - 1) - 1;
         if (eh < 0 || ew < 0) return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: kernel larger than the padded input");
         const int64_t OH = eh / sy + 1, OW = ew / sx + 1;
-        if (C * H * W >= (1ll << 31) || C * KH * KW >= (1ll << 31) || N * OH * OW >= (1ll << 37) || (KH - 1) * dy >= 32768 || (KW - 1) * dx >= 65536)
+        if (!elems_fit({C, H, W}) || !elems_fit({C, KH, KW}) || !elems_fit({N, OH, OW}) || !elems_fit({N, C, H, W}) ||
+            !elems_fit({Co, C, KH, KW}) || !elems_fit({N, Co, OH, OW}) || Co >= (1ll << 31))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: shape out of range");
+        if (C * H * W >= (1ll << 31) || C * KH * KW >= (1ll << 24) || N * OH * OW >= (1ll << 37) || (KH - 1) * dy >= 32768 || (KW - 1) * dx >= 65536)
             return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: shape out of range");
         const uint64_t e = dtype_bytes(d.dtype);
         int a = 0;
@@ -521,6 +540,8 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
             H >= (1 << 30) || W >= (1 << 30))
             return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: bad shape or stride/padding/dilation");
         if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16) return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: dtype must be F32 or BF16");
+        if (!elems_fit({planes, H, W}) || KH >= (1 << 30) || KW >= (1 << 30))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: tensor too large");
         const int64_t eh = H + 2 * py - (int64_t)dy * (KH - 1) - 1, ew = W + 2 * px - (int64_t)dx * (KW - 1) - 1;
         if (eh < 0 || ew < 0) return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: window larger than the padded input");
         const uint64_t e = dtype_bytes(d.dtype);
@@ -545,8 +566,8 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
                 return c->fail(ZHIP_KERNEL_COMPILATION, "index_select: output shape must equal the input's outside the axis");
             nx *= (uint64_t)d.dims[k];
             no *= (uint64_t)d.dims[4 + k];
+            if (nx >= (1ull << 40) || no >= (1ull << 40)) return c->fail(ZHIP_KERNEL_COMPILATION, "index: tensor too large"); // < 2^71 here
         }
-        if (nx >= (1ull << 40) || no >= (1ull << 40)) return c->fail(ZHIP_KERNEL_COMPILATION, "index: tensor too large");
         const uint64_t e = dtype_bytes(d.dtype), ie = dtype_bytes(idt);
         if (e == 0) return c->fail(ZHIP_KERNEL_COMPILATION, "index: bad dtype");
         if (d.flags == ZHIP_INDEX_SCATTER) {
@@ -569,7 +590,7 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
     case ZHIP_K_ATTENTION:
     case ZHIP_K_ATTENTION_BWD: {
         const int64_t B = d.dims[0], T = d.dims[1], H = d.dims[2], dh = d.dims[3];
-        if (B < 0 || T < 0 || H <= 0 || dh <= 0 || dh > 256 || B * H > 65535 || T >= (1ll << 24) || B * T * 3 * H * dh >= (1ll << 40))
+        if (B < 0 || T < 0 || H <= 0 || dh <= 0 || dh > 256 || B > 65535 || H > 65535 || B * H > 65535 || T >= (1ll << 24) || B * T * 3 * H * dh >= (1ll << 40))
             return c->fail(ZHIP_KERNEL_COMPILATION, "attention: shape out of range (dh <= 256, B*H <= 65535)");
         if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16) return c->fail(ZHIP_KERNEL_COMPILATION, "attention: dtype must be F32 or BF16");
         if ((d.flags & ~(ZHIP_ATTN_LSE | ZHIP_ATTN_CAUSAL)) || d.fparams[0] < 0.0f || !(d.fparams[1] >= 0.0f && d.fparams[1] < 1.0f))
