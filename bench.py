@@ -172,6 +172,53 @@ def extra_streaming(dev, pool, kernels, steps=20, warmup=5):
     return out
 
 
+def extra_graph(dev, pool, steps=60, warmup=10):
+    """Config 1 through the generic path: the training step written as graph nodes (zyx_amd/graph.py), differentiated
+    by the reverse rules, lowered to generated kernels (products optionally matched to the GEMM kernel), kept as one
+    plan; per step two host writes (batch, one-hot labels), one plan launch, four device-side parameter assignments."""
+    import zyx_amd
+    from zyx_amd.graph import Tape
+    from zyx_amd.ir import BOp, UOp
+    F32 = zyx_amd.DType.F32
+    B, NIN, H, NOUT, LR = 64, 784, 128, 10, 0.01
+    out = {}
+    for match in (False, True):
+        rng = np.random.default_rng(42069)  # the same parameters and batches for both runs
+        tape = Tape(dev, pool, match=match)
+        g = tape.graph
+        k1, k2 = 1 / np.sqrt(NIN), 1 / np.sqrt(H)
+        x, onehot = tape.tensor(np.zeros((B, NIN)), F32), tape.tensor(np.zeros((B, NOUT)), F32)
+        params = [tape.tensor(rng.uniform(-k1, k1, (H, NIN)), F32), tape.tensor(rng.uniform(-k1, k1, (H,)), F32),
+                  tape.tensor(rng.uniform(-k2, k2, (NOUT, H)), F32), tape.tensor(rng.uniform(-k2, k2, (NOUT,)), F32)]
+        h = g.relu(g.binary_b(g.dot(x, g.t(params[0])), params[1], BOp.Add))
+        logits = g.binary_b(g.dot(h, g.t(params[2])), params[3], BOp.Add)
+        per_row = g.reduce(g.binary(g.ln_softmax(logits, [-1]), onehot, BOp.Mul), BOp.Add, [1])
+        loss = g.binary(g.unary(g.sum_all(per_row), UOp.Neg), g.const(float(B), F32), BOp.Div)
+        lr = g.const(LR, F32)
+        new = [g.binary(p, g.binary(gr, lr, BOp.Mul), BOp.Sub) for p, gr in zip(params, tape.gradient(loss, params))]
+        t0 = time.perf_counter()
+        plan = tape.plan(new + [loss])
+        build_ms = (time.perf_counter() - t0) * 1e3
+        xs = rng.standard_normal((steps + warmup, B, NIN), dtype=np.float32)
+        hot = np.eye(NOUT, dtype=np.float32)[rng.integers(0, NOUT, (steps + warmup, B))]
+        for i in range(steps + warmup):
+            if i == warmup:
+                tape.sync()
+                t0 = time.perf_counter()
+            tape.write(x, xs[i])
+            tape.write(onehot, hot[i])
+            plan.launch()
+            for p, n in zip(params, new):
+                tape.assign(p, n)
+        final = float(tape.numpy(loss)[0])
+        sps = steps / (time.perf_counter() - t0)
+        out["matched_to_gemm" if match else "generated_kernels_only"] = {
+            "steps_per_s": round(sps, 1), "launches_per_step": plan.launches, "lower_and_compile_ms": round(build_ms, 1),
+            "final_loss": round(final, 5)}
+        tape.close()
+    return out
+
+
 def extra_ir(dev, pool, kernels, steps=20, warmup=5):
     """Kernels generated at run time from a linearized zyx kernel (Device::compile): the config-2 softmax rows written
     as such a kernel (row in registers, local-memory reductions) beside the hand-written one, and an elementwise map."""
@@ -361,6 +408,7 @@ def main():
     ap.add_argument("--streaming-only", action="store_true", help="run only the memory-bound kernel leg")
     ap.add_argument("--attention-only", action="store_true", help="run only the attention core leg")
     ap.add_argument("--ir-only", action="store_true", help="run only the generated-kernel leg")
+    ap.add_argument("--graph-only", action="store_true", help="run only the config-1 training step through the graph path")
     ap.add_argument("--counters", action="store_true",
                     help="short run for `rocprofv3 --pmc`: a few launches of the fused kernel and of a plain copy "
                          "kernel over the same 8192x4096 f32 tensor (known traffic: 134217728 B read + written), "
@@ -382,7 +430,7 @@ def main():
         pool.deinitialize()
         return
 
-    if args.conv_only or args.block_only or args.streaming_only or args.attention_only or args.mlp_only or args.ir_only:
+    if args.conv_only or args.block_only or args.streaming_only or args.attention_only or args.mlp_only or args.ir_only or args.graph_only:
         if args.mlp_only:
             res = {"config1_mlp_train": extra_mlp(dev, pool, cpu=not args.no_cpu)}
         elif args.conv_only:
@@ -393,6 +441,8 @@ def main():
             res = {"config5_attention_core": extra_attention(dev, pool, kernels)}
         elif args.ir_only:
             res = {"generated_kernels": extra_ir(dev, pool, kernels)}
+        elif args.graph_only:
+            res = {"config1_mlp_train_graph_path": extra_graph(dev, pool)}
         else:
             res = {"config5_transformer_block": extra_block(dev, pool, steps=args.steps if args.steps != 200 else 20, cpu=not args.no_cpu)}
         print(json.dumps(res))
@@ -479,7 +529,8 @@ def main():
                         "config5_attention_core": extra_attention(dev, pool, kernels),
                         "config5_transformer_block": extra_block(dev, pool, cpu=not args.no_cpu),
                         "memory_bound_kernels": extra_streaming(dev, pool, kernels),
-                        "generated_kernels": extra_ir(dev, pool, kernels)}
+                        "generated_kernels": extra_ir(dev, pool, kernels),
+                        "config1_mlp_train_graph_path": extra_graph(dev, pool)}
     pool.deinitialize()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(x)

@@ -283,3 +283,34 @@ def test_softmax_runs_on_the_fused_kernel(hip):
         np.testing.assert_allclose(got, e / e.sum(-1, keepdims=True), rtol=2e-6, atol=1e-12)
     finally:
         tape.close()
+
+
+@pytest.mark.parametrize("match", [False, True])
+def test_training_steps_as_a_cached_plan(hip, oracle, match):
+    """Twelve SGD steps of the MNIST-size network: the whole step (forward, cross entropy, gradients by the reverse
+    rules, updates) is lowered once, kept as one plan and replayed; new batches are written into the leaves and the
+    updated parameters assigned back on the device. Loss curve and final parameters against the CPU oracle's
+    training step on the same data."""
+    from graph_cases import mlp_training_graph
+    tape, leaves, (loss, new, params, (x, onehot)) = matched_tape(hip, mlp_training_graph, match=match)
+    try:
+        plan = tape.plan(new + [loss])
+        r = np.random.default_rng(11)
+        p = [leaves[i].copy() for i in params]
+        for step in range(12):
+            xs = r.standard_normal((64, 784)).astype(np.float32)
+            lab = r.integers(0, 10, 64).astype(np.int32)
+            tape.write(x, xs)
+            tape.write(onehot, np.eye(10, dtype=np.float32)[lab])
+            plan.launch()
+            got_loss = tape.numpy(loss)
+            for leaf_id, n in zip(params, new):
+                tape.assign(leaf_id, n)
+            want_loss, *p, _ = oracle.mlp_step(xs, lab, *p, 0.01)
+            np.testing.assert_allclose(got_loss, [want_loss], rtol=2e-5)
+        for leaf_id, w in zip(params, p):
+            np.testing.assert_allclose(tape.numpy(leaf_id), w, rtol=1e-4, atol=1e-6)
+        assert (tape.matched >= 5) == bool(match)
+        print(f"match={match}: {plan.launches} launches per step")
+    finally:
+        tape.close()

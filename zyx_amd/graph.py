@@ -779,6 +779,7 @@ class Tape:
         self._programs: dict[bytes, int] = {}
         self._keep: list = []
         self._last = None  # event of the most recent launch: launches form one chain
+        self._plans: list = []
 
     def tensor(self, array, dtype: DType) -> int:
         a = np.ascontiguousarray(array, storage_dtype(dtype))
@@ -811,6 +812,53 @@ class Tape:
             if self._last is not None:
                 waits.append(self._last)
             self._last = self.dev.launch(prog, self.pool, [self._buf[i] for i in kern.inputs] + [self._buf[kern.output]], waits)
+
+    def plan(self, nodes: Sequence[int]) -> "TapePlan":
+        """The schedule of `nodes` as one cached plan (a HIP graph): the analogue of the reference's plan cache
+        (zyx/src/graph/plan.rs:58-237). Leaves may be rewritten with `write` between launches; every launch
+        recomputes all the plan's nodes from the leaves' current contents."""
+        if self.match == "time":
+            self.realize(nodes)  # settles which candidate each product runs on; the plan reuses the buffers
+        self.sync()
+        launches = []
+        stored = [n for n in self._buf if self.graph[n].kind == "leaf"]  # everything else is computed by the plan
+        for kern in lower(self.graph, list(nodes), stored=stored, match=bool(self.match)):
+            if isinstance(kern, (Contraction, SoftmaxRows)):
+                kern = self._matched_or_generated(kern)
+            prog = self._programs.get(kern.image)
+            if prog is None:
+                prog = self._programs[kern.image] = self.dev.compile(kern.image)
+            if kern.output not in self._buf:
+                self._alloc(kern.output)
+            launches.append((prog, [self._buf[i] for i in kern.inputs] + [self._buf[kern.output]]))
+        self.sync()
+        return TapePlan(self, self.dev.create_plan(launches), len(launches))
+
+    def write(self, leaf: int, array):
+        """New contents for a leaf (same shape and dtype); later launches read them."""
+        n = self.graph[leaf]
+        a = np.ascontiguousarray(array, storage_dtype(n.dtype))
+        if n.kind != "leaf" or a.shape != n.shape:
+            raise ValueError("write takes a leaf and an array of its shape")
+        self._keep.append(a)
+        waits = [self._ev.pop(leaf)] if leaf in self._ev else []
+        if self._last is not None:  # a running launch may still read the old contents
+            waits.append(self._last)
+            self._last = None
+        self._ev[leaf] = self.pool.host_to_pool(a, self._buf[leaf], waits)
+
+    def assign(self, leaf: int, node: int):
+        """leaf <- node, device to device (`Tensor::assign` of an updated parameter): later launches read the new
+        contents."""
+        a, b = self.graph[leaf], self.graph[node]
+        if a.kind != "leaf" or a.shape != b.shape or a.dtype != b.dtype or node not in self._buf:
+            raise ValueError("assign takes a leaf and a realised node of the same shape and dtype")
+        waits = [self._ev.pop(i) for i in (leaf, node) if i in self._ev]
+        if self._last is not None:
+            waits.append(self._last)
+            self._last = None
+        nbytes = max(_numel(a.shape), 1) * np.dtype(storage_dtype(a.dtype)).itemsize
+        self._ev[leaf] = self.pool.copy_range(self._buf[node], 0, self._buf[leaf], 0, nbytes, waits)
 
     def _matched_or_generated(self, c) -> LoweredKernel:
         from .kernels import gemm_desc, softmax_rows_desc
@@ -861,9 +909,26 @@ class Tape:
 
     def close(self):
         self.sync()
+        for pl in self._plans:
+            self.dev.destroy_plan(pl)
+        self._plans.clear()
         for prog in self._programs.values():
             self.dev.release(prog)
         for buf in self._buf.values():
             self.pool.deallocate(buf, [])
         self._programs.clear()
         self._buf.clear()
+
+
+class TapePlan:
+    """A realised schedule kept as one replayable unit; `launch` runs it after everything the tape has outstanding."""
+
+    def __init__(self, tape: Tape, plan_id: int, launches: int):
+        self.tape, self.id, self.launches = tape, plan_id, launches
+        tape._plans.append(plan_id)
+
+    def launch(self):
+        t = self.tape
+        waits = list(t._ev.values()) + ([t._last] if t._last is not None else [])
+        t._ev.clear()
+        t._last = t.dev.launch_plan(self.id, waits)
