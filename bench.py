@@ -348,9 +348,9 @@ def zyx_dtype_bf16():
 
 def extra_mlp(dev, pool, steps=100, cpu=True):
     """Config 1: MLP 784->128->10, batch 64, SGD 0.01, 100 steps; steps 10..99 timed. GPU: per step two
-    device-to-device batch copies out of the resident dataset and one cached plan launch (9 launch nodes: the weight
-    updates ride in the weight-gradient GEMMs' epilogues, the bias updates and the loss mean in their reduces, the
-    ReLU gradient in the epilogue of the product that feeds it)."""
+    device-to-device batch copies out of the resident dataset and one cached plan launch (8 launch nodes: the weight
+    updates ride in the weight-gradient GEMMs' epilogues, the bias updates in their column sums, the loss mean in the
+    cross-entropy launch, the ReLU gradient in the epilogue of the product that feeds it)."""
     from zyx_amd.training import MLPTrainStep
     B, NIN, H, NOUT, LR = 64, 784, 128, 10, 0.01
     rng = np.random.default_rng(42069)

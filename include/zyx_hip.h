@@ -160,8 +160,9 @@ enum zhip_kernel_kind {
      * (zyx/src/tensor/mod.rs:1639-1655; ln_softmax :1427-1431; one-hot by equal(arange)
      * :1920-1946). flags: ZHIP_CE_LOSS writes the per-sample loss[rows] (ReduceOp::None),
      * ZHIP_CE_GRAD writes d(fparams[0] * sum(loss))/d(logits) = (softmax - onehot) *
-     * fparams[0] into grad[rows, cols] (fparams[0] = 1/rows for the Mean reduction).
-     * args: logits, labels, (loss), (grad). */
+     * fparams[0] into grad[rows, cols] (fparams[0] = 1/rows for the Mean reduction),
+     * ZHIP_CE_MEAN (rows <= 4096) writes mean[1] = sum(loss) / rows (ReduceOp::Mean) from the same launch.
+     * args: logits, labels, (loss), (grad), (mean). */
     ZHIP_K_CROSS_ENTROPY = 6,
     /* Tensor::conv for 4-D NCHW input, groups = 1 (zyx/src/tensor/mod.rs:2583-2680; layer
      * zyx-nn/src/conv2d.rs:60-70): y[N,Cout,OH,OW] = x[N,C,H,W] (*) w[Cout,C,KH,KW] (+ bias[Cout])
@@ -224,6 +225,7 @@ enum zhip_kernel_kind {
 #define ZHIP_NORM_ADD 8
 #define ZHIP_CE_LOSS 1
 #define ZHIP_CE_GRAD 2
+#define ZHIP_CE_MEAN 4
 #define ZHIP_INDEX_GATHER 0
 #define ZHIP_INDEX_SELECT 1
 #define ZHIP_INDEX_SCATTER 2

@@ -111,3 +111,24 @@ def test_norm_backward_bf16_config5_rows(hip, oracle):
     for g, wv, scale in zip(got, want, (1.0, 90.0, 90.0)):   # column sums of 8192 N(0,1) terms are ~90 in size
         gf, wf = oracle.bf16_to_f32(g).astype(np.float64), oracle.bf16_to_f32(wv).astype(np.float64)
         assert np.all(np.abs(gf - wf) <= 2.0 ** -7 * np.abs(wf) + 1e-4 * scale)
+
+
+@pytest.mark.parametrize("shape", [(64, 10), (1, 3), (333, 1000), (4096, 17)])
+def test_cross_entropy_with_batch_mean(hip, oracle, shape):
+    """ZHIP_CE_MEAN: loss, gradient and the batch mean from one launch; rows and gradient equal the plain kernel's
+    bit for bit, the mean is sum(loss) / rows to summation order."""
+    dev, pool = hip
+    r = oracle.Rng(shape[0])
+    x, lab = r.randn(shape, 3.0), r.randint(shape[0], 0, shape[1])
+    loss, grad = cross_entropy(dev, pool, x, lab, 1.0 / shape[0])
+    loss2, grad2, mean = cross_entropy(dev, pool, x, lab, 1.0 / shape[0], mean=True)
+    assert np.array_equal(loss, loss2) and np.array_equal(grad, grad2)
+    np.testing.assert_allclose(mean, [loss.astype(np.float64).mean()], rtol=2e-6)
+
+
+def test_cross_entropy_mean_row_limit(hip):
+    from zyx_amd import BackendError
+    from zyx_amd.kernels import cross_entropy_desc
+    dev, pool = hip
+    with pytest.raises(BackendError):
+        dev.register_kernel(cross_entropy_desc(4097, 10, True, False, 1.0, mean=True))

@@ -202,7 +202,9 @@ struct CrossEntropy {
     const float *x;
     const int32_t *labels;
     float *loss, *grad;
+    float *mean = nullptr; // [1]: sum(loss) / rows, by a single workgroup (rows <= kCrossEntropyMeanRows)
 };
+constexpr int64_t kCrossEntropyMeanRows = 4096;
 hipError_t cross_entropy(const CrossEntropy &p, hipStream_t stream);
 
 } // namespace zk

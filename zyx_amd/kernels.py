@@ -243,7 +243,7 @@ def gemm(dev: HIPDevice, pool: HIPMemoryPool, a: np.ndarray, b: np.ndarray, bias
 # ---- LayerNorm / RMSNorm (ZHIP_K_NORM_ROWS), cross entropy (ZHIP_K_CROSS_ENTROPY) --------------------
 K_NORM_ROWS, K_CROSS_ENTROPY = 5, 6
 NORM_RMS, NORM_WEIGHT, NORM_BIAS = 1, 2, 4
-CE_LOSS, CE_GRAD = 1, 2
+CE_LOSS, CE_GRAD, CE_MEAN = 1, 2, 4
 
 
 def norm_rows_desc(rows: int, cols: int, rms=False, weight=True, bias=True, eps=1e-5, dtype: DType = DType.F32) -> KernelDesc:
@@ -275,21 +275,23 @@ def norm_rows(dev: HIPDevice, pool: HIPMemoryPool, x, w=None, b=None, rms=False,
     return y
 
 
-def cross_entropy_desc(rows: int, cols: int, loss=True, grad=False, gscale: float = 1.0) -> KernelDesc:
+def cross_entropy_desc(rows: int, cols: int, loss=True, grad=False, gscale: float = 1.0, mean=False) -> KernelDesc:
+    """args: logits, labels, (loss[rows]), (grad[rows, cols]), (mean[1])."""
     d = KernelDesc()
     d.kind, d.dtype, d.out_dtype = K_CROSS_ENTROPY, DType.F32, DType.F32
-    d.flags = (CE_LOSS if loss else 0) | (CE_GRAD if grad else 0)
+    d.flags = (CE_LOSS if loss else 0) | (CE_GRAD if grad else 0) | (CE_MEAN if mean else 0)
     d.dims[0], d.dims[1] = rows, cols
     d.fparams[0] = gscale
     return d
 
 
-def cross_entropy(dev: HIPDevice, pool: HIPMemoryPool, logits, labels, grad_scale=None):
-    """-> (per-sample loss, grad or None); grad = d(grad_scale * sum(loss)) / d(logits)."""
+def cross_entropy(dev: HIPDevice, pool: HIPMemoryPool, logits, labels, grad_scale=None, mean=False):
+    """-> (per-sample loss, grad or None); grad = d(grad_scale * sum(loss)) / d(logits). With mean=True a third
+    value, the batch mean from the same launch."""
     x = np.ascontiguousarray(logits, np.float32)
     lab = np.ascontiguousarray(labels, np.int32)
     rows, cols = x.shape
-    prog = dev.register_kernel(cross_entropy_desc(rows, cols, True, grad_scale is not None, grad_scale or 0.0))
+    prog = dev.register_kernel(cross_entropy_desc(rows, cols, True, grad_scale is not None, grad_scale or 0.0, mean))
     xb, e0 = to_device(pool, x)
     lb, e1 = to_device(pool, lab)
     ob, e2 = alloc_like(pool, rows, 4)
@@ -298,13 +300,18 @@ def cross_entropy(dev: HIPDevice, pool: HIPMemoryPool, logits, labels, grad_scal
         gb, e3 = alloc_like(pool, rows * cols, 4)
         outs.append(gb)
         waits.append(e3)
+    if mean:
+        mb, e4 = alloc_like(pool, 1, 4)
+        outs.append(mb)
+        waits.append(e4)
     done = dev.launch(prog, pool, [xb, lb] + outs, waits)
     loss = to_host(pool, ob, (rows,), np.float32, [done])
     grad = to_host(pool, outs[1], (rows, cols), np.float32) if grad_scale is not None else None
+    mean_v = to_host(pool, outs[-1], (1,), np.float32) if mean else None
     for bb in [xb, lb] + outs:
         pool.deallocate(bb, [])
     dev.release(prog)
-    return loss, grad
+    return (loss, grad, mean_v) if mean else (loss, grad)
 
 
 # ---- conv2d / max_pool2d (ZHIP_K_CONV2D, ZHIP_K_MAX_POOL2D) ---------------------------------------------

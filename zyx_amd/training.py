@@ -76,9 +76,10 @@ class MLPTrainStep:
         nodes = [
             (prog(K.gemm_desc(batch, hidden, n_in, f32, f32, trans_b=True, epilogue="bias_relu")), [x, w1, b1, h]),
             (prog(K.gemm_desc(batch, n_out, hidden, f32, f32, trans_b=True, epilogue="bias")), [h, w2, b2, logits]),
-            (prog(K.cross_entropy_desc(batch, n_out, True, True, 1.0 / batch)), [logits, y, loss, dlogits]),
-        ] + ([(prog(K.reduce_desc(1, batch, "sum", div=float(batch))), [loss, mean_loss])] if fused_update else
-             [(prog(K.reduce_desc(1, batch, "sum")), [loss, loss_sum]), (prog(scale.desc()), [loss_sum, mean_loss])]) + [
+        ] + ([(prog(K.cross_entropy_desc(batch, n_out, True, True, 1.0 / batch, mean=True)), [logits, y, loss, dlogits, mean_loss])]
+             if fused_update and batch <= 4096 else
+             [(prog(K.cross_entropy_desc(batch, n_out, True, True, 1.0 / batch)), [logits, y, loss, dlogits]),
+              (prog(K.reduce_desc(1, batch, "sum")), [loss, loss_sum]), (prog(scale.desc()), [loss_sum, mean_loss])]) + [
             dw2_node,
             # bias gradients are column sums; the fused form stores b - lr * sum straight into the new bias
             (prog(K.reduce_desc(batch, n_out, "sum", axis0=True, mul=-lr, base=True)), [dlogits, b2, nb2]) if fused_update else
