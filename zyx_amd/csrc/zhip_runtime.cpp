@@ -78,6 +78,7 @@ struct Program {
     // A program's workspace is shared by all its launches: each launch waits for the previous one's event on
     // whatever stream that ran, so two launches with unrelated wait lists never overlap on the scratch memory.
     hipEvent_t ws_event = nullptr;
+    int ws_last = 0;           // where the scratch was last used: 0 nowhere yet, 1 a launch (ws_event), 2 a plan (the context's plan_done)
     int plan_refs = 0;         // live plans whose graphs hold this program's kernels, workspace and code
 };
 
@@ -134,6 +135,7 @@ struct zhip_ctx {
     Slab<Program> programs;
     Slab<Plan> plans;
     hipStream_t plan_stream = nullptr; // plans are captured on and replayed into this stream
+    hipEvent_t plan_done = nullptr;    // recorded after every plan launch that uses program scratch: one record for all of them
     hipEvent_t prof_a = nullptr, prof_b = nullptr;
 
     int32_t fail(int32_t status, const char *fmt, ...) __attribute__((format(printf, 3, 4))) {
@@ -979,7 +981,8 @@ ZHIP_EXPORT int32_t zhip_init(const zhip_config *cfg, zhip_ctx **out) {
             return bail(ZHIP_INITIALIZATION, "hipStreamCreate", e);
     if ((e = hipStreamCreateWithFlags(&c->plan_stream, hipStreamNonBlocking)) != hipSuccess)
         return bail(ZHIP_INITIALIZATION, "hipStreamCreate", e);
-    if ((e = hipEventCreate(&c->prof_a)) != hipSuccess || (e = hipEventCreate(&c->prof_b)) != hipSuccess)
+    if ((e = hipEventCreate(&c->prof_a)) != hipSuccess || (e = hipEventCreate(&c->prof_b)) != hipSuccess ||
+        (e = hipEventCreateWithFlags(&c->plan_done, hipEventDisableTiming)) != hipSuccess)
         return bail(ZHIP_INITIALIZATION, "hipEventCreate", e);
     if ((e = zk::gemm_bf16_init()) != hipSuccess) return bail(ZHIP_INITIALIZATION, "raising the LDS limit of the GEMM kernels", e);
     fill_info(c);
@@ -1016,6 +1019,7 @@ ZHIP_EXPORT int32_t zhip_deinit(zhip_ctx *c) {
         for (EventSlot &s : c->events) (void)hipEventDestroy(s.ev);
         (void)hipEventDestroy(c->prof_a);
         (void)hipEventDestroy(c->prof_b);
+        if (c->plan_done) (void)hipEventDestroy(c->plan_done);
         (void)hipStreamDestroy(c->pool_stream);
         for (auto s : c->launch_streams) (void)hipStreamDestroy(s);
     }
@@ -1371,10 +1375,14 @@ ZHIP_EXPORT int32_t zhip_launch(zhip_ctx *c, zhip_prog prog, const zhip_buf *arg
     rc = wait_and_consume(c, si, evs, n_evs, ZHIP_KERNEL_LAUNCH);
     if (rc != ZHIP_OK) return rc;
     if (c->debug & 32) fprintf(stderr, "[zyx-hip] launch program %u (kind %d) on stream %d\n", prog, p->desc.kind, si);
-    if (p->ws_event) HIPCHK(c, hipStreamWaitEvent(c->launch_streams[si], p->ws_event, 0), ZHIP_KERNEL_LAUNCH);
+    if (p->ws_event && p->ws_last)
+        HIPCHK(c, hipStreamWaitEvent(c->launch_streams[si], p->ws_last == 2 ? c->plan_done : p->ws_event, 0), ZHIP_KERNEL_LAUNCH);
     hipError_t e = program_enqueue(*p, ptr, c->launch_streams[si]);
     if (e != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "launch of program %u failed: %s", prog, hipGetErrorString(e));
-    if (p->ws_event) HIPCHK(c, hipEventRecord(p->ws_event, c->launch_streams[si]), ZHIP_KERNEL_LAUNCH);
+    if (p->ws_event) {
+        HIPCHK(c, hipEventRecord(p->ws_event, c->launch_streams[si]), ZHIP_KERNEL_LAUNCH);
+        p->ws_last = 1;
+    }
     return event_record(c, si, ZHIP_KERNEL_LAUNCH, ev);
 }
 
@@ -1387,7 +1395,7 @@ ZHIP_EXPORT int32_t zhip_time_kernel(zhip_ctx *c, zhip_prog prog, const zhip_buf
     if (rc != ZHIP_OK) return rc;
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
     hipStream_t st = c->launch_streams[0];
-    if (p->ws_event) HIPCHK(c, hipEventSynchronize(p->ws_event), ZHIP_KERNEL_SYNC);
+    if (p->ws_event && p->ws_last) HIPCHK(c, hipEventSynchronize(p->ws_last == 2 ? c->plan_done : p->ws_event), ZHIP_KERNEL_SYNC);
     HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
     auto t0 = std::chrono::steady_clock::now();
     hipError_t e = program_enqueue(*p, ptr, st);
@@ -1410,7 +1418,7 @@ ZHIP_EXPORT int32_t zhip_profile_kernel(zhip_ctx *c, zhip_prog prog, const zhip_
     }
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
     hipStream_t st = c->launch_streams[0];
-    if (p->ws_event) HIPCHK(c, hipEventSynchronize(p->ws_event), ZHIP_KERNEL_SYNC);
+    if (p->ws_event && p->ws_last) HIPCHK(c, hipEventSynchronize(p->ws_last == 2 ? c->plan_done : p->ws_event), ZHIP_KERNEL_SYNC);
     HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
     HIPCHK(c, hipEventRecord(c->prof_a, st), ZHIP_KERNEL_LAUNCH);
     for (int32_t i = 0; i < iters; i++) {
@@ -1478,11 +1486,21 @@ ZHIP_EXPORT int32_t zhip_plan_launch(zhip_ctx *c, zhip_plan plan, const zhip_eve
     int32_t rc = wait_and_consume(c, -2, evs, n_evs, ZHIP_KERNEL_LAUNCH);
     if (rc != ZHIP_OK) return rc;
     Plan &pl = c->plans.items[plan];
-    for (zhip_prog q : pl.progs)
-        if (hipEvent_t we = c->programs.items[q].ws_event) HIPCHK(c, hipStreamWaitEvent(c->plan_stream, we, 0), ZHIP_KERNEL_LAUNCH);
+    // Program scratch: a program last used by a single launch on another stream is waited for; one last used by a
+    // plan needs nothing (plans replay in order on one stream). Afterwards one event covers every program of the plan.
+    bool any_ws = false;
+    for (zhip_prog q : pl.progs) {
+        Program &pr = c->programs.items[q];
+        if (!pr.ws_event) continue;
+        any_ws = true;
+        if (pr.ws_last == 1) HIPCHK(c, hipStreamWaitEvent(c->plan_stream, pr.ws_event, 0), ZHIP_KERNEL_LAUNCH);
+    }
     HIPCHK(c, hipGraphLaunch(pl.exec, c->plan_stream), ZHIP_KERNEL_LAUNCH);
-    for (zhip_prog q : pl.progs)
-        if (hipEvent_t we = c->programs.items[q].ws_event) HIPCHK(c, hipEventRecord(we, c->plan_stream), ZHIP_KERNEL_LAUNCH);
+    if (any_ws) {
+        HIPCHK(c, hipEventRecord(c->plan_done, c->plan_stream), ZHIP_KERNEL_LAUNCH);
+        for (zhip_prog q : pl.progs)
+            if (c->programs.items[q].ws_event) c->programs.items[q].ws_last = 2;
+    }
     return event_record(c, -2, ZHIP_KERNEL_LAUNCH, ev);
 }
 
