@@ -59,6 +59,12 @@ struct EventSlot {
     int16_t stream = -1; // launch stream index, -1 = pool stream
     uint64_t seq = 0;    // position in that stream's record order
     bool live = false;
+    // An event handle first only names a position in its stream. The hipEvent is recorded when somebody has to wait
+    // for it from another stream or from the host -- at the stream's end as it is then, which is at or after the
+    // position and so waits for nothing less. Work chained on one stream (the common case: streams run in order and
+    // a same-stream wait is skipped) never pays for a record. No wait cycle can arise: whatever was enqueued between
+    // the position and the record only waits for events that existed before it, hence before the new waiter.
+    bool recorded = false;
 };
 
 struct CachedBlock {
@@ -192,16 +198,19 @@ int32_t event_record(zhip_ctx *c, int stream_idx, int32_t status, zhip_event *ou
         idx = (uint32_t)c->events.size() - 1;
     }
     EventSlot &s = c->events[idx];
-    hipError_t e = hipEventRecord(s.ev, stream_of(c, stream_idx));
-    if (e != hipSuccess) {
-        c->free_events.push_back(idx);
-        return c->fail(status, "hipEventRecord failed: %s", hipGetErrorString(e));
-    }
     s.live = true;
+    s.recorded = false;
     s.stream = (int16_t)stream_idx;
     s.seq = ++c->stream_seq[stream_idx == -1 ? kLaunchStreams : stream_idx == -2 ? kLaunchStreams + 1 : stream_idx];
     *out = ((uint64_t)s.gen << 32) | (uint64_t)(idx + 1);
     return ZHIP_OK;
+}
+// Records the event if nobody needed it so far (see EventSlot::recorded).
+hipError_t event_materialise(zhip_ctx *c, EventSlot *s) {
+    if (s->recorded) return hipSuccess;
+    hipError_t e = hipEventRecord(s->ev, stream_of(c, s->stream));
+    if (e == hipSuccess) s->recorded = true;
+    return e;
 }
 void event_retire(zhip_ctx *c, EventSlot *s) {
     s->live = false;
@@ -230,7 +239,8 @@ int32_t wait_and_consume(zhip_ctx *c, int stream_idx, const zhip_event *evs, siz
     }
     for (EventSlot *s : latest)
         if (s) {
-            hipError_t e = hipStreamWaitEvent(stream_of(c, stream_idx), s->ev, 0);
+            hipError_t e = event_materialise(c, s);
+            if (e == hipSuccess) e = hipStreamWaitEvent(stream_of(c, stream_idx), s->ev, 0);
             if (e != hipSuccess) rc = c->fail(status, "hipStreamWaitEvent failed: %s", hipGetErrorString(e));
         }
     for (size_t i = 0; i < n; i++)
@@ -257,7 +267,7 @@ void trim_cache(zhip_ctx *c, uint64_t limit) {
         if (it->second.empty()) c->cache.erase(it);
         for (zhip_event h : blk.pending)
             if (EventSlot *s = event_lookup(c, h)) {
-                (void)hipEventSynchronize(s->ev);
+                if (event_materialise(c, s) == hipSuccess) (void)hipEventSynchronize(s->ev);
                 event_retire(c, s);
             }
         (void)hipFree(blk.ptr);
@@ -1204,7 +1214,8 @@ ZHIP_EXPORT int32_t zhip_sync_events(zhip_ctx *c, const zhip_event *evs, size_t 
             rc = c->fail(ZHIP_KERNEL_SYNC, "event %zu is not live (stale or already consumed handle)", i);
             continue;
         }
-        hipError_t e = hipEventSynchronize(s->ev);
+        hipError_t e = event_materialise(c, s);
+        if (e == hipSuccess) e = hipEventSynchronize(s->ev);
         if (e != hipSuccess) rc = c->fail(ZHIP_KERNEL_SYNC, "hipEventSynchronize failed: %s", hipGetErrorString(e));
         event_retire(c, s);
     }
@@ -1501,7 +1512,13 @@ ZHIP_EXPORT int32_t zhip_plan_launch(zhip_ctx *c, zhip_plan plan, const zhip_eve
         for (zhip_prog q : pl.progs)
             if (c->programs.items[q].ws_event) c->programs.items[q].ws_last = 2;
     }
-    return event_record(c, -2, ZHIP_KERNEL_LAUNCH, ev);
+    // A plan is a coarse unit whose end other streams typically wait for while the next plan is already queued (batch
+    // copies of a training loop): its event is recorded right here, so that such a wait covers this plan only.
+    int32_t rc2 = event_record(c, -2, ZHIP_KERNEL_LAUNCH, ev);
+    if (rc2 == ZHIP_OK)
+        if (EventSlot *s = event_lookup(c, *ev))
+            if (event_materialise(c, s) != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "hipEventRecord failed");
+    return rc2;
 }
 
 ZHIP_EXPORT int32_t zhip_plan_destroy(zhip_ctx *c, zhip_plan plan) {
