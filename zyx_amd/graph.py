@@ -25,7 +25,6 @@ from .ir import BOp, Kernel, MemScope, ParamKind, UOp
 
 _BOOL_OPS = (BOp.Cmplt, BOp.Cmpgt, BOp.Cmpge, BOp.NotEq, BOp.Eq, BOp.Or, BOp.And)
 _NO_GRAD_BOPS = _BOOL_OPS + (BOp.BitXor, BOp.BitOr, BOp.BitAnd, BOp.BitShiftLeft, BOp.BitShiftRight)
-_FLOATS = (DType.BF16, DType.F16, DType.F32, DType.F64)
 _NP = {DType.BF16: np.uint16, DType.F16: np.float16, DType.F32: np.float32, DType.F64: np.float64, DType.U8: np.uint8,
        DType.U16: np.uint16, DType.U32: np.uint32, DType.U64: np.uint64, DType.I8: np.int8, DType.I16: np.int16,
        DType.I32: np.int32, DType.I64: np.int64, DType.Bool: np.uint8}
