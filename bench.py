@@ -299,13 +299,17 @@ def extra_block(dev, pool, steps=20, warmup=5, cpu=True):
     """Config 5: pre-norm transformer block B=8 T=1024 d=1024 16 heads, bf16, forward and forward + backward, each
     one cached plan launch (8 and 24 kernels). FLOPs counted: the matrix products only (240.5 GFLOP forward)."""
     import zyx_amd
-    import oracle
     from zyx_amd.block import TransformerBlock
     B, T, D, H = 8, 1024, 1024, 16
     fwd_flop = 2.0 * B * T * (3 * D * D + D * D + 8 * D * D) + 4.0 * B * H * T * T * (D // H)
     blk = TransformerBlock(dev, pool, B, T, D, H, zyx_amd.DType.BF16)
     trunc = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
-    params = oracle.block_init(D, H)
+    # config 5's parameters: Linear weights 0.02 * randn and zero biases (nanogpt.rs:121-125), LayerNorm weight 1 / bias 0
+    prng = np.random.default_rng(42069)
+    w = lambda *shape: (0.02 * prng.standard_normal(shape)).astype(np.float32)
+    z = lambda n: np.zeros(n, np.float32)
+    params = dict(ln1_w=np.ones(D, np.float32), ln1_b=z(D), attn_w=w(3 * D, D), attn_b=z(3 * D), proj_w=w(D, D), proj_b=z(D),
+                  ln2_w=np.ones(D, np.float32), ln2_b=z(D), fc_w=w(4 * D, D), fc_b=z(4 * D), proj2_w=w(D, 4 * D), proj2_b=z(D))
     blk.set_params({k: trunc(v) for k, v in params.items()})
     rng = np.random.default_rng(5)
     x = rng.standard_normal((B * T, D), dtype=np.float32)
@@ -325,6 +329,7 @@ def extra_block(dev, pool, steps=20, warmup=5, cpu=True):
         res[name] = {"ms": round(ms, 3), "TFLOP/s": round(flop / ms / 1e9, 1), "frac_of_2.5PF_bf16_peak": round(flop / ms / 1e9 / 2500.0, 4)}
     blk.close()
     if cpu:
+        import oracle  # the CPU comparison leg only
         # one attention head pair and 64 rows of each Linear on the host cores, scaled to the whole forward
         sub = trunc(rng.standard_normal((1, T, 3 * 128), dtype=np.float32))
         t0 = time.perf_counter()
