@@ -314,3 +314,23 @@ def test_training_steps_as_a_cached_plan(hip, oracle, match):
         print(f"match={match}: {plan.launches} launches per step")
     finally:
         tape.close()
+
+
+def test_long_reductions_run_on_the_reduce_kernel(hip):
+    """Row sums, a maximum over the trailing axes and an integer column sum of tensors with buffers are launched as
+    the two-stage reduce kernel; integers and maxima exact, float sums to 1e-5 of sum |x|."""
+    def build(g, leaf):
+        r = np.random.default_rng(8)
+        x = leaf(r.standard_normal((64, 16, 4096)), DType.F32)
+        y = leaf(r.integers(-100, 100, (5000, 33)), DType.I32)
+        return (g.reduce(x, BOp.Add, [2]), g.reduce(x, BOp.Max, [1, 2]), g.reduce(y, BOp.Add, [0])), (x, y)
+
+    tape, leaves, ((rs, mx, cs), (x, y)) = matched_tape(hip, build)
+    try:
+        tape.realize([rs, mx, cs])
+        assert tape.matched == 3
+        xv = leaves[x].astype(np.float64)
+        np.testing.assert_allclose(tape.numpy(rs), xv.sum(2), rtol=0, atol=1e-5 * np.abs(xv).sum(2).max())
+        assert np.array_equal(tape.numpy(mx), leaves[x].max((1, 2))) and np.array_equal(tape.numpy(cs), leaves[y].sum(0, dtype=np.int32))
+    finally:
+        tape.close()

@@ -7,7 +7,7 @@ import pytest
 from graph_cases import CASES, mixed_graph, mlp_graph
 from oracle import graph_eval, ir_interp
 from zyx_amd import DType
-from zyx_amd.graph import Contraction, Graph, SoftmaxRows, lower, match_softmax, match_contraction, storage_dtype, view_of
+from zyx_amd.graph import Contraction, Graph, RowColReduce, SoftmaxRows, lower, match_reduce, match_softmax, match_contraction, storage_dtype, view_of
 from zyx_amd.ir import BOp, UOp
 
 _FLOAT = (DType.F32, DType.F64)
@@ -37,6 +37,13 @@ def run_lowered(g, leaves, outputs, match=False, seen=None):
             A = A.transpose(0, 2, 1) if kern.trans_a else A
             B = B.transpose(0, 2, 1) if kern.trans_b else B
             bufs[kern.out] = np.matmul(A.astype(np.float64), B.astype(np.float64)).astype(A.dtype).reshape(-1)
+            if seen is not None:
+                seen.append(kern)
+            continue
+        if isinstance(kern, RowColReduce):
+            x = bufs[kern.x].reshape(kern.rows, kern.cols)
+            f = np.sum if kern.op == "sum" else np.max
+            bufs[kern.out] = f(x.astype(np.float64) if x.dtype.kind == "f" else x, axis=0 if kern.axis0 else 1).astype(x.dtype).reshape(-1)
             if seen is not None:
                 seen.append(kern)
             continue
@@ -350,3 +357,31 @@ def test_softmax_match():
     got = run_lowered(g, leaves, [sm], match=True, seen=seen)
     assert len(seen) == 1
     np.testing.assert_allclose(got[sm], run_lowered(g, leaves, [sm])[sm], rtol=1e-6)
+
+
+def test_reduce_match():
+    """Long reductions over the trailing or the leading axes of a tensor that has a buffer go to the reduce kernel;
+    short ones, middle axes and operands that are expressions stay generated (fused)."""
+    g = Graph()
+    x = g.leaf((6, 4, 512), DType.F32)
+    m = match_reduce(g, g.reduce(x, BOp.Add, [2]), set())
+    assert (m.x, m.rows, m.cols, m.axis0, m.op) == (x, 24, 512, False, "sum")
+    m = match_reduce(g, g.reduce(x, BOp.Max, [1, 2]), set())
+    assert (m.rows, m.cols, m.axis0, m.op) == (6, 2048, False, "max")
+    y = g.leaf((300, 7, 3), DType.I32)
+    m = match_reduce(g, g.reduce(g.reshape(y, [300, 21]), BOp.Add, [0]), set())
+    assert (m.x, m.rows, m.cols, m.axis0) == (y, 300, 21, True)
+    assert match_reduce(g, g.reduce(x, BOp.Add, [1]), set()) is None                      # a middle axis
+    assert match_reduce(g, g.reduce(x, BOp.Add, [0]), set()) is None                      # 6 elements per result
+    e = g.unary(x, UOp.Exp)
+    assert match_reduce(g, g.reduce(e, BOp.Add, [2]), set()) is None                      # an expression: stays fused
+    assert match_reduce(g, g.reduce(e, BOp.Add, [2]), {e}) is not None                    # unless it has a buffer anyway
+    assert match_reduce(g, g.reduce(g.permute(x, [1, 0, 2]), BOp.Add, [2]), set()) is None
+    leaves = {x: np.random.default_rng(1).standard_normal((6, 4, 512)).astype(np.float32),
+              y: np.random.default_rng(2).integers(-9, 9, (300, 7, 3)).astype(np.int32)}
+    outs = [g.reduce(x, BOp.Add, [2]), g.reduce(x, BOp.Max, [1, 2]), g.reduce(g.reshape(y, [300, 21]), BOp.Add, [0])]
+    seen = []
+    got, want = run_lowered(g, leaves, outs, match=True, seen=seen), run_lowered(g, leaves, outs)
+    assert len(seen) == 3
+    np.testing.assert_allclose(got[outs[0]], want[outs[0]], rtol=1e-5, atol=1e-5)
+    assert np.array_equal(got[outs[1]], want[outs[1]]) and np.array_equal(got[outs[2]], want[outs[2]])

@@ -540,6 +540,43 @@ def match_softmax(graph: Graph, nid: int):
     return SoftmaxRows(base, nid, _numel(n.shape[:-1]), n.shape[-1])
 
 
+@dataclasses.dataclass
+class RowColReduce:
+    """`out = reduce(x)` over the last axis (x seen as [rows, cols] -> [rows]) or over the leading axis (-> [cols]) of a
+    tensor that already has a buffer: the shapes the two-stage reduce kernel takes."""
+    x: int
+    out: int
+    rows: int
+    cols: int
+    axis0: bool
+    op: str
+    dtype: DType
+
+
+def match_reduce(graph: Graph, nid: int, stored) -> RowColReduce | None:
+    """A Reduce(Add | Max) whose operand is a plain view of a whole buffer that exists already (a leaf or a node in
+    `stored`: an operand that is an expression stays fused into the generated reduce), reduced over its trailing axes
+    or over its leading axes, with enough elements per result for the tree-shaped kernel to pay."""
+    r = graph[nid]
+    if r.kind != "reduce" or r.dtype not in (DType.F32, DType.BF16, DType.F16, DType.I32):
+        return None
+    x = r.src[0]
+    xs = graph[x].shape
+    base, st = view_of(graph, x)
+    if st != _contiguous(xs) or _numel(graph[base].shape) != _numel(xs) or not (graph[base].kind == "leaf" or base in stored):
+        return None
+    k, n = len(r.arg), len(xs)
+    if r.arg == tuple(range(n - k, n)):
+        rows, cols, axis0 = _numel(xs[:n - k]), _numel(xs[n - k:]), False
+    elif r.arg == tuple(range(k)):
+        rows, cols, axis0 = _numel(xs[:k]), _numel(xs[k:]), True
+    else:
+        return None
+    if (rows if axis0 else cols) < 256:
+        return None  # short reductions: one serial loop per result is as good and needs no second launch
+    return RowColReduce(base, nid, rows, cols, axis0, "sum" if r.op == BOp.Add else "max", r.dtype)
+
+
 # ---- lowering ---------------------------------------------------------------------------------------------------------
 
 @dataclasses.dataclass
@@ -731,7 +768,7 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
         n = graph[nid]
         if n.kind == "leaf" or nid in have:
             return
-        c = (match_contraction(graph, nid) or match_softmax(graph, nid)) if match else None
+        c = (match_contraction(graph, nid) or match_softmax(graph, nid) or match_reduce(graph, nid, have)) if match else None
         if c is not None:
             for s in ((c.a, c.b) if isinstance(c, Contraction) else (c.x,)):
                 need(s, True)
@@ -798,7 +835,7 @@ class Tape:
 
     def realize(self, nodes: Sequence[int]):
         for kern in lower(self.graph, [n for n in nodes if n not in self._buf], stored=list(self._buf), match=self.match):
-            if isinstance(kern, (Contraction, SoftmaxRows)):
+            if isinstance(kern, (Contraction, SoftmaxRows, RowColReduce)):
                 kern = self._matched_or_generated(kern)
             prog = self._programs.get(kern.image)
             if prog is None:
@@ -822,7 +859,7 @@ class Tape:
         launches = []
         stored = [n for n in self._buf if self.graph[n].kind == "leaf"]  # everything else is computed by the plan
         for kern in lower(self.graph, list(nodes), stored=stored, match=bool(self.match)):
-            if isinstance(kern, (Contraction, SoftmaxRows)):
+            if isinstance(kern, (Contraction, SoftmaxRows, RowColReduce)):
                 kern = self._matched_or_generated(kern)
             prog = self._programs.get(kern.image)
             if prog is None:
@@ -860,10 +897,13 @@ class Tape:
         self._ev[leaf] = self.pool.copy_range(self._buf[node], 0, self._buf[leaf], 0, nbytes, waits)
 
     def _matched_or_generated(self, c) -> LoweredKernel:
-        from .kernels import gemm_desc, softmax_rows_desc
+        from .kernels import gemm_desc, reduce_desc, softmax_rows_desc
         if isinstance(c, Contraction):
             desc = gemm_desc(c.m, c.n, c.k, c.dtype, c.dtype, c.trans_a, c.trans_b, batch=c.batch)
             inputs, elements = [c.a, c.b], c.batch * c.m * c.n
+        elif isinstance(c, RowColReduce):
+            desc = reduce_desc(c.rows, c.cols, c.op, c.axis0, c.dtype)
+            inputs, elements = [c.x], c.cols if c.axis0 else c.rows
         else:
             desc = softmax_rows_desc(c.rows, c.cols, y=True, rowsum=False, argmax=False)
             inputs, elements = [c.x], c.rows * c.cols
