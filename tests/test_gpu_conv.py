@@ -185,3 +185,32 @@ def test_max_pool_2x2_fast_path(hip, oracle, shape):
     assert np.array_equal(got, want) and got[0, 0, 0, 2] == np.float32(-3.4028234663852886e38)
     xb = oracle.f32_to_bf16(x)
     assert np.array_equal(max_pool2d(dev, pool, xb, *args, dtype=DType.BF16), oracle.max_pool2d(xb, *args, dtype=oracle.BF16))
+
+
+@pytest.mark.parametrize("shape", [(2, 16, 16, 56, 128), (1, 64, 56, 56, 128), (3, 32, 28, 16, 256), (2, 48, 8, 112, 128), (1, 16, 56, 8, 128)])
+@pytest.mark.parametrize("bias,relu", [(True, True), (False, False)])
+def test_conv3x3_direct_bf16(hip, oracle, shape, bias, relu):
+    """3 x 3 / stride 1 / padding 1 bf16 shapes whose rows tile into 448-pixel blocks take the direct kernel (input
+    tile in LDS, nine shifted views, no patch matrix): against the oracle, bf16 and f32 results, first / last rows and
+    columns (the zero border) included; the f32 result is also checked against the f64 convolution."""
+    dev, pool = hip
+    n, c, h, w, co = shape
+    r = oracle.Rng(n * 1000 + c + w)
+    x, wt = oracle.f32_to_bf16(r.randn((n, c, h, w))), oracle.f32_to_bf16(r.randn((co, c, 3, 3), 0.1))
+    b = oracle.f32_to_bf16(r.randn(co, 0.1)) if bias else None
+    mag = oracle.conv2d(np.abs(oracle.bf16_to_f32(x)), np.abs(oracle.bf16_to_f32(wt)), None if b is None else np.abs(oracle.bf16_to_f32(b)), (1, 1), (1, 1))
+    got32 = conv2d(dev, pool, x, wt, b, (1, 1), (1, 1), (1, 1), relu=relu, dtype=DType.BF16, out_dtype=DType.F32)
+    want32 = oracle.conv2d(x, wt, b, (1, 1), (1, 1), (1, 1), relu, oracle.BF16, oracle.F32)
+    assert np.all(np.abs(got32 - want32) <= 1e-3 * np.abs(want32) + 2e-5 * mag)
+    got = conv2d(dev, pool, x, wt, b, (1, 1), (1, 1), (1, 1), relu=relu, dtype=DType.BF16)
+    want = oracle.conv2d(x, wt, b, (1, 1), (1, 1), (1, 1), relu, oracle.BF16)
+    g, wv = oracle.bf16_to_f32(got), oracle.bf16_to_f32(want)
+    assert np.all(np.abs(g - wv) <= 2.0 ** -7 * np.abs(wv) + 1e-3 * mag)
+    # borders: a ones image with ones weights counts the taps inside the image
+    ones_x, ones_w = oracle.f32_to_bf16(np.ones((1, c, h, w), np.float32)), oracle.f32_to_bf16(np.ones((co, c, 3, 3), np.float32))
+    cnt = conv2d(dev, pool, ones_x, ones_w, None, (1, 1), (1, 1), (1, 1), dtype=DType.BF16, out_dtype=DType.F32)
+    taps = np.full((h, w), 9.0)
+    taps[0, :] = taps[-1, :] = 6
+    taps[:, 0] = taps[:, -1] = 6
+    taps[0, 0] = taps[0, -1] = taps[-1, 0] = taps[-1, -1] = 4
+    assert np.array_equal(cnt[0, 0], taps * c) and np.array_equal(cnt[0, -1], taps * c)

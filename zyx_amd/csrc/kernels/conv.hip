@@ -327,6 +327,7 @@ bool conv_gathers_in_gemm(const Conv2d &p) {
 
 // scratch = [zero bias (for ReLU without bias)] [patch matrix K x pixels bf16]
 uint64_t conv2d_scratch_bytes(const Conv2d &p) {
+    if (conv3x3_direct_ok(p)) return kZeroBiasBytes + conv3x3_scratch_bytes(p); // the direct kernel: re-laid weights only
     if (!conv_uses_gemm(p) || p.Cout > 4096) return 0;
     if (conv_gathers_in_gemm(p)) // padded input (+ 16 bytes: the last 128-bit load may start 7 elements before the end)
         return kZeroBiasBytes + (uint64_t)p.N * p.C * (p.H + 2 * p.py) * (p.W + 2 * p.px) * 2 + 16;
@@ -336,6 +337,7 @@ uint64_t conv2d_scratch_bytes(const Conv2d &p) {
 hipError_t conv2d(const Conv2d &p, hipStream_t st) {
     const int64_t P = (int64_t)p.N * p.OH * p.OW;
     if (P <= 0 || p.Cout <= 0) return hipSuccess;
+    if (p.scratch && conv3x3_direct_ok(p)) return conv3x3_direct(p, (char *)p.scratch + kZeroBiasBytes, st);
     if (p.scratch && conv2d_scratch_bytes(p)) {
         // im2col (transposed) + GEMM: C[pixel, co] = sum_k a[k, pixel] * w[co, k], stored as NCHW by the epilogue
         uint16_t *a = (uint16_t *)((char *)p.scratch + kZeroBiasBytes);

@@ -1,0 +1,270 @@
+// Direct 3 x 3 convolution, bf16, unit stride, padding 1 (the convolution block of a vision network:
+// Tensor::conv, zyx/src/tensor/mod.rs:2583-2680, padding rule zyx/src/kernel/linearize.rs:349-382), on the matrix
+// cores without a patch matrix, a padded copy of the input, or a second pass over it.
+//
+// A workgroup owns R whole output rows of one image (R * W = 448 pixels = 14 MFMA blocks of 32) and 128 output
+// channels. It copies the R + 2 input rows of all C channels into LDS once, channel-innermost ([row][col][C], borders
+// zero), so that the nine taps are nine shifted views of the same tile: the B operand of tap (ky, kx) and channel
+// block cb for pixel (r, c) is the 16 bytes at [r + ky][c + kx][cb*16 + half*8], one ds_read_b128, whatever the shift
+// (the pixel stride is padded by 16 bytes, which spreads the 16 lanes of a read phase over all 64 banks). Every input
+// element is fetched once and used 9 * 128 times. The weights are re-laid once per launch by a small kernel as
+// [tap][C/16][Cout][16], so the A operand (32 output channels x 16 input channels of one tap) is 1 KiB of consecutive
+// bytes read straight from L1 / L2, one k step ahead of its use.
+//
+// The product is formed transposed, acc[cout][pixel] = W . X^T, so that a lane owns a pixel column and the 32 lanes of
+// a store cover 32 consecutive pixels of one output channel: NCHW rows are written in 64-byte (bf16) or 128-byte (f32)
+// runs. 4 waves as 2 (pixel halves) x 2 (channel halves), 2 x 7 accumulator tiles of 32 x 32 each = 224 registers.
+#include <algorithm>
+
+#include "dtypes.hpp"
+#include "kernels.hpp"
+
+namespace zk {
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+#define ZK_LDS __attribute__((address_space(3)))
+
+constexpr int PB = 7;                 // 32-pixel blocks per wave
+constexpr int TILE_PIX = 2 * PB * 32; // 448 pixels per workgroup
+constexpr int TILE_CO = 128;          // output channels per workgroup
+
+// w[Cout][C][3][3] -> wt[tap][C/16][Cout][16]. One thread per (cout, cin): the nine taps of a pair are 18 consecutive
+// bytes, and the 16 threads of a channel block write 32 consecutive bytes of each tap's slice.
+__global__ __launch_bounds__(256) void conv3x3_weights_k(const uint16_t *__restrict__ w, uint16_t *__restrict__ wt, int C, int Cout) {
+    const int i = blockIdx.x * 256 + threadIdx.x; // = co * C + c
+    if (i >= C * Cout) return;
+    const int co = i / C, c = i - co * C, cb = c >> 4, ci = c & 15;
+    uint16_t v[9];
+#pragma unroll
+    for (int t = 0; t < 9; t++) v[t] = w[(int64_t)i * 9 + t];
+#pragma unroll
+    for (int t = 0; t < 9; t++) wt[(((int64_t)t * (C >> 4) + cb) * Cout + co) * 16 + ci] = v[t];
+}
+
+// floor(q / d) for 0 <= q < 2^22, inv = 1.0f / d: the rounding errors of the reciprocal and of the product are far
+// smaller than the distance 0.5 / d of (q + 0.5) / d from the nearest integer
+__device__ __forceinline__ int small_div(int q, float inv) { return (int)(((float)q + 0.5f) * inv); }
+
+template <bool OUT_BF16, bool RELU>
+__global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restrict__ x, const uint16_t *__restrict__ wt,
+                                                         const uint16_t *__restrict__ bias, void *__restrict__ y, int C, int H,
+                                                         int W, int Cout, int R) {
+    // A workgroup is alone on its compute unit, one wave per SIMD: nothing hides instruction issue outside the matrix
+    // loop, so every phase below is written for a small instruction count (no integer division, no per-element branch).
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
+    ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int tiles_per_image = H / R;
+    const int n = blockIdx.x / tiles_per_image, rb = blockIdx.x - n * tiles_per_image;
+    const int co0 = blockIdx.y * TILE_CO;
+    const int PS = C * 2 + 16;            // bytes between neighbouring pixels in LDS
+    const int Wp = W + 2, w8 = W >> 3;
+
+    // ---- input tile: rows rb*R - 1 .. rb*R + R of every channel, channel-innermost, zero outside the image ----------
+    // One item = 8 consecutive columns of two neighbouring channels of one row: two 16-byte reads, eight 4-byte LDS
+    // writes (channel pair packed). Consecutive lanes take consecutive channel pairs, so one write instruction covers
+    // C/2 consecutive words per pixel and (8 pixels apart = 32 banks apart) a second group: conflict-free for C >= 64.
+    {
+        constexpr int U = 5; // items whose reads are in flight together
+        const int C2 = C >> 1, items = C2 * (R + 2) * w8;
+        const float inv_c2 = 1.0f / (float)C2, inv_w8 = 1.0f / (float)w8;
+        const int64_t plane = (int64_t)H * W;
+        const uint16_t *xn = x + (int64_t)n * C * plane;
+        for (int q0 = tid; q0 < items; q0 += 256 * U) {
+            u32x4 va[U], vb[U];
+            int dsto[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int q = q0 + u * 256;
+                const int rest = small_div(q, inv_c2), cp = q - __mul24(rest, C2);
+                const int r = small_div(rest, inv_w8), ch = rest - __mul24(r, w8);
+                const int iy = rb * R - 1 + r;
+                va[u] = vb[u] = u32x4{0u, 0u, 0u, 0u};
+                if (q < items && iy >= 0 && iy < H) {
+                    const uint16_t *src = xn + (int64_t)(2 * cp) * plane + __mul24(iy, W) + ch * 8;
+                    va[u] = *(const u32x4 *)src;
+                    vb[u] = *(const u32x4 *)(src + plane);
+                }
+                dsto[u] = q < items ? __mul24(__mul24(r, Wp) + 1 + ch * 8, PS) + cp * 4 : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                if (dsto[u] < 0) continue;
+                ZK_LDS uint8_t *dst = smem + dsto[u];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    *(ZK_LDS uint32_t *)(dst + (2 * e) * PS) = __builtin_amdgcn_perm(vb[u][e], va[u][e], 0x05040100u);
+                    *(ZK_LDS uint32_t *)(dst + (2 * e + 1) * PS) = __builtin_amdgcn_perm(vb[u][e], va[u][e], 0x07060302u);
+                }
+            }
+        }
+        const int edge = (R + 2) * 2 * (C >> 3); // columns 0 and W + 1 of every row: C * 2 bytes each, 16 at a time
+        for (int q = tid; q < edge; q += 256) {
+            const int part = q % (C >> 3), side = (q / (C >> 3)) & 1, r = q / (C >> 3) / 2;
+            *(ZK_LDS u32x4 *)(smem + (r * Wp + (side ? W + 1 : 0)) * PS + part * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+
+    // per-lane byte offsets of this wave's pixels (tap 0, channel block 0) and of its weight rows
+    int xoff[PB];
+    {
+        const float inv_w = 1.0f / (float)W;
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++) {
+            const int p = wm * (PB * 32) + pb * 32 + l32, pr = small_div(p, inv_w), pc = p - __mul24(pr, W);
+            xoff[pb] = __mul24(__mul24(pr, Wp) + pc, PS) + half * 16;
+        }
+    }
+    const int cblocks = C >> 4;
+    // weight fragment of (tap, cb, nb): 16 bytes at ((tap * cblocks + cb) * Cout + co) * 32 + half * 16
+    const uint8_t *wlane = (const uint8_t *)wt + ((int64_t)(co0 + wn * 64 + l32)) * 32 + half * 16;
+    const int64_t wstep = (int64_t)Cout * 32; // bytes between (tap, cb) slices
+
+    f32x16 acc[2][PB];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[nb][pb][r] = 0.0f;
+
+    // k step s: tap = s / cblocks, cb = s % cblocks (the order of wt's slices). The weights of a step are requested two
+    // steps before their use and the input fragments one step before, each into one of three register sets (the step
+    // count 9 * cblocks is a multiple of three), so that a step's matrix instructions never wait for what they read.
+    const int steps = 9 * cblocks;
+    int tap = 0, cb = 0;
+    auto next_toff = [&]() { // tile offset of the next step's tap and channel block (the last step's again past the end)
+        const int tp = tap < 9 ? tap : 8, cc = tap < 9 ? cb : cblocks - 1;
+        const int ky = tp / 3, kx = tp - ky * 3;
+        if (++cb == cblocks) {
+            cb = 0;
+            tap++;
+        }
+        return (ky * Wp + kx) * PS + cc * 32;
+    };
+    auto load_w = [&](bf16x8(&wf)[2], int s) {
+        const uint8_t *src = wlane + (s < steps ? s : steps - 1) * wstep;
+        wf[0] = *(const bf16x8 *)src;
+        wf[1] = *(const bf16x8 *)(src + 32 * 32);
+    };
+    auto k_step = [&](const bf16x8(&wf)[2], const bf16x8(&xf)[PB], bf16x8(&xnext)[PB]) {
+        const int toff = next_toff();
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++) {
+            xnext[pb] = *(const ZK_LDS bf16x8 *)(smem + xoff[pb] + toff);
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++) acc[nb][pb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[nb], xf[pb], acc[nb][pb], 0, 0, 0);
+        }
+        // issue order: one LDS read of the next step, two matrix instructions of this one, seven times
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        }
+    };
+    bf16x8 w0[2], w1[2], w2[2], xa[PB], xb[PB], xc[PB];
+    load_w(w0, 0);
+    load_w(w1, 1);
+    __syncthreads(); // the tile is complete
+    {
+        const int toff = next_toff();
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++) xa[pb] = *(const ZK_LDS bf16x8 *)(smem + xoff[pb] + toff);
+    }
+    for (int s = 0; s < steps; s += 3) { // the barriers keep the scheduler from sinking a request towards its use
+        load_w(w2, s + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        k_step(w0, xa, xb);
+        load_w(w0, s + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        k_step(w1, xb, xc);
+        load_w(w1, s + 4);
+        __builtin_amdgcn_sched_barrier(0);
+        k_step(w2, xc, xa);
+    }
+
+    // ---- epilogue: register r of lane l is output channel 8*(r/4) + 4*(l/32) + r%4 of the block, pixel l%32 -----------
+    const int64_t plane = (int64_t)H * W;
+    const int co_lane = co0 + wn * 64 + half * 4;
+    float bv[2][16];
+    {
+        // all 32 reads are issued together; without a bias they read (and discard) the first weights instead
+        const uint16_t *bsrc = bias ? bias + co_lane : wt;
+        const uint32_t keep = bias ? 0xffffffffu : 0u;
+        uint16_t raw[2][16];
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) raw[nb][r] = bsrc[nb * 32 + (r >> 2) * 8 + (r & 3)];
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) bv[nb][r] = __uint_as_float(((uint32_t)raw[nb][r] << 16) & keep);
+    }
+    // the tile's pixels are consecutive in the image plane
+    const int64_t o0 = ((int64_t)n * Cout + co_lane) * plane + (int64_t)rb * R * W + wm * (PB * 32) + l32;
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int64_t o = o0 + (nb * 32 + (r >> 2) * 8 + (r & 3)) * plane;
+#pragma unroll
+            for (int pb = 0; pb < PB; pb++) {
+                float v = acc[nb][pb][r] + bv[nb][r];
+                if (RELU) v = (v > 0.0f ? 1.0f : 0.0f) * v;
+                if (OUT_BF16) ((uint16_t *)y)[o + pb * 32] = f32_to_bf16_trunc(v);
+                else ((float *)y)[o + pb * 32] = v;
+            }
+        }
+}
+
+int tile_rows(const Conv2d &p) { return p.W > 0 && TILE_PIX % p.W == 0 ? TILE_PIX / p.W : 0; }
+uint64_t lds_bytes(const Conv2d &p) { return (uint64_t)(tile_rows(p) + 2) * (p.W + 2) * (p.C * 2 + 16); }
+
+} // namespace
+
+bool conv3x3_direct_ok(const Conv2d &p) { // shape only: the same answer at registration and at every launch
+    const int R = tile_rows(p);
+    return p.dtype == DT_BF16 && (p.out_dtype == DT_BF16 || p.out_dtype == DT_F32) && p.KH == 3 && p.KW == 3 && p.sy == 1 && p.sx == 1 &&
+           p.dy == 1 && p.dx == 1 && p.py == 1 && p.px == 1 && p.C >= 16 && p.C % 16 == 0 && p.Cout % TILE_CO == 0 && p.W % 8 == 0 &&
+           R >= 1 && p.H % R == 0 && lds_bytes(p) <= 160 * 1024 && p.N > 0 && (int64_t)p.N * (p.H / R) < (1ll << 31) &&
+           p.Cout / TILE_CO <= 65535 && (int64_t)p.N * p.C * p.H * p.W < (1ll << 31) && (int64_t)p.N * p.Cout * p.H * p.W < (1ll << 40);
+}
+
+uint64_t conv3x3_scratch_bytes(const Conv2d &p) { return (uint64_t)9 * p.C * p.Cout * 2; }
+
+hipError_t conv3x3_init() {
+    // the input tile is larger than the default per-workgroup LDS limit
+    hipError_t e = hipSuccess;
+    const void *variants[4] = {(const void *)conv3x3_bf16_k<false, false>, (const void *)conv3x3_bf16_k<false, true>,
+                               (const void *)conv3x3_bf16_k<true, false>, (const void *)conv3x3_bf16_k<true, true>};
+    for (const void *f : variants)
+        if (e == hipSuccess) e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    return e;
+}
+
+// `wt` holds conv3x3_scratch_bytes(p) bytes for the re-laid weights.
+hipError_t conv3x3_direct(const Conv2d &p, void *wt, hipStream_t st) {
+    if ((uintptr_t)p.x % 16 || (uintptr_t)p.y % 4 || (uintptr_t)wt % 16) return hipErrorInvalidValue; // pool blocks are 256-byte aligned
+    const int R = tile_rows(p);
+    hipLaunchKernelGGL(conv3x3_weights_k, dim3((unsigned)((p.C * p.Cout + 255) / 256)), dim3(256), 0, st, (const uint16_t *)p.w,
+                       (uint16_t *)wt, p.C, p.Cout);
+    dim3 grid((unsigned)(p.N * (p.H / R)), (unsigned)(p.Cout / TILE_CO));
+    const bool out_bf16 = p.out_dtype == DT_BF16;
+#define ZK_LAUNCH(OB, RL)                                                                                                         \
+    hipLaunchKernelGGL((conv3x3_bf16_k<OB, RL>), grid, dim3(256), lds_bytes(p), st, (const uint16_t *)p.x, (const uint16_t *)wt, \
+                       (const uint16_t *)p.bias, p.y, p.C, p.H, p.W, p.Cout, R)
+    if (out_bf16 && p.relu) ZK_LAUNCH(true, true);
+    else if (out_bf16) ZK_LAUNCH(true, false);
+    else if (p.relu) ZK_LAUNCH(false, true);
+    else ZK_LAUNCH(false, false);
+#undef ZK_LAUNCH
+    return hipGetLastError();
+}
+
+} // namespace zk

@@ -147,6 +147,12 @@ struct Conv2d {
 };
 uint64_t conv2d_scratch_bytes(const Conv2d &p);
 hipError_t conv2d(const Conv2d &p, hipStream_t stream);
+// Direct 3 x 3 / stride 1 / padding 1 bf16 convolution (conv3x3.hip): shapes it takes, bytes for its re-laid weights,
+// one-time set-up of the kernel's LDS limit, launch.
+bool conv3x3_direct_ok(const Conv2d &p);
+uint64_t conv3x3_scratch_bytes(const Conv2d &p);
+hipError_t conv3x3_init();
+hipError_t conv3x3_direct(const Conv2d &p, void *weights_scratch, hipStream_t stream);
 
 // max-pool over the last two axes of `planes` images [H, W] -> [OH, OW]
 struct MaxPool2d {

@@ -995,6 +995,7 @@ ZHIP_EXPORT int32_t zhip_init(const zhip_config *cfg, zhip_ctx **out) {
         (e = hipEventCreateWithFlags(&c->plan_done, hipEventDisableTiming)) != hipSuccess)
         return bail(ZHIP_INITIALIZATION, "hipEventCreate", e);
     if ((e = zk::gemm_bf16_init()) != hipSuccess) return bail(ZHIP_INITIALIZATION, "raising the LDS limit of the GEMM kernels", e);
+    if ((e = zk::conv3x3_init()) != hipSuccess) return bail(ZHIP_INITIALIZATION, "raising the LDS limit of the convolution kernel", e);
     fill_info(c);
     if (c->debug & 1)
         fprintf(stderr, "[zyx-hip] device %d: %s (%s), %u CUs, %.1f GiB free\n", c->device, c->info.name, c->info.arch,
