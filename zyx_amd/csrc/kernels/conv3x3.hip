@@ -11,9 +11,12 @@
 // [tap][C/16][Cout][16], so the A operand (32 output channels x 16 input channels of one tap) is 1 KiB of consecutive
 // bytes read straight from L1 / L2, one k step ahead of its use.
 //
-// The product is formed transposed, acc[cout][pixel] = W . X^T, so that a lane owns a pixel column and the 32 lanes of
-// a store cover 32 consecutive pixels of one output channel: NCHW rows are written in 64-byte (bf16) or 128-byte (f32)
-// runs. 4 waves as 2 (pixel halves) x 2 (channel halves), 2 x 7 accumulator tiles of 32 x 32 each = 224 registers.
+// 4 waves as 2 (pixel halves) x 2 (channel halves), 2 x 7 accumulator tiles of 32 x 32 each = 224 registers, which start
+// at the bias. In a tile a lane owns one output channel and 16 pixels in runs of four. The epilogue stages the finished
+// tile in LDS (the input tile is dead by then) as [channel][pixel], 8 or 16 bytes per write, and copies it out in 16-byte
+// pieces, 896 (bf16) or 1792 (f32) consecutive bytes per channel row of NCHW: the memory pipeline takes one vector
+// instruction in about 16 cycles whatever its width, so narrow stores straight from the accumulators cost more than
+// the matrix loop.
 #include <algorithm>
 
 #include "dtypes.hpp"
@@ -26,11 +29,13 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 #define ZK_LDS __attribute__((address_space(3)))
 
 constexpr int PB = 7;                 // 32-pixel blocks per wave
 constexpr int TILE_PIX = 2 * PB * 32; // 448 pixels per workgroup
 constexpr int TILE_CO = 128;          // output channels per workgroup
+constexpr int STAGE_BYTES = 128 * (TILE_PIX * 2 + 16); // the epilogue's [channel][pixel] copy of the tile (bf16: 128 rows, f32: 64 rows twice)
 
 // w[Cout][C][3][3] -> wt[tap][C/16][Cout][16]. One thread per (cout, cin): the nine taps of a pair are 18 consecutive
 // bytes, and the 16 threads of a channel block write 32 consecutive bytes of each tap's slice.
@@ -67,30 +72,38 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
 
     // ---- input tile: rows rb*R - 1 .. rb*R + R of every channel, channel-innermost, zero outside the image ----------
     // One item = 8 consecutive columns of two neighbouring channels of one row: two 16-byte reads, eight 4-byte LDS
-    // writes (channel pair packed). Consecutive lanes take consecutive channel pairs, so one write instruction covers
-    // C/2 consecutive words per pixel and (8 pixels apart = 32 banks apart) a second group: conflict-free for C >= 64.
+    // writes (channel pair packed). The lanes of a wave take 4 neighbouring items of a row for each of 16 channel pairs
+    // (8 x 8 when C / 2 is not a multiple of 16): the texture unit takes one cache line per cycle, so neighbouring
+    // lanes share lines, while the writes of one instruction still spread over 32 banks (pixels 8 apart are 32 banks
+    // apart, 16 channel pairs are 16 consecutive words).
     {
-        constexpr int U = 5; // items whose reads are in flight together
-        const int C2 = C >> 1, items = C2 * (R + 2) * w8;
-        const float inv_c2 = 1.0f / (float)C2, inv_w8 = 1.0f / (float)w8;
+        constexpr int U = 9; // items whose reads are in flight together (one pass for 64 channels x 10 rows x 56 columns)
+        const int C2 = C >> 1, RC = (R + 2) * w8;          // channel pairs; 8-column pieces of one channel's rows
+        const int KB = (C2 & 15) ? 3 : 2;                  // log2(items of a row per wave instruction)
+        const int k = lane & ((1 << KB) - 1), cp_lo = lane >> KB, cp_lanes = 64 >> KB;
+        const int cpblocks = C2 / cp_lanes, groups = (RC + (1 << KB) - 1) >> KB, wave_items = cpblocks * groups;
+        const float inv_w8 = 1.0f / (float)w8;
         const int64_t plane = (int64_t)H * W;
         const uint16_t *xn = x + (int64_t)n * C * plane;
-        for (int q0 = tid; q0 < items; q0 += 256 * U) {
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        for (int t0 = wave_u; t0 < wave_items; t0 += 4 * U) {
             u32x4 va[U], vb[U];
             int dsto[U];
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const int q = q0 + u * 256;
-                const int rest = small_div(q, inv_c2), cp = q - __mul24(rest, C2);
-                const int r = small_div(rest, inv_w8), ch = rest - __mul24(r, w8);
+                const int t = t0 + 4 * u;                   // uniform over the wave
+                const int g = t / cpblocks, cpb = t - g * cpblocks;
+                const int rc = (g << KB) + k, cp = cpb * cp_lanes + cp_lo;
+                const int r = small_div(rc, inv_w8), ch = rc - __mul24(r, w8);
                 const int iy = rb * R - 1 + r;
+                const bool live = t < wave_items && rc < RC;
                 va[u] = vb[u] = u32x4{0u, 0u, 0u, 0u};
-                if (q < items && iy >= 0 && iy < H) {
+                if (live && iy >= 0 && iy < H) {
                     const uint16_t *src = xn + (int64_t)(2 * cp) * plane + __mul24(iy, W) + ch * 8;
                     va[u] = *(const u32x4 *)src;
                     vb[u] = *(const u32x4 *)(src + plane);
                 }
-                dsto[u] = q < items ? __mul24(__mul24(r, Wp) + 1 + ch * 8, PS) + cp * 4 : -1;
+                dsto[u] = live ? __mul24(__mul24(r, Wp) + 1 + ch * 8, PS) + cp * 4 : -1;
             }
 #pragma unroll
             for (int u = 0; u < U; u++) {
@@ -125,13 +138,15 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
     const uint8_t *wlane = (const uint8_t *)wt + ((int64_t)(co0 + wn * 64 + l32)) * 32 + half * 16;
     const int64_t wstep = (int64_t)Cout * 32; // bytes between (tap, cb) slices
 
-    f32x16 acc[2][PB];
+    f32x16 acc[2][PB]; // [nb][pb]: rows = pixels, columns = output channels; lane l owns channel l % 32 of block nb
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++)
+    for (int nb = 0; nb < 2; nb++) {
+        const float bv = bias ? bf16_to_f32(bias[co0 + wn * 64 + nb * 32 + l32]) : 0.0f;
 #pragma unroll
         for (int pb = 0; pb < PB; pb++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[nb][pb][r] = 0.0f;
+            for (int r = 0; r < 16; r++) acc[nb][pb][r] = bv;
+    }
 
     // k step s: tap = s / cblocks, cb = s % cblocks (the order of wt's slices). The weights of a step are requested two
     // steps before their use and the input fragments one step before, each into one of three register sets (the step
@@ -158,7 +173,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
         for (int pb = 0; pb < PB; pb++) {
             xnext[pb] = *(const ZK_LDS bf16x8 *)(smem + xoff[pb] + toff);
 #pragma unroll
-            for (int nb = 0; nb < 2; nb++) acc[nb][pb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[nb], xf[pb], acc[nb][pb], 0, 0, 0);
+            for (int nb = 0; nb < 2; nb++) acc[nb][pb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[pb], wf[nb], acc[nb][pb], 0, 0, 0);
         }
         // issue order: one LDS read of the next step, two matrix instructions of this one, seven times
 #pragma unroll
@@ -188,43 +203,60 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
         k_step(w2, xc, xa);
     }
 
-    // ---- epilogue: register r of lane l is output channel 8*(r/4) + 4*(l/32) + r%4 of the block, pixel l%32 -----------
+    // ---- epilogue: register r of lane l is pixel 8*(r/4) + 4*(l/32) + r%4 of block pb, channel l%32 of block nb --------
+    constexpr int ES = OUT_BF16 ? 2 : 4;          // bytes per output element
+    constexpr int RS = TILE_PIX * ES + 16;        // bytes per staged channel row
+    constexpr int CPR = TILE_PIX * ES / 16;       // 16-byte pieces per row
+    constexpr int PASSES = OUT_BF16 ? 1 : 2;      // f32: one channel block (nb) per pass, 64 rows each
     const int64_t plane = (int64_t)H * W;
-    const int co_lane = co0 + wn * 64 + half * 4;
-    float bv[2][16];
-    {
-        // all 32 reads are issued together; without a bias they read (and discard) the first weights instead
-        const uint16_t *bsrc = bias ? bias + co_lane : wt;
-        const uint32_t keep = bias ? 0xffffffffu : 0u;
-        uint16_t raw[2][16];
-#pragma unroll
-        for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) raw[nb][r] = bsrc[nb * 32 + (r >> 2) * 8 + (r & 3)];
-#pragma unroll
-        for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) bv[nb][r] = __uint_as_float(((uint32_t)raw[nb][r] << 16) & keep);
-    }
     // the tile's pixels are consecutive in the image plane
-    const int64_t o0 = ((int64_t)n * Cout + co_lane) * plane + (int64_t)rb * R * W + wm * (PB * 32) + l32;
+    uint8_t *ytile = (uint8_t *)y + (((int64_t)n * Cout + co0) * plane + (int64_t)rb * R * W) * ES;
+    __syncthreads(); // every wave has read its last input fragment
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++)
+    for (int pass = 0; pass < PASSES; pass++) {
+        if (pass) __syncthreads(); // the previous pass has been copied out
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int64_t o = o0 + (nb * 32 + (r >> 2) * 8 + (r & 3)) * plane;
+        for (int nb = 0; nb < 2; nb++) {
+            if (!OUT_BF16 && nb != pass) continue;
+            const int row = OUT_BF16 ? wn * 64 + nb * 32 + l32 : wn * 32 + l32;
+            ZK_LDS uint8_t *dst = smem + row * RS + (wm * (PB * 32) + 4 * half) * ES;
 #pragma unroll
-            for (int pb = 0; pb < PB; pb++) {
-                float v = acc[nb][pb][r] + bv[nb][r];
-                if (RELU) v = (v > 0.0f ? 1.0f : 0.0f) * v;
-                if (OUT_BF16) ((uint16_t *)y)[o + pb * 32] = f32_to_bf16_trunc(v);
-                else ((float *)y)[o + pb * 32] = v;
-            }
+            for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        v[e] = acc[nb][pb][g * 4 + e];
+                        if (RELU) v[e] = (v[e] > 0.0f ? 1.0f : 0.0f) * v[e];
+                    }
+                    ZK_LDS uint8_t *d = dst + (pb * 32 + g * 8) * ES;
+                    if (OUT_BF16) {
+                        // truncation to bf16 = the upper halves of the four words
+                        u32x2 pk = {__builtin_amdgcn_perm(__float_as_uint(v[1]), __float_as_uint(v[0]), 0x07060302u),
+                                    __builtin_amdgcn_perm(__float_as_uint(v[3]), __float_as_uint(v[2]), 0x07060302u)};
+                        *(ZK_LDS u32x2 *)d = pk;
+                    } else {
+                        *(ZK_LDS u32x4 *)d = u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])};
+                    }
+                }
         }
+        __syncthreads();
+        constexpr int ROWS = OUT_BF16 ? 128 : 64;
+#pragma unroll 4
+        for (int idx = tid; idx < ROWS * CPR; idx += 256) {
+            const int row = idx / CPR, col = idx - row * CPR;
+            const int co = OUT_BF16 ? row : (row >> 5) * 64 + pass * 32 + (row & 31);
+            const u32x4 v = *(const ZK_LDS u32x4 *)(smem + row * RS + col * 16);
+            *(u32x4 *)(ytile + (int64_t)co * plane * ES + col * 16) = v;
+        }
+    }
 }
 
 int tile_rows(const Conv2d &p) { return p.W > 0 && TILE_PIX % p.W == 0 ? TILE_PIX / p.W : 0; }
-uint64_t lds_bytes(const Conv2d &p) { return (uint64_t)(tile_rows(p) + 2) * (p.W + 2) * (p.C * 2 + 16); }
+uint64_t lds_bytes(const Conv2d &p) { // the input tile, later reused for the staged output tile
+    return std::max<uint64_t>((uint64_t)(tile_rows(p) + 2) * (p.W + 2) * (p.C * 2 + 16), STAGE_BYTES);
+}
 
 } // namespace
 
@@ -250,7 +282,7 @@ hipError_t conv3x3_init() {
 
 // `wt` holds conv3x3_scratch_bytes(p) bytes for the re-laid weights.
 hipError_t conv3x3_direct(const Conv2d &p, void *wt, hipStream_t st) {
-    if ((uintptr_t)p.x % 16 || (uintptr_t)p.y % 4 || (uintptr_t)wt % 16) return hipErrorInvalidValue; // pool blocks are 256-byte aligned
+    if ((uintptr_t)p.x % 16 || (uintptr_t)p.y % 16 || (uintptr_t)wt % 16) return hipErrorInvalidValue; // pool blocks are 256-byte aligned
     const int R = tile_rows(p);
     hipLaunchKernelGGL(conv3x3_weights_k, dim3((unsigned)((p.C * p.Cout + 255) / 256)), dim3(256), 0, st, (const uint16_t *)p.w,
                        (uint16_t *)wt, p.C, p.Cout);
