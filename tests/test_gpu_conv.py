@@ -214,3 +214,30 @@ def test_conv3x3_direct_bf16(hip, oracle, shape, bias, relu):
     taps[:, 0] = taps[:, -1] = 6
     taps[0, 0] = taps[0, -1] = taps[-1, 0] = taps[-1, -1] = 4
     assert np.array_equal(cnt[0, 0], taps * c) and np.array_equal(cnt[0, -1], taps * c)
+
+
+@pytest.mark.parametrize("shape", [(2, 16, 16, 56, 128), (1, 64, 56, 56, 128), (3, 32, 28, 16, 256), (2, 48, 8, 112, 128), (1, 16, 56, 8, 128)])
+@pytest.mark.parametrize("bias,relu", [(True, True), (False, False)])
+def test_conv3x3_direct_f32(hip, oracle, shape, bias, relu):
+    """The same direct kernel on f32 data (v_mfma_f32_32x32x2_f32): 2e-5 of the magnitude sum against the oracle (the
+    order of the k sum differs), zero borders by tap counting, and linearity in the input."""
+    dev, pool = hip
+    n, c, h, w, co = shape
+    r = oracle.Rng(n * 2000 + c + w)
+    x, wt = r.randn((n, c, h, w)), r.randn((co, c, 3, 3), 0.1)
+    b = r.randn(co, 0.1) if bias else None
+    args = ((1, 1), (1, 1), (1, 1))
+    mag = oracle.conv2d(np.abs(x), np.abs(wt), None if b is None else np.abs(b), *args)
+    got = conv2d(dev, pool, x, wt, b, *args, relu=relu)
+    want = oracle.conv2d(x, wt, b, *args, relu)
+    assert got.dtype == np.float32 and np.all(np.abs(got - want) <= 2e-5 * mag + 1e-30), np.max(np.abs(got - want) / (mag + 1e-30))
+    cnt = conv2d(dev, pool, np.ones((1, c, h, w), np.float32), np.ones((co, c, 3, 3), np.float32), None, *args)
+    taps = np.full((h, w), 9.0)
+    taps[0, :] = taps[-1, :] = 6
+    taps[:, 0] = taps[:, -1] = 6
+    taps[0, 0] = taps[0, -1] = taps[-1, 0] = taps[-1, -1] = 4
+    assert np.array_equal(cnt[0, 0], taps * c) and np.array_equal(cnt[0, -1], taps * c)
+    if not relu and b is None:
+        x2 = r.randn((n, c, h, w))
+        both = conv2d(dev, pool, x + x2, wt, None, *args)
+        assert np.allclose(both, got + conv2d(dev, pool, x2, wt, None, *args), rtol=1e-4, atol=2e-4)

@@ -37,27 +37,34 @@ constexpr int TILE_PIX = 2 * PB * 32; // 448 pixels per workgroup
 constexpr int TILE_CO = 128;          // output channels per workgroup
 constexpr int STAGE_BYTES = 128 * (TILE_PIX * 2 + 16); // the epilogue's [channel][pixel] copy of the tile (bf16: 128 rows, f32: 64 rows twice)
 
-// w[Cout][C][3][3] -> wt[tap][C/16][Cout][16]. One thread per (cout, cin): the nine taps of a pair are 18 consecutive
-// bytes, and the 16 threads of a channel block write 32 consecutive bytes of each tap's slice.
-__global__ __launch_bounds__(256) void conv3x3_weights_k(const uint16_t *__restrict__ w, uint16_t *__restrict__ wt, int C, int Cout) {
+// w[Cout][C][3][3] -> wt[tap][C/G][Cout][G], G = 16 (bf16) or 8 (f32) channels = the 32 bytes per output channel that one
+// k step reads. One thread per (cout, cin): the nine taps of a pair are consecutive, and the G threads of a channel
+// block write 32 consecutive bytes of each tap's slice.
+template <typename T, int LOG_G>
+__global__ __launch_bounds__(256) void conv3x3_weights_k(const T *__restrict__ w, T *__restrict__ wt, int C, int Cout) {
     const int i = blockIdx.x * 256 + threadIdx.x; // = co * C + c
     if (i >= C * Cout) return;
-    const int co = i / C, c = i - co * C, cb = c >> 4, ci = c & 15;
-    uint16_t v[9];
+    const int co = i / C, c = i - co * C, cb = c >> LOG_G, ci = c & ((1 << LOG_G) - 1);
+    T v[9];
 #pragma unroll
     for (int t = 0; t < 9; t++) v[t] = w[(int64_t)i * 9 + t];
 #pragma unroll
-    for (int t = 0; t < 9; t++) wt[(((int64_t)t * (C >> 4) + cb) * Cout + co) * 16 + ci] = v[t];
+    for (int t = 0; t < 9; t++) wt[((((int64_t)t * (C >> LOG_G) + cb) * Cout + co) << LOG_G) + ci] = v[t];
 }
 
 // floor(q / d) for 0 <= q < 2^22, inv = 1.0f / d: the rounding errors of the reciprocal and of the product are far
 // smaller than the distance 0.5 / d of (q + 0.5) / d from the nearest integer
 __device__ __forceinline__ int small_div(int q, float inv) { return (int)(((float)q + 0.5f) * inv); }
 
-template <bool OUT_BF16, bool RELU>
-__global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restrict__ x, const uint16_t *__restrict__ wt,
-                                                         const uint16_t *__restrict__ bias, void *__restrict__ y, int C, int H,
-                                                         int W, int Cout, int R) {
+// F32_IN: f32 input, weights, bias and output on v_mfma_f32_32x32x2_f32 (a k step is 8 channels of one tap: lane half h
+// holds channels 4h .. 4h + 3 of the block, and the j-th of four matrix instructions multiplies channels j and 4 + j);
+// otherwise bf16 input on v_mfma_f32_32x32x16_bf16 (a k step is 16 channels of one tap).
+template <bool F32_IN, bool OUT_BF16, bool RELU>
+__global__ __launch_bounds__(256, 1) void conv3x3_k(const void *__restrict__ x_, const void *__restrict__ wt,
+                                                    const void *__restrict__ bias, void *__restrict__ y, int C, int H, int W,
+                                                    int Cout, int R) {
+    static_assert(!(F32_IN && OUT_BF16), "f32 input gives f32 output");
+    constexpr int ES_IN = F32_IN ? 4 : 2;
     // A workgroup is alone on its compute unit, one wave per SIMD: nothing hides instruction issue outside the matrix
     // loop, so every phase below is written for a small instruction count (no integer division, no per-element branch).
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
@@ -67,8 +74,8 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
     const int tiles_per_image = H / R;
     const int n = blockIdx.x / tiles_per_image, rb = blockIdx.x - n * tiles_per_image;
     const int co0 = blockIdx.y * TILE_CO;
-    const int PS = C * 2 + 16;            // bytes between neighbouring pixels in LDS
-    const int Wp = W + 2, w8 = W >> 3;
+    const int PS = C * ES_IN + 16;        // bytes between neighbouring pixels in LDS
+    const int Wp = W + 2;
 
     // ---- input tile: rows rb*R - 1 .. rb*R + R of every channel, channel-innermost, zero outside the image ----------
     // One item = 8 consecutive columns of two neighbouring channels of one row: two 16-byte reads, eight 4-byte LDS
@@ -76,7 +83,9 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
     // (8 x 8 when C / 2 is not a multiple of 16): the texture unit takes one cache line per cycle, so neighbouring
     // lanes share lines, while the writes of one instruction still spread over 32 banks (pixels 8 apart are 32 banks
     // apart, 16 channel pairs are 16 consecutive words).
-    {
+    if constexpr (!F32_IN) {
+        const uint16_t *x = (const uint16_t *)x_;
+        const int w8 = W >> 3;
         constexpr int U = 9; // items whose reads are in flight together (one pass for 64 channels x 10 rows x 56 columns)
         const int C2 = C >> 1, RC = (R + 2) * w8;          // channel pairs; 8-column pieces of one channel's rows
         const int KB = (C2 & 15) ? 3 : 2;                  // log2(items of a row per wave instruction)
@@ -116,9 +125,46 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
                 }
             }
         }
-        const int edge = (R + 2) * 2 * (C >> 3); // columns 0 and W + 1 of every row: C * 2 bytes each, 16 at a time
+    } else {
+        // f32: one item = 4 consecutive columns of one channel (16 bytes), four 4-byte LDS writes; the lanes of a wave take
+        // 4 neighbouring items of a row for each of 16 channels (writes: pixels 4 apart are 16 banks apart for C = 64).
+        const float *x = (const float *)x_;
+        constexpr int U = 12;
+        const int w4 = W >> 2, RC = (R + 2) * w4;
+        const int k = lane & 3, c_lo = lane >> 2;
+        const int cblocks16 = C >> 4, groups = (RC + 3) >> 2, wave_items = cblocks16 * groups;
+        const float inv_w4 = 1.0f / (float)w4;
+        const int64_t plane = (int64_t)H * W;
+        const float *xn = x + (int64_t)n * C * plane;
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        for (int t0 = wave_u; t0 < wave_items; t0 += 4 * U) {
+            u32x4 v[U];
+            int dsto[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int t = t0 + 4 * u;                   // uniform over the wave
+                const int g = t / cblocks16, cbk = t - g * cblocks16;
+                const int rc = (g << 2) + k, c = cbk * 16 + c_lo;
+                const int r = small_div(rc, inv_w4), pc = rc - __mul24(r, w4);
+                const int iy = rb * R - 1 + r;
+                const bool live = t < wave_items && rc < RC;
+                v[u] = u32x4{0u, 0u, 0u, 0u};
+                if (live && iy >= 0 && iy < H) v[u] = *(const u32x4 *)(xn + (int64_t)c * plane + __mul24(iy, W) + pc * 4);
+                dsto[u] = live ? __mul24(__mul24(r, Wp) + 1 + pc * 4, PS) + c * 4 : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                if (dsto[u] < 0) continue;
+                ZK_LDS uint8_t *dst = smem + dsto[u];
+#pragma unroll
+                for (int e = 0; e < 4; e++) *(ZK_LDS uint32_t *)(dst + e * PS) = v[u][e];
+            }
+        }
+    }
+    {
+        const int parts = C * ES_IN / 16, edge = (R + 2) * 2 * parts; // columns 0 and W + 1 of every row, 16 bytes at a time
         for (int q = tid; q < edge; q += 256) {
-            const int part = q % (C >> 3), side = (q / (C >> 3)) & 1, r = q / (C >> 3) / 2;
+            const int part = q % parts, side = (q / parts) & 1, r = q / parts / 2;
             *(ZK_LDS u32x4 *)(smem + (r * Wp + (side ? W + 1 : 0)) * PS + part * 16) = u32x4{0u, 0u, 0u, 0u};
         }
     }
@@ -133,7 +179,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
             xoff[pb] = __mul24(__mul24(pr, Wp) + pc, PS) + half * 16;
         }
     }
-    const int cblocks = C >> 4;
+    const int cblocks = F32_IN ? C >> 3 : C >> 4; // k steps per tap
     // weight fragment of (tap, cb, nb): 16 bytes at ((tap * cblocks + cb) * Cout + co) * 32 + half * 16
     const uint8_t *wlane = (const uint8_t *)wt + ((int64_t)(co0 + wn * 64 + l32)) * 32 + half * 16;
     const int64_t wstep = (int64_t)Cout * 32; // bytes between (tap, cb) slices
@@ -141,7 +187,8 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
     f32x16 acc[2][PB]; // [nb][pb]: rows = pixels, columns = output channels; lane l owns channel l % 32 of block nb
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
-        const float bv = bias ? bf16_to_f32(bias[co0 + wn * 64 + nb * 32 + l32]) : 0.0f;
+        const int co = co0 + wn * 64 + nb * 32 + l32;
+        const float bv = !bias ? 0.0f : F32_IN ? ((const float *)bias)[co] : bf16_to_f32(((const uint16_t *)bias)[co]);
 #pragma unroll
         for (int pb = 0; pb < PB; pb++)
 #pragma unroll
@@ -162,34 +209,45 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
         }
         return (ky * Wp + kx) * PS + cc * 32;
     };
-    auto load_w = [&](bf16x8(&wf)[2], int s) {
+    auto load_w = [&](u32x4(&wf)[2], int s) {
         const uint8_t *src = wlane + (s < steps ? s : steps - 1) * wstep;
-        wf[0] = *(const bf16x8 *)src;
-        wf[1] = *(const bf16x8 *)(src + 32 * 32);
+        wf[0] = *(const u32x4 *)src;
+        wf[1] = *(const u32x4 *)(src + 32 * 32);
     };
-    auto k_step = [&](const bf16x8(&wf)[2], const bf16x8(&xf)[PB], bf16x8(&xnext)[PB]) {
+    auto k_step = [&](const u32x4(&wf)[2], const u32x4(&xf)[PB], u32x4(&xnext)[PB]) {
         const int toff = next_toff();
 #pragma unroll
-        for (int pb = 0; pb < PB; pb++) {
-            xnext[pb] = *(const ZK_LDS bf16x8 *)(smem + xoff[pb] + toff);
+        for (int pb = 0; pb < PB; pb++) xnext[pb] = *(const ZK_LDS u32x4 *)(smem + xoff[pb] + toff);
+        if constexpr (F32_IN) {
 #pragma unroll
-            for (int nb = 0; nb < 2; nb++) acc[nb][pb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[pb], wf[nb], acc[nb][pb], 0, 0, 0);
+            for (int j = 0; j < 4; j++) // j outermost: 14 independent instructions between two on the same accumulator
+#pragma unroll
+                for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                    for (int nb = 0; nb < 2; nb++)
+                        acc[nb][pb] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(xf[pb][j]), __uint_as_float(wf[nb][j]), acc[nb][pb], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                for (int nb = 0; nb < 2; nb++)
+                    acc[nb][pb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, xf[pb]), __builtin_bit_cast(bf16x8, wf[nb]), acc[nb][pb], 0, 0, 0);
         }
-        // issue order: one LDS read of the next step, two matrix instructions of this one, seven times
+        // issue order: one LDS read of the next step, then this step's share of matrix instructions, seven times
 #pragma unroll
         for (int pb = 0; pb < PB; pb++) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, F32_IN ? 8 : 2, 0);
         }
     };
-    bf16x8 w0[2], w1[2], w2[2], xa[PB], xb[PB], xc[PB];
+    u32x4 w0[2], w1[2], w2[2], xa[PB], xb[PB], xc[PB];
     load_w(w0, 0);
     load_w(w1, 1);
     __syncthreads(); // the tile is complete
     {
         const int toff = next_toff();
 #pragma unroll
-        for (int pb = 0; pb < PB; pb++) xa[pb] = *(const ZK_LDS bf16x8 *)(smem + xoff[pb] + toff);
+        for (int pb = 0; pb < PB; pb++) xa[pb] = *(const ZK_LDS u32x4 *)(smem + xoff[pb] + toff);
     }
     for (int s = 0; s < steps; s += 3) { // the barriers keep the scheduler from sinking a request towards its use
         load_w(w2, s + 2);
@@ -228,6 +286,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         v[e] = acc[nb][pb][g * 4 + e];
+                        asm volatile("" : "+v"(v[e])); // a copy in a vector register, here: the accumulators stay where they are
                         if (RELU) v[e] = (v[e] > 0.0f ? 1.0f : 0.0f) * v[e];
                     }
                     ZK_LDS uint8_t *d = dst + (pb * 32 + g * 8) * ES;
@@ -239,6 +298,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
                     } else {
                         *(ZK_LDS u32x4 *)d = u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])};
                     }
+                    __builtin_amdgcn_sched_barrier(0); // or the scheduler reads all 224 accumulators first and spills
                 }
         }
         __syncthreads();
@@ -254,27 +314,30 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_k(const uint16_t *__restr
 }
 
 int tile_rows(const Conv2d &p) { return p.W > 0 && TILE_PIX % p.W == 0 ? TILE_PIX / p.W : 0; }
+int elem_bytes(const Conv2d &p) { return p.dtype == DT_F32 ? 4 : 2; }
 uint64_t lds_bytes(const Conv2d &p) { // the input tile, later reused for the staged output tile
-    return std::max<uint64_t>((uint64_t)(tile_rows(p) + 2) * (p.W + 2) * (p.C * 2 + 16), STAGE_BYTES);
+    return std::max<uint64_t>((uint64_t)(tile_rows(p) + 2) * (p.W + 2) * (p.C * elem_bytes(p) + 16), STAGE_BYTES);
 }
 
 } // namespace
 
 bool conv3x3_direct_ok(const Conv2d &p) { // shape only: the same answer at registration and at every launch
     const int R = tile_rows(p);
-    return p.dtype == DT_BF16 && (p.out_dtype == DT_BF16 || p.out_dtype == DT_F32) && p.KH == 3 && p.KW == 3 && p.sy == 1 && p.sx == 1 &&
-           p.dy == 1 && p.dx == 1 && p.py == 1 && p.px == 1 && p.C >= 16 && p.C % 16 == 0 && p.Cout % TILE_CO == 0 && p.W % 8 == 0 &&
-           R >= 1 && p.H % R == 0 && lds_bytes(p) <= 160 * 1024 && p.N > 0 && (int64_t)p.N * (p.H / R) < (1ll << 31) &&
-           p.Cout / TILE_CO <= 65535 && (int64_t)p.N * p.C * p.H * p.W < (1ll << 31) && (int64_t)p.N * p.Cout * p.H * p.W < (1ll << 40);
+    const bool types = (p.dtype == DT_BF16 && (p.out_dtype == DT_BF16 || p.out_dtype == DT_F32)) || (p.dtype == DT_F32 && p.out_dtype == DT_F32);
+    return types && p.KH == 3 && p.KW == 3 && p.sy == 1 && p.sx == 1 && p.dy == 1 && p.dx == 1 && p.py == 1 && p.px == 1 && p.C >= 16 &&
+           p.C % 16 == 0 && p.Cout % TILE_CO == 0 && p.W % 8 == 0 && R >= 1 && p.H % R == 0 && lds_bytes(p) <= 160 * 1024 && p.N > 0 &&
+           (int64_t)p.N * (p.H / R) < (1ll << 31) && p.Cout / TILE_CO <= 65535 && (int64_t)p.N * p.C * p.H * p.W < (1ll << 31) &&
+           (int64_t)p.N * p.Cout * p.H * p.W < (1ll << 40) && (int64_t)p.C * p.Cout < (1ll << 26);
 }
 
-uint64_t conv3x3_scratch_bytes(const Conv2d &p) { return (uint64_t)9 * p.C * p.Cout * 2; }
+uint64_t conv3x3_scratch_bytes(const Conv2d &p) { return (uint64_t)9 * p.C * p.Cout * elem_bytes(p); }
 
 hipError_t conv3x3_init() {
     // the input tile is larger than the default per-workgroup LDS limit
     hipError_t e = hipSuccess;
-    const void *variants[4] = {(const void *)conv3x3_bf16_k<false, false>, (const void *)conv3x3_bf16_k<false, true>,
-                               (const void *)conv3x3_bf16_k<true, false>, (const void *)conv3x3_bf16_k<true, true>};
+    const void *variants[6] = {(const void *)conv3x3_k<false, false, false>, (const void *)conv3x3_k<false, false, true>,
+                               (const void *)conv3x3_k<false, true, false>,  (const void *)conv3x3_k<false, true, true>,
+                               (const void *)conv3x3_k<true, false, false>,  (const void *)conv3x3_k<true, false, true>};
     for (const void *f : variants)
         if (e == hipSuccess) e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     return e;
@@ -284,17 +347,24 @@ hipError_t conv3x3_init() {
 hipError_t conv3x3_direct(const Conv2d &p, void *wt, hipStream_t st) {
     if ((uintptr_t)p.x % 16 || (uintptr_t)p.y % 16 || (uintptr_t)wt % 16) return hipErrorInvalidValue; // pool blocks are 256-byte aligned
     const int R = tile_rows(p);
-    hipLaunchKernelGGL(conv3x3_weights_k, dim3((unsigned)((p.C * p.Cout + 255) / 256)), dim3(256), 0, st, (const uint16_t *)p.w,
-                       (uint16_t *)wt, p.C, p.Cout);
+    const dim3 wgrid((unsigned)((p.C * p.Cout + 255) / 256));
+    if (p.dtype == DT_F32) hipLaunchKernelGGL((conv3x3_weights_k<float, 3>), wgrid, dim3(256), 0, st, (const float *)p.w, (float *)wt, p.C, p.Cout);
+    else hipLaunchKernelGGL((conv3x3_weights_k<uint16_t, 4>), wgrid, dim3(256), 0, st, (const uint16_t *)p.w, (uint16_t *)wt, p.C, p.Cout);
     dim3 grid((unsigned)(p.N * (p.H / R)), (unsigned)(p.Cout / TILE_CO));
     const bool out_bf16 = p.out_dtype == DT_BF16;
-#define ZK_LAUNCH(OB, RL)                                                                                                         \
-    hipLaunchKernelGGL((conv3x3_bf16_k<OB, RL>), grid, dim3(256), lds_bytes(p), st, (const uint16_t *)p.x, (const uint16_t *)wt, \
-                       (const uint16_t *)p.bias, p.y, p.C, p.H, p.W, p.Cout, R)
-    if (out_bf16 && p.relu) ZK_LAUNCH(true, true);
-    else if (out_bf16) ZK_LAUNCH(true, false);
-    else if (p.relu) ZK_LAUNCH(false, true);
-    else ZK_LAUNCH(false, false);
+#define ZK_LAUNCH(FI, OB, RL)                                                                                                     \
+    hipLaunchKernelGGL((conv3x3_k<FI, OB, RL>), grid, dim3(256), lds_bytes(p), st, p.x, (const void *)wt, p.bias, p.y, p.C, p.H, p.W, \
+                       p.Cout, R)
+    if (p.dtype == DT_F32) {
+        if (p.relu) ZK_LAUNCH(true, false, true);
+        else ZK_LAUNCH(true, false, false);
+    } else if (out_bf16) {
+        if (p.relu) ZK_LAUNCH(false, true, true);
+        else ZK_LAUNCH(false, true, false);
+    } else {
+        if (p.relu) ZK_LAUNCH(false, false, true);
+        else ZK_LAUNCH(false, false, false);
+    }
 #undef ZK_LAUNCH
     return hipGetLastError();
 }
