@@ -101,6 +101,7 @@ def extra_conv(dev, pool, kernels, steps=50, warmup=50):
         mp = dev.register_kernel(kernels.max_pool2d_desc(N * CO, HW, HW, dtype=dt))
         dev.profile_kernel(conv, [[xb, wb, yb]], warmup)
         us = dev.profile_kernel(conv, [[xb, wb, yb]], steps)
+        dev.profile_kernel(mp, [[yb, pb]], warmup)
         us_p = dev.profile_kernel(mp, [[yb, pb]], steps)
         pool_bytes = (N * CO * HW * HW + N * CO * (HW // 2) ** 2) * isz
         peak = 157.3 if isz == 4 else 2500.0
