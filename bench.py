@@ -103,11 +103,16 @@ def extra_conv(dev, pool, kernels, steps=50, warmup=50):
         us = dev.profile_kernel(conv, [[xb, wb, yb]], steps)
         dev.profile_kernel(mp, [[yb, pb]], warmup)
         us_p = dev.profile_kernel(mp, [[yb, pb]], steps)
+        fused = dev.register_kernel(kernels.conv2d_desc(N, C, HW, HW, CO, 3, 3, padding=(1, 1), relu=True, dtype=dt, pool=True))
+        dev.profile_kernel(fused, [[xb, wb, pb]], warmup)
+        us_f = dev.profile_kernel(fused, [[xb, wb, pb]], steps)
+        dev.release(fused)
         pool_bytes = (N * CO * HW * HW + N * CO * (HW // 2) ** 2) * isz
         peak = 157.3 if isz == 4 else 2500.0
         out[name] = {"conv_relu_us": round(us, 2), "conv_TFLOP/s": round(flop / us / 1e6, 1),
                      "conv_frac_of_peak": round(flop / us / 1e6 / peak, 4), "peak_TFLOP/s": peak,
-                     "max_pool_us": round(us_p, 2), "max_pool_GB/s": round(pool_bytes / us_p / 1e3, 1)}
+                     "max_pool_us": round(us_p, 2), "max_pool_GB/s": round(pool_bytes / us_p / 1e3, 1),
+                     "conv_relu_pool_one_launch_us": round(us_f, 2), "conv_relu_pool_two_launches_us": round(us + us_p, 2)}
         dev.release(conv)
         dev.release(mp)
         for b_ in (xb, wb, yb, pb):

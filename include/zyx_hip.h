@@ -167,9 +167,12 @@ enum zhip_kernel_kind {
     /* Tensor::conv for 4-D NCHW input, groups = 1 (zyx/src/tensor/mod.rs:2583-2680; layer
      * zyx-nn/src/conv2d.rs:60-70): y[N,Cout,OH,OW] = x[N,C,H,W] (*) w[Cout,C,KH,KW] (+ bias[Cout])
      * (then ReLU), zero padding, OH = (H + 2*py - dy*(KH-1) - 1) / sy + 1 (OW likewise).
-     * dims = {N, C, H, W, Cout, KH, KW}; iparams = {sy, sx, py, px, dy, dx, has_bias, relu};
+     * dims = {N, C, H, W, Cout, KH, KW}; iparams = {sy, sx, py, px, dy, dx, has_bias, relu, pool};
      * dtype F32 or BF16 for x, w, bias; out_dtype = dtype, or F32 for BF16 operands. Products
-     * and sums are f32. args: x, w, (bias), y. */
+     * and sums are f32. pool = 1: y is Tensor::max_pool([2, 2]) of that result (stride 2, no
+     * padding; mod.rs:2706-2741), y[N,Cout,OH/2,OW/2], from the same launch; taken for
+     * 3x3 / stride 1 / dilation 1 / padding 1 shapes with C % 16 = 0, Cout % 128 = 0, W % 8 = 0,
+     * W a divisor of 224 and H a multiple of 448 / W, refused otherwise. args: x, w, (bias), y. */
     ZHIP_K_CONV2D = 7,
     /* Tensor::max_pool over the last two axes (zyx/src/tensor/mod.rs:2706-2741): padding counts
      * as the dtype's lowest value. dims = {planes (product of the leading axes), H, W, KH, KW};

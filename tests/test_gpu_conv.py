@@ -241,3 +241,42 @@ def test_conv3x3_direct_f32(hip, oracle, shape, bias, relu):
         x2 = r.randn((n, c, h, w))
         both = conv2d(dev, pool, x + x2, wt, None, *args)
         assert np.allclose(both, got + conv2d(dev, pool, x2, wt, None, *args), rtol=1e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("shape", [(2, 16, 16, 56, 128), (2, 64, 56, 56, 128), (3, 32, 28, 16, 256), (2, 48, 8, 112, 128)])
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "bf16->f32"])
+def test_conv3x3_fused_max_pool(hip, oracle, shape, dtype):
+    """conv + bias + ReLU + 2 x 2 max-pool in one launch (only the pooled tensor is written) equals the two-launch
+    result bit for bit, and the oracle's pooled convolution within the convolution's tolerance; without ReLU negative
+    maxima survive. A shape whose tiles hold an odd number of rows is refused."""
+    dev, pool = hip
+    n, c, h, w, co = shape
+    r = oracle.Rng(n * 3000 + c + w)
+    x, wt, b = r.randn((n, c, h, w)), r.randn((co, c, 3, 3), 0.1), r.randn(co, 0.1)
+    dt = DType.F32 if dtype == "f32" else DType.BF16
+    odt = DType.BF16 if dtype == "bf16" else DType.F32
+    if dt == DType.BF16:
+        x, wt, b = oracle.f32_to_bf16(x), oracle.f32_to_bf16(wt), oracle.f32_to_bf16(b)
+    args = ((1, 1), (1, 1), (1, 1))
+    for relu in (True, False):
+        y, pooled = conv2d(dev, pool, x, wt, b, *args, relu=relu, dtype=dt, out_dtype=odt, pool_kernel=(2, 2))
+        fused = conv2d(dev, pool, x, wt, b, *args, relu=relu, dtype=dt, out_dtype=odt, fused_pool=True)
+        assert fused.shape == (n, co, h // 2, w // 2) and fused.dtype == pooled.dtype
+        assert np.array_equal(fused, pooled)
+        ref = y.reshape(n, co, h // 2, 2, w // 2, 2)
+        ref = oracle.bf16_to_f32(ref) if odt == DType.BF16 else ref
+        got = oracle.bf16_to_f32(fused) if odt == DType.BF16 else fused
+        assert np.array_equal(got, ref.max(axis=(3, 5)))
+        if not relu:
+            assert (got < 0).any()
+    if dtype == "f32" and shape == (2, 16, 16, 56, 128):
+        xf = oracle.Rng(1).randn((1, 16, 4, 56))
+        with pytest.raises(Exception):  # 448 / 56 = 8 rows per tile, H = 4 is not a multiple
+            conv2d(dev, pool, xf, wt, b, *args, relu=True, fused_pool=True)
+        xf = oracle.Rng(1).randn((1, 16, 8, 56))
+        want = oracle.max_pool2d(oracle.conv2d(xf, wt, b, *args, True), (2, 2), (2, 2), (0, 0), (1, 1))
+        mag = oracle.max_pool2d(oracle.conv2d(np.abs(xf), np.abs(wt), np.abs(b), *args), (2, 2), (2, 2), (0, 0), (1, 1))
+        got = conv2d(dev, pool, xf, wt, b, *args, relu=True, fused_pool=True)
+        assert np.all(np.abs(got - want) <= 2e-5 * mag)
+        with pytest.raises(Exception):  # W = 448: one row per tile
+            conv2d(dev, pool, np.zeros((1, 16, 2, 448), np.float32), wt, b, *args, fused_pool=True)

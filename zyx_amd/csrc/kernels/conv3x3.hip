@@ -58,8 +58,10 @@ __device__ __forceinline__ int small_div(int q, float inv) { return (int)(((floa
 
 // F32_IN: f32 input, weights, bias and output on v_mfma_f32_32x32x2_f32 (a k step is 8 channels of one tap: lane half h
 // holds channels 4h .. 4h + 3 of the block, and the j-th of four matrix instructions multiplies channels j and 4 + j);
-// otherwise bf16 input on v_mfma_f32_32x32x16_bf16 (a k step is 16 channels of one tap).
-template <bool F32_IN, bool OUT_BF16, bool RELU>
+// otherwise bf16 input on v_mfma_f32_32x32x16_bf16 (a k step is 16 channels of one tap). POOL: the tile leaves through a
+// 2 x 2 / stride 2 max-pool (its rows are whole and even in number, so every window lies inside it): y is
+// [N, Cout, H / 2, W / 2] and the full-size result never reaches memory.
+template <bool F32_IN, bool OUT_BF16, bool RELU, bool POOL>
 __global__ __launch_bounds__(256, 1) void conv3x3_k(const void *__restrict__ x_, const void *__restrict__ wt,
                                                     const void *__restrict__ bias, void *__restrict__ y, int C, int H, int W,
                                                     int Cout, int R) {
@@ -303,6 +305,47 @@ __global__ __launch_bounds__(256, 1) void conv3x3_k(const void *__restrict__ x_,
         }
         __syncthreads();
         constexpr int ROWS = OUT_BF16 ? 128 : 64;
+        if constexpr (POOL) {
+            // a channel's pooled tile is (R / 2) x (W / 2) = 112 values, consecutive in the pooled plane; a thread makes
+            // 16 bytes of them. The running maximum starts at the dtype's lowest finite value and takes the window in
+            // row order, like the separate pooling kernel.
+            constexpr int PV = TILE_PIX / 4, VPC = 16 / ES, PCR = PV / VPC;
+            const int W2 = W >> 1;
+            const float inv_w2 = 1.0f / (float)W2;
+            const float lowest = OUT_BF16 ? -3.3895313892515355e38f : -3.4028234663852886e38f;
+            const int64_t pplane = plane >> 2;
+            uint8_t *ptile = (uint8_t *)y + (((int64_t)n * Cout + co0) * pplane + (int64_t)rb * PV) * ES;
+            for (int idx = tid; idx < ROWS * PCR; idx += 256) {
+                const int row = idx / PCR, piece = idx - row * PCR;
+                const int co = OUT_BF16 ? row : (row >> 5) * 64 + pass * 32 + (row & 31);
+                float m[VPC];
+#pragma unroll
+                for (int e = 0; e < VPC; e++) {
+                    const int q = piece * VPC + e, pr = small_div(q, inv_w2), pc = q - __mul24(pr, W2);
+                    const ZK_LDS uint8_t *src = smem + row * RS + (__mul24(2 * pr, W) + 2 * pc) * ES;
+                    float a0, a1, b0, b1;
+                    if (OUT_BF16) {
+                        const uint32_t u0 = *(const ZK_LDS uint32_t *)src, u1 = *(const ZK_LDS uint32_t *)(src + W * ES);
+                        a0 = __uint_as_float(u0 << 16), a1 = __uint_as_float(u0 & 0xffff0000u);
+                        b0 = __uint_as_float(u1 << 16), b1 = __uint_as_float(u1 & 0xffff0000u);
+                    } else {
+                        const u32x2 u0 = *(const ZK_LDS u32x2 *)src, u1 = *(const ZK_LDS u32x2 *)(src + W * ES);
+                        a0 = __uint_as_float(u0[0]), a1 = __uint_as_float(u0[1]), b0 = __uint_as_float(u1[0]), b1 = __uint_as_float(u1[1]);
+                    }
+                    m[e] = fmaxf(b1, fmaxf(b0, fmaxf(a1, fmaxf(a0, lowest))));
+                }
+                u32x4 v;
+                if (OUT_BF16) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = __builtin_amdgcn_perm(__float_as_uint(m[(2 * e + 1) % VPC]), __float_as_uint(m[(2 * e) % VPC]), 0x07060302u);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = __float_as_uint(m[e % VPC]);
+                }
+                *(u32x4 *)(ptile + (int64_t)co * pplane * ES + piece * 16) = v;
+            }
+            continue;
+        }
 #pragma unroll 4
         for (int idx = tid; idx < ROWS * CPR; idx += 256) {
             const int row = idx / CPR, col = idx - row * CPR;
@@ -323,6 +366,7 @@ uint64_t lds_bytes(const Conv2d &p) { // the input tile, later reused for the st
 
 bool conv3x3_direct_ok(const Conv2d &p) { // shape only: the same answer at registration and at every launch
     const int R = tile_rows(p);
+    if (p.pool && R % 2) return false; // pooling windows must not straddle two tiles
     const bool types = (p.dtype == DT_BF16 && (p.out_dtype == DT_BF16 || p.out_dtype == DT_F32)) || (p.dtype == DT_F32 && p.out_dtype == DT_F32);
     return types && p.KH == 3 && p.KW == 3 && p.sy == 1 && p.sx == 1 && p.dy == 1 && p.dx == 1 && p.py == 1 && p.px == 1 && p.C >= 16 &&
            p.C % 16 == 0 && p.Cout % TILE_CO == 0 && p.W % 8 == 0 && R >= 1 && p.H % R == 0 && lds_bytes(p) <= 160 * 1024 && p.N > 0 &&
@@ -335,9 +379,10 @@ uint64_t conv3x3_scratch_bytes(const Conv2d &p) { return (uint64_t)9 * p.C * p.C
 hipError_t conv3x3_init() {
     // the input tile is larger than the default per-workgroup LDS limit
     hipError_t e = hipSuccess;
-    const void *variants[6] = {(const void *)conv3x3_k<false, false, false>, (const void *)conv3x3_k<false, false, true>,
-                               (const void *)conv3x3_k<false, true, false>,  (const void *)conv3x3_k<false, true, true>,
-                               (const void *)conv3x3_k<true, false, false>,  (const void *)conv3x3_k<true, false, true>};
+#define ZK_V(FI, OB) (const void *)conv3x3_k<FI, OB, false, false>, (const void *)conv3x3_k<FI, OB, true, false>, \
+                     (const void *)conv3x3_k<FI, OB, false, true>, (const void *)conv3x3_k<FI, OB, true, true>
+    const void *variants[12] = {ZK_V(false, false), ZK_V(false, true), ZK_V(true, false)};
+#undef ZK_V
     for (const void *f : variants)
         if (e == hipSuccess) e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     return e;
@@ -352,19 +397,20 @@ hipError_t conv3x3_direct(const Conv2d &p, void *wt, hipStream_t st) {
     else hipLaunchKernelGGL((conv3x3_weights_k<uint16_t, 4>), wgrid, dim3(256), 0, st, (const uint16_t *)p.w, (uint16_t *)wt, p.C, p.Cout);
     dim3 grid((unsigned)(p.N * (p.H / R)), (unsigned)(p.Cout / TILE_CO));
     const bool out_bf16 = p.out_dtype == DT_BF16;
-#define ZK_LAUNCH(FI, OB, RL)                                                                                                     \
-    hipLaunchKernelGGL((conv3x3_k<FI, OB, RL>), grid, dim3(256), lds_bytes(p), st, p.x, (const void *)wt, p.bias, p.y, p.C, p.H, p.W, \
-                       p.Cout, R)
-    if (p.dtype == DT_F32) {
-        if (p.relu) ZK_LAUNCH(true, false, true);
-        else ZK_LAUNCH(true, false, false);
-    } else if (out_bf16) {
-        if (p.relu) ZK_LAUNCH(false, true, true);
-        else ZK_LAUNCH(false, true, false);
-    } else {
-        if (p.relu) ZK_LAUNCH(false, false, true);
-        else ZK_LAUNCH(false, false, false);
-    }
+#define ZK_LAUNCH(FI, OB, RL, PL)                                                                                                 \
+    hipLaunchKernelGGL((conv3x3_k<FI, OB, RL, PL>), grid, dim3(256), lds_bytes(p), st, p.x, (const void *)wt, p.bias, p.y, p.C, p.H, \
+                       p.W, p.Cout, R)
+#define ZK_LAUNCH2(FI, OB)                                                                                                        \
+    do {                                                                                                                          \
+        if (p.relu && p.pool) ZK_LAUNCH(FI, OB, true, true);                                                                      \
+        else if (p.relu) ZK_LAUNCH(FI, OB, true, false);                                                                          \
+        else if (p.pool) ZK_LAUNCH(FI, OB, false, true);                                                                          \
+        else ZK_LAUNCH(FI, OB, false, false);                                                                                     \
+    } while (0)
+    if (p.dtype == DT_F32) ZK_LAUNCH2(true, false);
+    else if (out_bf16) ZK_LAUNCH2(false, true);
+    else ZK_LAUNCH2(false, false);
+#undef ZK_LAUNCH2
 #undef ZK_LAUNCH
     return hipGetLastError();
 }

@@ -140,6 +140,7 @@ struct Conv2d {
     int N, C, H, W, Cout, KH, KW, OH, OW;
     int sy, sx, py, px, dy, dx;
     int dtype, out_dtype, relu;
+    int pool; // 1: y is the 2 x 2 / stride 2 max-pool of the (activated) result; only the direct 3 x 3 kernel does this
     const void *x, *w, *bias;
     void *y;
     const int32_t *koff, *kdyx;

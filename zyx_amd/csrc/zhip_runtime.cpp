@@ -295,7 +295,7 @@ zk::Conv2d conv_args(const zhip_kernel_desc &d) {
     a.sy = d.iparams[0]; a.sx = d.iparams[1]; a.py = d.iparams[2]; a.px = d.iparams[3]; a.dy = d.iparams[4]; a.dx = d.iparams[5];
     a.OH = (a.H + 2 * a.py - a.dy * (a.KH - 1) - 1) / a.sy + 1;
     a.OW = (a.W + 2 * a.px - a.dx * (a.KW - 1) - 1) / a.sx + 1;
-    a.dtype = d.dtype; a.out_dtype = d.out_dtype; a.relu = d.iparams[7];
+    a.dtype = d.dtype; a.out_dtype = d.out_dtype; a.relu = d.iparams[7]; a.pool = d.iparams[8];
     return a;
 }
 // the two int32 tap tables at the head of a conv program's workspace, rounded so what follows stays aligned
@@ -542,6 +542,11 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         if (d.iparams[6]) p.need[a++] = (uint64_t)Co * e;
         p.n_in = a;
         p.need[a] = (uint64_t)N * Co * OH * OW * dtype_bytes(d.out_dtype);
+        if (d.iparams[8]) { // fused 2 x 2 / stride 2 max-pool: the direct 3 x 3 kernel's shapes with an even number of rows per tile
+            if (d.iparams[8] != 1 || !zk::conv3x3_direct_ok(conv_args(d)))
+                return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: the fused 2x2 max-pool needs a 3x3 / stride 1 / padding 1 shape of the direct kernel (C a multiple of 16, Cout of 128, W of 8 and a divisor of 224, H a multiple of 448 / W)");
+            p.need[a] = (uint64_t)N * Co * (OH / 2) * (OW / 2) * dtype_bytes(d.out_dtype);
+        }
         p.n_out = 1;
         // two int32 tables filled at registration, then (bf16 shapes that run on the tiled GEMM) a zero bias
         // and the patch matrix

@@ -323,12 +323,14 @@ def conv_out(size: int, k: int, stride: int, pad: int, dil: int) -> int:
 
 
 def conv2d_desc(n, c, h, w, cout, kh, kw, stride=(1, 1), padding=(0, 0), dilation=(1, 1), bias=False, relu=False,
-                dtype: DType = DType.F32, out_dtype: DType | None = None) -> KernelDesc:
+                dtype: DType = DType.F32, out_dtype: DType | None = None, pool=False) -> KernelDesc:
+    """pool: the launch also applies max_pool([2, 2]) and writes only the pooled [n, cout, oh / 2, ow / 2] result
+    (shapes of the direct 3 x 3 kernel; registration refuses others)."""
     d = KernelDesc()
     d.kind, d.dtype, d.out_dtype = K_CONV2D, DType(dtype), DType(dtype if out_dtype is None else out_dtype)
     for i, v in enumerate((n, c, h, w, cout, kh, kw)):
         d.dims[i] = v
-    for i, v in enumerate((stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1], int(bias), int(relu))):
+    for i, v in enumerate((stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1], int(bias), int(relu), int(pool))):
         d.iparams[i] = v
     return d
 
@@ -345,9 +347,10 @@ def max_pool2d_desc(planes, h, w, kernel=(2, 2), stride=(2, 2), padding=(0, 0), 
 
 
 def conv2d(dev: HIPDevice, pool: HIPMemoryPool, x, w, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
-           relu=False, dtype: DType = DType.F32, out_dtype: DType | None = None, pool_kernel=None):
+           relu=False, dtype: DType = DType.F32, out_dtype: DType | None = None, pool_kernel=None, fused_pool=False):
     """Conv2d::forward (+ ReLU) and optionally max_pool(pool_kernel, stride = kernel) as two launches whose
-    second waits on the first's event. Returns y, or (y, pooled)."""
+    second waits on the first's event. Returns y, or (y, pooled). fused_pool: one launch that returns only the
+    2 x 2 pooled result."""
     st = _NP_STORE[DType(dtype)]
     out_dtype = DType(dtype if out_dtype is None else out_dtype)
     x, w = np.ascontiguousarray(x, st), np.ascontiguousarray(w, st)
@@ -355,7 +358,9 @@ def conv2d(dev: HIPDevice, pool: HIPMemoryPool, x, w, bias=None, stride=(1, 1), 
     co, _, kh, kw = w.shape
     oh, ow = conv_out(h, kh, stride[0], padding[0], dilation[0]), conv_out(wd, kw, stride[1], padding[1], dilation[1])
     prog = dev.register_kernel(conv2d_desc(n, c, h, wd, co, kh, kw, stride, padding, dilation, bias is not None, relu,
-                                           dtype, out_dtype))
+                                           dtype, out_dtype, pool=fused_pool))
+    if fused_pool:
+        oh, ow = oh // 2, ow // 2
     bufs, waits = [], []
     for arr in (x, w) + ((np.ascontiguousarray(bias, st),) if bias is not None else ()):
         bb, e = to_device(pool, arr)
