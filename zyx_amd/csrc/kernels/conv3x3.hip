@@ -319,10 +319,15 @@ __global__ __launch_bounds__(256, 1) void conv3x3_k(const void *__restrict__ x_,
                 const int row = idx / PCR, piece = idx - row * PCR;
                 const int co = OUT_BF16 ? row : (row >> 5) * 64 + pass * 32 + (row & 31);
                 float m[VPC];
+                int pr = small_div(piece * VPC, inv_w2), pc = piece * VPC - __mul24(pr, W2); // pooled row, column of value 0
+                const ZK_LDS uint8_t *rowp = smem + row * RS + __mul24(2 * pr, W) * ES;
 #pragma unroll
                 for (int e = 0; e < VPC; e++) {
-                    const int q = piece * VPC + e, pr = small_div(q, inv_w2), pc = q - __mul24(pr, W2);
-                    const ZK_LDS uint8_t *src = smem + row * RS + (__mul24(2 * pr, W) + 2 * pc) * ES;
+                    const ZK_LDS uint8_t *src = rowp + 2 * pc * ES;
+                    if (++pc == W2) { // the next value starts the next pooled row
+                        pc = 0;
+                        rowp += 2 * W * ES;
+                    }
                     float a0, a1, b0, b1;
                     if (OUT_BF16) {
                         const uint32_t u0 = *(const ZK_LDS uint32_t *)src, u1 = *(const ZK_LDS uint32_t *)(src + W * ES);
