@@ -1,15 +1,17 @@
-// Direct 3 x 3 convolution, bf16, unit stride, padding 1 (the convolution block of a vision network:
+// Direct 3 x 3 convolution, bf16 or f32, unit stride, padding 1 (the convolution block of a vision network:
 // Tensor::conv, zyx/src/tensor/mod.rs:2583-2680, padding rule zyx/src/kernel/linearize.rs:349-382), on the matrix
-// cores without a patch matrix, a padded copy of the input, or a second pass over it.
+// cores without a patch matrix, a padded copy of the input, or a second pass over it; optionally followed by the
+// block's 2 x 2 max-pool (Tensor::max_pool, mod.rs:2706-2741) before anything is written. Described for bf16; the f32
+// differences are at the kernel.
 //
 // A workgroup owns R whole output rows of one image (R * W = 448 pixels = 14 MFMA blocks of 32) and 128 output
 // channels. It copies the R + 2 input rows of all C channels into LDS once, channel-innermost ([row][col][C], borders
-// zero), so that the nine taps are nine shifted views of the same tile: the B operand of tap (ky, kx) and channel
+// zero), so that the nine taps are nine shifted views of the same tile: the input operand of tap (ky, kx) and channel
 // block cb for pixel (r, c) is the 16 bytes at [r + ky][c + kx][cb*16 + half*8], one ds_read_b128, whatever the shift
 // (the pixel stride is padded by 16 bytes, which spreads the 16 lanes of a read phase over all 64 banks). Every input
 // element is fetched once and used 9 * 128 times. The weights are re-laid once per launch by a small kernel as
-// [tap][C/16][Cout][16], so the A operand (32 output channels x 16 input channels of one tap) is 1 KiB of consecutive
-// bytes read straight from L1 / L2, one k step ahead of its use.
+// [tap][C/16][Cout][16], so the weight operand (32 output channels x 16 input channels of one tap) is 1 KiB of
+// consecutive bytes read straight from L1 / L2, two k steps ahead of its use.
 //
 // 4 waves as 2 (pixel halves) x 2 (channel halves), 2 x 7 accumulator tiles of 32 x 32 each = 224 registers, which start
 // at the bias. In a tile a lane owns one output channel and 16 pixels in runs of four. The epilogue stages the finished

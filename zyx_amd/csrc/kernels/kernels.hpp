@@ -148,7 +148,7 @@ struct Conv2d {
 };
 uint64_t conv2d_scratch_bytes(const Conv2d &p);
 hipError_t conv2d(const Conv2d &p, hipStream_t stream);
-// Direct 3 x 3 / stride 1 / padding 1 bf16 convolution (conv3x3.hip): shapes it takes, bytes for its re-laid weights,
+// Direct 3 x 3 / stride 1 / padding 1 convolution, bf16 or f32, optional fused 2 x 2 max-pool (conv3x3.hip): shapes it takes, bytes for its re-laid weights,
 // one-time set-up of the kernel's LDS limit, launch.
 bool conv3x3_direct_ok(const Conv2d &p);
 uint64_t conv3x3_scratch_bytes(const Conv2d &p);
