@@ -378,7 +378,8 @@ bool conv3x3_direct_ok(const Conv2d &p) { // shape only: the same answer at regi
     return types && p.KH == 3 && p.KW == 3 && p.sy == 1 && p.sx == 1 && p.dy == 1 && p.dx == 1 && p.py == 1 && p.px == 1 && p.C >= 16 &&
            p.C % 16 == 0 && p.Cout % TILE_CO == 0 && p.W % 8 == 0 && R >= 1 && p.H % R == 0 && lds_bytes(p) <= 160 * 1024 && p.N > 0 &&
            (int64_t)p.N * (p.H / R) < (1ll << 31) && p.Cout / TILE_CO <= 65535 && (int64_t)p.N * p.C * p.H * p.W < (1ll << 31) &&
-           (int64_t)p.N * p.Cout * p.H * p.W < (1ll << 40) && (int64_t)p.C * p.Cout < (1ll << 26);
+           (int64_t)p.N * p.Cout * p.H * p.W < (1ll << 40) && (int64_t)p.C * p.Cout < (1ll << 26) &&
+           p.H < (1 << 22); // row numbers go through 24-bit multiplies
 }
 
 uint64_t conv3x3_scratch_bytes(const Conv2d &p) { return (uint64_t)9 * p.C * p.Cout * elem_bytes(p); }
