@@ -124,13 +124,18 @@ __global__ __launch_bounds__(256) void softmax_rows_generic_k(const float *__res
 
 template <int NV> static hipError_t launch_wave(const SoftmaxRows &p, hipStream_t st) {
     dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
+    // Rows of 16 vectors per lane on a grid of several rounds: an unused LDS request holds a compute unit at 3 workgroups
+    // (12 waves) instead of 8, so that the rounds overlap and one round's stores run beside the next one's loads; with
+    // every wave resident at once all of them load, then all of them store (measured 47.8 against 48.0 us at
+    // 8192 x 4096; 2, 4, 5, 6 and 8 workgroups per unit were all slower than 3).
+    const unsigned lds_pad = (NV == 16 && grid.x >= 1536) ? 54000u : 0u;
     int rows = (int)p.rows, cols = (int)p.cols;
     int sel = (p.y ? 1 : 0) | (p.rowsum ? 2 : 0) | (p.arg ? 4 : 0);
     bool full = p.cols == 256 * NV;
 #define ZK_CASE(S, A, B, C)                                                                                           \
     case S:                                                                                                           \
         if (full)                                                                                                     \
-            hipLaunchKernelGGL((softmax_rows_wave_k<NV, true, A, B, C>), grid, block, 0, st, p.x, p.y, p.rowsum,     \
+            hipLaunchKernelGGL((softmax_rows_wave_k<NV, true, A, B, C>), grid, block, lds_pad, st, p.x, p.y, p.rowsum,     \
                                p.arg, rows, cols);                                                                    \
         else                                                                                                          \
             hipLaunchKernelGGL((softmax_rows_wave_k<NV, false, A, B, C>), grid, block, 0, st, p.x, p.y, p.rowsum,    \
