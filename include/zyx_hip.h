@@ -436,6 +436,22 @@ int32_t zhip_time_kernel(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args, si
 int32_t zhip_profile_kernel(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args, size_t n_args, size_t arg_sets,
                             int32_t iters, float *avg_us);
 
+/* No counterpart in the reference: an entry point for callers that cannot allocate device memory -- code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. It is the ZHIP_K_REDUCE kernel pair
+ * (sum: op = 0, max: op = 1; over the last axis: axis0 = 0, over axis 0: axis0 = 1; dtype F32 / BF16 / F16 / I32,
+ * no scale / base epilogue) on raw device pointers x[rows, cols] -> out[rows] or out[cols], enqueued on the
+ * caller's `stream` (a hipStream_t, NULL = the null stream) of ctx's device; asynchronous, the caller orders it
+ * against its other work. The partial results of the two-stage variants go to a 1 MiB array that is part of the
+ * library's code object (one copy per GPU, held until the process ends) instead of a per-program allocation:
+ * no hipMalloc, hipFree or other allocating routine is called. A shape whose partials need more than 1 MiB is
+ * refused with ZHIP_KERNEL_COMPILATION and the needed size in zhip_last_error (register the kernel instead).
+ * Results are bit-identical to a ZHIP_K_REDUCE program launched with zhip_launch on the same data. All calls on one
+ * GPU share the array: calls that overlap in time on one GPU (different streams, different contexts) race on it,
+ * so the caller keeps them in one stream or orders them; nothing in it has to be cleared between calls (every
+ * partial a call reads it has written itself). */
+int32_t zhip_reduce_static(zhip_ctx *ctx, int32_t dtype, int32_t op, int32_t axis0, int64_t rows, int64_t cols,
+                           const void *x, void *out, void *stream);
+
 /* --- cached execution plans ----------------------------------------------------- */
 
 /* The steady state of Tape::realize / FrozenTape::replay is a fixed list of Launch nodes on

@@ -131,7 +131,7 @@ _EXPORTS = ["zhip_device_count", "zhip_init", "zhip_deinit", "zhip_last_error", 
             "zhip_get_variable", "zhip_h2d", "zhip_d2h", "zhip_d2d", "zhip_sync_events", "zhip_release_events",
             "zhip_buffer_ptr", "zhip_register_kernel", "zhip_compile_ir", "zhip_ir_generate", "zhip_program_source", "zhip_launch",
             "zhip_release_program",
-            "zhip_time_kernel", "zhip_profile_kernel", "zhip_plan_create", "zhip_plan_launch", "zhip_plan_destroy"]
+            "zhip_reduce_static", "zhip_time_kernel", "zhip_profile_kernel", "zhip_plan_create", "zhip_plan_launch", "zhip_plan_destroy"]
 
 
 def load_library() -> C.CDLL:
@@ -354,6 +354,14 @@ class HIPDevice:
         self._ctx.check(self._ctx.lib.zhip_launch(self._ctx.ptr, C.c_uint32(program_id), a, C.c_size_t(len(args)), arr,
                                                   n, C.byref(ev)))
         return Event(ev.value)
+
+    def reduce_static(self, dtype: DType, op: int, axis0: bool, rows: int, cols: int, x_ptr: int, out_ptr: int,
+                      stream: int = 0):
+        """zhip_reduce_static: sum (op 0) / max (op 1) of x[rows, cols] given as raw device addresses, enqueued on the
+        caller's hipStream_t (0 = null stream) without any device allocation; asynchronous."""
+        self._ctx.check(self._ctx.lib.zhip_reduce_static(self._ctx.ptr, C.c_int32(int(dtype)), C.c_int32(op),
+                                                         C.c_int32(int(bool(axis0))), C.c_int64(rows), C.c_int64(cols),
+                                                         C.c_void_p(x_ptr), C.c_void_p(out_ptr), C.c_void_p(stream)))
 
     def release(self, program_id: int):
         self._ctx.check(self._ctx.lib.zhip_release_program(self._ctx.ptr, C.c_uint32(program_id)))

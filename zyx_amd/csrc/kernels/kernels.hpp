@@ -52,6 +52,8 @@ struct Reduce {
     float mul = 0.0f, div = 0.0f;   // float dtypes: out = (reduce * mul) / div + base, a 0 / null step is left out
     const void *base = nullptr;     // [len(out)] of the same dtype
 };
+// rows * cols below 2^40 elements and every grid dimension of the launches within 32 bits
+bool reduce_shape_ok(int64_t rows, int64_t cols, int axis0);
 uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int axis0);
 hipError_t reduce(const Reduce &p, hipStream_t stream);
 

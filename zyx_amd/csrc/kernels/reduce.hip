@@ -288,6 +288,13 @@ template <int DT, int OP> hipError_t launch(const Reduce &p, hipStream_t st) {
 
 } // namespace
 
+bool reduce_shape_ok(int64_t rows, int64_t cols, int axis0) {
+    if (rows < 0 || cols < 0 || (cols && rows > (1ll << 40) / cols)) return false;
+    if (rows == 0 || cols == 0) return (axis0 ? cols : rows) < (1ll << 33); // the fill of an empty reduce: 4 results per workgroup
+    if (!axis0) return rows * plan_rows(rows, cols).segs < (1ll << 33); // 4 (row, segment) items per workgroup, grid.x < 2^31
+    return (cols + 63) / 64 < (1ll << 31); // column strips along grid.x; chunks <= 4096 along grid.y
+}
+
 uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int axis0) {
     if (rows <= 0 || cols <= 0) return 0;
     if (!axis0) {

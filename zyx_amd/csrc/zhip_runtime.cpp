@@ -41,6 +41,7 @@ constexpr int kLaunchStreams = 8; // zyx/src/backend/hip.rs:242-274
 constexpr int kMaxArgs = ZHIP_IR_MAX_PARAMS; // arguments of one launch (hand-written kernels take at most 8)
 constexpr uint64_t kDefaultCacheBytes = 1ull << 30;
 constexpr uint64_t kAllocAlign = 256;
+constexpr uint64_t kStaticScratchBytes = 1ull << 20;
 
 thread_local std::string g_init_error;
 
@@ -118,6 +119,11 @@ template <class T> struct Slab { // dense ids, lowest free id reused (zyx/src/sl
 
 } // namespace
 
+// Partial results of zhip_reduce_static: device memory that exists from the moment the code object is loaded,
+// one copy per GPU, so that entry point never allocates. In host code the name only stands for the symbol;
+// its device address is looked up once per context (zhip_init) and kept in zhip_ctx::static_scratch.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 struct zhip_ctx {
     std::mutex mu;
     int device = 0;
@@ -143,6 +149,7 @@ struct zhip_ctx {
     hipStream_t plan_stream = nullptr; // plans are captured on and replayed into this stream
     hipEvent_t plan_done = nullptr;    // recorded after every plan launch that uses program scratch: one record for all of them
     hipEvent_t prof_a = nullptr, prof_b = nullptr;
+    void *static_scratch = nullptr; // this device's copy of `scratch`
 
     int32_t fail(int32_t status, const char *fmt, ...) __attribute__((format(printf, 3, 4))) {
         char buf[512];
@@ -423,7 +430,7 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
     }
     case ZHIP_K_REDUCE: {
         int64_t rows = d.dims[0], cols = d.dims[1];
-        if (rows < 0 || cols < 0 || (cols && rows > (1ll << 40) / cols))
+        if (!zk::reduce_shape_ok(rows, cols, d.flags & 1))
             return c->fail(ZHIP_KERNEL_COMPILATION, "reduce: rows/cols out of range");
         if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16 && d.dtype != ZHIP_F16 && d.dtype != ZHIP_I32)
             return c->fail(ZHIP_KERNEL_COMPILATION, "reduce: dtype %d not implemented", d.dtype);
@@ -999,6 +1006,8 @@ ZHIP_EXPORT int32_t zhip_init(const zhip_config *cfg, zhip_ctx **out) {
     if ((e = hipEventCreate(&c->prof_a)) != hipSuccess || (e = hipEventCreate(&c->prof_b)) != hipSuccess ||
         (e = hipEventCreateWithFlags(&c->plan_done, hipEventDisableTiming)) != hipSuccess)
         return bail(ZHIP_INITIALIZATION, "hipEventCreate", e);
+    if ((e = hipGetSymbolAddress((void **)&c->static_scratch, HIP_SYMBOL(scratch))) != hipSuccess || !c->static_scratch)
+        return bail(ZHIP_INITIALIZATION, "hipGetSymbolAddress of the static scratch array", e);
     if ((e = zk::gemm_bf16_init()) != hipSuccess) return bail(ZHIP_INITIALIZATION, "raising the LDS limit of the GEMM kernels", e);
     if ((e = zk::conv3x3_init()) != hipSuccess) return bail(ZHIP_INITIALIZATION, "raising the LDS limit of the convolution kernel", e);
     fill_info(c);
@@ -1401,6 +1410,38 @@ ZHIP_EXPORT int32_t zhip_launch(zhip_ctx *c, zhip_prog prog, const zhip_buf *arg
         p->ws_last = 1;
     }
     return event_record(c, si, ZHIP_KERNEL_LAUNCH, ev);
+}
+
+ZHIP_EXPORT int32_t zhip_reduce_static(zhip_ctx *c, int32_t dtype, int32_t op, int32_t axis0, int64_t rows, int64_t cols,
+                                       const void *x, void *out, void *stream) {
+    if (!c) return ZHIP_KERNEL_LAUNCH;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (dtype != ZHIP_F32 && dtype != ZHIP_BF16 && dtype != ZHIP_F16 && dtype != ZHIP_I32)
+        return c->fail(ZHIP_KERNEL_COMPILATION, "reduce_static: dtype %d not implemented", dtype);
+    if ((op != 0 && op != 1) || (axis0 != 0 && axis0 != 1)) return c->fail(ZHIP_KERNEL_COMPILATION, "reduce_static: bad op/axis");
+    if (!zk::reduce_shape_ok(rows, cols, axis0)) return c->fail(ZHIP_KERNEL_COMPILATION, "reduce_static: rows/cols out of range");
+    const uint64_t need = zk::reduce_workspace_bytes(rows, cols, axis0);
+    if (need > kStaticScratchBytes)
+        return c->fail(ZHIP_KERNEL_COMPILATION,
+                       "reduce_static: a %lld x %lld reduce over axis %d needs %llu bytes of partial results, the static "
+                       "scratch holds %llu; use zhip_register_kernel + zhip_launch for this shape",
+                       (long long)rows, (long long)cols, axis0 ? 0 : 1, (unsigned long long)need, (unsigned long long)kStaticScratchBytes);
+    const int64_t n_in = rows * cols, n_out = axis0 ? cols : rows;
+    if ((n_in && !x) || (n_out && !out)) return c->fail(ZHIP_INCORRECT_KERNEL_ARG, "reduce_static: null device pointer");
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
+    zk::Reduce a{};
+    a.rows = rows;
+    a.cols = cols;
+    a.dtype = dtype;
+    a.op = op;
+    a.axis0 = axis0;
+    a.x = x;
+    a.out = out;
+    a.workspace = c->static_scratch;
+    a.workspace_bytes = kStaticScratchBytes;
+    hipError_t e = zk::reduce(a, (hipStream_t)stream);
+    if (e != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "reduce_static: launch failed: %s", hipGetErrorString(e));
+    return ZHIP_OK;
 }
 
 ZHIP_EXPORT int32_t zhip_time_kernel(zhip_ctx *c, zhip_prog prog, const zhip_buf *args, size_t n_args, uint64_t *ns) {
