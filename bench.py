@@ -21,6 +21,8 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+from zyx_amd.rng import Rng  # zyx's own generator (zyx/src/rng.rs): every input below is drawn from it, outside the timed regions
+
 ROWS, COLS = 8192, 4096
 # x read once + y written once + rowsum and argmax written once
 ALGO_BYTES = ROWS * COLS * 4 * 2 + 2 * ROWS * 4
@@ -57,10 +59,10 @@ def cpu_baseline(x: np.ndarray, budget_s: float = 10.0):
 def extra_gemm(dev, pool, kernels, steps=100, warmup=200):
     """Config 3: bf16 4096^3 GEMM (f32 accumulate), raw and with the fused bias+GELU epilogue."""
     n = 4096
-    rng = np.random.default_rng(1)
+    rng = Rng(1)
     trunc = lambda a: (a.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)  # bf16 by truncation, as zyx does
-    a, b = trunc(rng.uniform(-1, 1, (n, n))), trunc(rng.uniform(-1, 1, (n, n)))
-    bias = trunc(rng.uniform(-1 / 64, 1 / 64, n))
+    a, b = trunc(rng.uniform((n, n), -1, 1)), trunc(rng.uniform((n, n), -1, 1))
+    bias = trunc(rng.uniform(n, -1 / 64, 1 / 64))
     ab, e1 = kernels.to_device(pool, a)
     bb, e2 = kernels.to_device(pool, b)
     biasb, e3 = kernels.to_device(pool, bias)
@@ -85,11 +87,11 @@ def extra_conv(dev, pool, kernels, steps=50, warmup=50):
     import zyx_amd
     N, C, HW, CO = 32, 64, 56, 128
     flop = 2.0 * N * CO * HW * HW * C * 9
-    rng = np.random.default_rng(4)
+    rng = Rng(4)
     out = {}
     for name, dt, isz in (("f32", zyx_amd.DType.F32, 4), ("bf16", zyx_amd.DType.BF16, 2)):
-        x = rng.standard_normal((N, C, HW, HW), dtype=np.float32)
-        w = (rng.standard_normal((CO, C, 3, 3), dtype=np.float32) * np.sqrt(2.0 / 576)).astype(np.float32)
+        x = rng.randn((N, C, HW, HW))
+        w = rng.randn((CO, C, 3, 3), float(np.sqrt(2.0 / 576)))
         if isz == 2:
             x, w = [(a.view(np.uint32) >> 16).astype(np.uint16) for a in (x, w)]
         xb, e1 = kernels.to_device(pool, x)
@@ -125,11 +127,11 @@ def extra_streaming(dev, pool, kernels, steps=20, warmup=5):
     LayerNorm forward and backward. GB/s = (bytes of every input + output tensor, each once) / kernel time."""
     import zyx_amd
     M, F, D = 8192, 4096, 1024
-    rng = np.random.default_rng(3)
+    rng = Rng(3)
     out = {}
 
     def dev_arr(shape, dt):
-        a = rng.standard_normal(shape, dtype=np.float32)
+        a = rng.randn(shape)
         if dt == zyx_amd.DType.BF16:
             a = (a.view(np.uint32) >> 16).astype(np.uint16)
         b, e = kernels.to_device(pool, a)
@@ -189,13 +191,13 @@ def extra_graph(dev, pool, steps=60, warmup=10):
     B, NIN, H, NOUT, LR = 64, 784, 128, 10, 0.01
     out = {}
     for match in (False, True):
-        rng = np.random.default_rng(42069)  # the same parameters and batches for both runs
+        rng = Rng(42069)  # the same parameters and batches for both runs
         tape = Tape(dev, pool, match=match)
         g = tape.graph
         k1, k2 = 1 / np.sqrt(NIN), 1 / np.sqrt(H)
         x, onehot = tape.tensor(np.zeros((B, NIN)), F32), tape.tensor(np.zeros((B, NOUT)), F32)
-        params = [tape.tensor(rng.uniform(-k1, k1, (H, NIN)), F32), tape.tensor(rng.uniform(-k1, k1, (H,)), F32),
-                  tape.tensor(rng.uniform(-k2, k2, (NOUT, H)), F32), tape.tensor(rng.uniform(-k2, k2, (NOUT,)), F32)]
+        params = [tape.tensor(rng.uniform((H, NIN), -k1, k1), F32), tape.tensor(rng.uniform((H,), -k1, k1), F32),
+                  tape.tensor(rng.uniform((NOUT, H), -k2, k2), F32), tape.tensor(rng.uniform((NOUT,), -k2, k2), F32)]
         h = g.relu(g.binary_b(g.dot(x, g.t(params[0])), params[1], BOp.Add))
         logits = g.binary_b(g.dot(h, g.t(params[2])), params[3], BOp.Add)
         per_row = g.reduce(g.binary(g.ln_softmax(logits, [-1]), onehot, BOp.Mul), BOp.Add, [1])
@@ -205,8 +207,8 @@ def extra_graph(dev, pool, steps=60, warmup=10):
         t0 = time.perf_counter()
         plan = tape.plan(new + [loss])
         build_ms = (time.perf_counter() - t0) * 1e3
-        xs = rng.standard_normal((steps + warmup, B, NIN), dtype=np.float32)
-        hot = np.eye(NOUT, dtype=np.float32)[rng.integers(0, NOUT, (steps + warmup, B))]
+        xs = rng.randn((steps + warmup, B, NIN))
+        hot = np.eye(NOUT, dtype=np.float32)[rng.randint((steps + warmup, B), 0, NOUT)]
         for i in range(steps + warmup):
             if i == warmup:
                 tape.sync()
@@ -230,9 +232,9 @@ def extra_ir(dev, pool, kernels, steps=20, warmup=5):
     as such a kernel (row in registers, local-memory reductions) beside the hand-written one, and an elementwise map."""
     import zyx_amd
     from zyx_amd import ir_examples
-    rng = np.random.default_rng(4)
+    rng = Rng(4)
     out = {}
-    x = (rng.standard_normal((ROWS, COLS), dtype=np.float32) * 3.0).astype(np.float32)
+    x = rng.randn((ROWS, COLS), 3.0)
     sets, pending = [], []
     for _ in range(N_SETS):  # rotating buffer sets, like the headline run: no launch finds its rows in the cache
         xb, e1 = kernels.to_device(pool, x)
@@ -274,10 +276,10 @@ def extra_attention(dev, pool, kernels, steps=30, warmup=10):
     10*B*H*T*T*dh backward (5 products; the two-kernel backward recomputes QK^T and dy.V^T, not counted)."""
     import zyx_amd
     B, T, H, DH = 8, 1024, 16, 64
-    rng = np.random.default_rng(6)
+    rng = Rng(6)
     trunc = lambda a: (a.view(np.uint32) >> 16).astype(np.uint16)
-    qkv = trunc(rng.standard_normal((B, T, 3 * H * DH), dtype=np.float32))
-    dy = trunc(rng.standard_normal((B, T, H * DH), dtype=np.float32))
+    qkv = trunc(rng.randn((B, T, 3 * H * DH)))
+    dy = trunc(rng.randn((B, T, H * DH)))
     xb, e0 = kernels.to_device(pool, qkv)
     db, e1 = kernels.to_device(pool, dy)
     yb, e2 = kernels.alloc_like(pool, B * T * H * DH, 2)
@@ -311,14 +313,14 @@ def extra_block(dev, pool, steps=20, warmup=5, cpu=True):
     blk = TransformerBlock(dev, pool, B, T, D, H, zyx_amd.DType.BF16)
     trunc = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
     # config 5's parameters: Linear weights 0.02 * randn and zero biases (nanogpt.rs:121-125), LayerNorm weight 1 / bias 0
-    prng = np.random.default_rng(42069)
-    w = lambda *shape: (0.02 * prng.standard_normal(shape)).astype(np.float32)
+    prng = Rng(42069)
+    w = lambda *shape: prng.randn(shape, 0.02)
     z = lambda n: np.zeros(n, np.float32)
     params = dict(ln1_w=np.ones(D, np.float32), ln1_b=z(D), attn_w=w(3 * D, D), attn_b=z(3 * D), proj_w=w(D, D), proj_b=z(D),
                   ln2_w=np.ones(D, np.float32), ln2_b=z(D), fc_w=w(4 * D, D), fc_b=z(4 * D), proj2_w=w(D, 4 * D), proj2_b=z(D))
     blk.set_params({k: trunc(v) for k, v in params.items()})
-    rng = np.random.default_rng(5)
-    x = rng.standard_normal((B * T, D), dtype=np.float32)
+    rng = Rng(5)
+    x = rng.randn((B * T, D))
     blk.write("x", trunc(x))
     blk.write("dout", trunc(np.ones((B * T, D), np.float32)))
     res = {"kernels_forward": len(blk.forward_nodes), "kernels_forward_backward": len(blk.forward_nodes) + len(blk.backward_nodes)}
@@ -337,7 +339,7 @@ def extra_block(dev, pool, steps=20, warmup=5, cpu=True):
     if cpu:
         import oracle  # the CPU comparison leg only
         # one attention head pair and 64 rows of each Linear on the host cores, scaled to the whole forward
-        sub = trunc(rng.standard_normal((1, T, 3 * 128), dtype=np.float32))
+        sub = trunc(rng.randn((1, T, 3 * 128)))
         t0 = time.perf_counter()
         oracle.attention(sub, 2, dtype=oracle.BF16)
         t_att = (time.perf_counter() - t0) * (B * H / 2)
@@ -345,7 +347,7 @@ def extra_block(dev, pool, steps=20, warmup=5, cpu=True):
         t0 = time.perf_counter()
         for w in ("attn_w", "proj_w", "fc_w"):
             oracle.linear(rows, trunc(params[w]), dtype=oracle.BF16)
-        oracle.linear(trunc(rng.standard_normal((64, 4 * D), dtype=np.float32)), trunc(params["proj2_w"]), dtype=oracle.BF16)
+        oracle.linear(trunc(rng.randn((64, 4 * D))), trunc(params["proj2_w"]), dtype=oracle.BF16)
         t_lin = (time.perf_counter() - t0) * (B * T / 64)
         res["cpu_oracle_forward_s_extrapolated"] = round(t_att + t_lin, 2)
         res["cpu_sample"] = "2 of 128 (batch, head) attention problems and 64 of 8192 rows of the four Linear layers"
@@ -364,12 +366,12 @@ def extra_mlp(dev, pool, steps=100, cpu=True):
     cross-entropy launch, the ReLU gradient in the epilogue of the product that feeds it)."""
     from zyx_amd.training import MLPTrainStep
     B, NIN, H, NOUT, LR = 64, 784, 128, 10, 0.01
-    rng = np.random.default_rng(42069)
+    rng = Rng(42069)
     k1, k2 = 1 / np.sqrt(NIN), 1 / np.sqrt(H)
-    w1, b1 = rng.uniform(-k1, k1, (H, NIN)).astype(np.float32), rng.uniform(-k1, k1, H).astype(np.float32)
-    w2, b2 = rng.uniform(-k2, k2, (NOUT, H)).astype(np.float32), rng.uniform(-k2, k2, NOUT).astype(np.float32)
-    xs = rng.standard_normal((steps, B, NIN), dtype=np.float32)
-    ys = rng.integers(0, NOUT, (steps, B)).astype(np.int32)
+    w1, b1 = rng.uniform((H, NIN), -k1, k1), rng.uniform(H, -k1, k1)
+    w2, b2 = rng.uniform((NOUT, H), -k2, k2), rng.uniform(NOUT, -k2, k2)
+    xs = rng.randn((steps, B, NIN))
+    ys = rng.randint((steps, B), 0, NOUT)
     m = MLPTrainStep(dev, pool, B, NIN, H, NOUT, LR, fused_update=True)
     m.set_params(w1, b1, w2, b2)
     from zyx_amd import kernels as K
@@ -460,8 +462,8 @@ def main():
         pool.deinitialize()
         return
 
-    rng = np.random.default_rng(42069)
-    x = (rng.standard_normal((ROWS, COLS), dtype=np.float32) * 3.0).astype(np.float32)
+    rng = Rng(42069)
+    x = rng.randn((ROWS, COLS), 3.0)
 
     prog = dev.register_kernel(kernels.softmax_rows_desc(ROWS, COLS))
     sets, pending = [], []
