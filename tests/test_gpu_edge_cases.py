@@ -114,3 +114,15 @@ def test_shapes_whose_byte_counts_would_overflow_are_refused(hip):
         e = KernelDesc.from_buffer_copy(bytes(d))
         e.dims[idx] = val
         refused(e)
+    # padding / dilation / stride near 2^31 must be refused, not wrap the output-size arithmetic
+    for ip, val in ((2, (1 << 31) - 1), (3, 1 << 30), (4, 1 << 30), (0, 1 << 30)):
+        e = K.conv2d_desc(1, 3, 8, 8, 4, 3, 3)
+        e.iparams[ip] = val
+        refused(e)
+        e = K.max_pool2d_desc(4, 8, 8)
+        e.iparams[ip] = val
+        refused(e)
+    # a last-axis reduce with more (row, segment) items than a 32-bit grid of 4-item workgroups holds
+    refused(K.reduce_desc(1 << 34, 1, "sum"))
+    refused(K.reduce_desc(1 << 34, 0, "sum"))
+    dev.release(dev.register_kernel(K.reduce_desc(1 << 32, 1, "sum")))  # 2^30 workgroups: fits

@@ -334,3 +334,35 @@ def test_long_reductions_run_on_the_reduce_kernel(hip):
         assert np.array_equal(tape.numpy(mx), leaves[x].max((1, 2))) and np.array_equal(tape.numpy(cs), leaves[y].sum(0, dtype=np.int32))
     finally:
         tape.close()
+
+
+def test_launch_chain_survives_a_write_to_an_unrelated_leaf(hip):
+    """realize -> write of a leaf the next kernel does not read -> realize of a dependant of the first result: the
+    second launch must still be ordered after the first (the chain continues in the copy's event). A long serial
+    reduce makes the first kernel slow enough that an unordered second launch would read unfinished data."""
+    dev, pool = hip
+    tape = Tape(dev, pool)
+    try:
+        g = tape.graph
+        n = 1 << 22
+        xa = np.arange(n, dtype=np.int32).reshape(4, n // 4) % 1000
+        x = tape.tensor(xa, DType.I32)
+        other = tape.tensor(np.zeros(16, np.int32), DType.I32)
+        other2 = tape.tensor(np.zeros(16, np.int32), DType.I32)
+        keep = g.binary(other, g.const(0, DType.I32), BOp.Add)
+        tape.realize([keep])
+        for rep in range(3):
+            a = g.reduce(g.binary(x, g.const(rep, DType.I32), BOp.Add), BOp.Add, [1])   # 4 serial sums of a million terms each
+            base = (xa + rep).sum(1, dtype=np.int32)
+            tape.realize([a])
+            tape.write(other, np.full(16, rep, np.int32))     # pool-stream copy between the two launches
+            b = g.binary(a, g.const(2 + rep, DType.I32), BOp.Mul)
+            tape.realize([b])
+            tape.assign(other2, keep)                          # a device-side copy between the next two
+            c = g.binary(b, g.const(1, DType.I32), BOp.Add)
+            tape.realize([c])
+            assert np.array_equal(tape.numpy(c), base * (2 + rep) + 1)
+            assert np.array_equal(tape.numpy(b), base * (2 + rep))
+        assert tape.numpy(other).tolist() == [2] * 16
+    finally:
+        tape.close()

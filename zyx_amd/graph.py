@@ -842,9 +842,12 @@ class Tape:
                 prog = self._programs[kern.image] = self.dev.compile(kern.image)
             if kern.output not in self._buf:
                 self._alloc(kern.output)
-            # A launch consumes the events it waits for. Every launch waits for the one before it, so a buffer whose
-            # event an earlier launch consumed is ready for all later ones too.
-            waits = [self._ev.pop(i) for i in kern.inputs + [kern.output] if i in self._ev]
+            # A launch consumes the events it waits for, and it waits for everything outstanding: the launch before it
+            # and every upload, copy or allocation whose event nobody has consumed yet (after `write` / `assign` the
+            # chain of launches continues in such an event, not in `_last`). The launches thus form one chain, and a
+            # buffer whose event an earlier launch consumed is ready for all later ones too.
+            waits = list(self._ev.values())
+            self._ev.clear()
             if self._last is not None:
                 waits.append(self._last)
             self._last = self.dev.launch(prog, self.pool, [self._buf[i] for i in kern.inputs] + [self._buf[kern.output]], waits)

@@ -23,9 +23,12 @@ def softmax_rows_desc(rows: int, cols: int, y=True, rowsum=True, argmax=True) ->
 def to_device(pool: HIPMemoryPool, array: np.ndarray):
     """`Runtime::new_tensor`-style upload: allocate bytes + one trash element, async copy.
     Returns (buffer id, event); `array` must outlive the event."""
-    array = np.ascontiguousarray(array)
-    buf, ev = pool.allocate(array.nbytes + array.itemsize)
-    ev2 = pool.host_to_pool(array, buf, [ev])
+    src = np.ascontiguousarray(array)
+    buf, ev = pool.allocate(src.nbytes + src.itemsize)
+    ev2 = pool.host_to_pool(src, buf, [ev])
+    if src is not array:  # a contiguous copy was made: only this frame keeps it alive, so the copy finishes here
+        pool.sync_events([ev2])
+        ev2 = Event(0)
     return buf, ev2
 
 
@@ -190,6 +193,38 @@ def reduce(dev: HIPDevice, pool: HIPMemoryPool, x: np.ndarray, op: str = "sum", 
         pool.deallocate(buf, [])
     dev.release(prog)
     return res
+
+
+K_ARGMAX = 13
+
+
+def argmax_desc(outer: int, n: int, inner: int, dtype: DType = DType.F32) -> KernelDesc:
+    """Tensor::argmax_axis over the middle axis of a dense [outer, n, inner] view; args: x, out (i32)."""
+    d = KernelDesc()
+    d.kind, d.dtype, d.out_dtype = K_ARGMAX, DType(dtype), DType.I32
+    d.dims[0], d.dims[1], d.dims[2] = outer, n, inner
+    return d
+
+
+def argmax_axis(dev: HIPDevice, pool: HIPMemoryPool, x: np.ndarray, axis: int, dtype: DType = DType.F32) -> np.ndarray:
+    """x.argmax_axis(axis) (zyx/src/tensor/mod.rs:2238-2243); `x` holds the storage values of `dtype`."""
+    x = np.ascontiguousarray(x, _NP_STORE[DType(dtype)])
+    axis = axis % x.ndim
+    outer, n, inner = int(np.prod(x.shape[:axis], dtype=np.int64)), x.shape[axis], int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    prog = dev.register_kernel(argmax_desc(outer, n, inner, dtype))
+    xb, e0 = to_device(pool, x)
+    ob, e1 = alloc_like(pool, outer * inner, 4)
+    done = dev.launch(prog, pool, [xb, ob], [e0, e1])
+    res = to_host(pool, ob, x.shape[:axis] + x.shape[axis + 1:], np.int32, [done])
+    pool.deallocate(xb, [])
+    pool.deallocate(ob, [])
+    dev.release(prog)
+    return res
+
+
+def argmax(dev: HIPDevice, pool: HIPMemoryPool, x: np.ndarray, dtype: DType = DType.F32) -> np.ndarray:
+    """x.argmax(): the flattened tensor's arg-max (zyx/src/tensor/mod.rs:2228-2230)."""
+    return argmax_axis(dev, pool, np.ascontiguousarray(x).reshape(-1), 0, dtype)
 
 
 # ---- GEMM (ZHIP_K_GEMM) ----------------------------------------------------------------------

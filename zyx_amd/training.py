@@ -105,6 +105,7 @@ class MLPTrainStep:
         self._copy_ev = []            # uploads of the batch the next step reads
         self._batch_no = 0            # batches set so far, and which of them each pair of batch buffers holds
         self._holds = [0, 0]
+        self._host = [None, None]     # host arrays of the batch last uploaded into each pair of batch buffers
 
     @property
     def _pending(self):
@@ -128,14 +129,16 @@ class MLPTrainStep:
         self.pool.sync_events(evs)
 
     def set_batch(self, x, labels):
-        """Uploads wait for the step before the previous one: it read the same pair of batch buffers."""
-        self._x = np.ascontiguousarray(x, np.float32)
-        self._y = np.ascontiguousarray(labels, np.int32)
+        """Uploads into this step's pair of batch buffers once the step before the previous one, which read them, is
+        done. That step also waited for its own uploads, so the host arrays they came from are free to drop here and
+        not before: a source of host_to_pool must outlive the copy."""
         xb, yb = self._batch_bufs[self._cur]
         if self._copy_ev:  # a batch that no step consumed
             self.pool.sync_events(self._copy_ev)
-        e1 = self.pool.host_to_pool(self._x, xb, self._take_plan_event(self._cur))
-        e2 = self.pool.host_to_pool(self._y, yb, [])
+        self.pool.sync_events(self._take_plan_event(self._cur))
+        self._host[self._cur] = (np.ascontiguousarray(x, np.float32), np.ascontiguousarray(labels, np.int32))
+        e1 = self.pool.host_to_pool(self._host[self._cur][0], xb, [])
+        e2 = self.pool.host_to_pool(self._host[self._cur][1], yb, [])
         self._copy_ev = [e1, e2]
         self._batch_no += 1
         self._holds[self._cur] = self._batch_no
