@@ -217,6 +217,13 @@ enum zhip_kernel_kind {
      * ZHIP_NORM_ADD (a tensor [rows, cols] that is added to dx: the skip branch of x + f(norm(x))).
      * args: x, (w), dy, (add), then dx, (dw), (db). */
     ZHIP_K_NORM_ROWS_BWD = 12,
+    /* Tensor::argmax_axis / argmax (zyx/src/tensor/mod.rs:2228-2269) along one axis of a dense tensor seen as
+     * x[outer, n, inner] (outer = product of the axes before it, inner = of those after; argmax() is outer = inner = 1):
+     * max_k((x == max_keepdim(x)) * k) as I32, i.e. the LARGEST index among equal maxima; the maximum is a reduce from
+     * the dtype's lowest finite value (zyx/src/kernel/linearize.rs:920-952) under fmax, so NaN entries are never
+     * chosen and a slice with no candidate gives 0. dims = {outer, n, inner}, n >= 1; dtype F32, BF16, F16 or I32.
+     * args: x, out[outer, inner] (I32). */
+    ZHIP_K_ARGMAX = 13,
     ZHIP_K_COUNT_
 };
 #define ZHIP_SOFTMAX_Y 1
@@ -346,6 +353,27 @@ typedef struct zhip_ir_op {
     uint64_t imm;
 } zhip_ir_op;
 
+/* --- host-side random numbers ---------------------------------------------------- */
+
+/* zyx draws every random tensor on the host from one generator (zyx/src/rng.rs: xoshiro256++ seeded by four
+ * splitmix64 rounds; default seed 42069, zyx/src/runtime.rs:178) and uploads it. These calls restate it, so seeded
+ * inputs match the reference's element for element. No device and no context are involved.
+ * zhip_rng_fill draws n elements in order:
+ *   ZHIP_RNG_RAND     Tensor::rand (zyx/src/tensor/mod.rs:516-597): F32 in [0, 1] via next_f32 (rng.rs:98-110), or
+ *                     the low bytes of one 64-bit draw per element for U8..U64 / I8..I64;
+ *   ZHIP_RNG_UNIFORM  Tensor::uniform (mod.rs:637-648), F32: rand * (hi - lo) + lo;
+ *   ZHIP_RNG_RANDN    Tensor::randn (mod.rs:603-613), F32: cos(2 pi u0) * sqrt(-2 ln(1 - u1)) over one rand([2, n])
+ *                     draw (all u0 first, then all u1), multiplied by hi when hi != 0; cos / ln / sqrt are the host
+ *                     libm's (the reference evaluates them on whatever device runs the kernel);
+ *   ZHIP_RNG_RANDINT  Tensor::randint (mod.rs:653-660, Rng::range rng.rs:186-208), I32 / I64 in [lo, hi):
+ *                     next_u64 % (hi - lo) + lo.
+ * Returns ZHIP_INCORRECT_KERNEL_ARG for a dtype the kind does not produce. */
+typedef struct zhip_rng { uint64_t s[4]; } zhip_rng;
+enum zhip_rng_kind { ZHIP_RNG_RAND = 0, ZHIP_RNG_UNIFORM = 1, ZHIP_RNG_RANDN = 2, ZHIP_RNG_RANDINT = 3 };
+void zhip_rng_seed(zhip_rng *rng, uint64_t seed);
+uint64_t zhip_rng_next_u64(zhip_rng *rng);
+int32_t zhip_rng_fill(zhip_rng *rng, int32_t kind, int32_t dtype, void *out, uint64_t n, double lo, double hi);
+
 /* --- backend lifetime ------------------------------------------------------- */
 
 /* Number of usable GPUs (device enumeration of hip.rs:190-215). */
@@ -451,6 +479,25 @@ int32_t zhip_profile_kernel(zhip_ctx *ctx, zhip_prog prog, const zhip_buf *args,
  * partial a call reads it has written itself). */
 int32_t zhip_reduce_static(zhip_ctx *ctx, int32_t dtype, int32_t op, int32_t axis0, int64_t rows, int64_t cols,
                            const void *x, void *out, void *stream);
+
+/* Ceilings measured on this device as it runs now. DeviceInfo.compute (zyx/src/backend/mod.rs:506-531) is a nominal
+ * figure; like the reference's autotuner (zyx/src/kernel/autotune.rs:775-798) this call finds out by launching and
+ * timing, so that kernel results can be priced against what the part sustains as well as against its data sheet:
+ *   memcpy_d2d_GBps   hipMemcpyDtoDAsync of `bytes`, read + written bytes per second;
+ *   copy_kernel_GBps  a plain 128-bit streaming copy kernel over the same buffers, read + written;
+ *   read_kernel_GBps  a read-only sum over `bytes`;
+ *   mfma_bf16_*       one wave per SIMD issuing 4096 v_mfma_f32_32x32x16_bf16 from registers (no memory traffic),
+ *                     with constant operands and with uniform(-1, 1) operands that change from instruction to
+ *                     instruction (real data draws more power, and the clock follows): TFLOP/s over the in-kernel
+ *                     duration, the shader clock read inside the kernel, and the launch-to-launch time in a queue of
+ *                     such launches.
+ * Allocates 2 x bytes of device memory for the duration of the call (bytes >= 1 MiB); blocks until done. */
+typedef struct zhip_ceilings {
+    float memcpy_d2d_GBps, copy_kernel_GBps, read_kernel_GBps;
+    float mfma_bf16_const_TFLOPs, mfma_bf16_const_MHz, mfma_bf16_const_launch_us;
+    float mfma_bf16_random_TFLOPs, mfma_bf16_random_MHz, mfma_bf16_random_launch_us;
+} zhip_ceilings;
+int32_t zhip_measure_ceilings(zhip_ctx *ctx, uint64_t bytes, zhip_ceilings *out);
 
 /* --- cached execution plans ----------------------------------------------------- */
 

@@ -198,6 +198,19 @@ def argmax_rows(x: np.ndarray) -> np.ndarray:
     return a
 
 
+def argmax_axis(x: np.ndarray, axis: int) -> np.ndarray:
+    """Tensor::argmax_axis (zyx/src/tensor/mod.rs:2238-2269) for any axis. Float tensors (given as f32 values) go
+    through the C row routine on a view with the axis moved last; integer tensors follow the reference's expression
+    literally, `max_k((x == max_keepdim(x)) * k)` cast to i32, in numpy integers."""
+    x = np.asarray(x)
+    axis = axis % x.ndim
+    if x.dtype.kind in "iu":
+        k = np.arange(x.shape[axis], dtype=np.int64).reshape([-1 if d == axis else 1 for d in range(x.ndim)])
+        return ((x == x.max(axis=axis, keepdims=True)) * k).max(axis=axis).astype(np.int32)
+    moved = np.moveaxis(x, axis, -1)
+    return argmax_rows(np.ascontiguousarray(moved, np.float32).reshape(-1, x.shape[axis])).reshape(moved.shape[:-1])
+
+
 def matmul(a: np.ndarray, b: np.ndarray, in_dtype: int = F32, out_dtype: int = F32, transb: bool = False,
            transa: bool = False) -> np.ndarray:
     """dot / dot_dtype of zyx/src/tensor/mod.rs:1469-1518 on 2-D operands (a stored [k,m] if transa,

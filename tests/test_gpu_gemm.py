@@ -70,6 +70,30 @@ def test_config3_full_size(hip, oracle):
     assert np.all(np.abs(lhs - rhs) <= 1e-4 * (np.abs(af) @ (np.abs(bf) @ np.abs(v))))
 
 
+def test_config3_full_size_bias_gelu(hip, oracle):
+    """Benchmark configuration 3 with its epilogue, gelu(A.B + bias) at 4096^3: the pre-activations have a standard
+    deviation of ~21, so most outputs lie where the reference's tanh = (e^2z - 1) / (e^2z + 1) has overflowed
+    (z > ~44, i.e. x > ~10: inf / inf, unspecified under its -ffast-math) or underflowed. The kernel saturates there
+    (gelu(x) -> x, resp. -> 0); everywhere it must be finite and match the formula of
+    zyx/src/tensor/elementwise.rs:168-170 evaluated in f64 on the f64-accumulated product of sampled rows."""
+    dev, pool = hip
+    a, b = make(oracle, 4096, 4096, 4096, 42069)
+    bias = oracle.f32_to_bf16(oracle.Rng(7).uniform(4096, -1 / 64, 1 / 64))
+    got = gemm(dev, pool, a, b, bias, epilogue="bias_gelu", bias_dtype=DType.BF16)
+    assert np.all(np.isfinite(got))
+    rows = np.arange(5, 4096, 64)
+    af, bf = oracle.bf16_to_f32(a).astype(np.float64), oracle.bf16_to_f32(b).astype(np.float64)
+    pre = af[rows] @ bf + oracle.bf16_to_f32(bias).astype(np.float64)[None, :]
+    mag = np.abs(af[rows]) @ np.abs(bf)
+    want = 0.5 * pre * (1 + np.tanh(np.sqrt(2 / np.pi) * (pre + 0.044715 * pre ** 3)))
+    # |gelu'| <= 1.13: the product's summation-order error (1e-5 of sum |a b|) passes through at most that much
+    assert np.all(np.abs(got[rows] - want) <= 1e-3 * np.abs(want) + 2e-5 * mag + 1e-6)
+    hi, lo = pre > 10, pre < -10
+    assert hi.sum() > 1000 and lo.sum() > 1000  # the sample does reach both saturated regions
+    assert np.all(np.abs(got[rows][hi] - pre[hi]) <= 2e-5 * mag[hi] + 1e-3 * np.abs(pre[hi]))
+    assert np.all(np.abs(got[rows][lo]) <= 1e-6)
+
+
 # ---- general kernel: f32, ragged shapes, narrow outputs, batches -------------------------------------
 
 def test_reference_matmul_goldens(hip):

@@ -310,3 +310,26 @@ def test_autotune_call_sequence(hip):
     dev.release(prog)
     for b in (rows, x, y):
         pool.deallocate(b, [])
+
+
+def test_reference_integer_matmuls_on_the_device(hip):
+    """Integer products are bit-exact on the GPU: the reference's i64 fixture (zyx/tests/xyz2.safetensors,
+    zyx/tests/05_misc.rs:639-661: x[256,512] . y[512,368] == z) and the closed-form i32 sweep of matmul_1
+    (05_misc.rs:210-237: x[i][j] = i + j, y[i][j] = i - j), through generated matmul kernels."""
+    import os
+    from zyx_amd import safetensors_io
+    t = safetensors_io.load(os.path.join(os.path.dirname(__file__), "golden", "xyz2.safetensors"))
+    x, y, z = (np.ascontiguousarray(t[k][1]) for k in "xyz")
+    assert x.dtype == np.int64 and x.shape == (256, 512) and y.shape == (512, 368)
+    for local in ((16, 16), (1, 1)):
+        (g, _), = both(hip, K.matmul(256, 368, 512, DType.I64, DType.I64, use_mad=True, local=local),
+                       [x, y, np.zeros((256, 368), np.int64)])
+        assert g.dtype == np.int64 and np.array_equal(g, z)
+    for m in range(56, 576, 259):
+        for k in range(12, 890, 231):
+            for n in range(5, 97, 71):
+                a = (np.arange(m)[:, None] + np.arange(k)[None, :]).astype(np.int32)
+                b = (np.arange(k)[:, None] - np.arange(n)[None, :]).astype(np.int32)
+                want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.int32)  # wraps like i32 accumulation
+                (g, c), = both(hip, K.matmul(m, n, k, DType.I32, DType.I32), [a, b, np.zeros((m, n), np.int32)])
+                assert np.array_equal(g, want) and np.array_equal(c, want), (m, k, n)

@@ -7,8 +7,8 @@ the f64 sum at 1e-5 of sum(|x|) (the bound both orders satisfy), and max is exac
 import numpy as np
 import pytest
 
-from zyx_amd import DType
-from zyx_amd.kernels import reduce
+from zyx_amd import BackendError, DType
+from zyx_amd.kernels import argmax_desc, reduce
 
 pytestmark = pytest.mark.gpu
 
@@ -99,3 +99,55 @@ def test_scale_is_refused_for_integers(hip):
     dev, pool = hip
     with pytest.raises(BackendError):
         dev.register_kernel(reduce_desc(4, 4, "sum", False, DType.I32, mul=2.0))
+
+
+# ---- argmax_axis (zyx/src/tensor/mod.rs:2238-2269) -------------------------------------------------------------
+def test_argmax_reference_goldens(hip):
+    """zyx/tests/08_indexing.rs:630-694 on the device, as i32 tensors (what the reference builds) and as f32."""
+    from zyx_amd.kernels import argmax, argmax_axis
+    dev, pool = hip
+    for dt, np_dt in ((DType.I32, np.int32), (DType.F32, np.float32)):
+        am = lambda x, ax: argmax_axis(dev, pool, np.array(x, np_dt), ax, dt).tolist()
+        assert am([1, 3, 2, 5], 0) == 3 or am([1, 3, 2, 5], 0) == [3]
+        x2 = [[1, 3, 2], [4, 6, 5], [7, 9, 8]]
+        assert argmax(dev, pool, np.array(x2, np_dt), dt).item() == 7
+        assert am(x2, 0) == [2, 2, 2] and am(x2, 1) == [1, 1, 1]
+        xn = [[-1, -3, -2], [-4, -6, -5]]
+        assert argmax(dev, pool, np.array(xn, np_dt), dt).item() == 0
+        assert am(xn, 0) == [0, 0, 0] and am(xn, 1) == [0, 0]
+        assert am([[42]], 0) == [0] and am([[42]], 1) == [0]
+        x3 = [[[1, 5, 2], [4, 0, 3]], [[7, 2, 6], [1, 8, 0]]]
+        assert am(x3, 0) == [[1, 0, 1], [0, 1, 0]] and am(x3, 1) == [[1, 0, 1], [0, 1, 0]] and am(x3, 2) == [[1, 0], [0, 1]]
+
+
+@pytest.mark.parametrize("shape,axis", [((8192, 4096), 1), ((8192, 4096), 0), ((3, 70000), 1), ((1, 1 << 21), 1),
+                                        ((5, 777, 33), 1), ((2, 9000, 3), 1), ((64, 10), 1), ((7, 5, 260), 0),
+                                        ((300, 1001), 1), ((4097, 2), 0)])
+def test_argmax_axis_matches_oracle(hip, oracle, shape, axis):
+    """Bit-exact arg-max on every layout the kernels split differently (one wave per row, segmented rows, strided
+    axis with and without chunks), with many ties (values drawn from 12 levels) and without."""
+    from zyx_amd.kernels import argmax_axis
+    dev, pool = hip
+    rng = np.random.default_rng(sum(shape) + axis)
+    ties = rng.integers(-6, 6, size=shape).astype(np.int32)
+    assert np.array_equal(argmax_axis(dev, pool, ties, axis, DType.I32), oracle.argmax_axis(ties, axis))
+    assert np.array_equal(argmax_axis(dev, pool, ties.astype(np.float32), axis, DType.F32), oracle.argmax_axis(ties.astype(np.float32), axis))
+    x = rng.standard_normal(shape).astype(np.float32)
+    assert np.array_equal(argmax_axis(dev, pool, x, axis, DType.F32), oracle.argmax_axis(x, axis))
+    xb = oracle.f32_to_bf16(x)  # storage bits; many ties after truncation
+    assert np.array_equal(argmax_axis(dev, pool, xb, axis, DType.BF16), oracle.argmax_axis(oracle.bf16_to_f32(xb), axis))
+
+
+def test_argmax_skips_nan_and_handles_lowest(hip, oracle):
+    from zyx_amd.kernels import argmax_axis
+    dev, pool = hip
+    x = np.array([[np.nan, 1.0, np.nan, 1.0, 0.5], [np.nan] * 5, [-np.inf] * 5, [-3.4028235e38, -np.inf, -3.4028235e38, -np.inf, -np.inf],
+                  [0.0, -0.0, 0.0, -0.0, -1.0]], np.float32)
+    got = argmax_axis(dev, pool, x, 1, DType.F32)
+    # fmax skips a NaN and a NaN equals nothing: the expression's IEEE reading. (The reference's C backend compiles
+    # with -ffast-math, which leaves NaN handling unspecified; the CPU oracle, built with the same flags, is therefore
+    # only consulted on the NaN-free rows.)
+    assert got.tolist() == [3, 0, 0, 2, 3]
+    assert np.array_equal(got[2:], oracle.argmax_axis(x[2:], 1))
+    with pytest.raises(BackendError):
+        dev.register_kernel(argmax_desc(4, 0, 4))

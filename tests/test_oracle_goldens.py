@@ -110,6 +110,44 @@ def test_argmax_goldens_and_ties(oracle):
         assert oracle.argmax_rows(row[None, :])[0] == want
 
 
+def test_argmax_axis_goldens(oracle):
+    """zyx/tests/08_indexing.rs:630-694 (argmax_comprehensive, argmax_1): every axis, int tensors as the reference
+    writes them and the same values as f32."""
+    cases = [
+        ([1, 3, 2, 5], 0, [3]),
+        ([[1, 3, 2], [4, 6, 5], [7, 9, 8]], 0, [2, 2, 2]),
+        ([[1, 3, 2], [4, 6, 5], [7, 9, 8]], 1, [1, 1, 1]),
+        ([[-1, -3, -2], [-4, -6, -5]], 0, [0, 0, 0]),
+        ([[-1, -3, -2], [-4, -6, -5]], 1, [0, 0]),
+        ([[42]], 0, [0]),
+        ([[42]], 1, [0]),
+        ([[[1, 5, 2], [4, 0, 3]], [[7, 2, 6], [1, 8, 0]]], 0, [[1, 0, 1], [0, 1, 0]]),
+        ([[[1, 5, 2], [4, 0, 3]], [[7, 2, 6], [1, 8, 0]]], 1, [[1, 0, 1], [0, 1, 0]]),
+        ([[[1, 5, 2], [4, 0, 3]], [[7, 2, 6], [1, 8, 0]]], 2, [[1, 0], [0, 1]]),
+    ]
+    for x, axis, want in cases:
+        for dt in (np.int32, np.float32):
+            got = oracle.argmax_axis(np.array(x, dt), axis)
+            if np.ndim(want) == 1 and np.ndim(x) == 1:
+                got = got.reshape(-1)
+            assert got.dtype == np.int32 and got.tolist() == want, (x, axis, dt)
+    # flattened argmax(): 08_indexing.rs:633,641,654,663
+    assert oracle.argmax_axis(np.array([[1, 3, 2], [4, 6, 5], [7, 9, 8]], np.int32).reshape(-1), 0).item() == 7
+    assert oracle.argmax_axis(np.array([[-1, -3, -2], [-4, -6, -5]], np.int32).reshape(-1), 0).item() == 0
+    # both routes give the largest index of tied maxima on every axis (brute force)
+    rng = np.random.default_rng(3)
+    for _ in range(100):
+        shape = tuple(rng.integers(1, 5, size=3))
+        x = rng.integers(-2, 2, size=shape)
+        for axis in range(3):
+            want = np.zeros([d for i, d in enumerate(shape) if i != axis], np.int64)
+            for idx in np.ndindex(*want.shape):
+                sl = x[idx[:axis] + (slice(None),) + idx[axis:]]
+                want[idx] = max(k for k in range(len(sl)) if sl[k] == sl.max())
+            assert np.array_equal(oracle.argmax_axis(x.astype(np.int32), axis), want)
+            assert np.array_equal(oracle.argmax_axis(x.astype(np.float32), axis), want)
+
+
 # ---- reductions: 04_reduce.rs (closed forms over ones / mod-10 pattern) ------------
 def test_reduce_goldens(oracle):
     assert oracle.reduce_rows_i32("sum", np.ones((8, 4096), np.int32)).tolist() == [4096] * 8
@@ -566,3 +604,71 @@ def test_block_f64_forward_pieces_and_backward_finite_differences(oracle):
             lo[i] -= 1e-6
             num[i] = (lossc(p, hi) - lossc(p, lo)) / 2e-6 if name == "x" else (lossc({**p, name: hi}, x) - lossc({**p, name: lo}, x)) / 2e-6
         assert np.allclose(gc["dx"] if name == "x" else gc[name], num, rtol=2e-5, atol=2e-6), name
+
+
+# ---- every entry of the oracle's unary / binary tables, on the reference's own test vectors ---------------------
+# zyx/tests/01_unary.rs:18-111 and zyx/tests/02_binary.rs:7-140 compare each op with the host language's scalar
+# function on these ten values (exact equality for + - * max and comparisons, is_equal otherwise). The expected
+# values here come from numpy in float64, rounded once: an independent libm, so a swapped table entry, a wrong
+# operand order or a missing composite step fails.
+_REF_X = np.array([-3.285, 0.001, 1.780, 5.675, -8.521, -0.456, 1.215, -3.474, -4.128, -7.657], np.float32)
+_REF_Y = np.array([2.772, -8.327, 1.945, 9.286, 3.989, 8.105, -5.307, 2.865, 3.106, 3.111], np.float32)
+
+
+def _close32(got, want64):
+    want = np.asarray(want64, np.float64).astype(np.float32)
+    both_nan = np.isnan(got) & np.isnan(want)
+    return np.all(both_nan | np.isclose(got, want, rtol=2e-6, atol=1e-37))
+
+
+def test_unary_table_closed_forms(oracle):
+    x, x64 = _REF_X, _REF_X.astype(np.float64)
+    with np.errstate(all="ignore"):
+        exact = {"neg": -x, "floor": np.floor(x), "trunc": np.trunc(x), "abs": np.abs(x),
+                 "relu": np.where(x > 0, x, np.float32(0)) * np.float32(1), "reciprocal": np.float32(1) / x,
+                 "sqrt": np.sqrt(x)}
+        close = {"exp": np.exp(x64), "exp2": np.exp2(x64), "ln": np.log(x64), "log2": np.log2(x64), "sin": np.sin(x64),
+                 "cos": np.cos(x64), "tanh": np.tanh(x64), "sigmoid": 1 / (1 + np.exp(-x64)),
+                 "rsqrt": np.sqrt(1 / x64),
+                 "gelu": 0.5 * x64 * (1 + np.tanh(np.sqrt(2 / np.pi) * (x64 + 0.044715 * x64 ** 3)))}
+    assert set(exact) | set(close) == set(oracle.UNARY), "a unary table entry without a pin"
+    for name, want in exact.items():
+        got = oracle.unary(name, x)
+        assert np.array_equal(got, want, equal_nan=True), name
+    for name, want in close.items():
+        got = oracle.unary(name, x)
+        if name in ("tanh", "gelu", "sigmoid"):  # compositions that carry one rounding of a value near 1
+            assert np.allclose(got, want.astype(np.float32), rtol=1e-5, atol=3e-7), name
+        else:
+            assert _close32(got, want), name
+    # values the reference asserts outright: 01_unary.rs:332-343 (abs), :9-16 (relu)
+    assert oracle.unary("abs", np.array([-2.0, 0.0, 3.0], np.float32)).tolist() == [2.0, 0.0, 3.0]
+    # sign of zero and special values survive the plain ops
+    assert np.signbit(oracle.unary("neg", np.array([0.0], np.float32)))[0]
+    assert oracle.unary("floor", np.array([-0.5, 2.5, -2.0], np.float32)).tolist() == [-1.0, 2.0, -2.0]
+    assert oracle.unary("trunc", np.array([-0.5, 2.5, -2.7], np.float32)).tolist() == [-0.0, 2.0, -2.0]
+
+
+def test_binary_table_closed_forms(oracle):
+    x, y = _REF_X, _REF_Y
+    exact = {"add": x + y, "sub": x - y, "mul": x * y, "div": x / y, "max": np.maximum(x, y),
+             "cmplt": (x < y).astype(np.float32), "cmpgt": (x > y).astype(np.float32),
+             "cmpge": (x >= y).astype(np.float32), "eq": (x == y).astype(np.float32),
+             "noteq": (x != y).astype(np.float32),
+             "mod": np.fmod(x.astype(np.int32), y.astype(np.int32)).astype(np.float32)}  # (int)x % (int)y, C truncation
+    assert set(exact) | {"pow"} == set(oracle.BINARY), "a binary table entry without a pin"
+    for name, want in exact.items():
+        got = oracle.binary(name, x, y)
+        assert np.array_equal(got, want), name
+    # sub and div are not commutative: swapped operands must change the answer
+    assert not np.array_equal(oracle.binary("sub", x, y), oracle.binary("sub", y, x))
+    assert np.array_equal(oracle.binary("cmpge", x, x), np.ones_like(x))
+    # pow is exp2(log2(x) * y) (zyx/src/kernel/fold_constants.rs:639-653): the textbook power for positive bases,
+    # NaN for every negative base, whatever the exponent (02_binary.rs:99-111 accepts NaN == NaN)
+    got = oracle.binary("pow", x, y)
+    with np.errstate(all="ignore"):
+        want = np.power(x.astype(np.float64), y.astype(np.float64))
+    pos = x > 0
+    assert np.allclose(got[pos], want[pos].astype(np.float32), rtol=2e-5) and np.all(np.isnan(got[~pos]))
+    p = oracle.binary("pow", np.array([-2.0, 2.0, 0.5], np.float32), np.array([2.0, 2.0, 0.5], np.float32))
+    assert np.isnan(p[0]) and abs(p[1] - 4.0) < 1e-5 and abs(p[2] - np.sqrt(0.5)) < 1e-6

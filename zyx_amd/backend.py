@@ -89,6 +89,12 @@ class KernelDesc(C.Structure):
                 ("dims", C.c_int64 * 8), ("fparams", C.c_float * 8), ("iparams", C.c_int32 * 24)]
 
 
+class _Ceilings(C.Structure):
+    _fields_ = [(n, C.c_float) for n in ("memcpy_d2d_GBps", "copy_kernel_GBps", "read_kernel_GBps",
+                                         "mfma_bf16_const_TFLOPs", "mfma_bf16_const_MHz", "mfma_bf16_const_launch_us",
+                                         "mfma_bf16_random_TFLOPs", "mfma_bf16_random_MHz", "mfma_bf16_random_launch_us")]
+
+
 @dataclass
 class DeviceInfo:
     """zyx/src/backend/mod.rs:506-531"""
@@ -131,7 +137,7 @@ _EXPORTS = ["zhip_device_count", "zhip_init", "zhip_deinit", "zhip_last_error", 
             "zhip_get_variable", "zhip_h2d", "zhip_d2h", "zhip_d2d", "zhip_sync_events", "zhip_release_events",
             "zhip_buffer_ptr", "zhip_register_kernel", "zhip_compile_ir", "zhip_ir_generate", "zhip_program_source", "zhip_launch",
             "zhip_release_program",
-            "zhip_reduce_static", "zhip_time_kernel", "zhip_profile_kernel", "zhip_plan_create", "zhip_plan_launch", "zhip_plan_destroy"]
+            "zhip_rng_seed", "zhip_rng_next_u64", "zhip_rng_fill", "zhip_reduce_static", "zhip_measure_ceilings", "zhip_time_kernel", "zhip_profile_kernel", "zhip_plan_create", "zhip_plan_launch", "zhip_plan_destroy"]
 
 
 def load_library() -> C.CDLL:
@@ -362,6 +368,12 @@ class HIPDevice:
         self._ctx.check(self._ctx.lib.zhip_reduce_static(self._ctx.ptr, C.c_int32(int(dtype)), C.c_int32(op),
                                                          C.c_int32(int(bool(axis0))), C.c_int64(rows), C.c_int64(cols),
                                                          C.c_void_p(x_ptr), C.c_void_p(out_ptr), C.c_void_p(stream)))
+
+    def measure_ceilings(self, nbytes: int = 128 << 20) -> dict:
+        """zhip_measure_ceilings: streaming and matrix-instruction rates this device sustains right now."""
+        raw = _Ceilings()
+        self._ctx.check(self._ctx.lib.zhip_measure_ceilings(self._ctx.ptr, C.c_uint64(nbytes), C.byref(raw)))
+        return {name: round(float(getattr(raw, name)), 1) for name, _ in _Ceilings._fields_}
 
     def release(self, program_id: int):
         self._ctx.check(self._ctx.lib.zhip_release_program(self._ctx.ptr, C.c_uint32(program_id)))

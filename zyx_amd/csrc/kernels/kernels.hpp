@@ -57,6 +57,20 @@ bool reduce_shape_ok(int64_t rows, int64_t cols, int axis0);
 uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int axis0);
 hipError_t reduce(const Reduce &p, hipStream_t stream);
 
+// Index of the maximum along the middle axis of a contiguous x[outer, n, inner] (any axis of a dense tensor), ties to
+// the largest index, NaN entries never chosen; out[outer, inner] is i32.
+struct ArgMax {
+    int64_t outer, n, inner;
+    int dtype; // F32, BF16, F16 or I32
+    const void *x;
+    int32_t *out;
+    void *workspace; // argmax_workspace_bytes(outer, n, inner)
+    uint64_t workspace_bytes;
+};
+bool argmax_shape_ok(int64_t outer, int64_t n, int64_t inner);
+uint64_t argmax_workspace_bytes(int64_t outer, int64_t n, int64_t inner);
+hipError_t argmax(const ArgMax &p, hipStream_t stream);
+
 // Geometry of a zero-padded NCHW input [images, C, Hp, Wp] from which gemm_bf16 gathers the patch matrix of a
 // convolution on the fly (khw == 0: not used). Offsets in elements; k = (c*KH + ky)*KW + kx.
 struct ConvGather {
@@ -203,6 +217,14 @@ struct AttentionBwd {
 };
 uint64_t attention_bwd_workspace_bytes(const Attention &p);
 hipError_t attention_bwd(const AttentionBwd &p, hipStream_t stream);
+
+// What this device sustains right now (ceilings.hip); the layout is zhip_ceilings of include/zyx_hip.h.
+struct Ceilings {
+    float memcpy_d2d_GBps, copy_kernel_GBps, read_kernel_GBps;
+    float mfma_bf16_const_TFLOPs, mfma_bf16_const_MHz, mfma_bf16_const_launch_us;
+    float mfma_bf16_random_TFLOPs, mfma_bf16_random_MHz, mfma_bf16_random_launch_us;
+};
+hipError_t measure_ceilings(uint64_t bytes, int compute_units, Ceilings *out, hipStream_t stream);
 
 // cross_entropy of f32 logits [rows, cols] with i32 class indices; loss / grad may be null.
 struct CrossEntropy {

@@ -286,6 +286,163 @@ template <int DT, int OP> hipError_t launch(const Reduce &p, hipStream_t st) {
     return hipGetLastError();
 }
 
+
+// ---- argmax along one axis of a contiguous [outer, n, inner] view -----------------------------------------------
+// Tensor::argmax_axis (zyx/src/tensor/mod.rs:2238-2269) is max_k((x == max_keepdim(x)) * k) cast to i32: the LARGEST
+// index among equal maxima; the maximum is a reduce from the dtype's lowest finite value in which a NaN never wins
+// (fmax), and a NaN never equals it, so NaN entries are skipped and a row without any finite candidate gives 0.
+// One pass keeps (best value, largest index holding it); pairs combine associatively, so lanes, waves and workgroups
+// may fold slices in any order and the result is the reference's.
+template <typename A> struct Best {
+    A v;
+    int i;
+};
+template <typename A> __device__ __forceinline__ A lowest();
+template <> __device__ __forceinline__ float lowest<float>() { return -FLT_MAX; }
+template <> __device__ __forceinline__ int lowest<int>() { return INT32_MIN; }
+template <typename A> __device__ __forceinline__ void best_take(Best<A> &b, A v, int i) {
+    if (v > b.v) {
+        b.v = v;
+        b.i = i;
+    } else if (v == b.v) {
+        b.i = max(b.i, i);
+    }
+}
+__device__ __forceinline__ float shfl_xor_any(float v, int m) { return __shfl_xor(v, m, 64); }
+__device__ __forceinline__ int shfl_xor_any(int v, int m) { return __shfl_xor(v, m, 64); }
+template <typename A> __device__ __forceinline__ Best<A> wave_best(Best<A> b) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        A ov = shfl_xor_any(b.v, m);
+        int oi = __shfl_xor(b.i, m, 64);
+        best_take(b, ov, oi);
+    }
+    return b;
+}
+
+// inner == 1: one wave per (row, segment) of x[rows, n]; lanes stride the span with 4-element loads when VEC.
+template <int DT, bool VEC>
+__global__ __launch_bounds__(256) void argmax_rows_k(const typename Elem<DT>::S *__restrict__ x, int32_t *__restrict__ out,
+                                                     typename Elem<DT>::A *__restrict__ pv, int32_t *__restrict__ pi,
+                                                     int64_t rows, int64_t n, int segs, int64_t seg_len) {
+    typedef typename Elem<DT>::A A;
+    const int lane = threadIdx.x & 63;
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= rows * segs) return; // whole wave
+    const int64_t row = item / segs;
+    const int seg = (int)(item - row * segs);
+    const int64_t c0 = seg * seg_len, c1 = min(n, c0 + seg_len);
+    const typename Elem<DT>::S *xr = x + row * n;
+    Best<A> b{lowest<A>(), 0};
+    if (VEC) {
+        const int64_t nv = (c1 - c0) >> 2;
+        for (int64_t i = lane; i < nv; i += 64) {
+            A v[4];
+            Elem<DT>::ld4(xr, c0 + i * 4, v);
+#pragma unroll
+            for (int k = 0; k < 4; k++) best_take(b, v[k], (int)(c0 + i * 4 + k));
+        }
+        for (int64_t c = c0 + nv * 4 + lane; c < c1; c += 64) best_take(b, Elem<DT>::ld(xr, c), (int)c);
+    } else {
+        for (int64_t c = c0 + lane; c < c1; c += 64) best_take(b, Elem<DT>::ld(xr, c), (int)c);
+    }
+    b = wave_best(b);
+    if (lane == 0) {
+        if (segs == 1) out[row] = b.i;
+        else {
+            pv[item] = b.v;
+            pi[item] = b.i;
+        }
+    }
+}
+// second stage of both layouts: result r folds partial pairs r * stride_r + s * stride_s, s < parts
+template <typename A>
+__global__ __launch_bounds__(256) void argmax_partials_k(const A *__restrict__ pv, const int32_t *__restrict__ pi,
+                                                         int32_t *__restrict__ out, int64_t n_out, int parts,
+                                                         int64_t stride_r, int64_t stride_s) {
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= n_out) return;
+    Best<A> b{lowest<A>(), 0};
+    for (int s = 0; s < parts; s++) best_take(b, pv[r * stride_r + s * stride_s], pi[r * stride_r + s * stride_s]);
+    out[r] = b.i;
+}
+// inner > 1: a workgroup owns 64 neighbouring inner positions of one outer slice (lane -> position, coalesced rows)
+// and a chunk of the axis split over its 4 waves; LDS joins the waves.
+template <int DT>
+__global__ __launch_bounds__(256) void argmax_mid_k(const typename Elem<DT>::S *__restrict__ x, int32_t *__restrict__ out,
+                                                    typename Elem<DT>::A *__restrict__ pv, int32_t *__restrict__ pi,
+                                                    int64_t n, int64_t inner, int strips, int chunks, int64_t chunk_len) {
+    typedef typename Elem<DT>::A A;
+    __shared__ A lv[4][64];
+    __shared__ int li[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t o = blockIdx.x / strips;
+    const int64_t c = (int64_t)(blockIdx.x % strips) * 64 + lane;
+    const int chunk = blockIdx.y;
+    const int64_t r0 = chunk * chunk_len, r1 = min(n, r0 + chunk_len);
+    Best<A> b{lowest<A>(), 0};
+    if (c < inner) {
+        const typename Elem<DT>::S *xo = x + o * n * inner + c;
+#pragma unroll 8
+        for (int64_t r = r0 + wave; r < r1; r += 4) best_take(b, Elem<DT>::ld(xo, r * inner), (int)r);
+    }
+    lv[wave][lane] = b.v;
+    li[wave][lane] = b.i;
+    __syncthreads(); // every thread arrives: no early exit above
+    if (wave == 0 && c < inner) {
+#pragma unroll
+        for (int w = 1; w < 4; w++) best_take(b, lv[w][lane], li[w][lane]);
+        if (chunks == 1) out[o * inner + c] = b.i;
+        else {
+            pv[(o * chunks + chunk) * inner + c] = b.v;
+            pi[(o * chunks + chunk) * inner + c] = b.i;
+        }
+    }
+}
+
+struct ArgPlan { int parts; int64_t len; int strips; };
+ArgPlan plan_argmax(int64_t outer, int64_t n, int64_t inner) {
+    if (inner == 1) {
+        RowPlan r = plan_rows(outer, n);
+        return {r.segs, r.seg_len, 0};
+    }
+    const int64_t strips = (inner + 63) / 64, blocks = strips * outer;
+    int chunks = 1;
+    if (blocks < 1024 && n >= 256) chunks = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>((1024 + blocks - 1) / blocks, n / 64), 4096));
+    int64_t len = (n + chunks - 1) / chunks;
+    chunks = (int)((n + len - 1) / len);
+    return {chunks, len, (int)strips};
+}
+
+template <int DT> hipError_t launch_argmax(const ArgMax &p, hipStream_t st) {
+    typedef typename Elem<DT>::S S;
+    typedef typename Elem<DT>::A A;
+    const S *x = (const S *)p.x;
+    const ArgPlan pl = plan_argmax(p.outer, p.n, p.inner);
+    const int64_t n_out = p.outer * p.inner;
+    A *pv = (A *)p.workspace;
+    int32_t *pi = (int32_t *)((char *)p.workspace + (uint64_t)n_out * pl.parts * 4);
+    if (pl.parts > 1 && (uint64_t)n_out * pl.parts * 8 > p.workspace_bytes) return hipErrorInvalidValue;
+    if (p.inner == 1) {
+        const bool vec = p.n % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+        dim3 grid((unsigned)((p.outer * pl.parts + 3) / 4)), block(256);
+        if (vec) hipLaunchKernelGGL((argmax_rows_k<DT, true>), grid, block, 0, st, x, p.out, pv, pi, p.outer, p.n, pl.parts, pl.len);
+        else hipLaunchKernelGGL((argmax_rows_k<DT, false>), grid, block, 0, st, x, p.out, pv, pi, p.outer, p.n, pl.parts, pl.len);
+        if (pl.parts > 1)
+            hipLaunchKernelGGL((argmax_partials_k<A>), dim3((unsigned)((n_out + 255) / 256)), block, 0, st, pv, pi, p.out, n_out, pl.parts, (int64_t)pl.parts, (int64_t)1);
+    } else {
+        dim3 grid((unsigned)(pl.strips * p.outer), (unsigned)pl.parts), block(256);
+        hipLaunchKernelGGL((argmax_mid_k<DT>), grid, block, 0, st, x, p.out, pv, pi, p.n, p.inner, pl.strips, pl.parts, pl.len);
+        if (pl.parts > 1) { // result (o, c) folds partial[(o * parts + s) * inner + c]: walk the outer slices one launch each
+            for (int64_t o = 0; o < p.outer; o++)
+                hipLaunchKernelGGL((argmax_partials_k<A>), dim3((unsigned)((p.inner + 255) / 256)), block, 0, st,
+                                   pv + o * pl.parts * p.inner, pi + o * pl.parts * p.inner, p.out + o * p.inner, p.inner,
+                                   pl.parts, (int64_t)1, p.inner);
+        }
+    }
+    return hipGetLastError();
+}
+
 } // namespace
 
 bool reduce_shape_ok(int64_t rows, int64_t cols, int axis0) {
@@ -336,6 +493,33 @@ hipError_t reduce(const Reduce &p, hipStream_t st) {
     case DT_F16 * 2 + 1: return launch<2, 1>(p, st);
     case DT_I32 * 2 + 0: return launch<3, 0>(p, st);
     case DT_I32 * 2 + 1: return launch<3, 1>(p, st);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+bool argmax_shape_ok(int64_t outer, int64_t n, int64_t inner) {
+    if (outer < 0 || n < 1 || inner < 0 || n >= (1ll << 31)) return false; // indices are i32; an empty axis has no arg-max
+    if (outer == 0 || inner == 0) return true;
+    if (outer > (1ll << 40) / inner || outer * inner > (1ll << 40) / n) return false;
+    if (inner == 1) return outer * plan_rows(outer, n).segs < (1ll << 33);
+    return (inner + 63) / 64 * outer < (1ll << 31);
+}
+
+uint64_t argmax_workspace_bytes(int64_t outer, int64_t n, int64_t inner) {
+    if (outer <= 0 || n <= 0 || inner <= 0) return 0;
+    const ArgPlan pl = plan_argmax(outer, n, inner);
+    return pl.parts > 1 ? (uint64_t)outer * inner * pl.parts * 8 : 0;
+}
+
+hipError_t argmax(const ArgMax &p, hipStream_t st) {
+    if (!argmax_shape_ok(p.outer, p.n, p.inner)) return hipErrorInvalidValue;
+    const int64_t n_out = p.outer * p.inner;
+    if (n_out == 0) return hipSuccess;
+    switch (p.dtype) {
+    case DT_F32: return launch_argmax<0>(p, st);
+    case DT_BF16: return launch_argmax<1>(p, st);
+    case DT_F16: return launch_argmax<2>(p, st);
+    case DT_I32: return launch_argmax<3>(p, st);
     default: return hipErrorInvalidValue;
     }
 }

@@ -300,8 +300,9 @@ zk::Conv2d conv_args(const zhip_kernel_desc &d) {
     a.N = (int)d.dims[0]; a.C = (int)d.dims[1]; a.H = (int)d.dims[2]; a.W = (int)d.dims[3];
     a.Cout = (int)d.dims[4]; a.KH = (int)d.dims[5]; a.KW = (int)d.dims[6];
     a.sy = d.iparams[0]; a.sx = d.iparams[1]; a.py = d.iparams[2]; a.px = d.iparams[3]; a.dy = d.iparams[4]; a.dx = d.iparams[5];
-    a.OH = (a.H + 2 * a.py - a.dy * (a.KH - 1) - 1) / a.sy + 1;
-    a.OW = (a.W + 2 * a.px - a.dx * (a.KW - 1) - 1) / a.sx + 1;
+    // 64-bit: registration has bounded every term, the sums of a hostile descriptor must not wrap before it has
+    a.OH = (int)(((int64_t)a.H + 2 * (int64_t)a.py - (int64_t)a.dy * (a.KH - 1) - 1) / a.sy + 1);
+    a.OW = (int)(((int64_t)a.W + 2 * (int64_t)a.px - (int64_t)a.dx * (a.KW - 1) - 1) / a.sx + 1);
     a.dtype = d.dtype; a.out_dtype = d.out_dtype; a.relu = d.iparams[7]; a.pool = d.iparams[8];
     return a;
 }
@@ -447,6 +448,20 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         p.workspace_bytes = zk::reduce_workspace_bytes(rows, cols, d.flags & 1);
         return ZHIP_OK;
     }
+    case ZHIP_K_ARGMAX: {
+        const int64_t outer = d.dims[0], n = d.dims[1], inner = d.dims[2];
+        if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16 && d.dtype != ZHIP_F16 && d.dtype != ZHIP_I32)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "argmax: dtype %d not implemented", d.dtype);
+        if (d.flags) return c->fail(ZHIP_KERNEL_COMPILATION, "argmax: bad flags");
+        if (!zk::argmax_shape_ok(outer, n, inner))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "argmax: shape out of range (axis length 1 .. 2^31 - 1)");
+        p.n_in = 1;
+        p.n_out = 1;
+        p.need[0] = (uint64_t)outer * n * inner * dtype_bytes(d.dtype);
+        p.need[1] = (uint64_t)outer * inner * 4;
+        p.workspace_bytes = zk::argmax_workspace_bytes(outer, n, inner);
+        return ZHIP_OK;
+    }
     case ZHIP_K_GEMM: {
         int64_t M = d.dims[0], N = d.dims[1], K = d.dims[2], batch = d.dims[3] ? d.dims[3] : 1;
         int epi = d.iparams[0];
@@ -534,7 +549,10 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
             return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: bad shape or stride/padding/dilation");
         if ((d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16) || (d.out_dtype != d.dtype && !(d.dtype == ZHIP_BF16 && d.out_dtype == ZHIP_F32)))
             return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: dtype %d -> %d not implemented", d.dtype, d.out_dtype);
-        const int64_t eh = H + 2 * py - (int64_t)dy * (KH - 1) - 1, ew = W + 2 * px - (int64_t)dx * (KW - 1) - 1;
+        if (H >= (1ll << 30) || W >= (1ll << 30) || KH >= (1ll << 20) || KW >= (1ll << 20) || sy >= (1 << 20) || sx >= (1 << 20) ||
+            py >= (1 << 20) || px >= (1 << 20) || dy >= (1 << 20) || dx >= (1 << 20))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: size, stride, padding or dilation out of range");
+        const int64_t eh = H + 2 * (int64_t)py - (int64_t)dy * (KH - 1) - 1, ew = W + 2 * (int64_t)px - (int64_t)dx * (KW - 1) - 1;
         if (eh < 0 || ew < 0) return c->fail(ZHIP_KERNEL_COMPILATION, "conv2d: kernel larger than the padded input");
         const int64_t OH = eh / sy + 1, OW = ew / sx + 1;
         if (!elems_fit({C, H, W}) || !elems_fit({C, KH, KW}) || !elems_fit({N, OH, OW}) || !elems_fit({N, C, H, W}) ||
@@ -569,7 +587,9 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16) return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: dtype must be F32 or BF16");
         if (!elems_fit({planes, H, W}) || KH >= (1 << 30) || KW >= (1 << 30))
             return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: tensor too large");
-        const int64_t eh = H + 2 * py - (int64_t)dy * (KH - 1) - 1, ew = W + 2 * px - (int64_t)dx * (KW - 1) - 1;
+        if (sy >= (1 << 20) || sx >= (1 << 20) || py >= (1 << 20) || px >= (1 << 20) || dy >= (1 << 20) || dx >= (1 << 20))
+            return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: stride, padding or dilation out of range");
+        const int64_t eh = H + 2 * (int64_t)py - (int64_t)dy * (KH - 1) - 1, ew = W + 2 * (int64_t)px - (int64_t)dx * (KW - 1) - 1;
         if (eh < 0 || ew < 0) return c->fail(ZHIP_KERNEL_COMPILATION, "max_pool2d: window larger than the padded input");
         const uint64_t e = dtype_bytes(d.dtype);
         p.n_in = 1;
@@ -710,6 +730,18 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         a.workspace_bytes = p.workspace_bytes;
         return zk::reduce(a, st);
     }
+    case ZHIP_K_ARGMAX: {
+        zk::ArgMax a{};
+        a.outer = d.dims[0];
+        a.n = d.dims[1];
+        a.inner = d.dims[2];
+        a.dtype = d.dtype;
+        a.x = ptr[0];
+        a.out = (int32_t *)ptr[1];
+        a.workspace = p.workspace;
+        a.workspace_bytes = p.workspace_bytes;
+        return zk::argmax(a, st);
+    }
     case ZHIP_K_GEMM: {
         const int64_t batch = d.dims[3] ? d.dims[3] : 1;
         const float alpha = d.fparams[0] == 0.0f ? 1.0f : d.fparams[0];
@@ -814,8 +846,8 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         zk::MaxPool2d a{};
         a.planes = d.dims[0]; a.H = (int)d.dims[1]; a.W = (int)d.dims[2]; a.KH = (int)d.dims[3]; a.KW = (int)d.dims[4];
         a.sy = d.iparams[0]; a.sx = d.iparams[1]; a.py = d.iparams[2]; a.px = d.iparams[3]; a.dy = d.iparams[4]; a.dx = d.iparams[5];
-        a.OH = (a.H + 2 * a.py - a.dy * (a.KH - 1) - 1) / a.sy + 1;
-        a.OW = (a.W + 2 * a.px - a.dx * (a.KW - 1) - 1) / a.sx + 1;
+        a.OH = (int)(((int64_t)a.H + 2 * (int64_t)a.py - (int64_t)a.dy * (a.KH - 1) - 1) / a.sy + 1);
+        a.OW = (int)(((int64_t)a.W + 2 * (int64_t)a.px - (int64_t)a.dx * (a.KW - 1) - 1) / a.sx + 1);
         a.dtype = d.dtype; a.x = ptr[0]; a.y = ptr[1];
         return zk::max_pool2d(a, st);
     }
@@ -1441,6 +1473,23 @@ ZHIP_EXPORT int32_t zhip_reduce_static(zhip_ctx *c, int32_t dtype, int32_t op, i
     a.workspace_bytes = kStaticScratchBytes;
     hipError_t e = zk::reduce(a, (hipStream_t)stream);
     if (e != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "reduce_static: launch failed: %s", hipGetErrorString(e));
+    return ZHIP_OK;
+}
+
+ZHIP_EXPORT int32_t zhip_measure_ceilings(zhip_ctx *c, uint64_t bytes, zhip_ceilings *out) {
+    static_assert(sizeof(zhip_ceilings) == sizeof(zk::Ceilings), "zhip_ceilings and zk::Ceilings are one layout");
+    if (!c) return ZHIP_DEVICE_QUERY;
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (!out || bytes < (1u << 20)) return c->fail(ZHIP_DEVICE_QUERY, "measure_ceilings: null result or fewer than 1 MiB");
+    HIPCHK(c, hipSetDevice(c->device), ZHIP_DEVICE_QUERY);
+    HIPCHK(c, hipStreamSynchronize(c->launch_streams[0]), ZHIP_KERNEL_SYNC);
+    zk::Ceilings r{};
+    hipError_t e = zk::measure_ceilings(bytes, (int)c->info.compute_units, &r, c->launch_streams[0]);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return c->fail(ZHIP_DEVICE_QUERY, "measure_ceilings failed: %s", hipGetErrorString(e));
+    }
+    memcpy(out, &r, sizeof r);
     return ZHIP_OK;
 }
 
