@@ -438,6 +438,13 @@ int32_t zhip_register_kernel(zhip_ctx *ctx, const zhip_kernel_desc *desc, zhip_p
  * Variable, a memory buffer otherwise. ZHIP_KERNEL_COMPILATION with the reason in zhip_last_error when the
  * image is malformed, uses an op this backend has no code for, or does not compile. */
 int32_t zhip_compile_ir(zhip_ctx *ctx, const void *ir, uint64_t ir_bytes, zhip_prog *prog);
+/* Code objects built at run time (zhip_compile_ir, large elementwise chains) are cached like the shared objects of
+ * the reference's C backend (zyx/src/backend/c.rs:165-186): in memory for the life of the process and on disk under
+ * $ZYX_HIP_CACHE_DIR, else $XDG_CONFIG_HOME/zyx/cache/hip, else $HOME/.config/zyx/cache/hip, keyed by a hash of the
+ * source text, the compiler options and the hiprtc version; ZYX_HIP_CACHE=0 switches the disk part off. A file that
+ * is truncated or fails its check word is ignored and rebuilt. counts[0..3] = compilations, memory hits, disk hits
+ * of this process so far. */
+void zhip_compile_cache_stats(uint64_t counts[3]);
 /* Source generation alone, no device and no context needed: checks the image and writes the HIP source
  * zhip_compile_ir would compile (ZHIP_OK), or the reason it is refused (ZHIP_KERNEL_COMPILATION), into buf
  * (up to cap - 1 bytes plus a terminator; *len = full length). */

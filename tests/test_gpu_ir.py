@@ -333,3 +333,58 @@ def test_reference_integer_matmuls_on_the_device(hip):
                 want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.int32)  # wraps like i32 accumulation
                 (g, c), = both(hip, K.matmul(m, n, k, DType.I32, DType.I32), [a, b, np.zeros((m, n), np.int32)])
                 assert np.array_equal(g, want) and np.array_equal(c, want), (m, k, n)
+
+
+def test_compiled_code_is_cached_in_memory_and_on_disk(hip, tmp_path):
+    """The reference's C backend keeps what it compiled on disk by kernel hash (zyx/src/backend/c.rs:165-186); here
+    the code object of a generated kernel is found again in memory by the same process and on disk by another one,
+    and a damaged cache file is rebuilt."""
+    import os
+    import subprocess
+    import sys
+    import time
+    from zyx_amd import backend
+    dev, pool = hip
+    old = os.environ.get("ZYX_HIP_CACHE_DIR")
+    os.environ["ZYX_HIP_CACHE_DIR"] = str(tmp_path)
+    try:
+        kernel = K.elementwise(977, 64, [UOp.Exp2, UOp.Sin, UOp.Neg])  # a shape no other test compiles
+        img = kernel.to_bytes()
+        s0 = backend.compile_cache_stats()
+        t0 = time.perf_counter()
+        p1 = dev.compile(img)
+        t1 = time.perf_counter()
+        p2 = dev.compile(img)
+        t2 = time.perf_counter()
+        s1 = backend.compile_cache_stats()
+        assert s1["compiled"] == s0["compiled"] + 1 and s1["memory_hits"] == s0["memory_hits"] + 1
+        assert t2 - t1 < 0.05 and t2 - t1 < t1 - t0
+        files = [f for f in os.listdir(tmp_path) if f.endswith(".hsaco")]
+        assert len(files) == 1
+        dev.release(p1)
+        dev.release(p2)
+        # another process finds the file; after the file is cut short it compiles again and repairs it
+        child = ("import sys, numpy as np; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+                 "import zyx_amd, ir_kernels as K\n"
+                 "from zyx_amd import backend\n"
+                 "from zyx_amd.ir import UOp\n"
+                 "pools, devs = zyx_amd.initialize_device(zyx_amd.HIPConfig(device_ids=[0]))\n"
+                 "devs[0].compile(K.elementwise(977, 64, [UOp.Exp2, UOp.Sin, UOp.Neg]).to_bytes())\n"
+                 "s = backend.compile_cache_stats(); print(s['compiled'], s['disk_hits'])\n"
+                 "pools[0].deinitialize()\n") % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                                                os.path.dirname(os.path.abspath(__file__)))
+        out = subprocess.run([sys.executable, "-c", child], capture_output=True, text=True, timeout=100, env=dict(os.environ))
+        assert out.returncode == 0, out.stderr[-2000:]
+        assert out.stdout.split()[-2:] == ["0", "1"]
+        path = os.path.join(tmp_path, files[0])
+        whole = open(path, "rb").read()
+        open(path, "wb").write(whole[:len(whole) // 2])
+        out = subprocess.run([sys.executable, "-c", child], capture_output=True, text=True, timeout=100, env=dict(os.environ))
+        assert out.returncode == 0, out.stderr[-2000:]
+        assert out.stdout.split()[-2:] == ["1", "0"]
+        assert len(open(path, "rb").read()) >= len(whole) // 2 + 1 and not [f for f in os.listdir(tmp_path) if ".tmp" in f]
+    finally:
+        if old is None:
+            del os.environ["ZYX_HIP_CACHE_DIR"]
+        else:
+            os.environ["ZYX_HIP_CACHE_DIR"] = old

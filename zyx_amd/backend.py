@@ -135,7 +135,7 @@ _lib = None
 _EXPORTS = ["zhip_device_count", "zhip_init", "zhip_deinit", "zhip_last_error", "zhip_get_device_info",
             "zhip_free_bytes", "zhip_free_compute", "zhip_alloc", "zhip_free", "zhip_store_variable",
             "zhip_get_variable", "zhip_h2d", "zhip_d2h", "zhip_d2d", "zhip_sync_events", "zhip_release_events",
-            "zhip_buffer_ptr", "zhip_register_kernel", "zhip_compile_ir", "zhip_ir_generate", "zhip_program_source", "zhip_launch",
+            "zhip_buffer_ptr", "zhip_register_kernel", "zhip_compile_ir", "zhip_compile_cache_stats", "zhip_ir_generate", "zhip_program_source", "zhip_launch",
             "zhip_release_program",
             "zhip_rng_seed", "zhip_rng_next_u64", "zhip_rng_fill", "zhip_reduce_static", "zhip_measure_ceilings", "zhip_time_kernel", "zhip_profile_kernel", "zhip_plan_create", "zhip_plan_launch", "zhip_plan_destroy"]
 
@@ -435,6 +435,14 @@ def generate_source(kernel_ir: bytes) -> str:
     if rc != 0:
         raise BackendError(ErrorStatus(rc), buf.value.decode())
     return buf.value.decode()
+
+
+def compile_cache_stats() -> dict:
+    """Run-time compilations, in-memory hits and on-disk hits of this process (zhip_compile_cache_stats)."""
+    lib = load_library()
+    raw = (C.c_uint64 * 3)()
+    lib.zhip_compile_cache_stats(raw)
+    return {"compiled": raw[0], "memory_hits": raw[1], "disk_hits": raw[2]}
 
 
 def device_count() -> int:

@@ -10,7 +10,7 @@
 // keeps U x (full-tensor operands) 128-bit loads in flight; streaming accesses are non-temporal.
 #include "kernels/kernels.hpp"
 
-#include <hip/hiprtc.h>
+#include "rtc_cache.hpp"
 
 #include <cstdarg>
 #include <cstdio>
@@ -221,35 +221,18 @@ EwJit *ew_jit_compile(const Elementwise &p, std::string &err) {
     for (int k = 0; k < p.n_in; k++) n_full += p.in_bcast[k] == 0;
     const int U = n_full <= 2 ? 4 : 2;
     const std::string src = ew_jit_source(p, V, U);
-    hiprtcProgram prog;
-    if (hiprtcCreateProgram(&prog, src.c_str(), "zk_ew.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
-        err = "hiprtcCreateProgram failed";
-        return nullptr;
-    }
     // same code generation switches as the ahead-of-time kernels: gfx950, packed-FP32 instructions off
     // -ffp-contract=on: a*b+c fuses only inside one source expression, as in the interpreting kernel's build,
     // never across two ops of the chain
-    const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=on", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
-    const hiprtcResult rc = hiprtcCompileProgram(prog, (int)(sizeof opts / sizeof opts[0]), opts);
-    if (rc != HIPRTC_SUCCESS) {
-        size_t ls = 0;
-        hiprtcGetProgramLogSize(prog, &ls);
-        std::string log(ls, 0);
-        if (ls) hiprtcGetProgramLog(prog, &log[0]);
-        err = std::string("hiprtc: ") + hiprtcGetErrorString(rc) + ": " + log.substr(0, 600);
-        hiprtcDestroyProgram(&prog);
-        return nullptr;
-    }
-    size_t cs = 0;
-    hiprtcGetCodeSize(prog, &cs);
-    std::vector<char> code(cs);
-    hiprtcGetCode(prog, code.data());
-    hiprtcDestroyProgram(&prog);
+    const std::vector<const char *> opts = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=on",
+                                            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+    const auto code = rtc_compile(src, opts, "zk_ew.hip", err);
+    if (!code) return nullptr;
     EwJit *j = new EwJit();
     j->V = V;
     j->U = U;
     j->nvec = p.rows * p.cols / V;
-    hipError_t e = hipModuleLoadData(&j->mod, code.data());
+    hipError_t e = hipModuleLoadData(&j->mod, code->data());
     if (e == hipSuccess) e = hipModuleGetFunction(&j->fn, j->mod, "zk_ew");
     if (e != hipSuccess) {
         err = std::string("module load: ") + hipGetErrorString(e);

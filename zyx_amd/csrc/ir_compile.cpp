@@ -8,7 +8,7 @@
 // Mad (-ffp-contract=off), so kernels without Mad round exactly like the scalar C loop.
 #include "ir_compile.hpp"
 
-#include <hip/hiprtc.h>
+#include "rtc_cache.hpp"
 
 #include <cmath>
 #include <cstdarg>
@@ -618,32 +618,15 @@ IrProgram *ir_compile(const void *image, uint64_t bytes, std::string &err) {
         delete p;
         return nullptr;
     }
-    hiprtcProgram prog;
-    if (hiprtcCreateProgram(&prog, p->source.c_str(), "zir_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
-        err = "hiprtcCreateProgram failed";
-        delete p;
-        return nullptr;
-    }
     // gfx950 only, packed-FP32 instructions off like every kernel of this library; no contraction, wrapping ints
-    const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fwrapv",
-                          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
-    const hiprtcResult rc = hiprtcCompileProgram(prog, (int)(sizeof opts / sizeof opts[0]), opts);
-    if (rc != HIPRTC_SUCCESS) {
-        size_t ls = 0;
-        hiprtcGetProgramLogSize(prog, &ls);
-        std::string log(ls, 0);
-        if (ls) hiprtcGetProgramLog(prog, &log[0]);
-        err = std::string("hiprtc: ") + hiprtcGetErrorString(rc) + ": " + log.substr(0, 800);
-        hiprtcDestroyProgram(&prog);
+    const std::vector<const char *> opts = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fwrapv",
+                                            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+    const auto code = rtc_compile(p->source, opts, "zir_kernel.hip", err);
+    if (!code) {
         delete p;
         return nullptr;
     }
-    size_t cs = 0;
-    hiprtcGetCodeSize(prog, &cs);
-    std::vector<char> code(cs);
-    hiprtcGetCode(prog, code.data());
-    hiprtcDestroyProgram(&prog);
-    hipError_t e = hipModuleLoadData(&p->mod, code.data());
+    hipError_t e = hipModuleLoadData(&p->mod, code->data());
     if (e == hipSuccess) e = hipModuleGetFunction(&p->fn, p->mod, "zir_kernel");
     if (e != hipSuccess) {
         err = std::string("loading the compiled kernel failed: ") + hipGetErrorString(e);

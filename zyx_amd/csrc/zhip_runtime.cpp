@@ -31,6 +31,7 @@
 #include <vector>
 
 #include "ir_compile.hpp"
+#include "rtc_cache.hpp"
 #include "kernels/kernels.hpp"
 
 #define ZHIP_EXPORT extern "C" __attribute__((visibility("default")))
@@ -1350,6 +1351,13 @@ ZHIP_EXPORT int32_t zhip_compile_ir(zhip_ctx *c, const void *ir, uint64_t ir_byt
     *prog = c->programs.push(p);
     if (c->debug & 128) fprintf(stderr, "[zyx-hip] program %u = generated kernel, %zu parameters\n", *prog, k->params.size());
     return ZHIP_OK;
+}
+
+ZHIP_EXPORT void zhip_compile_cache_stats(uint64_t counts[3]) {
+    const zk::RtcCacheStats s = zk::rtc_cache_stats();
+    counts[0] = s.compiled;
+    counts[1] = s.memory_hits;
+    counts[2] = s.disk_hits;
 }
 
 ZHIP_EXPORT int32_t zhip_ir_generate(const void *ir, uint64_t ir_bytes, char *buf, uint64_t cap, uint64_t *len) {
