@@ -46,8 +46,25 @@ constexpr uint64_t kStaticScratchBytes = 1ull << 20;
 
 thread_local std::string g_init_error;
 
+constexpr int kStreams = kLaunchStreams + 2; // launch streams, then the pool stream, then the plan stream
+
+// Where in which stream a buffer was last written and, per stream, last read. The caller's events say what an
+// operation must wait for -- but zyx files one event under ALL buffers of a kernel and consumes it on the first later
+// use of ANY of them (zyx/src/runtime.rs:1-16, zyx/src/graph/plan.rs:311-327), so a buffer can lose its event to an
+// operation that never touched it. The backend therefore keeps its own record and orders every operation after the
+// conflicting accesses of its buffers, whatever the wait list holds; stream positions suffice (no event objects).
+struct Stamp {
+    int16_t stream = -3; // stream index as in stream_of(); -3 = none
+    uint64_t seq = 0;
+};
+struct Access {
+    Stamp writer;
+    uint64_t read_seq[kStreams] = {0}; // latest read per stream slot, 0 = none since the last write
+};
+
 struct Buffer {
     enum Kind : uint8_t { Free, Memory, Variable } kind = Free;
+    Access acc;
     void *ptr = nullptr;
     uint64_t bytes = 0;    // what the caller asked for (bookkeeping unit of free_bytes)
     uint64_t capacity = 0; // size class actually backing it
@@ -67,11 +84,13 @@ struct EventSlot {
     // a same-stream wait is skipped) never pays for a record. No wait cycle can arise: whatever was enqueued between
     // the position and the record only waits for events that existed before it, hence before the new waiter.
     bool recorded = false;
+    uint64_t covers = 0; // once recorded: the position of its stream the record stands for (>= seq)
 };
 
 struct CachedBlock {
     void *ptr;
     std::vector<zhip_event> pending; // last users; owned by the cache
+    Access acc;                      // and where they ran: the next owner's first operation is ordered after them
 };
 
 struct Program {
@@ -96,6 +115,7 @@ struct Plan {
     hipGraphExec_t exec = nullptr;
     size_t n_nodes = 0;
     std::vector<zhip_prog> progs; // distinct programs of the plan
+    std::vector<std::pair<zhip_buf, bool>> uses; // every memory buffer of the plan once; true = some node writes it
 };
 
 template <class T> struct Slab { // dense ids, lowest free id reused (zyx/src/slab.rs)
@@ -136,7 +156,12 @@ struct zhip_ctx {
 
     hipStream_t pool_stream = nullptr;
     hipStream_t launch_streams[kLaunchStreams] = {nullptr};
-    uint64_t stream_seq[kLaunchStreams + 2] = {0}; // [kLaunchStreams] = pool stream, [+1] = plan stream
+    uint64_t stream_seq[kStreams] = {0}; // [kLaunchStreams] = pool stream, [+1] = plan stream
+    // seen[w][s]: stream w is ordered after everything stream s held up to this position (through a wait that was
+    // enqueued in w); done[s]: the host has seen stream s complete up to this position
+    uint64_t seen[kStreams][kStreams] = {{0}};
+    uint64_t done[kStreams] = {0};
+    hipEvent_t order_ev[kStreams] = {nullptr}; // one per source stream, re-recorded for every cross-stream ordering
     int rr = 0;
 
     uint64_t free_bytes = 0;
@@ -172,6 +197,9 @@ struct zhip_ctx {
 
 namespace {
 
+int slot_of(int stream_idx);
+hipStream_t stream_of(zhip_ctx *c, int idx);
+
 uint64_t size_class(uint64_t bytes) {
     if (bytes < kAllocAlign) return kAllocAlign;
     // 8 classes per power of two: at most 12.5% slack, few distinct sizes to cache
@@ -185,6 +213,47 @@ uint64_t size_class(uint64_t bytes) {
 hipStream_t stream_of(zhip_ctx *c, int idx) {
     return idx == -1 ? c->pool_stream : idx == -2 ? c->plan_stream : c->launch_streams[idx];
 }
+
+// Stream slot w now runs after stream slot `from` up to position `upto`, hence also after whatever `from` had been
+// ordered after by then. (What `from` waits for later does not carry over; the table only ever under-states.)
+void note_ordered(zhip_ctx *c, int w, int from, uint64_t upto) {
+    if (c->seen[w][from] < upto) c->seen[w][from] = upto;
+    if (upto >= c->stream_seq[from]) // ordered after the stream's present end: its own waits carry over
+        for (int k = 0; k < kStreams; k++)
+            if (k != w && c->seen[w][k] < c->seen[from][k]) c->seen[w][k] = c->seen[from][k];
+}
+
+// Orders stream `stream_idx` after position `st`: nothing to do inside one stream, or when a wait already enqueued
+// there, or the host, covers the position; else the source stream's ordering event is recorded at its present end
+// (at or after the position) and waited for.
+int32_t order_after(zhip_ctx *c, int stream_idx, const Stamp &st, int32_t status) {
+    if (st.stream == -3 || st.stream == stream_idx) return ZHIP_OK;
+    const int w = slot_of(stream_idx), from = slot_of(st.stream);
+    if (c->seen[w][from] >= st.seq || c->done[from] >= st.seq) return ZHIP_OK;
+    HIPCHK(c, hipEventRecord(c->order_ev[from], stream_of(c, st.stream)), status);
+    HIPCHK(c, hipStreamWaitEvent(stream_of(c, stream_idx), c->order_ev[from], 0), status);
+    note_ordered(c, w, from, c->stream_seq[from]);
+    return ZHIP_OK;
+}
+// Before an operation in `stream_idx` reads (write == false) or writes a buffer: after its writer, and a write also
+// after every reader.
+int32_t order_access(zhip_ctx *c, int stream_idx, const Access &a, bool write, int32_t status) {
+    int32_t rc = order_after(c, stream_idx, a.writer, status);
+    for (int k = 0; k < kStreams && write && rc == ZHIP_OK; k++)
+        if (a.read_seq[k]) rc = order_after(c, stream_idx, Stamp{(int16_t)(k == kLaunchStreams ? -1 : k == kLaunchStreams + 1 ? -2 : k), a.read_seq[k]}, status);
+    return rc;
+}
+// After it was enqueued at position seq.
+void stamp_access(Access &a, int stream_idx, uint64_t seq, bool write) {
+    if (write) {
+        a = Access();
+        a.writer = Stamp{(int16_t)stream_idx, seq};
+    } else {
+        a.read_seq[slot_of(stream_idx)] = seq;
+    }
+}
+
+int slot_of(int stream_idx) { return stream_idx == -1 ? kLaunchStreams : stream_idx == -2 ? kLaunchStreams + 1 : stream_idx; }
 
 // --- events ---------------------------------------------------------------------
 EventSlot *event_lookup(zhip_ctx *c, zhip_event h) {
@@ -209,7 +278,8 @@ int32_t event_record(zhip_ctx *c, int stream_idx, int32_t status, zhip_event *ou
     s.live = true;
     s.recorded = false;
     s.stream = (int16_t)stream_idx;
-    s.seq = ++c->stream_seq[stream_idx == -1 ? kLaunchStreams : stream_idx == -2 ? kLaunchStreams + 1 : stream_idx];
+    s.seq = ++c->stream_seq[slot_of(stream_idx)];
+    s.covers = 0;
     *out = ((uint64_t)s.gen << 32) | (uint64_t)(idx + 1);
     return ZHIP_OK;
 }
@@ -217,7 +287,10 @@ int32_t event_record(zhip_ctx *c, int stream_idx, int32_t status, zhip_event *ou
 hipError_t event_materialise(zhip_ctx *c, EventSlot *s) {
     if (s->recorded) return hipSuccess;
     hipError_t e = hipEventRecord(s->ev, stream_of(c, s->stream));
-    if (e == hipSuccess) s->recorded = true;
+    if (e == hipSuccess) {
+        s->recorded = true;
+        s->covers = c->stream_seq[slot_of(s->stream)]; // the stream's end as it is now
+    }
     return e;
 }
 void event_retire(zhip_ctx *c, EventSlot *s) {
@@ -232,7 +305,7 @@ int32_t wait_and_consume(zhip_ctx *c, int stream_idx, const zhip_event *evs, siz
     int32_t rc = ZHIP_OK;
     // Streams run in order: of several events recorded on one stream only the latest needs a wait (a cross-stream
     // wait is the expensive part of a launch on the host). Slot -1 / -2 are the pool and plan streams.
-    EventSlot *latest[kLaunchStreams + 2] = {nullptr};
+    EventSlot *latest[kStreams] = {nullptr};
     for (size_t i = 0; i < n; i++) {
         if (evs[i] == 0) continue;
         EventSlot *s = event_lookup(c, evs[i]);
@@ -241,15 +314,18 @@ int32_t wait_and_consume(zhip_ctx *c, int stream_idx, const zhip_event *evs, siz
             continue;
         }
         if (s->stream != stream_idx) {
-            EventSlot *&l = latest[s->stream == -1 ? kLaunchStreams : s->stream == -2 ? kLaunchStreams + 1 : s->stream];
+            EventSlot *&l = latest[slot_of(s->stream)];
             if (!l || s->seq > l->seq) l = s;
         }
     }
     for (EventSlot *s : latest)
         if (s) {
+            const int w = slot_of(stream_idx), from = slot_of(s->stream);
+            if (c->seen[w][from] >= s->seq || c->done[from] >= s->seq) continue; // already ordered after that position
             hipError_t e = event_materialise(c, s);
             if (e == hipSuccess) e = hipStreamWaitEvent(stream_of(c, stream_idx), s->ev, 0);
             if (e != hipSuccess) rc = c->fail(status, "hipStreamWaitEvent failed: %s", hipGetErrorString(e));
+            else note_ordered(c, w, from, s->covers);
         }
     for (size_t i = 0; i < n; i++)
         if (evs[i] != 0)
@@ -929,7 +1005,29 @@ int32_t resolve_args(zhip_ctx *c, zhip_prog prog, const zhip_buf *args, size_t n
     return ZHIP_OK;
 }
 
-int pick_stream(zhip_ctx *c, const zhip_event *evs, size_t n) {
+// The buffers of a launch: inputs are read, outputs written (a generated kernel may read its outputs as well: a write
+// is ordered after everything anyway). Scalar variables are not memory.
+int32_t order_args(zhip_ctx *c, int stream_idx, const Program &p, const zhip_buf *args, size_t n_args, int32_t status) {
+    for (size_t i = 0; i < n_args; i++) {
+        Buffer *b = buffer_lookup(c, args[i]);
+        if (!b || b->kind != Buffer::Memory) continue;
+        const bool write = p.ir ? p.ir->params[i].kind == ZHIP_IR_GLOBAL_MUT : i >= (size_t)p.n_in;
+        int32_t rc = order_access(c, stream_idx, b->acc, write, status);
+        if (rc != ZHIP_OK) return rc;
+    }
+    return ZHIP_OK;
+}
+void stamp_args(zhip_ctx *c, int stream_idx, uint64_t seq, const Program &p, const zhip_buf *args, size_t n_args) {
+    for (int pass = 0; pass < 2; pass++) // reads first: a buffer that is input and output ends up written
+        for (size_t i = 0; i < n_args; i++) {
+            Buffer *b = buffer_lookup(c, args[i]);
+            if (!b || b->kind != Buffer::Memory) continue;
+            const bool write = p.ir ? p.ir->params[i].kind == ZHIP_IR_GLOBAL_MUT : i >= (size_t)p.n_in;
+            if (write == (pass == 1)) stamp_access(b->acc, stream_idx, seq, write);
+        }
+}
+
+int pick_stream(zhip_ctx *c, const zhip_event *evs, size_t n, const zhip_buf *args, size_t n_args) {
     int best = -1;
     uint64_t best_seq = 0;
     for (size_t i = 0; i < n; i++)
@@ -939,6 +1037,11 @@ int pick_stream(zhip_ctx *c, const zhip_event *evs, size_t n) {
                 best_seq = s->seq;
             }
     if (best >= 0) return best;
+    // no event names a launch stream: follow the stream that last wrote one of the buffers (outputs first), where the
+    // launch needs no cross-stream wait for it
+    for (size_t i = n_args; i-- > 0;)
+        if (Buffer *b = buffer_lookup(c, args[i]))
+            if (b->kind == Buffer::Memory && b->acc.writer.stream >= 0 && c->done[b->acc.writer.stream] < b->acc.writer.seq) return b->acc.writer.stream;
     c->rr = (c->rr + 1) % kLaunchStreams;
     return c->rr;
 }
@@ -1039,6 +1142,8 @@ ZHIP_EXPORT int32_t zhip_init(const zhip_config *cfg, zhip_ctx **out) {
     if ((e = hipEventCreate(&c->prof_a)) != hipSuccess || (e = hipEventCreate(&c->prof_b)) != hipSuccess ||
         (e = hipEventCreateWithFlags(&c->plan_done, hipEventDisableTiming)) != hipSuccess)
         return bail(ZHIP_INITIALIZATION, "hipEventCreate", e);
+    for (int k = 0; k < kStreams; k++)
+        if ((e = hipEventCreateWithFlags(&c->order_ev[k], hipEventDisableTiming)) != hipSuccess) return bail(ZHIP_INITIALIZATION, "hipEventCreate", e);
     if ((e = hipGetSymbolAddress((void **)&c->static_scratch, HIP_SYMBOL(scratch))) != hipSuccess || !c->static_scratch)
         return bail(ZHIP_INITIALIZATION, "hipGetSymbolAddress of the static scratch array", e);
     if ((e = zk::gemm_bf16_init()) != hipSuccess) return bail(ZHIP_INITIALIZATION, "raising the LDS limit of the GEMM kernels", e);
@@ -1078,6 +1183,8 @@ ZHIP_EXPORT int32_t zhip_deinit(zhip_ctx *c) {
         (void)hipEventDestroy(c->prof_a);
         (void)hipEventDestroy(c->prof_b);
         if (c->plan_done) (void)hipEventDestroy(c->plan_done);
+        for (hipEvent_t ev : c->order_ev)
+            if (ev) (void)hipEventDestroy(ev);
         (void)hipStreamDestroy(c->pool_stream);
         for (auto s : c->launch_streams) (void)hipStreamDestroy(s);
     }
@@ -1117,6 +1224,7 @@ ZHIP_EXPORT int32_t zhip_alloc(zhip_ctx *c, uint64_t bytes, zhip_buf *buf, zhip_
         if (it->second.empty()) c->cache.erase(it);
         c->cached_bytes -= cap;
         b.ptr = blk.ptr;
+        b.acc = blk.acc; // the first operation on the new buffer is ordered after the block's last users
         if (!blk.pending.empty()) {
             // the previous users' completion becomes the new owner's first dependency
             int32_t rc = wait_and_consume(c, -1, blk.pending.data(), blk.pending.size(), ZHIP_MEMORY_ALLOCATION);
@@ -1156,7 +1264,7 @@ ZHIP_EXPORT int32_t zhip_free(zhip_ctx *c, zhip_buf id, const zhip_event *evs, s
         return ZHIP_OK;
     }
     (void)hipSetDevice(c->device);
-    CachedBlock blk{b->ptr, {}};
+    CachedBlock blk{b->ptr, {}, b->acc};
     for (size_t i = 0; i < n; i++)
         if (evs[i] != 0 && event_lookup(c, evs[i])) blk.pending.push_back(evs[i]);
     c->free_bytes += b->bytes;
@@ -1207,8 +1315,12 @@ ZHIP_EXPORT int32_t zhip_h2d(zhip_ctx *c, const void *src, uint64_t bytes, zhip_
     if (bytes > b->bytes)
         return c->fail(ZHIP_MEMORY_COPY_H2P, "copy of %llu bytes into buffer %u of %llu bytes", (unsigned long long)bytes,
                        dst, (unsigned long long)b->bytes);
+    rc = order_access(c, -1, b->acc, true, ZHIP_MEMORY_COPY_H2P);
+    if (rc != ZHIP_OK) return rc;
     if (bytes) HIPCHK(c, hipMemcpyAsync(b->ptr, src, bytes, hipMemcpyHostToDevice, c->pool_stream), ZHIP_MEMORY_COPY_H2P);
-    return event_record(c, -1, ZHIP_MEMORY_COPY_H2P, ev);
+    rc = event_record(c, -1, ZHIP_MEMORY_COPY_H2P, ev);
+    stamp_access(b->acc, -1, c->stream_seq[kLaunchStreams], true);
+    return rc;
 }
 
 ZHIP_EXPORT int32_t zhip_d2h(zhip_ctx *c, zhip_buf src, void *dst, uint64_t bytes, const zhip_event *evs, size_t n) {
@@ -1221,8 +1333,14 @@ ZHIP_EXPORT int32_t zhip_d2h(zhip_ctx *c, zhip_buf src, void *dst, uint64_t byte
     if (bytes > b->bytes)
         return c->fail(ZHIP_MEMORY_COPY_P2H, "copy of %llu bytes out of buffer %u of %llu bytes", (unsigned long long)bytes,
                        src, (unsigned long long)b->bytes);
+    rc = order_access(c, -1, b->acc, false, ZHIP_MEMORY_COPY_P2H);
+    if (rc != ZHIP_OK) return rc;
     if (bytes) HIPCHK(c, hipMemcpyAsync(dst, b->ptr, bytes, hipMemcpyDeviceToHost, c->pool_stream), ZHIP_MEMORY_COPY_P2H);
     HIPCHK(c, hipStreamSynchronize(c->pool_stream), ZHIP_MEMORY_COPY_P2H);
+    // the pool stream has drained, and with it everything it was ordered after
+    c->done[kLaunchStreams] = c->stream_seq[kLaunchStreams];
+    for (int k = 0; k < kStreams; k++)
+        if (c->done[k] < c->seen[kLaunchStreams][k]) c->done[k] = c->seen[kLaunchStreams][k];
     return ZHIP_OK;
 }
 
@@ -1240,6 +1358,9 @@ ZHIP_EXPORT int32_t zhip_d2d(zhip_ctx *c, zhip_buf src, uint64_t src_off, zhip_b
     if (src_off > s->bytes || bytes > s->bytes - src_off || dst_off > d->bytes || bytes > d->bytes - dst_off)
         return c->fail(ZHIP_MEMORY_COPY_H2P, "d2d: %llu bytes at offsets %llu -> %llu exceed a buffer", (unsigned long long)bytes,
                        (unsigned long long)src_off, (unsigned long long)dst_off);
+    rc = order_access(c, -1, s->acc, false, ZHIP_MEMORY_COPY_H2P);
+    if (rc == ZHIP_OK) rc = order_access(c, -1, d->acc, true, ZHIP_MEMORY_COPY_H2P);
+    if (rc != ZHIP_OK) return rc;
     if (bytes) {
         char *to = (char *)d->ptr + dst_off;
         const char *from = (const char *)s->ptr + src_off;
@@ -1249,7 +1370,10 @@ ZHIP_EXPORT int32_t zhip_d2d(zhip_ctx *c, zhip_buf src, uint64_t src_off, zhip_b
         if (bytes <= (4u << 20) && !overlap) HIPCHK(c, zk::copy_range(to, from, bytes, c->pool_stream), ZHIP_MEMORY_COPY_H2P);
         else HIPCHK(c, hipMemcpyAsync(to, from, bytes, hipMemcpyDeviceToDevice, c->pool_stream), ZHIP_MEMORY_COPY_H2P);
     }
-    return event_record(c, -1, ZHIP_MEMORY_COPY_H2P, ev);
+    rc = event_record(c, -1, ZHIP_MEMORY_COPY_H2P, ev);
+    if (s != d) stamp_access(s->acc, -1, c->stream_seq[kLaunchStreams], false);
+    stamp_access(d->acc, -1, c->stream_seq[kLaunchStreams], true);
+    return rc;
 }
 
 ZHIP_EXPORT int32_t zhip_sync_events(zhip_ctx *c, const zhip_event *evs, size_t n) {
@@ -1265,6 +1389,10 @@ ZHIP_EXPORT int32_t zhip_sync_events(zhip_ctx *c, const zhip_event *evs, size_t 
         hipError_t e = event_materialise(c, s);
         if (e == hipSuccess) e = hipEventSynchronize(s->ev);
         if (e != hipSuccess) rc = c->fail(ZHIP_KERNEL_SYNC, "hipEventSynchronize failed: %s", hipGetErrorString(e));
+        else {
+            const int from = slot_of(s->stream);
+            if (c->done[from] < s->covers) c->done[from] = s->covers;
+        }
         event_retire(c, s);
     }
     return rc;
@@ -1437,8 +1565,9 @@ ZHIP_EXPORT int32_t zhip_launch(zhip_ctx *c, zhip_prog prog, const zhip_buf *arg
         return rc;
     }
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
-    int si = pick_stream(c, evs, n_evs);
+    int si = pick_stream(c, evs, n_evs, args, n_args);
     rc = wait_and_consume(c, si, evs, n_evs, ZHIP_KERNEL_LAUNCH);
+    if (rc == ZHIP_OK) rc = order_args(c, si, *p, args, n_args, ZHIP_KERNEL_LAUNCH);
     if (rc != ZHIP_OK) return rc;
     if (c->debug & 32) fprintf(stderr, "[zyx-hip] launch program %u (kind %d) on stream %d\n", prog, p->desc.kind, si);
     if (p->ws_event && p->ws_last)
@@ -1449,7 +1578,9 @@ ZHIP_EXPORT int32_t zhip_launch(zhip_ctx *c, zhip_prog prog, const zhip_buf *arg
         HIPCHK(c, hipEventRecord(p->ws_event, c->launch_streams[si]), ZHIP_KERNEL_LAUNCH);
         p->ws_last = 1;
     }
-    return event_record(c, si, ZHIP_KERNEL_LAUNCH, ev);
+    rc = event_record(c, si, ZHIP_KERNEL_LAUNCH, ev);
+    stamp_args(c, si, c->stream_seq[si], *p, args, n_args);
+    return rc;
 }
 
 ZHIP_EXPORT int32_t zhip_reduce_static(zhip_ctx *c, int32_t dtype, int32_t op, int32_t axis0, int64_t rows, int64_t cols,
@@ -1511,11 +1642,15 @@ ZHIP_EXPORT int32_t zhip_time_kernel(zhip_ctx *c, zhip_prog prog, const zhip_buf
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
     hipStream_t st = c->launch_streams[0];
     if (p->ws_event && p->ws_last) HIPCHK(c, hipEventSynchronize(p->ws_last == 2 ? c->plan_done : p->ws_event), ZHIP_KERNEL_SYNC);
+    rc = order_args(c, 0, *p, args, n_args, ZHIP_KERNEL_LAUNCH);
+    if (rc != ZHIP_OK) return rc;
     HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
     auto t0 = std::chrono::steady_clock::now();
     hipError_t e = program_enqueue(*p, ptr, st);
     if (e != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "launch of program %u failed: %s", prog, hipGetErrorString(e));
     HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
+    stamp_args(c, 0, ++c->stream_seq[0], *p, args, n_args);
+    c->done[0] = c->stream_seq[0];
     *ns = (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t0).count();
     return ZHIP_OK;
 }
@@ -1534,6 +1669,10 @@ ZHIP_EXPORT int32_t zhip_profile_kernel(zhip_ctx *c, zhip_prog prog, const zhip_
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
     hipStream_t st = c->launch_streams[0];
     if (p->ws_event && p->ws_last) HIPCHK(c, hipEventSynchronize(p->ws_last == 2 ? c->plan_done : p->ws_event), ZHIP_KERNEL_SYNC);
+    for (size_t s = 0; s < arg_sets; s++) {
+        int32_t rc = order_args(c, 0, *p, args + s * n_args, n_args, ZHIP_KERNEL_LAUNCH);
+        if (rc != ZHIP_OK) return rc;
+    }
     HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
     HIPCHK(c, hipEventRecord(c->prof_a, st), ZHIP_KERNEL_LAUNCH);
     for (int32_t i = 0; i < iters; i++) {
@@ -1545,6 +1684,9 @@ ZHIP_EXPORT int32_t zhip_profile_kernel(zhip_ctx *c, zhip_prog prog, const zhip_
     float ms = 0.0f;
     HIPCHK(c, hipEventElapsedTime(&ms, c->prof_a, c->prof_b), ZHIP_KERNEL_SYNC);
     *avg_us = ms * 1000.0f / (float)iters;
+    ++c->stream_seq[0];
+    for (size_t s = 0; s < arg_sets; s++) stamp_args(c, 0, c->stream_seq[0], *p, args + s * n_args, n_args);
+    c->done[0] = c->stream_seq[0]; // the second event was waited for
     return ZHIP_OK;
 }
 
@@ -1584,6 +1726,20 @@ ZHIP_EXPORT int32_t zhip_plan_create(zhip_ctx *c, const zhip_prog *progs, const 
     for (size_t i = 0; i < n_nodes; i++)
         if (std::find(pl.progs.begin(), pl.progs.end(), progs[i]) == pl.progs.end()) pl.progs.push_back(progs[i]);
     for (zhip_prog q : pl.progs) c->programs.items[q].plan_refs++;
+    off = 0;
+    for (size_t i = 0; i < n_nodes; i++) {
+        const Program &pr = *ps[i];
+        for (size_t a = 0; a < n_args[i]; a++) {
+            const zhip_buf id = args_flat[off + a];
+            Buffer *b = buffer_lookup(c, id);
+            if (!b || b->kind != Buffer::Memory) continue;
+            const bool write = pr.ir ? pr.ir->params[a].kind == ZHIP_IR_GLOBAL_MUT : a >= (size_t)pr.n_in;
+            auto it = std::find_if(pl.uses.begin(), pl.uses.end(), [id](const std::pair<zhip_buf, bool> &u) { return u.first == id; });
+            if (it == pl.uses.end()) pl.uses.push_back({id, write});
+            else it->second = it->second || write;
+        }
+        off += n_args[i];
+    }
     *plan = c->plans.push(pl);
     return ZHIP_OK;
 }
@@ -1610,6 +1766,11 @@ ZHIP_EXPORT int32_t zhip_plan_launch(zhip_ctx *c, zhip_plan plan, const zhip_eve
         any_ws = true;
         if (pr.ws_last == 1) HIPCHK(c, hipStreamWaitEvent(c->plan_stream, pr.ws_event, 0), ZHIP_KERNEL_LAUNCH);
     }
+    for (const auto &u : pl.uses)
+        if (Buffer *b = buffer_lookup(c, u.first)) {
+            rc = order_access(c, -2, b->acc, u.second, ZHIP_KERNEL_LAUNCH);
+            if (rc != ZHIP_OK) return rc;
+        }
     HIPCHK(c, hipGraphLaunch(pl.exec, c->plan_stream), ZHIP_KERNEL_LAUNCH);
     if (any_ws) {
         HIPCHK(c, hipEventRecord(c->plan_done, c->plan_stream), ZHIP_KERNEL_LAUNCH);
@@ -1619,6 +1780,8 @@ ZHIP_EXPORT int32_t zhip_plan_launch(zhip_ctx *c, zhip_plan plan, const zhip_eve
     // A plan is a coarse unit whose end other streams typically wait for while the next plan is already queued (batch
     // copies of a training loop): its event is recorded right here, so that such a wait covers this plan only.
     int32_t rc2 = event_record(c, -2, ZHIP_KERNEL_LAUNCH, ev);
+    for (const auto &u : pl.uses)
+        if (Buffer *b = buffer_lookup(c, u.first)) stamp_access(b->acc, -2, c->stream_seq[kLaunchStreams + 1], u.second);
     if (rc2 == ZHIP_OK)
         if (EventSlot *s = event_lookup(c, *ev))
             if (event_materialise(c, s) != hipSuccess) return c->fail(ZHIP_KERNEL_LAUNCH, "hipEventRecord failed");
