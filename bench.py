@@ -79,6 +79,26 @@ def extra_gemm(dev, pool, kernels, steps=100, warmup=200):
         dev.release(prog)
     for b_ in (ab, bb, biasb, cb):
         pool.deallocate(b_, [])
+    # the other operand dtypes of Tensor::dot: f16 on the same LDS-tiled kernel, f32 (what the reference's own AOT
+    # matchers claim, zyx/src/backend/cblas.rs:265-268; zyx/tests/05_misc.rs:820-842 multiplies 1024^3) at 1024^3 and 4096^3
+    import zyx_amd
+    to_f16 = lambda x: x.astype(np.float16).view(np.uint16)
+    for name, dt, n2, peak, conv in (("f16_4096", zyx_amd.DType.F16, 4096, 2500.0, to_f16),
+                                     ("f32_1024", zyx_amd.DType.F32, 1024, 157.3, lambda x: x),
+                                     ("f32_4096", zyx_amd.DType.F32, 4096, 157.3, lambda x: x)):
+        a2, b2 = conv(rng.uniform((n2, n2), -1, 1)), conv(rng.uniform((n2, n2), -1, 1))
+        ab, e1 = kernels.to_device(pool, a2)
+        bb, e2 = kernels.to_device(pool, b2)
+        cb, e3 = pool.allocate(n2 * n2 * 4 + 4)
+        pool.sync_events([e1, e2, e3])
+        prog = dev.register_kernel(kernels.gemm_desc(n2, n2, n2, dtype=dt))
+        dev.profile_kernel(prog, [[ab, bb, cb]], max(20, warmup // 4))
+        us = dev.profile_kernel(prog, [[ab, bb, cb]], max(10, steps // 4))
+        tf = 2.0 * n2**3 / us / 1e6
+        out[name] = {"avg_launch_us": round(us, 2), "TFLOP/s": round(tf, 1), "peak_TFLOP/s": peak, "frac_of_peak": round(tf / peak, 4)}
+        dev.release(prog)
+        for b_ in (ab, bb, cb):
+            pool.deallocate(b_, [])
     return out
 
 

@@ -33,7 +33,9 @@ int gemm_bf16_splits(int64_t, int64_t, int64_t) { return 2; }
 uint64_t gemm_bf16_workspace_bytes(int64_t, int64_t, int64_t) { return kScratch; }
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K) { return M % 256 == 0 && N % 128 == 0 && K % 64 == 0; }
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K, int, int, int) { return M >= 64 && N >= 64 && K % 64 == 0; }
+int64_t gemm_bf16_column_split(int64_t, int64_t, int64_t) { return 0; }
 hipError_t gemm_bf16_init() { return hipSuccess; }
+hipError_t gemm_f16_init() { return hipSuccess; }
 hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t st) { return rec(st, "gemm_bf16", {p.A, p.B, p.bias, p.residual}, {p.C, p.workspace}); }
 uint64_t gemm_generic_workspace_bytes(int64_t, int64_t, int64_t, int64_t) { return kScratch; }
 hipError_t gemm_generic(const GemmGeneric &p, hipStream_t st) { return rec(st, "gemm_generic", {p.A, p.B, p.bias, p.residual}, {p.C, p.workspace}); }

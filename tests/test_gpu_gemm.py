@@ -324,3 +324,96 @@ def test_relu_mask_epilogue(hip, oracle, dtype, mnk):
         np.testing.assert_allclose(got, want, rtol=0, atol=2e-6 * np.abs(plain).max() * np.sqrt(k))
         assert np.array_equal(got == 0, want == 0)
     assert (got[0] == 0).all() and got[1, 0] == 0
+
+
+# ---- f16 on the LDS-tiled kernel (v_mfma_f32_32x32x16_f16) -----------------------------------------------------------
+
+def _f16_operands(oracle, m, n, k, seed, trans_a, trans_b):
+    r = oracle.Rng(seed)
+    a = oracle.f32_to_f16(r.uniform((k, m) if trans_a else (m, k), -1, 1))
+    b = oracle.f32_to_f16(r.uniform((n, k) if trans_b else (k, n), -1, 1))
+    af, bf = oracle.f16_to_f32(a).astype(np.float64), oracle.f16_to_f32(b).astype(np.float64)
+    af, bf = (af.T if trans_a else af), (bf.T if trans_b else bf)
+    return a, b, af @ bf, np.abs(af) @ np.abs(bf)
+
+
+@pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("mnk", [(256, 256, 64), (512, 256, 576), (1024, 2048, 512), (256, 384, 256), (264, 136, 64), (1000, 1000, 256),
+                                 (256, 256, 4096)])
+def test_f16_tiled_gemm_layouts(hip, oracle, mnk, trans_a, trans_b):
+    """Whole tiles, edge tiles, the 128-wide tile and split-K, all four layouts; 1e-3 of the f32-accumulated product."""
+    dev, pool = hip
+    m, n, k = mnk
+    a, b, want, mag = _f16_operands(oracle, m, n, k, m + 3 * n + k, trans_a, trans_b)
+    got = gemm(dev, pool, a, b, dtype=DType.F16, trans_a=trans_a, trans_b=trans_b)
+    assert np.all(np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-5 * mag), np.max(np.abs(got - want) / (mag + 1e-30))
+
+
+def test_f16_small_integers_are_exact(hip, oracle):
+    dev, pool = hip
+    rng = np.random.default_rng(2)
+    a = rng.integers(-4, 5, size=(256, 192)).astype(np.float32)
+    b = rng.integers(-4, 5, size=(192, 256)).astype(np.float32)
+    assert np.array_equal(gemm(dev, pool, oracle.f32_to_f16(a), oracle.f32_to_f16(b), dtype=DType.F16), a @ b)
+
+
+@pytest.mark.parametrize("mnk", [(256, 512, 128), (512, 256, 4096), (300, 200, 128)])
+@pytest.mark.parametrize("epilogue", ["bias", "bias_relu", "bias_gelu"])
+def test_f16_epilogues_result_and_residual(hip, oracle, mnk, epilogue):
+    """Linear (weights [out, in]) with f16 bias, activation, f16 result by the C backend's truncating store
+    (zyx/src/codegen/c.rs:475-490) and the fused residual add."""
+    dev, pool = hip
+    m, n, k = mnk
+    a, b, want, mag = _f16_operands(oracle, m, n, k, 17, False, True)
+    r = oracle.Rng(6)
+    bias, res = oracle.f32_to_f16(r.uniform((n,), -1, 1)), oracle.f32_to_f16(r.randn((m, n)))
+    want = want + oracle.f16_to_f32(bias).astype(np.float64)
+    if epilogue == "bias_relu":
+        want = np.maximum(want, 0.0)
+    if epilogue == "bias_gelu":
+        want = 0.5 * want * (1 + np.tanh(np.sqrt(2 / np.pi) * (want + 0.044715 * want ** 3)))
+    kw = dict(bias=bias, epilogue=epilogue, bias_dtype=DType.F16, trans_b=True, dtype=DType.F16)
+    for residual in (None, res):
+        w = want + (oracle.f16_to_f32(res).astype(np.float64) if residual is not None else 0.0)
+        got32 = gemm(dev, pool, a, b, out_dtype=DType.F32, residual=None if residual is None else oracle.f16_to_f32(res), **kw)
+        assert np.all(np.abs(got32 - w) <= 1e-3 * np.abs(w) + 2e-5 * mag + 1e-6)
+        got16 = gemm(dev, pool, a, b, out_dtype=DType.F16, residual=residual, **kw)
+        assert np.array_equal(got16, oracle.f32_to_f16(got32))  # the f16 result is the f32 one truncated
+
+
+# ---- f32 on the LDS-tiled kernel (v_mfma_f32_32x32x2_f32) ------------------------------------------------------------
+
+@pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("mnk", [(1024, 1024, 1024), (512, 1024, 96), (2048, 2048, 64), (768, 640, 224), (4096, 128, 32)])
+def test_f32_tiled_gemm(hip, oracle, mnk, trans_a, trans_b):
+    """zyx/tests/05_misc.rs:820-842 multiplies 1024^3 in f32 against a textbook sgemm: here against the f64-accumulated
+    product at 1e-5 of sum |a b|, on both tile sizes (128 x 128 when the grid is large, 64 x 64 otherwise)."""
+    dev, pool = hip
+    m, n, k = mnk
+    r = oracle.Rng(m + n * 3 + k * 7)
+    a = r.uniform((k, m) if trans_a else (m, k), -1, 1)
+    b = r.uniform((n, k) if trans_b else (k, n), -1, 1)
+    got = gemm(dev, pool, a, b, dtype=DType.F32, trans_a=trans_a, trans_b=trans_b)
+    ad, bd = a.astype(np.float64), b.astype(np.float64)
+    ad, bd = (ad.T if trans_a else ad), (bd.T if trans_b else bd)
+    want, mag = ad @ bd, np.abs(ad) @ np.abs(bd)
+    assert np.all(np.abs(got - want) <= 1e-5 * mag + 1e-30), np.max(np.abs(got - want) / (mag + 1e-30))
+
+
+def test_f32_tiled_integer_products_and_epilogues(hip, oracle):
+    dev, pool = hip
+    rng = np.random.default_rng(4)
+    a = rng.integers(-8, 9, size=(1024, 512)).astype(np.float32)
+    b = rng.integers(-8, 9, size=(512, 1024)).astype(np.float32)
+    assert np.array_equal(gemm(dev, pool, a, b, dtype=DType.F32), a @ b)  # exact in f32 whatever the order
+    r = oracle.Rng(12)
+    x, w, bias = r.randn((1024, 256)), r.uniform((1024, 256), -0.06, 0.06), r.uniform(1024, -0.06, 0.06)
+    res = r.randn((1024, 1024))
+    lin = x.astype(np.float64) @ w.astype(np.float64).T + bias
+    mag = np.abs(x) @ np.abs(w.T) + np.abs(bias)
+    for epi, f in (("bias", lambda v: v), ("bias_relu", lambda v: np.maximum(v, 0)),
+                   ("bias_gelu", lambda v: 0.5 * v * (1 + np.tanh(np.sqrt(2 / np.pi) * (v + 0.044715 * v ** 3))))):
+        got = gemm(dev, pool, x, w, bias, dtype=DType.F32, trans_b=True, epilogue=epi, residual=res)
+        assert np.all(np.abs(got - (f(lin) + res)) <= 2e-5 * mag + 1e-6), epi
+    mask = gemm(dev, pool, x, w, dtype=DType.F32, trans_b=True, residual=res, relu_mask=True)
+    assert np.all(np.abs(mask - (x.astype(np.float64) @ w.astype(np.float64).T) * (res > 0)) <= 2e-5 * mag)

@@ -330,6 +330,7 @@ hipError_t gemm_generic(const GemmGeneric &p0, hipStream_t st) {
 #undef ZK_S
         return hipGetLastError();
     }
+    if (gemm_f32_tiled_ok(p)) return gemm_f32_tiled(p, st);
     p.splits = gemm_generic_splits(p.M, p.N, p.K, p.batch, &p.k_len);
     if (p.splits > 1 && (!p.workspace || (int64_t)p.batch * p.splits > 65535)) return hipErrorInvalidValue;
     dim3 grid((unsigned)((p.N + GN - 1) / GN), (unsigned)((p.M + GM - 1) / GM), (unsigned)(p.batch * p.splits)), block(256);

@@ -88,8 +88,9 @@ struct GemmBf16 {
     int64_t M, N, K;
     int trans_a, trans_b;
     int epilogue;      // 0 none, 1 bias, 2 bias+relu, 3 bias+gelu
-    int bias_dtype;    // DT_BF16 or DT_F32
-    int out_bf16;
+    int bias_dtype;    // DT_BF16, DT_F16 or DT_F32
+    int out_bf16;      // C and the residual are stored in the operands' 16-bit dtype
+    int f16;           // operands (and a 16-bit C) are f16 instead of bf16
     int plane; // 0, or C is stored [M / plane, N, plane] (rows of one group of `plane` are contiguous per column)
     int64_t ldn; // 0, or the launch computes N columns of a product ldn columns wide (row stride of C, residual, [K,N] B)
     ConvGather gather; // with plane != 0 and gather.khw != 0: A is the padded input, not a matrix
@@ -102,8 +103,11 @@ int gemm_bf16_splits(int64_t M, int64_t N, int64_t K);
 uint64_t gemm_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K); // every tile whole
 bool gemm_bf16_supported(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, int out_bf16); // edge tiles allowed
+int64_t gemm_bf16_column_split(int64_t M, int64_t N, int64_t K);
 hipError_t gemm_bf16_init(); // once per device, before the first launch
-hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t stream);
+hipError_t gemm_bf16(const GemmBf16 &p, hipStream_t stream); // either 16-bit dtype (p.f16)
+hipError_t gemm_f16_init();
+hipError_t gemm_f16(const GemmBf16 &p, hipStream_t stream);
 
 // Any-shape GEMM: dtype F32 / BF16 / F16 operands, f32 accumulate, C stored as F32 or as
 // the operand dtype (truncating). `batch` independent products at element strides
@@ -124,6 +128,9 @@ struct GemmGeneric {
 };
 uint64_t gemm_generic_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t batch);
 hipError_t gemm_generic(const GemmGeneric &p, hipStream_t stream);
+// The LDS-tiled f32 kernel (gemm_f32.hip) for whole 64 x 64 x 32 tiles; gemm_generic hands such products over.
+bool gemm_f32_tiled_ok(const GemmGeneric &p);
+hipError_t gemm_f32_tiled(const GemmGeneric &p, hipStream_t stream);
 
 // LayerNorm (rms == 0) / RMSNorm (rms == 1) over the last axis; w, b may be null.
 struct NormRows {

@@ -407,12 +407,13 @@ zk::Elementwise elementwise_args(const zhip_kernel_desc &d) {
 
 // bf16 problems of K a multiple of 64 and M, N of at least 64 (aligned for 128-bit loads) run on the 256-row
 // LDS-tiled kernel, everything else on the general one.
+// 16-bit problems (bf16, f16) of K a multiple of 64 and M, N of at least 64 run on the LDS-tiled kernels.
 bool gemm_takes_fast_path(const zhip_kernel_desc &d) {
     const int64_t batch = d.dims[3] ? d.dims[3] : 1;
     const float alpha = d.fparams[0] == 0.0f ? 1.0f : d.fparams[0];
-    return d.dtype == ZHIP_BF16 && batch == 1 && alpha == 1.0f && (d.iparams[0] == 0 || d.iparams[1] != ZHIP_F16) && d.iparams[2] != 2 &&
+    return (d.dtype == ZHIP_BF16 || d.dtype == ZHIP_F16) && batch == 1 && alpha == 1.0f && d.iparams[2] != 2 &&
            zk::gemm_bf16_supported(d.dims[0], d.dims[1], d.dims[2], d.flags & ZHIP_GEMM_TRANS_A ? 1 : 0,
-                                   d.flags & ZHIP_GEMM_TRANS_B ? 1 : 0, d.out_dtype == ZHIP_BF16);
+                                   d.flags & ZHIP_GEMM_TRANS_B ? 1 : 0, d.out_dtype != ZHIP_F32);
 }
 
 // Shape and scalar parameters of the two attention kinds.
@@ -836,7 +837,8 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
             a.B = ptr[1];
             a.bias = a.epilogue ? ptr[2] : nullptr;
             a.residual = residual;
-            a.out_bf16 = d.out_dtype == ZHIP_BF16;
+            a.out_bf16 = d.out_dtype != ZHIP_F32;
+            a.f16 = d.dtype == ZHIP_F16;
             a.C = ptr[p.n_in];
             a.workspace = p.workspace;
             return zk::gemm_bf16(a, st);
@@ -1146,7 +1148,8 @@ ZHIP_EXPORT int32_t zhip_init(const zhip_config *cfg, zhip_ctx **out) {
         if ((e = hipEventCreateWithFlags(&c->order_ev[k], hipEventDisableTiming)) != hipSuccess) return bail(ZHIP_INITIALIZATION, "hipEventCreate", e);
     if ((e = hipGetSymbolAddress((void **)&c->static_scratch, HIP_SYMBOL(scratch))) != hipSuccess || !c->static_scratch)
         return bail(ZHIP_INITIALIZATION, "hipGetSymbolAddress of the static scratch array", e);
-    if ((e = zk::gemm_bf16_init()) != hipSuccess) return bail(ZHIP_INITIALIZATION, "raising the LDS limit of the GEMM kernels", e);
+    if ((e = zk::gemm_bf16_init()) != hipSuccess || (e = zk::gemm_f16_init()) != hipSuccess)
+        return bail(ZHIP_INITIALIZATION, "raising the LDS limit of the GEMM kernels", e);
     if ((e = zk::conv3x3_init()) != hipSuccess) return bail(ZHIP_INITIALIZATION, "raising the LDS limit of the convolution kernel", e);
     fill_info(c);
     if (c->debug & 1)
