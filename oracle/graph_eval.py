@@ -1,5 +1,5 @@
 """TEST INFRASTRUCTURE, not product code: evaluates a graph of zyx node kinds (Leaf, Const, Unary, Binary, Cast,
-Reshape, Expand, Permute, Flip, Reduce -- zyx/src/graph/mod.rs `Node`) with numpy, node by node, as the checker for
+Reshape, Expand, Permute, Flip, Pad, Narrow, Reduce -- zyx/src/graph/mod.rs `Node`) with numpy, node by node, as the checker for
 the kernels the HIP backend generates from such a graph.
 
 Element arithmetic is the C backend's (oracle/ir_interp.py `unary` / `binary` / `_c_cast`, which restate
@@ -97,6 +97,16 @@ def evaluate(nodes, leaves: dict, wanted) -> dict:
             return np.transpose(x, n.arg)
         if n.kind == "flip":
             return np.flip(x, n.arg)
+        if n.kind == "narrow":  # Node::Narrow: elements start .. start + len of one axis
+            axis, start = n.arg
+            return x[(slice(None),) * axis + (slice(start, start + n.shape[axis]),)]
+        if n.kind == "pad":  # Node::Pad: element i of the axis is x[i - lp] where that exists, else 0
+            axis, lp = n.arg
+            out = np.zeros(n.shape, x.dtype)
+            lo, hi = max(0, lp), min(n.shape[axis], lp + x.shape[axis])  # positions of the result that come from x
+            pre = (slice(None),) * axis
+            out[pre + (slice(lo, hi),)] = x[pre + (slice(lo - lp, hi - lp),)]
+            return out
         if n.kind == "reduce":
             axes = tuple(n.arg)
             keep = [a for a in range(x.ndim) if a not in axes]

@@ -7,7 +7,7 @@ import pytest
 from graph_cases import CASES, mixed_graph, mlp_graph
 from oracle import graph_eval, ir_interp
 from zyx_amd import DType
-from zyx_amd.graph import Contraction, Graph, RowColReduce, SoftmaxRows, lower, match_reduce, match_softmax, match_contraction, storage_dtype, view_of
+from zyx_amd.graph import Contraction, Conv2dMatch, Graph, MaxPoolMatch, RowColReduce, SoftmaxRows, lower, match_reduce, match_softmax, match_contraction, storage_dtype, view_of
 from zyx_amd.ir import BOp, UOp
 
 _FLOAT = (DType.F32, DType.F64)
@@ -23,6 +23,36 @@ def _build(build, *args, **kw):
         return nid
 
     return g, leaves, build(g, leaf, *args, **kw)
+
+
+def conv_textbook(x, w, bias, stride, dilation, padding):
+    """y[n,o,i,j] = bias[o] + sum_{c,p,q} xpad[n,c,i*sh + p*dh, j*sw + q*dw] * w[o,c,p,q], in f64; padding = [(top, bottom),
+    (left, right)]."""
+    x, w = np.asarray(x, np.float64), np.asarray(w, np.float64)
+    xp = np.pad(x, [(0, 0), (0, 0), tuple(padding[0]), tuple(padding[1])])
+    (sh, sw), (dh, dw) = stride, dilation
+    co, _, kh, kw = w.shape
+    oh = (xp.shape[2] - dh * (kh - 1) - 1) // sh + 1
+    ow = (xp.shape[3] - dw * (kw - 1) - 1) // sw + 1
+    y = np.zeros((x.shape[0], co, oh, ow))
+    for p in range(kh):
+        for q in range(kw):
+            win = xp[:, :, p * dh: p * dh + (oh - 1) * sh + 1: sh, q * dw: q * dw + (ow - 1) * sw + 1: sw]
+            y += np.einsum("ncij,oc->noij", win, w[:, :, p, q])
+    return y if bias is None else y + np.asarray(bias, np.float64).reshape(1, -1, 1, 1)
+
+
+def max_pool_textbook(x, kernel, stride, dilation, padding):
+    """x: [planes, h, w]; padding = (ph, pw) on both sides with -inf."""
+    xp = np.pad(x, [(0, 0), (padding[0],) * 2, (padding[1],) * 2], constant_values=-np.inf)
+    oh = (xp.shape[1] - dilation[0] * (kernel[0] - 1) - 1) // stride[0] + 1
+    ow = (xp.shape[2] - dilation[1] * (kernel[1] - 1) - 1) // stride[1] + 1
+    y = np.full((x.shape[0], oh, ow), -np.inf, x.dtype)
+    for p in range(kernel[0]):
+        for q in range(kernel[1]):
+            y = np.maximum(y, xp[:, p * dilation[0]: p * dilation[0] + (oh - 1) * stride[0] + 1: stride[0],
+                                 q * dilation[1]: q * dilation[1] + (ow - 1) * stride[1] + 1: stride[1]])
+    return y
 
 
 def run_lowered(g, leaves, outputs, match=False, seen=None):
@@ -51,6 +81,21 @@ def run_lowered(g, leaves, outputs, match=False, seen=None):
             x = bufs[kern.x].reshape(kern.rows, kern.cols).astype(np.float64)
             e = np.exp(x - x.max(1, keepdims=True))
             bufs[kern.out] = (e / e.sum(1, keepdims=True)).astype(np.float32).reshape(-1)
+            if seen is not None:
+                seen.append(kern)
+            continue
+        if isinstance(kern, Conv2dMatch):
+            n, c, h, w, co, kh, kw = kern.dims
+            y = conv_textbook(bufs[kern.x].reshape(n, c, h, w), bufs[kern.w].reshape(co, c, kh, kw),
+                              None if kern.bias is None else bufs[kern.bias], kern.stride, kern.dilation,
+                              [(kern.padding[0],) * 2, (kern.padding[1],) * 2])
+            bufs[kern.out] = (np.maximum(y, 0) if kern.relu else y).astype(np.float32).reshape(-1)
+            if seen is not None:
+                seen.append(kern)
+            continue
+        if isinstance(kern, MaxPoolMatch):
+            x = bufs[kern.x].reshape(kern.planes, *kern.hw)
+            bufs[kern.out] = max_pool_textbook(x, kern.kernel, kern.stride, kern.dilation, kern.padding).reshape(-1)
             if seen is not None:
                 seen.append(kern)
             continue

@@ -69,6 +69,8 @@ def _numel(shape) -> int:
 class Graph:
     def __init__(self):
         self.nodes: list[Node] = []
+        self.convs: dict[int, dict] = {}  # result node of `conv` -> its operands and parameters
+        self.pools: dict[int, dict] = {}  # result node of a 2-D `max_pool` -> its operand and parameters
 
     def _push(self, node: Node) -> int:
         self.nodes.append(node)
@@ -132,6 +134,37 @@ class Graph:
     def flip(self, x: int, axes) -> int:
         xs = self[x].shape
         return self._push(Node("flip", self[x].dtype, xs, (x,), arg=tuple(sorted({int(a) % len(xs) for a in axes}))))
+
+    @staticmethod
+    def _axis(axis: int, rank: int) -> int:
+        axis = int(axis)
+        if not -rank <= axis < rank:
+            raise ValueError(f"axis {axis} out of range for rank {rank}")
+        return axis % rank
+
+    def pad(self, x: int, axis: int, lp: int, length: int) -> int:
+        """`Node::Pad { x, axis, lp, len }` (zyx/src/graph/mod.rs:118-127): element i of `axis` is x[i - lp] where that
+        exists and 0 elsewhere; `length` is the new extent of the axis. A negative `lp` drops leading elements, a
+        `length` short of lp + the old extent drops trailing ones (`Tensor::pad_axis`, zyx/src/tensor/mod.rs:1126-1138)."""
+        xs = self[x].shape
+        axis = self._axis(axis, len(xs))
+        lp, length = int(lp), int(length)
+        if length < 1 or lp + xs[axis] <= 0 or lp >= length:
+            raise ValueError(f"padding lp={lp}, len={length} leaves nothing of an axis of extent {xs[axis]}")
+        if lp == 0 and length == xs[axis]:
+            return x
+        return self._push(Node("pad", self[x].dtype, xs[:axis] + (length,) + xs[axis + 1:], (x,), arg=(axis, lp)))
+
+    def narrow(self, x: int, axis: int, start: int, length: int) -> int:
+        """`Node::Narrow { x, axis, start, len }` (zyx/src/graph/mod.rs:132-137): elements start .. start + len of `axis`."""
+        xs = self[x].shape
+        axis = self._axis(axis, len(xs))
+        start, length = int(start), int(length)
+        if start < 0 or length < 1 or start + length > xs[axis]:
+            raise ValueError(f"cannot narrow an axis of extent {xs[axis]} to [{start}, {start + length})")
+        if start == 0 and length == xs[axis]:
+            return x
+        return self._push(Node("narrow", self[x].dtype, xs[:axis] + (length,) + xs[axis + 1:], (x,), arg=(axis, start)))
 
     def reduce(self, x: int, rop: BOp, axes) -> int:
         """Reduced dims are dropped; reducing every axis leaves shape [1]."""
@@ -207,6 +240,135 @@ class Graph:
 
     def max_all(self, x: int) -> int:
         return self.reduce(x, BOp.Max, range(len(self[x].shape)))
+
+    # -- padding, slicing, pooling and convolution as the reference composes them ----------------------------------
+    def pad_zeros(self, x: int, padding) -> int:
+        """`Tensor::pad_zeros` (zyx/src/tensor/mod.rs:1161-1179): `padding[i] = (left, right)` for axis i, first axis
+        first; negative amounts crop."""
+        for axis, (l, r) in enumerate(padding):
+            if l or r:
+                x = self.pad(x, axis, l, self[x].shape[axis] + l + r)
+        return x
+
+    def rpad_zeros(self, x: int, padding) -> int:
+        """`Tensor::rpad_zeros` (mod.rs:1202-1222): the first pair pads the LAST axis."""
+        padding = list(padding)
+        rank = len(self[x].shape)
+        return self.pad_zeros(x, ([(0, 0)] * (rank - len(padding)) + padding[::-1]))
+
+    def pad_value(self, x: int, padding, value) -> int:
+        """`Tensor::pad` (mod.rs:1257-1275): `pad_zeros(x) + pad_zeros(ones).where_(zeros, value)`, where_ being
+        `m * a + (1 - m) * b` (mod.rs:1617-1624)."""
+        dt, xs = self[x].dtype, self[x].shape
+        m = self.pad_zeros(self.expand(self.const(1, dt), xs), padding)
+        shape = self[m].shape
+        zeros, val = self.expand(self.const(0, dt), shape), self.expand(self.const(value, dt), shape)
+        one_minus = self.binary(self.expand(self.const(1, dt), shape), m, BOp.Sub)
+        filler = self.binary(self.binary(m, zeros, BOp.Mul), self.binary(one_minus, val, BOp.Mul), BOp.Add)
+        return self.binary(self.pad_zeros(x, padding), filler, BOp.Add)
+
+    def slice(self, x: int, ranges) -> int:
+        """`Tensor::slice` with plain `start..stop` ranges for the leading axes."""
+        for axis, (start, stop) in enumerate(ranges):
+            x = self.narrow(x, axis, start, stop - start)
+        return x
+
+    def repeat(self, x: int, repeats) -> int:
+        """`Tensor::repeat` (mod.rs:2766-2783): reshape to [1, d]..., expand to [r, d]..., reshape to [r * d]...."""
+        repeats, xs = [int(r) for r in repeats], self[x].shape
+        base = (1,) * (len(repeats) - len(xs)) + xs
+        x = self.reshape(x, [v for d in base for v in (1, d)])
+        x = self.expand(x, [v for r, d in zip(repeats, base) for v in (r, d)])
+        return self.reshape(x, [r * d for r, d in zip(repeats, base)])
+
+    def pool(self, x: int, kernel, stride=1, dilation=1) -> int:
+        """`Tensor::pool` (mod.rs:2442-2544): the trailing len(kernel) axes [.., i..] become [.., o.., k..] windows,
+        by repeat / slice / reshape only (no gather): element [.., o, k] is x[.., o * s + k * d]."""
+        k_ = [int(k) for k in kernel]
+        nk = len(k_)
+        s_ = [int(stride)] * nk if np.isscalar(stride) else [int(v) for v in stride]
+        d_ = [int(dilation)] * nk if np.isscalar(dilation) else [int(v) for v in dilation]
+        if len(s_) == 1: s_ = s_ * nk
+        if len(d_) == 1: d_ = d_ * nk
+        shape = self[x].shape
+        lead = list(shape[:len(shape) - nk])
+        i_ = list(shape[len(shape) - nk:])
+        o_ = [-(-(i - d * (k - 1)) // s) for i, d, k, s in zip(i_, d_, k_, s_)]
+        full = [(0, d) for d in lead]
+        x = self.repeat(x, [1] * len(lead) + [-(-(k * (i + d)) // i) for k, i, d in zip(k_, i_, d_)])
+        x = self.slice(x, full + [(0, k * (i + d)) for k, i, d in zip(k_, i_, d_)])
+        x = self.reshape(x, lead + [v for k, i, d in zip(k_, i_, d_) for v in (k, i + d)])
+        x = self.slice(x, full + [r for k, o, s in zip(k_, o_, s_) for r in ((0, k), (0, o * s))])
+        x = self.reshape(x, lead + [v for k, o, s in zip(k_, o_, s_) for v in (k, o, s)])
+        x = self.slice(x, full + [r for k, o in zip(k_, o_) for r in ((0, k), (0, o), (0, 1))])
+        x = self.reshape(x, lead + [v for k, o in zip(k_, o_) for v in (k, o)])
+        n = len(lead)
+        return self.permute(x, list(range(n)) + [n + 2 * i + 1 for i in range(nk)] + [n + 2 * i for i in range(nk)])
+
+    def conv(self, x: int, w: int, bias: int | None = None, groups: int = 1, stride=1, dilation=1, padding=0) -> int:
+        """`Tensor::conv` (mod.rs:2583-2680): pad, pool into windows, broadcast against the reshaped weight, sum over
+        (cin, kernel). `padding`: one amount, one per spatial axis (both sides), 2 * nk amounts running from the last axis
+        to the first as (before, after, before, after, ...) like the reference's, or one (before, after) pair per spatial
+        axis, first axis first. The result node is remembered in `self.convs` with its operands and parameters, so that a 2-D
+        convolution can be handed to the hand-written kernel as a whole (`match_conv`)."""
+        xs, ws = self[x].shape, self[w].shape
+        bs, cin_, (cout, cin), hw = xs[0], xs[1], ws[:2], list(ws[2:])
+        nk = len(hw)
+        if groups * cin != cin_ or len(xs) != len(ws):
+            raise ValueError(f"input shape {xs} does not match the weights {ws}")
+        if not np.isscalar(padding) and all(not np.isscalar(q) for q in padding):
+            # (before, after) per spatial axis, first axis first
+            if len(padding) != nk or any(len(q) != 2 for q in padding):
+                raise ValueError(f"padding {padding} does not name {nk} (before, after) pairs")
+            padding = [int(v) for q in reversed(list(padding)) for v in q]
+        pads = [int(padding)] * (2 * nk) if np.isscalar(padding) else [int(v) for v in padding]
+        if len(pads) == nk:  # one amount per spatial axis, both sides
+            pads = [v for q in pads for v in (q, q)][::-1]
+        elif len(pads) == 1:
+            pads = pads * (2 * nk)
+        stride = [int(stride)] * nk if np.isscalar(stride) else [int(v) for v in stride]
+        dilation = [int(dilation)] * nk if np.isscalar(dilation) else [int(v) for v in dilation]
+        px = self.rpad_zeros(x, [(pads[2 * i], pads[2 * i + 1]) for i in range(nk)])
+        pooled = self.pool(px, hw, stride, dilation)
+        rcout = cout // groups
+        oyx = list(self[pooled].shape[2:2 + nk])
+        t = self.reshape(pooled, [bs, groups, cin, 1] + oyx + hw)
+        t = self.expand(t, [bs, groups, cin, rcout] + oyx + hw)
+        t = self.permute(t, [0, 1, 3] + [4 + i for i in range(nk)] + [2] + [4 + nk + i for i in range(nk)])
+        wr = self.reshape(w, [1, groups, rcout] + [1] * nk + [cin] + hw)
+        prod = self.binary_b(t, wr, BOp.Mul)
+        rank = len(self[prod].shape)
+        out = self.reshape(self.reduce(prod, BOp.Add, [rank - 1 - i for i in range(nk + 1)]), [bs, cout] + oyx)
+        core = out
+        if bias is not None:
+            out = self.binary_b(out, self.reshape(bias, [1, cout] + [1] * nk), BOp.Add)
+        if nk == 2 and groups == 1:
+            # rpad_zeros pairs run last axis first: (left, right) of W, then (top, bottom) of H
+            info = dict(x=x, w=w, bias=bias, stride=tuple(stride), dilation=tuple(dilation), padding=(pads[2], pads[0]),
+                        symmetric=pads[0] == pads[1] and pads[2] == pads[3], core=core)
+            self.convs[out] = info
+        return out
+
+    def max_pool(self, x: int, kernel, stride=None, dilation=1, padding=None) -> int:
+        """`Tensor::max_pool` (mod.rs:2706-2741): pad the trailing axes with the dtype's lowest value, pool, maximum over
+        the window axes. `padding[i] = (before, after)` for the i-th of the trailing axes, first of them first."""
+        nk = len(kernel)
+        stride = list(kernel) if stride is None else stride
+        rank = len(self[x].shape)
+        orig = x
+        if padding is not None and any(l or r for l, r in padding):
+            x = self.pad_value(x, [(0, 0)] * (rank - nk) + list(padding), min_constant(self[x].dtype))
+        pooled = self.pool(x, kernel, stride, dilation)
+        prank = len(self[pooled].shape)
+        out = self.reduce(pooled, BOp.Max, range(prank - nk, prank))
+        if nk == 2:
+            pads = [(0, 0), (0, 0)] if padding is None else [tuple(q) for q in padding]
+            s2 = [int(stride)] * 2 if np.isscalar(stride) else [int(v) for v in stride]
+            d2 = [int(dilation)] * 2 if np.isscalar(dilation) else [int(v) for v in dilation]
+            if all(l == r for l, r in pads):
+                self.pools[out] = dict(x=orig, kernel=tuple(int(k) for k in kernel), stride=tuple(s2), dilation=tuple(d2),
+                                       padding=(pads[0][0], pads[1][0]))
+        return out
 
     # -- reverse mode ---------------------------------------------------------------------------------------------
     def _grad_order(self, target: int, sources: set) -> list:
@@ -325,6 +487,16 @@ class Graph:
                 acc(n.src[0], self.permute(grad, inv))
             elif n.kind == "flip":
                 acc(n.src[0], self.flip(grad, n.arg))
+            elif n.kind == "pad":
+                # `todo!()` in the reference (autograd.rs:252-254). The padding received no contribution from x and
+                # cropped elements none from the result: the gradient is the same window moved back, i.e. a Pad by -lp
+                # to x's extent.
+                axis, lp = n.arg
+                acc(n.src[0], self.pad(grad, axis, -lp, self[n.src[0]].shape[axis]))
+            elif n.kind == "narrow":
+                # `todo!()` in the reference (autograd.rs:255-257): zeros around the window that was kept
+                axis, start = n.arg
+                acc(n.src[0], self.pad(grad, axis, start, self[n.src[0]].shape[axis]))
             elif n.kind == "reduce":
                 x = n.src[0]
                 xs = self[x].shape
@@ -577,6 +749,103 @@ def match_reduce(graph: Graph, nid: int, stored) -> RowColReduce | None:
     return RowColReduce(base, nid, rows, cols, axis0, "sum" if r.op == BOp.Add else "max", r.dtype)
 
 
+@dataclasses.dataclass
+class Conv2dMatch:
+    """`out = conv(x, w) (+ bias) (then relu)` for NCHW x and [Cout, C, KH, KW] w, groups = 1, equal padding on both sides
+    of an axis: what ZHIP_K_CONV2D computes in one launch. x, w, bias are the nodes whose buffers it reads."""
+    x: int
+    w: int
+    bias: int | None
+    out: int
+    dims: tuple      # N, C, H, W, Cout, KH, KW
+    stride: tuple
+    padding: tuple
+    dilation: tuple
+    relu: bool
+    dtype: DType
+    fallback: object = None
+
+
+@dataclasses.dataclass
+class MaxPoolMatch:
+    """`out = max_pool(x)` over the last two axes (ZHIP_K_MAX_POOL2D)."""
+    x: int
+    out: int
+    planes: int
+    hw: tuple
+    kernel: tuple
+    stride: tuple
+    padding: tuple
+    dilation: tuple
+    dtype: DType
+
+
+def _is_relu_of(graph: Graph, nid: int):
+    """The node x when `nid` is `x.cmpgt(0) * x` (`Tensor::relu`, zyx/src/tensor/elementwise.rs:289-293), else None."""
+    n = graph[nid]
+    if n.kind != "binary" or n.op != BOp.Mul:
+        return None
+    c, x = graph[n.src[0]], n.src[1]
+    if c.kind == "binary" and c.op == BOp.Cmpgt and c.src[0] == x:
+        z = graph[c.src[1]]
+        if z.kind == "const" and z.arg == 0:
+            return x
+    return None
+
+
+def match_conv(graph: Graph, nid: int, users: dict | None = None) -> Conv2dMatch | None:
+    """A node `Graph.conv` built, or the `relu` of one whose only consumers are that relu's two nodes (`users`: node ->
+    its consumers among the nodes being computed, -1 standing for the caller; without it no relu is folded in). The composition of pads, window
+    views and the broadcast product is recognised by where it came from rather than by its thirty-odd movement nodes:
+    `Graph.conv` notes operands and parameters next to the node it returns."""
+    relu, c = False, nid
+    inner = _is_relu_of(graph, nid)
+    if inner is not None and inner in graph.convs and users is not None and users.get(inner, set()) == {graph[nid].src[0], nid}:
+        relu, c = True, inner
+    info = graph.convs.get(c)
+    if info is None or not info["symmetric"] or graph[nid].dtype not in (DType.F32, DType.BF16):
+        return None
+    xs, ws = graph[info["x"]].shape, graph[info["w"]].shape
+    return Conv2dMatch(info["x"], info["w"], info["bias"], nid, (xs[0], xs[1], xs[2], xs[3], ws[0], ws[2], ws[3]), info["stride"],
+                       info["padding"], info["dilation"], relu, graph[nid].dtype)
+
+
+def consumers(graph: Graph, outputs: Sequence[int], stored=()) -> dict:
+    """node -> the nodes that read it, among those `outputs` are computed from (not looking behind stored nodes)."""
+    users: dict[int, set] = {o: {-1} for o in outputs}  # the caller reads the outputs
+    seen, stack = set(stored), list(outputs)
+    while stack:
+        i = stack.pop()
+        if i in seen:
+            continue
+        seen.add(i)
+        for s in graph[i].src:
+            users.setdefault(s, set()).add(i)
+            stack.append(s)
+    return users
+
+
+def match_max_pool(graph: Graph, nid: int) -> MaxPoolMatch | None:
+    info = graph.pools.get(nid)
+    if info is None or graph[nid].dtype not in (DType.F32, DType.BF16):
+        return None
+    xs = graph[info["x"]].shape
+    return MaxPoolMatch(info["x"], nid, _numel(xs[:-2]), (xs[-2], xs[-1]), info["kernel"], info["stride"], info["padding"],
+                        info["dilation"], graph[nid].dtype)
+
+
+def match_operands(m) -> tuple:
+    """Nodes whose buffers a matched kernel reads."""
+    if isinstance(m, Contraction):
+        return (m.a, m.b)
+    if isinstance(m, Conv2dMatch):
+        return (m.x, m.w) + ((m.bias,) if m.bias is not None else ())
+    return (m.x,)
+
+
+MATCHED = (Contraction, SoftmaxRows, RowColReduce, Conv2dMatch, MaxPoolMatch)
+
+
 # ---- lowering ---------------------------------------------------------------------------------------------------------
 
 @dataclasses.dataclass
@@ -600,6 +869,7 @@ class _Emitter:
 
     def __init__(self, graph: Graph, stored: set):
         self.g, self.stored = graph, stored
+        self.relu_mask: dict[int, int] = {}  # `v > 0` node of a relu whose v is not stored -> the stored relu(v)
 
     # index arithmetic with constant folding
     def _ix(self, v):
@@ -666,6 +936,7 @@ class _Emitter:
             v = k.unary(self.value(n.src[0], idx), n.op)
         elif n.kind == "binary":
             x, y = n.src
+            x = self.relu_mask.get(nid, x)
             dt = self.g.operand_dtype(x, y)
             v = k.binary(self.operand(x, idx, dt), self.operand(y, idx, dt), n.op)
         elif n.kind == "cast":
@@ -681,6 +952,40 @@ class _Emitter:
             for i, a in enumerate(n.arg):
                 x_idx[a] = idx[i]
             v = self.value(n.src[0], x_idx)
+        elif n.kind == "narrow":
+            axis, start = n.arg
+            x_idx = list(idx)
+            x_idx[axis] = self.add(idx[axis], start)
+            v = self.value(n.src[0], x_idx)
+        elif n.kind == "pad":
+            # the reference's rule (zyx/src/kernel/linearize.rs:349-382): pc = (0 <= j < extent); the load happens at
+            # pc * j and its value is multiplied by pc
+            axis, lp = n.arg
+            ext = self.g[n.src[0]].shape[axis]
+            i = idx[axis]
+            x_idx = list(idx)
+            if not isinstance(i, _V):
+                j = i - lp
+                if 0 <= j < ext:
+                    x_idx[axis] = j
+                    v = self.value(n.src[0], x_idx)
+                else:
+                    v = k.const(0, n.dtype)
+            else:
+                j = self.add(i, -lp) if lp <= 0 else _V(k.sub(i.id, self._ix(lp)))
+                inside = None
+                if lp > 0:
+                    inside = k.cmpge(j.id, self._ix(0))
+                if n.shape[axis] - lp > ext:
+                    hi = k.cmplt(j.id, self._ix(ext))
+                    inside = hi if inside is None else k.and_(inside, hi)
+                if inside is None:  # a pure crop: every index of the result exists in x
+                    x_idx[axis] = j
+                    v = self.value(n.src[0], x_idx)
+                else:
+                    pc_i = k.cast(inside, DType.I64)
+                    x_idx[axis] = _V(k.mul(j.id, pc_i))
+                    v = k.binary(self.value(n.src[0], x_idx), k.cast(inside, n.dtype), BOp.Mul)
         elif n.kind == "flip":
             x_idx = list(idx)
             for a in n.arg:
@@ -707,8 +1012,8 @@ class _Emitter:
                 seen.add(nid)
                 order.append(nid)
             return
-        for s in n.src:
-            self._inputs(s, False, seen, order)
+        for i, s in enumerate(n.src):
+            self._inputs(self.relu_mask.get(nid, s) if i == 0 else s, False, seen, order)
 
     def kernel(self, nid: int) -> LoweredKernel:
         n = self.g[nid]
@@ -763,17 +1068,28 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
     have = set(stored)
     emitter = _Emitter(graph, have)
     schedule: list = []
+    users = consumers(graph, outputs, stored) if match else {}
 
     def need(nid: int, root: bool):
         n = graph[nid]
         if n.kind == "leaf" or nid in have:
             return
-        c = (match_contraction(graph, nid) or match_softmax(graph, nid) or match_reduce(graph, nid, have)) if match else None
+        if match and nid in graph.convs:
+            # a convolution read only by its relu is never stored: the relu's launch computes both, and the relu's mask
+            # `conv > 0`, which the reverse pass reads, is taken from the relu's result (`relu(v) > 0` is `v > 0`)
+            for r in users.get(nid, ()):
+                if _is_relu_of(graph, r) == nid and match_conv(graph, r, users) is not None:
+                    need(r, True)
+                    return
+        c = (match_conv(graph, nid, users) or match_max_pool(graph, nid) or match_contraction(graph, nid) or match_softmax(graph, nid)
+             or match_reduce(graph, nid, have)) if match else None
         if c is not None:
-            for s in ((c.a, c.b) if isinstance(c, Contraction) else (c.x,)):
+            for s in match_operands(c):
                 need(s, True)
             if isinstance(c, Contraction):
                 c.fallback = emitter.kernel(nid)
+            if isinstance(c, Conv2dMatch) and c.relu:
+                emitter.relu_mask[graph[nid].src[0]] = nid
             schedule.append(c)
             have.add(nid)
             return
@@ -835,7 +1151,7 @@ class Tape:
 
     def realize(self, nodes: Sequence[int]):
         for kern in lower(self.graph, [n for n in nodes if n not in self._buf], stored=list(self._buf), match=self.match):
-            if isinstance(kern, (Contraction, SoftmaxRows, RowColReduce)):
+            if isinstance(kern, MATCHED):
                 kern = self._matched_or_generated(kern)
             prog = self._programs.get(kern.image)
             if prog is None:
@@ -862,7 +1178,7 @@ class Tape:
         launches = []
         stored = [n for n in self._buf if self.graph[n].kind == "leaf"]  # everything else is computed by the plan
         for kern in lower(self.graph, list(nodes), stored=stored, match=bool(self.match)):
-            if isinstance(kern, (Contraction, SoftmaxRows, RowColReduce)):
+            if isinstance(kern, MATCHED):
                 kern = self._matched_or_generated(kern)
             prog = self._programs.get(kern.image)
             if prog is None:
@@ -900,8 +1216,15 @@ class Tape:
         self._ev[leaf] = self.pool.copy_range(self._buf[node], 0, self._buf[leaf], 0, nbytes, waits)
 
     def _matched_or_generated(self, c) -> LoweredKernel:
-        from .kernels import gemm_desc, reduce_desc, softmax_rows_desc
-        if isinstance(c, Contraction):
+        from .kernels import conv2d_desc, gemm_desc, max_pool2d_desc, reduce_desc, softmax_rows_desc
+        if isinstance(c, Conv2dMatch):
+            n_, c_, h, w, co, kh, kw = c.dims
+            desc = conv2d_desc(n_, c_, h, w, co, kh, kw, c.stride, c.padding, c.dilation, c.bias is not None, c.relu, c.dtype)
+            inputs, elements = list(match_operands(c)), _numel(self.graph[c.out].shape)
+        elif isinstance(c, MaxPoolMatch):
+            desc = max_pool2d_desc(c.planes, c.hw[0], c.hw[1], c.kernel, c.stride, c.padding, c.dilation, c.dtype)
+            inputs, elements = [c.x], _numel(self.graph[c.out].shape)
+        elif isinstance(c, Contraction):
             desc = gemm_desc(c.m, c.n, c.k, c.dtype, c.dtype, c.trans_a, c.trans_b, batch=c.batch)
             inputs, elements = [c.a, c.b], c.batch * c.m * c.n
         elif isinstance(c, RowColReduce):
