@@ -210,8 +210,8 @@ def extra_graph(dev, pool, steps=60, warmup=10):
     F32 = zyx_amd.DType.F32
     B, NIN, H, NOUT, LR = 64, 784, 128, 10, 0.01
     out = {}
-    for match in (False, True):
-        rng = Rng(42069)  # the same parameters and batches for both runs
+    for match, in_place in ((False, False), (True, False), (True, True)):
+        rng = Rng(42069)  # the same parameters and batches for all runs
         tape = Tape(dev, pool, match=match)
         g = tape.graph
         k1, k2 = 1 / np.sqrt(NIN), 1 / np.sqrt(H)
@@ -220,12 +220,11 @@ def extra_graph(dev, pool, steps=60, warmup=10):
                   tape.tensor(rng.uniform((NOUT, H), -k2, k2), F32), tape.tensor(rng.uniform((NOUT,), -k2, k2), F32)]
         h = g.relu(g.binary_b(g.dot(x, g.t(params[0])), params[1], BOp.Add))
         logits = g.binary_b(g.dot(h, g.t(params[2])), params[3], BOp.Add)
-        per_row = g.reduce(g.binary(g.ln_softmax(logits, [-1]), onehot, BOp.Mul), BOp.Add, [1])
-        loss = g.binary(g.unary(g.sum_all(per_row), UOp.Neg), g.const(float(B), F32), BOp.Div)
+        loss = g.cross_entropy(logits, onehot, "mean")
         lr = g.const(LR, F32)
         new = [g.binary(p, g.binary(gr, lr, BOp.Mul), BOp.Sub) for p, gr in zip(params, tape.gradient(loss, params))]
         t0 = time.perf_counter()
-        plan = tape.plan(new + [loss])
+        plan = tape.plan(new + [loss], updates=dict(zip(params, new)) if in_place else None, inputs=[x, onehot] if in_place else ())
         build_ms = (time.perf_counter() - t0) * 1e3
         xs = rng.randn((steps + warmup, B, NIN))
         hot = np.eye(NOUT, dtype=np.float32)[rng.randint((steps + warmup, B), 0, NOUT)]
@@ -236,11 +235,12 @@ def extra_graph(dev, pool, steps=60, warmup=10):
             tape.write(x, xs[i])
             tape.write(onehot, hot[i])
             plan.launch()
-            for p, n in zip(params, new):
-                tape.assign(p, n)
+            if not in_place:
+                for p, n in zip(params, new):
+                    tape.assign(p, n)
         final = float(tape.numpy(loss)[0])
         sps = steps / (time.perf_counter() - t0)
-        out["matched_to_gemm" if match else "generated_kernels_only"] = {
+        out["matched_updates_in_place" if in_place else "matched_to_kernels" if match else "generated_kernels_only"] = {
             "steps_per_s": round(sps, 1), "launches_per_step": plan.launches, "lower_and_compile_ms": round(build_ms, 1),
             "final_loss": round(final, 5)}
         tape.close()

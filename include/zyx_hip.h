@@ -162,7 +162,10 @@ enum zhip_kernel_kind {
      * ZHIP_CE_GRAD writes d(fparams[0] * sum(loss))/d(logits) = (softmax - onehot) *
      * fparams[0] into grad[rows, cols] (fparams[0] = 1/rows for the Mean reduction),
      * ZHIP_CE_MEAN (rows <= 4096) writes mean[1] = sum(loss) / rows (ReduceOp::Mean) from the same launch.
-     * args: logits, labels, (loss), (grad), (mean). */
+     * ZHIP_CE_DENSE: the targets are an f32 tensor of the logits' shape instead (the `target` of
+     * :1641-1646 when it already has the logits' shape): loss = sum_c -ln_softmax * target,
+     * grad = (softmax * sum_c target - target) * fparams[0].
+     * args: logits, labels | targets, (loss), (grad), (mean). */
     ZHIP_K_CROSS_ENTROPY = 6,
     /* Tensor::conv for 4-D NCHW input, groups = 1 (zyx/src/tensor/mod.rs:2583-2680; layer
      * zyx-nn/src/conv2d.rs:60-70): y[N,Cout,OH,OW] = x[N,C,H,W] (*) w[Cout,C,KH,KW] (+ bias[Cout])
@@ -236,6 +239,7 @@ enum zhip_kernel_kind {
 #define ZHIP_CE_LOSS 1
 #define ZHIP_CE_GRAD 2
 #define ZHIP_CE_MEAN 4
+#define ZHIP_CE_DENSE 8 /* the second argument is an f32 [rows, cols] target tensor (one-hot or soft labels) */
 #define ZHIP_INDEX_GATHER 0
 #define ZHIP_INDEX_SELECT 1
 #define ZHIP_INDEX_SCATTER 2

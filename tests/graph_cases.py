@@ -223,7 +223,7 @@ def attention_graph(g, leaf, b=2, h=2, t=24, dh=8, seed=3, causal=False, p=0.0, 
 
 def mlp_training_graph(g, leaf, batch=64, n_in=784, hidden=128, n_out=10, lr=0.01, seed=4):
     """The MNIST network's training step as one graph (zyx/tests/mnist.rs:54-66): Linear, relu, Linear,
-    cross_entropy = mean over the batch of -sum(ln_softmax(logits) * one_hot(labels)) (tensor/mod.rs:1639-1655),
+    cross_entropy(one_hot(labels), Mean) (tensor/mod.rs:1639-1655),
     gradients by the reverse rules, `w - g * lr`. Returns (loss, new parameters, parameter leaves, (x, onehot))."""
     r = np.random.default_rng(seed)
     k1, k2 = 1 / np.sqrt(n_in), 1 / np.sqrt(hidden)
@@ -233,8 +233,7 @@ def mlp_training_graph(g, leaf, batch=64, n_in=784, hidden=128, n_out=10, lr=0.0
     w2, b2 = leaf(r.uniform(-k2, k2, (n_out, hidden)), F32), leaf(r.uniform(-k2, k2, (n_out,)), F32)
     h = g.relu(g.binary_b(g.dot(x, g.t(w1)), b1, BOp.Add))
     logits = g.binary_b(g.dot(h, g.t(w2)), b2, BOp.Add)
-    per_row = g.reduce(g.binary(g.ln_softmax(logits, [-1]), onehot, BOp.Mul), BOp.Add, [1])
-    loss = g.binary(g.unary(g.sum_all(per_row), UOp.Neg), g.const(float(batch), F32), BOp.Div)
+    loss = g.cross_entropy(logits, onehot, "mean")
     params = [w1, b1, w2, b2]
     grads = g.gradient(loss, params)
     lr_c = g.const(lr, F32)

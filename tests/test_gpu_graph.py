@@ -316,6 +316,57 @@ def test_training_steps_as_a_cached_plan(hip, oracle, match):
         tape.close()
 
 
+def test_training_steps_with_fused_launches_and_in_place_updates(hip, oracle):
+    """The same twelve steps with every matcher on and the parameter updates declared to the plan: eight launches per
+    step (the list zyx_amd/training.py writes by hand), no copies between steps; loss curve and final parameters
+    against the CPU oracle's training step."""
+    from graph_cases import mlp_training_graph
+    tape, leaves, (loss, new, params, (x, onehot)) = matched_tape(hip, mlp_training_graph, match=True)
+    try:
+        plan = tape.plan(new + [loss], updates=dict(zip(params, new)), inputs=[x, onehot])
+        assert plan.launches == 8 and tape.matched == 8
+        r = np.random.default_rng(11)
+        p = [leaves[i].copy() for i in params]
+        for step in range(12):
+            xs = r.standard_normal((64, 784)).astype(np.float32)
+            lab = r.integers(0, 10, 64).astype(np.int32)
+            tape.write(x, xs)
+            tape.write(onehot, np.eye(10, dtype=np.float32)[lab])
+            plan.launch()
+            want_loss, *p, _ = oracle.mlp_step(xs, lab, *p, 0.01)
+            if step % 5 == 0 or step == 11:
+                np.testing.assert_allclose(tape.numpy(loss), [want_loss], rtol=2e-5)
+                for leaf_id, w in zip(params, p):  # the leaves hold the updated parameters after every launch
+                    np.testing.assert_allclose(tape.numpy(leaf_id), w, rtol=1e-4, atol=1e-6)
+        with pytest.raises(ValueError):
+            tape.plan(new + [loss], updates={params[0]: new[1]})
+    finally:
+        tape.close()
+
+
+def test_cross_entropy_with_dense_targets(hip, oracle):
+    """ZHIP_K_CROSS_ENTROPY with an f32 target tensor: one-hot targets give what class indices give; soft targets give
+    -sum(ln_softmax * t) and (softmax * sum t - t) * scale."""
+    from zyx_amd import kernels
+    dev, pool = hip
+    r = np.random.default_rng(3)
+    for rows, cols in ((64, 10), (33, 1000), (5, 1)):
+        X = (r.standard_normal((rows, cols)) * 3).astype(np.float32)
+        lab = r.integers(0, cols, rows).astype(np.int32)
+        l0, g0, m0 = kernels.cross_entropy(dev, pool, X, lab, 1.0 / rows, mean=True)
+        l1, g1, m1 = kernels.cross_entropy(dev, pool, X, np.eye(cols, dtype=np.float32)[lab], 1.0 / rows, mean=True, dense=True)
+        np.testing.assert_allclose(l1, l0, rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(g1, g0, rtol=1e-6, atol=1e-8)
+        np.testing.assert_allclose(m1, m0, rtol=1e-6)
+        T = r.random((rows, cols)).astype(np.float32)
+        l2, g2 = kernels.cross_entropy(dev, pool, X, T, 0.5, dense=True)
+        x64 = X.astype(np.float64)
+        m = x64 - x64.max(1, keepdims=True)
+        ls = m - np.log(np.exp(m).sum(1, keepdims=True))
+        np.testing.assert_allclose(l2, (-ls * T).sum(1), rtol=2e-5, atol=1e-6)
+        np.testing.assert_allclose(g2, (np.exp(ls) * T.sum(1, keepdims=True) - T) * 0.5, rtol=2e-5, atol=1e-6)
+
+
 def test_long_reductions_run_on_the_reduce_kernel(hip):
     """Row sums, a maximum over the trailing axes and an integer column sum of tensors with buffers are launched as
     the two-stage reduce kernel; integers and maxima exact, float sums to 1e-5 of sum |x|."""

@@ -7,7 +7,7 @@ import pytest
 from graph_cases import CASES, mixed_graph, mlp_graph
 from oracle import graph_eval, ir_interp
 from zyx_amd import DType
-from zyx_amd.graph import Contraction, Conv2dMatch, Graph, MaxPoolMatch, RowColReduce, SoftmaxRows, lower, match_reduce, match_softmax, match_contraction, storage_dtype, view_of
+from zyx_amd.graph import Contraction, Conv2dMatch, CrossEntropyMatch, Graph, MaxPoolMatch, RowColReduce, SoftmaxRows, lower, match_reduce, match_softmax, match_contraction, storage_dtype, view_of
 from zyx_amd.ir import BOp, UOp
 
 _FLOAT = (DType.F32, DType.F64)
@@ -66,14 +66,39 @@ def run_lowered(g, leaves, outputs, match=False, seen=None):
             B = bufs[kern.b].reshape((kern.batch, kern.n, kern.k) if kern.trans_b else (kern.batch, kern.k, kern.n))
             A = A.transpose(0, 2, 1) if kern.trans_a else A
             B = B.transpose(0, 2, 1) if kern.trans_b else B
-            bufs[kern.out] = np.matmul(A.astype(np.float64), B.astype(np.float64)).astype(A.dtype).reshape(-1)
+            acc = np.matmul(A.astype(np.float64), B.astype(np.float64)) * np.float64(np.float32(kern.alpha))
+            if kern.bias is not None:
+                acc = acc + bufs[kern.bias].astype(np.float64).reshape(1, 1, -1)
+            if kern.epilogue == "bias_relu":
+                acc = np.maximum(acc, 0)
+            elif kern.epilogue == "bias_gelu":
+                acc = acc * 0.5 * (np.tanh((acc + acc ** 3 * 0.044715) * np.sqrt(2 / np.pi)) + 1)
+            if kern.residual is not None:
+                res = bufs[kern.residual].astype(np.float64).reshape(acc.shape)
+                acc = acc * (res > 0) if kern.relu_mask else acc + res
+            bufs[kern.out] = acc.astype(A.dtype).reshape(-1)
+            if seen is not None:
+                seen.append(kern)
+            continue
+        if isinstance(kern, CrossEntropyMatch):
+            x = bufs[kern.x].reshape(kern.rows, kern.cols).astype(np.float64)
+            t = bufs[kern.target].reshape(kern.rows, kern.cols).astype(np.float64)
+            m = x - x.max(1, keepdims=True)
+            ls = m - np.log(np.exp(m).sum(1, keepdims=True))
+            if kern.mean is not None:
+                bufs[kern.mean] = np.array([(-ls * t).sum(1).mean()], np.float32)
+            if kern.grad is not None:
+                bufs[kern.grad] = ((np.exp(ls) * t.sum(1, keepdims=True) - t) * kern.gscale).astype(np.float32).reshape(-1)
             if seen is not None:
                 seen.append(kern)
             continue
         if isinstance(kern, RowColReduce):
             x = bufs[kern.x].reshape(kern.rows, kern.cols)
             f = np.sum if kern.op == "sum" else np.max
-            bufs[kern.out] = f(x.astype(np.float64) if x.dtype.kind == "f" else x, axis=0 if kern.axis0 else 1).astype(x.dtype).reshape(-1)
+            red = f(x.astype(np.float64) if x.dtype.kind == "f" else x, axis=0 if kern.axis0 else 1)
+            if kern.base is not None:
+                red = red * np.float64(np.float32(kern.mul)) + bufs[kern.base].astype(np.float64).reshape(-1)
+            bufs[kern.out] = red.astype(x.dtype).reshape(-1)
             if seen is not None:
                 seen.append(kern)
             continue

@@ -240,6 +240,7 @@ struct CrossEntropy {
     const float *x;
     const int32_t *labels;
     float *loss, *grad;
+    const float *dense = nullptr; // f32 targets [rows, cols] in place of class indices
     float *mean = nullptr; // [1]: sum(loss) / rows, by a single workgroup (rows <= kCrossEntropyMeanRows)
 };
 constexpr int64_t kCrossEntropyMeanRows = 4096;

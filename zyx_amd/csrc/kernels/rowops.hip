@@ -261,12 +261,13 @@ __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename R
     }
 }
 
-// Cross-entropy with class-index targets, one wave per sample. loss[r] = -(ln_softmax(x)[label])
-// computed as the reference does: m = x - max; ls = m - ln(sum exp(m)); loss = sum_c -ls[c] * onehot[c].
-// grad (optional) = (softmax(x) - onehot) * gscale, the gradient of gscale * sum_r loss[r].
-// A label outside [0, cols) matches no class (all-zero one-hot): loss 0, grad = softmax * gscale.
+// Cross-entropy, one wave per sample. loss[r] = sum_c -(ln_softmax(x)[r,c]) * target[r,c], computed as the reference
+// does: m = x - max; ls = m - ln(sum exp(m)). Targets are class indices (target[r,c] = (c == label[r]); a label outside
+// [0, cols) matches no class: loss 0) or, DENSE, an f32 [rows, cols] tensor of their own (one-hot or soft labels).
+// grad (optional) = (softmax(x) * sum_c target - target) * gscale, the gradient of gscale * sum_r loss[r].
 // One row by one wave; returns the row's loss (in every lane).
-__device__ __forceinline__ float cross_entropy_row(const float *__restrict__ x, const int32_t *__restrict__ labels,
+template <bool DENSE>
+__device__ __forceinline__ float cross_entropy_row(const float *__restrict__ x, const void *__restrict__ target,
                                                    float *__restrict__ loss, float *__restrict__ grad, int64_t row, int cols,
                                                    float gscale, int lane) {
     const float *xr = x + row * cols;
@@ -277,37 +278,54 @@ __device__ __forceinline__ float cross_entropy_row(const float *__restrict__ x, 
     for (int c = lane; c < cols; c += 64) s += expf(xr[c] - mx);
     s = wave_allreduce_f32(s, OpAdd());
     const float lns = logf(s);
-    const int label = labels[row];
-    float l = 0.0f;
-    if (label >= 0 && label < cols) l = -((xr[label] - mx) - lns);
+    float l = 0.0f, tsum = 1.0f;
+    int label = -1;
+    const float *tr = nullptr;
+    if (DENSE) {
+        tr = (const float *)target + row * cols;
+        float ts = 0.0f;
+        for (int c = lane; c < cols; c += 64) {
+            const float t = tr[c];
+            l += -((xr[c] - mx) - lns) * t;
+            ts += t;
+        }
+        l = wave_allreduce_f32(l, OpAdd());
+        tsum = wave_allreduce_f32(ts, OpAdd());
+    } else {
+        label = ((const int32_t *)target)[row];
+        if (label >= 0 && label < cols) l = -((xr[label] - mx) - lns);
+    }
     if (loss && lane == 0) loss[row] = l;
     if (grad) {
         const float inv = 1.0f / s;
         for (int c = lane; c < cols; c += 64) {
             float p = expf(xr[c] - mx) * inv;
-            grad[row * cols + c] = (p - (c == label ? 1.0f : 0.0f)) * gscale;
+            if (DENSE) grad[row * cols + c] = (p * tsum - tr[c]) * gscale;
+            else grad[row * cols + c] = (p - (c == label ? 1.0f : 0.0f)) * gscale;
         }
     }
     return l;
 }
 
-__global__ __launch_bounds__(256) void cross_entropy_k(const float *__restrict__ x, const int32_t *__restrict__ labels,
+template <bool DENSE>
+__global__ __launch_bounds__(256) void cross_entropy_k(const float *__restrict__ x, const void *__restrict__ target,
                                                        float *__restrict__ loss, float *__restrict__ grad, int64_t rows,
                                                        int cols, float gscale) {
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
-    cross_entropy_row(x, labels, loss, grad, row, cols, gscale, threadIdx.x & 63);
+    cross_entropy_row<DENSE>(x, target, loss, grad, row, cols, gscale, threadIdx.x & 63);
 }
 
 // The whole batch in one workgroup of 16 waves, which also leaves mean[0] = sum(loss) / rows (ReduceOp::Mean): every
 // wave adds its rows' losses in row order, the 16 partial sums are added in wave order.
-__global__ __launch_bounds__(1024) void cross_entropy_mean_k(const float *__restrict__ x, const int32_t *__restrict__ labels,
+template <bool DENSE>
+__global__ __launch_bounds__(1024) void cross_entropy_mean_k(const float *__restrict__ x, const void *__restrict__ target,
                                                              float *__restrict__ loss, float *__restrict__ grad,
                                                              float *__restrict__ mean, int64_t rows, int cols, float gscale) {
     __shared__ float part[16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float sum = 0.0f;
-    for (int64_t row = wave; row < rows; row += 16) sum += cross_entropy_row(x, labels, loss, grad, row, cols, gscale, lane);
+    for (int64_t row = wave; row < rows; row += 16) sum += cross_entropy_row<DENSE>(x, target, loss, grad, row, cols, gscale, lane);
     if (lane == 0) part[wave] = sum;
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -550,14 +568,16 @@ hipError_t norm_rows_bwd(const NormRowsBwd &p, hipStream_t st) {
 hipError_t cross_entropy(const CrossEntropy &p, hipStream_t st) {
     if (p.rows <= 0 || p.cols <= 0) return hipSuccess;
     if (p.cols >= (1ll << 31) || (p.rows + 3) / 4 >= (1ll << 31)) return hipErrorInvalidValue;
+    const void *target = p.dense ? (const void *)p.dense : (const void *)p.labels;
     if (p.mean) {
         if (p.rows > kCrossEntropyMeanRows) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(cross_entropy_mean_k, dim3(1), dim3(1024), 0, st, p.x, p.labels, p.loss, p.grad, p.mean, p.rows,
-                           (int)p.cols, p.gscale);
+        if (p.dense) hipLaunchKernelGGL(cross_entropy_mean_k<true>, dim3(1), dim3(1024), 0, st, p.x, target, p.loss, p.grad, p.mean, p.rows, (int)p.cols, p.gscale);
+        else hipLaunchKernelGGL(cross_entropy_mean_k<false>, dim3(1), dim3(1024), 0, st, p.x, target, p.loss, p.grad, p.mean, p.rows, (int)p.cols, p.gscale);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL(cross_entropy_k, dim3((unsigned)((p.rows + 3) / 4)), dim3(256), 0, st, p.x, p.labels, p.loss, p.grad,
-                       p.rows, (int)p.cols, p.gscale);
+    const dim3 grid((unsigned)((p.rows + 3) / 4));
+    if (p.dense) hipLaunchKernelGGL(cross_entropy_k<true>, grid, dim3(256), 0, st, p.x, target, p.loss, p.grad, p.rows, (int)p.cols, p.gscale);
+    else hipLaunchKernelGGL(cross_entropy_k<false>, grid, dim3(256), 0, st, p.x, target, p.loss, p.grad, p.rows, (int)p.cols, p.gscale);
     return hipGetLastError();
 }
 

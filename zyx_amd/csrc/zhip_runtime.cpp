@@ -607,12 +607,12 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
         if (rows < 0 || cols < 0 || cols >= (1ll << 31) || (cols && rows > (1ll << 40) / cols))
             return c->fail(ZHIP_KERNEL_COMPILATION, "cross_entropy: rows/cols out of range");
         if (d.dtype != ZHIP_F32) return c->fail(ZHIP_KERNEL_COMPILATION, "cross_entropy: logits must be F32");
-        if ((d.flags & 7) == 0 || (d.flags & ~7)) return c->fail(ZHIP_KERNEL_COMPILATION, "cross_entropy: bad output flags");
+        if ((d.flags & 7) == 0 || (d.flags & ~15)) return c->fail(ZHIP_KERNEL_COMPILATION, "cross_entropy: bad output flags");
         if ((d.flags & ZHIP_CE_MEAN) && (rows < 1 || rows > zk::kCrossEntropyMeanRows))
             return c->fail(ZHIP_KERNEL_COMPILATION, "cross_entropy: the mean output takes 1 to %lld rows", (long long)zk::kCrossEntropyMeanRows);
         p.n_in = 2;
         p.need[0] = (uint64_t)rows * cols * 4;
-        p.need[1] = (uint64_t)rows * 4;
+        p.need[1] = (d.flags & ZHIP_CE_DENSE) ? (uint64_t)rows * cols * 4 : (uint64_t)rows * 4;
         int o = 2;
         if (d.flags & ZHIP_CE_LOSS) p.need[o++] = (uint64_t)rows * 4;
         if (d.flags & ZHIP_CE_GRAD) p.need[o++] = (uint64_t)rows * cols * 4;
@@ -906,7 +906,8 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st) {
         a.cols = d.dims[1];
         a.gscale = d.fparams[0];
         a.x = (const float *)ptr[0];
-        a.labels = (const int32_t *)ptr[1];
+        if (d.flags & ZHIP_CE_DENSE) a.dense = (const float *)ptr[1];
+        else a.labels = (const int32_t *)ptr[1];
         int o = 2;
         if (d.flags & ZHIP_CE_LOSS) a.loss = (float *)ptr[o++];
         if (d.flags & ZHIP_CE_GRAD) a.grad = (float *)ptr[o++];

@@ -195,6 +195,19 @@ class Graph:
         """`self.cmpgt(0) * self` (zyx/src/tensor/elementwise.rs:289-293)."""
         return self.binary(self.binary(x, self.const(0, self[x].dtype), BOp.Cmpgt), x, BOp.Mul)
 
+    def tanh(self, x: int) -> int:
+        """`e = (x + x).exp(); (e - 1) / (e + 1)` (zyx/src/tensor/elementwise.rs:585-588)."""
+        dt = self[x].dtype
+        e = self.unary(self.binary(x, x, BOp.Add), UOp.Exp)
+        return self.binary(self.binary(e, self.const(1, dt), BOp.Sub), self.binary(e, self.const(1, dt), BOp.Add), BOp.Div)
+
+    def gelu(self, x: int) -> int:
+        """`x * 0.5 * (tanh((x + x * x * x * 0.044715) * sqrt(2 / pi)) + 1)` (zyx/src/tensor/elementwise.rs:168-170)."""
+        dt = self[x].dtype
+        cube = self.binary(self.binary(self.binary(x, x, BOp.Mul), x, BOp.Mul), self.const(0.044715, dt), BOp.Mul)
+        inner = self.binary(self.binary(x, cube, BOp.Add), self.const(float(np.sqrt(np.float32(2.0) / np.float32(np.pi))), dt), BOp.Mul)
+        return self.binary(self.binary(x, self.const(0.5, dt), BOp.Mul), self.binary(self.tanh(inner), self.const(1, dt), BOp.Add), BOp.Mul)
+
     def t(self, x: int) -> int:
         r = len(self[x].shape)
         return x if r < 2 else self.permute(x, tuple(range(r - 2)) + (r - 1, r - 2))
@@ -240,6 +253,30 @@ class Graph:
 
     def max_all(self, x: int) -> int:
         return self.reduce(x, BOp.Max, range(len(self[x].shape)))
+
+    def mean(self, x: int, axes=()) -> int:
+        """`sum(axes) / n` with n the number of elements reduced, as a constant of x's dtype (`ReduceOp::Mean`,
+        zyx/src/tensor/reduce_ops.rs:102-110); no axes: all of them."""
+        xs = self[x].shape
+        axes = [self._axis(a, len(xs)) for a in axes] or list(range(len(xs)))
+        n = _numel([xs[a] for a in axes])
+        return self.binary(self.reduce(x, BOp.Add, axes), self.const(n, self[x].dtype), BOp.Div)
+
+    def cross_entropy(self, logits: int, target: int, reduction: str = "mean") -> int:
+        """`Tensor::cross_entropy` (zyx/src/tensor/mod.rs:1639-1655) for a target of the logits' shape (one-hot or soft
+        labels): `(-ln_softmax(logits, [classes]) * target).sum([classes])`, then the mean, the sum, or nothing;
+        the class axis is 0 for 1-D logits and 1 otherwise."""
+        if self[logits].shape != self[target].shape:
+            raise ValueError(f"target shape {self[target].shape} is not the logits' {self[logits].shape}")
+        cd = 0 if len(self[logits].shape) <= 1 else 1
+        per_sample = self.reduce(self.binary(self.unary(self.ln_softmax(logits, [cd]), UOp.Neg), target, BOp.Mul), BOp.Add, [cd])
+        if reduction == "mean":
+            return self.mean(per_sample)
+        if reduction == "sum":
+            return self.sum_all(per_sample)
+        if reduction == "none":
+            return per_sample
+        raise ValueError("invalid reduction for cross_entropy, expected mean, sum or none")
 
     # -- padding, slicing, pooling and convolution as the reference composes them ----------------------------------
     def pad_zeros(self, x: int, padding) -> int:
@@ -538,6 +575,14 @@ class Contraction:
     trans_b: bool
     dtype: DType
     fallback: object = None   # the generated kernel for the same node, reading the same operand buffers (set by `lower`)
+    # what the GEMM's epilogue applies before it stores (found by `match_linear`): out = act(alpha * product + bias),
+    # then + residual, or * (residual > 0)
+    epilogue: str = "none"    # "none" | "bias" | "bias_relu" | "bias_gelu"
+    bias: int | None = None
+    alpha: float = 1.0
+    residual: int | None = None
+    relu_mask: bool = False   # the residual operand is a relu's input or output: multiply by (residual > 0)
+    mask_node: int | None = None  # the `v > 0` node of a relu folded into the epilogue (its v is never stored)
 
 
 def _reshape_strides(old_shape, old_strides, new_shape):
@@ -723,6 +768,8 @@ class RowColReduce:
     axis0: bool
     op: str
     dtype: DType
+    mul: float = 0.0          # out = reduce * mul + base when a base is named (`base - reduce * c` is mul = -c)
+    base: int | None = None
 
 
 def match_reduce(graph: Graph, nid: int, stored) -> RowColReduce | None:
@@ -834,16 +881,306 @@ def match_max_pool(graph: Graph, nid: int) -> MaxPoolMatch | None:
                         info["dilation"], graph[nid].dtype)
 
 
+
+
+# ---- matching by template: an expression has the shape of one the builders above produce -----------------------------
+
+def same_tree(graph: Graph, nid: int, tgraph: Graph, tid: int, bind: dict) -> bool:
+    """True when the expression below `nid` is, node for node, the expression below `tid` of `tgraph`; the leaves of
+    the template stand for any node of their shape and dtype. `bind` (template node -> graph node) is extended; a
+    template node reached twice has to meet the same graph node both times."""
+    todo = [(nid, tid)]
+    while todo:
+        a, t = todo.pop()
+        if t in bind:
+            if bind[t] != a:
+                return False
+            continue
+        na, nt = graph[a], tgraph[t]
+        if na.shape != nt.shape or na.dtype != nt.dtype:
+            return False
+        if nt.kind != "leaf":
+            if na.kind != nt.kind or na.op != nt.op or len(na.src) != len(nt.src) or na.arg != nt.arg:
+                return False
+            todo.extend(zip(na.src, nt.src))
+        bind[t] = a
+    return True
+
+
+_TEMPLATES: dict = {}
+
+
+def _template(key, build):
+    """Templates are built once per (kind, shape, dtype, ...)."""
+    if key not in _TEMPLATES:
+        if len(_TEMPLATES) > 256:
+            _TEMPLATES.clear()
+        t = Graph()
+        _TEMPLATES[key] = (t, build(t))
+    return _TEMPLATES[key]
+
+
+def _is_gelu_of(graph: Graph, nid: int):
+    """The node x when `nid` is `Graph.gelu(x)`, else None."""
+    n = graph[nid]
+    if n.kind != "binary" or n.op != BOp.Mul or n.dtype not in (DType.F32, DType.BF16, DType.F16):
+        return None
+
+    def build(t):
+        x = t.leaf(n.shape, n.dtype)
+        return x, t.gelu(x)
+
+    t, (x, root) = _template(("gelu", n.shape, n.dtype), build)
+    bind: dict = {}
+    return bind[x] if same_tree(graph, nid, t, root, bind) else None
+
+
+def _interior(graph: Graph, root: int, stop: int) -> set:
+    """Nodes strictly between `root` and `stop` (the expression of root in terms of stop)."""
+    seen, stack = set(), [root]
+    while stack:
+        i = stack.pop()
+        for s_ in graph[i].src:
+            if s_ != stop and s_ not in seen and graph[s_].kind != "const":
+                seen.add(s_)
+                stack.append(s_)
+    return seen
+
+
+def _plain(graph: Graph, nid: int):
+    """The node whose buffer holds `nid` element for element (reshapes and permutes that keep the linear order), or
+    None when `nid` is a strided or broadcast view."""
+    base, st = view_of(graph, nid)
+    shape = graph[nid].shape
+    if _numel(graph[base].shape) != _numel(shape):
+        return None
+    want = _contiguous(shape)
+    return base if all(d == 1 or a == b for d, a, b in zip(shape, st, want)) else None
+
+
+def _row_vector(graph: Graph, nid: int):
+    """The [n] node that `nid` ([.., n]) repeats along all its leading axes, or None."""
+    base, st = view_of(graph, nid)
+    shape = graph[nid].shape
+    if not shape or _numel(graph[base].shape) != shape[-1] or shape[-1] == 1:
+        return None
+    if st[-1] != 1 or any(d != 1 and v != 0 for d, v in zip(shape[:-1], st[:-1])):
+        return None
+    return base
+
+
+def _const_value(graph: Graph, nid: int):
+    """The scalar a node broadcasts, or None."""
+    base, _ = view_of(graph, nid)
+    n = graph[base]
+    return n.arg if n.kind == "const" else None
+
+
+def match_linear(graph: Graph, nid: int, users: dict, relu_mask: dict):
+    """A product summed over shared axes together with what the GEMM kernel's epilogue can apply to it on the way out
+    (`Linear::forward` zyx-nn/src/linear.rs:38-44 with the activation behind it, and the three products of its reverse
+    pass with the SGD step zyx-optim/src/sgd.rs:45-84 behind them):
+      act(product + bias)            act = relu | gelu | nothing, bias repeated along the rows
+      w - product * c                a parameter update: alpha = -c, residual = w
+      product * (v > 0)              the reverse of a relu: residual = v (or relu(v) where only that is stored)
+    `users`: node -> consumers among the nodes being computed; an inner node folded away must have no other reader.
+    Returns a `Contraction` whose `out` is `nid`, or None."""
+    n = graph[nid]
+    if n.dtype not in (DType.F32, DType.BF16, DType.F16) or n.kind not in ("binary", "reduce", "reshape", "permute"):
+        return None
+
+    def only_reader(node, *readers):
+        return users.get(node, set()) <= set(readers)
+
+    def product(node, reader):
+        """The Contraction of the reduce that `node` shows element for element, if `reader` alone reads it."""
+        base = _plain(graph, node)
+        if base is None or graph[base].kind != "reduce":
+            return None
+        chain, i = [], node
+        while i != base:  # the views between node and the reduce: each read by the next only
+            chain.append(i)
+            i = graph[i].src[0]
+        chain.append(base)
+        for j, v in enumerate(chain):
+            if not only_reader(v, reader if j == 0 else chain[j - 1]):
+                return None
+        return match_contraction(graph, base)
+
+    cur, act, mask_node = nid, None, None
+    v = _is_relu_of(graph, cur)
+    if v is not None and users.get(v, set()) == {graph[cur].src[0], cur}:
+        act, mask_node, cur = "relu", graph[cur].src[0], v
+    else:
+        v = _is_gelu_of(graph, cur)
+        if v is not None:
+            inner = _interior(graph, cur, v)
+            if all(users.get(i, set()) <= inner | {cur} for i in inner | {v}):
+                act, cur = "gelu", v
+    c = graph[cur]
+    if c.kind == "binary" and c.op == BOp.Add:
+        for core, other in (c.src, c.src[::-1]):
+            bias = _row_vector(graph, other)
+            if bias is None or graph[bias].dtype != n.dtype:
+                continue
+            m = product(core, cur)
+            if m is not None and m.batch == 1 and _numel(graph[bias].shape) == m.n:
+                m.out, m.bias, m.mask_node = nid, bias, mask_node
+                m.epilogue = {None: "bias", "relu": "bias_relu", "gelu": "bias_gelu"}[act]
+                return m
+        return None
+    if act is not None:
+        return None  # an activation straight on a product: the kernel has no such epilogue
+    if c.kind == "binary" and c.op == BOp.Sub:
+        w, scaled = c.src
+        sc = graph[scaled]
+        wb = _plain(graph, w)
+        if wb is None or sc.kind != "binary" or sc.op != BOp.Mul:
+            return None
+        for core, other in (sc.src, sc.src[::-1]):
+            k = _const_value(graph, other)
+            if k is None or not only_reader(scaled, cur):
+                continue
+            m = product(core, scaled)
+            if m is not None and m.batch == 1:
+                m.out, m.alpha, m.residual = nid, -float(k), wb
+                return m
+        return None
+    if c.kind == "binary" and c.op == BOp.Mul:
+        for core, other in (c.src, c.src[::-1]):
+            o = graph[other]
+            if o.kind != "binary" or o.op != BOp.Cmpgt or _const_value(graph, o.src[1]) != 0:
+                continue
+            shown = relu_mask.get(other)
+            if shown is None:  # relu(v) > 0 is v > 0: where the relu itself is computed, read that
+                shown = next((r for r in users.get(o.src[0], ()) if r >= 0 and _is_relu_of(graph, r) == o.src[0]), o.src[0])
+            vb = _plain(graph, shown)
+            if vb is None or graph[vb].dtype != n.dtype:
+                continue
+            m = product(core, cur)
+            if m is not None and m.batch == 1:
+                m.out, m.residual, m.relu_mask = nid, vb, True
+                return m
+    return None
+
+
+def match_reduce_update(graph: Graph, nid: int, users: dict) -> RowColReduce | None:
+    """`b - reduce(x) * c` with x a whole buffer that exists (a bias update, zyx-optim/src/sgd.rs:45-84 applied to
+    the column sums the reverse pass of a broadcast bias leaves): one launch of the reduce kernel with its scale and
+    base operands, whatever the length of the reduction."""
+    n = graph[nid]
+    if n.kind != "binary" or n.op != BOp.Sub or n.dtype != DType.F32:
+        return None
+    b, scaled = n.src
+    bb, sc = _plain(graph, b), graph[scaled]
+    if bb is None or sc.kind != "binary" or sc.op != BOp.Mul:
+        return None
+    if not users.get(scaled, set()) <= {nid}:
+        return None
+    for core, other in (sc.src, sc.src[::-1]):
+        k = _const_value(graph, other)
+        base = _plain(graph, core)
+        if k is None or base is None or graph[base].kind != "reduce" or graph[base].op != BOp.Add:
+            continue
+        r = graph[base]
+        x = r.src[0]
+        xs = graph[x].shape
+        xb = _plain(graph, x)
+        if xb is None:
+            continue
+        kk, rank = len(r.arg), len(xs)
+        if r.arg == tuple(range(rank - kk, rank)):
+            rows, cols, axis0 = _numel(xs[:rank - kk]), _numel(xs[rank - kk:]), False
+        elif r.arg == tuple(range(kk)):
+            rows, cols, axis0 = _numel(xs[:kk]), _numel(xs[kk:]), True
+        else:
+            continue
+        return RowColReduce(xb, nid, rows, cols, axis0, "sum", r.dtype, mul=-float(k), base=bb)
+    return None
+
+
+@dataclasses.dataclass
+class CrossEntropyMatch:
+    """`Graph.cross_entropy(x, target, "mean")` and / or its gradient with respect to x, found in the graph: one launch
+    of ZHIP_K_CROSS_ENTROPY with dense targets writes both."""
+    x: int
+    target: int
+    rows: int
+    cols: int
+    gscale: float
+    grad: int | None = None
+    mean: int | None = None
+
+    @property
+    def out(self):
+        return self.grad if self.grad is not None else self.mean
+
+
+def _ce_template(rows: int, cols: int, reduction: str):
+    def build(t):
+        x, y = t.leaf((rows, cols), DType.F32), t.leaf((rows, cols), DType.F32)
+        loss = t.cross_entropy(x, y, reduction)
+        (gx,) = t.gradient(loss, [x])
+        return x, y, loss, gx
+
+    return _template(("ce", rows, cols, reduction), build)
+
+
+def scan_cross_entropy(graph: Graph, nodes) -> dict:
+    """node -> CrossEntropyMatch for the mean cross-entropy losses among `nodes` and the gradients the reverse rules
+    derive from such a loss (mean or sum) for its logits. The gradient's template is what `Graph.gradient` makes of
+    the template loss: the same rules applied to the same expression give the same expression, so the comparison is
+    node for node. A loss and a gradient over the same logits and target share one match (one launch)."""
+    found: dict[tuple, CrossEntropyMatch] = {}
+    by_node: dict[int, CrossEntropyMatch] = {}
+    for nid in nodes:
+        n = graph[nid]
+        if n.dtype != DType.F32 or n.kind != "binary":
+            continue
+        if n.shape == (1,) and n.op == BOp.Div:
+            r = graph[n.src[0]]
+            per = graph[r.src[0]] if r.kind == "reduce" and r.src else None
+            prod = graph[per.src[0]] if per is not None and per.kind == "reduce" else None
+            if prod is None or len(prod.shape) != 2:
+                continue
+            rows, cols = prod.shape
+            t, (tx, ty, tloss, _) = _ce_template(rows, cols, "mean")
+            bind: dict = {}
+            if same_tree(graph, nid, t, tloss, bind):
+                m = found.setdefault((bind[tx], bind[ty]), CrossEntropyMatch(bind[tx], bind[ty], rows, cols, 1.0 / rows))
+                if m.mean is None:
+                    m.mean = nid
+                    by_node[nid] = m
+        elif len(n.shape) == 2:
+            rows, cols = n.shape
+            for reduction, gscale in (("mean", 1.0 / rows), ("sum", 1.0)):
+                t, (tx, ty, _, tgx) = _ce_template(rows, cols, reduction)
+                if graph[nid].op != t[tgx].op:
+                    continue
+                bind = {}
+                if same_tree(graph, nid, t, tgx, bind) and tx in bind and ty in bind:
+                    m = found.setdefault((bind[tx], bind[ty]), CrossEntropyMatch(bind[tx], bind[ty], rows, cols, gscale))
+                    if m.grad is None and m.gscale == gscale:
+                        m.grad = nid
+                        by_node[nid] = m
+                    break
+    return by_node
+
+
 def match_operands(m) -> tuple:
-    """Nodes whose buffers a matched kernel reads."""
+    """Nodes whose buffers a matched kernel reads, in argument order."""
     if isinstance(m, Contraction):
-        return (m.a, m.b)
+        return (m.a, m.b) + ((m.bias,) if m.bias is not None else ()) + ((m.residual,) if m.residual is not None else ())
+    if isinstance(m, RowColReduce):
+        return (m.x,) + ((m.base,) if m.base is not None else ())
+    if isinstance(m, CrossEntropyMatch):
+        return (m.x, m.target)
     if isinstance(m, Conv2dMatch):
         return (m.x, m.w) + ((m.bias,) if m.bias is not None else ())
     return (m.x,)
 
 
-MATCHED = (Contraction, SoftmaxRows, RowColReduce, Conv2dMatch, MaxPoolMatch)
+MATCHED = (Contraction, SoftmaxRows, RowColReduce, Conv2dMatch, MaxPoolMatch, CrossEntropyMatch)
 
 
 # ---- lowering ---------------------------------------------------------------------------------------------------------
@@ -854,6 +1191,7 @@ class LoweredKernel:
     inputs: list      # node ids of the buffers read, in parameter order
     output: int       # node id of the buffer written
     elements: int
+    more_outputs: tuple = ()  # further buffers written, after `output` in the argument list
 
 
 class _V:
@@ -1069,29 +1407,38 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
     emitter = _Emitter(graph, have)
     schedule: list = []
     users = consumers(graph, outputs, stored) if match else {}
+    losses = scan_cross_entropy(graph, [i for i in users if i >= 0] + list(outputs)) if match else {}
+
+    def find(nid: int):
+        return (losses.get(nid) or match_conv(graph, nid, users) or match_max_pool(graph, nid)
+                or match_linear(graph, nid, users, emitter.relu_mask) or match_contraction(graph, nid)
+                or match_softmax(graph, nid) or match_reduce_update(graph, nid, users) or match_reduce(graph, nid, have))
 
     def need(nid: int, root: bool):
         n = graph[nid]
         if n.kind == "leaf" or nid in have:
             return
-        if match and nid in graph.convs:
-            # a convolution read only by its relu is never stored: the relu's launch computes both, and the relu's mask
-            # `conv > 0`, which the reverse pass reads, is taken from the relu's result (`relu(v) > 0` is `v > 0`)
+        if match:
+            # A convolution or a Linear read only by its relu is never stored: the relu's launch computes both, and the
+            # relu's mask `v > 0`, which the reverse pass reads, is taken from the relu's result (`relu(v) > 0` is `v > 0`).
             for r in users.get(nid, ()):
-                if _is_relu_of(graph, r) == nid and match_conv(graph, r, users) is not None:
-                    need(r, True)
-                    return
-        c = (match_conv(graph, nid, users) or match_max_pool(graph, nid) or match_contraction(graph, nid) or match_softmax(graph, nid)
-             or match_reduce(graph, nid, have)) if match else None
+                if r >= 0 and _is_relu_of(graph, r) == nid:
+                    m = match_conv(graph, r, users) or match_linear(graph, r, users, emitter.relu_mask)
+                    if m is not None and (getattr(m, "relu", False) or getattr(m, "mask_node", None) is not None):
+                        need(r, True)
+                        return
+        c = find(nid) if match else None
         if c is not None:
             for s in match_operands(c):
                 need(s, True)
-            if isinstance(c, Contraction):
+            if isinstance(c, Contraction) and c.epilogue == "none" and c.residual is None:
                 c.fallback = emitter.kernel(nid)
             if isinstance(c, Conv2dMatch) and c.relu:
                 emitter.relu_mask[graph[nid].src[0]] = nid
+            if isinstance(c, Contraction) and c.mask_node is not None:
+                emitter.relu_mask[c.mask_node] = nid
             schedule.append(c)
-            have.add(nid)
+            have.update(i for i in ((c.grad, c.mean) if isinstance(c, CrossEntropyMatch) else (nid,)) if i is not None)
             return
         for s in n.src:
             need(s, False)
@@ -1132,6 +1479,7 @@ class Tape:
         self._keep: list = []
         self._last = None  # event of the most recent launch: launches form one chain
         self._plans: list = []
+        self._spare: list = []  # second buffers of the input leaves of plans
 
     def tensor(self, array, dtype: DType) -> int:
         a = np.ascontiguousarray(array, storage_dtype(dtype))
@@ -1156,8 +1504,9 @@ class Tape:
             prog = self._programs.get(kern.image)
             if prog is None:
                 prog = self._programs[kern.image] = self.dev.compile(kern.image)
-            if kern.output not in self._buf:
-                self._alloc(kern.output)
+            for o in (kern.output,) + tuple(kern.more_outputs):
+                if o not in self._buf:
+                    self._alloc(o)
             # A launch consumes the events it waits for, and it waits for everything outstanding: the launch before it
             # and every upload, copy or allocation whose event nobody has consumed yet (after `write` / `assign` the
             # chain of launches continues in such an event, not in `_last`). The launches thus form one chain, and a
@@ -1166,12 +1515,30 @@ class Tape:
             self._ev.clear()
             if self._last is not None:
                 waits.append(self._last)
-            self._last = self.dev.launch(prog, self.pool, [self._buf[i] for i in kern.inputs] + [self._buf[kern.output]], waits)
+            self._last = self.dev.launch(prog, self.pool, [self._buf[i] for i in kern.inputs + [kern.output] + list(kern.more_outputs)], waits)
 
-    def plan(self, nodes: Sequence[int]) -> "TapePlan":
+    def plan(self, nodes: Sequence[int], updates: dict | None = None, inputs: Sequence[int] = ()) -> "TapePlan":
         """The schedule of `nodes` as one cached plan (a HIP graph): the analogue of the reference's plan cache
         (zyx/src/graph/plan.rs:58-237). Leaves may be rewritten with `write` between launches; every launch
-        recomputes all the plan's nodes from the leaves' current contents."""
+        recomputes all the plan's nodes from the leaves' current contents.
+
+        updates: {leaf: node} -- after every launch the leaf holds what the launch computed for the node
+        (`Tensor::assign` of every updated parameter, as an optimizer step ends: zyx-optim/src/sgd.rs:45-84), without
+        a copy: a kernel's outputs never alias its inputs, so the plan exists twice, over the two buffers of each pair
+        in either role, and the pairs swap after each launch. Between launches the node's own value is the leaf's
+        previous one.
+
+        inputs: leaves the caller rewrites before every launch (the batch). Each gets a second buffer and the two
+        copies of the plan read them alternately, so `write` fills the one the running launch does not read and the
+        upload of the next batch overlaps the current step."""
+        updates = dict(updates or {})
+        for leaf in inputs:
+            if self.graph[leaf].kind != "leaf" or leaf in updates:
+                raise ValueError("inputs are leaves that no update writes")
+        for leaf, node in updates.items():
+            a, b = self.graph[leaf], self.graph[node]
+            if a.kind != "leaf" or a.shape != b.shape or a.dtype != b.dtype or node not in nodes or self.graph[node].kind == "leaf":
+                raise ValueError("updates map leaves to nodes of the plan with the leaf's shape and dtype")
         if self.match == "time":
             self.realize(nodes)  # settles which candidate each product runs on; the plan reuses the buffers
         self.sync()
@@ -1183,11 +1550,27 @@ class Tape:
             prog = self._programs.get(kern.image)
             if prog is None:
                 prog = self._programs[kern.image] = self.dev.compile(kern.image)
-            if kern.output not in self._buf:
-                self._alloc(kern.output)
-            launches.append((prog, [self._buf[i] for i in kern.inputs] + [self._buf[kern.output]]))
+            outs = [kern.output] + list(kern.more_outputs)
+            for o in outs:
+                if o not in self._buf:
+                    self._alloc(o)
+            launches.append((prog, [self._buf[i] for i in kern.inputs + outs]))
         self.sync()
-        return TapePlan(self, self.dev.create_plan(launches), len(launches))
+        ids = [self.dev.create_plan(launches)]
+        pairs = dict(updates)
+        for leaf in inputs:  # the alternate of an input leaf is a buffer of its own, filled by the next `write`
+            n = self.graph[leaf]
+            buf, ev = self.pool.allocate(max(_numel(n.shape), 1) * np.dtype(storage_dtype(n.dtype)).itemsize)
+            self.pool.sync_events([ev])
+            pairs[leaf] = ("alt", buf)
+            self._spare.append(buf)
+        if pairs:
+            swap = {}
+            for leaf, other in pairs.items():
+                ob = other[1] if isinstance(other, tuple) else self._buf[other]
+                swap[self._buf[leaf]], swap[ob] = ob, self._buf[leaf]
+            ids.append(self.dev.create_plan([(prog, [swap.get(b, b) for b in bufs]) for prog, bufs in launches]))
+        return TapePlan(self, ids, len(launches), pairs)
 
     def write(self, leaf: int, array):
         """New contents for a leaf (same shape and dtype); later launches read them."""
@@ -1196,10 +1579,12 @@ class Tape:
         if n.kind != "leaf" or a.shape != n.shape:
             raise ValueError("write takes a leaf and an array of its shape")
         self._keep.append(a)
+        if len(self._keep) > 1024:  # bound the host arrays kept alive: after a sync none is still being read
+            self.sync()
+            self._keep.append(a)
+        # No wait for the launch in flight: the runtime orders a copy after every earlier access of its destination by
+        # itself, and a launch that does not touch this buffer has no reason to hold the upload back.
         waits = [self._ev.pop(leaf)] if leaf in self._ev else []
-        if self._last is not None:  # a running launch may still read the old contents
-            waits.append(self._last)
-            self._last = None
         self._ev[leaf] = self.pool.host_to_pool(a, self._buf[leaf], waits)
 
     def assign(self, leaf: int, node: int):
@@ -1216,7 +1601,8 @@ class Tape:
         self._ev[leaf] = self.pool.copy_range(self._buf[node], 0, self._buf[leaf], 0, nbytes, waits)
 
     def _matched_or_generated(self, c) -> LoweredKernel:
-        from .kernels import conv2d_desc, gemm_desc, max_pool2d_desc, reduce_desc, softmax_rows_desc
+        from .kernels import conv2d_desc, cross_entropy_desc, gemm_desc, max_pool2d_desc, reduce_desc, softmax_rows_desc
+        more = ()
         if isinstance(c, Conv2dMatch):
             n_, c_, h, w, co, kh, kw = c.dims
             desc = conv2d_desc(n_, c_, h, w, co, kh, kw, c.stride, c.padding, c.dilation, c.bias is not None, c.relu, c.dtype)
@@ -1225,19 +1611,25 @@ class Tape:
             desc = max_pool2d_desc(c.planes, c.hw[0], c.hw[1], c.kernel, c.stride, c.padding, c.dilation, c.dtype)
             inputs, elements = [c.x], _numel(self.graph[c.out].shape)
         elif isinstance(c, Contraction):
-            desc = gemm_desc(c.m, c.n, c.k, c.dtype, c.dtype, c.trans_a, c.trans_b, batch=c.batch)
-            inputs, elements = [c.a, c.b], c.batch * c.m * c.n
+            bias_dtype = self.graph[c.bias].dtype if c.bias is not None else DType.F32
+            desc = gemm_desc(c.m, c.n, c.k, c.dtype, c.dtype, c.trans_a, c.trans_b, c.epilogue, bias_dtype, c.batch, c.alpha,
+                             "relu_mask" if c.relu_mask else c.residual is not None)
+            inputs, elements = list(match_operands(c)), c.batch * c.m * c.n
         elif isinstance(c, RowColReduce):
-            desc = reduce_desc(c.rows, c.cols, c.op, c.axis0, c.dtype)
-            inputs, elements = [c.x], c.cols if c.axis0 else c.rows
+            desc = reduce_desc(c.rows, c.cols, c.op, c.axis0, c.dtype, mul=c.mul, base=c.base is not None)
+            inputs, elements = list(match_operands(c)), c.cols if c.axis0 else c.rows
+        elif isinstance(c, CrossEntropyMatch):
+            desc = cross_entropy_desc(c.rows, c.cols, False, c.grad is not None, c.gscale, c.mean is not None, dense=True)
+            inputs, elements = [c.x, c.target], c.rows * c.cols if c.grad is not None else 1
+            more = (c.mean,) if c.grad is not None and c.mean is not None else ()
         else:
             desc = softmax_rows_desc(c.rows, c.cols, y=True, rowsum=False, argmax=False)
             inputs, elements = [c.x], c.rows * c.cols
         key = bytes(desc)
         if key not in self._programs:
             self._programs[key] = self.dev.register_kernel(desc)
-        gemm = LoweredKernel(key, inputs, c.out, elements)
-        if self.match == "time" and isinstance(c, Contraction):
+        gemm = LoweredKernel(key, inputs, c.out, elements, more)
+        if self.match == "time" and isinstance(c, Contraction) and c.fallback is not None:
             pair = (key, c.fallback.image)
             if pair not in self._choice:
                 if c.fallback.image not in self._programs:
@@ -1279,8 +1671,9 @@ class Tape:
         self._plans.clear()
         for prog in self._programs.values():
             self.dev.release(prog)
-        for buf in self._buf.values():
+        for buf in list(self._buf.values()) + self._spare:
             self.pool.deallocate(buf, [])
+        self._spare.clear()
         self._programs.clear()
         self._buf.clear()
 
@@ -1288,12 +1681,23 @@ class Tape:
 class TapePlan:
     """A realised schedule kept as one replayable unit; `launch` runs it after everything the tape has outstanding."""
 
-    def __init__(self, tape: Tape, plan_id: int, launches: int):
-        self.tape, self.id, self.launches = tape, plan_id, launches
-        tape._plans.append(plan_id)
+    def __init__(self, tape: Tape, plan_ids: list, launches: int, updates: dict | None = None):
+        self.tape, self.ids, self.launches, self.updates = tape, plan_ids, launches, dict(updates or {})
+        self._parity = 0
+        tape._plans.extend(plan_ids)
 
     def launch(self):
         t = self.tape
         waits = list(t._ev.values()) + ([t._last] if t._last is not None else [])
         t._ev.clear()
-        t._last = t.dev.launch_plan(self.id, waits)
+        t._last = t.dev.launch_plan(self.ids[self._parity], waits)
+        if self.updates:
+            for leaf, other in self.updates.items():
+                if isinstance(other, tuple):  # an input leaf: the next `write` goes to the buffer this launch does not read
+                    spare = other[1]
+                    self.updates[leaf] = ("alt", t._buf[leaf])
+                    t._spare[t._spare.index(spare)] = t._buf[leaf]
+                    t._buf[leaf] = spare
+                else:
+                    t._buf[leaf], t._buf[other] = t._buf[other], t._buf[leaf]
+            self._parity ^= 1

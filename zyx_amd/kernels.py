@@ -278,7 +278,7 @@ def gemm(dev: HIPDevice, pool: HIPMemoryPool, a: np.ndarray, b: np.ndarray, bias
 # ---- LayerNorm / RMSNorm (ZHIP_K_NORM_ROWS), cross entropy (ZHIP_K_CROSS_ENTROPY) --------------------
 K_NORM_ROWS, K_CROSS_ENTROPY = 5, 6
 NORM_RMS, NORM_WEIGHT, NORM_BIAS = 1, 2, 4
-CE_LOSS, CE_GRAD, CE_MEAN = 1, 2, 4
+CE_LOSS, CE_GRAD, CE_MEAN, CE_DENSE = 1, 2, 4, 8
 
 
 def norm_rows_desc(rows: int, cols: int, rms=False, weight=True, bias=True, eps=1e-5, dtype: DType = DType.F32) -> KernelDesc:
@@ -310,23 +310,25 @@ def norm_rows(dev: HIPDevice, pool: HIPMemoryPool, x, w=None, b=None, rms=False,
     return y
 
 
-def cross_entropy_desc(rows: int, cols: int, loss=True, grad=False, gscale: float = 1.0, mean=False) -> KernelDesc:
-    """args: logits, labels, (loss[rows]), (grad[rows, cols]), (mean[1])."""
+def cross_entropy_desc(rows: int, cols: int, loss=True, grad=False, gscale: float = 1.0, mean=False, dense=False) -> KernelDesc:
+    """args: logits, labels (dense: f32 targets[rows, cols]), (loss[rows]), (grad[rows, cols]), (mean[1])."""
     d = KernelDesc()
     d.kind, d.dtype, d.out_dtype = K_CROSS_ENTROPY, DType.F32, DType.F32
-    d.flags = (CE_LOSS if loss else 0) | (CE_GRAD if grad else 0) | (CE_MEAN if mean else 0)
+    d.flags = (CE_LOSS if loss else 0) | (CE_GRAD if grad else 0) | (CE_MEAN if mean else 0) | (CE_DENSE if dense else 0)
     d.dims[0], d.dims[1] = rows, cols
     d.fparams[0] = gscale
     return d
 
 
-def cross_entropy(dev: HIPDevice, pool: HIPMemoryPool, logits, labels, grad_scale=None, mean=False):
+def cross_entropy(dev: HIPDevice, pool: HIPMemoryPool, logits, labels, grad_scale=None, mean=False, dense=False):
     """-> (per-sample loss, grad or None); grad = d(grad_scale * sum(loss)) / d(logits). With mean=True a third
-    value, the batch mean from the same launch."""
+    value, the batch mean from the same launch. dense: `labels` is an f32 target tensor of the logits' shape."""
     x = np.ascontiguousarray(logits, np.float32)
-    lab = np.ascontiguousarray(labels, np.int32)
+    lab = np.ascontiguousarray(labels, np.float32 if dense else np.int32)
     rows, cols = x.shape
-    prog = dev.register_kernel(cross_entropy_desc(rows, cols, True, grad_scale is not None, grad_scale or 0.0, mean))
+    if dense and lab.shape != x.shape:
+        raise ValueError("dense targets have the logits' shape")
+    prog = dev.register_kernel(cross_entropy_desc(rows, cols, True, grad_scale is not None, grad_scale or 0.0, mean, dense))
     xb, e0 = to_device(pool, x)
     lb, e1 = to_device(pool, lab)
     ob, e2 = alloc_like(pool, rows, 4)
