@@ -30,8 +30,20 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 N_SETS = 4              # 4 x 268 MB working set > Infinity Cache
 # HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
 # by the same counter's reading for a plain copy kernel of known size in the same run
-# (profiles/softmax_rows_f32_8192x4096.md): 134,352,818 B fetched + 134,461,653 B written.
-TRAFFIC_BYTES = 268814470
+# (profiles/softmax_rows_f32_8192x4096.md): 134,351,537 B fetched + 134,443,294 B written.
+TRAFFIC_BYTES = 268794831
+
+
+def measured_ceilings(dev, nbytes: int = 1 << 30):
+    """What this device sustains right now, beside the published peaks the roofline fractions are quoted against:
+    hipMemcpy device to device and a float4 copy kernel over `nbytes` (bytes read + written per second), a read-only
+    kernel (bytes read), and a register-resident v_mfma_f32_32x32x16_bf16 loop on all compute units with constant
+    operands (the clock holds) and with random ones (the power limit lowers it): rate, average clock, launch time."""
+    c = dev.measure_ceilings(nbytes)
+    c["bytes"] = nbytes
+    c["frac_of_8TB/s"] = {k: round(c[k] / HBM_PEAK_GBPS, 4) for k in ("memcpy_d2d_GBps", "copy_kernel_GBps", "read_kernel_GBps")}
+    c["frac_of_2.5PF"] = {k: round(c[k] / 2500.0, 4) for k in ("mfma_bf16_const_TFLOPs", "mfma_bf16_random_TFLOPs")}
+    return c
 
 
 def cpu_baseline(x: np.ndarray, budget_s: float = 10.0):
@@ -442,6 +454,9 @@ def main():
     ap.add_argument("--attention-only", action="store_true", help="run only the attention core leg")
     ap.add_argument("--ir-only", action="store_true", help="run only the generated-kernel leg")
     ap.add_argument("--graph-only", action="store_true", help="run only the config-1 training step through the graph path")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="run only the ceiling probes (hipMemcpy device to device, copy and read-only kernels, bf16 "
+                         "matrix-instruction loops on constant and on random operands) and print them")
     ap.add_argument("--counters", action="store_true",
                     help="short run for `rocprofv3 --pmc`: a few launches of the fused kernel and of a plain copy "
                          "kernel over the same 8192x4096 f32 tensor (known traffic: 134217728 B read + written), "
@@ -458,8 +473,15 @@ def main():
     pool, dev = pools[0], devices[0]
     info = dev.info()
 
+    if args.mfma_ceiling:
+        print(json.dumps({"measured_ceilings": measured_ceilings(dev)}))
+        pool.deinitialize()
+        return
+
     if args.gemm_only:
-        print(json.dumps({"config3_gemm_bf16_4096": extra_gemm(dev, pool, kernels, steps=args.steps, warmup=max(args.warmup, 100))}))
+        res = extra_gemm(dev, pool, kernels, steps=args.steps, warmup=max(args.warmup, 100))
+        res["measured_ceilings"] = measured_ceilings(dev)
+        print(json.dumps({"config3_gemm_bf16_4096": res}))
         pool.deinitialize()
         return
 
@@ -554,6 +576,9 @@ def main():
         for b in s:
             pool.deallocate(b, [])
     dev.release(prog)
+    ceil = measured_ceilings(dev)
+    out["config"]["measured_ceilings"] = ceil
+    out["roofline"]["frac_of_measured_copy_kernel"] = round(achieved / ceil["copy_kernel_GBps"], 4) if ceil["copy_kernel_GBps"] else None
     if not args.no_extra:
         # other configs of the same backend, reported beside the headline (not part of `value`)
         out["extra"] = {"config3_gemm_bf16_4096": extra_gemm(dev, pool, kernels),

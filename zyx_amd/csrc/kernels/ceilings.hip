@@ -13,18 +13,16 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-// dst[i] = src[i], 16 bytes per lane and trip, 4 trips in flight, streaming accesses
+// dst[i] = src[i]: every wave moves one contiguous 16 KiB piece, its 16 loads of 16 bytes per lane all in flight before
+// the first store (the access pattern of the row kernels), streaming accesses. n16 is a multiple of 4096.
 __global__ __launch_bounds__(256) void probe_copy_k(const f32x4 *__restrict__ src, f32x4 *__restrict__ dst, int64_t n16) {
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    for (; i + 3 * stride < n16; i += 4 * stride) {
-        f32x4 a = load_stream(src + i), b = load_stream(src + i + stride), c = load_stream(src + i + 2 * stride), d = load_stream(src + i + 3 * stride);
-        store_stream(a, dst + i);
-        store_stream(b, dst + i + stride);
-        store_stream(c, dst + i + 2 * stride);
-        store_stream(d, dst + i + 3 * stride);
-    }
-    for (; i < n16; i += stride) store_stream(load_stream(src + i), dst + i);
+    const int64_t base = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 1024 + (threadIdx.x & 63);
+    if (base >= n16) return;
+    f32x4 v[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) v[k] = load_stream(src + base + k * 64);
+#pragma unroll
+    for (int k = 0; k < 16; k++) store_stream(v[k], dst + base + k * 64);
 }
 // out[block] = sum of a slice: the read-only ceiling
 __global__ __launch_bounds__(256) void probe_read_k(const f32x4 *__restrict__ src, float *__restrict__ out, int64_t n16) {
@@ -86,7 +84,7 @@ __global__ __launch_bounds__(256, 1) void probe_mfma_k(float *__restrict__ out, 
 
 hipError_t measure_ceilings(uint64_t bytes, int compute_units, Ceilings *out, hipStream_t st) {
     *out = Ceilings{};
-    bytes = bytes / 4096 * 4096;
+    bytes = bytes / 65536 * 65536; // whole 16 KiB pieces for every wave of a copy workgroup
     if (bytes < (1u << 20) || compute_units <= 0) return hipErrorInvalidValue;
     char *a = nullptr, *b = nullptr;
     long long *clk = nullptr;
@@ -118,7 +116,7 @@ hipError_t measure_ceilings(uint64_t bytes, int compute_units, Ceilings *out, hi
     if (e == hipSuccess) out->memcpy_d2d_GBps = 2.0f * (float)bytes / us / 1e3f;
     timed([&] {
         flip ^= 1;
-        hipLaunchKernelGGL(probe_copy_k, dim3(blocks), dim3(256), 0, st, (const f32x4 *)(flip ? a : b), (f32x4 *)(flip ? b : a), n16);
+        hipLaunchKernelGGL(probe_copy_k, dim3((unsigned)(n16 / 4096)), dim3(256), 0, st, (const f32x4 *)(flip ? a : b), (f32x4 *)(flip ? b : a), n16);
         return hipGetLastError();
     }, 10, &us);
     if (e == hipSuccess) out->copy_kernel_GBps = 2.0f * (float)bytes / us / 1e3f;
