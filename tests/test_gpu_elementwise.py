@@ -245,7 +245,9 @@ def test_generated_unary_bf16(hip, oracle, op):
     c = Chain(*BIG, out_dtype=DType.BF16)
     getattr(c.load(c.input(DType.BF16)), op)()
     got, want = oracle.bf16_to_f32(run_chain(dev, pool, c, [x])), oracle.bf16_to_f32(oracle.ew_chain(c, [x]))
-    ok = np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + 1e-6   # one truncating store apart at most
+    # one truncating store apart at most; the absolute term covers the tails, where the reference's own expression
+    # rounds 1 + tanh to 0 (gelu'(-5.06) = -1.03e-6 comes out as 0 there, the kernel returns the value itself)
+    ok = np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + (2e-6 if op == "gelu_grad" else 1e-6)
     assert np.all(ok | (np.isnan(want) & (np.isnan(got) | np.isfinite(got))))
 
 

@@ -100,18 +100,22 @@ std::string ew_jit_source(const Elementwise &p, int V, int U) {
     const bool ireg = p.reg_class == DT_I32;
     const char *R = ireg ? "int" : "float";
     const int64_t n = p.rows * p.cols, nvec = n / V;
+    // A result stored in 16 bits keeps 8 or 11 significant bits: the sigmoid family then runs on the hardware's
+    // exp2 and reciprocal approximations (1 ulp of f32 each) instead of the library routines.
+    const bool fast16 = esize(p.out_dtype) == 2;
     Gen g;
     g.s = kPrelude;
     g.f("\ntypedef unsigned int u32x4 __attribute__((ext_vector_type(4)));\ntypedef unsigned int u32x2 __attribute__((ext_vector_type(2)));\n");
     g.f("extern \"C\" __global__ __launch_bounds__(256) void zk_ew(const char *__restrict__ in0, const char *__restrict__ in1,\n"
         "        const char *__restrict__ in2, const char *__restrict__ in3, char *__restrict__ out) {\n");
-    g.f("    const long NVEC = %lldL, T = (long)gridDim.x * 256L;\n", (long long)nvec);
+    g.f("    const long NVEC = %lldL;\n", (long long)nvec);
     for (int c = 0; c < 8; c++) {
         uint32_t bits;
         memcpy(&bits, &p.consts[c], 4);
         g.f("    const %s c%d = (%s)__uint_as_float(0x%08xu);\n", R, c, R, bits);
     }
-    g.f("    long v = (long)blockIdx.x * 256L + threadIdx.x;\n");
+    // every wave owns U consecutive pieces of 64 vectors: its requests cover one contiguous stretch of every operand
+    g.f("    const long v = ((long)blockIdx.x * 4L + (threadIdx.x >> 6)) * %dL + (threadIdx.x & 63);\n", 64 * U);
 
     // which inputs does the program read?
     bool used[4] = {false, false, false, false};
@@ -126,13 +130,13 @@ std::string ew_jit_source(const Elementwise &p, int V, int U) {
             if (!used[k] || p.in_bcast[k] != 0) continue;
             char name[32], off[64], ptr[16];
             snprintf(name, sizeof name, "r%d_%d_", u, k);
-            snprintf(off, sizeof off, "(v + %d * T) * %d", u, V * esize(p.in_dtype[k]));
+            snprintf(off, sizeof off, "(v + %d) * %d", u * 64, V * esize(p.in_dtype[k]));
             snprintf(ptr, sizeof ptr, "in%d", k);
             emit_load(g, name, ptr, off, V * esize(p.in_dtype[k]), true);
         }
     };
     auto body = [&](int u) {
-        g.f("        {\n        const long i0 = (v + %d * T) * %d;\n", u, V);
+        g.f("        {\n        const long i0 = (v + %d) * %d;\n", u * 64, V);
         if (p.need_rowcol) {
             if (n < (1ll << 31)) g.f("        const unsigned int row = (unsigned int)i0 / %uu, col = (unsigned int)i0 - row * %uu;\n", (unsigned)p.cols, (unsigned)p.cols);
             else g.f("        const long row = i0 / %lldL, col = i0 - row * %lldL;\n", (long long)p.cols, (long long)p.cols);
@@ -179,7 +183,8 @@ std::string ew_jit_source(const Elementwise &p, int V, int U) {
             for (int e = 0; e < V; e++) {
                 const std::string A = unary ? std::string("(") + R + ")0" : operand(sa, e);
                 const std::string B = three ? operand(sb, e) : std::string("(") + R + ")0";
-                g.f("        a%d = zkew::%s(%d, a%d, %s, %s);\n", e, ireg ? "op_i" : "op_f", op, e, A.c_str(), B.c_str());
+                const bool quick = !ireg && fast16 && (op == 39 || op == 40 || op == 41 || op == 44);
+                g.f("        a%d = zkew::%s(%d, a%d, %s, %s);\n", e, ireg ? "op_i" : quick ? "op_f_quick" : "op_f", op, e, A.c_str(), B.c_str());
             }
         }
         // store
@@ -201,12 +206,16 @@ std::string ew_jit_source(const Elementwise &p, int V, int U) {
                 g.f("        __builtin_nontemporal_store(u32x4{o%d, o%d, o%d, o%d}, (u32x4 *)(out + i0 * %d + %d));\n", 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3, oes, 16 * q);
         g.f("        }\n");
     };
-    g.f("    for (; v + %d * T < NVEC; v += %d * T) {\n", U - 1, U);
+    g.f("    if (v + %d < NVEC) {\n", (U - 1) * 64); // all requests of the thread in flight before the first use
     for (int u = 0; u < U; u++) loads(u);
     for (int u = 0; u < U; u++) body(u);
-    g.f("    }\n    for (; v < NVEC; v += T) {\n");
-    loads(0);
-    body(0);
+    g.f("    } else {\n");
+    for (int u = 0; u < U; u++) {
+        g.f("    if (v + %d < NVEC) {\n", u * 64);
+        loads(u);
+        body(u);
+        g.f("    }\n");
+    }
     g.f("    }\n}\n");
     return g.s;
 }
@@ -219,7 +228,7 @@ EwJit *ew_jit_compile(const Elementwise &p, std::string &err) {
     }
     int n_full = 0;
     for (int k = 0; k < p.n_in; k++) n_full += p.in_bcast[k] == 0;
-    const int U = n_full <= 2 ? 4 : 2;
+    const int U = n_full <= 1 ? 8 : n_full == 2 ? 4 : 2;
     const std::string src = ew_jit_source(p, V, U);
     // same code generation switches as the ahead-of-time kernels: gfx950, packed-FP32 instructions off
     // -ffp-contract=on: a*b+c fuses only inside one source expression, as in the interpreting kernel's build,
@@ -259,9 +268,8 @@ bool ew_jit_can_launch(const EwJit *j, const Elementwise &p) {
 }
 
 hipError_t ew_jit_launch(const EwJit *j, const Elementwise &p, hipStream_t st) {
-    int64_t blocks = (j->nvec + 256 * j->U - 1) / (256 * j->U);
-    if (blocks < 1) blocks = 1;
-    if (blocks > 256 * 16) blocks = 256 * 16;
+    const int64_t blocks = (j->nvec + 256 * j->U - 1) / (256 * j->U); // one pass: a thread's U vectors are all it does
+    if (blocks < 1 || blocks >= (1ll << 31)) return hipErrorInvalidValue;
     const void *in[4] = {p.in[0], p.in[1], p.in[2], p.in[3]};
     void *out = p.out;
     void *args[5] = {&in[0], &in[1], &in[2], &in[3], &out};

@@ -44,6 +44,28 @@ __device__ __forceinline__ float ref_gelu_grad(float x) {
     return 0.5f * (1.0f + t) + (0.5f * x) * ((1.0f - t * t) * (k * (1.0f + 0.134145f * x2)));
 }
 
+// The sigmoid family on v_exp_f32 / v_rcp_f32 (about 1 ulp of f32 each), for results that are stored in 16 bits:
+// 0.5 (1 + tanh(u)) = sigmoid(2u) = 1 / (1 + 2^(-2u log2 e)), so gelu(x) = x * sigmoid(2u) and
+// gelu'(x) = s + x * 2 s (1 - s) * k (1 + 3 * 0.044715 x^2) with s = sigmoid(2u). All of them saturate where e^{2u}
+// overflows, like ref_tanh.
+__device__ __forceinline__ float quick_sigmoid(float z) { // 1 / (1 + e^-z)
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * -1.44269504088896340736f));
+}
+__device__ __forceinline__ float op_f_quick(int op, float x, float a, float b) {
+    (void)a;
+    (void)b;
+    const float k = 0.79788456080286535588f;
+    switch (op) {
+    case 39: return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * 2.88539008177792681472f) + 1.0f);
+    case 40: return x * quick_sigmoid((x + ((x * x) * x) * 0.044715f) * (2.0f * k));
+    case 41: return quick_sigmoid(x);
+    default: { // 44
+        const float x2 = x * x, s = quick_sigmoid((x + (x2 * x) * 0.044715f) * (2.0f * k));
+        return s + (x * s) * ((2.0f - 2.0f * s) * (k * (1.0f + 0.134145f * x2)));
+    }
+    }
+}
+
 __device__ __forceinline__ float op_f(int op, float x, float a, float b) {
     switch (op) {
     case 0: return a;                                  // LOAD

@@ -53,6 +53,15 @@ template <> struct Elem<1> {
         v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
         v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
     }
+    static __device__ __forceinline__ void ld8(const uint16_t *p, int64_t i, float (&v)[8]) {
+        uint4 t = *(const uint4 *)(p + i);
+        const unsigned w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            v[2 * k] = __uint_as_float(w[k] << 16);
+            v[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
+        }
+    }
     static __device__ __forceinline__ void st(uint16_t *p, int64_t i, float v) { p[i] = f32_to_bf16_trunc(v); }
 };
 template <> struct Elem<2> {
@@ -62,6 +71,15 @@ template <> struct Elem<2> {
         uint2 t = *(const uint2 *)(p + i);
         v[0] = f16_to_f32((uint16_t)t.x); v[1] = f16_to_f32((uint16_t)(t.x >> 16));
         v[2] = f16_to_f32((uint16_t)t.y); v[3] = f16_to_f32((uint16_t)(t.y >> 16));
+    }
+    static __device__ __forceinline__ void ld8(const uint16_t *p, int64_t i, float (&v)[8]) {
+        uint4 t = *(const uint4 *)(p + i);
+        const unsigned w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            v[2 * k] = f16_to_f32((uint16_t)w[k]);
+            v[2 * k + 1] = f16_to_f32((uint16_t)(w[k] >> 16));
+        }
     }
     static __device__ __forceinline__ void st(uint16_t *p, int64_t i, float v) { p[i] = f32_to_f16_trunc(v); }
 };
@@ -162,17 +180,16 @@ __global__ __launch_bounds__(256) void reduce_partials_k(const typename Elem<DT>
     if (lane == 0) store_result<DT>(out, row, acc, epi);
 }
 
-// columns: a workgroup owns a strip of 256 columns (lane -> 4 adjacent columns when VEC,
-// else thread -> 1 column of a 64-wide strip per wave... kept simple: VEC strips are 256
-// wide, scalar strips 64 wide) and a chunk of rows split over its 4 waves.
-template <int DT, int OP, bool VEC>
+// columns: a workgroup owns a strip of 64 * W columns (lane -> W adjacent columns: 16 bytes per lane and row where
+// width and alignment allow, W = 4 for 32-bit and 8 for 16-bit elements; W = 1 otherwise) and a chunk of rows split
+// over its 4 waves.
+template <int DT, int OP, int W>
 __global__ __launch_bounds__(256) void reduce_cols_k(const typename Elem<DT>::S *__restrict__ x,
                                                      typename Elem<DT>::S *__restrict__ out,
                                                      typename Elem<DT>::A *__restrict__ partial, int64_t rows,
                                                      int64_t cols, int chunks, int64_t chunk_len, const Epilogue epi) {
     typedef typename Elem<DT>::A A;
     typedef Fold<OP, A> F;
-    constexpr int W = VEC ? 4 : 1;
     __shared__ A lds[4][64 * W];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t c = ((int64_t)blockIdx.x * 64 + lane) * W;
@@ -184,7 +201,12 @@ __global__ __launch_bounds__(256) void reduce_cols_k(const typename Elem<DT>::S 
     if (c < cols) {
 #pragma unroll 8
         for (int64_t r = r0 + wave; r < r1; r += 4) { // unrolled: 8 independent row loads in flight per thread
-            if (VEC) {
+            if constexpr (W == 8) {
+                A v[8];
+                Elem<DT>::ld8(x, r * cols + c, v);
+#pragma unroll
+                for (int k = 0; k < W; k++) acc[k] = F::f(acc[k], v[k]);
+            } else if constexpr (W == 4) {
                 A v[4];
                 Elem<DT>::ld4(x, r * cols + c, v);
 #pragma unroll
@@ -242,11 +264,14 @@ RowPlan plan_rows(int64_t rows, int64_t cols) {
     return {segs, seg_len};
 }
 struct ColPlan { int chunks; int64_t chunk_len; };
-ColPlan plan_cols(int64_t rows, int64_t cols, bool vec) {
-    int64_t strips = (cols + (vec ? 255 : 63)) / (vec ? 256 : 64);
+ColPlan plan_cols(int64_t rows, int64_t cols, int width) { // width of a strip: 64, 256 or 512 columns
+    int64_t strips = (cols + width - 1) / width;
     int chunks = 1;
-    if (strips < 1024 && rows >= 256) {
-        int64_t want = (1024 + strips - 1) / strips;
+    // two workgroups per compute unit (one for the widest strips) measured best at 8192 x 4096: more, shorter chunks
+    // pay their start-up and the second stage's longer fold, fewer leave units idle
+    const int64_t target = width >= 512 ? 256 : 512;
+    if (strips < target && rows >= 256) {
+        int64_t want = (target + strips - 1) / strips;
         chunks = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, rows / 64), 4096));
     }
     int64_t chunk_len = (rows + chunks - 1) / chunks;
@@ -273,13 +298,17 @@ template <int DT, int OP> hipError_t launch(const Reduce &p, hipStream_t st) {
         if (pl.segs > 1)
             hipLaunchKernelGGL((reduce_partials_k<DT, OP>), dim3((unsigned)((p.rows + 3) / 4)), block, 0, st, ws, out, p.rows, pl.segs, epi);
     } else {
-        bool vec = p.cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
-        ColPlan pl = plan_cols(p.rows, p.cols, vec);
+        const bool al16 = reinterpret_cast<uintptr_t>(x) % 16 == 0;
+        const int W = (esz == 2 && al16 && p.cols % 8 == 0) ? 8 : (al16 && p.cols % 4 == 0) ? 4 : 1;
+        ColPlan pl = plan_cols(p.rows, p.cols, 64 * W);
         if (pl.chunks > 1 && (uint64_t)pl.chunks * p.cols * sizeof(A) > p.workspace_bytes) return hipErrorInvalidValue;
-        int64_t strips = (p.cols + (vec ? 255 : 63)) / (vec ? 256 : 64);
+        int64_t strips = (p.cols + 64 * W - 1) / (64 * W);
         dim3 grid((unsigned)strips, (unsigned)pl.chunks), block(256);
-        if (vec) hipLaunchKernelGGL((reduce_cols_k<DT, OP, true>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len, epi);
-        else hipLaunchKernelGGL((reduce_cols_k<DT, OP, false>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len, epi);
+        if constexpr (sizeof(S) == 2) {
+            if (W == 8) hipLaunchKernelGGL((reduce_cols_k<DT, OP, 8>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len, epi);
+        }
+        if (W == 4) hipLaunchKernelGGL((reduce_cols_k<DT, OP, 4>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len, epi);
+        else if (W == 1) hipLaunchKernelGGL((reduce_cols_k<DT, OP, 1>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.chunks, pl.chunk_len, epi);
         if (pl.chunks > 1)
             hipLaunchKernelGGL((reduce_col_partials_k<DT, OP>), dim3((unsigned)((p.cols + 63) / 64)), block, 0, st, ws, out, p.cols, pl.chunks, epi);
     }
@@ -458,9 +487,8 @@ uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int axis0) {
         RowPlan pl = plan_rows(rows, cols);
         return pl.segs > 1 ? (uint64_t)rows * pl.segs * 4 : 0;
     }
-    // the vectorised plan never needs more chunks than the scalar one for the same shape
-    ColPlan a = plan_cols(rows, cols, true), b = plan_cols(rows, cols, false);
-    int chunks = std::max(a.chunks, b.chunks);
+    // whichever strip width the launch picks (alignment and dtype decide), its partials fit
+    const int chunks = std::max(plan_cols(rows, cols, 64).chunks, std::max(plan_cols(rows, cols, 256).chunks, plan_cols(rows, cols, 512).chunks));
     return chunks > 1 ? (uint64_t)chunks * cols * 4 : 0;
 }
 
