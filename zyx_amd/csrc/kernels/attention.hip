@@ -34,7 +34,9 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int QB = 128, KB = 64, DH = 64;
 constexpr int TILE = KB * DH * 2;   // one K or V tile: 8 KiB
 constexpr int STAGE = 2 * TILE;     // K tile then V tile
+constexpr int NSTAGE = 2;           // tiles kt+1 and kt+2 are on their way while tile kt is multiplied
 constexpr float kLog2e = 1.44269504088896340736f, kLn2 = 0.69314718055994530942f;
+constexpr float kSlack = 8.0f;
 
 // K tile: [key][16-byte chunk ^ ((key >> 1) & 7)], 128-byte rows: ds_read_b128 of 16 consecutive keys
 // at one logical chunk touches 16 different slots modulo 256 bytes.
@@ -47,18 +49,33 @@ __device__ __forceinline__ int v_slot(int key, int chunk) {
 
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
+// 64 lanes x 16 bytes from global memory straight into LDS at `lds` (wave-uniform byte address) + 16 * lane.
+// Written as an instruction, not through the compiler's builtin: for the builtin the compiler waits for every such
+// load in flight (vmcnt(0)) before the next LDS read that may touch the same array, which stops a wave for a full
+// global-memory latency in every tile although the data it waits for belongs to a later tile. Here completion is
+// tracked by hand: callers wait with s_waitcnt vmcnt and a workgroup barrier before anybody reads what was loaded.
+// The compiler's own vmcnt bookkeeping stays safe: these loads only ever make the counter larger than it assumes.
+__device__ __forceinline__ void load16_to_lds(const void *g, ZK_LDS void *lds) {
+    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(base), "v"(g) : "memory");
+}
+
 // CAUSAL: query t sees keys 0..t. A workgroup then stops at the key tile that holds its last query, a wave leaves out
 // tiles that lie wholly after its queries, and the tiles the diagonal crosses get -inf where key > query.
-template <bool LSE, bool CAUSAL>
+// QW: 32-query blocks per wave (the workgroup takes 128 * QW queries). Every K and V fragment a wave reads from LDS
+// serves QW matrix instructions: at QW = 1 the LDS port, which all four SIMDs share, carries 16 KiB per 32 x 64 score
+// block and is the busiest unit of the kernel; QW = 2 halves that.
+template <bool LSE, bool CAUSAL, int QW>
 __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__restrict__ qkv, uint16_t *__restrict__ y,
                                                           float *__restrict__ lse, int T, int H, float c, float out_scale) {
-    __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[2 * STAGE];
+    constexpr int WQ = 32 * QW, QBW = QB * QW; // queries per wave and per workgroup
+    __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[NSTAGE * STAGE];
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
 
     // Workgroups whose ids are congruent mod 8 share an XCD (and its L2): give every XCD whole heads, so
     // the K and V of a head are fetched into one L2 only.
-    const int QT = T / QB, NB = CAUSAL ? (QT + 1) / 2 : QT, BH = (int)gridDim.x / NB; // NB blocks of the grid per head
+    const int QT = T / QBW, NB = CAUSAL ? (QT + 1) / 2 : QT, BH = (int)gridDim.x / NB; // NB blocks of the grid per head
     int bh, qt;
     if (BH % 8 == 0) {
         const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
@@ -69,7 +86,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
         qt = blockIdx.x % NB;
     }
     // Causal work grows with qt: a workgroup takes the query blocks qt and QT-1-qt one after the other, so every
-    // workgroup streams the same number of key tiles (2 QT + 2) whatever CU it lands on.
+    // workgroup streams the same number of key tiles whatever CU it lands on.
     const int qt_first = qt;
 #pragma nounroll
     for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
@@ -80,11 +97,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
     const int bb = bh / H, h = bh % H;
     const int64_t ld = 3 * (int64_t)H * DH;
     const uint16_t *qp = qkv + (int64_t)bb * T * ld + h * DH, *kp = qp + H * DH, *vp = kp + H * DH;
-    const int tq = qt * QB + wave * 32 + (lane & 31);
+    const int q0w = qt * QBW + wave * WQ; // first query of this wave
+    const int tq0 = q0w + (lane & 31);    // this lane's query in block 0; block b: + 32 b
 
-    bf16x8 qf[4]; // B operand of S^T: lane -> query lane % 32, dh = ks*16 + (lane / 32)*8 .. +7
+    bf16x8 qf[QW][4]; // B operand of S^T: lane -> query lane % 32, dh = ks*16 + (lane / 32)*8 .. +7
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) qf[ks] = *(const bf16x8 *)(qp + (int64_t)tq * ld + ks * 16 + hh * 8);
+    for (int b = 0; b < QW; b++)
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) qf[b][ks] = *(const bf16x8 *)(qp + (int64_t)(tq0 + 32 * b) * ld + ks * 16 + hh * 8);
 
     // staging: direct global -> LDS loads (a wave-load lays 64 x 16 bytes down contiguously: 8 tile rows). The
     // swizzle is applied on the source side: lane l fetches the chunk that belongs at row l/8, physical slot l%8.
@@ -103,10 +123,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             const int rows = (i * 32 + wave * 8) * 128;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)((const uint8_t *)kp + base + gk[i]),
-                                             (ZK_LDS void *)(smem + stage + rows), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)((const uint8_t *)vp + base + gv[i]),
-                                             (ZK_LDS void *)(smem + stage + TILE + rows), 16, 0, 0);
+            load16_to_lds((const uint8_t *)kp + base + gk[i], (ZK_LDS void *)(smem + stage + rows));
+            load16_to_lds((const uint8_t *)vp + base + gv[i], (ZK_LDS void *)(smem + stage + TILE + rows));
         }
     };
 
@@ -121,72 +139,101 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
             vf[db] = TILE + (4 * (g16 >> 1) + kr) * 128 + ((db ^ ((kr >> 1) & 1)) << 6) + ((g16 & 1) * 16 + (r & 3) * 4) * 2;
     }
 
-    f32x16 o[2];
+    f32x16 o[QW][2];
+    float m[QW], l[QW];
 #pragma unroll
-    for (int db = 0; db < 2; db++)
+    for (int b = 0; b < QW; b++) {
+        m[b] = -INFINITY;
+        l[b] = 0.0f;
 #pragma unroll
-        for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
-    float m = -INFINITY, l = 0.0f;
+        for (int db = 0; db < 2; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[b][db][r] = 0.0f;
+    }
 
-    const int NT = CAUSAL ? 2 * qt + 2 : T / KB;
-    const int q0w = qt * QB + wave * 32; // first query of this wave
+    const int NT = CAUSAL ? (qt + 1) * (QBW / KB) : T / KB;
+    // A stage_tile is 4 loads per wave; they complete in order, so "at most 4 outstanding" means every tile but the
+    // newest has landed. Tiles kt+1 .. kt+NSTAGE-1 are in flight or landed while tile kt is multiplied.
     stage_tile(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): this wave's part of tile 0 has landed in LDS
+    if (NSTAGE > 2 && NT > 1) {
+        stage_tile(1, STAGE);
+        __builtin_amdgcn_s_waitcnt(0x0f74); // vmcnt(4): this wave's part of tile 0 has landed in LDS
+    } else {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+    }
     __syncthreads();
-    int stage = 0;
+    int stage = 0, fill = (NSTAGE - 1) * STAGE; // stage of tile kt; the stage last read before the previous barrier
     for (int kt = 0; kt < NT; kt++) {
-        if (kt + 1 < NT) stage_tile(kt + 1, stage ^ STAGE); // the other stage was last read before the previous barrier
+        if (kt + NSTAGE - 1 < NT) stage_tile(kt + NSTAGE - 1, fill);
 
-        if (!CAUSAL || kt * KB <= q0w + 31) {
-        f32x16 s[2];
+        if (!CAUSAL || kt * KB <= q0w + WQ - 1) {
+        f32x16 s[QW][2];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) s[kb][r] = 0.0f;
+            for (int b = 0; b < QW; b++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[b][kb][r] = 0.0f;
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
                 const bf16x8 a = *(const ZK_LDS bf16x8 *)(smem + stage + kb * 32 * 128 + kf + (((ks * 2 + hh) ^ key7) << 4));
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s[kb], 0, 0, 0);
+#pragma unroll
+                for (int b = 0; b < QW; b++) s[b][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[b][ks], s[b][kb], 0, 0, 0);
             }
         }
 
-        if (CAUSAL && kt * KB + KB - 1 > q0w) { // register r of block kb is key kb*32 + 8*(r/4) + 4*hh + r%4 of the tile
+        float m_new[QW];
+        bool moved = false;
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+        for (int b = 0; b < QW; b++) {
+            if (CAUSAL && kt * KB + KB - 1 > q0w + 32 * b) { // register r of block kb is key kb*32 + 8*(r/4) + 4*hh + r%4 of the tile
 #pragma unroll
-                for (int r = 0; r < 16; r++)
-                    if (kt * KB + kb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3) > tq) s[kb][r] = -INFINITY;
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        if (kt * KB + kb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3) > tq0 + 32 * b) s[b][kb][r] = -INFINITY;
+            }
+            float bm = s[b][0][0];
+#pragma unroll
+            for (int r = 1; r < 16; r++) bm = fmaxf(bm, s[b][0][r]);
+#pragma unroll
+            for (int r = 0; r < 16; r++) bm = fmaxf(bm, s[b][1][r]);
+            bm = fmaxf(bm, xor32(bm));
+            // The reference point m of a query's exponentials follows its running maximum only in steps of more than
+            // kSlack (in log2 units): exponentials may then reach 2^kSlack instead of 1, which f32 sums and bf16
+            // products carry at the same relative precision, and the accumulators are rescaled when a query makes such
+            // a step (the first tile it sees, then rarely) instead of whenever any of the wave's maxima moves (nearly
+            // every tile). A block of a causal tile that lies wholly after its queries has bm = -inf and changes nothing.
+            m_new[b] = bm * c > m[b] + kSlack ? bm * c : m[b];
+            moved |= m_new[b] != m[b];
         }
-        float bm = s[0][0];
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
 #pragma unroll
-        for (int r = 1; r < 16; r++) bm = fmaxf(bm, s[0][r]);
+            for (int b = 0; b < QW; b++) {
+                const float alpha = m[b] == m_new[b] ? 1.0f : __builtin_amdgcn_exp2f(m[b] - m_new[b]);
 #pragma unroll
-        for (int r = 0; r < 16; r++) bm = fmaxf(bm, s[1][r]);
-        bm = fmaxf(bm, xor32(bm));
-        const float m_new = fmaxf(m, bm * c);
-        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
-        m = m_new;
-        // the accumulator needs rescaling only when some query's running maximum moved: rare after the first tiles
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+                for (int db = 0; db < 2; db++)
 #pragma unroll
-            for (int db = 0; db < 2; db++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+                    for (int r = 0; r < 16; r++) o[b][db][r] *= alpha;
+                l[b] *= alpha;
+                m[b] = m_new[b];
+            }
         }
-        float ps = 0.0f;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) { // exponentiate one 32-key block, feed it to the matrix pipe, then the next
-            bf16x8 pf[2];
+            bf16x8 pf[QW][2];
 #pragma unroll
-            for (int s2 = 0; s2 < 2; s2++) {
-                f32x8 p;
+            for (int b = 0; b < QW; b++)
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][8 * s2 + e], c, -m_new));
-                    ps += p[e];
+                for (int s2 = 0; s2 < 2; s2++) {
+                    f32x8 p;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[b][kb][8 * s2 + e], c, -m[b]));
+                        l[b] += p[e];
+                    }
+                    pf[b][s2] = __builtin_convertvector(p, bf16x8);
                 }
-                pf[s2] = __builtin_convertvector(p, bf16x8);
-            }
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++)
 #pragma unroll
@@ -195,30 +242,36 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
                     const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(smem + off));
                     const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ZK_LDS bf16x4 *)(smem + off + 8 * 128));
                     const bf16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[s2], o[db], 0, 0, 0);
+#pragma unroll
+                    for (int b = 0; b < QW; b++) o[b][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[b][s2], o[b][db], 0, 0, 0);
                 }
         }
-        l = __builtin_fmaf(l, alpha, ps);
         }
 
-        __builtin_amdgcn_s_waitcnt(0x0f70); // this wave's loads of tile kt+1 have landed
+        if (NSTAGE > 2 && kt + 2 < NT) __builtin_amdgcn_s_waitcnt(0x0f74); // this wave's loads of tile kt+1 have landed, kt+2 may be in flight
+        else __builtin_amdgcn_s_waitcnt(0x0f70);
         __syncthreads();
-        stage ^= STAGE;
+        fill = stage;
+        stage = stage + STAGE == NSTAGE * STAGE ? 0 : stage + STAGE;
     }
 
-    l += xor32(l);
-    const float inv = out_scale / l;
-    uint16_t *yp = y + ((int64_t)bb * T + tq) * ((int64_t)H * DH) + h * DH;
 #pragma unroll
-    for (int db = 0; db < 2; db++)
+    for (int b = 0; b < QW; b++) {
+        const int tq = tq0 + 32 * b;
+        const float lt = l[b] + xor32(l[b]);
+        const float inv = out_scale / lt;
+        uint16_t *yp = y + ((int64_t)bb * T + tq) * ((int64_t)H * DH) + h * DH;
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            uint32_t w0 = (uint32_t)f32_to_bf16_trunc(o[db][4 * g + 0] * inv) | ((uint32_t)f32_to_bf16_trunc(o[db][4 * g + 1] * inv) << 16);
-            uint32_t w1 = (uint32_t)f32_to_bf16_trunc(o[db][4 * g + 2] * inv) | ((uint32_t)f32_to_bf16_trunc(o[db][4 * g + 3] * inv) << 16);
-            u32x2 w = {w0, w1};
-            *(u32x2 *)(yp + db * 32 + 8 * g + 4 * hh) = w;
-        }
-    if (LSE && hh == 0) lse[(int64_t)bh * T + tq] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+        for (int db = 0; db < 2; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                uint32_t w0 = (uint32_t)f32_to_bf16_trunc(o[b][db][4 * g + 0] * inv) | ((uint32_t)f32_to_bf16_trunc(o[b][db][4 * g + 1] * inv) << 16);
+                uint32_t w1 = (uint32_t)f32_to_bf16_trunc(o[b][db][4 * g + 2] * inv) | ((uint32_t)f32_to_bf16_trunc(o[b][db][4 * g + 3] * inv) << 16);
+                u32x2 w = {w0, w1};
+                *(u32x2 *)(yp + db * 32 + 8 * g + 4 * hh) = w;
+            }
+        if (LSE && hh == 0) lse[(int64_t)bh * T + tq] = (m[b] + __builtin_amdgcn_logf(lt)) * kLn2;
+    }
     }
 }
 
@@ -292,11 +345,19 @@ bool attention_fast_path(const Attention &p) {
 hipError_t attention_fwd(const Attention &p, hipStream_t st) {
     if (p.B <= 0 || p.T <= 0 || p.H <= 0 || p.dh <= 0) return hipSuccess;
     if (attention_fast_path(p)) {
-        const int qblocks = p.T / QB;
+        // 64 queries per wave where the sequence divides into such workgroups and they still fill the device twice
+        const bool wide = !p.causal && p.T % (2 * QB) == 0 && (int64_t)p.B * p.H * (p.T / (2 * QB)) >= 512;
+        const int qblocks = p.T / (wide ? 2 * QB : QB);
         dim3 grid((unsigned)(p.B * p.H * (p.causal ? (qblocks + 1) / 2 : qblocks))), block(256);
 #define ZK_ATTN(L, CA)                                                                                                \
-    hipLaunchKernelGGL((attn_fwd_bf16_k<L, CA>), grid, block, 0, st, (const uint16_t *)p.qkv, (uint16_t *)p.y, p.lse, p.T, p.H, \
-                       p.scale * kLog2e, 1.0f / p.keep)
+    do {                                                                                                              \
+        if (wide)                                                                                                     \
+            hipLaunchKernelGGL((attn_fwd_bf16_k<L, CA, 2>), grid, block, 0, st, (const uint16_t *)p.qkv, (uint16_t *)p.y, p.lse, p.T, \
+                               p.H, p.scale * kLog2e, 1.0f / p.keep);                                                 \
+        else                                                                                                          \
+            hipLaunchKernelGGL((attn_fwd_bf16_k<L, CA, 1>), grid, block, 0, st, (const uint16_t *)p.qkv, (uint16_t *)p.y, p.lse, p.T, \
+                               p.H, p.scale * kLog2e, 1.0f / p.keep);                                                 \
+    } while (0)
         if (p.lse) {
             if (p.causal) ZK_ATTN(true, true);
             else ZK_ATTN(true, false);
