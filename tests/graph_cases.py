@@ -239,3 +239,36 @@ def mlp_training_graph(g, leaf, batch=64, n_in=784, hidden=128, n_out=10, lr=0.0
     lr_c = g.const(lr, F32)
     new = [g.binary(p, g.binary(gr, lr_c, BOp.Mul), BOp.Sub) for p, gr in zip(params, grads)]
     return loss, new, params, (x, onehot)
+
+
+BLOCK_PARAMS = ("ln1_w", "ln1_b", "attn_w", "attn_b", "proj_w", "proj_b", "ln2_w", "ln2_b", "fc_w", "fc_b", "proj2_w", "proj2_b")
+
+
+def block_graph(g, leaf, b=2, t=16, d=32, n_head=4, dtype=F32, seed=7, params=None, x=None, dout=None):
+    """One pre-norm transformer block `x = x + attn(ln_1(x)); x = x + mlp(ln_2(x))` (zyx-examples/examples/nanogpt.rs:
+    68-98) from zyx-nn modules written as graph nodes: LayerNorm, CausalSelfAttention (c_attn Linear, the attention
+    core, c_proj Linear), MLP = Linear d -> 4d, gelu, Linear 4d -> d; rows are (batch, position) pairs. The loss is
+    sum(out * dout), so the gradients are those of the block for the upstream gradient dout.
+    Returns (out, loss, parameter leaves by name, x leaf, dout leaf)."""
+    r = np.random.default_rng(seed)
+    f = 4 * d
+    shapes = dict(ln1_w=(d,), ln1_b=(d,), attn_w=(3 * d, d), attn_b=(3 * d,), proj_w=(d, d), proj_b=(d,),
+                  ln2_w=(d,), ln2_b=(d,), fc_w=(f, d), fc_b=(f,), proj2_w=(d, f), proj2_b=(d,))
+    if params is None:
+        params = {n: (1.0 + 0.1 * r.standard_normal(s)) if n in ("ln1_w", "ln2_w") else 0.02 * r.standard_normal(s) if n.endswith("_w")
+                  else 0.01 * r.standard_normal(s) for n, s in shapes.items()}
+    P = {n: leaf(np.asarray(params[n]).reshape(shapes[n]), dtype) for n in BLOCK_PARAMS}
+    xl = leaf(r.standard_normal((b, t, d)) if x is None else x, dtype)
+    dl = leaf(r.standard_normal((b, t, d)) if dout is None else dout, dtype)
+
+    def linear(v, w, bias):  # zyx-nn/src/linear.rs:38-44
+        return g.binary_b(g.dot(v, g.t(P[w])), P[bias], BOp.Add)
+
+    n1 = g.layer_norm(xl, P["ln1_w"], P["ln1_b"])
+    att = g.self_attention(linear(n1, "attn_w", "attn_b"), n_head)
+    x2 = g.binary(linear(att, "proj_w", "proj_b"), xl, BOp.Add)
+    n2 = g.layer_norm(x2, P["ln2_w"], P["ln2_b"])
+    hid = g.gelu(linear(n2, "fc_w", "fc_b"))
+    out = g.binary(linear(hid, "proj2_w", "proj2_b"), x2, BOp.Add)
+    loss = g.sum_all(g.binary(out, dl, BOp.Mul))
+    return out, loss, P, xl, dl

@@ -210,3 +210,53 @@ def test_config5_block_full_size(hip, oracle):
     da = F(t["datt"]).reshape(B, T, d)
     assert np.all(np.abs(dv - da.sum(1)) <= 2.0 ** -6 * np.abs(da).sum(1) + 1e-6)
     blk.close()
+
+
+@pytest.mark.parametrize("dtype", [DType.BF16, DType.F32])
+def test_block_written_as_graph_nodes_gives_the_hand_written_launch_list(hip, oracle, dtype):
+    """The same block built from graph nodes (layer_norm, Linear, self_attention, gelu, skip connections), its
+    gradients taken by the reverse rules and everything lowered with matching on: 24 launches like the list in
+    zyx_amd/block.py, the same kernel kinds, and the results of that list. bf16: the two paths share every
+    hand-written kernel and differ in gelu / gelu' (generated from the expression here, one fused op there): both
+    store bf16, so values agree to a few bf16 steps of the tensors they go through; bit equality is asserted where
+    only shared kernels are involved (n1, qkv, att, x2, n2, h)."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from graph_cases import BLOCK_PARAMS, block_graph
+    from zyx_amd.graph import Alias, Tape, lower, storage_dtype
+    dev, pool = hip
+    B, T, d, H = 2, 128, 256, 4
+    blk, p, x, dout = make_block(hip, oracle, B, T, d, H, dtype, std=0.05)
+    blk.forward_backward()
+    tape, leaves = Tape(dev, pool, match=True), {}
+
+    def leaf(array, dt):
+        a = np.ascontiguousarray(array)
+        nid = tape.tensor(a, dt)
+        leaves[nid] = a
+        return nid
+
+    g = tape.graph
+    out, loss, P, xl, dl = block_graph(g, leaf, B, T, d, H, dtype, params=p, x=x.reshape(B, T, d), dout=dout.reshape(B, T, d))
+    grads = tape.gradient(loss, [P[n] for n in BLOCK_PARAMS] + [xl])
+    nodes = [out] + grads
+    sched = [k for k in lower(g, nodes, stored=list(leaves), match=True) if not isinstance(k, Alias)]
+    assert len(sched) == len(blk.forward_nodes) + len(blk.backward_nodes) == 24
+    tape.realize(nodes)
+    assert tape.matched == 24 - 2 if dtype == DType.BF16 else tape.matched >= 18  # all but gelu and gelu' (f32 at this size: short column sums are generated too)
+    F = lambda a: f64(oracle, np.asarray(a))
+    inter = {"n1": None, "qkv": None, "att": None, "x2": None, "n2": None, "h": None}
+    comps = [k for k, v in g.composites.items()]
+    by_name = {"n1": comps[0], "att": comps[1], "n2": comps[2]}
+    for name, nid in by_name.items():
+        assert np.array_equal(tape.numpy(nid).reshape(-1), blk.read(name).reshape(-1)), name
+    scale = lambda a: np.abs(F(a)).max()
+    got_out, want_out = tape.numpy(out).reshape(B * T, d), blk.read("out")
+    assert np.abs(F(got_out) - F(want_out)).max() <= 2.0 ** -6 * scale(want_out)
+    for n, gid in zip(list(BLOCK_PARAMS) + ["x"], grads):
+        want = blk.read("dx" if n == "x" else "d_" + n)
+        got = tape.numpy(gid).reshape(want.shape)
+        assert np.abs(F(got) - F(want)).max() <= 2.0 ** -5 * scale(want), n
+    del inter
+    tape.close()
+    blk.close()

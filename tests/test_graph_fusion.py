@@ -150,3 +150,54 @@ def test_folded_relu_is_the_only_thing_stored():
     stored = {k.out if not isinstance(k, LoweredKernel) else k.output for k in sched}
     assert pre not in stored and h in stored
     assert sched[3].relu_mask and sched[3].residual == h
+
+
+def test_transformer_block_lowers_to_the_module_level_launches():
+    """The block of zyx_amd/block.py written as graph nodes: with matching on, forward and backward come out as the
+    launches that file lists by hand (norms, products with their epilogues, attention, column sums, the two norm
+    backward passes with the skip gradient added in) plus generated elementwise kernels for gelu and gelu'."""
+    from graph_cases import BLOCK_PARAMS, block_graph
+    from zyx_amd.graph import AttentionBwdMatch, AttentionMatch, NormBwdMatch, NormRowsMatch
+    g, leaves, (out, loss, P, xl, dl) = _build(block_graph)
+    grads = g.gradient(loss, [P[n] for n in BLOCK_PARAMS] + [xl])
+    outs = [out] + grads
+    seen = []
+    got = run_lowered(g, leaves, outs, match=True, seen=seen)
+    want = graph_eval.evaluate(g.nodes, leaves, outs)
+    for o in outs:
+        np.testing.assert_allclose(got[o], want[o], rtol=2e-4, atol=2e-5)
+    from zyx_amd.graph import Alias
+    kinds = [type(k).__name__ for k in lower(g, outs, match=True) if not isinstance(k, Alias)]
+    count = {k: kinds.count(k) for k in set(kinds)}
+    assert len(kinds) == 24                 # 8 forward + 16 backward: the list zyx_amd/block.py writes by hand
+    assert count["NormRowsMatch"] == 2 and count["NormBwdMatch"] == 2 and count["AttentionMatch"] == 1 and count["AttentionBwdMatch"] == 1
+    assert count["Contraction"] == 12       # 4 Linear forward, 4 x (dW, dX) backward
+    assert count.get("RowColReduce", 0) + count["LoweredKernel"] == 4 + 2   # the bias gradients' column sums; gelu and gelu'
+    fwd = [k for k in seen if isinstance(k, Contraction) and k.epilogue == "bias"]
+    assert sum(k.residual is not None for k in fwd) == 2          # both skip connections ride on a Linear's epilogue
+    nb = [k for k in seen if isinstance(k, NormBwdMatch)]
+    assert all(k.add is not None and k.dw is not None and k.db is not None for k in nb)
+    assert [k.lse for k in seen if isinstance(k, AttentionMatch)] == [True]
+    # forward alone: no row log-sum-exps asked of the attention kernel
+    assert [k.lse for k in lower(g, [out], match=True) if isinstance(k, AttentionMatch)] == [False]
+    # ... and gelu, whose input nothing reads any more, folds into the product before it: 7 launches
+    assert len([k for k in lower(g, [out], match=True) if not isinstance(k, Alias)]) == 7
+
+
+def test_norm_composites_against_closed_forms():
+    rng = np.random.default_rng(4)
+    X, W, T = rng.standard_normal((5, 12)), rng.standard_normal(12), rng.standard_normal((5, 12))
+    g = Graph()
+    x, w, t = (g.leaf(a.shape, DType.F64) for a in (X, W, T))
+    y = g.rms_norm(x, w)
+    (gx, gw) = g.gradient(g.sum_all(g.binary(y, t, BOp.Mul)), [x, w])
+    got = graph_eval.evaluate(g.nodes, {x: X, w: W, t: T}, [y, gx, gw])
+    r = np.sqrt(1.0 / ((X * X).mean(1, keepdims=True) + 1e-6))
+    np.testing.assert_allclose(got[y], X * r * W, rtol=1e-12)
+    gg = T * W
+    np.testing.assert_allclose(got[gx], r * gg - r ** 3 * X * (gg * X).sum(1, keepdims=True) / 12, rtol=1e-10)
+    np.testing.assert_allclose(got[gw], (T * X * r).sum(0), rtol=1e-10)
+    seen = []
+    low = run_lowered(g, {x: X.astype(np.float32), w: W.astype(np.float32), t: T.astype(np.float32)}, [y, gx, gw], match=True, seen=seen)
+    assert seen == []  # f64 graphs stay on generated kernels
+    del low

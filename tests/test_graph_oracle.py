@@ -7,7 +7,7 @@ import pytest
 from graph_cases import CASES, mixed_graph, mlp_graph
 from oracle import graph_eval, ir_interp
 from zyx_amd import DType
-from zyx_amd.graph import Contraction, Conv2dMatch, CrossEntropyMatch, Graph, MaxPoolMatch, RowColReduce, SoftmaxRows, lower, match_reduce, match_softmax, match_contraction, storage_dtype, view_of
+from zyx_amd.graph import (Alias, AttentionBwdMatch, AttentionMatch, Contraction, Conv2dMatch, CrossEntropyMatch, Graph, NormBwdMatch, NormRowsMatch, MaxPoolMatch, RowColReduce, SoftmaxRows, lower, match_reduce, match_softmax, match_contraction, storage_dtype, view_of)
 from zyx_amd.ir import BOp, UOp
 
 _FLOAT = (DType.F32, DType.F64)
@@ -61,6 +61,9 @@ def run_lowered(g, leaves, outputs, match=False, seen=None):
     (trans_a) times [batch, k, n] or [batch, n, k] (trans_b), written as [batch, m, n]."""
     bufs = {i: a.reshape(-1).copy() for i, a in leaves.items()}
     for kern in lower(g, outputs, match=match):
+        if isinstance(kern, Alias):
+            bufs[kern.out] = bufs[kern.base]
+            continue
         if isinstance(kern, Contraction):
             A = bufs[kern.a].reshape((kern.batch, kern.k, kern.m) if kern.trans_a else (kern.batch, kern.m, kern.k))
             B = bufs[kern.b].reshape((kern.batch, kern.n, kern.k) if kern.trans_b else (kern.batch, kern.k, kern.n))
@@ -77,6 +80,65 @@ def run_lowered(g, leaves, outputs, match=False, seen=None):
                 res = bufs[kern.residual].astype(np.float64).reshape(acc.shape)
                 acc = acc * (res > 0) if kern.relu_mask else acc + res
             bufs[kern.out] = acc.astype(A.dtype).reshape(-1)
+            if seen is not None:
+                seen.append(kern)
+            continue
+        if isinstance(kern, NormRowsMatch):
+            x = bufs[kern.x].reshape(kern.rows, kern.cols).astype(np.float64)
+            if kern.rms:
+                y = x * np.sqrt(1.0 / ((x * x).mean(1, keepdims=True) + kern.eps))
+            else:
+                y = (x - x.mean(1, keepdims=True)) / np.sqrt(x.var(1, ddof=1, keepdims=True) + kern.eps)
+            if kern.w is not None:
+                y = y * bufs[kern.w].astype(np.float64).reshape(1, -1)
+            if kern.b is not None:
+                y = y + bufs[kern.b].astype(np.float64).reshape(1, -1)
+            bufs[kern.out] = y.astype(bufs[kern.x].dtype).reshape(-1)
+            if seen is not None:
+                seen.append(kern)
+            continue
+        if isinstance(kern, NormBwdMatch):
+            x = bufs[kern.x].reshape(kern.rows, kern.cols).astype(np.float64)
+            dy = bufs[kern.dy].reshape(kern.rows, kern.cols).astype(np.float64)
+            gg = dy * bufs[kern.w].astype(np.float64).reshape(1, -1) if kern.w is not None else dy
+            n = kern.cols
+            if kern.rms:
+                r = np.sqrt(1.0 / ((x * x).mean(1, keepdims=True) + kern.eps))
+                xh = x * r
+                dx = r * gg - r ** 3 * x * (gg * x).sum(1, keepdims=True) / n
+            else:
+                r = 1.0 / np.sqrt(x.var(1, ddof=1, keepdims=True) + kern.eps)
+                xh = (x - x.mean(1, keepdims=True)) * r
+                dx = r * (gg - gg.mean(1, keepdims=True) - xh * (gg * xh).sum(1, keepdims=True) / (n - 1))
+            if kern.add is not None:
+                dx = dx + bufs[kern.add].reshape(kern.rows, kern.cols).astype(np.float64)
+            st = bufs[kern.x].dtype
+            bufs[kern.dx] = dx.astype(st).reshape(-1)
+            if kern.dw is not None:
+                bufs[kern.dw] = (dy * xh).sum(0).astype(st)
+            if kern.db is not None:
+                bufs[kern.db] = dy.sum(0).astype(st)
+            if seen is not None:
+                seen.append(kern)
+            continue
+        if isinstance(kern, (AttentionMatch, AttentionBwdMatch)):
+            b_, t_, h_, dh_ = kern.dims
+            qkv = bufs[kern.qkv].reshape(b_, t_, 3, h_, dh_).astype(np.float64)
+            q, k, v = (qkv[:, :, i].transpose(0, 2, 1, 3) for i in range(3))
+            sc = np.einsum("bhtd,bhsd->bhts", q, k) * kern.scale
+            p = np.exp(sc - sc.max(-1, keepdims=True))
+            p /= p.sum(-1, keepdims=True)
+            if isinstance(kern, AttentionMatch):
+                y = np.einsum("bhts,bhsd->bhtd", p, v).transpose(0, 2, 1, 3).reshape(b_, t_, h_ * dh_)
+                bufs[kern.out] = y.astype(bufs[kern.qkv].dtype).reshape(-1)
+            else:
+                dy = bufs[kern.dy].reshape(b_, t_, h_, dh_).astype(np.float64).transpose(0, 2, 1, 3)
+                dv = np.einsum("bhts,bhtd->bhsd", p, dy)
+                dp = np.einsum("bhtd,bhsd->bhts", dy, v)
+                ds = p * (dp - (dp * p).sum(-1, keepdims=True)) * kern.scale
+                dq, dk = np.einsum("bhts,bhsd->bhtd", ds, k), np.einsum("bhts,bhtd->bhsd", ds, q)
+                out = np.stack([a.transpose(0, 2, 1, 3) for a in (dq, dk, dv)], 2).reshape(b_, t_, 3 * h_ * dh_)
+                bufs[kern.out] = out.astype(bufs[kern.qkv].dtype).reshape(-1)
             if seen is not None:
                 seen.append(kern)
             continue

@@ -71,6 +71,12 @@ class Graph:
         self.nodes: list[Node] = []
         self.convs: dict[int, dict] = {}  # result node of `conv` -> its operands and parameters
         self.pools: dict[int, dict] = {}  # result node of a 2-D `max_pool` -> its operand and parameters
+        # Module-level expressions the hand-written kernels compute whole (`layer_norm`, `rms_norm`, `self_attention`):
+        # result node -> dict(kind, inputs, params). The reverse pass differentiates such an expression as a unit (the
+        # same primitive rules, applied to its own nodes only) and notes the gradient nodes in `fused_bwd`, so that the
+        # lowering can hand forward and backward to one launch each.
+        self.composites: dict[int, dict] = {}
+        self.fused_bwd: dict[int, dict] = {}   # gradient node of a composite's input -> dict(kind, fwd, dy, inputs, grads, params)
 
     def _push(self, node: Node) -> int:
         self.nodes.append(node)
@@ -262,6 +268,59 @@ class Graph:
         n = _numel([xs[a] for a in axes])
         return self.binary(self.reduce(x, BOp.Add, axes), self.const(n, self[x].dtype), BOp.Div)
 
+    def var(self, x: int, axes, correction: int = 1, keepdim: bool = False) -> int:
+        """`ReduceOp::Var` (zyx/src/tensor/reduce_ops.rs:111-123): `d = x - mean_keepdim(x); sum(d * d) / (n - correction)`."""
+        xs = self[x].shape
+        axes = [self._axis(a, len(xs)) for a in axes] or list(range(len(xs)))
+        n = _numel([xs[a] for a in axes])
+        dt = self[x].dtype
+        mean = self.binary(self.reduce_keepdim(x, BOp.Add, axes), self.const(n, dt), BOp.Div)
+        d = self.binary_b(x, mean, BOp.Sub)
+        sq = self.binary(d, d, BOp.Mul)
+        red = self.reduce_keepdim(sq, BOp.Add, axes) if keepdim else self.reduce(sq, BOp.Add, axes)
+        return self.binary(red, self.const(n - correction, dt), BOp.Div)
+
+    def layer_norm(self, x: int, weight: int | None = None, bias: int | None = None, eps: float = 1e-5) -> int:
+        """`LayerNorm::forward` over the last axis (zyx-nn/src/layer_norm.rs:98-135): `(x - mean) / sqrt(var + eps)`
+        (`var_keepdim`, correction 1), then `* weight`, `+ bias`."""
+        dt, n = self[x].dtype, self[x].shape[-1]
+        mean = self.binary(self.reduce_keepdim(x, BOp.Add, [-1]), self.const(n, dt), BOp.Div)
+        variance = self.var(x, [-1], 1, keepdim=True)
+        out = self.binary_b(self.binary_b(x, mean, BOp.Sub),
+                            self.unary(self.binary(variance, self.const(eps, dt), BOp.Add), UOp.Sqrt), BOp.Div)
+        if weight is not None:
+            out = self.binary_b(out, weight, BOp.Mul)
+        if bias is not None:
+            out = self.binary_b(out, bias, BOp.Add)
+        self.composites[out] = dict(kind="layer_norm", inputs=(x, weight, bias), params=dict(eps=float(eps)))
+        return out
+
+    def rms_norm(self, x: int, scale: int, eps: float = 1e-6) -> int:
+        """`RMSNorm::forward` (zyx-nn/src/rms_norm.rs:26-32): `x * (mean_keepdim(x * x, [-1]) + eps).rsqrt() * scale`,
+        rsqrt being `reciprocal().sqrt()` (zyx/src/tensor/elementwise.rs:305-307)."""
+        dt, n = self[x].dtype, self[x].shape[-1]
+        ms = self.binary(self.reduce_keepdim(self.binary(x, x, BOp.Mul), BOp.Add, [-1]), self.const(n, dt), BOp.Div)
+        r = self.unary(self.unary(self.binary(ms, self.const(eps, dt), BOp.Add), UOp.Reciprocal), UOp.Sqrt)
+        out = self.binary_b(self.binary_b(x, r, BOp.Mul), scale, BOp.Mul)
+        self.composites[out] = dict(kind="rms_norm", inputs=(x, scale, None), params=dict(eps=float(eps)))
+        return out
+
+    def self_attention(self, qkv: int, n_head: int) -> int:
+        """The core of `CausalSelfAttention::forward` between c_attn and c_proj (zyx-nn/src/causal_self_attention.rs:
+        39-69; the reference applies no mask and, in evaluation, no dropout): qkv[B, T, 3C] is split along the last axis,
+        each part viewed as [B, H, T, C / H], `softmax(q . k^T * scale, [-1]) . v`, back to [B, T, C]."""
+        b, t, c3 = self[qkv].shape
+        c = c3 // 3
+        if c * 3 != c3 or c % n_head:
+            raise ValueError(f"qkv of shape {self[qkv].shape} does not split into 3 x {n_head} heads")
+        dh, dt = c // n_head, self[qkv].dtype
+        q, k, v = (self.permute(self.reshape(self.narrow(qkv, 2, i * c, c), (b, t, n_head, dh)), (0, 2, 1, 3)) for i in range(3))
+        scale = float(np.float32(1.0 / np.sqrt(float(dh))))
+        att = self.softmax(self.binary(self.dot(q, self.t(k)), self.const(scale, dt), BOp.Mul), [-1])
+        y = self.reshape(self.permute(self.dot(att, v), (0, 2, 1, 3)), (b, t, c))
+        self.composites[y] = dict(kind="attention", inputs=(qkv,), params=dict(n_head=int(n_head), scale=scale))
+        return y
+
     def cross_entropy(self, logits: int, target: int, reduction: str = "mean") -> int:
         """`Tensor::cross_entropy` (zyx/src/tensor/mod.rs:1639-1655) for a target of the logits' shape (one-hot or soft
         labels): `(-ln_softmax(logits, [classes]) * target).sum([classes])`, then the mean, the sum, or nothing;
@@ -435,11 +494,12 @@ class Graph:
         # node ids are topological (operands are created before their users): descending id = reverse topological
         return sorted((i for i, d in needs.items() if d), reverse=True)
 
-    def gradient(self, target: int, sources: Sequence[int]) -> list:
+    def gradient(self, target: int, sources: Sequence[int], seed: int | None = None, _inside: int | None = None) -> list:
         """d target / d source for every source, as new nodes (`Runtime::gradient`, autograd.rs:14-424). The seed is
-        1 in the target's dtype; a source the target does not depend on gets zeros of its shape and dtype."""
+        1 in the target's dtype (or the node `seed`, of the target's shape: the gradient arriving from above); a source
+        the target does not depend on gets zeros of its shape and dtype."""
         src_set = set(sources)
-        grads: dict[int, int] = {target: self.expand(self.const(1, self[target].dtype), self[target].shape)}
+        grads: dict[int, int] = {target: self.expand(self.const(1, self[target].dtype), self[target].shape) if seed is None else seed}
         order = self._grad_order(target, src_set)
         wanted = set(order) | src_set
 
@@ -451,6 +511,16 @@ class Graph:
             if cid not in grads:
                 continue
             grad, n = grads[cid], self[cid]
+            comp = self.composites.get(cid)
+            if comp is not None and cid != _inside:
+                # a module-level expression: the same rules, applied to its own nodes with the arriving gradient as seed
+                ins = [i for i in comp["inputs"] if i is not None]
+                gs = self.gradient(cid, ins, seed=grad, _inside=cid)
+                record = dict(kind=comp["kind"], fwd=cid, dy=grad, inputs=comp["inputs"], grads=dict(zip(ins, gs)), params=comp["params"])
+                for i, gi in zip(ins, gs):
+                    self.fused_bwd[gi] = record
+                    acc(i, gi)
+                continue
             if n.kind == "unary":
                 (x,) = n.src
                 u = n.op
@@ -488,8 +558,13 @@ class Graph:
                     acc(x, grad)
                     acc(y, self.unary(grad, UOp.Neg))
                 elif b == BOp.Mul:
-                    acc(x, self.binary(grad, y, BOp.Mul))
-                    acc(y, self.binary(grad, x, BOp.Mul))
+                    # 1 * v is v: the product with a gradient that is all ones (the seed seen through views) is not materialised
+                    def times(v):
+                        if _const_value(self, grad) == 1 and self[v].shape == self[grad].shape and self[v].dtype == n.dtype:
+                            return v
+                        return self.binary(grad, v, BOp.Mul)
+                    acc(x, times(y))
+                    acc(y, times(x))
                 elif b == BOp.Div:
                     acc(x, self.binary(grad, y, BOp.Div))
                     x_mul = self.binary(self.unary(grad, UOp.Neg), x, BOp.Mul)
@@ -1028,6 +1103,19 @@ def match_linear(graph: Graph, nid: int, users: dict, relu_mask: dict):
                 m.out, m.bias, m.mask_node = nid, bias, mask_node
                 m.epilogue = {None: "bias", "relu": "bias_relu", "gelu": "bias_gelu"}[act]
                 return m
+        if act is None:  # (product + bias) + a tensor of the result's shape: the skip connection around a Linear
+            for inner, res in (c.src, c.src[::-1]):
+                rb, ni = _plain(graph, res), graph[inner]
+                if rb is None or graph[rb].dtype != n.dtype or ni.kind != "binary" or ni.op != BOp.Add or not only_reader(inner, cur):
+                    continue
+                for core, other in (ni.src, ni.src[::-1]):
+                    bias = _row_vector(graph, other)
+                    if bias is None or graph[bias].dtype != n.dtype:
+                        continue
+                    m = product(core, inner)
+                    if m is not None and m.batch == 1 and _numel(graph[bias].shape) == m.n:
+                        m.out, m.bias, m.epilogue, m.residual = nid, bias, "bias", rb
+                        return m
         return None
     if act is not None:
         return None  # an activation straight on a product: the kernel has no such epilogue
@@ -1167,8 +1255,151 @@ def scan_cross_entropy(graph: Graph, nodes) -> dict:
     return by_node
 
 
+@dataclasses.dataclass
+class NormRowsMatch:
+    """`out = layer_norm(x, w, b)` or `rms_norm(x, scale)` over the last axis (ZHIP_K_NORM_ROWS)."""
+    x: int
+    w: int | None
+    b: int | None
+    out: int
+    rows: int
+    cols: int
+    rms: bool
+    eps: float
+    dtype: DType
+
+
+@dataclasses.dataclass
+class NormBwdMatch:
+    """The gradients of a norm with respect to x, weight and bias for the arriving gradient dy, optionally with the
+    gradient of a skip branch added to dx in the same pass (ZHIP_K_NORM_ROWS_BWD). `dx`, `dw`, `db`: the nodes that
+    receive the results (None: not asked for)."""
+    x: int
+    w: int | None
+    dy: int
+    add: int | None
+    dx: int
+    dw: int | None
+    db: int | None
+    rows: int
+    cols: int
+    rms: bool
+    eps: float
+    dtype: DType
+
+    @property
+    def out(self):
+        return self.dx
+
+
+@dataclasses.dataclass
+class AttentionMatch:
+    """`y = self_attention(qkv)` (ZHIP_K_ATTENTION); `lse`: the launch also leaves the row log-sum-exps the backward
+    kernel reads, in a buffer that belongs to `out` and is no graph node."""
+    qkv: int
+    out: int
+    dims: tuple      # B, T, H, dh
+    scale: float
+    lse: bool
+    dtype: DType
+
+
+@dataclasses.dataclass
+class AttentionBwdMatch:
+    """d qkv of `self_attention` for the arriving gradient dy (ZHIP_K_ATTENTION_BWD): reads qkv, the forward's y and
+    row log-sum-exps."""
+    qkv: int
+    y: int
+    dy: int
+    out: int
+    dims: tuple
+    scale: float
+    dtype: DType
+
+
+def _rows_cols(shape):
+    return _numel(shape[:-1]), shape[-1]
+
+
+def match_norm(graph: Graph, nid: int) -> NormRowsMatch | None:
+    comp = graph.composites.get(nid)
+    if comp is None or comp["kind"] not in ("layer_norm", "rms_norm") or graph[nid].dtype not in (DType.F32, DType.BF16):
+        return None
+    x, w, b = comp["inputs"]
+    cols = graph[nid].shape[-1]
+    if any(v is not None and (_numel(graph[v].shape) != cols or graph[v].dtype != graph[nid].dtype) for v in (w, b)):
+        return None
+    rows, cols = _rows_cols(graph[nid].shape)
+    return NormRowsMatch(x, w, b, nid, rows, cols, comp["kind"] == "rms_norm", comp["params"]["eps"], graph[nid].dtype)
+
+
+def match_norm_bwd(graph: Graph, nid: int, users: dict) -> NormBwdMatch | None:
+    """`nid` is one of the gradients a norm's reverse pass produced, or the sum of its dx and one other gradient of
+    the same tensor (the skip branch of a pre-norm block) where nothing else reads dx."""
+    n = graph[nid]
+    rec, add, dx_node = graph.fused_bwd.get(nid), None, None
+    if rec is None and n.kind == "binary" and n.op == BOp.Add:
+        for a, other in (n.src, n.src[::-1]):
+            r = graph.fused_bwd.get(a)
+            if r is not None and r["kind"] in ("layer_norm", "rms_norm") and r["grads"].get(r["inputs"][0]) == a \
+                    and users.get(a, set()) <= {nid} and graph[other].shape == n.shape:
+                rec, add, dx_node = r, other, nid
+                break
+    if rec is None or rec["kind"] not in ("layer_norm", "rms_norm") or n.dtype not in (DType.F32, DType.BF16):
+        return None
+    x, w, b = rec["inputs"]
+    gx = rec["grads"][x]
+    if dx_node is None:  # reached through dw or db: dx goes where it would go when reached through itself
+        dx_node = gx
+        readers = users.get(gx, set())
+        if len(readers) == 1:
+            (u,) = readers
+            if u >= 0 and graph[u].kind == "binary" and graph[u].op == BOp.Add and gx in graph[u].src and graph[u].shape == graph[gx].shape \
+                    and graph[u].src[0] != graph[u].src[1]:
+                dx_node, add = u, [v for v in graph[u].src if v != gx][0]
+
+    def wanted(v):
+        return v is not None and (rec["grads"][v] in users or rec["grads"][v] == nid)
+
+    rows, cols = _rows_cols(graph[x].shape)
+    return NormBwdMatch(x, w, rec["dy"], add, dx_node, rec["grads"][w] if wanted(w) else None, rec["grads"][b] if wanted(b) else None,
+                        rows, cols, rec["kind"] == "rms_norm", rec["params"]["eps"], n.dtype)
+
+
+def match_attention(graph: Graph, nid: int, users: dict) -> AttentionMatch | None:
+    comp = graph.composites.get(nid)
+    if comp is None or comp["kind"] != "attention" or graph[nid].dtype not in (DType.F32, DType.BF16):
+        return None
+    (qkv,) = comp["inputs"]
+    b, t, c = graph[nid].shape
+    h = comp["params"]["n_head"]
+    gq = None
+    for g_, rec in graph.fused_bwd.items():  # does a backward of this forward belong to what is being computed?
+        if rec["fwd"] == nid and (g_ in users):
+            gq = g_
+    return AttentionMatch(qkv, nid, (b, t, h, c // h), comp["params"]["scale"], gq is not None, graph[nid].dtype)
+
+
+def match_attention_bwd(graph: Graph, nid: int) -> AttentionBwdMatch | None:
+    rec = graph.fused_bwd.get(nid)
+    if rec is None or rec["kind"] != "attention" or graph[nid].dtype not in (DType.F32, DType.BF16):
+        return None
+    (qkv,) = rec["inputs"]
+    b, t, c = graph[rec["fwd"]].shape
+    h = rec["params"]["n_head"]
+    return AttentionBwdMatch(qkv, rec["fwd"], rec["dy"], nid, (b, t, h, c // h), rec["params"]["scale"], graph[nid].dtype)
+
+
 def match_operands(m) -> tuple:
     """Nodes whose buffers a matched kernel reads, in argument order."""
+    if isinstance(m, NormRowsMatch):
+        return (m.x,) + tuple(v for v in (m.w, m.b) if v is not None)
+    if isinstance(m, NormBwdMatch):
+        return (m.x,) + ((m.w,) if m.w is not None else ()) + (m.dy,) + ((m.add,) if m.add is not None else ())
+    if isinstance(m, AttentionMatch):
+        return (m.qkv,)
+    if isinstance(m, AttentionBwdMatch):
+        return (m.qkv, m.y, m.dy)
     if isinstance(m, Contraction):
         return (m.a, m.b) + ((m.bias,) if m.bias is not None else ()) + ((m.residual,) if m.residual is not None else ())
     if isinstance(m, RowColReduce):
@@ -1180,10 +1411,18 @@ def match_operands(m) -> tuple:
     return (m.x,)
 
 
-MATCHED = (Contraction, SoftmaxRows, RowColReduce, Conv2dMatch, MaxPoolMatch, CrossEntropyMatch)
+MATCHED = (Contraction, SoftmaxRows, RowColReduce, Conv2dMatch, MaxPoolMatch, CrossEntropyMatch, NormRowsMatch, NormBwdMatch,
+           AttentionMatch, AttentionBwdMatch)
 
 
 # ---- lowering ---------------------------------------------------------------------------------------------------------
+
+@dataclasses.dataclass
+class Alias:
+    """`out` shows `base` element for element (a reshape, or permutes that cancel): it shares base's buffer."""
+    out: int
+    base: int
+
 
 @dataclasses.dataclass
 class LoweredKernel:
@@ -1410,7 +1649,8 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
     losses = scan_cross_entropy(graph, [i for i in users if i >= 0] + list(outputs)) if match else {}
 
     def find(nid: int):
-        return (losses.get(nid) or match_conv(graph, nid, users) or match_max_pool(graph, nid)
+        return (losses.get(nid) or match_norm(graph, nid) or match_norm_bwd(graph, nid, users) or match_attention(graph, nid, users)
+                or match_attention_bwd(graph, nid) or match_conv(graph, nid, users) or match_max_pool(graph, nid)
                 or match_linear(graph, nid, users, emitter.relu_mask) or match_contraction(graph, nid)
                 or match_softmax(graph, nid) or match_reduce_update(graph, nid, users) or match_reduce(graph, nid, have))
 
@@ -1428,7 +1668,20 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
                         need(r, True)
                         return
         c = find(nid) if match else None
+        if c is None and match and root:
+            base = _plain(graph, nid)
+            if base is not None and base != nid and graph[base].kind != "const":
+                need(base, True)
+                schedule.append(Alias(nid, base))
+                have.add(nid)
+                return
         if c is not None:
+            for attr in ("x", "w", "b", "dy", "add", "qkv", "bias", "residual", "target", "base"):
+                v = getattr(c, attr, None)  # an operand that only re-views a tensor reads that tensor's buffer
+                if isinstance(v, int) and not isinstance(c, (Conv2dMatch, MaxPoolMatch)):
+                    shown = _plain(graph, v)
+                    if shown is not None and graph[shown].kind != "const":
+                        setattr(c, attr, shown)
             for s in match_operands(c):
                 need(s, True)
             if isinstance(c, Contraction) and c.epilogue == "none" and c.residual is None:
@@ -1438,7 +1691,8 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
             if isinstance(c, Contraction) and c.mask_node is not None:
                 emitter.relu_mask[c.mask_node] = nid
             schedule.append(c)
-            have.update(i for i in ((c.grad, c.mean) if isinstance(c, CrossEntropyMatch) else (nid,)) if i is not None)
+            outs = (c.grad, c.mean) if isinstance(c, CrossEntropyMatch) else (c.dx, c.dw, c.db) if isinstance(c, NormBwdMatch) else (nid,)
+            have.update(i for i in outs if i is not None)
             return
         for s in n.src:
             need(s, False)
@@ -1497,8 +1751,18 @@ class Tape:
     def gradient(self, target: int, sources: Sequence[int]) -> list:
         return self.graph.gradient(target, sources)
 
+    def _aux(self, key, nbytes: int):
+        """A buffer that belongs to a matched kernel and is no graph node (row log-sum-exps, an unwanted output)."""
+        if key not in self._buf:
+            buf, ev = self.pool.allocate(max(int(nbytes), 1))
+            self._buf[key], self._ev[key] = buf, ev
+        return key
+
     def realize(self, nodes: Sequence[int]):
-        for kern in lower(self.graph, [n for n in nodes if n not in self._buf], stored=list(self._buf), match=self.match):
+        for kern in lower(self.graph, [n for n in nodes if n not in self._buf], stored=[n for n in self._buf if isinstance(n, int)], match=self.match):
+            if isinstance(kern, Alias):
+                self._buf[kern.out] = self._buf[kern.base]
+                continue
             if isinstance(kern, MATCHED):
                 kern = self._matched_or_generated(kern)
             prog = self._programs.get(kern.image)
@@ -1543,8 +1807,13 @@ class Tape:
             self.realize(nodes)  # settles which candidate each product runs on; the plan reuses the buffers
         self.sync()
         launches = []
-        stored = [n for n in self._buf if self.graph[n].kind == "leaf"]  # everything else is computed by the plan
+        stored = [n for n in self._buf if isinstance(n, int) and self.graph[n].kind == "leaf"]  # everything else is computed by the plan
         for kern in lower(self.graph, list(nodes), stored=stored, match=bool(self.match)):
+            if isinstance(kern, Alias):
+                if kern.out in updates.values():
+                    raise ValueError("an update has to be computed, not a view of another tensor")
+                self._buf[kern.out] = self._buf[kern.base]
+                continue
             if isinstance(kern, MATCHED):
                 kern = self._matched_or_generated(kern)
             prog = self._programs.get(kern.image)
@@ -1601,9 +1870,34 @@ class Tape:
         self._ev[leaf] = self.pool.copy_range(self._buf[node], 0, self._buf[leaf], 0, nbytes, waits)
 
     def _matched_or_generated(self, c) -> LoweredKernel:
-        from .kernels import conv2d_desc, cross_entropy_desc, gemm_desc, max_pool2d_desc, reduce_desc, softmax_rows_desc
+        from .kernels import (attention_bwd_desc, attention_desc, conv2d_desc, cross_entropy_desc, gemm_desc, max_pool2d_desc,
+                              norm_rows_bwd_desc, norm_rows_desc, reduce_desc, softmax_rows_desc)
         more = ()
-        if isinstance(c, Conv2dMatch):
+        isz = np.dtype(storage_dtype(c.dtype)).itemsize if hasattr(c, "dtype") else 4
+        if isinstance(c, NormRowsMatch):
+            desc = norm_rows_desc(c.rows, c.cols, c.rms, c.w is not None, c.b is not None, c.eps, c.dtype)
+            inputs, elements = list(match_operands(c)), c.rows * c.cols
+        elif isinstance(c, NormBwdMatch):
+            want_db = c.db is not None and not c.rms
+            desc = norm_rows_bwd_desc(c.rows, c.cols, c.rms, c.w is not None, want_db, c.add is not None, c.eps, c.dtype)
+            inputs, elements = list(match_operands(c)), c.rows * c.cols
+            if c.w is not None:  # the kernel writes dw whenever there is a weight
+                more += (c.dw if c.dw is not None else self._aux(("dw", c.dx), c.cols * isz),)
+            if want_db:
+                more += (c.db,)
+        elif isinstance(c, AttentionMatch):
+            b_, t_, h_, dh_ = c.dims
+            desc = attention_desc(b_, t_, h_, dh_, c.dtype, c.scale, 0.0, c.lse, False)
+            inputs, elements = [c.qkv], b_ * t_ * h_ * dh_
+            if c.lse:
+                more = (self._aux(("lse", c.out), b_ * h_ * t_ * 4),)
+        elif isinstance(c, AttentionBwdMatch):
+            b_, t_, h_, dh_ = c.dims
+            desc = attention_bwd_desc(b_, t_, h_, dh_, c.dtype, c.scale, 0.0, False)
+            inputs, elements = [c.qkv, c.y, c.dy, ("lse", c.y)], 3 * b_ * t_ * h_ * dh_
+            if ("lse", c.y) not in self._buf:
+                raise RuntimeError("the attention forward of this backward was realised without its row log-sum-exps")
+        elif isinstance(c, Conv2dMatch):
             n_, c_, h, w, co, kh, kw = c.dims
             desc = conv2d_desc(n_, c_, h, w, co, kh, kw, c.stride, c.padding, c.dilation, c.bias is not None, c.relu, c.dtype)
             inputs, elements = list(match_operands(c)), _numel(self.graph[c.out].shape)
@@ -1671,7 +1965,7 @@ class Tape:
         self._plans.clear()
         for prog in self._programs.values():
             self.dev.release(prog)
-        for buf in list(self._buf.values()) + self._spare:
+        for buf in sorted(set(self._buf.values()) | set(self._spare)):  # aliases share a buffer
             self.pool.deallocate(buf, [])
         self._spare.clear()
         self._programs.clear()
