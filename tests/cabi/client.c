@@ -36,6 +36,19 @@ static int layout(void) {
            offsetof(zhip_ir_op, c), offsetof(zhip_ir_op, aux), offsetof(zhip_ir_op, imm));
     printf("ir %zu %u %d %d %d %d %d %d\n", sizeof(zhip_ir_header), ZHIP_IR_MAGIC, ZHIP_IR_BARRIER, ZHIP_IR_REDUCE, ZHIP_IR_ABS, ZHIP_IR_EQ,
            ZHIP_IR_GLOBAL_MUT, ZHIP_IR_SCOPE_REGISTER);
+    printf("zhip_ceilings %zu memcpy_d2d_GBps %zu read_kernel_GBps %zu mfma_bf16_const_TFLOPs %zu mfma_bf16_random_launch_us %zu\n",
+           sizeof(zhip_ceilings), offsetof(zhip_ceilings, memcpy_d2d_GBps), offsetof(zhip_ceilings, read_kernel_GBps),
+           offsetof(zhip_ceilings, mfma_bf16_const_TFLOPs), offsetof(zhip_ceilings, mfma_bf16_random_launch_us));
+    printf("zhip_rng %zu kinds %d %d %d %d argmax %d ce_dense %d\n", sizeof(zhip_rng), ZHIP_RNG_RAND, ZHIP_RNG_UNIFORM, ZHIP_RNG_RANDN,
+           ZHIP_RNG_RANDINT, ZHIP_K_ARGMAX, ZHIP_CE_DENSE);
+    {   /* the generator needs no device: the reference's known answer starts from seed 42069 (zyx/tests/05_misc.rs:768-774) */
+        zhip_rng r;
+        uint64_t counts[3] = {0, 0, 0};
+        zhip_rng_seed(&r, 42069);
+        printf("rng %llu\n", (unsigned long long)zhip_rng_next_u64(&r));
+        zhip_compile_cache_stats(counts);
+        printf("cache %llu %llu %llu\n", (unsigned long long)counts[0], (unsigned long long)counts[1], (unsigned long long)counts[2]);
+    }
     return 0;
 }
 

@@ -21,7 +21,8 @@ hipError_t softmax_rows(const SoftmaxRows &p, hipStream_t st) { return rec(st, "
 hipError_t elementwise(const Elementwise &p, hipStream_t st) { return rec(st, "elementwise", {p.in[0], p.in[1], p.in[2], p.in[3]}, {p.out}); }
 
 bool reduce_shape_ok(int64_t rows, int64_t cols, int) { return rows >= 0 && cols >= 0 && (cols == 0 || rows <= (1ll << 40) / cols); }
-uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int) { return rows > 0 && cols > 0 ? kScratch : 0; }
+// 7777 rows: a shape whose partial results exceed any scratch, for the callers' refusal paths
+uint64_t reduce_workspace_bytes(int64_t rows, int64_t cols, int) { return rows == 7777 ? (64ull << 20) : rows > 0 && cols > 0 ? kScratch : 0; }
 hipError_t reduce(const Reduce &p, hipStream_t st) { return rec(st, "reduce", {p.x, p.base}, {p.out, p.workspace}); }
 
 bool argmax_shape_ok(int64_t outer, int64_t n, int64_t inner) { return outer >= 0 && n >= 1 && inner >= 0; }

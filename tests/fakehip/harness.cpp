@@ -463,6 +463,12 @@ static void reduce_static_allocates_nothing() {
     EXPECT(hipStreamEndCapture(st, &graph) == hipSuccess);
     EXPECT(fakehip_calls("hipMalloc") == m0 && fakehip_calls("hipFree") == f0 && fakehip_calls("hipEventCreate") == ev0);
     EXPECT(zhip_reduce_static(ctx, ZHIP_F64, 0, 1, 4, 4, xp, sp, st) == ZHIP_KERNEL_COMPILATION);
+    // partial results beyond the static scratch: refused with the sizes, before any pointer is looked at
+    EXPECT(zhip_reduce_static(ctx, ZHIP_F32, 0, 1, 7777, 64, nullptr, nullptr, st) == ZHIP_KERNEL_COMPILATION);
+    EXPECT(strstr(zhip_last_error(ctx), "67108864") && strstr(zhip_last_error(ctx), "1048576"));
+    // null pointers are an argument error, not a launch
+    EXPECT(zhip_reduce_static(ctx, ZHIP_F32, 0, 1, 64, 64, nullptr, sp, st) == ZHIP_INCORRECT_KERNEL_ARG);
+    EXPECT(zhip_reduce_static(ctx, ZHIP_F32, 0, 1, 64, 64, xp, nullptr, st) == ZHIP_INCORRECT_KERNEL_ARG);
     no_hazards("reduce_static");
     (void)hipGraphDestroy(graph);
     (void)hipStreamSynchronize(st);

@@ -41,6 +41,15 @@ def test_header_is_c_and_layouts_match_the_python_mirror(client):
     assert {op[i]: int(op[i + 1]) for i in range(2, len(op), 2)} == {f[0]: getattr(ir.IrOp, f[0]).offset for f in ir.IrOp._fields_}
     assert [int(v) for v in out[5].split()[1:]] == [ctypes.sizeof(ir.IrHeader), ir.MAGIC, ir.Opcode.BARRIER, ir.Opcode.REDUCE, ir.UOp.Abs,
                                                     ir.BOp.Eq, ir.ParamKind.GlobalMut, ir.MemScope.Register]
+    ce = out[6].split()
+    assert ce[0] == "zhip_ceilings" and int(ce[1]) == ctypes.sizeof(backend._Ceilings) == 36
+    assert {ce[i]: int(ce[i + 1]) for i in range(2, len(ce), 2)} == {n: getattr(backend._Ceilings, n).offset for n in ce[2::2]}
+    rg = out[7].split()
+    assert rg[:2] == ["zhip_rng", "32"] and [int(v) for v in rg[3:7]] == [0, 1, 2, 3]
+    assert int(rg[8]) == K.K_ARGMAX and int(rg[10]) == K.CE_DENSE
+    from zyx_amd.rng import Rng
+    assert int(out[8].split()[1]) == Rng(42069).next_u64()   # the generator driven from C and through the Python mirror
+    assert out[9].split()[0] == "cache" and len(out[9].split()) == 4
 
 
 @pytest.mark.gpu

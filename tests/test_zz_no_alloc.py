@@ -88,13 +88,15 @@ def test_single_stage_shapes_and_empty(hip):
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
 
 
-def test_shape_beyond_the_static_scratch_is_refused(hip):
+def test_null_pointers_and_unsupported_dtypes_are_refused(hip):
+    """Nothing is launched for a call that cannot be right. Only null pointers are used here: a made-up non-null
+    pointer would fault the device if a refusal ever went missing. (No shape the reduce planner produces needs more
+    than the 1 MiB of static scratch any more -- its partials are bounded by two workgroups per compute unit -- so that
+    refusal is exercised on the CPU, against the host model of the runtime: tests/fakehip/harness.cpp.)"""
     dev, pool = hip
-    # 256 x 196608 over axis 0 is sized for 3 chunks x 196608 f32 partials (the split 16-bit rows would take) = 2.25 MiB;
-    # refused before any pointer is used
     with pytest.raises(zyx_amd.BackendError) as ei:
-        dev.reduce_static(DType.F32, 0, True, 256, 196608, 256, 256, 0)
+        dev.reduce_static(DType.F32, 0, True, 256, 4096, 0, 0, 0)
+    assert ei.value.status == zyx_amd.ErrorStatus.IncorrectKernelArg and "null" in ei.value.context
+    with pytest.raises(zyx_amd.BackendError) as ei:
+        dev.reduce_static(DType.F64, 0, True, 4, 4, 0, 0, 0)
     assert ei.value.status == zyx_amd.ErrorStatus.KernelCompilation
-    assert "2359296" in ei.value.context and "1048576" in ei.value.context
-    with pytest.raises(zyx_amd.BackendError):
-        dev.reduce_static(DType.F64, 0, True, 4, 4, 256, 256, 0)
