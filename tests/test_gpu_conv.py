@@ -280,3 +280,52 @@ def test_conv3x3_fused_max_pool(hip, oracle, shape, dtype):
         assert np.all(np.abs(got - want) <= 2e-5 * mag)
         with pytest.raises(Exception):  # W = 448: one row per tile
             conv2d(dev, pool, np.zeros((1, 16, 2, 448), np.float32), wt, b, *args, fused_pool=True)
+
+
+def test_relaid_weights_follow_every_write_of_the_weight_buffer(hip, oracle):
+    """The direct 3 x 3 kernel keeps a re-laid copy of its weights in the program's scratch and makes it again only when
+    the weight buffer has been written since (host upload, device copy, another launch's output) or another buffer is
+    passed: launches with unchanged weights give the same bits, every change of the weights shows in the next launch,
+    whichever way it was made, inside a plan too."""
+    from zyx_amd import kernels as K
+    dev, pool = hip
+    r = oracle.Rng(7)
+    n, c, hw, co = 1, 64, 56, 128
+    x = r.randn((n, c, hw, hw))
+    w1, w2 = r.randn((co, c, 3, 3), 0.05), r.randn((co, c, 3, 3), 0.05)
+    prog = dev.register_kernel(K.conv2d_desc(n, c, hw, hw, co, 3, 3, (1, 1), (1, 1), (1, 1), False, False, DType.F32))
+    xb, e0 = K.to_device(pool, x)
+    wa, e1 = K.to_device(pool, w1)
+    wb, e2 = K.to_device(pool, w2)
+    yb, e3 = K.alloc_like(pool, n * co * hw * hw, 4)
+    pool.sync_events([e0, e1, e2, e3])
+
+    def run(wbuf):
+        ev = dev.launch(prog, pool, [xb, wbuf, yb], [])
+        return K.to_host(pool, yb, (n, co, hw, hw), np.float32, [ev])
+
+    y1 = run(wa)
+    assert np.array_equal(run(wa), y1)                       # copy kept
+    y2 = run(wb)                                             # another buffer
+    assert not np.array_equal(y2, y1) and np.array_equal(run(wb), y2)
+    assert np.array_equal(run(wa), y1)                       # and back
+    pool.sync_events([pool.host_to_pool(np.ascontiguousarray(w2, np.float32), wa, [])])
+    assert np.array_equal(run(wa), y2)                       # same buffer, new contents from the host
+    pool.sync_events([pool.host_to_pool(np.ascontiguousarray(w1, np.float32), wb, [])])
+    pool.sync_events([pool.copy_range(wb, 0, wa, 0, w1.size * 4, [])])
+    assert np.array_equal(run(wa), y1)                       # new contents by a device copy
+    plan = dev.create_plan([(prog, [xb, wb, yb])])           # a plan re-lays from its own weights every time
+    pool.sync_events([dev.launch_plan(plan, [])])
+    assert np.array_equal(K.to_host(pool, yb, (n, co, hw, hw), np.float32), y1)   # wb holds w1 now
+    assert np.array_equal(run(wa), y1)
+    pool.sync_events([pool.host_to_pool(np.ascontiguousarray(w2, np.float32), wb, [])])
+    pool.sync_events([dev.launch_plan(plan, [])])
+    assert np.array_equal(K.to_host(pool, yb, (n, co, hw, hw), np.float32), y2)
+    assert np.array_equal(run(wa), y1)                       # the plan's re-layout does not pass for wa's
+    want = oracle.conv2d(x, w1, None, (1, 1), (1, 1), (1, 1))
+    mag = oracle.conv2d(np.abs(x), np.abs(w1), None, (1, 1), (1, 1), (1, 1))
+    assert np.all(np.abs(y1 - want) <= 2e-5 * mag)
+    dev.destroy_plan(plan)
+    dev.release(prog)
+    for b_ in (xb, wa, wb, yb):
+        pool.deallocate(b_, [])

@@ -401,7 +401,9 @@ hipError_t conv3x3_direct(const Conv2d &p, void *wt, hipStream_t st) {
     if ((uintptr_t)p.x % 16 || (uintptr_t)p.y % 16 || (uintptr_t)wt % 16) return hipErrorInvalidValue; // pool blocks are 256-byte aligned
     const int R = tile_rows(p);
     const dim3 wgrid((unsigned)((p.C * p.Cout + 255) / 256));
-    if (p.dtype == DT_F32) hipLaunchKernelGGL((conv3x3_weights_k<float, 3>), wgrid, dim3(256), 0, st, (const float *)p.w, (float *)wt, p.C, p.Cout);
+    if (p.weights_ready) {
+        // the caller knows that w has not been written since the launch that left its re-laid copy in wt
+    } else if (p.dtype == DT_F32) hipLaunchKernelGGL((conv3x3_weights_k<float, 3>), wgrid, dim3(256), 0, st, (const float *)p.w, (float *)wt, p.C, p.Cout);
     else hipLaunchKernelGGL((conv3x3_weights_k<uint16_t, 4>), wgrid, dim3(256), 0, st, (const uint16_t *)p.w, (uint16_t *)wt, p.C, p.Cout);
     dim3 grid((unsigned)(p.N * (p.H / R)), (unsigned)(p.Cout / TILE_CO));
     const bool out_bf16 = p.out_dtype == DT_BF16;

@@ -168,6 +168,7 @@ struct Conv2d {
     void *y;
     const int32_t *koff, *kdyx;
     void *scratch; // conv2d_scratch_bytes(p) bytes when the product runs on the tiled MFMA GEMM, else unused
+    bool weights_ready = false; // the direct kernel's re-laid copy of w in `scratch` is current: skip the re-layout launch
 };
 uint64_t conv2d_scratch_bytes(const Conv2d &p);
 hipError_t conv2d(const Conv2d &p, hipStream_t stream);
