@@ -1447,6 +1447,7 @@ class _Emitter:
     def __init__(self, graph: Graph, stored: set):
         self.g, self.stored = graph, stored
         self.relu_mask: dict[int, int] = {}  # `v > 0` node of a relu whose v is not stored -> the stored relu(v)
+        self.inline: set = set()  # reduces computed inside the kernel of the one expression that reads them element for element
 
     # index arithmetic with constant folding
     def _ix(self, v):
@@ -1507,6 +1508,8 @@ class _Emitter:
         n, k = self.g[nid], self.k
         if (n.kind == "leaf" or nid in self.stored) and not root:
             v = k.load(self.params[nid], self._ix(self.ravel(idx, n.shape)))
+        elif n.kind == "reduce":
+            v = self._reduce(n, idx)
         elif n.kind == "const":
             v = k.const(n.arg, n.dtype)
         elif n.kind == "unary":
@@ -1592,6 +1595,27 @@ class _Emitter:
         for i, s in enumerate(n.src):
             self._inputs(self.relu_mask.get(nid, s) if i == 0 else s, False, seen, order)
 
+    def _reduce(self, n, idx):
+        """Element `idx` of a Reduce as one serial loop with a register accumulator, where it is asked for. What the loop
+        body defines stays inside the loop: the memo and the constant table are put back afterwards."""
+        k = self.k
+        x = n.src[0]
+        xs = self.g[x].shape
+        red = [xs[a] for a in n.arg]
+        zero = self._ix(0)
+        accu = k.storage(n.dtype, MemScope.Register, 1)
+        k.store(accu, k.const(0 if n.op == BOp.Add else min_constant(n.dtype), n.dtype), zero)
+        r = _V(k.loop(self._ix(_numel(red))))
+        outer_consts, outer_memo = dict(self.consts), dict(self.memo)
+        r_idx = self.unravel(r, red)
+        kept = iter(idx if len(n.arg) < len(xs) else [])
+        x_idx = [r_idx[n.arg.index(i)] if i in n.arg else next(kept) for i in range(len(xs))]
+        v = self.value(x, x_idx)
+        k.store(accu, k.binary(v, k.load(accu, zero), n.op), zero)  # x (op) acc, linearize.rs:943-946
+        k.end_loop()
+        self.consts, self.memo = outer_consts, outer_memo
+        return k.load(accu, zero)
+
     def kernel(self, nid: int) -> LoweredKernel:
         n = self.g[nid]
         self.k = k = Kernel()
@@ -1610,25 +1634,7 @@ class _Emitter:
             k.if_(k.cmplt(self._ix(lin), self._ix(total)))
             self.consts = {}  # constants created from here on live inside the If
         idx = self.unravel(lin, n.shape) if n.shape else []
-        if n.kind == "reduce":
-            x = n.src[0]
-            xs = self.g[x].shape
-            red = [xs[a] for a in n.arg]
-            zero = self._ix(0)
-            accu = k.storage(n.dtype, MemScope.Register, 1)
-            k.store(accu, k.const(0 if n.op == BOp.Add else min_constant(n.dtype), n.dtype), zero)
-            r = _V(k.loop(self._ix(_numel(red))))
-            outer, self.consts = dict(self.consts), dict(self.consts)
-            r_idx = self.unravel(r, red)
-            kept = iter(idx if len(n.arg) < len(xs) else [])
-            x_idx = [r_idx[n.arg.index(i)] if i in n.arg else next(kept) for i in range(len(xs))]
-            v = self.value(x, x_idx)
-            k.store(accu, k.binary(v, k.load(accu, zero), n.op), zero)  # x (op) acc, linearize.rs:943-946
-            k.end_loop()
-            self.consts = outer
-            v = k.load(accu, zero)
-        else:
-            v = self.value(nid, idx, root=True)
+        v = self._reduce(n, idx) if n.kind == "reduce" else self.value(nid, idx, root=True)
         k.store(out, v, self._ix(lin))
         if guarded:
             k.end_if()
@@ -1645,7 +1651,7 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
     have = set(stored)
     emitter = _Emitter(graph, have)
     schedule: list = []
-    users = consumers(graph, outputs, stored) if match else {}
+    users = consumers(graph, outputs, stored)
     losses = scan_cross_entropy(graph, [i for i in users if i >= 0] + list(outputs)) if match else {}
 
     def find(nid: int):
@@ -1654,9 +1660,11 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
                 or match_linear(graph, nid, users, emitter.relu_mask) or match_contraction(graph, nid)
                 or match_softmax(graph, nid) or match_reduce_update(graph, nid, users) or match_reduce(graph, nid, have))
 
-    def need(nid: int, root: bool):
+    def need(nid: int, root: bool, via: int | None = None):
+        """via: the node that reads `nid` when every node between the kernel's root and `nid` keeps the element order
+        (unary, cast, reshape, binary with an operand of its own shape), else None."""
         n = graph[nid]
-        if n.kind == "leaf" or nid in have:
+        if n.kind == "leaf" or nid in have or nid in emitter.inline:
             return
         if match:
             # A convolution or a Linear read only by its relu is never stored: the relu's launch computes both, and the
@@ -1694,8 +1702,30 @@ def lower(graph: Graph, outputs: Sequence[int], stored: Sequence[int] = (), matc
             outs = (c.grad, c.mean) if isinstance(c, CrossEntropyMatch) else (c.dx, c.dw, c.db) if isinstance(c, NormBwdMatch) else (nid,)
             have.update(i for i in outs if i is not None)
             return
+        if n.kind == "reduce" and not root and via is not None and users.get(nid, set()) == {via}:
+            # read once, element for element, by an expression whose thread i wants exactly element i: the loop runs
+            # inside that expression's kernel and the reduce gets no buffer and no launch of its own
+            emitter.inline.add(nid)
+            for s in n.src:
+                need(s, False)
+            return
         for s in n.src:
-            need(s, False)
+            keeps = (n.kind in ("unary", "cast", "reshape") or (n.kind == "binary" and graph[s].shape == n.shape)) and n.kind != "reduce"
+            reader = nid if keeps and (root or via is not None) else None
+            if reader is not None and graph[s].kind in ("reshape", "permute"):
+                # a chain of views that shows a reduce element for element (transposes that cancel): same thing
+                b = _plain(graph, s)
+                if b is not None and b != s and graph[b].kind == "reduce" and b not in have and b not in emitter.inline:
+                    chain, i = [], s
+                    while i != b:
+                        chain.append(i)
+                        i = graph[i].src[0]
+                    if all(users.get(c, set()) == {r} for c, r in zip(chain + [b], [nid] + chain)) and not (match and find(b) is not None):
+                        emitter.inline.add(b)
+                        for q in graph[b].src:
+                            need(q, False)
+                        continue
+            need(s, False, reader)
         if root or n.kind == "reduce":
             schedule.append(emitter.kernel(nid))
             have.add(nid)
