@@ -9,16 +9,18 @@
 // Ps is recomputed from the saved lse = ln sum exp(scale q k^T) instead of being stored.
 //
 // Matrix-core path (bf16, dh = 64, T % 128 == 0), three launches:
-//   attn_bwd_d_k    D[B,H,T] into the program's workspace;
+//   attn_bwd_d_k    -D keep [B,H,T] and lse log2(e) into the program's workspace;
 //   attn_bwd_dkv_k  one workgroup per (batch, head, 128 keys), a wave owns 32 keys and streams query
 //                   tiles; S = Q.K^T is formed queries x keys so that a lane owns a key column and the
 //                   exponentiated / differentiated tiles, packed to bf16, are the B operands of
 //                   dV^T += dy^T.P and dK^T += Q^T.dS (dy^T and Q^T come through the transposing LDS read);
+//                   the three steps of a 32-query sub-tile run in three consecutive iterations (software pipeline);
 //   attn_bwd_dq_k   one workgroup per (batch, head, 128 queries), S^T = K.Q^T keys x queries (a lane owns
 //                   a query, lse and D are per-lane scalars), dQ^T += K^T.dS^T.
 // No atomics: every output element has one owner, results are reproducible.
 //
 // attn_bwd_small_*: any dh <= 256 and T, f32 or bf16 storage, f32 arithmetic, one wave per query / key.
+#include <type_traits>
 #include "attn_common.hpp"
 #include "kernels.hpp"
 
@@ -30,13 +32,17 @@ namespace {
 
 constexpr int STAGE_BWD = 2 * TILE + 512; // two tiles + lse*log2(e) [64] + D [64]
 
-// D[bh, t] = sum_d dy[b,t,h,d] * y[b,t,h,d]; 8 lanes per row of 64.
+// D[bh, t] = sum_d dy[b,t,h,d] * y[b,t,h,d], 8 lanes per row of 64, stored as Dn = -D * keep; and lse2 = lse * log2(e).
 __global__ __launch_bounds__(256) void attn_bwd_d_k(const uint16_t *__restrict__ y, const uint16_t *__restrict__ dy,
-                                                    float *__restrict__ D, int64_t rows, int T, int H) {
-    const int64_t row = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3); // row = (b*T + t)*H + h
+                                                    const float *__restrict__ lse, float *__restrict__ Dn,
+                                                    float *__restrict__ lse2, int64_t rows, int T, int H, float keep) {
+    // rows are taken in the order of the results, o = (b*H + h)*T + t: eight lanes read the 128 bytes of row
+    // (b*T + t)*H + h of y and dy, and the three results of 32 consecutive t leave as whole cache lines
+    const int64_t o = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3);
     const int part = threadIdx.x & 7;
     float a = 0.0f;
-    if (row < rows) {
+    if (o < rows) {
+        const int64_t bhh = o / T, t = o % T, b = bhh / H, h = bhh % H, row = (b * T + t) * H + h;
         const u32x4 u = *(const u32x4 *)(y + row * DH + part * 8), v = *(const u32x4 *)(dy + row * DH + part * 8);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -47,22 +53,39 @@ __global__ __launch_bounds__(256) void attn_bwd_d_k(const uint16_t *__restrict__
     a += dpp_f32<kDppQuadXor1>(a);
     a += dpp_f32<kDppQuadXor2>(a);
     a += dpp_f32<kDppRowHalfMirror>(a);
-    if (row < rows && part == 0) {
-        const int64_t bt = row / H, h = row % H, b = bt / T, t = bt % T;
-        D[(b * H + h) * T + t] = a;
+    if (o < rows && part == 0) {
+        Dn[o] = -a * keep; // what the dP accumulators start from: dP - D keep = keep (dP / keep - D)
+        lse2[o] = lse[o] * kLog2e; // the exponent the kernels subtract, in exp2 units
     }
 }
 
-// CAUSAL (both kernels below): pairs with key > query carry probability 0. Tiles that hold only such pairs are not
-// visited (the workgroup's loop bounds) or not computed (a wave's own keys / queries), and the tiles the diagonal
-// crosses zero the masked probabilities, which zeroes dS too. The number of tiles then depends on the block, so a
-// workgroup takes blocks j and nblk-1-j one after the other: equal work for every workgroup, on whatever CU.
+// 64 lanes x 16 (or 4) bytes from global memory straight into LDS at `lds` (wave-uniform byte address) + 16 (4) * lane.
+// Written as instructions, not through the compiler's builtin: for the builtin the compiler waits for every such
+// load in flight (vmcnt(0)) before the next LDS read that may touch the same array. Completion is tracked by hand:
+// callers wait with s_waitcnt vmcnt and a workgroup barrier before anybody reads what was loaded. The compiler's own
+// vmcnt bookkeeping stays safe: these loads only ever make the counter larger than it assumes.
+__device__ __forceinline__ void load16_to_lds(const void *g, ZK_LDS void *lds) {
+    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(base), "v"(g) : "memory");
+}
+__device__ __forceinline__ void load4_to_lds(const void *g, ZK_LDS void *lds) {
+    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(base), "v"(g) : "memory");
+}
+
+// dK and dV as one software pipeline per workgroup (128 keys, a wave owns 32) over sub-tiles of 32 queries: iteration
+// j issues S = Q.K^T and dP = dy.V^T of sub-tile j+1 and the products dV^T += dy^T.P, dK^T += Q^T.dS of sub-tile j-1
+// (16 matrix instructions) between slices of sub-tile j's vector work (exp2, dS = P o (dP/keep - D), bf16 packing),
+// in an order pinned by scheduling fences, so that inside one wave the matrix pipe and the vector unit always have
+// independent work. Q / dy tiles of 64 queries with their lse*log2(e) and D rows live in a ring of 4 LDS stages
+// filled by direct global->LDS loads three tiles ahead; one workgroup barrier per tile.
 template <bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ dy,
-                                                         const float *__restrict__ lse, const float *__restrict__ D,
+                                                         const float *__restrict__ lse2, const float *__restrict__ Dn,
                                                          uint16_t *__restrict__ dqkv, int T, int H, float c, float scale,
                                                          float inv_keep) {
-    __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[2 * STAGE_BWD];
+    constexpr int NS = 4;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[NS * STAGE_BWD];
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
     int bh, kblk;
@@ -74,12 +97,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restr
     if (CAUSAL && pass) {
         kblk = nblk - 1 - blk_first;
         if (kblk == blk_first) break;
+        __syncthreads(); // the first block's last tile has been read by every wave
     }
     const int bb = bh / H, h = bh % H;
     const int64_t C = (int64_t)H * DH, ld = 3 * C;
     const uint16_t *qp = qkv + (int64_t)bb * T * ld + h * DH, *kp = qp + C, *vp = kp + C;
     const uint16_t *dop = dy + (int64_t)bb * T * C + h * DH;
-    const float *lsep = lse + (int64_t)bh * T, *Dp = D + (int64_t)bh * T;
+    const float *lsep = lse2 + (int64_t)bh * T, *Dp = Dn + (int64_t)bh * T;
     const int tk = kblk * 128 + wave * 32 + (lane & 31);
 
     bf16x8 kfr[4], vfr[4]; // B operands: lane -> key, k-slots = dh
@@ -89,33 +113,24 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restr
         vfr[ks] = *(const bf16x8 *)(vp + (int64_t)tk * ld + ks * 16 + hh * 8);
     }
 
-    u32x4 rq[2], rdo[2];
-    float rstat = 0.0f; // threads 0..63: lse of query tid; 64..127: D of query tid - 64
-    int sl[2];
+    // staging: lane l of a wave-load fetches the chunk that belongs at row l/8, physical slot l%8 of 8 tile rows;
+    // wave w moves rows i*32 + w*8 .. +7 (i = 0, 1) of both tiles, waves 0 and 1 also the 64 lse and the 64 D values
     uint32_t gq[2], gdo[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        const int ch = tid + 256 * i, row = ch >> 3, cc = ch & 7;
+        const int row = i * 32 + wave * 8 + (lane >> 3), cc = (lane & 7) ^ tile_f(row);
         gq[i] = (uint32_t)(row * ld + cc * 8) * 2;
         gdo[i] = (uint32_t)(row * C + cc * 8) * 2;
-        sl[i] = tile_slot(row, cc);
     }
-    auto gload = [&](int qt) {
+    auto stage_tile = [&](int qt, int stage) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            rq[i] = *(const u32x4 *)((const uint8_t *)qp + (int64_t)qt * TROWS * ld * 2 + gq[i]);
-            rdo[i] = *(const u32x4 *)((const uint8_t *)dop + (int64_t)qt * TROWS * C * 2 + gdo[i]);
+            const int rows = (i * 32 + wave * 8) * 128;
+            load16_to_lds((const uint8_t *)qp + (int64_t)qt * TROWS * ld * 2 + gq[i], (ZK_LDS void *)(smem + stage + rows));
+            load16_to_lds((const uint8_t *)dop + (int64_t)qt * TROWS * C * 2 + gdo[i], (ZK_LDS void *)(smem + stage + TILE + rows));
         }
-        if (tid < 64) rstat = lsep[qt * TROWS + tid] * kLog2e;
-        else if (tid < 128) rstat = Dp[qt * TROWS + tid - 64];
-    };
-    auto lwrite = [&](int stage) {
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            *(ZK_LDS u32x4 *)(smem + stage + sl[i]) = rq[i];
-            *(ZK_LDS u32x4 *)(smem + stage + TILE + sl[i]) = rdo[i];
-        }
-        if (tid < 128) *(ZK_LDS float *)(smem + stage + 2 * TILE + tid * 4) = rstat;
+        if (wave == 0) load4_to_lds(lsep + qt * TROWS + lane, (ZK_LDS void *)(smem + stage + 2 * TILE));
+        else if (wave == 1) load4_to_lds(Dp + qt * TROWS + lane, (ZK_LDS void *)(smem + stage + 2 * TILE + 256));
     };
 
     int fr[4], ft[2][2];
@@ -133,90 +148,179 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restr
 #pragma unroll
         for (int r = 0; r < 16; r++) dkT[db][r] = dvT[db][r] = 0.0f;
 
-    const int NT = T / TROWS;
-    const int QT0 = CAUSAL ? 2 * kblk : 0;        // first query tile that holds a query >= this block's first key
-    const int k0w = kblk * 128 + wave * 32;       // first key of this wave
-    gload(QT0);
-    lwrite(0);
+    const int QT0 = CAUSAL ? 2 * kblk : 0; // first query tile that holds a query >= this block's first key
+    const int NTQ = T / TROWS - QT0;       // tiles this block streams, u = 0 .. NTQ-1 is query tile QT0 + u
+    const int k0w = kblk * 128 + wave * 32; // first key of this wave
+#pragma unroll
+    for (int u = 0; u < 3; u++)
+        if (u < NTQ) stage_tile(QT0 + u, u * STAGE_BWD);
+    __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
-    int stage = 0;
-    for (int qt = QT0; qt < NT; qt++) {
-        if (qt + 1 < NT) gload(qt + 1);
-        const bool diag = CAUSAL && qt * TROWS < k0w + 31; // some query of the tile is before some key of this wave
-        if (!CAUSAL || qt * TROWS + TROWS - 1 >= k0w) {
+
+    const f32x16 zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    f32x16 sA, dpA, sB, dpB;
+    u32x4 pbA[2], dsA[2], pbB[2], dsB[2]; // P and dS of a sub-tile as bf16 pairs: [16-query half]
 #pragma unroll
-        for (int qb = 0; qb < 2; qb++) {
-            f32x16 s, dp;
+    for (int s2 = 0; s2 < 2; s2++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.0f;
+        for (int e = 0; e < 4; e++) pbB[s2][e] = dsB[s2][e] = 0u;
+    // register r of a lane's S / dP tile is query 8*(r/4) + 4*hh + r%4 of the sub-tile: the dP accumulators start at that
+    // query's -D keep, read from the stage's D row four at a time
+    auto dp_start = [&](int stat) {
+        f32x4 d[4];
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                const bf16x8 a = frag_row(smem, stage + qb * 32 * 128 + fr[ks]);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kfr[ks], s, 0, 0, 0);
-            }
+        for (int g = 0; g < 4; g++) d[g] = *(const ZK_LDS f32x4 *)(smem + stat + 256 + (8 * g + 4 * hh) * 4);
+        f32x16 v;
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                const bf16x8 a = frag_row(smem, stage + TILE + qb * 32 * 128 + fr[ks]);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vfr[ks], dp, 0, 0, 0);
-            }
-            // register r of this lane is query qb*32 + 8*(r/4) + 4*hh + r%4
-            bf16x8 pb[2], dsb[2];
+        for (int r = 0; r < 16; r++) v[r] = d[r >> 2][r & 3];
+        return v;
+    };
+    dpA = dp_start(2 * TILE);
 #pragma unroll
-            for (int s2 = 0; s2 < 2; s2++) {
-                f32x8 p, ds;
-#pragma unroll
-                for (int g = 0; g < 2; g++) {
-                    const int q0 = qb * 32 + 8 * (2 * s2 + g) + 4 * hh;
-                    const f32x4 l2 = *(const ZK_LDS f32x4 *)(smem + stage + 2 * TILE + q0 * 4);
-                    const f32x4 dd = *(const ZK_LDS f32x4 *)(smem + stage + 2 * TILE + 256 + q0 * 4);
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const int r = 8 * s2 + 4 * g + j;
-                        float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], c, -l2[j]));
-                        if (CAUSAL && diag && qt * TROWS + q0 + j < tk) pv = 0.0f;
-                        p[4 * g + j] = pv;
-                        ds[4 * g + j] = pv * __builtin_fmaf(dp[r], inv_keep, -dd[j]);
-                    }
-                }
-                pb[s2] = __builtin_convertvector(p, bf16x8);
-                dsb[s2] = __builtin_convertvector(ds, bf16x8);
-            }
-#pragma unroll
-            for (int s2 = 0; s2 < 2; s2++)
-#pragma unroll
-                for (int db = 0; db < 2; db++) {
-                    const int base = stage + (qb * 32 + 16 * s2) * 128;
-                    const bf16x8 doT = frag_tr(smem, base + TILE + ft[db][0], base + TILE + ft[db][1]);
-                    dvT[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(doT, pb[s2], dvT[db], 0, 0, 0);
-                    const bf16x8 qT = frag_tr(smem, base + ft[db][0], base + ft[db][1]);
-                    dkT[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qT, dsb[s2], dkT[db], 0, 0, 0);
-                }
-        }
-        }
-        if (qt + 1 < NT) lwrite(stage ^ STAGE_BWD);
-        __syncthreads();
-        stage ^= STAGE_BWD;
+    for (int ks = 0; ks < 4; ks++) {
+        sA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(smem, fr[ks]), kfr[ks], ks == 0 ? zero16 : sA, 0, 0, 0);
+        dpA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(smem, TILE + fr[ks]), vfr[ks], dpA, 0, 0, 0);
     }
 
+    // One sub-tile. st1: stage and 32-row half that sub-tile j+1's Q / dy rows are read from; st3: the same for
+    // sub-tile j-1 (transposed reads); stat, stat1: where the lse and D rows of sub-tiles j and j+1 are; qbase: first
+    // query of sub-tile j.
+    auto sub = [&](auto mask_, int st1, int st3, int stat, int stat1, int qbase, const f32x16 &sc, const f32x16 &dpc, f32x16 &sn, f32x16 &dpn,
+                   const u32x4 (&pbp)[2], const u32x4 (&dsp)[2], u32x4 (&pbn)[2], u32x4 (&dsn)[2]) {
+        constexpr bool MASK = decltype(mask_)::value;
+        f32x16 dstart; // what sub-tile j+1's dP accumulators start from
+        // Issue order, pinned by fences: matrix instruction i, then the LDS reads of the fragment DIST instructions
+        // ahead, then slice i of the vector work, written so that no instruction reads the result of the one before
+        // it: slice i scales and shifts element i+1 (two fma), exponentiates element i, multiplies element i-1 and
+        // packs a finished pair.
+        constexpr int DIST = 4;
+        bf16x8 frg[16]; // 0..7: transposed dy^T / Q^T fragments of sub-tile j-1 (s2, db, which); 8..15: rows of Q / dy of j+1 (ks, which)
+        auto read_frag = [&](int f) {
+            if (f < 8) {
+                const int s2 = f >> 2, db = (f >> 1) & 1, isq = f & 1;
+                const int base = st3 + 16 * s2 * 128 + (isq ? 0 : TILE);
+                frg[f] = frag_tr(smem, base + ft[db][0], base + ft[db][1]);
+            } else {
+                const int ks = (f - 8) >> 1, isdo = f & 1;
+                frg[f] = frag_row(smem, st1 + (isdo ? TILE : 0) + fr[ks]);
+            }
+        };
+        auto matrix = [&](int f) {
+            if (f < 8) {
+                const int s2 = f >> 2, db = (f >> 1) & 1, isq = f & 1;
+                if (isq) dkT[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frg[f], __builtin_bit_cast(bf16x8, dsp[s2]), dkT[db], 0, 0, 0);
+                else dvT[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frg[f], __builtin_bit_cast(bf16x8, pbp[s2]), dvT[db], 0, 0, 0);
+            } else {
+                const int ks = (f - 8) >> 1, isdo = f & 1;
+                if (isdo) dpn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frg[f], vfr[ks], ks == 0 ? dstart : dpn, 0, 0, 0);
+                else sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frg[f], kfr[ks], ks == 0 ? zero16 : sn, 0, 0, 0);
+            }
+        };
+        // register r of this lane is query qbase + 8*(r/4) + 4*hh + r%4; its lse and D come in groups of four
+        f32x4 l2[4];
+        auto read_stat = [&](int g) { l2[g] = *(const ZK_LDS f32x4 *)(smem + stat + (8 * g + 4 * hh) * 4); };
+        // element r: scale and shift (slot r-1) -> exp2 (slot r) -> product with dP - D keep (slot r+1); a pair is
+        // packed one slot after its second product
+        float arg[2], pv[4], ds[4];
+        auto shift = [&](int r) { arg[r & 1] = __builtin_fmaf(sc[r], c, -l2[r >> 2][r & 3]); };
+        auto expo = [&](int r) {
+            pv[r & 3] = __builtin_amdgcn_exp2f(arg[r & 1]);
+            if (MASK && qbase + 8 * (r >> 2) + 4 * hh + (r & 3) < tk) pv[r & 3] = 0.0f; // query before key
+        };
+        auto product = [&](int r) { ds[r & 3] = pv[r & 3] * dpc[r]; }; // keep . dS: 1 / keep goes into dK's final scale
+        auto pack = [&](int r) { // elements r-1, r (r odd)
+            uint32_t w0, w1; // two f32 -> two bf16, round to nearest even; written as instructions so that they stay in their slot
+            asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(w0) : "v"(pv[(r - 1) & 3]), "v"(pv[r & 3]));
+            asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(w1) : "v"(ds[(r - 1) & 3]), "v"(ds[r & 3]));
+            pbn[r >> 3][(r >> 1) & 3] = w0;
+            dsn[r >> 3][(r >> 1) & 3] = w1;
+        };
+        read_stat(0);
+        read_stat(1);
+#pragma unroll
+        for (int f = 0; f < DIST; f++) read_frag(f);
+        __builtin_amdgcn_sched_barrier(0);
+        shift(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            matrix(i);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + DIST < 16) read_frag(i + DIST);
+            if (i == 2) read_stat(2);
+            if (i == 4) dstart = dp_start(stat1);
+            if (i == 6) read_stat(3);
+            if (i > 0) product(i - 1);
+            expo(i);
+            if (i + 1 < 16) shift(i + 1);
+            if (i >= 3 && (i & 1)) pack(i - 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        product(15);
+        pack(15);
+        // pinned here: left alone, the compiler moves the vector work down to its first use in the next iteration
+#pragma unroll
+        for (int s2 = 0; s2 < 2; s2++) asm volatile("" : "+v"(pbn[s2]), "+v"(dsn[s2]));
+    };
+    const std::true_type masked;
+    const std::false_type plain;
+    // tile u: sub-tiles 2u (rows 0..31) and 2u+1. Sub-tile 2u reads the second half of tile u for j+1 and the second
+    // half of tile u-1 for j-1 (sub-tile 0: any landed rows, against a zero P); sub-tile 2u+1 reads the first half of
+    // tile u+1 (past the end: rows nobody uses the product of) and the first half of tile u.
+    int su = 0, sprev = 0; // stages of tile u and of tile u-1
+    for (int u = 0; u < NTQ; u++) {
+        const int snext = su + STAGE_BWD == NS * STAGE_BWD ? 0 : su + STAGE_BWD;
+        const int q0 = (QT0 + u) * TROWS;
+        const bool diag = CAUSAL && q0 < k0w + 31; // some query of the tile is before some key of this wave
+        if (CAUSAL && diag) sub(masked, su + 32 * 128, sprev + 32 * 128, su + 2 * TILE, su + 2 * TILE + 128, q0, sA, dpA, sB, dpB, pbB, dsB, pbA, dsA);
+        else sub(plain, su + 32 * 128, sprev + 32 * 128, su + 2 * TILE, su + 2 * TILE + 128, q0, sA, dpA, sB, dpB, pbB, dsB, pbA, dsA);
+        // tile u+1 must have landed, tile u-1 is no longer read: its stage takes tile u+3
+        if (u + 2 < NTQ) {
+            if (wave < 2) __builtin_amdgcn_s_waitcnt(0x0f70 | 5);
+            else __builtin_amdgcn_s_waitcnt(0x0f70 | 4);
+        } else __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        if (u + 3 < NTQ) stage_tile(QT0 + u + 3, sprev == su ? 3 * STAGE_BWD : sprev);
+        if (CAUSAL && diag) sub(masked, snext, su, su + 2 * TILE + 128, snext + 2 * TILE, q0 + 32, sB, dpB, sA, dpA, pbA, dsA, pbB, dsB);
+        else sub(plain, snext, su, su + 2 * TILE + 128, snext + 2 * TILE, q0 + 32, sB, dpB, sA, dpA, pbA, dsA, pbB, dsB);
+        sprev = su;
+        su = snext;
+    }
+    // the products of the last sub-tile (second half of the last tile, stage sprev)
+#pragma unroll
+    for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+        for (int db = 0; db < 2; db++) {
+            const int base = sprev + (32 + 16 * s2) * 128;
+            dvT[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(smem, base + TILE + ft[db][0], base + TILE + ft[db][1]), __builtin_bit_cast(bf16x8, pbB[s2]), dvT[db], 0, 0, 0);
+            dkT[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(smem, base + ft[db][0], base + ft[db][1]), __builtin_bit_cast(bf16x8, dsB[s2]), dkT[db], 0, 0, 0);
+        }
+
     // result register r of lane: d = db*32 + 8*(r/4) + 4*hh + r%4, key = lane % 32
+    const float ks_ = scale * inv_keep; // dK accumulated keep . dS
     uint16_t *dk = dqkv + ((int64_t)bb * T + tk) * ld + C + h * DH, *dv = dk + C;
 #pragma unroll
     for (int db = 0; db < 2; db++)
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const int d = db * 32 + 8 * g + 4 * hh;
-            *(u32x2 *)(dk + d) = pack4_trunc(dkT[db][4 * g] * scale, dkT[db][4 * g + 1] * scale, dkT[db][4 * g + 2] * scale, dkT[db][4 * g + 3] * scale);
+            *(u32x2 *)(dk + d) = pack4_trunc(dkT[db][4 * g] * ks_, dkT[db][4 * g + 1] * ks_, dkT[db][4 * g + 2] * ks_, dkT[db][4 * g + 3] * ks_);
             *(u32x2 *)(dv + d) = pack4_trunc(dvT[db][4 * g] * inv_keep, dvT[db][4 * g + 1] * inv_keep, dvT[db][4 * g + 2] * inv_keep, dvT[db][4 * g + 3] * inv_keep);
         }
     }
 }
 
+// dQ in the same software pipeline, one workgroup per (batch, head, 128 queries), a wave owns 32 queries and streams key
+// tiles in sub-tiles of 32 keys: iteration j issues S^T = K.Q^T and dP^T = V.dy^T of sub-tile j+1 and dQ^T += K^T.dS^T of
+// sub-tile j-1 (12 matrix instructions) between the vector work of sub-tile j. A lane owns a query: its lse log2(e) and
+// -D keep are scalars, and the dP^T accumulators start at -D keep.
 template <bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ dy,
-                                                        const float *__restrict__ lse, const float *__restrict__ D,
+                                                        const float *__restrict__ lse2, const float *__restrict__ Dn,
                                                         uint16_t *__restrict__ dqkv, int T, int H, float c, float scale,
                                                         float inv_keep) {
-    __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[4 * TILE];
+    constexpr int NS = 4, STAGE = 2 * TILE; // K tile then V tile
+    __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[NS * STAGE];
     ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
     int bh, qblk;
@@ -228,6 +332,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restri
     if (CAUSAL && pass) {
         qblk = nblk - 1 - blk_first;
         if (qblk == blk_first) break;
+        __syncthreads(); // the first block's last tile has been read by every wave
     }
     const int bb = bh / H, h = bh % H;
     const int64_t C = (int64_t)H * DH, ld = 3 * C;
@@ -240,29 +345,23 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restri
         qfr[ks] = *(const bf16x8 *)(qp + (int64_t)tq * ld + ks * 16 + hh * 8);
         dofr[ks] = *(const bf16x8 *)(dy + ((int64_t)bb * T + tq) * C + h * DH + ks * 16 + hh * 8);
     }
-    const float l2 = lse[(int64_t)bh * T + tq] * kLog2e, dd = D[(int64_t)bh * T + tq];
+    const float l2 = lse2[(int64_t)bh * T + tq], dn = Dn[(int64_t)bh * T + tq];
+    f32x16 dstart;
+#pragma unroll
+    for (int r = 0; r < 16; r++) dstart[r] = dn;
 
-    u32x4 rk[2], rv[2];
-    int sl[2];
     uint32_t go[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        const int ch = tid + 256 * i, row = ch >> 3, cc = ch & 7;
+        const int row = i * 32 + wave * 8 + (lane >> 3), cc = (lane & 7) ^ tile_f(row);
         go[i] = (uint32_t)(row * ld + cc * 8) * 2;
-        sl[i] = tile_slot(row, cc);
     }
-    auto gload = [&](int kt) {
+    auto stage_tile = [&](int kt, int stage) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            rk[i] = *(const u32x4 *)((const uint8_t *)kp + (int64_t)kt * TROWS * ld * 2 + go[i]);
-            rv[i] = *(const u32x4 *)((const uint8_t *)vp + (int64_t)kt * TROWS * ld * 2 + go[i]);
-        }
-    };
-    auto lwrite = [&](int stage) {
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            *(ZK_LDS u32x4 *)(smem + stage + sl[i]) = rk[i];
-            *(ZK_LDS u32x4 *)(smem + stage + TILE + sl[i]) = rv[i];
+            const int rows = (i * 32 + wave * 8) * 128;
+            load16_to_lds((const uint8_t *)kp + (int64_t)kt * TROWS * ld * 2 + go[i], (ZK_LDS void *)(smem + stage + rows));
+            load16_to_lds((const uint8_t *)vp + (int64_t)kt * TROWS * ld * 2 + go[i], (ZK_LDS void *)(smem + stage + TILE + rows));
         }
     };
     int fr[4], ft[2][2];
@@ -282,63 +381,120 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restri
 
     const int NT = CAUSAL ? 2 * qblk + 2 : T / TROWS;
     const int q0w = qblk * 128 + wave * 32; // first query of this wave
-    gload(0);
-    lwrite(0);
+#pragma unroll
+    for (int u = 0; u < 3; u++)
+        if (u < NT) stage_tile(u, u * STAGE);
+    __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
-    int stage = 0;
-    for (int kt = 0; kt < NT; kt++) {
-        if (kt + 1 < NT) gload(kt + 1);
-        const bool diag = CAUSAL && kt * TROWS + TROWS - 1 > q0w;
-        if (!CAUSAL || kt * TROWS <= q0w + 31) {
+
+    const f32x16 zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    f32x16 sA, dpA, sB, dpB;
+    u32x4 dsA[2], dsB[2]; // dS^T of a sub-tile as bf16 pairs: [16-key half]
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-            f32x16 s, dp;
+    for (int s2 = 0; s2 < 2; s2++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.0f;
+        for (int e = 0; e < 4; e++) dsB[s2][e] = 0u;
+    dpA = dstart;
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                const bf16x8 a = frag_row(smem, stage + kb * 32 * 128 + fr[ks]);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qfr[ks], s, 0, 0, 0);
-            }
-#pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                const bf16x8 a = frag_row(smem, stage + TILE + kb * 32 * 128 + fr[ks]);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dofr[ks], dp, 0, 0, 0);
-            }
-            bf16x8 dsb[2];
-#pragma unroll
-            for (int s2 = 0; s2 < 2; s2++) {
-                f32x8 ds;
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 * s2 + e], c, -l2));
-                    // register r = 8*s2 + e is key kb*32 + 8*(r/4) + 4*hh + r%4 of the tile
-                    if (CAUSAL && diag && kt * TROWS + kb * 32 + 8 * (2 * s2 + (e >> 2)) + 4 * hh + (e & 3) > tq) pv = 0.0f;
-                    ds[e] = pv * __builtin_fmaf(dp[8 * s2 + e], inv_keep, -dd);
-                }
-                dsb[s2] = __builtin_convertvector(ds, bf16x8);
-            }
-#pragma unroll
-            for (int s2 = 0; s2 < 2; s2++)
-#pragma unroll
-                for (int db = 0; db < 2; db++) {
-                    const int base = stage + (kb * 32 + 16 * s2) * 128;
-                    const bf16x8 kT = frag_tr(smem, base + ft[db][0], base + ft[db][1]);
-                    dqT[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kT, dsb[s2], dqT[db], 0, 0, 0);
-                }
-        }
-        }
-        if (kt + 1 < NT) lwrite(stage ^ (2 * TILE));
-        __syncthreads();
-        stage ^= 2 * TILE;
+    for (int ks = 0; ks < 4; ks++) {
+        sA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(smem, fr[ks]), qfr[ks], ks == 0 ? zero16 : sA, 0, 0, 0);
+        dpA = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(smem, TILE + fr[ks]), dofr[ks], dpA, 0, 0, 0);
     }
+
+    // One sub-tile. st1: stage and 32-row half that sub-tile j+1's K / V rows are read from; st3: the same for sub-tile
+    // j-1's K rows (transposed reads); kbase: first key of sub-tile j.
+    auto sub = [&](auto mask_, int st1, int st3, int kbase, const f32x16 &sc, const f32x16 &dpc, f32x16 &sn, f32x16 &dpn,
+                   const u32x4 (&dsp)[2], u32x4 (&dsn)[2]) {
+        constexpr bool MASK = decltype(mask_)::value;
+        constexpr int DIST = 4;
+        bf16x8 frg[12]; // 0..3: K^T fragments of sub-tile j-1 (s2, db); 4..11: rows of K / V of sub-tile j+1 (ks, which)
+        auto read_frag = [&](int f) {
+            if (f < 4) {
+                const int s2 = f >> 1, db = f & 1, base = st3 + 16 * s2 * 128;
+                frg[f] = frag_tr(smem, base + ft[db][0], base + ft[db][1]);
+            } else {
+                const int ks = (f - 4) >> 1, isv = f & 1;
+                frg[f] = frag_row(smem, st1 + (isv ? TILE : 0) + fr[ks]);
+            }
+        };
+        auto matrix = [&](int f) {
+            if (f < 4) dqT[f & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frg[f], __builtin_bit_cast(bf16x8, dsp[f >> 1]), dqT[f & 1], 0, 0, 0);
+            else {
+                const int ks = (f - 4) >> 1, isv = f & 1;
+                if (isv) dpn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frg[f], dofr[ks], ks == 0 ? dstart : dpn, 0, 0, 0);
+                else sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frg[f], qfr[ks], ks == 0 ? zero16 : sn, 0, 0, 0);
+            }
+        };
+        // element r (key kbase + 8*(r/4) + 4*hh + r%4): scale and shift -> exp2 -> product with dP - D keep, one step
+        // apart, so that no instruction reads the result of the one before it; a pair is packed one step after its
+        // second product. 18 steps over the 12 slots behind the matrix instructions.
+        float arg[2], pv[4], ds[4];
+        auto step = [&](int k) {
+            if (k >= 1 && k <= 16) ds[(k - 1) & 3] = pv[(k - 1) & 3] * dpc[k - 1];
+            if (k < 16) {
+                pv[k & 3] = __builtin_amdgcn_exp2f(arg[k & 1]);
+                if (MASK && kbase + 8 * (k >> 2) + 4 * hh + (k & 3) > tq) pv[k & 3] = 0.0f; // key after query
+            }
+            if (k + 1 < 16) arg[(k + 1) & 1] = __builtin_fmaf(sc[k + 1], c, -l2);
+            if (k >= 3 && (k & 1)) { // elements k-3, k-2
+                uint32_t w; // two f32 -> two bf16, round to nearest even; written as an instruction so that it stays in its slot
+                asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(w) : "v"(ds[(k - 3) & 3]), "v"(ds[(k - 2) & 3]));
+                dsn[(k - 2) >> 3][((k - 2) >> 1) & 3] = w;
+            }
+        };
+#pragma unroll
+        for (int f = 0; f < DIST; f++) read_frag(f);
+        __builtin_amdgcn_sched_barrier(0);
+        arg[0] = __builtin_fmaf(sc[0], c, -l2);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 12; i++) {
+            matrix(i);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + DIST < 12) read_frag(i + DIST);
+#pragma unroll
+            for (int k = (i * 18) / 12; k < ((i + 1) * 18) / 12; k++) step(k);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // pinned here: left alone, the compiler moves the vector work down to its first use in the next iteration
+#pragma unroll
+        for (int s2 = 0; s2 < 2; s2++) asm volatile("" : "+v"(dsn[s2]));
+    };
+    const std::true_type masked;
+    const std::false_type plain;
+    int su = 0, sprev = 0; // stages of tile u and of tile u-1
+    for (int u = 0; u < NT; u++) {
+        const int snext = su + STAGE == NS * STAGE ? 0 : su + STAGE;
+        const bool diag = CAUSAL && u * TROWS + TROWS - 1 > q0w; // some key of the tile is after some query of this wave
+        if (CAUSAL && diag) sub(masked, su + 32 * 128, sprev + 32 * 128, u * TROWS, sA, dpA, sB, dpB, dsB, dsA);
+        else sub(plain, su + 32 * 128, sprev + 32 * 128, u * TROWS, sA, dpA, sB, dpB, dsB, dsA);
+        // tile u+1 must have landed, tile u-1 is no longer read: its stage takes tile u+3
+        if (u + 2 < NT) __builtin_amdgcn_s_waitcnt(0x0f70 | 4);
+        else __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        if (u + 3 < NT) stage_tile(u + 3, sprev == su ? 3 * STAGE : sprev);
+        if (CAUSAL && diag) sub(masked, snext, su, u * TROWS + 32, sB, dpB, sA, dpA, dsA, dsB);
+        else sub(plain, snext, su, u * TROWS + 32, sB, dpB, sA, dpA, dsA, dsB);
+        sprev = su;
+        su = snext;
+    }
+    // the product of the last sub-tile (second half of the last tile, stage sprev)
+#pragma unroll
+    for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+        for (int db = 0; db < 2; db++) {
+            const int base = sprev + (32 + 16 * s2) * 128;
+            dqT[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(smem, base + ft[db][0], base + ft[db][1]), __builtin_bit_cast(bf16x8, dsB[s2]), dqT[db], 0, 0, 0);
+        }
+
+    const float qs = scale * inv_keep; // dQ accumulated keep . dS
     uint16_t *dq = dqkv + ((int64_t)bb * T + tq) * ld + h * DH;
 #pragma unroll
     for (int db = 0; db < 2; db++)
 #pragma unroll
         for (int g = 0; g < 4; g++)
             *(u32x2 *)(dq + db * 32 + 8 * g + 4 * hh) =
-                pack4_trunc(dqT[db][4 * g] * scale, dqT[db][4 * g + 1] * scale, dqT[db][4 * g + 2] * scale, dqT[db][4 * g + 3] * scale);
+                pack4_trunc(dqT[db][4 * g] * qs, dqT[db][4 * g + 1] * qs, dqT[db][4 * g + 2] * qs, dqT[db][4 * g + 3] * qs);
     }
 }
 
@@ -443,7 +599,7 @@ __global__ __launch_bounds__(64) void attn_bwd_small_k(const void *__restrict__ 
 } // namespace
 
 uint64_t attention_bwd_workspace_bytes(const Attention &p) {
-    return attention_fast_path(p) ? (uint64_t)p.B * p.H * p.T * 4 : 0;
+    return attention_fast_path(p) ? 2 * (uint64_t)p.B * p.H * p.T * 4 : 0; // -D * keep and lse * log2(e)
 }
 
 hipError_t attention_bwd(const AttentionBwd &p, hipStream_t st) {
@@ -452,21 +608,21 @@ hipError_t attention_bwd(const AttentionBwd &p, hipStream_t st) {
     if (attention_fast_path(f)) {
         if (!p.workspace) return hipErrorInvalidValue;
         const int64_t rows = (int64_t)f.B * f.T * f.H;
-        float *D = (float *)p.workspace;
+        float *Dn = (float *)p.workspace, *L2 = Dn + (int64_t)f.B * f.H * f.T;
         hipLaunchKernelGGL(attn_bwd_d_k, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, st, (const uint16_t *)f.y,
-                           (const uint16_t *)p.dy, D, rows, f.T, f.H);
+                           (const uint16_t *)p.dy, f.lse, Dn, L2, rows, f.T, f.H, f.keep);
         const int nblk = f.T / 128;
         dim3 grid((unsigned)(f.B * f.H * (f.causal ? (nblk + 1) / 2 : nblk))), block(256);
         const float c = f.scale * kLog2e, ik = 1.0f / f.keep;
-#define ZK_BWD(K)                                                                                                     \
-    hipLaunchKernelGGL(K, grid, block, 0, st, (const uint16_t *)f.qkv, (const uint16_t *)p.dy, f.lse, D, (uint16_t *)p.dqkv, \
+#define ZK_BWD(K, LSE, DD)                                                                                            \
+    hipLaunchKernelGGL(K, grid, block, 0, st, (const uint16_t *)f.qkv, (const uint16_t *)p.dy, LSE, DD, (uint16_t *)p.dqkv, \
                        f.T, f.H, c, f.scale, ik)
         if (f.causal) {
-            ZK_BWD(attn_bwd_dkv_k<true>);
-            ZK_BWD(attn_bwd_dq_k<true>);
+            ZK_BWD(attn_bwd_dkv_k<true>, L2, Dn);
+            ZK_BWD(attn_bwd_dq_k<true>, L2, Dn);
         } else {
-            ZK_BWD(attn_bwd_dkv_k<false>);
-            ZK_BWD(attn_bwd_dq_k<false>);
+            ZK_BWD(attn_bwd_dkv_k<false>, L2, Dn);
+            ZK_BWD(attn_bwd_dq_k<false>, L2, Dn);
         }
 #undef ZK_BWD
         return hipGetLastError();
