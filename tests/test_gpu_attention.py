@@ -3,8 +3,9 @@ reference's goldens (zyx/tests/05_misc.rs:1073-1163, zyx-nn/src/causal_self_atte
 
 Tolerances: f32 storage 1e-5 relative to max(|y|, sum_j p_j |v_j|) =: mag. bf16 storage: 1e-3 * mag (north star
 for f32-accumulated bf16 matrix products) + 2^-9 * mag (the probabilities enter att.dot(v) as bf16 values, as the
-reference's bf16 `att` tensor does; round-to-nearest moves each by at most half a bf16 ulp) + 2^-7 * |y| (the
-truncating bf16 store of y)."""
+reference's bf16 `att` tensor does; round-to-nearest moves each by at most half a bf16 ulp, which is 2^-8 relative in
+the worst case and averages below 2^-9 over rows of many comparable terms: the test whose rows are carried by a few
+keys uses 2^-8) + 2^-7 * |y| (the truncating bf16 store of y)."""
 import numpy as np
 import pytest
 
@@ -94,6 +95,30 @@ def test_structured_inputs_bf16(hip, oracle):
     q = np.full((b, t, h * dh), 2.0, np.float32)  # score of key 77: 64*32/8 = 256, others 0
     y = oracle.bf16_to_f32(attention(dev, pool, oracle.f32_to_bf16(np.concatenate([q, k, v], 2)), h))
     assert np.array_equal(y, np.broadcast_to(v[:, 77:78, :], v.shape))
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(1, 512, 2, 64), (8, 256, 64, 64)])  # 32 and 64 queries per wave
+def test_scores_that_keep_growing_bf16(hip, oracle, shape, causal):
+    """Scores rise by ~37 (in powers of two) from one block of 32 keys to the next, so the reference point of the
+    running exponentials has to move several times inside a row, and every probability but the last few underflows."""
+    dev, pool = hip
+    b, t, h, dh = shape
+    rng = np.random.default_rng(t + h)
+    q = (1.0 + 0.1 * rng.standard_normal((b, t, h * dh))).astype(np.float32)
+    k = np.broadcast_to((0.1 * np.arange(t, dtype=np.float32))[None, :, None], (b, t, h * dh))
+    v = rng.standard_normal((b, t, h * dh)).astype(np.float32)
+    # packed layout [B, T, 3, H, dh]
+    qkv = oracle.f32_to_bf16(np.stack([q.reshape(b, t, h, dh), k.reshape(b, t, h, dh), v.reshape(b, t, h, dh)], 2).reshape(b, t, 3 * h * dh))
+    y, lse = attention(dev, pool, qkv, h, DType.BF16, want_lse=True, causal=causal)
+    want, mag, lse64 = sdpa64(oracle.bf16_to_f32(qkv), h, causal=causal)
+    got = oracle.bf16_to_f32(y).astype(np.float64)
+    assert np.all(np.isfinite(got)) and np.all(np.isfinite(lse))
+    # a handful of keys carry each row here, so the roundings of their probabilities to bf16 do not average out: the
+    # bar is the worst case of round-to-nearest on 8 significant bits, 2^-8 * mag, instead of the 2^-9 that rows of
+    # many comparable terms are held to
+    assert np.all(np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + (1e-3 + 2.0 ** -8) * mag)
+    assert np.allclose(lse, lse64, rtol=1e-4, atol=1e-4)
 
 
 def test_config5_attention_full_size(hip, oracle):

@@ -36,7 +36,7 @@ constexpr int TILE = KB * DH * 2;   // one K or V tile: 8 KiB
 constexpr int STAGE = 2 * TILE;     // K tile then V tile
 constexpr int NSTAGE = 2;           // tiles kt+1 and kt+2 are on their way while tile kt is multiplied
 constexpr float kLog2e = 1.44269504088896340736f, kLn2 = 0.69314718055994530942f;
-constexpr float kSlack = 8.0f;
+constexpr float kBig = 1.8446744e19f; // 2^64: a block's sum of exponentials beyond this moves the query's reference point
 
 // K tile: [key][16-byte chunk ^ ((key >> 1) & 7)], 128-byte rows: ds_read_b128 of 16 consecutive keys
 // at one logical chunk touches 16 different slots modulo 256 bytes.
@@ -182,58 +182,69 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
             }
         }
 
-        float m_new[QW];
-        bool moved = false;
+        if (CAUSAL) {
 #pragma unroll
-        for (int b = 0; b < QW; b++) {
-            if (CAUSAL && kt * KB + KB - 1 > q0w + 32 * b) { // register r of block kb is key kb*32 + 8*(r/4) + 4*hh + r%4 of the tile
+            for (int b = 0; b < QW; b++)
+                if (kt * KB + KB - 1 > q0w + 32 * b) { // register r of block kb is key kb*32 + 8*(r/4) + 4*hh + r%4 of the tile
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++)
+                    for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        if (kt * KB + kb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3) > tq0 + 32 * b) s[b][kb][r] = -INFINITY;
-            }
-            float bm = s[b][0][0];
-#pragma unroll
-            for (int r = 1; r < 16; r++) bm = fmaxf(bm, s[b][0][r]);
-#pragma unroll
-            for (int r = 0; r < 16; r++) bm = fmaxf(bm, s[b][1][r]);
-            bm = fmaxf(bm, xor32(bm));
-            // The reference point m of a query's exponentials follows its running maximum only in steps of more than
-            // kSlack (in log2 units): exponentials may then reach 2^kSlack instead of 1, which f32 sums and bf16
-            // products carry at the same relative precision, and the accumulators are rescaled when a query makes such
-            // a step (the first tile it sees, then rarely) instead of whenever any of the wave's maxima moves (nearly
-            // every tile). A block of a causal tile that lies wholly after its queries has bm = -inf and changes nothing.
-            m_new[b] = bm * c > m[b] + kSlack ? bm * c : m[b];
-            moved |= m_new[b] != m[b];
-        }
-        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
-#pragma unroll
-            for (int b = 0; b < QW; b++) {
-                const float alpha = m[b] == m_new[b] ? 1.0f : __builtin_amdgcn_exp2f(m[b] - m_new[b]);
-#pragma unroll
-                for (int db = 0; db < 2; db++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) o[b][db][r] *= alpha;
-                l[b] *= alpha;
-                m[b] = m_new[b];
-            }
+                        for (int r = 0; r < 16; r++)
+                            if (kt * KB + kb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3) > tq0 + 32 * b) s[b][kb][r] = -INFINITY;
+                }
         }
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) { // exponentiate one 32-key block, feed it to the matrix pipe, then the next
+            // The exponentials are taken against the reference point m the query already has, and checked afterwards:
+            // f32 sums and bf16 products carry 2^60 at the same relative precision as 1, so m only has to move when a
+            // block's sum leaves that range (or is not a number: the first block of a query, whose m is -inf). Only then
+            // is the block's maximum computed, the accumulators rescaled and the block exponentiated again; a query
+            // usually sets m once, from the first block it sees, instead of computing a maximum for every block.
+            float lt[QW];
+            f32x8 p[QW][2];
+            auto exponentiate = [&]() {
+#pragma unroll
+                for (int b = 0; b < QW; b++) {
+                    lt[b] = 0.0f;
+#pragma unroll
+                    for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            p[b][s2][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[b][kb][8 * s2 + e], c, -m[b]));
+                            lt[b] += p[b][s2][e];
+                        }
+                }
+            };
+            exponentiate();
+            bool redo = false;
+#pragma unroll
+            for (int b = 0; b < QW; b++) redo |= !(lt[b] < kBig);
+            if (__builtin_amdgcn_ballot_w64(redo) != 0) {
+#pragma unroll
+                for (int b = 0; b < QW; b++) {
+                    float bm = s[b][kb][0];
+#pragma unroll
+                    for (int r = 1; r < 16; r++) bm = fmaxf(bm, s[b][kb][r]);
+                    bm = fmaxf(bm, xor32(bm));
+                    // a block that lies wholly after its queries (causal) has bm = -inf and changes nothing
+                    const float m_new = fmaxf(m[b], bm * c);
+                    const float alpha = m[b] == m_new ? 1.0f : __builtin_amdgcn_exp2f(m[b] - m_new);
+#pragma unroll
+                    for (int db = 0; db < 2; db++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) o[b][db][r] *= alpha;
+                    l[b] *= alpha;
+                    m[b] = m_new;
+                }
+                exponentiate();
+            }
             bf16x8 pf[QW][2];
 #pragma unroll
-            for (int b = 0; b < QW; b++)
+            for (int b = 0; b < QW; b++) {
+                l[b] += lt[b];
 #pragma unroll
-                for (int s2 = 0; s2 < 2; s2++) {
-                    f32x8 p;
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[b][kb][8 * s2 + e], c, -m[b]));
-                        l[b] += p[e];
-                    }
-                    pf[b][s2] = __builtin_convertvector(p, bf16x8);
-                }
+                for (int s2 = 0; s2 < 2; s2++) pf[b][s2] = __builtin_convertvector(p[b][s2], bf16x8);
+            }
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++)
 #pragma unroll
