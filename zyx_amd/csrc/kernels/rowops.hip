@@ -48,6 +48,50 @@ template <> struct RowIO<1> {
         *(uint2 *)(p + i) = make_uint2((__float_as_uint(v[0]) >> 16) | (__float_as_uint(v[1]) & 0xffff0000u),
                                        (__float_as_uint(v[2]) >> 16) | (__float_as_uint(v[3]) & 0xffff0000u));
     }
+    // 8 consecutive elements, one 16-byte access
+    static __device__ __forceinline__ void ld8(const uint16_t *p, int64_t i, float (&a)[4], float (&b)[4]) {
+        const uint4 t = *(const uint4 *)(p + i);
+        a[0] = __uint_as_float(t.x << 16); a[1] = __uint_as_float(t.x & 0xffff0000u);
+        a[2] = __uint_as_float(t.y << 16); a[3] = __uint_as_float(t.y & 0xffff0000u);
+        b[0] = __uint_as_float(t.z << 16); b[1] = __uint_as_float(t.z & 0xffff0000u);
+        b[2] = __uint_as_float(t.w << 16); b[3] = __uint_as_float(t.w & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void st8(uint16_t *p, int64_t i, const float (&a)[4], const float (&b)[4]) {
+        *(uint4 *)(p + i) = make_uint4((__float_as_uint(a[0]) >> 16) | (__float_as_uint(a[1]) & 0xffff0000u),
+                                       (__float_as_uint(a[2]) >> 16) | (__float_as_uint(a[3]) & 0xffff0000u),
+                                       (__float_as_uint(b[0]) >> 16) | (__float_as_uint(b[1]) & 0xffff0000u),
+                                       (__float_as_uint(b[2]) >> 16) | (__float_as_uint(b[3]) & 0xffff0000u));
+    }
+};
+
+// A row of 256*NV columns held by one wave as NV vectors of 4 values per lane. f32, or an odd NV: vector j of a lane is
+// columns (lane + 64*j)*4 .. +3. bf16 with an even NV: vectors 2q and 2q+1 are the two halves of the 8 columns
+// (lane + 64*q)*8 .. +7, moved as one 16-byte access (the memory pipeline takes a vector instruction in about the same
+// time whatever its width). Every access of the wave covers consecutive bytes either way.
+template <int DT, int NV> struct RegRow {
+    typedef RowIO<DT> IO;
+    typedef typename IO::S S;
+    static constexpr bool WIDE = DT == 1 && NV % 2 == 0;
+    static __device__ __forceinline__ int col(int lane, int j) { return WIDE ? (lane + 64 * (j >> 1)) * 8 + (j & 1) * 4 : (lane + 64 * j) * 4; }
+    static __device__ __forceinline__ void load(const S *p, int lane, float (&v)[NV][4]) {
+        if constexpr (WIDE) {
+#pragma unroll
+            for (int q = 0; q < NV / 2; q++) IO::ld8(p, (lane + 64 * q) * 8, v[2 * q], v[2 * q + 1]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NV; j++) IO::ld4(p, (lane + 64 * j) * 4, v[j]);
+        }
+    }
+    // vectors j0 (and j0 + 1 when WIDE; j0 even then)
+    static __device__ __forceinline__ void load_at(const S *p, int lane, int j0, float (&a)[4], float (&b)[4]) {
+        if constexpr (WIDE) IO::ld8(p, (lane + 64 * (j0 >> 1)) * 8, a, b);
+        else IO::ld4(p, (lane + 64 * j0) * 4, a);
+    }
+    static __device__ __forceinline__ void store_at(S *p, int lane, int j0, const float (&a)[4], const float (&b)[4]) {
+        if constexpr (WIDE) IO::st8(p, (lane + 64 * (j0 >> 1)) * 8, a, b);
+        else IO::st4(p, (lane + 64 * j0) * 4, a);
+    }
+    static constexpr int STEP = WIDE ? 2 : 1; // vectors per access
 };
 
 // sum over one row of f(x[c]) with lanes striding over columns
@@ -122,9 +166,9 @@ __global__ __launch_bounds__(256) void norm_rows_reg_k(const typename RowIO<DT>:
     if (row >= rows) return;
     const typename IO::S *xr = x + row * cols;
     typename IO::S *yr = y + row * cols;
+    typedef RegRow<DT, NV> RR;
     float v[NV][4];
-#pragma unroll
-    for (int j = 0; j < NV; j++) IO::ld4(xr, (lane + 64 * j) * 4, v[j]);
+    RR::load(xr, lane, v);
     float mean = 0.0f, scale;
     if (MODE == 0) {
         float s = 0.0f;
@@ -146,24 +190,28 @@ __global__ __launch_bounds__(256) void norm_rows_reg_k(const typename RowIO<DT>:
         scale = sqrtf(1.0f / (wave_allreduce_f32(q, OpAdd()) / (float)cols + eps));
     }
 #pragma unroll
-    for (int j = 0; j < NV; j++) {
-        const int c = (lane + 64 * j) * 4;
-        float wv[4] = {1.0f, 1.0f, 1.0f, 1.0f}, bv[4] = {0.0f, 0.0f, 0.0f, 0.0f}, o[4];
-        if (w) IO::ld4(w, c, wv);
-        if (b) IO::ld4(b, c, bv);
+    for (int j0 = 0; j0 < NV; j0 += RR::STEP) {
+        float o[2][4];
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            o[k] = MODE == 0 ? (v[j][k] - mean) * scale : v[j][k] * scale;
-            if (w) o[k] *= wv[k];
-            if (b) o[k] += bv[k];
+        for (int h = 0; h < RR::STEP; h++) {
+            const int j = j0 + h, c = RR::col(lane, j);
+            float wv[4] = {1.0f, 1.0f, 1.0f, 1.0f}, bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (w) IO::ld4(w, c, wv);
+            if (b) IO::ld4(b, c, bv);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                o[h][k] = MODE == 0 ? (v[j][k] - mean) * scale : v[j][k] * scale;
+                if (w) o[h][k] *= wv[k];
+                if (b) o[h][k] += bv[k];
+            }
         }
-        IO::st4(yr, c, o);
+        RR::store_at(yr, lane, j0, o[0], o[1]);
     }
 }
 
 // dx for rows of 256*NV columns with x and dy held in registers (one read of each), and the parameter gradients in
 // the same pass: a workgroup of WAVES waves walks rows blockIdx*WAVES + wave, + gridDim*WAVES, ..., every lane keeps
-// running sums of dy*xh and dy for its 4*NV columns, the waves of a workgroup fold theirs through LDS in wave order
+// running sums of dy*xh and dy for its 4*NV columns, the waves of a workgroup add theirs up through LDS in wave order
 // and the workgroup leaves one partial row pair in part[(blockIdx*2 + {0,1})*cols + c] for norm_bwd_param_sum_k.
 // The order of every sum is fixed by the launch shape: results are reproducible. part may be null (no dw / db).
 template <int DT, int MODE, int NV, int WAVES>
@@ -174,8 +222,9 @@ __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename R
                                                                 typename RowIO<DT>::S *__restrict__ dx, float *__restrict__ part,
                                                                 int64_t rows, float eps) {
     typedef RowIO<DT> IO;
+    typedef RegRow<DT, NV> RR;
     constexpr int cols = 256 * NV;
-    __shared__ float fold[2][cols];
+    __shared__ float fold[WAVES][2][cols]; // 128 KiB at most (16 waves x 1024 columns, 8 waves x 2048)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float pw[NV][4], pb[NV][4];
 #pragma unroll
@@ -187,11 +236,8 @@ __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename R
     for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < rows; row += (int64_t)gridDim.x * WAVES) {
         const int64_t base = row * cols;
         float xv[NV][4], g[NV][4];
-#pragma unroll
-        for (int j = 0; j < NV; j++) {
-            IO::ld4(x + base, (lane + 64 * j) * 4, xv[j]);
-            IO::ld4(dy + base, (lane + 64 * j) * 4, g[j]);
-        }
+        RR::load(x + base, lane, xv);
+        RR::load(dy + base, lane, g);
         float mean = 0.0f, rstd;
         if (MODE == 0) {
             float s = 0.0f;
@@ -216,7 +262,7 @@ __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename R
 #pragma unroll
         for (int j = 0; j < NV; j++) {
             float wv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-            if (w) IO::ld4(w, (lane + 64 * j) * 4, wv); // L1 / L2 hit: every row reads the same 4*NV values
+            if (w) IO::ld4(w, RR::col(lane, j), wv); // L1 / L2 hit: every row reads the same 4*NV values
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 const float xh = (xv[j][k] - mean) * rstd; // mean is 0 for RMSNorm
@@ -231,33 +277,37 @@ __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename R
         s2 = wave_allreduce_f32(s2, OpAdd());
         const float k1 = s1 / (float)cols, k2 = MODE == 0 ? s2 / (float)(cols - 1) : rstd * rstd * rstd * s2 / (float)cols;
 #pragma unroll
-        for (int j = 0; j < NV; j++) {
-            const int c = (lane + 64 * j) * 4;
-            float o[4], av[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (add) IO::ld4(add + base, c, av);
+        for (int j0 = 0; j0 < NV; j0 += RR::STEP) {
+            float o[2][4], av[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+            if (add) RR::load_at(add + base, lane, j0, av[0], av[1]);
 #pragma unroll
-            for (int k = 0; k < 4; k++)
-                o[k] = (MODE == 0 ? rstd * ((g[j][k] - k1) - ((xv[j][k] - mean) * rstd) * k2) : rstd * g[j][k] - xv[j][k] * k2) + av[k];
-            IO::st4(dx + base, c, o);
+            for (int h = 0; h < RR::STEP; h++)
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const int j = j0 + h;
+                    o[h][k] = (MODE == 0 ? rstd * ((g[j][k] - k1) - ((xv[j][k] - mean) * rstd) * k2) : rstd * g[j][k] - xv[j][k] * k2) + av[h][k];
+                }
+            RR::store_at(dx + base, lane, j0, o[0], o[1]);
         }
     }
     if (!part) return; // uniform over the workgroup
-    for (int v = 0; v < WAVES; v++) {
-        if (wave == v) {
+    // every wave lays its sums down, then a thread adds a column's WAVES values in wave order
 #pragma unroll
-            for (int j = 0; j < NV; j++)
-#pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const int c = (lane + 64 * j) * 4 + k;
-                    fold[0][c] = v == 0 ? pw[j][k] : fold[0][c] + pw[j][k];
-                    fold[1][c] = v == 0 ? pb[j][k] : fold[1][c] + pb[j][k];
-                }
-        }
-        __syncthreads();
+    for (int j = 0; j < NV; j++) {
+        const int c = RR::col(lane, j);
+        *(f32x4 *)&fold[wave][0][c] = f32x4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]};
+        *(f32x4 *)&fold[wave][1][c] = f32x4{pb[j][0], pb[j][1], pb[j][2], pb[j][3]};
     }
+    __syncthreads();
     for (int c = threadIdx.x; c < cols; c += WAVES * 64) {
-        part[((int64_t)blockIdx.x * 2) * cols + c] = fold[0][c];
-        part[((int64_t)blockIdx.x * 2 + 1) * cols + c] = fold[1][c];
+        float a = fold[0][0][c], b = fold[0][1][c];
+#pragma unroll
+        for (int v = 1; v < WAVES; v++) {
+            a += fold[v][0][c];
+            b += fold[v][1][c];
+        }
+        part[((int64_t)blockIdx.x * 2) * cols + c] = a;
+        part[((int64_t)blockIdx.x * 2 + 1) * cols + c] = b;
     }
 }
 
