@@ -8,15 +8,15 @@
 //   dQ = scale dS . k,   dK = scale dS^T . q
 // Ps is recomputed from the saved lse = ln sum exp(scale q k^T) instead of being stored.
 //
-// Matrix-core path (bf16, dh = 64, T % 128 == 0), three launches:
-//   attn_bwd_d_k    -D keep [B,H,T] and lse log2(e) into the program's workspace;
-//   attn_bwd_dkv_k  one workgroup per (batch, head, 128 keys), a wave owns 32 keys and streams query
+// Matrix-core path (bf16, dh = 64, T % 128 == 0), two launches:
+//   attn_bwd_dkv_k  (second) one workgroup per (batch, head, 128 keys), a wave owns 32 keys and streams query
 //                   tiles; S = Q.K^T is formed queries x keys so that a lane owns a key column and the
 //                   exponentiated / differentiated tiles, packed to bf16, are the B operands of
 //                   dV^T += dy^T.P and dK^T += Q^T.dS (dy^T and Q^T come through the transposing LDS read);
 //                   the three steps of a 32-query sub-tile run in three consecutive iterations (software pipeline);
-//   attn_bwd_dq_k   one workgroup per (batch, head, 128 queries), S^T = K.Q^T keys x queries (a lane owns
-//                   a query, lse and D are per-lane scalars), dQ^T += K^T.dS^T.
+//   attn_bwd_dq_k   (first) one workgroup per (batch, head, 128 queries), S^T = K.Q^T keys x queries (a lane owns
+//                   a query, lse and D are per-lane scalars), dQ^T += K^T.dS^T; leaves -D keep and lse log2(e) of its
+//                   queries in the program's workspace;
 // No atomics: every output element has one owner, results are reproducible.
 //
 // attn_bwd_small_*: any dh <= 256 and T, f32 or bf16 storage, f32 arithmetic, one wave per query / key.
@@ -31,33 +31,6 @@ using namespace attn;
 namespace {
 
 constexpr int STAGE_BWD = 2 * TILE + 512; // two tiles + lse*log2(e) [64] + D [64]
-
-// D[bh, t] = sum_d dy[b,t,h,d] * y[b,t,h,d], 8 lanes per row of 64, stored as Dn = -D * keep; and lse2 = lse * log2(e).
-__global__ __launch_bounds__(256) void attn_bwd_d_k(const uint16_t *__restrict__ y, const uint16_t *__restrict__ dy,
-                                                    const float *__restrict__ lse, float *__restrict__ Dn,
-                                                    float *__restrict__ lse2, int64_t rows, int T, int H, float keep) {
-    // rows are taken in the order of the results, o = (b*H + h)*T + t: eight lanes read the 128 bytes of row
-    // (b*T + t)*H + h of y and dy, and the three results of 32 consecutive t leave as whole cache lines
-    const int64_t o = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3);
-    const int part = threadIdx.x & 7;
-    float a = 0.0f;
-    if (o < rows) {
-        const int64_t bhh = o / T, t = o % T, b = bhh / H, h = bhh % H, row = (b * T + t) * H + h;
-        const u32x4 u = *(const u32x4 *)(y + row * DH + part * 8), v = *(const u32x4 *)(dy + row * DH + part * 8);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            a = __builtin_fmaf(__uint_as_float(u[i] << 16), __uint_as_float(v[i] << 16), a);
-            a = __builtin_fmaf(__uint_as_float(u[i] & 0xffff0000u), __uint_as_float(v[i] & 0xffff0000u), a);
-        }
-    }
-    a += dpp_f32<kDppQuadXor1>(a);
-    a += dpp_f32<kDppQuadXor2>(a);
-    a += dpp_f32<kDppRowHalfMirror>(a);
-    if (o < rows && part == 0) {
-        Dn[o] = -a * keep; // what the dP accumulators start from: dP - D keep = keep (dP / keep - D)
-        lse2[o] = lse[o] * kLog2e; // the exponent the kernels subtract, in exp2 units
-    }
-}
 
 // 64 lanes x 16 (or 4) bytes from global memory straight into LDS at `lds` (wave-uniform byte address) + 16 (4) * lane.
 // Written as instructions, not through the compiler's builtin: for the builtin the compiler waits for every such
@@ -315,8 +288,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restr
 // sub-tile j-1 (12 matrix instructions) between the vector work of sub-tile j. A lane owns a query: its lse log2(e) and
 // -D keep are scalars, and the dP^T accumulators start at -D keep.
 template <bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ dy,
-                                                        const float *__restrict__ lse2, const float *__restrict__ Dn,
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ y,
+                                                        const uint16_t *__restrict__ dy, const float *__restrict__ lse,
+                                                        float *__restrict__ lse2, float *__restrict__ Dn,
                                                         uint16_t *__restrict__ dqkv, int T, int H, float c, float scale,
                                                         float inv_keep) {
     constexpr int NS = 4, STAGE = 2 * TILE; // K tile then V tile
@@ -345,7 +319,25 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restri
         qfr[ks] = *(const bf16x8 *)(qp + (int64_t)tq * ld + ks * 16 + hh * 8);
         dofr[ks] = *(const bf16x8 *)(dy + ((int64_t)bb * T + tq) * C + h * DH + ks * 16 + hh * 8);
     }
-    const float l2 = lse2[(int64_t)bh * T + tq], dn = Dn[(int64_t)bh * T + tq];
+    // D = sum_d dy o y of this lane's query (each half-wave holds half of the row), kept as -D keep; with lse log2(e) it
+    // also goes to the workspace, where the dK / dV kernel (launched after this one) reads both
+    float dsum = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+        const u32x4 o = *(const u32x4 *)(y + ((int64_t)bb * T + tq) * C + h * DH + ks * 16 + hh * 8);
+        const u32x4 g = __builtin_bit_cast(u32x4, dofr[ks]);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            dsum = __builtin_fmaf(__uint_as_float(o[i] << 16), __uint_as_float(g[i] << 16), dsum);
+            dsum = __builtin_fmaf(__uint_as_float(o[i] & 0xffff0000u), __uint_as_float(g[i] & 0xffff0000u), dsum);
+        }
+    }
+    dsum += xor32(dsum);
+    const float l2 = lse[(int64_t)bh * T + tq] * kLog2e, dn = -dsum / inv_keep;
+    if (hh == 0) {
+        lse2[(int64_t)bh * T + tq] = l2;
+        Dn[(int64_t)bh * T + tq] = dn;
+    }
     f32x16 dstart;
 #pragma unroll
     for (int r = 0; r < 16; r++) dstart[r] = dn;
@@ -607,23 +599,25 @@ hipError_t attention_bwd(const AttentionBwd &p, hipStream_t st) {
     if (f.B <= 0 || f.T <= 0 || f.H <= 0 || f.dh <= 0) return hipSuccess;
     if (attention_fast_path(f)) {
         if (!p.workspace) return hipErrorInvalidValue;
-        const int64_t rows = (int64_t)f.B * f.T * f.H;
         float *Dn = (float *)p.workspace, *L2 = Dn + (int64_t)f.B * f.H * f.T;
-        hipLaunchKernelGGL(attn_bwd_d_k, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, st, (const uint16_t *)f.y,
-                           (const uint16_t *)p.dy, f.lse, Dn, L2, rows, f.T, f.H, f.keep);
         const int nblk = f.T / 128;
         dim3 grid((unsigned)(f.B * f.H * (f.causal ? (nblk + 1) / 2 : nblk))), block(256);
         const float c = f.scale * kLog2e, ik = 1.0f / f.keep;
-#define ZK_BWD(K, LSE, DD)                                                                                            \
-    hipLaunchKernelGGL(K, grid, block, 0, st, (const uint16_t *)f.qkv, (const uint16_t *)p.dy, LSE, DD, (uint16_t *)p.dqkv, \
-                       f.T, f.H, c, f.scale, ik)
+        // the dQ kernel also leaves -D keep and lse log2(e) of its rows in the workspace for the dK / dV kernel
+#define ZK_BWD_DQ(K)                                                                                                  \
+    hipLaunchKernelGGL(K, grid, block, 0, st, (const uint16_t *)f.qkv, (const uint16_t *)f.y, (const uint16_t *)p.dy, f.lse, L2, Dn, \
+                       (uint16_t *)p.dqkv, f.T, f.H, c, f.scale, ik)
+#define ZK_BWD(K)                                                                                                     \
+    hipLaunchKernelGGL(K, grid, block, 0, st, (const uint16_t *)f.qkv, (const uint16_t *)p.dy, L2, Dn, (uint16_t *)p.dqkv, f.T, \
+                       f.H, c, f.scale, ik)
         if (f.causal) {
-            ZK_BWD(attn_bwd_dkv_k<true>, L2, Dn);
-            ZK_BWD(attn_bwd_dq_k<true>, L2, Dn);
+            ZK_BWD_DQ(attn_bwd_dq_k<true>);
+            ZK_BWD(attn_bwd_dkv_k<true>);
         } else {
-            ZK_BWD(attn_bwd_dkv_k<false>, L2, Dn);
-            ZK_BWD(attn_bwd_dq_k<false>, L2, Dn);
+            ZK_BWD_DQ(attn_bwd_dq_k<false>);
+            ZK_BWD(attn_bwd_dkv_k<false>);
         }
+#undef ZK_BWD_DQ
 #undef ZK_BWD
         return hipGetLastError();
     }
