@@ -75,25 +75,23 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
 
     // Workgroups whose ids are congruent mod 8 share an XCD (and its L2): give every XCD whole heads, so
     // the K and V of a head are fetched into one L2 only.
-    const int QT = T / QBW, NB = CAUSAL ? (QT + 1) / 2 : QT, BH = (int)gridDim.x / NB; // NB blocks of the grid per head
+    const int QT = T / QBW, BH = (int)gridDim.x / QT; // QT blocks of the grid per head
     int bh, qt;
-    if (BH % 8 == 0) {
+    if (CAUSAL) {
+        // causal work grows with the query block: the blocks with the most key tiles come first in the grid, so that
+        // short workgroups fill in behind long ones (ids congruent mod 8 still share a head's XCD when the number of
+        // heads is a multiple of 8)
+        bh = blockIdx.x % BH;
+        qt = QT - 1 - blockIdx.x / BH;
+    } else if (BH % 8 == 0) {
         const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
-        bh = (i / NB) * 8 + x;
-        qt = i % NB;
+        bh = (i / QT) * 8 + x;
+        qt = i % QT;
     } else {
-        bh = blockIdx.x / NB;
-        qt = blockIdx.x % NB;
+        bh = blockIdx.x / QT;
+        qt = blockIdx.x % QT;
     }
-    // Causal work grows with qt: a workgroup takes the query blocks qt and QT-1-qt one after the other, so every
-    // workgroup streams the same number of key tiles whatever CU it lands on.
-    const int qt_first = qt;
-#pragma nounroll
-    for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
-    if (CAUSAL && pass) {
-        qt = QT - 1 - qt_first;
-        if (qt == qt_first) break; // odd QT: the middle block has no partner
-    }
+    {
     const int bb = bh / H, h = bh % H;
     const int64_t ld = 3 * (int64_t)H * DH;
     const uint16_t *qp = qkv + (int64_t)bb * T * ld + h * DH, *kp = qp + H * DH, *vp = kp + H * DH;
@@ -359,7 +357,7 @@ hipError_t attention_fwd(const Attention &p, hipStream_t st) {
         // 64 queries per wave where the sequence divides into such workgroups and they still fill the device twice
         const bool wide = !p.causal && p.T % (2 * QB) == 0 && (int64_t)p.B * p.H * (p.T / (2 * QB)) >= 512;
         const int qblocks = p.T / (wide ? 2 * QB : QB);
-        dim3 grid((unsigned)(p.B * p.H * (p.causal ? (qblocks + 1) / 2 : qblocks))), block(256);
+        dim3 grid((unsigned)(p.B * p.H * qblocks)), block(256);
 #define ZK_ATTN(L, CA)                                                                                                \
     do {                                                                                                              \
         if (wide)                                                                                                     \

@@ -63,15 +63,17 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_k(const uint16_t *__restr
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
     int bh, kblk;
     const int nblk = T / 128;
-    head_and_block(CAUSAL ? (nblk + 1) / 2 : nblk, bh, kblk);
-    const int blk_first = kblk;
-#pragma nounroll
-    for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
-    if (CAUSAL && pass) {
-        kblk = nblk - 1 - blk_first;
-        if (kblk == blk_first) break;
-        __syncthreads(); // the first block's last tile has been read by every wave
-    }
+    // CAUSAL: pairs with key > query carry probability 0; tiles that hold only such pairs are not visited (the loop
+    // bounds), and the tiles the diagonal crosses zero the masked probabilities, which zeroes dS too. The number of tiles
+    // then depends on the block: the blocks with the most tiles (here: the first keys) come first in the grid, so that
+    // short workgroups fill in behind long ones. Ids congruent mod 8 still share a head (and its XCD's L2) when the number
+    // of heads is a multiple of 8.
+    if (CAUSAL) {
+        const int BH = (int)gridDim.x / nblk;
+        bh = blockIdx.x % BH;
+        kblk = blockIdx.x / BH;
+    } else head_and_block(nblk, bh, kblk);
+    {
     const int bb = bh / H, h = bh % H;
     const int64_t C = (int64_t)H * DH, ld = 3 * C;
     const uint16_t *qp = qkv + (int64_t)bb * T * ld + h * DH, *kp = qp + C, *vp = kp + C;
@@ -299,15 +301,12 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_k(const uint16_t *__restri
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hh = lane >> 5;
     int bh, qblk;
     const int nblk = T / 128;
-    head_and_block(CAUSAL ? (nblk + 1) / 2 : nblk, bh, qblk);
-    const int blk_first = qblk;
-#pragma nounroll
-    for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
-    if (CAUSAL && pass) {
-        qblk = nblk - 1 - blk_first;
-        if (qblk == blk_first) break;
-        __syncthreads(); // the first block's last tile has been read by every wave
-    }
+    if (CAUSAL) { // as in the dK / dV kernel: the last queries (most key tiles) first
+        const int BH = (int)gridDim.x / nblk;
+        bh = blockIdx.x % BH;
+        qblk = nblk - 1 - blockIdx.x / BH;
+    } else head_and_block(nblk, bh, qblk);
+    {
     const int bb = bh / H, h = bh % H;
     const int64_t C = (int64_t)H * DH, ld = 3 * C;
     const uint16_t *qp = qkv + (int64_t)bb * T * ld + h * DH, *kp = qp + C, *vp = kp + C;
@@ -601,7 +600,7 @@ hipError_t attention_bwd(const AttentionBwd &p, hipStream_t st) {
         if (!p.workspace) return hipErrorInvalidValue;
         float *Dn = (float *)p.workspace, *L2 = Dn + (int64_t)f.B * f.H * f.T;
         const int nblk = f.T / 128;
-        dim3 grid((unsigned)(f.B * f.H * (f.causal ? (nblk + 1) / 2 : nblk))), block(256);
+        dim3 grid((unsigned)(f.B * f.H * nblk)), block(256);
         const float c = f.scale * kLog2e, ik = 1.0f / f.keep;
         // the dQ kernel also leaves -D keep and lse log2(e) of its rows in the workspace for the dK / dV kernel
 #define ZK_BWD_DQ(K)                                                                                                  \
