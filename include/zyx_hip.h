@@ -104,7 +104,9 @@ typedef struct zhip_device_info {
 enum zhip_kernel_kind {
     /* x[rows,cols] -> y = softmax(x, -1), rowsum = y.sum(-1), arg = y.argmax_axis(-1).
      * dims = {rows, cols}; flags selects outputs (ZHIP_SOFTMAX_*); args: x, then the
-     * selected outputs in the order y, rowsum, arg.
+     * selected outputs in the order y, rowsum, arg. dtype ZHIP_F32, ZHIP_BF16 or ZHIP_F16 (x, y, rowsum; arg is
+     * i32): 16-bit elements widen to f32 registers, y is truncated on store, and the sum and argmax read the stored
+     * y, as the C backend's kernels do (zyx/src/codegen/c.rs:456-497).
      * zyx/src/tensor/mod.rs:1457-1461, 2245-2269; zyx/src/tensor/reduce_ops.rs:197-199 */
     ZHIP_K_SOFTMAX_ROWS = 1,
     /* Fused elementwise chain over a [rows, cols] view (dims = {rows, cols}): up to 4

@@ -170,8 +170,17 @@ def reduce_rows_i32(op: str, x: np.ndarray) -> np.ndarray:
     return y
 
 
-def softmax_rows(x: np.ndarray, want_y=True, want_sum=True, want_arg=True):
-    """Returns (y, rowsum, argmax) of the reference's softmax -> sum / argmax_axis(-1) chain."""
+def softmax_rows(x: np.ndarray, want_y=True, want_sum=True, want_arg=True, dtype: int = F32):
+    """Returns (y, rowsum, argmax) of the reference's softmax -> sum / argmax_axis(-1) chain. dtype BF16 / F16: x, y and
+    rowsum are bit patterns (uint16); y is narrowed on store and the sum and argmax read the stored y."""
+    if dtype != F32:
+        x = np.ascontiguousarray(x, np.uint16)
+        rows, cols = x.shape
+        y = np.empty_like(x) if want_y else None
+        s = np.empty(rows, np.uint16) if want_sum else None
+        a = np.empty(rows, np.int32) if want_arg else None
+        lib().zo_softmax_rows(dtype, _p(x), _p(y), _p(s), _p(a), _I64(rows), _I64(cols))
+        return y, s, a
     x = np.ascontiguousarray(x, np.float32)
     rows, cols = x.shape
     y = np.empty_like(x) if want_y else None

@@ -361,6 +361,50 @@ ZO_API void zo_softmax_rows_f32(const float *x, float *y, float *rowsum, int32_t
     }
 }
 
+/* The same chain on 16-bit storage (bf16 / f16; dtype codes as everywhere in this file): elements widen to f32
+ * registers, softmax's max / sub / exp / sum / div stay in f32 inside its kernel (zyx/src/codegen/c.rs:615-629) and y is
+ * narrowed by truncation on store (:491-496); the sum and the argmax that follow are kernels of their own and read the
+ * stored y; the sum is stored truncated. Built from the f32 row function above and the load / store conversions that
+ * the narrow-store goldens pin. y, rowsum and arg may each be NULL. */
+ZO_API void zo_softmax_rows(int dtype, const void *x, void *y, void *rowsum, int32_t *arg, int64_t rows, int64_t cols) {
+    if (dtype == ZO_F32) {
+        zo_softmax_rows_f32((const float *)x, (float *)y, (float *)rowsum, arg, rows, cols);
+        return;
+    }
+#pragma omp parallel for
+    for (int64_t r = 0; r < rows; r++) {
+        float *tmp = (float *)malloc(sizeof(float) * (size_t)(cols > 0 ? cols : 1));
+        float m = -FLT_MAX;
+        for (int64_t c = 0; c < cols; c++) m = fmaxf(load_as_f32(x, dtype, r * cols + c), m);
+        float s = 0.0f;
+        for (int64_t c = 0; c < cols; c++) {
+            tmp[c] = expf(load_as_f32(x, dtype, r * cols + c) - m);
+            s = tmp[c] + s;
+        }
+        uint16_t *stored = (uint16_t *)malloc(sizeof(uint16_t) * (size_t)(cols > 0 ? cols : 1));
+        for (int64_t c = 0; c < cols; c++) store_from_f32(stored, dtype, c, tmp[c] / s);
+        float ys = 0.0f, ymax = -FLT_MAX;
+        for (int64_t c = 0; c < cols; c++) {
+            tmp[c] = load_as_f32(stored, dtype, c);
+            ys = tmp[c] + ys;
+            ymax = fmaxf(tmp[c], ymax);
+        }
+        if (y)
+            for (int64_t c = 0; c < cols; c++) ((uint16_t *)y)[r * cols + c] = stored[c];
+        if (rowsum) store_from_f32(rowsum, dtype, r, ys);
+        if (arg) {
+            int32_t a = INT32_MIN;
+            for (int64_t c = 0; c < cols; c++) {
+                int32_t idx = (int32_t)(tmp[c] == ymax) * (int32_t)c;
+                a = idx > a ? idx : a;
+            }
+            arg[r] = a;
+        }
+        free(stored);
+        free(tmp);
+    }
+}
+
 /* Same rows, but every accumulation in double: the "what the mathematics fixes"
  * companion used to bound how far serial f32 summation itself is from the truth. */
 ZO_API void zo_softmax_rows_f64acc(const float *x, float *y, float *rowsum, int64_t rows, int64_t cols) {

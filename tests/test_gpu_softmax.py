@@ -169,3 +169,41 @@ def test_undersized_argument_is_rejected(hip):
     for b in (x, y, s, a):
         pool.deallocate(b, [])
     dev.release(prog)
+
+
+# ---- 16-bit storage -----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("shape", [(1, 1), (5, 10), (64, 252), (33, 256), (9, 1000), (130, 1024), (6, 4092), (5, 4096), (3, 4097),
+                                   (2, 16384), (2048, 320)])
+def test_sixteen_bit_storage(hip, oracle, shape, dt):
+    """bf16 / f16 rows: elements widen to f32 registers, y is truncated on store, the row sum and the argmax read the stored
+    y (zyx/src/codegen/c.rs:456-497, 491-496). Against the oracle's restatement: the device's exp differs from expf in the
+    last bits of an f32, which can move a truncated y by one unit of its last place; the argmax follows the stored y."""
+    from zyx_amd import DType
+    dev, pool = hip
+    code, dtype, to16, to32, ulp = ((oracle.BF16, DType.BF16, oracle.f32_to_bf16, oracle.bf16_to_f32, 2.0 ** -7) if dt == "bf16" else
+                                    (oracle.F16, DType.F16, oracle.f32_to_f16, oracle.f16_to_f32, 2.0 ** -10))
+    x = to16(oracle.Rng(shape[0] * 7 + shape[1]).randn(shape, 3.0))
+    y, s, a = kernels.softmax_rows(dev, pool, x, dtype=dtype)
+    yo, so, ao = oracle.softmax_rows(x, dtype=code)
+    yf, yof = to32(y).astype(np.float64), to32(yo).astype(np.float64)
+    assert np.all(np.abs(yf - yof) <= ulp * yof + (1e-37 if dt == "bf16" else 6e-8))  # at most one step (f16: one subnormal step)
+    assert np.mean(y == yo) > 0.98
+    # the row sum of the stored values, itself stored truncated: a few steps of the 16-bit format around the oracle's
+    assert np.all(np.abs(to32(s).astype(np.float64) - to32(so)) <= 4 * ulp)
+    exact = to32(y).astype(np.float32).sum(1, dtype=np.float64)
+    assert np.all(np.abs(to32(s) - exact) <= 2 * ulp * exact + 1e-3 * ulp)
+    # argmax: the largest column among the maxima of the device's own stored row
+    yf32 = to32(y)
+    want = np.array([np.flatnonzero(r == r.max())[-1] for r in yf32], np.int32)
+    assert np.array_equal(a, want)
+    assert np.mean(a == ao) > 0.95
+
+
+def test_sixteen_bit_descriptor_is_checked(hip):
+    from zyx_amd import DType
+    dev, _ = hip
+    d = kernels.softmax_rows_desc(4, 8, dtype=DType.F64)
+    with pytest.raises(BackendError) as e:
+        dev.register_kernel(d)
+    assert e.value.status == ErrorStatus.KernelCompilation

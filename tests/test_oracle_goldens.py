@@ -672,3 +672,23 @@ def test_binary_table_closed_forms(oracle):
     assert np.allclose(got[pos], want[pos].astype(np.float32), rtol=2e-5) and np.all(np.isnan(got[~pos]))
     p = oracle.binary("pow", np.array([-2.0, 2.0, 0.5], np.float32), np.array([2.0, 2.0, 0.5], np.float32))
     assert np.isnan(p[0]) and abs(p[1] - 4.0) < 1e-5 and abs(p[2] - np.sqrt(0.5)) < 1e-6
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_softmax_rows_on_sixteen_bit_storage_is_the_f32_chain_with_narrow_stores(dt):
+    """zo_softmax_rows(dtype) against the same chain assembled from functions pinned above: the f32 primitives (max, sub,
+    exp, serial sum, div) on the widened row, the truncating store, then sum and argmax of the stored row."""
+    import oracle
+    code, to16, to32 = ((oracle.BF16, oracle.f32_to_bf16, oracle.bf16_to_f32) if dt == "bf16" else (oracle.F16, oracle.f32_to_f16, oracle.f16_to_f32))
+    for shape in [(3, 5), (7, 130), (2, 1000)]:
+        x = to16(oracle.Rng(shape[1]).randn(shape, 2.0))
+        y, s, a = oracle.softmax_rows(x, dtype=code)
+        xf = to32(x)
+        m = oracle.reduce_rows("max", xf)
+        e = oracle.unary("exp", oracle.binary("sub", xf, np.repeat(m[:, None], shape[1], 1)))
+        q = oracle.binary("div", e, np.repeat(oracle.reduce_rows("sum", e)[:, None], shape[1], 1))
+        want_y = to16(q)
+        assert np.array_equal(y, want_y)
+        stored = to32(want_y)
+        assert np.array_equal(s, to16(oracle.reduce_rows("sum", stored)))
+        assert np.array_equal(a, oracle.argmax_rows(stored))

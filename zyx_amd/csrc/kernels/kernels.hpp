@@ -10,9 +10,10 @@ namespace zk {
 
 struct SoftmaxRows {
     int64_t rows, cols;
-    const float *x;
-    float *y;       // may be null
-    float *rowsum;  // may be null
+    int dtype = 2;  // DT_F32 (2), DT_BF16 (0) or DT_F16 (1): storage of x, y and rowsum
+    const void *x;
+    void *y;        // may be null
+    void *rowsum;   // may be null
     int32_t *arg;   // may be null
 };
 hipError_t softmax_rows(const SoftmaxRows &p, hipStream_t stream);

@@ -1,4 +1,4 @@
-// Fused row softmax (+ row sum of the result, + row argmax of the result), f32.
+// Fused row softmax (+ row sum of the result, + row argmax of the result), f32; bf16 / f16 storage further down.
 //
 // Computes what zyx evaluates as >= 5 kernels for
 //   y = x.softmax([-1]); s = y.sum([-1]); a = y.argmax_axis(-1)
@@ -10,6 +10,7 @@
 // instruction of a wave covers 1 KiB of consecutive bytes). The three row
 // reductions (max, sum of exp, sum/argmax of y) are DPP + readlane wave reductions:
 // no LDS, no barriers. Four waves per workgroup -> rows/4 workgroups.
+#include "dtypes.hpp"
 #include "kernels.hpp"
 #include "wave.hpp"
 
@@ -122,6 +123,132 @@ __global__ __launch_bounds__(256) void softmax_rows_generic_k(const float *__res
     }
 }
 
+// 16-bit storage (bf16 / f16), as the C backend computes it: elements widen to f32 registers, the exponentials, their
+// sum and the quotient are f32, y is narrowed by truncation on store (zyx/src/codegen/c.rs:456-497, 491-496), and the
+// row sum and the argmax that follow read the stored y, i.e. the truncated values; the row sum is stored truncated too.
+template <int DT> __device__ __forceinline__ float widen(uint16_t h) { return DT == DT_BF16 ? bf16_to_f32(h) : f16_to_f32(h); }
+template <int DT> __device__ __forceinline__ uint16_t narrow(float v) { return DT == DT_BF16 ? f32_to_bf16_trunc(v) : f32_to_f16_trunc(v); }
+
+// One wave per row of up to 4096 columns held in registers, 4 columns (8 bytes) per lane and access.
+template <int DT, int NV>
+__global__ __launch_bounds__(256) void softmax_rows_wave16_k(const uint16_t *__restrict__ x, uint16_t *__restrict__ y,
+                                                             uint16_t *__restrict__ rowsum, int32_t *__restrict__ arg,
+                                                             int rows, int cols) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int nvec = cols >> 2;
+    const uint2 *xr = reinterpret_cast<const uint2 *>(x + (size_t)row * cols);
+    float v[NV][4];
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + 64 * j;
+        if (i < nvec) {
+            const uint2 t = xr[i];
+            v[j][0] = widen<DT>((uint16_t)t.x); v[j][1] = widen<DT>((uint16_t)(t.x >> 16));
+            v[j][2] = widen<DT>((uint16_t)t.y); v[j][3] = widen<DT>((uint16_t)(t.y >> 16));
+        } else v[j][0] = v[j][1] = v[j][2] = v[j][3] = -FLT_MAX;
+        m = fmaxf(fmaxf(fmaxf(v[j][0], v[j][1]), fmaxf(v[j][2], v[j][3])), m);
+    }
+    m = wave_allreduce_f32(m, OpMaxF());
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const bool live = lane + 64 * j < nvec;
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[j][k] = live ? exp_neg(v[j][k] - m) : 0.0f;
+        s += (v[j][0] + v[j][1]) + (v[j][2] + v[j][3]);
+    }
+    s = wave_allreduce_f32(s, OpAdd());
+    const float inv = 1.0f / s;
+    const float ymax = widen<DT>(narrow<DT>(inv)); // the stored y of the row maximum (its exponential is exactly 1)
+    float ys = 0.0f;
+    int best = 0;
+    uint2 *yr = reinterpret_cast<uint2 *>(y + (size_t)row * cols);
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + 64 * j;
+        if (i >= nvec) continue;
+        uint16_t t[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            t[k] = narrow<DT>(v[j][k] * inv);
+            const float f = widen<DT>(t[k]);
+            ys += f;
+            best = f == ymax ? max(best, i * 4 + k) : best; // largest column among ties
+        }
+        if (y) yr[i] = make_uint2((uint32_t)t[0] | ((uint32_t)t[1] << 16), (uint32_t)t[2] | ((uint32_t)t[3] << 16));
+    }
+    if (rowsum) {
+        ys = wave_allreduce_f32(ys, OpAdd());
+        if (lane == 0) rowsum[row] = narrow<DT>(ys);
+    }
+    if (arg) {
+        best = wave_allreduce_i32(best, OpMaxI());
+        if (lane == 0) arg[row] = best;
+    }
+}
+
+// Any cols / alignment: one workgroup per row, three passes over the row.
+template <int DT>
+__global__ __launch_bounds__(256) void softmax_rows_generic16_k(const uint16_t *__restrict__ x, uint16_t *__restrict__ y,
+                                                                uint16_t *__restrict__ rowsum, int32_t *__restrict__ arg,
+                                                                int rows, int64_t cols) {
+    __shared__ float lds[4];
+    __shared__ int ldsi[4];
+    const int64_t row = blockIdx.x;
+    const uint16_t *xr = x + row * cols;
+    float m = -FLT_MAX;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) m = fmaxf(widen<DT>(xr[c]), m);
+    m = block_allreduce_f32(m, OpMaxF(), lds);
+    float s = 0.0f;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) s += exp_neg(widen<DT>(xr[c]) - m);
+    s = block_allreduce_f32(s, OpAdd(), lds);
+    const float inv = 1.0f / s, ymax = widen<DT>(narrow<DT>(inv));
+    float ys = 0.0f;
+    int best = 0;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) {
+        const uint16_t t = narrow<DT>(exp_neg(widen<DT>(xr[c]) - m) * inv);
+        const float f = widen<DT>(t);
+        ys += f;
+        best = f == ymax ? max(best, (int)c) : best;
+        if (y) y[row * cols + c] = t;
+    }
+    if (rowsum) {
+        ys = block_allreduce_f32(ys, OpAdd(), lds);
+        if (threadIdx.x == 0) rowsum[row] = narrow<DT>(ys);
+    }
+    if (arg) {
+        best = wave_allreduce_i32(best, OpMaxI());
+        if ((threadIdx.x & 63) == 0) ldsi[threadIdx.x >> 6] = best;
+        __syncthreads();
+        if (threadIdx.x == 0) arg[row] = max(max(ldsi[0], ldsi[1]), max(ldsi[2], ldsi[3]));
+    }
+}
+
+template <int DT> static hipError_t softmax_rows16(const SoftmaxRows &p, hipStream_t st) {
+    const uint16_t *x = (const uint16_t *)p.x;
+    uint16_t *y = (uint16_t *)p.y, *rs = (uint16_t *)p.rowsum;
+    const bool vec_ok = (p.cols % 4 == 0) && p.cols <= 4096 && (reinterpret_cast<uintptr_t>(p.x) % 8 == 0) &&
+                        (p.y == nullptr || reinterpret_cast<uintptr_t>(p.y) % 8 == 0) && p.rows < (1ll << 31) - 4;
+    if (vec_ok) {
+        dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
+        const int64_t nvec = p.cols / 4;
+#define ZK_W16(NV) hipLaunchKernelGGL((softmax_rows_wave16_k<DT, NV>), grid, block, 0, st, x, y, rs, p.arg, (int)p.rows, (int)p.cols)
+        if (nvec <= 64) ZK_W16(1);
+        else if (nvec <= 128) ZK_W16(2);
+        else if (nvec <= 256) ZK_W16(4);
+        else if (nvec <= 512) ZK_W16(8);
+        else ZK_W16(16);
+#undef ZK_W16
+        return hipGetLastError();
+    }
+    if (p.rows >= (1ll << 31) || p.cols >= (1ll << 31)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(softmax_rows_generic16_k<DT>, dim3((unsigned)p.rows), dim3(256), 0, st, x, y, rs, p.arg, (int)p.rows, p.cols);
+    return hipGetLastError();
+}
+
 template <int NV> static hipError_t launch_wave(const SoftmaxRows &p, hipStream_t st) {
     dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
     // Rows of 16 vectors per lane on a grid of several rounds: an unused LDS request holds a compute unit at 3 workgroups
@@ -135,10 +262,10 @@ template <int NV> static hipError_t launch_wave(const SoftmaxRows &p, hipStream_
 #define ZK_CASE(S, A, B, C)                                                                                           \
     case S:                                                                                                           \
         if (full)                                                                                                     \
-            hipLaunchKernelGGL((softmax_rows_wave_k<NV, true, A, B, C>), grid, block, lds_pad, st, p.x, p.y, p.rowsum,     \
+            hipLaunchKernelGGL((softmax_rows_wave_k<NV, true, A, B, C>), grid, block, lds_pad, st, (const float *)p.x, (float *)p.y, (float *)p.rowsum, \
                                p.arg, rows, cols);                                                                    \
         else                                                                                                          \
-            hipLaunchKernelGGL((softmax_rows_wave_k<NV, false, A, B, C>), grid, block, 0, st, p.x, p.y, p.rowsum,    \
+            hipLaunchKernelGGL((softmax_rows_wave_k<NV, false, A, B, C>), grid, block, 0, st, (const float *)p.x, (float *)p.y, (float *)p.rowsum, \
                                p.arg, rows, cols);                                                                    \
         break;
     switch (sel) {
@@ -153,6 +280,9 @@ template <int NV> static hipError_t launch_wave(const SoftmaxRows &p, hipStream_
 
 hipError_t softmax_rows(const SoftmaxRows &p, hipStream_t st) {
     if (p.rows <= 0 || p.cols <= 0) return hipSuccess; // empty tensor: nothing to write
+    if (p.dtype == DT_BF16) return softmax_rows16<DT_BF16>(p, st);
+    if (p.dtype == DT_F16) return softmax_rows16<DT_F16>(p, st);
+    if (p.dtype != DT_F32) return hipErrorInvalidValue;
     bool vec_ok = (p.cols % 4 == 0) && p.cols <= 4096 && (reinterpret_cast<uintptr_t>(p.x) % 16 == 0) &&
                   (p.y == nullptr || reinterpret_cast<uintptr_t>(p.y) % 16 == 0) && p.rows < (1ll << 31) - 4;
     if (vec_ok) {
@@ -164,7 +294,7 @@ hipError_t softmax_rows(const SoftmaxRows &p, hipStream_t st) {
         return launch_wave<16>(p, st);
     }
     if (p.rows >= (1ll << 31) || p.cols >= (1ll << 31)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(softmax_rows_generic_k, dim3((unsigned)p.rows), dim3(256), 0, st, p.x, p.y, p.rowsum, p.arg,
+    hipLaunchKernelGGL(softmax_rows_generic_k, dim3((unsigned)p.rows), dim3(256), 0, st, (const float *)p.x, (float *)p.y, (float *)p.rowsum, p.arg,
                        (int)p.rows, p.cols);
     return hipGetLastError();
 }

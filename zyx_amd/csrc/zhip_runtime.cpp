@@ -470,15 +470,17 @@ int32_t program_from_desc(zhip_ctx *c, const zhip_kernel_desc &d, Program &p) {
     switch (d.kind) {
     case ZHIP_K_SOFTMAX_ROWS: {
         int64_t rows = d.dims[0], cols = d.dims[1];
-        if (d.dtype != ZHIP_F32) return c->fail(ZHIP_KERNEL_COMPILATION, "softmax_rows: only f32 is implemented");
+        if (d.dtype != ZHIP_F32 && d.dtype != ZHIP_BF16 && d.dtype != ZHIP_F16)
+            return c->fail(ZHIP_KERNEL_COMPILATION, "softmax_rows: dtype must be f32, bf16 or f16");
+        const uint64_t es = d.dtype == ZHIP_F32 ? 4 : 2;
         if (rows < 0 || cols < 0 || rows >= (1ll << 31) || cols >= (1ll << 31))
             return c->fail(ZHIP_KERNEL_COMPILATION, "softmax_rows: rows/cols out of range");
         if ((d.flags & 7) == 0 || (d.flags & ~7)) return c->fail(ZHIP_KERNEL_COMPILATION, "softmax_rows: bad output flags");
         p.n_in = 1;
-        p.need[0] = (uint64_t)rows * cols * 4;
+        p.need[0] = (uint64_t)rows * cols * es;
         int o = 1;
-        if (d.flags & ZHIP_SOFTMAX_Y) p.need[o++] = (uint64_t)rows * cols * 4;
-        if (d.flags & ZHIP_SOFTMAX_ROWSUM) p.need[o++] = (uint64_t)rows * 4;
+        if (d.flags & ZHIP_SOFTMAX_Y) p.need[o++] = (uint64_t)rows * cols * es;
+        if (d.flags & ZHIP_SOFTMAX_ROWSUM) p.need[o++] = (uint64_t)rows * es;
         if (d.flags & ZHIP_SOFTMAX_ARGMAX) p.need[o++] = (uint64_t)rows * 4;
         p.n_out = o - 1;
         return ZHIP_OK;
@@ -800,10 +802,11 @@ hipError_t program_enqueue(const Program &p, void *const *ptr, hipStream_t st, b
         zk::SoftmaxRows a{};
         a.rows = d.dims[0];
         a.cols = d.dims[1];
-        a.x = (const float *)ptr[0];
+        a.dtype = d.dtype;
+        a.x = ptr[0];
         int o = 1;
-        if (d.flags & ZHIP_SOFTMAX_Y) a.y = (float *)ptr[o++];
-        if (d.flags & ZHIP_SOFTMAX_ROWSUM) a.rowsum = (float *)ptr[o++];
+        if (d.flags & ZHIP_SOFTMAX_Y) a.y = ptr[o++];
+        if (d.flags & ZHIP_SOFTMAX_ROWSUM) a.rowsum = ptr[o++];
         if (d.flags & ZHIP_SOFTMAX_ARGMAX) a.arg = (int32_t *)ptr[o++];
         return zk::softmax_rows(a, st);
     }

@@ -12,9 +12,9 @@ K_SOFTMAX_ROWS = 1
 SOFTMAX_Y, SOFTMAX_ROWSUM, SOFTMAX_ARGMAX = 1, 2, 4
 
 
-def softmax_rows_desc(rows: int, cols: int, y=True, rowsum=True, argmax=True) -> KernelDesc:
+def softmax_rows_desc(rows: int, cols: int, y=True, rowsum=True, argmax=True, dtype: DType = DType.F32) -> KernelDesc:
     d = KernelDesc()
-    d.kind, d.dtype, d.out_dtype = K_SOFTMAX_ROWS, DType.F32, DType.F32
+    d.kind, d.dtype, d.out_dtype = K_SOFTMAX_ROWS, DType(dtype), DType(dtype)
     d.flags = (SOFTMAX_Y if y else 0) | (SOFTMAX_ROWSUM if rowsum else 0) | (SOFTMAX_ARGMAX if argmax else 0)
     d.dims[0], d.dims[1] = rows, cols
     return d
@@ -42,14 +42,16 @@ def alloc_like(pool: HIPMemoryPool, n_elems: int, itemsize: int):
     return pool.allocate((n_elems + 1) * itemsize)
 
 
-def softmax_rows(dev: HIPDevice, pool: HIPMemoryPool, x: np.ndarray, y=True, rowsum=True, argmax=True):
-    """Upload x, run the fused kernel, read back (y, rowsum, argmax); entries not asked for are None."""
-    x = np.ascontiguousarray(x, np.float32)
+def softmax_rows(dev: HIPDevice, pool: HIPMemoryPool, x: np.ndarray, y=True, rowsum=True, argmax=True, dtype: DType = DType.F32):
+    """Upload x, run the fused kernel, read back (y, rowsum, argmax); entries not asked for are None. bf16 / f16: x, y and
+    rowsum are bit patterns (uint16)."""
+    st = np.float32 if DType(dtype) == DType.F32 else np.uint16
+    x = np.ascontiguousarray(x, st)
     rows, cols = x.shape
-    prog = dev.register_kernel(softmax_rows_desc(rows, cols, y, rowsum, argmax))
+    prog = dev.register_kernel(softmax_rows_desc(rows, cols, y, rowsum, argmax, dtype))
     xb, ev = to_device(pool, x)
     waits, outs = [ev], []
-    for want, n, isz in ((y, rows * cols, 4), (rowsum, rows, 4), (argmax, rows, 4)):
+    for want, n, isz in ((y, rows * cols, x.itemsize), (rowsum, rows, x.itemsize), (argmax, rows, 4)):
         if want:
             b, e = alloc_like(pool, n, isz)
             outs.append(b)
@@ -57,7 +59,7 @@ def softmax_rows(dev: HIPDevice, pool: HIPMemoryPool, x: np.ndarray, y=True, row
     done = dev.launch(prog, pool, [xb] + outs, waits)
     res, it = [], iter(outs)
     first = True
-    for want, shape, dt in ((y, (rows, cols), np.float32), (rowsum, (rows,), np.float32), (argmax, (rows,), np.int32)):
+    for want, shape, dt in ((y, (rows, cols), st), (rowsum, (rows,), st), (argmax, (rows,), np.int32)):
         if not want:
             res.append(None)
             continue
