@@ -5,7 +5,8 @@
 // (zyx/src/tensor/mod.rs:1457-1461, 2245-2269; zyx/src/tensor/reduce_ops.rs:45-147)
 // in one pass over HBM: x is read once, y written once.
 //
-// Register-resident variant: one 64-lane wave owns one row of up to 4096 columns,
+// Register-resident variants. Many full rows of 1024 / 2048 / 4096 columns: four waves share a row (softmax_rows_split_k
+// below; the benchmark's shape). Otherwise: one 64-lane wave owns one row of up to 4096 columns,
 // each lane holding NV float4 (lane + 64*j addressing, so every load/store
 // instruction of a wave covers 1 KiB of consecutive bytes). The three row
 // reductions (max, sum of exp, sum/argmax of y) are DPP + readlane wave reductions:
@@ -76,6 +77,92 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_k(const float *__restri
     if (WA) {
         best = wave_allreduce_i32(best, OpMaxI());
         if (lane == 0) arg[row] = best;
+    }
+}
+
+// The same row split over W waves of a workgroup (W = 2 or 4; 4 / W rows per workgroup), NVL float4 per lane: a wave's
+// requests cover 1024 * NVL / 256 KiB of consecutive bytes instead of the whole row, and there are W times as many
+// waves to issue them; the three row reductions go through LDS (one barrier each). cols == 256 * NVL * W exactly.
+template <int NVL, int W, bool WY, bool WS, bool WA>
+__global__ __launch_bounds__(W < 4 ? 256 : 64 * W) void softmax_rows_split_k(const float *__restrict__ x, float *__restrict__ y,
+                                                            float *__restrict__ rowsum, int32_t *__restrict__ arg, int rows) {
+    constexpr int RPB = W < 4 ? 4 / W : 1, cols = 256 * NVL * W; // rows per workgroup
+    __shared__ float red[3][16];
+    __shared__ int redi[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, part = wave % W, rw = wave / W;
+    const int row = blockIdx.x * RPB + rw;
+    const bool live = row < rows; // every wave reaches every barrier
+    const size_t base = (size_t)(live ? row : 0) * cols + (size_t)part * (256 * NVL);
+    const f32x4 *xr = reinterpret_cast<const f32x4 *>(x + base);
+    f32x4 v[NVL];
+#pragma unroll
+    for (int j = 0; j < NVL; j++) v[j] = load_stream(xr + lane + 64 * j);
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < NVL; j++) m = fmaxf(fmaxf(fmaxf(v[j].x, v[j].y), fmaxf(v[j].z, v[j].w)), m);
+    m = wave_allreduce_f32(m, OpMaxF());
+    if (lane == 0) red[0][wave] = m;
+    __syncthreads();
+    m = red[0][rw * W];
+#pragma unroll
+    for (int k = 1; k < W; k++) m = fmaxf(m, red[0][rw * W + k]);
+
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+        v[j].x = exp_neg(v[j].x - m);
+        v[j].y = exp_neg(v[j].y - m);
+        v[j].z = exp_neg(v[j].z - m);
+        v[j].w = exp_neg(v[j].w - m);
+        s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+    }
+    s = wave_allreduce_f32(s, OpAdd());
+    if (lane == 0) red[1][wave] = s;
+    __syncthreads();
+    s = red[1][rw * W];
+#pragma unroll
+    for (int k = 1; k < W; k++) s += red[1][rw * W + k]; // the parts in column order, in every wave of the row
+    const float inv = 1.0f / s;
+
+    float ys = 0.0f;
+    int best = 0;
+    f32x4 *yr = reinterpret_cast<f32x4 *>(y + base);
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+        const int i = lane + 64 * j;
+        f32x4 o = v[j] * inv;
+        if (WS) ys += (o.x + o.y) + (o.z + o.w);
+        if (WA) {
+            const int c = part * (256 * NVL) + i * 4;
+            best = o.x == inv ? max(best, c) : best;
+            best = o.y == inv ? max(best, c + 1) : best;
+            best = o.z == inv ? max(best, c + 2) : best;
+            best = o.w == inv ? max(best, c + 3) : best;
+        }
+        if (WY && live) store_stream(o, yr + i);
+    }
+    if (WS || WA) {
+        if (WS) ys = wave_allreduce_f32(ys, OpAdd());
+        if (WA) best = wave_allreduce_i32(best, OpMaxI());
+        if (lane == 0) {
+            red[2][wave] = ys;
+            redi[wave] = best;
+        }
+        __syncthreads();
+        if (part == 0 && lane == 0 && live) {
+            if (WS) {
+                float t = red[2][rw * W];
+#pragma unroll
+                for (int k = 1; k < W; k++) t += red[2][rw * W + k];
+                rowsum[row] = t;
+            }
+            if (WA) {
+                int t = redi[rw * W];
+#pragma unroll
+                for (int k = 1; k < W; k++) t = max(t, redi[rw * W + k]);
+                arg[row] = t;
+            }
+        }
     }
 }
 
@@ -249,6 +336,28 @@ template <int DT> static hipError_t softmax_rows16(const SoftmaxRows &p, hipStre
     return hipGetLastError();
 }
 
+// Four waves per row. Measured at 8192 x 4096 (all three outputs): 44.2 us against 47.8 us for one wave per row (two waves
+// per row 45.5, eight 44.4, sixteen 50.7), and 43.4 us when an unused LDS request holds a compute unit at 4 workgroups
+// (16 waves) on a grid of several rounds, so that one round's stores run beside the next one's loads.
+template <int NVL> static hipError_t launch_split(const SoftmaxRows &p, hipStream_t st) {
+    dim3 grid((unsigned)p.rows), block(256);
+    const unsigned lds_pad = p.rows >= 4096 ? 40000u : 0u;
+    const int sel = (p.y ? 1 : 0) | (p.rowsum ? 2 : 0) | (p.arg ? 4 : 0);
+#define ZK_CASE(S, A, B, C)                                                                                           \
+    case S:                                                                                                           \
+        hipLaunchKernelGGL((softmax_rows_split_k<NVL, 4, A, B, C>), grid, block, lds_pad, st, (const float *)p.x, (float *)p.y, \
+                           (float *)p.rowsum, p.arg, (int)p.rows);                                                    \
+        break;
+    switch (sel) {
+        ZK_CASE(1, true, false, false) ZK_CASE(2, false, true, false) ZK_CASE(3, true, true, false)
+        ZK_CASE(4, false, false, true) ZK_CASE(5, true, false, true) ZK_CASE(6, false, true, true)
+        ZK_CASE(7, true, true, true)
+    default: return hipErrorInvalidValue;
+    }
+#undef ZK_CASE
+    return hipGetLastError();
+}
+
 template <int NV> static hipError_t launch_wave(const SoftmaxRows &p, hipStream_t st) {
     dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
     // Rows of 16 vectors per lane on a grid of several rounds: an unused LDS request holds a compute unit at 3 workgroups
@@ -287,6 +396,10 @@ hipError_t softmax_rows(const SoftmaxRows &p, hipStream_t st) {
                   (p.y == nullptr || reinterpret_cast<uintptr_t>(p.y) % 16 == 0) && p.rows < (1ll << 31) - 4;
     if (vec_ok) {
         int64_t nvec = p.cols / 4;
+        // many full rows of 1024, 2048 or 4096 columns: four waves per row
+        if (p.rows >= 1024 && p.cols == 1024) return launch_split<1>(p, st);
+        if (p.rows >= 1024 && p.cols == 2048) return launch_split<2>(p, st);
+        if (p.rows >= 1024 && p.cols == 4096) return launch_split<4>(p, st);
         if (nvec <= 64) return launch_wave<1>(p, st);
         if (nvec <= 128) return launch_wave<2>(p, st);
         if (nvec <= 256) return launch_wave<4>(p, st);
