@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 N_SETS = 4              # 4 x 268 MB working set > Infinity Cache
 # HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
 # by the same counter's reading for a plain copy kernel of known size in the same run
-# (profiles/softmax_rows_f32_8192x4096.md): 134,351,537 B fetched + 134,443,294 B written.
+# (profiles/softmax_rows_f32_8192x4096.md): 134,262,878 B fetched + 134,739,929 B written.
 TRAFFIC_BYTES = 269002807
 
 
