@@ -13,7 +13,7 @@ from zyx_amd.kernels import argmax_desc, reduce
 pytestmark = pytest.mark.gpu
 
 SHAPES = [(1, 1), (3, 5), (8, 4096), (1, 131072), (1, 1 << 22), (4096, 512), (100, 1000), (513, 257), (70000, 12),
-          (2, 100003), (64, 128), (64, 10), (8192, 4096)]
+          (2, 100003), (64, 128), (64, 10), (8192, 4096), (2048, 2050), (2100, 2500), (2048, 16384)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
@@ -61,6 +61,23 @@ def test_16bit_inputs_accumulate_in_f32(hip, oracle, dt):
         assert np.all(np.abs(got - ref) <= ulp + 1e-6)
         assert np.array_equal(reduce(dev, pool, x, "max", axis0, dt),
                               (oracle.reduce_cols if axis0 else oracle.reduce_rows)("max", x, code))
+
+
+@pytest.mark.parametrize("cols", [4096, 4100, 4103, 12296])
+def test_rows_shared_by_a_workgroup(hip, oracle, cols):
+    """Many rows of 8-64 KiB: four waves take a quarter of the row each. Integer sums (wrapping) and maxima are exact
+    whatever the split; 16-bit rows whose quarters are not whole 16-byte pieces take the narrower loads."""
+    dev, pool = hip
+    rng = np.random.default_rng(cols)
+    x = rng.integers(-2**31, 2**31, size=(2048, cols), dtype=np.int64).astype(np.int32)
+    assert np.array_equal(reduce(dev, pool, x, "sum", False, DType.I32), oracle.reduce_rows_i32("sum", x))
+    assert np.array_equal(reduce(dev, pool, x, "max", False, DType.I32), x.max(1))
+    xb = oracle.f32_to_bf16(oracle.Rng(cols).randn((2048, cols)))
+    assert np.array_equal(reduce(dev, pool, xb, "max", False, DType.BF16), oracle.reduce_rows("max", xb, oracle.BF16))
+    got = oracle.bf16_to_f32(reduce(dev, pool, xb, "sum", False, DType.BF16))
+    ref = oracle.bf16_to_f32(oracle.reduce_rows("sum", xb, oracle.BF16))
+    ulp = 2.0 ** (np.floor(np.log2(np.abs(ref) + 1e-30)) - 7)
+    assert np.all(np.abs(got - ref) <= ulp + 1e-4 * np.sqrt(cols))
 
 
 def test_empty_axes(hip):

@@ -129,9 +129,38 @@ __device__ __forceinline__ typename Elem<DT>::A fold_row_span(const typename Ele
     typedef typename Elem<DT>::A A;
     typedef Fold<OP, A> F;
     A acc = F::init();
+    if constexpr (sizeof(typename Elem<DT>::S) == 2) {
+        // 16-bit rows whose span is whole 16-byte pieces: 8 elements per request, eight requests in flight per lane
+        if (VEC && ((c1 - c0) & 7) == 0 && (c0 & 7) == 0 && (reinterpret_cast<uintptr_t>(xr) & 15) == 0) {
+            const int64_t nv = (c1 - c0) >> 3;
+            int64_t i = lane;
+            for (; i + 7 * nlanes < nv; i += 8 * nlanes) {
+                A v[8][8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) Elem<DT>::ld8(xr, c0 + (i + u * nlanes) * 8, v[u]);
+#pragma unroll
+                for (int u = 0; u < 8; u++)
+                    acc = F::f(acc, F::f(F::f(F::f(v[u][0], v[u][1]), F::f(v[u][2], v[u][3])), F::f(F::f(v[u][4], v[u][5]), F::f(v[u][6], v[u][7]))));
+            }
+            for (; i < nv; i += nlanes) {
+                A v[8];
+                Elem<DT>::ld8(xr, c0 + i * 8, v);
+                acc = F::f(acc, F::f(F::f(F::f(v[0], v[1]), F::f(v[2], v[3])), F::f(F::f(v[4], v[5]), F::f(v[6], v[7]))));
+            }
+            return acc;
+        }
+    }
     if (VEC) {
         int64_t nv = (c1 - c0) >> 2;
-        for (int64_t i = lane; i < nv; i += nlanes) {
+        int64_t i = lane;
+        for (; i + 7 * nlanes < nv; i += 8 * nlanes) { // eight requests in flight per lane
+            A v[8][4];
+#pragma unroll
+            for (int u = 0; u < 8; u++) Elem<DT>::ld4(xr, c0 + (i + u * nlanes) * 4, v[u]);
+#pragma unroll
+            for (int u = 0; u < 8; u++) acc = F::f(acc, F::f(F::f(v[u][0], v[u][1]), F::f(v[u][2], v[u][3])));
+        }
+        for (; i < nv; i += nlanes) {
             A v[4];
             Elem<DT>::ld4(xr, c0 + i * 4, v);
             acc = F::f(acc, F::f(F::f(v[0], v[1]), F::f(v[2], v[3])));
@@ -162,6 +191,26 @@ __global__ __launch_bounds__(256) void reduce_rows_wave_k(const typename Elem<DT
         if (segs == 1) store_result<DT>(out, row, acc, epi);
         else partial[item] = acc;
     }
+}
+
+// rows, many of middling length: a workgroup per row, its 4 waves take a quarter each (a wave's requests then cover a
+// few KiB of consecutive memory, which the memory system serves faster than one wave walking the whole row) and the
+// quarters meet in LDS. quarter is a multiple of 8 elements.
+template <int DT, int OP, bool VEC>
+__global__ __launch_bounds__(256) void reduce_rows_group_k(const typename Elem<DT>::S *__restrict__ x,
+                                                           typename Elem<DT>::S *__restrict__ out, int64_t cols,
+                                                           int64_t quarter, const Epilogue epi) {
+    typedef typename Elem<DT>::A A;
+    typedef Fold<OP, A> F;
+    __shared__ A part[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row = blockIdx.x;
+    const int64_t c0 = min(cols, wave * quarter), c1 = min(cols, c0 + quarter);
+    A acc = fold_row_span<DT, OP, VEC>(x + row * cols, c0, c1, lane, 64);
+    acc = wave_fold<OP>(acc);
+    if (lane == 0) part[wave] = acc;
+    __syncthreads(); // every thread arrives: no early exit above
+    if (threadIdx.x == 0) store_result<DT>(out, row, F::f(F::f(part[0], part[1]), F::f(part[2], part[3])), epi);
 }
 
 // second stage: fold `segs` raw partials per row (accumulator type), store as DT.
@@ -291,6 +340,14 @@ template <int DT, int OP> hipError_t launch(const Reduce &p, hipStream_t st) {
         bool vec = (p.cols * esz) % (4 * esz) == 0 && p.cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
         RowPlan pl = plan_rows(p.rows, p.cols);
         if (pl.segs > 1 && (uint64_t)p.rows * pl.segs * sizeof(A) > p.workspace_bytes) return hipErrorInvalidValue;
+        const int64_t row_bytes = p.cols * esz;
+        if (pl.segs == 1 && p.rows >= 2048 && p.rows <= 0x7fffffff && row_bytes >= 8192 && row_bytes <= 65536) {
+            const int64_t quarter = ((p.cols + 3) / 4 + 7) / 8 * 8;
+            dim3 grid((unsigned)p.rows), block(256);
+            if (vec) hipLaunchKernelGGL((reduce_rows_group_k<DT, OP, true>), grid, block, 0, st, x, out, p.cols, quarter, epi);
+            else hipLaunchKernelGGL((reduce_rows_group_k<DT, OP, false>), grid, block, 0, st, x, out, p.cols, quarter, epi);
+            return hipGetLastError();
+        }
         int64_t items = p.rows * pl.segs;
         dim3 grid((unsigned)((items + 3) / 4)), block(256);
         if (vec) hipLaunchKernelGGL((reduce_rows_wave_k<DT, OP, true>), grid, block, 0, st, x, out, ws, p.rows, p.cols, pl.segs, pl.seg_len, epi);
