@@ -209,6 +209,9 @@ def extra_streaming(dev, pool, kernels, steps=20, warmup=5):
         timeit(f"add_{tag}_8192x4096", c.desc(), lambda: [full(), full(), out_arr(M * F, isz)], 3 * M * F * isz)
         timeit(f"colsum_{tag}_8192x4096", kernels.reduce_desc(M, F, "sum", axis0=True, dtype=dt), lambda: [full(), out_arr(F, isz)], M * F * isz)
         timeit(f"rowsum_{tag}_8192x4096", kernels.reduce_desc(M, F, "sum", dtype=dt), lambda: [full(), out_arr(M, isz)], M * F * isz)
+        c = kernels.Chain(M, D, out_dtype=dt)
+        c.load(c.input(dt))
+        timeit(f"copy_{tag}_8192x1024", c.desc(), lambda: [dev_arr(row, dt), out_arr(M * D, isz)], 2 * M * D * isz)  # what a launch this small can reach
         w, bb = dev_arr(vec, dt), dev_arr(vec, dt)  # the affine parameters are shared by every set, as in a model
         timeit(f"layernorm_{tag}_8192x1024", kernels.norm_rows_desc(M, D, dtype=dt), lambda: [dev_arr(row, dt), w, bb, out_arr(M * D, isz)], 2 * M * D * isz)
         w, bb = dev_arr(vec, dt), dev_arr(vec, dt)

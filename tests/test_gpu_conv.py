@@ -187,11 +187,14 @@ def test_max_pool_2x2_fast_path(hip, oracle, shape):
     assert np.array_equal(max_pool2d(dev, pool, xb, *args, dtype=DType.BF16), oracle.max_pool2d(xb, *args, dtype=oracle.BF16))
 
 
-@pytest.mark.parametrize("shape", [(2, 16, 16, 56, 128), (1, 64, 56, 56, 128), (3, 32, 28, 16, 256), (2, 48, 8, 112, 128), (1, 16, 56, 8, 128)])
+@pytest.mark.parametrize("shape", [(2, 16, 16, 56, 128), (1, 64, 56, 56, 128), (3, 32, 28, 16, 256), (2, 48, 8, 112, 128), (1, 16, 56, 8, 128),
+                                   (2, 64, 16, 28, 128), (1, 96, 8, 56, 128), (1, 32, 2, 224, 128)])
 @pytest.mark.parametrize("bias,relu", [(True, True), (False, False)])
 def test_conv3x3_direct_bf16(hip, oracle, shape, bias, relu):
     """3 x 3 / stride 1 / padding 1 bf16 shapes whose rows tile into 448-pixel blocks take the direct kernel (input
-    tile in LDS, nine shifted views, no patch matrix): against the oracle, bf16 and f32 results, first / last rows and
+    tile in LDS, nine shifted views, no patch matrix; 224-pixel tiles on 16 x 16 x 32 matrix instructions when the
+    channel count is a multiple of 32 -- an odd and an even number of 32-channel steps, 1 to 14 rows per tile -- and
+    448-pixel tiles otherwise): against the oracle, bf16 and f32 results, first / last rows and
     columns (the zero border) included; the f32 result is also checked against the f64 convolution."""
     dev, pool = hip
     n, c, h, w, co = shape

@@ -58,6 +58,123 @@ __global__ __launch_bounds__(256) void conv3x3_weights_k(const T *__restrict__ w
 // smaller than the distance 0.5 / d of (q + 0.5) / d from the nearest integer
 __device__ __forceinline__ int small_div(int q, float inv) { return (int)(((float)q + 0.5f) * inv); }
 
+// The bf16 input tile: rows rb*R - 1 .. rb*R + R of every channel of image n, channel-innermost in LDS, zero outside
+// the image. One item = 8 consecutive columns of two neighbouring channels of one row: two 16-byte reads, eight 4-byte
+// LDS writes (channel pair packed). The lanes of a wave take 4 neighbouring items of a row for each of 16 channel pairs
+// (8 x 8 when C / 2 is not a multiple of 16): the texture unit takes one cache line per cycle, so neighbouring lanes
+// share lines, while the writes of one instruction still spread over 32 banks. U items' reads are in flight together.
+template <int U>
+__device__ __forceinline__ void load_tile_bf16(ZK_LDS uint8_t *smem, const void *x_, int n, int rb, int R, int C, int H, int W,
+                                               int PS, int lane, int wave) {
+    const int Wp = W + 2;
+    const uint16_t *x = (const uint16_t *)x_;
+    const int w8 = W >> 3;
+    const int C2 = C >> 1, RC = (R + 2) * w8;          // channel pairs; 8-column pieces of one channel's rows
+    const int KB = (C2 & 15) ? 3 : 2;                  // log2(items of a row per wave instruction)
+    const int k = lane & ((1 << KB) - 1), cp_lo = lane >> KB, cp_lanes = 64 >> KB;
+    const int cpblocks = C2 / cp_lanes, groups = (RC + (1 << KB) - 1) >> KB, wave_items = cpblocks * groups;
+    const float inv_w8 = 1.0f / (float)w8;
+    const int64_t plane = (int64_t)H * W;
+    const uint16_t *xn = x + (int64_t)n * C * plane;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    for (int t0 = wave_u; t0 < wave_items; t0 += 4 * U) {
+        u32x4 va[U], vb[U];
+        int dsto[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int t = t0 + 4 * u;                   // uniform over the wave
+            const int g = t / cpblocks, cpb = t - g * cpblocks;
+            const int rc = (g << KB) + k, cp = cpb * cp_lanes + cp_lo;
+            const int r = small_div(rc, inv_w8), ch = rc - __mul24(r, w8);
+            const int iy = rb * R - 1 + r;
+            const bool live = t < wave_items && rc < RC;
+            va[u] = vb[u] = u32x4{0u, 0u, 0u, 0u};
+            if (live && iy >= 0 && iy < H) {
+                const uint16_t *src = xn + (int64_t)(2 * cp) * plane + __mul24(iy, W) + ch * 8;
+                va[u] = *(const u32x4 *)src;
+                vb[u] = *(const u32x4 *)(src + plane);
+            }
+            dsto[u] = live ? __mul24(__mul24(r, Wp) + 1 + ch * 8, PS) + cp * 4 : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            if (dsto[u] < 0) continue;
+            ZK_LDS uint8_t *dst = smem + dsto[u];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                *(ZK_LDS uint32_t *)(dst + (2 * e) * PS) = __builtin_amdgcn_perm(vb[u][e], va[u][e], 0x05040100u);
+                *(ZK_LDS uint32_t *)(dst + (2 * e + 1) * PS) = __builtin_amdgcn_perm(vb[u][e], va[u][e], 0x07060302u);
+            }
+        }
+    }
+}
+
+// The staged tile ([channel][pixel], TP pixels = whole rows of the image, RS bytes per channel row; 128 channel rows for
+// 16-bit output, 64 per pass for 32-bit) leaves for y in 16-byte pieces, or, POOL, through 2 x 2 windows: a channel's
+// pooled tile is TP / 4 values, consecutive in the pooled plane, a thread makes 16 bytes of them; the running maximum
+// starts at the dtype's lowest finite value and takes the window in row order, like the separate pooling kernel.
+template <int TP, bool OUT_BF16, bool POOL>
+__device__ __forceinline__ void copy_out(const ZK_LDS uint8_t *smem, void *__restrict__ y, int n, int Cout, int co0, int H, int W,
+                                         int rb, int pass, int tid) {
+    constexpr int ES = OUT_BF16 ? 2 : 4;
+    constexpr int RS = TP * ES + 16;
+    constexpr int CPR = TP * ES / 16;
+    constexpr int ROWS = OUT_BF16 ? 128 : 64;
+    const int64_t plane = (int64_t)H * W;
+    if constexpr (POOL) {
+        constexpr int PV = TP / 4, VPC = 16 / ES, PCR = PV / VPC;
+        const int W2 = W >> 1;
+        const float inv_w2 = 1.0f / (float)W2;
+        const float lowest = OUT_BF16 ? -3.3895313892515355e38f : -3.4028234663852886e38f;
+        const int64_t pplane = plane >> 2;
+        uint8_t *ptile = (uint8_t *)y + (((int64_t)n * Cout + co0) * pplane + (int64_t)rb * PV) * ES;
+        for (int idx = tid; idx < ROWS * PCR; idx += 256) {
+            const int row = idx / PCR, piece = idx - row * PCR;
+            const int co = OUT_BF16 ? row : (row >> 5) * 64 + pass * 32 + (row & 31);
+            float m[VPC];
+            int pr = small_div(piece * VPC, inv_w2), pc = piece * VPC - __mul24(pr, W2); // pooled row, column of value 0
+            const ZK_LDS uint8_t *rowp = smem + row * RS + __mul24(2 * pr, W) * ES;
+#pragma unroll
+            for (int e = 0; e < VPC; e++) {
+                const ZK_LDS uint8_t *src = rowp + 2 * pc * ES;
+                if (++pc == W2) { // the next value starts the next pooled row
+                    pc = 0;
+                    rowp += 2 * W * ES;
+                }
+                float a0, a1, b0, b1;
+                if (OUT_BF16) {
+                    const uint32_t u0 = *(const ZK_LDS uint32_t *)src, u1 = *(const ZK_LDS uint32_t *)(src + W * ES);
+                    a0 = __uint_as_float(u0 << 16), a1 = __uint_as_float(u0 & 0xffff0000u);
+                    b0 = __uint_as_float(u1 << 16), b1 = __uint_as_float(u1 & 0xffff0000u);
+                } else {
+                    const u32x2 u0 = *(const ZK_LDS u32x2 *)src, u1 = *(const ZK_LDS u32x2 *)(src + W * ES);
+                    a0 = __uint_as_float(u0[0]), a1 = __uint_as_float(u0[1]), b0 = __uint_as_float(u1[0]), b1 = __uint_as_float(u1[1]);
+                }
+                m[e] = fmaxf(b1, fmaxf(b0, fmaxf(a1, fmaxf(a0, lowest))));
+            }
+            u32x4 v;
+            if (OUT_BF16) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = __builtin_amdgcn_perm(__float_as_uint(m[(2 * e + 1) % VPC]), __float_as_uint(m[(2 * e) % VPC]), 0x07060302u);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = __float_as_uint(m[e % VPC]);
+            }
+            *(u32x4 *)(ptile + (int64_t)co * pplane * ES + piece * 16) = v;
+        }
+    } else {
+        // the tile's pixels are consecutive in the image plane
+        uint8_t *ytile = (uint8_t *)y + (((int64_t)n * Cout + co0) * plane + (int64_t)rb * TP) * ES;
+#pragma unroll 4
+        for (int idx = tid; idx < ROWS * CPR; idx += 256) {
+            const int row = idx / CPR, col = idx - row * CPR;
+            const int co = OUT_BF16 ? row : (row >> 5) * 64 + pass * 32 + (row & 31);
+            const u32x4 v = *(const ZK_LDS u32x4 *)(smem + row * RS + col * 16);
+            *(u32x4 *)(ytile + (int64_t)co * plane * ES + col * 16) = v;
+        }
+    }
+}
+
 // F32_IN: f32 input, weights, bias and output on v_mfma_f32_32x32x2_f32 (a k step is 8 channels of one tap: lane half h
 // holds channels 4h .. 4h + 3 of the block, and the j-th of four matrix instructions multiplies channels j and 4 + j);
 // otherwise bf16 input on v_mfma_f32_32x32x16_bf16 (a k step is 16 channels of one tap). POOL: the tile leaves through a
@@ -88,47 +205,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_k(const void *__restrict__ x_,
     // lanes share lines, while the writes of one instruction still spread over 32 banks (pixels 8 apart are 32 banks
     // apart, 16 channel pairs are 16 consecutive words).
     if constexpr (!F32_IN) {
-        const uint16_t *x = (const uint16_t *)x_;
-        const int w8 = W >> 3;
-        constexpr int U = 9; // items whose reads are in flight together (one pass for 64 channels x 10 rows x 56 columns)
-        const int C2 = C >> 1, RC = (R + 2) * w8;          // channel pairs; 8-column pieces of one channel's rows
-        const int KB = (C2 & 15) ? 3 : 2;                  // log2(items of a row per wave instruction)
-        const int k = lane & ((1 << KB) - 1), cp_lo = lane >> KB, cp_lanes = 64 >> KB;
-        const int cpblocks = C2 / cp_lanes, groups = (RC + (1 << KB) - 1) >> KB, wave_items = cpblocks * groups;
-        const float inv_w8 = 1.0f / (float)w8;
-        const int64_t plane = (int64_t)H * W;
-        const uint16_t *xn = x + (int64_t)n * C * plane;
-        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-        for (int t0 = wave_u; t0 < wave_items; t0 += 4 * U) {
-            u32x4 va[U], vb[U];
-            int dsto[U];
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const int t = t0 + 4 * u;                   // uniform over the wave
-                const int g = t / cpblocks, cpb = t - g * cpblocks;
-                const int rc = (g << KB) + k, cp = cpb * cp_lanes + cp_lo;
-                const int r = small_div(rc, inv_w8), ch = rc - __mul24(r, w8);
-                const int iy = rb * R - 1 + r;
-                const bool live = t < wave_items && rc < RC;
-                va[u] = vb[u] = u32x4{0u, 0u, 0u, 0u};
-                if (live && iy >= 0 && iy < H) {
-                    const uint16_t *src = xn + (int64_t)(2 * cp) * plane + __mul24(iy, W) + ch * 8;
-                    va[u] = *(const u32x4 *)src;
-                    vb[u] = *(const u32x4 *)(src + plane);
-                }
-                dsto[u] = live ? __mul24(__mul24(r, Wp) + 1 + ch * 8, PS) + cp * 4 : -1;
-            }
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                if (dsto[u] < 0) continue;
-                ZK_LDS uint8_t *dst = smem + dsto[u];
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    *(ZK_LDS uint32_t *)(dst + (2 * e) * PS) = __builtin_amdgcn_perm(vb[u][e], va[u][e], 0x05040100u);
-                    *(ZK_LDS uint32_t *)(dst + (2 * e + 1) * PS) = __builtin_amdgcn_perm(vb[u][e], va[u][e], 0x07060302u);
-                }
-            }
-        }
+        load_tile_bf16<9>(smem, x_, n, rb, R, C, H, W, PS, lane, wave);
     } else {
         // f32: one item = 4 consecutive columns of one channel (16 bytes), four 4-byte LDS writes; the lanes of a wave take
         // 4 neighbouring items of a row for each of 16 channels (writes: pixels 4 apart are 16 banks apart for C = 64).
@@ -268,11 +345,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_k(const void *__restrict__ x_,
     // ---- epilogue: register r of lane l is pixel 8*(r/4) + 4*(l/32) + r%4 of block pb, channel l%32 of block nb --------
     constexpr int ES = OUT_BF16 ? 2 : 4;          // bytes per output element
     constexpr int RS = TILE_PIX * ES + 16;        // bytes per staged channel row
-    constexpr int CPR = TILE_PIX * ES / 16;       // 16-byte pieces per row
     constexpr int PASSES = OUT_BF16 ? 1 : 2;      // f32: one channel block (nb) per pass, 64 rows each
-    const int64_t plane = (int64_t)H * W;
-    // the tile's pixels are consecutive in the image plane
-    uint8_t *ytile = (uint8_t *)y + (((int64_t)n * Cout + co0) * plane + (int64_t)rb * R * W) * ES;
     __syncthreads(); // every wave has read its last input fragment
 #pragma unroll
     for (int pass = 0; pass < PASSES; pass++) {
@@ -306,60 +379,152 @@ __global__ __launch_bounds__(256, 1) void conv3x3_k(const void *__restrict__ x_,
                 }
         }
         __syncthreads();
-        constexpr int ROWS = OUT_BF16 ? 128 : 64;
-        if constexpr (POOL) {
-            // a channel's pooled tile is (R / 2) x (W / 2) = 112 values, consecutive in the pooled plane; a thread makes
-            // 16 bytes of them. The running maximum starts at the dtype's lowest finite value and takes the window in
-            // row order, like the separate pooling kernel.
-            constexpr int PV = TILE_PIX / 4, VPC = 16 / ES, PCR = PV / VPC;
-            const int W2 = W >> 1;
-            const float inv_w2 = 1.0f / (float)W2;
-            const float lowest = OUT_BF16 ? -3.3895313892515355e38f : -3.4028234663852886e38f;
-            const int64_t pplane = plane >> 2;
-            uint8_t *ptile = (uint8_t *)y + (((int64_t)n * Cout + co0) * pplane + (int64_t)rb * PV) * ES;
-            for (int idx = tid; idx < ROWS * PCR; idx += 256) {
-                const int row = idx / PCR, piece = idx - row * PCR;
-                const int co = OUT_BF16 ? row : (row >> 5) * 64 + pass * 32 + (row & 31);
-                float m[VPC];
-                int pr = small_div(piece * VPC, inv_w2), pc = piece * VPC - __mul24(pr, W2); // pooled row, column of value 0
-                const ZK_LDS uint8_t *rowp = smem + row * RS + __mul24(2 * pr, W) * ES;
+        copy_out<TILE_PIX, OUT_BF16, POOL>(smem, y, n, Cout, co0, H, W, rb, pass, tid);
+    }
+}
+
+// The same convolution for bf16 input with half the tile, two workgroups to a compute unit: a workgroup's phases
+// (fetch the tile, matrix loop, copy out) do not overlap one another, so a second resident workgroup fills the matrix
+// pipeline while the first one waits for memory. R * W = 224 pixels x 128 output channels; 4 waves as 2 pixel halves x 2
+// channel halves on v_mfma_f32_16x16x32_bf16: 7 pixel blocks x 4 channel blocks of 16 x 16 per wave = 112 accumulator
+// registers, and one LDS read still feeds four matrix instructions of 16 cycles (the ratio of the large tile). A k step
+// is 32 channels of one tap (C % 32 = 0): lane l holds pixel (or channel) l % 16 and channels 8 * (l / 16) .. + 7 of
+// the step; weights re-laid as [tap][C / 32][Cout][32]. Register r of lane l of a block is pixel 4 * (l / 16) + r,
+// channel l % 16.
+constexpr int SPB = 7;                     // 16-pixel blocks per wave
+constexpr int S_TILE_PIX = 2 * SPB * 16;   // 224
+constexpr int S_STAGE_BYTES = 128 * (S_TILE_PIX * 2 + 16);
+typedef float f32x4a __attribute__((ext_vector_type(4)));
+
+template <bool OUT_BF16, bool RELU, bool POOL>
+__global__ __launch_bounds__(256, 2) void conv3x3_half_k(const void *__restrict__ x_, const void *__restrict__ wt,
+                                                         const void *__restrict__ bias, void *__restrict__ y, int C, int H, int W,
+                                                         int Cout, int R) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
+    ZK_LDS uint8_t *smem = (ZK_LDS uint8_t *)smem_raw;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, quad = lane >> 4, l16 = lane & 15;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int tiles_per_image = H / R;
+    const int n = blockIdx.x / tiles_per_image, rb = blockIdx.x - n * tiles_per_image;
+    const int co0 = blockIdx.y * TILE_CO;
+    const int PS = C * 2 + 16;
+    const int Wp = W + 2;
+
+    load_tile_bf16<6>(smem, x_, n, rb, R, C, H, W, PS, lane, wave);
+    {
+        const int parts = C * 2 / 16, edge = (R + 2) * 2 * parts; // columns 0 and W + 1 of every row, 16 bytes at a time
+        for (int q = tid; q < edge; q += 256) {
+            const int part = q % parts, side = (q / parts) & 1, r = q / parts / 2;
+            *(ZK_LDS u32x4 *)(smem + (r * Wp + (side ? W + 1 : 0)) * PS + part * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+
+    int xoff[SPB];
+    {
+        const float inv_w = 1.0f / (float)W;
 #pragma unroll
-                for (int e = 0; e < VPC; e++) {
-                    const ZK_LDS uint8_t *src = rowp + 2 * pc * ES;
-                    if (++pc == W2) { // the next value starts the next pooled row
-                        pc = 0;
-                        rowp += 2 * W * ES;
-                    }
-                    float a0, a1, b0, b1;
-                    if (OUT_BF16) {
-                        const uint32_t u0 = *(const ZK_LDS uint32_t *)src, u1 = *(const ZK_LDS uint32_t *)(src + W * ES);
-                        a0 = __uint_as_float(u0 << 16), a1 = __uint_as_float(u0 & 0xffff0000u);
-                        b0 = __uint_as_float(u1 << 16), b1 = __uint_as_float(u1 & 0xffff0000u);
-                    } else {
-                        const u32x2 u0 = *(const ZK_LDS u32x2 *)src, u1 = *(const ZK_LDS u32x2 *)(src + W * ES);
-                        a0 = __uint_as_float(u0[0]), a1 = __uint_as_float(u0[1]), b0 = __uint_as_float(u1[0]), b1 = __uint_as_float(u1[1]);
-                    }
-                    m[e] = fmaxf(b1, fmaxf(b0, fmaxf(a1, fmaxf(a0, lowest))));
+        for (int pb = 0; pb < SPB; pb++) {
+            const int p = wm * (SPB * 16) + pb * 16 + l16, pr = small_div(p, inv_w), pc = p - __mul24(pr, W);
+            xoff[pb] = __mul24(__mul24(pr, Wp) + pc, PS) + quad * 16;
+        }
+    }
+    const int cblocks = C >> 5; // k steps per tap
+    // weight fragment of (tap, cb, nb): 16 bytes at ((tap * cblocks + cb) * Cout + co) * 64 + quad * 16
+    const uint8_t *wlane = (const uint8_t *)wt + ((int64_t)(co0 + wn * 64 + l16)) * 64 + quad * 16;
+    const int64_t wstep = (int64_t)Cout * 64;
+
+    f32x4a acc[4][SPB]; // [nb][pb]
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int co = co0 + wn * 64 + nb * 16 + l16;
+        const float bv = !bias ? 0.0f : bf16_to_f32(((const uint16_t *)bias)[co]);
+#pragma unroll
+        for (int pb = 0; pb < SPB; pb++) acc[nb][pb] = f32x4a{bv, bv, bv, bv};
+    }
+
+    // k step s: tap = s / cblocks, cb = s % cblocks. Weights and input fragments of a step are requested during the
+    // step before, into the other of two register sets.
+    const int steps = 9 * cblocks;
+    int tap = 0, cb = 0;
+    auto next_toff = [&]() {
+        const int tp = tap < 9 ? tap : 8, cc = tap < 9 ? cb : cblocks - 1;
+        const int ky = tp / 3, kx = tp - ky * 3;
+        if (++cb == cblocks) {
+            cb = 0;
+            tap++;
+        }
+        return (ky * Wp + kx) * PS + cc * 64;
+    };
+    auto load_w = [&](u32x4(&wf)[4], int s) {
+        const uint8_t *src = wlane + (s < steps ? s : steps - 1) * wstep;
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) wf[nb] = *(const u32x4 *)(src + nb * 16 * 64);
+    };
+    auto k_step = [&](const u32x4(&wf)[4], const u32x4(&xf)[SPB], u32x4(&xnext)[SPB]) {
+        const int toff = next_toff();
+#pragma unroll
+        for (int pb = 0; pb < SPB; pb++) xnext[pb] = *(const ZK_LDS u32x4 *)(smem + xoff[pb] + toff);
+#pragma unroll
+        for (int pb = 0; pb < SPB; pb++)
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++)
+                acc[nb][pb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xf[pb]), __builtin_bit_cast(bf16x8, wf[nb]), acc[nb][pb], 0, 0, 0);
+#pragma unroll
+        for (int pb = 0; pb < SPB; pb++) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        }
+    };
+    u32x4 w0[4], w1[4], xa[SPB], xb[SPB];
+    load_w(w0, 0);
+    __syncthreads(); // the tile is complete
+    {
+        const int toff = next_toff();
+#pragma unroll
+        for (int pb = 0; pb < SPB; pb++) xa[pb] = *(const ZK_LDS u32x4 *)(smem + xoff[pb] + toff);
+    }
+    for (int s = 0; s < steps; s += 2) {
+        load_w(w1, s + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        k_step(w0, xa, xb);
+        load_w(w0, s + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s + 1 < steps) k_step(w1, xb, xa); // uniform
+    }
+
+    // ---- epilogue ------------------------------------------------------------------------------------------------
+    constexpr int ES = OUT_BF16 ? 2 : 4;
+    constexpr int RS = S_TILE_PIX * ES + 16;
+    constexpr int PASSES = OUT_BF16 ? 1 : 2; // f32: two channel blocks per pass, 64 rows each
+    __syncthreads(); // every wave has read its last input fragment
+#pragma unroll
+    for (int pass = 0; pass < PASSES; pass++) {
+        if (pass) __syncthreads(); // the previous pass has been copied out
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+            if (!OUT_BF16 && (nb >> 1) != pass) continue;
+            const int row = OUT_BF16 ? wn * 64 + nb * 16 + l16 : wn * 32 + (nb & 1) * 16 + l16;
+            ZK_LDS uint8_t *dst = smem + row * RS + (wm * (SPB * 16) + 4 * quad) * ES;
+#pragma unroll
+            for (int pb = 0; pb < SPB; pb++) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    v[e] = acc[nb][pb][e];
+                    if (RELU) v[e] = (v[e] > 0.0f ? 1.0f : 0.0f) * v[e];
                 }
-                u32x4 v;
+                ZK_LDS uint8_t *d = dst + pb * 16 * ES;
                 if (OUT_BF16) {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) v[e] = __builtin_amdgcn_perm(__float_as_uint(m[(2 * e + 1) % VPC]), __float_as_uint(m[(2 * e) % VPC]), 0x07060302u);
+                    u32x2 pk = {__builtin_amdgcn_perm(__float_as_uint(v[1]), __float_as_uint(v[0]), 0x07060302u),
+                                __builtin_amdgcn_perm(__float_as_uint(v[3]), __float_as_uint(v[2]), 0x07060302u)};
+                    *(ZK_LDS u32x2 *)d = pk;
                 } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) v[e] = __float_as_uint(m[e % VPC]);
+                    *(ZK_LDS u32x4 *)d = u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])};
                 }
-                *(u32x4 *)(ptile + (int64_t)co * pplane * ES + piece * 16) = v;
             }
-            continue;
         }
-#pragma unroll 4
-        for (int idx = tid; idx < ROWS * CPR; idx += 256) {
-            const int row = idx / CPR, col = idx - row * CPR;
-            const int co = OUT_BF16 ? row : (row >> 5) * 64 + pass * 32 + (row & 31);
-            const u32x4 v = *(const ZK_LDS u32x4 *)(smem + row * RS + col * 16);
-            *(u32x4 *)(ytile + (int64_t)co * plane * ES + col * 16) = v;
-        }
+        __syncthreads();
+        copy_out<S_TILE_PIX, OUT_BF16, POOL>(smem, y, n, Cout, co0, H, W, rb, pass, tid);
     }
 }
 
@@ -368,12 +533,21 @@ int elem_bytes(const Conv2d &p) { return p.dtype == DT_F32 ? 4 : 2; }
 uint64_t lds_bytes(const Conv2d &p) { // the input tile, later reused for the staged output tile
     return std::max<uint64_t>((uint64_t)(tile_rows(p) + 2) * (p.W + 2) * (p.C * elem_bytes(p) + 16), STAGE_BYTES);
 }
-
+// the half-tile kernel: bf16, 32-channel k steps, whole rows in 224 pixels, two workgroups within a compute unit's LDS
+int half_rows(const Conv2d &p) { return p.W > 0 && S_TILE_PIX % p.W == 0 ? S_TILE_PIX / p.W : 0; }
+uint64_t half_lds_bytes(const Conv2d &p) {
+    return std::max<uint64_t>((uint64_t)(half_rows(p) + 2) * (p.W + 2) * (p.C * 2 + 16), S_STAGE_BYTES);
+}
+bool half_ok(const Conv2d &p) {
+    const int R = half_rows(p);
+    return p.dtype == DT_BF16 && p.C % 32 == 0 && R >= 1 && p.H % R == 0 && !(p.pool && R % 2) && half_lds_bytes(p) <= 80 * 1024 &&
+           (int64_t)p.N * (p.H / R) < (1ll << 31);
+}
 } // namespace
 
 bool conv3x3_direct_ok(const Conv2d &p) { // shape only: the same answer at registration and at every launch
     const int R = tile_rows(p);
-    if (p.pool && R % 2) return false; // pooling windows must not straddle two tiles
+    if (p.pool && R % 2) return false; // pooling windows must not straddle two tiles (either tile: half the rows otherwise)
     const bool types = (p.dtype == DT_BF16 && (p.out_dtype == DT_BF16 || p.out_dtype == DT_F32)) || (p.dtype == DT_F32 && p.out_dtype == DT_F32);
     return types && p.KH == 3 && p.KW == 3 && p.sy == 1 && p.sx == 1 && p.dy == 1 && p.dx == 1 && p.py == 1 && p.px == 1 && p.C >= 16 &&
            p.C % 16 == 0 && p.Cout % TILE_CO == 0 && p.W % 8 == 0 && R >= 1 && p.H % R == 0 && lds_bytes(p) <= 160 * 1024 && p.N > 0 &&
@@ -393,17 +567,25 @@ hipError_t conv3x3_init() {
 #undef ZK_V
     for (const void *f : variants)
         if (e == hipSuccess) e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+#define ZK_V(OB) (const void *)conv3x3_half_k<OB, false, false>, (const void *)conv3x3_half_k<OB, true, false>, \
+                 (const void *)conv3x3_half_k<OB, false, true>, (const void *)conv3x3_half_k<OB, true, true>
+    const void *halves[8] = {ZK_V(false), ZK_V(true)};
+#undef ZK_V
+    for (const void *f : halves)
+        if (e == hipSuccess) e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
     return e;
 }
 
 // `wt` holds conv3x3_scratch_bytes(p) bytes for the re-laid weights.
 hipError_t conv3x3_direct(const Conv2d &p, void *wt, hipStream_t st) {
     if ((uintptr_t)p.x % 16 || (uintptr_t)p.y % 16 || (uintptr_t)wt % 16) return hipErrorInvalidValue; // pool blocks are 256-byte aligned
-    const int R = tile_rows(p);
+    const bool half = half_ok(p); // by shape only: a program's launches all take the same kernel and weight layout
+    const int R = half ? half_rows(p) : tile_rows(p);
     const dim3 wgrid((unsigned)((p.C * p.Cout + 255) / 256));
     if (p.weights_ready) {
         // the caller knows that w has not been written since the launch that left its re-laid copy in wt
-    } else if (p.dtype == DT_F32) hipLaunchKernelGGL((conv3x3_weights_k<float, 3>), wgrid, dim3(256), 0, st, (const float *)p.w, (float *)wt, p.C, p.Cout);
+    } else if (half) hipLaunchKernelGGL((conv3x3_weights_k<uint16_t, 5>), wgrid, dim3(256), 0, st, (const uint16_t *)p.w, (uint16_t *)wt, p.C, p.Cout);
+    else if (p.dtype == DT_F32) hipLaunchKernelGGL((conv3x3_weights_k<float, 3>), wgrid, dim3(256), 0, st, (const float *)p.w, (float *)wt, p.C, p.Cout);
     else hipLaunchKernelGGL((conv3x3_weights_k<uint16_t, 4>), wgrid, dim3(256), 0, st, (const uint16_t *)p.w, (uint16_t *)wt, p.C, p.Cout);
     dim3 grid((unsigned)(p.N * (p.H / R)), (unsigned)(p.Cout / TILE_CO));
     const bool out_bf16 = p.out_dtype == DT_BF16;
@@ -417,7 +599,22 @@ hipError_t conv3x3_direct(const Conv2d &p, void *wt, hipStream_t st) {
         else if (p.pool) ZK_LAUNCH(FI, OB, false, true);                                                                          \
         else ZK_LAUNCH(FI, OB, false, false);                                                                                     \
     } while (0)
-    if (p.dtype == DT_F32) ZK_LAUNCH2(true, false);
+    if (half) {
+#define ZK_HALF(OB, RL, PL)                                                                                                       \
+    hipLaunchKernelGGL((conv3x3_half_k<OB, RL, PL>), grid, dim3(256), half_lds_bytes(p), st, p.x, (const void *)wt, p.bias, p.y, p.C, \
+                       p.H, p.W, p.Cout, R)
+#define ZK_HALF2(OB)                                                                                                              \
+    do {                                                                                                                          \
+        if (p.relu && p.pool) ZK_HALF(OB, true, true);                                                                            \
+        else if (p.relu) ZK_HALF(OB, true, false);                                                                                \
+        else if (p.pool) ZK_HALF(OB, false, true);                                                                                \
+        else ZK_HALF(OB, false, false);                                                                                           \
+    } while (0)
+        if (out_bf16) ZK_HALF2(true);
+        else ZK_HALF2(false);
+#undef ZK_HALF2
+#undef ZK_HALF
+    } else if (p.dtype == DT_F32) ZK_LAUNCH2(true, false);
     else if (out_bf16) ZK_LAUNCH2(false, true);
     else ZK_LAUNCH2(false, false);
 #undef ZK_LAUNCH2

@@ -92,6 +92,36 @@ template <int DT, int NV> struct RegRow {
         else IO::st4(p, (lane + 64 * j0) * 4, a);
     }
     static constexpr int STEP = WIDE ? 2 : 1; // vectors per access
+    // The lane's part of a row as it lies in memory (32-bit words), for a row fetched ahead of its use: 16-bit rows
+    // stay packed until unpack(), half the registers of their f32 form.
+    static constexpr int NW = NV * (int)sizeof(S);
+    static __device__ __forceinline__ void load_raw(const S *p, int lane, uint32_t (&r)[NW]) {
+        if constexpr (DT == 0 || WIDE) {
+#pragma unroll
+            for (int q = 0; q < NW / 4; q++) {
+                const uint4 t = *(const uint4 *)(p + (lane + 64 * q) * (16 / (int)sizeof(S)));
+                r[4 * q] = t.x; r[4 * q + 1] = t.y; r[4 * q + 2] = t.z; r[4 * q + 3] = t.w;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const uint2 t = *(const uint2 *)(p + (lane + 64 * j) * 4);
+                r[2 * j] = t.x; r[2 * j + 1] = t.y;
+            }
+        }
+    }
+    static __device__ __forceinline__ void unpack(const uint32_t (&r)[NW], float (&v)[NV][4]) {
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            if constexpr (DT == 0) {
+#pragma unroll
+                for (int k = 0; k < 4; k++) v[j][k] = __uint_as_float(r[4 * j + k]);
+            } else { // words 2j, 2j+1 hold vector j in both 16-bit layouts
+                v[j][0] = __uint_as_float(r[2 * j] << 16); v[j][1] = __uint_as_float(r[2 * j] & 0xffff0000u);
+                v[j][2] = __uint_as_float(r[2 * j + 1] << 16); v[j][3] = __uint_as_float(r[2 * j + 1] & 0xffff0000u);
+            }
+        }
+    }
 };
 
 // sum over one row of f(x[c]) with lanes striding over columns
@@ -214,7 +244,7 @@ __global__ __launch_bounds__(256) void norm_rows_reg_k(const typename RowIO<DT>:
 // running sums of dy*xh and dy for its 4*NV columns, the waves of a workgroup add theirs up through LDS in wave order
 // and the workgroup leaves one partial row pair in part[(blockIdx*2 + {0,1})*cols + c] for norm_bwd_param_sum_k.
 // The order of every sum is fixed by the launch shape: results are reproducible. part may be null (no dw / db).
-template <int DT, int MODE, int NV, int WAVES>
+template <int DT, int MODE, int NV, int WAVES, bool AHEAD>
 __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename RowIO<DT>::S *__restrict__ x,
                                                                 const typename RowIO<DT>::S *__restrict__ w,
                                                                 const typename RowIO<DT>::S *__restrict__ dy,
@@ -231,13 +261,38 @@ __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename R
     for (int j = 0; j < NV; j++)
 #pragma unroll
         for (int k = 0; k < 4; k++) pw[j][k] = pb[j][k] = 0.0f;
-    // (Fetching 16-bit rows one row ahead was tried: the 24 extra registers spill in a 16-wave workgroup and the
-    // kernel gets slower, 25.9 us against 18.7 us at 8192 x 1024.)
-    for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < rows; row += (int64_t)gridDim.x * WAVES) {
+    // AHEAD: the wave's next row (x, dy, add) is requested before the current one is worked on, in its memory form
+    // (f32 rows of 1024 in an 8-wave workgroup: 29.3 us against 32.5 us at 8192 rows; the registers this takes spill
+    // in a 16-wave workgroup, and 16-bit rows gain nothing from it).
+    const int64_t stride = (int64_t)gridDim.x * WAVES;
+    int64_t row = (int64_t)blockIdx.x * WAVES + wave;
+    uint32_t nx[RR::NW], ng[RR::NW], na[RR::NW];
+#pragma unroll
+    for (int i = 0; i < RR::NW; i++) na[i] = 0u;
+    if (AHEAD && row < rows) {
+        RR::load_raw(x + row * cols, lane, nx);
+        RR::load_raw(dy + row * cols, lane, ng);
+        if (add) RR::load_raw(add + row * cols, lane, na);
+    }
+    for (; row < rows; row += stride) {
         const int64_t base = row * cols;
         float xv[NV][4], g[NV][4];
-        RR::load(x + base, lane, xv);
-        RR::load(dy + base, lane, g);
+        uint32_t ca[RR::NW];
+        if constexpr (AHEAD) {
+            RR::unpack(nx, xv);
+            RR::unpack(ng, g);
+#pragma unroll
+            for (int i = 0; i < RR::NW; i++) ca[i] = na[i];
+            if (row + stride < rows) {
+                const int64_t nb = (row + stride) * cols;
+                RR::load_raw(x + nb, lane, nx);
+                RR::load_raw(dy + nb, lane, ng);
+                if (add) RR::load_raw(add + nb, lane, na);
+            }
+        } else {
+            RR::load(x + base, lane, xv);
+            RR::load(dy + base, lane, g);
+        }
         float mean = 0.0f, rstd;
         if (MODE == 0) {
             float s = 0.0f;
@@ -276,16 +331,22 @@ __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename R
         s1 = wave_allreduce_f32(s1, OpAdd());
         s2 = wave_allreduce_f32(s2, OpAdd());
         const float k1 = s1 / (float)cols, k2 = MODE == 0 ? s2 / (float)(cols - 1) : rstd * rstd * rstd * s2 / (float)cols;
+        float av[NV][4];
+        if constexpr (AHEAD) RR::unpack(ca, av); // zeros without add
 #pragma unroll
         for (int j0 = 0; j0 < NV; j0 += RR::STEP) {
-            float o[2][4], av[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
-            if (add) RR::load_at(add + base, lane, j0, av[0], av[1]);
+            float o[2][4];
+            if constexpr (!AHEAD) {
+#pragma unroll
+                for (int k = 0; k < 4; k++) av[j0][k] = av[j0 + RR::STEP - 1][k] = 0.0f;
+                if (add) RR::load_at(add + base, lane, j0, av[j0], av[j0 + RR::STEP - 1]);
+            }
 #pragma unroll
             for (int h = 0; h < RR::STEP; h++)
 #pragma unroll
                 for (int k = 0; k < 4; k++) {
                     const int j = j0 + h;
-                    o[h][k] = (MODE == 0 ? rstd * ((g[j][k] - k1) - ((xv[j][k] - mean) * rstd) * k2) : rstd * g[j][k] - xv[j][k] * k2) + av[h][k];
+                    o[h][k] = (MODE == 0 ? rstd * ((g[j][k] - k1) - ((xv[j][k] - mean) * rstd) * k2) : rstd * g[j][k] - xv[j][k] * k2) + av[j][k];
                 }
             RR::store_at(dx + base, lane, j0, o[0], o[1]);
         }
@@ -535,13 +596,14 @@ __global__ __launch_bounds__(1024) void norm_bwd_param_sum_k(const float *__rest
 int norm_bwd_chunks(int64_t rows) { return (int)(rows < 256 * 32 ? (rows + 31) / 32 : 256); }
 // the fused register kernel: one workgroup per CU's worth of waves, at most 256 partial row pairs
 constexpr int kFusedBlocks = 256;
-template <int NV> constexpr int fused_waves() { return NV <= 4 ? 16 : 8; }
+template <int DT, int NV> constexpr bool fused_ahead() { return DT == 0 && NV == 4; }
+template <int DT, int NV> constexpr int fused_waves() { return NV <= 4 && !fused_ahead<DT, NV>() ? 16 : 8; }
 
 template <int DT, int MODE, int NV> void launch_norm_bwd_reg(const NormRowsBwd &p, float *part, int &chunks, hipStream_t st) {
     typedef typename RowIO<DT>::S S;
-    constexpr int WAVES = fused_waves<NV>();
+    constexpr int WAVES = fused_waves<DT, NV>();
     chunks = (int)((p.rows + WAVES - 1) / WAVES < kFusedBlocks ? (p.rows + WAVES - 1) / WAVES : kFusedBlocks);
-    hipLaunchKernelGGL((norm_bwd_dx_reg_k<DT, MODE, NV, WAVES>), dim3((unsigned)chunks), dim3(WAVES * 64), 0, st, (const S *)p.x,
+    hipLaunchKernelGGL((norm_bwd_dx_reg_k<DT, MODE, NV, WAVES, fused_ahead<DT, NV>()>), dim3((unsigned)chunks), dim3(WAVES * 64), 0, st, (const S *)p.x,
                        (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, (p.dw || p.db) ? part : nullptr, p.rows, p.eps);
 }
 
