@@ -583,33 +583,29 @@ __global__ __launch_bounds__(256) void norm_bwd_param_k(const typename RowIO<DT>
         }
     }
 }
-// lane -> column of a 64-column strip, the 16 waves split the chunks (independent loads, a few per wave)
+// A workgroup folds one of the two partial rows (blockIdx.y: 0 dw, 1 db) over 32 columns: lane % 32 -> column, the 32
+// half-waves split the chunks (a few independent loads each), LDS joins them in a fixed order.
 template <int DT>
 __global__ __launch_bounds__(1024) void norm_bwd_param_sum_k(const float *__restrict__ part, typename RowIO<DT>::S *__restrict__ dw,
                                                              typename RowIO<DT>::S *__restrict__ db, int cols, int chunks) {
-    __shared__ float lds[16][2][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int c = blockIdx.x * 64 + lane;
-    float sw = 0.0f, sb = 0.0f;
+    __shared__ float lds[32][32];
+    const int which = blockIdx.y;
+    typename RowIO<DT>::S *out = which ? db : dw;
+    if (!out) return; // uniform over the workgroup
+    const int lane = threadIdx.x & 63, l32 = lane & 31, grp = (threadIdx.x >> 6) * 2 + (lane >> 5);
+    const int c = blockIdx.x * 32 + l32;
+    float s = 0.0f;
     if (c < cols) {
 #pragma unroll 8
-        for (int k = wave; k < chunks; k += 16) {
-            sw += part[((int64_t)k * 2) * cols + c];
-            sb += part[((int64_t)k * 2 + 1) * cols + c];
-        }
+        for (int k = grp; k < chunks; k += 32) s += part[((int64_t)k * 2 + which) * cols + c];
     }
-    lds[wave][0][lane] = sw;
-    lds[wave][1][lane] = sb;
+    lds[grp][l32] = s;
     __syncthreads();
-    if (wave == 0 && c < cols) {
-        float tw = 0.0f, tb = 0.0f;
+    if (threadIdx.x < 32 && c < cols) {
+        float t = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            tw += lds[v][0][lane];
-            tb += lds[v][1][lane];
-        }
-        if (dw) RowIO<DT>::st(dw, c, tw);
-        if (db) RowIO<DT>::st(db, c, tb);
+        for (int v = 0; v < 32; v++) t += lds[v][threadIdx.x];
+        RowIO<DT>::st(out, c, t);
     }
 }
 
@@ -649,7 +645,7 @@ template <int DT, int MODE> hipError_t launch_norm_bwd(const NormRowsBwd &p, hip
             if (vec) hipLaunchKernelGGL((norm_bwd_param_k<DT, true>), dim3((unsigned)((p.cols + 255) / 256), (unsigned)chunks), block, 0, st, (const S *)p.x, (const S *)p.dy, stats, part, p.rows, (int)p.cols, rpc);
             else hipLaunchKernelGGL((norm_bwd_param_k<DT, false>), dim3((unsigned)((p.cols + 63) / 64), (unsigned)chunks), block, 0, st, (const S *)p.x, (const S *)p.dy, stats, part, p.rows, (int)p.cols, rpc);
         }
-        hipLaunchKernelGGL((norm_bwd_param_sum_k<DT>), dim3((unsigned)((p.cols + 63) / 64)), dim3(1024), 0, st, part, (S *)p.dw, (S *)p.db, (int)p.cols, chunks);
+        hipLaunchKernelGGL((norm_bwd_param_sum_k<DT>), dim3((unsigned)((p.cols + 31) / 32), 2), dim3(1024), 0, st, part, (S *)p.dw, (S *)p.db, (int)p.cols, chunks);
     }
     return hipGetLastError();
 }
