@@ -396,7 +396,7 @@ constexpr int S_TILE_PIX = 2 * SPB * 16;   // 224
 constexpr int S_STAGE_BYTES = 128 * (S_TILE_PIX * 2 + 16);
 typedef float f32x4a __attribute__((ext_vector_type(4)));
 
-template <bool OUT_BF16, bool RELU, bool POOL>
+template <bool OUT_BF16, bool RELU, bool POOL, int CB>
 __global__ __launch_bounds__(256, 2) void conv3x3_half_k(const void *__restrict__ x_, const void *__restrict__ wt,
                                                          const void *__restrict__ bias, void *__restrict__ y, int C, int H, int W,
                                                          int Cout, int R) {
@@ -410,7 +410,6 @@ __global__ __launch_bounds__(256, 2) void conv3x3_half_k(const void *__restrict_
     const int PS = C * 2 + 16;
     const int Wp = W + 2;
 
-    load_tile_bf16<6>(smem, x_, n, rb, R, C, H, W, PS, lane, wave);
     {
         const int parts = C * 2 / 16, edge = (R + 2) * 2 * parts; // columns 0 and W + 1 of every row, 16 bytes at a time
         for (int q = tid; q < edge; q += 256) {
@@ -430,8 +429,13 @@ __global__ __launch_bounds__(256, 2) void conv3x3_half_k(const void *__restrict_
     }
     const int cblocks = C >> 5; // k steps per tap
     // weight fragment of (tap, cb, nb): 16 bytes at ((tap * cblocks + cb) * Cout + co) * 64 + quad * 16
-    const uint8_t *wlane = (const uint8_t *)wt + ((int64_t)(co0 + wn * 64 + l16)) * 64 + quad * 16;
-    const int64_t wstep = (int64_t)Cout * 64;
+    // (buffer loads: a fixed 32-bit lane offset plus a scalar offset that moves with the step, so the loads need no
+    // address registers of their own, which the allocator would otherwise recycle from a load still in flight and
+    // wait for it)
+    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((const uint8_t *)wt + (int64_t)co0 * 64), 0, (int)((int64_t)9 * C * Cout * 2 - (int64_t)co0 * 64), 0x00020000);
+    const int wl = (wn * 64 + l16) * 64 + quad * 16;
+    const int wstep = Cout * 64;
 
     f32x4a acc[4][SPB]; // [nb][pb]
 #pragma unroll
@@ -442,54 +446,95 @@ __global__ __launch_bounds__(256, 2) void conv3x3_half_k(const void *__restrict_
         for (int pb = 0; pb < SPB; pb++) acc[nb][pb] = f32x4a{bv, bv, bv, bv};
     }
 
-    // k step s: tap = s / cblocks, cb = s % cblocks. Weights and input fragments of a step are requested during the
-    // step before, into the other of two register sets.
+    // k step s: tap = s / cblocks, cb = s % cblocks. The input fragments of a step are read from LDS during the step
+    // before, into the other of two register sets; the weights of a step are requested three steps before their use
+    // (an L2 round trip is longer than one step's matrix instructions), the first three before the input tile is
+    // fetched. CB > 0: C = 32 * CB and the 9 * CB steps are unrolled, so that the tile and weight offsets of a step
+    // are constants of the launch and a step is little more than its matrix instructions, seven LDS reads and four
+    // loads (one wave per SIMD issues everything in order: at ~90 instructions per step the matrix pipe waited for
+    // the scalar bookkeeping of the looping form, 717 cycles per step against 448 of matrix instructions).
     const int steps = 9 * cblocks;
-    int tap = 0, cb = 0;
-    auto next_toff = [&]() {
-        const int tp = tap < 9 ? tap : 8, cc = tap < 9 ? cb : cblocks - 1;
-        const int ky = tp / 3, kx = tp - ky * 3;
-        if (++cb == cblocks) {
-            cb = 0;
-            tap++;
-        }
-        return (ky * Wp + kx) * PS + cc * 64;
-    };
-    auto load_w = [&](u32x4(&wf)[4], int s) {
-        const uint8_t *src = wlane + (s < steps ? s : steps - 1) * wstep;
+    auto read_x = [&](u32x4(&xf)[SPB], int toff) {
 #pragma unroll
-        for (int nb = 0; nb < 4; nb++) wf[nb] = *(const u32x4 *)(src + nb * 16 * 64);
+        for (int pb = 0; pb < SPB; pb++) xf[pb] = *(const ZK_LDS u32x4 *)(smem + xoff[pb] + toff);
     };
-    auto k_step = [&](const u32x4(&wf)[4], const u32x4(&xf)[SPB], u32x4(&xnext)[SPB]) {
-        const int toff = next_toff();
+    auto load_w = [&](u32x4(&wf)[4], int s) { // s < steps, uniform
+        const int soff = s * wstep;
 #pragma unroll
-        for (int pb = 0; pb < SPB; pb++) xnext[pb] = *(const ZK_LDS u32x4 *)(smem + xoff[pb] + toff);
+        for (int nb = 0; nb < 4; nb++) wf[nb] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wl + nb * 16 * 64, soff, 0));
+    };
+    auto multiply = [&](const u32x4(&wf)[4], const u32x4(&xf)[SPB]) {
 #pragma unroll
         for (int pb = 0; pb < SPB; pb++)
 #pragma unroll
             for (int nb = 0; nb < 4; nb++)
                 acc[nb][pb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xf[pb]), __builtin_bit_cast(bf16x8, wf[nb]), acc[nb][pb], 0, 0, 0);
 #pragma unroll
-        for (int pb = 0; pb < SPB; pb++) {
+        for (int pb = 0; pb < SPB; pb++) { // issue order: one LDS read of the next step, four matrix instructions
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
         }
     };
-    u32x4 w0[4], w1[4], xa[SPB], xb[SPB];
-    load_w(w0, 0);
+    u32x4 wq[4][4], xq[2][SPB];
+    load_w(wq[0], 0);
+    load_w(wq[1], 1);
+    load_w(wq[2], 2);
+    load_tile_bf16<6>(smem, x_, n, rb, R, C, H, W, PS, lane, wave);
     __syncthreads(); // the tile is complete
-    {
-        const int toff = next_toff();
+    read_x(xq[0], 0);
+    if constexpr (CB > 0) {
+        constexpr int STEPS = 9 * CB;
+        auto toff_of = [&](int s) { // constant folding leaves a few scalar instructions per step
+            const int tp = s / CB, cc = s - tp * CB, ky = tp / 3, kx = tp - ky * 3;
+            return (ky * Wp + kx) * PS + cc * 64;
+        };
 #pragma unroll
-        for (int pb = 0; pb < SPB; pb++) xa[pb] = *(const ZK_LDS u32x4 *)(smem + xoff[pb] + toff);
-    }
-    for (int s = 0; s < steps; s += 2) {
-        load_w(w1, s + 1);
-        __builtin_amdgcn_sched_barrier(0);
-        k_step(w0, xa, xb);
-        load_w(w0, s + 2);
-        __builtin_amdgcn_sched_barrier(0);
-        if (s + 1 < steps) k_step(w1, xb, xa); // uniform
+        for (int s = 0; s < STEPS; s++) {
+            if (s + 3 < STEPS) load_w(wq[(s + 3) & 3], s + 3);
+            __builtin_amdgcn_sched_barrier(0);
+            if (s + 1 < STEPS) read_x(xq[(s + 1) & 1], toff_of(s + 1));
+            multiply(wq[s & 3], xq[s & 1]);
+        }
+    } else {
+        int cb = 0, kx = 0, ky = 0, toff = 0; // of the step whose fragments are read next
+        auto next_toff = [&]() {
+            toff += 64;
+            if (++cb == cblocks) {
+                cb = 0;
+                toff += PS - cblocks * 64;
+                if (++kx == 3) {
+                    kx = 0;
+                    toff += (Wp - 3) * PS;
+                    ++ky;
+                }
+            }
+            return ky < 3 ? toff : 0; // past the last step: any address inside the tile
+        };
+        auto k_step = [&](int s, const u32x4(&wf)[4], const u32x4(&xf)[SPB], u32x4(&xnext)[SPB]) {
+            read_x(xnext, next_toff());
+            multiply(wf, xf);
+        };
+        auto ahead = [&](u32x4(&wf)[4], int s) { load_w(wf, s < steps ? s : steps - 1); };
+        for (int s = 0; s < steps; s += 4) { // the tests on s are uniform
+            ahead(wq[3], s + 3);
+            __builtin_amdgcn_sched_barrier(0);
+            k_step(s, wq[0], xq[0], xq[1]);
+            if (s + 1 < steps) {
+                ahead(wq[0], s + 4);
+                __builtin_amdgcn_sched_barrier(0);
+                k_step(s + 1, wq[1], xq[1], xq[0]);
+            }
+            if (s + 2 < steps) {
+                ahead(wq[1], s + 5);
+                __builtin_amdgcn_sched_barrier(0);
+                k_step(s + 2, wq[2], xq[0], xq[1]);
+            }
+            if (s + 3 < steps) {
+                ahead(wq[2], s + 6);
+                __builtin_amdgcn_sched_barrier(0);
+                k_step(s + 3, wq[3], xq[1], xq[0]);
+            }
+        }
     }
 
     // ---- epilogue ------------------------------------------------------------------------------------------------
@@ -567,9 +612,9 @@ hipError_t conv3x3_init() {
 #undef ZK_V
     for (const void *f : variants)
         if (e == hipSuccess) e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-#define ZK_V(OB) (const void *)conv3x3_half_k<OB, false, false>, (const void *)conv3x3_half_k<OB, true, false>, \
-                 (const void *)conv3x3_half_k<OB, false, true>, (const void *)conv3x3_half_k<OB, true, true>
-    const void *halves[8] = {ZK_V(false), ZK_V(true)};
+#define ZK_V(OB, CB) (const void *)conv3x3_half_k<OB, false, false, CB>, (const void *)conv3x3_half_k<OB, true, false, CB>, \
+                     (const void *)conv3x3_half_k<OB, false, true, CB>, (const void *)conv3x3_half_k<OB, true, true, CB>
+    const void *halves[24] = {ZK_V(false, 0), ZK_V(true, 0), ZK_V(false, 2), ZK_V(true, 2), ZK_V(false, 4), ZK_V(true, 4)};
 #undef ZK_V
     for (const void *f : halves)
         if (e == hipSuccess) e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
@@ -600,9 +645,15 @@ hipError_t conv3x3_direct(const Conv2d &p, void *wt, hipStream_t st) {
         else ZK_LAUNCH(FI, OB, false, false);                                                                                     \
     } while (0)
     if (half) {
+#define ZK_HALF_CB(OB, RL, PL, CB)                                                                                                \
+    hipLaunchKernelGGL((conv3x3_half_k<OB, RL, PL, CB>), grid, dim3(256), half_lds_bytes(p), st, p.x, (const void *)wt, p.bias, p.y, \
+                       p.C, p.H, p.W, p.Cout, R)
 #define ZK_HALF(OB, RL, PL)                                                                                                       \
-    hipLaunchKernelGGL((conv3x3_half_k<OB, RL, PL>), grid, dim3(256), half_lds_bytes(p), st, p.x, (const void *)wt, p.bias, p.y, p.C, \
-                       p.H, p.W, p.Cout, R)
+    do {                                                                                                                          \
+        if (p.C == 64) ZK_HALF_CB(OB, RL, PL, 2);                                                                                 \
+        else if (p.C == 128) ZK_HALF_CB(OB, RL, PL, 4);                                                                           \
+        else ZK_HALF_CB(OB, RL, PL, 0);                                                                                           \
+    } while (0)
 #define ZK_HALF2(OB)                                                                                                              \
     do {                                                                                                                          \
         if (p.relu && p.pool) ZK_HALF(OB, true, true);                                                                            \
@@ -614,6 +665,7 @@ hipError_t conv3x3_direct(const Conv2d &p, void *wt, hipStream_t st) {
         else ZK_HALF2(false);
 #undef ZK_HALF2
 #undef ZK_HALF
+#undef ZK_HALF_CB
     } else if (p.dtype == DT_F32) ZK_LAUNCH2(true, false);
     else if (out_bf16) ZK_LAUNCH2(false, true);
     else ZK_LAUNCH2(false, false);
