@@ -66,16 +66,20 @@ __device__ __forceinline__ int small_div(int q, float inv) { return (int)(((floa
 template <int U>
 __device__ __forceinline__ void load_tile_bf16(ZK_LDS uint8_t *smem, const void *x_, int n, int rb, int R, int C, int H, int W,
                                                int PS, int lane, int wave) {
+    // Buffer loads with 32-bit byte offsets from the image's first element (conv3x3_direct_ok bounds the tensor by
+    // 2^31 elements): no 64-bit address arithmetic, and an item outside the image or past the end of the list gets
+    // an offset beyond the buffer, for which the load returns zeros without a branch.
     const int Wp = W + 2;
-    const uint16_t *x = (const uint16_t *)x_;
     const int w8 = W >> 3;
     const int C2 = C >> 1, RC = (R + 2) * w8;          // channel pairs; 8-column pieces of one channel's rows
     const int KB = (C2 & 15) ? 3 : 2;                  // log2(items of a row per wave instruction)
     const int k = lane & ((1 << KB) - 1), cp_lo = lane >> KB, cp_lanes = 64 >> KB;
     const int cpblocks = C2 / cp_lanes, groups = (RC + (1 << KB) - 1) >> KB, wave_items = cpblocks * groups;
-    const float inv_w8 = 1.0f / (float)w8;
-    const int64_t plane = (int64_t)H * W;
-    const uint16_t *xn = x + (int64_t)n * C * plane;
+    const float inv_w8 = 1.0f / (float)w8, inv_cpb = 1.0f / (float)cpblocks;
+    const int plane = H * W;
+    const uint32_t image_bytes = (uint32_t)C * (uint32_t)plane * 2u;
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((const uint16_t *)x_ + (int64_t)n * C * plane), 0, (int)image_bytes, 0x00020000);
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     for (int t0 = wave_u; t0 < wave_items; t0 += 4 * U) {
         u32x4 va[U], vb[U];
@@ -83,17 +87,15 @@ __device__ __forceinline__ void load_tile_bf16(ZK_LDS uint8_t *smem, const void 
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int t = t0 + 4 * u;                   // uniform over the wave
-            const int g = t / cpblocks, cpb = t - g * cpblocks;
+            const int g = small_div(t, inv_cpb), cpb = t - g * cpblocks;
             const int rc = (g << KB) + k, cp = cpb * cp_lanes + cp_lo;
             const int r = small_div(rc, inv_w8), ch = rc - __mul24(r, w8);
             const int iy = rb * R - 1 + r;
             const bool live = t < wave_items && rc < RC;
-            va[u] = vb[u] = u32x4{0u, 0u, 0u, 0u};
-            if (live && iy >= 0 && iy < H) {
-                const uint16_t *src = xn + (int64_t)(2 * cp) * plane + __mul24(iy, W) + ch * 8;
-                va[u] = *(const u32x4 *)src;
-                vb[u] = *(const u32x4 *)(src + plane);
-            }
+            const bool inside = live && iy >= 0 && iy < H;
+            const uint32_t off = (uint32_t)(__mul24(2 * cp, plane) + __mul24(iy, W) + ch * 8) * 2u;
+            va[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(inside ? off : 0xfffffff0u), 0, 0));
+            vb[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(inside ? off + (uint32_t)plane * 2u : 0xfffffff0u), 0, 0));
             dsto[u] = live ? __mul24(__mul24(r, Wp) + 1 + ch * 8, PS) + cp * 4 : -1;
         }
 #pragma unroll
