@@ -66,8 +66,8 @@ __device__ __forceinline__ int small_div(int q, float inv) { return (int)(((floa
 template <int U>
 __device__ __forceinline__ void load_tile_bf16(ZK_LDS uint8_t *smem, const void *x_, int n, int rb, int R, int C, int H, int W,
                                                int PS, int lane, int wave) {
-    // Buffer loads with 32-bit byte offsets from the image's first element (conv3x3_direct_ok bounds the tensor by
-    // 2^31 elements): no 64-bit address arithmetic, and an item outside the image or past the end of the list gets
+    // Buffer loads with 32-bit byte offsets from the image's first element (conv3x3_direct_ok bounds an image by
+    // 2^32 bytes): no 64-bit address arithmetic, and an item outside the image or past the end of the list gets
     // an offset beyond the buffer, for which the load returns zeros without a branch.
     const int Wp = W + 2;
     const int w8 = W >> 3;
@@ -93,7 +93,7 @@ __device__ __forceinline__ void load_tile_bf16(ZK_LDS uint8_t *smem, const void 
             const int iy = rb * R - 1 + r;
             const bool live = t < wave_items && rc < RC;
             const bool inside = live && iy >= 0 && iy < H;
-            const uint32_t off = (uint32_t)(__mul24(2 * cp, plane) + __mul24(iy, W) + ch * 8) * 2u;
+            const uint32_t off = (uint32_t)(2 * cp * plane + __mul24(iy, W) + ch * 8) * 2u; // (a plane may exceed 24 bits)
             va[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(inside ? off : 0xfffffff0u), 0, 0));
             vb[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(inside ? off + (uint32_t)plane * 2u : 0xfffffff0u), 0, 0));
             dsto[u] = live ? __mul24(__mul24(r, Wp) + 1 + ch * 8, PS) + cp * 4 : -1;
@@ -211,14 +211,15 @@ __global__ __launch_bounds__(256, 1) void conv3x3_k(const void *__restrict__ x_,
     } else {
         // f32: one item = 4 consecutive columns of one channel (16 bytes), four 4-byte LDS writes; the lanes of a wave take
         // 4 neighbouring items of a row for each of 16 channels (writes: pixels 4 apart are 16 banks apart for C = 64).
-        const float *x = (const float *)x_;
+        // (buffer loads with 32-bit byte offsets within the image, as in load_tile_bf16)
         constexpr int U = 12;
         const int w4 = W >> 2, RC = (R + 2) * w4;
         const int k = lane & 3, c_lo = lane >> 2;
         const int cblocks16 = C >> 4, groups = (RC + 3) >> 2, wave_items = cblocks16 * groups;
-        const float inv_w4 = 1.0f / (float)w4;
-        const int64_t plane = (int64_t)H * W;
-        const float *xn = x + (int64_t)n * C * plane;
+        const float inv_w4 = 1.0f / (float)w4, inv_cb16 = 1.0f / (float)cblocks16;
+        const int plane = H * W;
+        const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)((const float *)x_ + (int64_t)n * C * plane), 0, (int)((uint32_t)C * (uint32_t)plane * 4u), 0x00020000);
         const int wave_u = __builtin_amdgcn_readfirstlane(wave);
         for (int t0 = wave_u; t0 < wave_items; t0 += 4 * U) {
             u32x4 v[U];
@@ -226,13 +227,13 @@ __global__ __launch_bounds__(256, 1) void conv3x3_k(const void *__restrict__ x_,
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const int t = t0 + 4 * u;                   // uniform over the wave
-                const int g = t / cblocks16, cbk = t - g * cblocks16;
+                const int g = small_div(t, inv_cb16), cbk = t - g * cblocks16;
                 const int rc = (g << 2) + k, c = cbk * 16 + c_lo;
                 const int r = small_div(rc, inv_w4), pc = rc - __mul24(r, w4);
                 const int iy = rb * R - 1 + r;
                 const bool live = t < wave_items && rc < RC;
-                v[u] = u32x4{0u, 0u, 0u, 0u};
-                if (live && iy >= 0 && iy < H) v[u] = *(const u32x4 *)(xn + (int64_t)c * plane + __mul24(iy, W) + pc * 4);
+                const uint32_t off = (uint32_t)(c * plane + __mul24(iy, W) + pc * 4) * 4u; // (a plane may exceed 24 bits)
+                v[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(live && iy >= 0 && iy < H ? off : 0xfffffff0u), 0, 0));
                 dsto[u] = live ? __mul24(__mul24(r, Wp) + 1 + pc * 4, PS) + c * 4 : -1;
             }
 #pragma unroll
@@ -600,7 +601,8 @@ bool conv3x3_direct_ok(const Conv2d &p) { // shape only: the same answer at regi
            p.C % 16 == 0 && p.Cout % TILE_CO == 0 && p.W % 8 == 0 && R >= 1 && p.H % R == 0 && lds_bytes(p) <= 160 * 1024 && p.N > 0 &&
            (int64_t)p.N * (p.H / R) < (1ll << 31) && p.Cout / TILE_CO <= 65535 && (int64_t)p.N * p.C * p.H * p.W < (1ll << 31) &&
            (int64_t)p.N * p.Cout * p.H * p.W < (1ll << 40) && (int64_t)p.C * p.Cout < (1ll << 26) &&
-           p.H < (1 << 22); // row numbers go through 24-bit multiplies
+           p.H < (1 << 22) && // row numbers go through 24-bit multiplies
+           (int64_t)p.C * p.H * p.W * elem_bytes(p) < (1ll << 32); // 32-bit byte offsets within an image
 }
 
 uint64_t conv3x3_scratch_bytes(const Conv2d &p) { return (uint64_t)9 * p.C * p.Cout * elem_bytes(p); }
