@@ -77,7 +77,8 @@ def test_cross_entropy(hip, oracle):
 
 
 # ---- gradients of the norms ---------------------------------------------------------------------------------
-@pytest.mark.parametrize("shape", [(5, 9), (64, 128), (130, 1024), (3, 1000), (2100, 64), (64, 256), (7, 512), (9, 2048)])
+@pytest.mark.parametrize("shape", [(5, 9), (64, 128), (130, 1024), (3, 1000), (2100, 64), (64, 256), (7, 512), (9, 2048),
+                                   (8192, 1024), (4099, 1024), (2051, 512)])  # several rows per wave: rows fetched ahead
 @pytest.mark.parametrize("rms", [False, True])
 def test_norm_backward_f32(hip, oracle, shape, rms):
     from zyx_amd.kernels import norm_rows_bwd
