@@ -207,6 +207,9 @@ def extra_streaming(dev, pool, kernels, steps=20, warmup=5):
         a, b = c.input(dt), c.input(dt)
         c.load(a).add(b)
         timeit(f"add_{tag}_8192x4096", c.desc(), lambda: [full(), full(), out_arr(M * F, isz)], 3 * M * F * isz)
+        # the fused softmax (y, row sum, arg-max) on this storage type: x read once, y written once
+        timeit(f"softmax_{tag}_8192x4096", kernels.softmax_rows_desc(M, F, dtype=dt),
+               lambda: [full(), out_arr(M * F, isz), out_arr(M, isz), out_arr(M, 4)], 2 * M * F * isz + M * (isz + 4))
         timeit(f"colsum_{tag}_8192x4096", kernels.reduce_desc(M, F, "sum", axis0=True, dtype=dt), lambda: [full(), out_arr(F, isz)], M * F * isz)
         timeit(f"rowsum_{tag}_8192x4096", kernels.reduce_desc(M, F, "sum", dtype=dt), lambda: [full(), out_arr(M, isz)], M * F * isz)
         c = kernels.Chain(M, D, out_dtype=dt)

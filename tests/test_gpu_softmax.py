@@ -174,7 +174,8 @@ def test_undersized_argument_is_rejected(hip):
 # ---- 16-bit storage -----------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dt", ["bf16", "f16"])
 @pytest.mark.parametrize("shape", [(1, 1), (5, 10), (64, 252), (33, 256), (9, 1000), (130, 1024), (6, 4092), (5, 4096), (3, 4097),
-                                   (2, 16384), (2048, 320)])
+                                   (2, 16384), (2048, 320),
+                                   (1025, 1024), (1024, 2048), (2050, 4096), (1027, 8192)])  # rows split over the waves of a workgroup
 def test_sixteen_bit_storage(hip, oracle, shape, dt):
     """bf16 / f16 rows: elements widen to f32 registers, y is truncated on store, the row sum and the argmax read the stored
     y (zyx/src/codegen/c.rs:456-497, 491-496). Against the oracle's restatement: the device's exp differs from expf in the
@@ -187,7 +188,14 @@ def test_sixteen_bit_storage(hip, oracle, shape, dt):
     y, s, a = kernels.softmax_rows(dev, pool, x, dtype=dtype)
     yo, so, ao = oracle.softmax_rows(x, dtype=code)
     yf, yof = to32(y).astype(np.float64), to32(yo).astype(np.float64)
-    assert np.all(np.abs(yf - yof) <= ulp * yof + (1e-37 if dt == "bf16" else 6e-8))  # at most one step (f16: one subnormal step)
+    close = np.abs(yf - yof) <= ulp * yof + (1e-37 if dt == "bf16" else 6e-8)  # at most one step (f16: one subnormal step)
+    if dt == "f16":
+        # the reference's f32 -> f16 conversion gives 0 below 2^-14 (no subnormals): a y whose f32 value lies within a few
+        # ulps of 2^-14 is stored as 2^-14 by one side and as 0 by the other
+        cliff = ((yf == 0) & (yof == 2.0 ** -14)) | ((yof == 0) & (yf == 2.0 ** -14))
+        assert cliff.sum() <= max(1, y.size // 100000)
+        close |= cliff
+    assert np.all(close)
     assert np.mean(y == yo) > 0.98
     # the row sum of the stored values, itself stored truncated: a few steps of the 16-bit format around the oracle's
     assert np.all(np.abs(to32(s).astype(np.float64) - to32(so)) <= 4 * ulp)

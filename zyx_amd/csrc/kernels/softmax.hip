@@ -314,11 +314,129 @@ __global__ __launch_bounds__(256) void softmax_rows_generic16_k(const uint16_t *
     }
 }
 
+// 16-bit rows split over W waves of a workgroup, NVL 16-byte vectors (8 elements) per lane: cols == 512 * NVL * W
+// exactly. A wave's requests cover NVL KiB of consecutive bytes (2 KiB at 4096 columns). For bf16 the exponential is
+// one multiply and one v_exp_f32: its relative error (about |x - max| * 6e-8) is far below the step of an 8-bit
+// mantissa, so the truncated y differs from the long form's in one element of several thousand, always by one step; the
+// eight-instruction form makes a kernel that moves half the bytes of the f32 one as slow as it (42 us at 8192 x 4096).
+// f16 keeps the long form: below 2^-14 its conversion gives 0, a cliff of a whole step at which a 1e-6 error shows.
+template <int DT, int NVL, int W>
+__global__ __launch_bounds__(W < 4 ? 256 : 64 * W) void softmax_rows_split16_k(const uint16_t *__restrict__ x, uint16_t *__restrict__ y,
+                                                                              uint16_t *__restrict__ rowsum,
+                                                                              int32_t *__restrict__ arg, int rows) {
+    constexpr int RPB = W < 4 ? 4 / W : 1, cols = 512 * NVL * W; // rows per workgroup
+    __shared__ float red[3][16];
+    __shared__ int redi[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, part = wave % W, rw = wave / W;
+    const int row = blockIdx.x * RPB + rw;
+    const bool live = row < rows; // every wave reaches every barrier
+    const size_t base = (size_t)(live ? row : 0) * cols + (size_t)part * (512 * NVL);
+    const uint4 *xr = reinterpret_cast<const uint4 *>(x + base);
+    float v[NVL][8];
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+        const uint4 t = xr[lane + 64 * j];
+        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            v[j][2 * k] = widen<DT>((uint16_t)w[k]);
+            v[j][2 * k + 1] = widen<DT>((uint16_t)(w[k] >> 16));
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) m = fmaxf(v[j][k], m);
+    }
+    m = wave_allreduce_f32(m, OpMaxF());
+    if (lane == 0) red[0][wave] = m;
+    __syncthreads();
+    m = red[0][rw * W];
+#pragma unroll
+    for (int k = 1; k < W; k++) m = fmaxf(m, red[0][rw * W + k]);
+
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            v[j][k] = DT == DT_BF16 ? __builtin_amdgcn_exp2f((v[j][k] - m) * 1.44269502162933349609375f) : exp_neg(v[j][k] - m);
+        s += ((v[j][0] + v[j][1]) + (v[j][2] + v[j][3])) + ((v[j][4] + v[j][5]) + (v[j][6] + v[j][7]));
+    }
+    s = wave_allreduce_f32(s, OpAdd());
+    if (lane == 0) red[1][wave] = s;
+    __syncthreads();
+    s = red[1][rw * W];
+#pragma unroll
+    for (int k = 1; k < W; k++) s += red[1][rw * W + k]; // the parts in column order, in every wave of the row
+    const float inv = 1.0f / s;
+    const float ymax = widen<DT>(narrow<DT>(inv)); // the stored y of the row maximum (its exponential is exactly 1)
+
+    float ys = 0.0f;
+    int best = 0;
+    uint4 *yr = reinterpret_cast<uint4 *>(y + base);
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+        const int c0 = part * (512 * NVL) + (lane + 64 * j) * 8;
+        uint32_t w[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint16_t lo = narrow<DT>(v[j][2 * k] * inv), hi = narrow<DT>(v[j][2 * k + 1] * inv);
+            const float flo = widen<DT>(lo), fhi = widen<DT>(hi);
+            ys += flo + fhi;
+            best = flo == ymax ? max(best, c0 + 2 * k) : best; // largest column among ties
+            best = fhi == ymax ? max(best, c0 + 2 * k + 1) : best;
+            w[k] = (uint32_t)lo | ((uint32_t)hi << 16);
+        }
+        if (y && live) yr[lane + 64 * j] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    if (rowsum || arg) {
+        ys = wave_allreduce_f32(ys, OpAdd());
+        best = wave_allreduce_i32(best, OpMaxI());
+        if (lane == 0) {
+            red[2][wave] = ys;
+            redi[wave] = best;
+        }
+        __syncthreads();
+        if (part == 0 && lane == 0 && live) {
+            float t = red[2][rw * W];
+            int b = redi[rw * W];
+#pragma unroll
+            for (int k = 1; k < W; k++) {
+                t += red[2][rw * W + k];
+                b = max(b, redi[rw * W + k]);
+            }
+            if (rowsum) rowsum[row] = narrow<DT>(t);
+            if (arg) arg[row] = b;
+        }
+    }
+}
+
 template <int DT> static hipError_t softmax_rows16(const SoftmaxRows &p, hipStream_t st) {
     const uint16_t *x = (const uint16_t *)p.x;
     uint16_t *y = (uint16_t *)p.y, *rs = (uint16_t *)p.rowsum;
     const bool vec_ok = (p.cols % 4 == 0) && p.cols <= 4096 && (reinterpret_cast<uintptr_t>(p.x) % 8 == 0) &&
                         (p.y == nullptr || reinterpret_cast<uintptr_t>(p.y) % 8 == 0) && p.rows < (1ll << 31) - 4;
+    const bool al16 = reinterpret_cast<uintptr_t>(p.x) % 16 == 0 && (p.y == nullptr || reinterpret_cast<uintptr_t>(p.y) % 16 == 0);
+    if (al16 && p.rows >= 1024 && p.rows < (1ll << 31) - 4) {
+        // (rows per workgroup: 4 / W for W < 4)
+        if (p.cols == 1024) {
+            hipLaunchKernelGGL((softmax_rows_split16_k<DT, 1, 2>), dim3((unsigned)((p.rows + 1) / 2)), dim3(256), 0, st, x, y, rs, p.arg, (int)p.rows);
+            return hipGetLastError();
+        }
+        if (p.cols == 2048) {
+            hipLaunchKernelGGL((softmax_rows_split16_k<DT, 1, 4>), dim3((unsigned)p.rows), dim3(256), 0, st, x, y, rs, p.arg, (int)p.rows);
+            return hipGetLastError();
+        }
+        if (p.cols == 4096) {
+            // (holding a compute unit at fewer workgroups with an unused LDS request, which helps the f32 kernel, does not
+            // help here: 24.6 us without, 24.6 .. 31.2 us with 20,000 .. 52,000 bytes)
+            hipLaunchKernelGGL((softmax_rows_split16_k<DT, 2, 4>), dim3((unsigned)p.rows), dim3(256), 0, st, x, y, rs, p.arg, (int)p.rows);
+            return hipGetLastError();
+        }
+        if (p.cols == 8192) {
+            hipLaunchKernelGGL((softmax_rows_split16_k<DT, 4, 4>), dim3((unsigned)p.rows), dim3(256), 0, st, x, y, rs, p.arg, (int)p.rows);
+            return hipGetLastError();
+        }
+    }
     if (vec_ok) {
         dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
         const int64_t nvec = p.cols / 4;
