@@ -106,6 +106,11 @@ struct Program {
     // whatever stream that ran, so two launches with unrelated wait lists never overlap on the scratch memory.
     hipEvent_t ws_event = nullptr;
     int ws_last = 0;           // where the scratch was last used: 0 nowhere yet, 1 a launch (ws_event), 2 a plan (the context's plan_done)
+    // A launch only notes its stream: the event is recorded when somebody else (another stream, a plan, the host) has to
+    // wait for the scratch, at that stream's end as it is then. Back-to-back launches on one stream, the usual case, pay
+    // no record (an event record after every two-kernel program left ~5.5 us between it and the next kernel).
+    int ws_stream = 0;
+    bool ws_recorded = false;
     int plan_refs = 0;         // live plans whose graphs hold this program's kernels, workspace and code
     // Direct convolution: which weights the re-laid copy in the workspace was made from (buffer, its device address and
     // the position of its last writer). A launch outside a plan that finds them unchanged skips the re-layout kernel.
@@ -1580,6 +1585,22 @@ ZHIP_EXPORT int32_t zhip_release_program(zhip_ctx *c, zhip_prog prog) {
     return ZHIP_OK;
 }
 
+// The event somebody else waits on for a program's scratch (ws_last != 0): the context's plan_done, or the program's own
+// event, recorded now on the stream of its last launch if that has not been done since.
+static hipError_t ws_wait_event(zhip_ctx *c, Program &p, hipEvent_t *out) {
+    if (p.ws_last == 2) {
+        *out = c->plan_done;
+        return hipSuccess;
+    }
+    if (!p.ws_recorded) {
+        hipError_t e = hipEventRecord(p.ws_event, c->launch_streams[p.ws_stream]);
+        if (e != hipSuccess) return e;
+        p.ws_recorded = true;
+    }
+    *out = p.ws_event;
+    return hipSuccess;
+}
+
 ZHIP_EXPORT int32_t zhip_launch(zhip_ctx *c, zhip_prog prog, const zhip_buf *args, size_t n_args, const zhip_event *evs,
                                 size_t n_evs, zhip_event *ev) {
     std::lock_guard<std::mutex> lk(c->mu);
@@ -1600,16 +1621,20 @@ ZHIP_EXPORT int32_t zhip_launch(zhip_ctx *c, zhip_prog prog, const zhip_buf *arg
     if (rc == ZHIP_OK) rc = order_args(c, si, *p, args, n_args, ZHIP_KERNEL_LAUNCH);
     if (rc != ZHIP_OK) return rc;
     if (c->debug & 32) fprintf(stderr, "[zyx-hip] launch program %u (kind %d) on stream %d\n", prog, p->desc.kind, si);
-    if (p->ws_event && p->ws_last)
-        HIPCHK(c, hipStreamWaitEvent(c->launch_streams[si], p->ws_last == 2 ? c->plan_done : p->ws_event, 0), ZHIP_KERNEL_LAUNCH);
+    if (p->ws_event && p->ws_last && !(p->ws_last == 1 && p->ws_stream == si)) { // the same stream is ordered by itself
+        hipEvent_t w;
+        HIPCHK(c, ws_wait_event(c, *p, &w), ZHIP_KERNEL_LAUNCH);
+        HIPCHK(c, hipStreamWaitEvent(c->launch_streams[si], w, 0), ZHIP_KERNEL_LAUNCH);
+    }
     hipError_t e = program_enqueue(*p, ptr, c->launch_streams[si], conv_weights_current(c, *p, args, n_args));
     if (e != hipSuccess) {
         p->conv_w_valid = false;
         return c->fail(ZHIP_KERNEL_LAUNCH, "launch of program %u failed: %s", prog, hipGetErrorString(e));
     }
     if (p->ws_event) {
-        HIPCHK(c, hipEventRecord(p->ws_event, c->launch_streams[si]), ZHIP_KERNEL_LAUNCH);
         p->ws_last = 1;
+        p->ws_stream = si;
+        p->ws_recorded = false;
     }
     rc = event_record(c, si, ZHIP_KERNEL_LAUNCH, ev);
     stamp_args(c, si, c->stream_seq[si], *p, args, n_args);
@@ -1674,7 +1699,11 @@ ZHIP_EXPORT int32_t zhip_time_kernel(zhip_ctx *c, zhip_prog prog, const zhip_buf
     if (rc != ZHIP_OK) return rc;
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
     hipStream_t st = c->launch_streams[0];
-    if (p->ws_event && p->ws_last) HIPCHK(c, hipEventSynchronize(p->ws_last == 2 ? c->plan_done : p->ws_event), ZHIP_KERNEL_SYNC);
+    if (p->ws_event && p->ws_last) {
+        hipEvent_t w;
+        HIPCHK(c, ws_wait_event(c, *p, &w), ZHIP_KERNEL_SYNC);
+        HIPCHK(c, hipEventSynchronize(w), ZHIP_KERNEL_SYNC);
+    }
     rc = order_args(c, 0, *p, args, n_args, ZHIP_KERNEL_LAUNCH);
     if (rc != ZHIP_OK) return rc;
     HIPCHK(c, hipStreamSynchronize(st), ZHIP_KERNEL_SYNC);
@@ -1703,7 +1732,11 @@ ZHIP_EXPORT int32_t zhip_profile_kernel(zhip_ctx *c, zhip_prog prog, const zhip_
     }
     HIPCHK(c, hipSetDevice(c->device), ZHIP_KERNEL_LAUNCH);
     hipStream_t st = c->launch_streams[0];
-    if (p->ws_event && p->ws_last) HIPCHK(c, hipEventSynchronize(p->ws_last == 2 ? c->plan_done : p->ws_event), ZHIP_KERNEL_SYNC);
+    if (p->ws_event && p->ws_last) {
+        hipEvent_t w;
+        HIPCHK(c, ws_wait_event(c, *p, &w), ZHIP_KERNEL_SYNC);
+        HIPCHK(c, hipEventSynchronize(w), ZHIP_KERNEL_SYNC);
+    }
     for (size_t s = 0; s < arg_sets; s++) {
         int32_t rc = order_args(c, 0, *p, args + s * n_args, n_args, ZHIP_KERNEL_LAUNCH);
         if (rc != ZHIP_OK) return rc;
@@ -1804,7 +1837,11 @@ ZHIP_EXPORT int32_t zhip_plan_launch(zhip_ctx *c, zhip_plan plan, const zhip_eve
         Program &pr = c->programs.items[q];
         if (!pr.ws_event) continue;
         any_ws = true;
-        if (pr.ws_last == 1) HIPCHK(c, hipStreamWaitEvent(c->plan_stream, pr.ws_event, 0), ZHIP_KERNEL_LAUNCH);
+        if (pr.ws_last == 1) {
+            hipEvent_t w;
+            HIPCHK(c, ws_wait_event(c, pr, &w), ZHIP_KERNEL_LAUNCH);
+            HIPCHK(c, hipStreamWaitEvent(c->plan_stream, w, 0), ZHIP_KERNEL_LAUNCH);
+        }
     }
     for (const auto &u : pl.uses)
         if (Buffer *b = buffer_lookup(c, u.first)) {
