@@ -13,7 +13,8 @@ from zyx_amd.kernels import argmax_desc, reduce
 pytestmark = pytest.mark.gpu
 
 SHAPES = [(1, 1), (3, 5), (8, 4096), (1, 131072), (1, 1 << 22), (4096, 512), (100, 1000), (513, 257), (70000, 12),
-          (2, 100003), (64, 128), (64, 10), (8192, 4096), (2048, 2050), (2100, 2500), (2048, 16384)]
+          (2, 100003), (64, 128), (64, 10), (8192, 4096), (2048, 2050), (2100, 2500), (2048, 16384),
+          (2047, 4096), (2048, 3072), (2049, 6140), (2048, 6144)]  # either side of the rows-per-workgroup and waves-per-row switches
 
 
 @pytest.mark.parametrize("shape", SHAPES)
