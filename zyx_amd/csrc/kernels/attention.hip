@@ -165,9 +165,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
         if (kt + NSTAGE - 1 < NT) stage_tile(kt + NSTAGE - 1, fill);
 
         if (!CAUSAL || kt * KB <= q0w + WQ - 1) {
+        // causal: the second 32-key block of the tile on the diagonal lies wholly after this wave's queries
+        const bool second_live = !CAUSAL || kt * KB + 32 <= q0w + WQ - 1; // uniform over the wave
         f32x16 s[QW][2];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
+            if (kb == 1 && !second_live) break;
 #pragma unroll
             for (int b = 0; b < QW; b++)
 #pragma unroll
@@ -185,14 +188,17 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_k(const uint16_t *__rest
             for (int b = 0; b < QW; b++)
                 if (kt * KB + KB - 1 > q0w + 32 * b) { // register r of block kb is key kb*32 + 8*(r/4) + 4*hh + r%4 of the tile
 #pragma unroll
-                    for (int kb = 0; kb < 2; kb++)
+                    for (int kb = 0; kb < 2; kb++) {
+                        if (kb == 1 && !second_live) break;
 #pragma unroll
                         for (int r = 0; r < 16; r++)
                             if (kt * KB + kb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3) > tq0 + 32 * b) s[b][kb][r] = -INFINITY;
+                    }
                 }
         }
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) { // exponentiate one 32-key block, feed it to the matrix pipe, then the next
+            if (kb == 1 && !second_live) break;
             // The exponentials are taken against the reference point m the query already has, and checked afterwards:
             // f32 sums and bf16 products carry 2^60 at the same relative precision as 1, so m only has to move when a
             // block's sum leaves that range (or is not a number: the first block of a query, whose m is -inf). Only then
