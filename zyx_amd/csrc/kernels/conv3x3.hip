@@ -594,15 +594,18 @@ bool half_ok(const Conv2d &p) {
 } // namespace
 
 bool conv3x3_direct_ok(const Conv2d &p) { // shape only: the same answer at registration and at every launch
-    const int R = tile_rows(p);
-    if (p.pool && R % 2) return false; // pooling windows must not straddle two tiles (either tile: half the rows otherwise)
     const bool types = (p.dtype == DT_BF16 && (p.out_dtype == DT_BF16 || p.out_dtype == DT_F32)) || (p.dtype == DT_F32 && p.out_dtype == DT_F32);
-    return types && p.KH == 3 && p.KW == 3 && p.sy == 1 && p.sx == 1 && p.dy == 1 && p.dx == 1 && p.py == 1 && p.px == 1 && p.C >= 16 &&
-           p.C % 16 == 0 && p.Cout % TILE_CO == 0 && p.W % 8 == 0 && R >= 1 && p.H % R == 0 && lds_bytes(p) <= 160 * 1024 && p.N > 0 &&
-           (int64_t)p.N * (p.H / R) < (1ll << 31) && p.Cout / TILE_CO <= 65535 && (int64_t)p.N * p.C * p.H * p.W < (1ll << 31) &&
-           (int64_t)p.N * p.Cout * p.H * p.W < (1ll << 40) && (int64_t)p.C * p.Cout < (1ll << 26) &&
-           p.H < (1 << 22) && // row numbers go through 24-bit multiplies
-           (int64_t)p.C * p.H * p.W * elem_bytes(p) < (1ll << 32); // 32-bit byte offsets within an image
+    const bool common = types && p.KH == 3 && p.KW == 3 && p.sy == 1 && p.sx == 1 && p.dy == 1 && p.dx == 1 && p.py == 1 && p.px == 1 &&
+                        p.C >= 16 && p.C % 16 == 0 && p.Cout % TILE_CO == 0 && p.W % 8 == 0 && p.N > 0 && p.H > 0 && p.Cout / TILE_CO <= 65535 &&
+                        (int64_t)p.N * p.C * p.H * p.W < (1ll << 31) && (int64_t)p.N * p.Cout * p.H * p.W < (1ll << 40) &&
+                        (int64_t)p.C * p.Cout < (1ll << 26) && p.H < (1 << 22) && // row numbers go through 24-bit multiplies
+                        (int64_t)p.C * p.H * p.W * elem_bytes(p) < (1ll << 32); // 32-bit byte offsets within an image
+    if (!common) return false;
+    // the 448-pixel tile, or the 224-pixel one (bf16, C % 32 = 0): whole rows, an even number of them under a fused pool
+    // (pooling windows must not straddle two tiles), the tile within LDS
+    const int R = tile_rows(p);
+    const bool full = R >= 1 && p.H % R == 0 && !(p.pool && R % 2) && lds_bytes(p) <= 160 * 1024 && (int64_t)p.N * (p.H / R) < (1ll << 31);
+    return full || half_ok(p);
 }
 
 uint64_t conv3x3_scratch_bytes(const Conv2d &p) { return (uint64_t)9 * p.C * p.Cout * elem_bytes(p); }
