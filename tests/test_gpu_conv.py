@@ -189,7 +189,8 @@ def test_max_pool_2x2_fast_path(hip, oracle, shape):
 
 @pytest.mark.parametrize("shape", [(2, 16, 16, 56, 128), (1, 64, 56, 56, 128), (3, 32, 28, 16, 256), (2, 48, 8, 112, 128), (1, 16, 56, 8, 128),
                                    (2, 64, 16, 28, 128), (1, 96, 8, 56, 128), (1, 32, 2, 224, 128), (1, 128, 28, 16, 128),
-                                   (2, 64, 28, 56, 128), (1, 32, 3, 224, 128)])  # heights only the 224-pixel tile divides
+                                   (2, 64, 28, 56, 128), (1, 32, 3, 224, 128),  # heights only the 224-pixel tile divides
+                                   (1, 128, 8, 56, 128)])  # 128 channels at this width fit the 448-pixel tile's LDS only
 @pytest.mark.parametrize("bias,relu", [(True, True), (False, False)])
 def test_conv3x3_direct_bf16(hip, oracle, shape, bias, relu):
     """3 x 3 / stride 1 / padding 1 bf16 shapes whose rows tile into 448-pixel blocks take the direct kernel (input
