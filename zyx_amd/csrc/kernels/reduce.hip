@@ -40,7 +40,7 @@ template <> struct Elem<0> {
     typedef float S; typedef float A;
     static __device__ __forceinline__ float ld(const float *p, int64_t i) { return p[i]; }
     static __device__ __forceinline__ void ld4(const float *p, int64_t i, float (&v)[4]) {
-        f32x4 t = *(const f32x4 *)(p + i);
+        f32x4 t = __builtin_nontemporal_load((const f32x4 *)(p + i)); // read once
         v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
     }
     static __device__ __forceinline__ void st(float *p, int64_t i, float v) { p[i] = v; }
@@ -49,12 +49,16 @@ template <> struct Elem<1> {
     typedef uint16_t S; typedef float A;
     static __device__ __forceinline__ float ld(const uint16_t *p, int64_t i) { return bf16_to_f32(p[i]); }
     static __device__ __forceinline__ void ld4(const uint16_t *p, int64_t i, float (&v)[4]) {
-        uint2 t = *(const uint2 *)(p + i);
+        typedef uint32_t u32x2nt __attribute__((ext_vector_type(2)));
+        const u32x2nt tt = __builtin_nontemporal_load((const u32x2nt *)(p + i)); // read once
+        const uint2 t = make_uint2(tt[0], tt[1]);
         v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
         v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
     }
     static __device__ __forceinline__ void ld8(const uint16_t *p, int64_t i, float (&v)[8]) {
-        uint4 t = *(const uint4 *)(p + i);
+        typedef uint32_t u32x4nt __attribute__((ext_vector_type(4)));
+        const u32x4nt tt = __builtin_nontemporal_load((const u32x4nt *)(p + i)); // read once
+        const uint4 t = make_uint4(tt[0], tt[1], tt[2], tt[3]);
         const unsigned w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
         for (int k = 0; k < 4; k++) {
@@ -68,12 +72,16 @@ template <> struct Elem<2> {
     typedef uint16_t S; typedef float A;
     static __device__ __forceinline__ float ld(const uint16_t *p, int64_t i) { return f16_to_f32(p[i]); }
     static __device__ __forceinline__ void ld4(const uint16_t *p, int64_t i, float (&v)[4]) {
-        uint2 t = *(const uint2 *)(p + i);
+        typedef uint32_t u32x2nt __attribute__((ext_vector_type(2)));
+        const u32x2nt tt = __builtin_nontemporal_load((const u32x2nt *)(p + i)); // read once
+        const uint2 t = make_uint2(tt[0], tt[1]);
         v[0] = f16_to_f32((uint16_t)t.x); v[1] = f16_to_f32((uint16_t)(t.x >> 16));
         v[2] = f16_to_f32((uint16_t)t.y); v[3] = f16_to_f32((uint16_t)(t.y >> 16));
     }
     static __device__ __forceinline__ void ld8(const uint16_t *p, int64_t i, float (&v)[8]) {
-        uint4 t = *(const uint4 *)(p + i);
+        typedef uint32_t u32x4nt __attribute__((ext_vector_type(4)));
+        const u32x4nt tt = __builtin_nontemporal_load((const u32x4nt *)(p + i)); // read once
+        const uint4 t = make_uint4(tt[0], tt[1], tt[2], tt[3]);
         const unsigned w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
         for (int k = 0; k < 4; k++) {
@@ -87,7 +95,7 @@ template <> struct Elem<3> {
     typedef int32_t S; typedef int A;
     static __device__ __forceinline__ int ld(const int32_t *p, int64_t i) { return p[i]; }
     static __device__ __forceinline__ void ld4(const int32_t *p, int64_t i, int (&v)[4]) {
-        i32x4 t = *(const i32x4 *)(p + i);
+        i32x4 t = __builtin_nontemporal_load((const i32x4 *)(p + i)); // read once
         v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
     }
     static __device__ __forceinline__ void st(int32_t *p, int64_t i, int v) { p[i] = v; }
