@@ -336,8 +336,9 @@ __global__ __launch_bounds__(W < 4 ? 256 : 64 * W) void softmax_rows_split16_k(c
     float m = -FLT_MAX;
 #pragma unroll
     for (int j = 0; j < NVL; j++) {
-        const uint4 t = xr[lane + 64 * j];
-        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+        typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
+        const u32x4s t = __builtin_nontemporal_load((const u32x4s *)(xr + lane + 64 * j)); // read once
+        const uint32_t w[4] = {t[0], t[1], t[2], t[3]};
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             v[j][2 * k] = widen<DT>((uint16_t)w[k]);
@@ -386,7 +387,8 @@ __global__ __launch_bounds__(W < 4 ? 256 : 64 * W) void softmax_rows_split16_k(c
             best = fhi == ymax ? max(best, c0 + 2 * k + 1) : best;
             w[k] = (uint32_t)lo | ((uint32_t)hi << 16);
         }
-        if (y && live) yr[lane + 64 * j] = make_uint4(w[0], w[1], w[2], w[3]);
+        typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
+        if (y && live) __builtin_nontemporal_store(u32x4s{w[0], w[1], w[2], w[3]}, (u32x4s *)(yr + lane + 64 * j));
     }
     if (rowsum || arg) {
         ys = wave_allreduce_f32(ys, OpAdd());
