@@ -162,7 +162,7 @@ __device__ __forceinline__ void copy_out(const ZK_LDS uint8_t *smem, void *__res
 #pragma unroll
                 for (int e = 0; e < 4; e++) v[e] = __float_as_uint(m[e % VPC]);
             }
-            *(u32x4 *)(ptile + (int64_t)co * pplane * ES + piece * 16) = v;
+            __builtin_nontemporal_store(v, (u32x4 *)(ptile + (int64_t)co * pplane * ES + piece * 16)); // written once
         }
     } else {
         // the tile's pixels are consecutive in the image plane
@@ -172,7 +172,7 @@ __device__ __forceinline__ void copy_out(const ZK_LDS uint8_t *smem, void *__res
             const int row = idx / CPR, col = idx - row * CPR;
             const int co = OUT_BF16 ? row : (row >> 5) * 64 + pass * 32 + (row & 31);
             const u32x4 v = *(const ZK_LDS u32x4 *)(smem + row * RS + col * 16);
-            *(u32x4 *)(ytile + (int64_t)co * plane * ES + col * 16) = v;
+            __builtin_nontemporal_store(v, (u32x4 *)(ytile + (int64_t)co * plane * ES + col * 16)); // written once
         }
     }
 }
