@@ -22,8 +22,6 @@ namespace zk {
 
 namespace {
 
-typedef uint32_t u32x2r __attribute__((ext_vector_type(2)));
-typedef uint32_t u32x4r __attribute__((ext_vector_type(4)));
 template <int DT> struct RowIO; // DT: 0 f32, 1 bf16 storage
 template <> struct RowIO<0> {
     typedef float S;
@@ -31,14 +29,6 @@ template <> struct RowIO<0> {
     static __device__ __forceinline__ void ld4(const float *p, int64_t i, float (&v)[4]) {
         f32x4 t = *(const f32x4 *)(p + i);
         v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
-    }
-    // rows (read once, written once) as against the affine parameters (read by every row): non-temporal
-    static __device__ __forceinline__ void ld4r(const float *p, int64_t i, float (&v)[4]) {
-        f32x4 t = __builtin_nontemporal_load((const f32x4 *)(p + i));
-        v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
-    }
-    static __device__ __forceinline__ void st4r(float *p, int64_t i, const float (&v)[4]) {
-        __builtin_nontemporal_store(f32x4{v[0], v[1], v[2], v[3]}, (f32x4 *)(p + i));
     }
     static __device__ __forceinline__ void st(float *p, int64_t i, float v) { p[i] = v; }
     static __device__ __forceinline__ void st4(float *p, int64_t i, const float (&v)[4]) {
@@ -57,28 +47,6 @@ template <> struct RowIO<1> {
     static __device__ __forceinline__ void st4(uint16_t *p, int64_t i, const float (&v)[4]) {
         *(uint2 *)(p + i) = make_uint2((__float_as_uint(v[0]) >> 16) | (__float_as_uint(v[1]) & 0xffff0000u),
                                        (__float_as_uint(v[2]) >> 16) | (__float_as_uint(v[3]) & 0xffff0000u));
-    }
-    static __device__ __forceinline__ void ld4r(const uint16_t *p, int64_t i, float (&v)[4]) {
-        const u32x2r t = __builtin_nontemporal_load((const u32x2r *)(p + i));
-        v[0] = __uint_as_float(t[0] << 16); v[1] = __uint_as_float(t[0] & 0xffff0000u);
-        v[2] = __uint_as_float(t[1] << 16); v[3] = __uint_as_float(t[1] & 0xffff0000u);
-    }
-    static __device__ __forceinline__ void st4r(uint16_t *p, int64_t i, const float (&v)[4]) {
-        __builtin_nontemporal_store(u32x2r{(__float_as_uint(v[0]) >> 16) | (__float_as_uint(v[1]) & 0xffff0000u),
-                                           (__float_as_uint(v[2]) >> 16) | (__float_as_uint(v[3]) & 0xffff0000u)}, (u32x2r *)(p + i));
-    }
-    static __device__ __forceinline__ void ld8r(const uint16_t *p, int64_t i, float (&a)[4], float (&b)[4]) {
-        const u32x4r t = __builtin_nontemporal_load((const u32x4r *)(p + i));
-        a[0] = __uint_as_float(t[0] << 16); a[1] = __uint_as_float(t[0] & 0xffff0000u);
-        a[2] = __uint_as_float(t[1] << 16); a[3] = __uint_as_float(t[1] & 0xffff0000u);
-        b[0] = __uint_as_float(t[2] << 16); b[1] = __uint_as_float(t[2] & 0xffff0000u);
-        b[2] = __uint_as_float(t[3] << 16); b[3] = __uint_as_float(t[3] & 0xffff0000u);
-    }
-    static __device__ __forceinline__ void st8r(uint16_t *p, int64_t i, const float (&a)[4], const float (&b)[4]) {
-        __builtin_nontemporal_store(u32x4r{(__float_as_uint(a[0]) >> 16) | (__float_as_uint(a[1]) & 0xffff0000u),
-                                           (__float_as_uint(a[2]) >> 16) | (__float_as_uint(a[3]) & 0xffff0000u),
-                                           (__float_as_uint(b[0]) >> 16) | (__float_as_uint(b[1]) & 0xffff0000u),
-                                           (__float_as_uint(b[2]) >> 16) | (__float_as_uint(b[3]) & 0xffff0000u)}, (u32x4r *)(p + i));
     }
     // 8 consecutive elements, one 16-byte access
     static __device__ __forceinline__ void ld8(const uint16_t *p, int64_t i, float (&a)[4], float (&b)[4]) {
@@ -108,39 +76,37 @@ template <int DT, int NV> struct RegRow {
     static __device__ __forceinline__ void load(const S *p, int lane, float (&v)[NV][4]) {
         if constexpr (WIDE) {
 #pragma unroll
-            for (int q = 0; q < NV / 2; q++) IO::ld8r(p, (lane + 64 * q) * 8, v[2 * q], v[2 * q + 1]);
+            for (int q = 0; q < NV / 2; q++) IO::ld8(p, (lane + 64 * q) * 8, v[2 * q], v[2 * q + 1]);
         } else {
 #pragma unroll
-            for (int j = 0; j < NV; j++) IO::ld4r(p, (lane + 64 * j) * 4, v[j]);
+            for (int j = 0; j < NV; j++) IO::ld4(p, (lane + 64 * j) * 4, v[j]);
         }
     }
     // vectors j0 (and j0 + 1 when WIDE; j0 even then)
     static __device__ __forceinline__ void load_at(const S *p, int lane, int j0, float (&a)[4], float (&b)[4]) {
-        if constexpr (WIDE) IO::ld8r(p, (lane + 64 * (j0 >> 1)) * 8, a, b);
-        else IO::ld4r(p, (lane + 64 * j0) * 4, a);
+        if constexpr (WIDE) IO::ld8(p, (lane + 64 * (j0 >> 1)) * 8, a, b);
+        else IO::ld4(p, (lane + 64 * j0) * 4, a);
     }
     static __device__ __forceinline__ void store_at(S *p, int lane, int j0, const float (&a)[4], const float (&b)[4]) {
-        if constexpr (WIDE) IO::st8r(p, (lane + 64 * (j0 >> 1)) * 8, a, b);
-        else IO::st4r(p, (lane + 64 * j0) * 4, a);
+        if constexpr (WIDE) IO::st8(p, (lane + 64 * (j0 >> 1)) * 8, a, b);
+        else IO::st4(p, (lane + 64 * j0) * 4, a);
     }
     static constexpr int STEP = WIDE ? 2 : 1; // vectors per access
     // The lane's part of a row as it lies in memory (32-bit words), for a row fetched ahead of its use: 16-bit rows
     // stay packed until unpack(), half the registers of their f32 form.
     static constexpr int NW = NV * (int)sizeof(S);
-    template <bool ROW> static __device__ __forceinline__ void load_raw(const S *p, int lane, uint32_t (&r)[NW]) { // ROW: read once
+    static __device__ __forceinline__ void load_raw(const S *p, int lane, uint32_t (&r)[NW]) {
         if constexpr (DT == 0 || WIDE) {
 #pragma unroll
             for (int q = 0; q < NW / 4; q++) {
-                const u32x4r *src = (const u32x4r *)(p + (lane + 64 * q) * (16 / (int)sizeof(S)));
-                const u32x4r t = ROW ? __builtin_nontemporal_load(src) : *src;
-                r[4 * q] = t[0]; r[4 * q + 1] = t[1]; r[4 * q + 2] = t[2]; r[4 * q + 3] = t[3];
+                const uint4 t = *(const uint4 *)(p + (lane + 64 * q) * (16 / (int)sizeof(S)));
+                r[4 * q] = t.x; r[4 * q + 1] = t.y; r[4 * q + 2] = t.z; r[4 * q + 3] = t.w;
             }
         } else {
 #pragma unroll
             for (int j = 0; j < NV; j++) {
-                const u32x2r *src = (const u32x2r *)(p + (lane + 64 * j) * 4);
-                const u32x2r t = ROW ? __builtin_nontemporal_load(src) : *src;
-                r[2 * j] = t[0]; r[2 * j + 1] = t[1];
+                const uint2 t = *(const uint2 *)(p + (lane + 64 * j) * 4);
+                r[2 * j] = t.x; r[2 * j + 1] = t.y;
             }
         }
     }
@@ -237,8 +203,8 @@ __global__ __launch_bounds__(256) void norm_rows_reg_k(const typename RowIO<DT>:
     constexpr bool EARLY = DT == 1 && NV <= 4; // (f32 rows lose by it: 13.9 us against 12.6 us at 8192 x 1024)
     uint32_t wr[RR::NW], br[RR::NW];
     if constexpr (EARLY) {
-        if (w) RR::template load_raw<false>(w, lane, wr);
-        if (b) RR::template load_raw<false>(b, lane, br);
+        if (w) RR::load_raw(w, lane, wr);
+        if (b) RR::load_raw(b, lane, br);
     }
     float mean = 0.0f, scale;
     if (MODE == 0) {
@@ -324,9 +290,9 @@ __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename R
 #pragma unroll
     for (int i = 0; i < RR::NW; i++) na[i] = 0u;
     if (AHEAD && row < rows) {
-        RR::template load_raw<true>(x + row * cols, lane, nx);
-        RR::template load_raw<true>(dy + row * cols, lane, ng);
-        if (add) RR::template load_raw<true>(add + row * cols, lane, na);
+        RR::load_raw(x + row * cols, lane, nx);
+        RR::load_raw(dy + row * cols, lane, ng);
+        if (add) RR::load_raw(add + row * cols, lane, na);
     }
     for (; row < rows; row += stride) {
         const int64_t base = row * cols;
@@ -339,9 +305,9 @@ __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename R
             for (int i = 0; i < RR::NW; i++) ca[i] = na[i];
             if (row + stride < rows) {
                 const int64_t nb = (row + stride) * cols;
-                RR::template load_raw<true>(x + nb, lane, nx);
-                RR::template load_raw<true>(dy + nb, lane, ng);
-                if (add) RR::template load_raw<true>(add + nb, lane, na);
+                RR::load_raw(x + nb, lane, nx);
+                RR::load_raw(dy + nb, lane, ng);
+                if (add) RR::load_raw(add + nb, lane, na);
             }
         } else {
             RR::load(x + base, lane, xv);
