@@ -73,7 +73,10 @@ def test_config2_full_size(hip, oracle):
 
 @pytest.mark.parametrize("shape", [(1, 1), (3, 4), (5, 10), (64, 10), (7, 252), (33, 256), (9, 1000), (130, 1024),
                                    (17, 2048), (6, 4092), (5, 4096), (3, 4097), (4, 5000), (2, 16384), (1, 100003),
-                                   (2048, 320), (1025, 12)])
+                                   (2048, 320), (1025, 12),
+                                   # rows held in the registers of 4, 8 or 16 waves: whole and ragged last parts
+                                   (3, 8192), (5, 8188), (3, 4100), (2, 12292), (3, 32768), (2, 20484), (2, 32772),
+                                   (1030, 3072), (1025, 2052), (1024, 4092)])
 def test_shapes(hip, oracle, shape):
     x = oracle.Rng(shape[0] * 131 + shape[1]).randn(shape, 3.0)
     run_and_check(hip, oracle, x)

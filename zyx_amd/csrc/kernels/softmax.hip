@@ -166,6 +166,90 @@ __global__ __launch_bounds__(W < 4 ? 256 : 64 * W) void softmax_rows_split_k(con
     }
 }
 
+// Rows of 4096 .. 32768 columns (a multiple of 4): one workgroup per row, W waves holding 1024 * NVL columns each in
+// registers (a ragged last part reads the fold's neutral value), so that a long row is still read from memory once;
+// the three row reductions go through LDS as in the split kernel. The three-pass kernel below, which these rows took
+// before, runs 8192 .. 32768 columns at 0.20-0.31 of 8 TB/s.
+template <int NVL, int W>
+__global__ __launch_bounds__(64 * W) void softmax_rows_wide_k(const float *__restrict__ x, float *__restrict__ y,
+                                                             float *__restrict__ rowsum, int32_t *__restrict__ arg, int cols) {
+    __shared__ float red[3][16];
+    __shared__ int redi[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row = blockIdx.x;
+    const int nvec = cols >> 2, v0 = wave * (64 * NVL) + lane; // this lane's first float4 of the row
+    const f32x4 *xr = reinterpret_cast<const f32x4 *>(x + row * cols);
+    f32x4 v[NVL];
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+        const int i = v0 + 64 * j;
+        v[j] = i < nvec ? load_stream(xr + i) : f32x4{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+        m = fmaxf(fmaxf(fmaxf(v[j].x, v[j].y), fmaxf(v[j].z, v[j].w)), m);
+    }
+    m = wave_allreduce_f32(m, OpMaxF());
+    if (lane == 0) red[0][wave] = m;
+    __syncthreads();
+    m = red[0][0];
+#pragma unroll
+    for (int k = 1; k < W; k++) m = fmaxf(m, red[0][k]);
+
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+        const bool live = v0 + 64 * j < nvec;
+        v[j].x = live ? exp_neg(v[j].x - m) : 0.0f;
+        v[j].y = live ? exp_neg(v[j].y - m) : 0.0f;
+        v[j].z = live ? exp_neg(v[j].z - m) : 0.0f;
+        v[j].w = live ? exp_neg(v[j].w - m) : 0.0f;
+        s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+    }
+    s = wave_allreduce_f32(s, OpAdd());
+    if (lane == 0) red[1][wave] = s;
+    __syncthreads();
+    s = red[1][0];
+#pragma unroll
+    for (int k = 1; k < W; k++) s += red[1][k]; // the parts in column order, in every wave
+    const float inv = 1.0f / s;
+
+    float ys = 0.0f;
+    int best = 0;
+    f32x4 *yr = reinterpret_cast<f32x4 *>(y + row * cols);
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+        const int i = v0 + 64 * j;
+        if (i >= nvec) continue;
+        const f32x4 o = v[j] * inv;
+        ys += (o.x + o.y) + (o.z + o.w);
+        const int c = i * 4; // largest column whose y equals max(y) = inv
+        best = o.x == inv ? max(best, c) : best;
+        best = o.y == inv ? max(best, c + 1) : best;
+        best = o.z == inv ? max(best, c + 2) : best;
+        best = o.w == inv ? max(best, c + 3) : best;
+        if (y) store_stream(o, yr + i);
+    }
+    if (rowsum || arg) {
+        ys = wave_allreduce_f32(ys, OpAdd());
+        best = wave_allreduce_i32(best, OpMaxI());
+        if (lane == 0) {
+            red[2][wave] = ys;
+            redi[wave] = best;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float t = red[2][0];
+            int b = redi[0];
+#pragma unroll
+            for (int k = 1; k < W; k++) {
+                t += red[2][k];
+                b = max(b, redi[k]);
+            }
+            if (rowsum) rowsum[row] = t;
+            if (arg) arg[row] = b;
+        }
+    }
+}
+
 // Any cols / alignment: one 256-thread workgroup per row, three passes over the row
 // (rows of this size stay in L2 between passes), LDS only for the cross-wave folds.
 template <class Op> __device__ __forceinline__ float block_allreduce_f32(float v, Op op, float *lds) {
@@ -520,6 +604,11 @@ hipError_t softmax_rows(const SoftmaxRows &p, hipStream_t st) {
         if (p.rows >= 1024 && p.cols == 1024) return launch_split<1>(p, st);
         if (p.rows >= 1024 && p.cols == 2048) return launch_split<2>(p, st);
         if (p.rows >= 1024 && p.cols == 4096) return launch_split<4>(p, st);
+        if (p.rows >= 1024 && p.cols > 2048) { // other lengths up to 4096: four waves per row as well, the last part ragged
+            hipLaunchKernelGGL((softmax_rows_wide_k<4, 4>), dim3((unsigned)p.rows), dim3(256), 0, st, (const float *)p.x, (float *)p.y,
+                               (float *)p.rowsum, p.arg, (int)p.cols);
+            return hipGetLastError();
+        }
         if (nvec <= 64) return launch_wave<1>(p, st);
         if (nvec <= 128) return launch_wave<2>(p, st);
         if (nvec <= 256) return launch_wave<4>(p, st);
@@ -527,6 +616,17 @@ hipError_t softmax_rows(const SoftmaxRows &p, hipStream_t st) {
         return launch_wave<16>(p, st);
     }
     if (p.rows >= (1ll << 31) || p.cols >= (1ll << 31)) return hipErrorInvalidValue;
+    if (p.cols % 4 == 0 && p.cols > 4096 && p.cols <= 32768 && reinterpret_cast<uintptr_t>(p.x) % 16 == 0 &&
+        (p.y == nullptr || reinterpret_cast<uintptr_t>(p.y) % 16 == 0)) {
+        const float *x = (const float *)p.x;
+        float *y = (float *)p.y, *rs = (float *)p.rowsum;
+        const dim3 grid((unsigned)p.rows);
+        // 4 KiB of a row per wave up to 16384 columns, 8 KiB beyond
+        if (p.cols <= 8192) hipLaunchKernelGGL((softmax_rows_wide_k<4, 8>), grid, dim3(512), 0, st, x, y, rs, p.arg, (int)p.cols);
+        else if (p.cols <= 16384) hipLaunchKernelGGL((softmax_rows_wide_k<4, 16>), grid, dim3(1024), 0, st, x, y, rs, p.arg, (int)p.cols);
+        else hipLaunchKernelGGL((softmax_rows_wide_k<8, 16>), grid, dim3(1024), 0, st, x, y, rs, p.arg, (int)p.cols);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(softmax_rows_generic_k, dim3((unsigned)p.rows), dim3(256), 0, st, (const float *)p.x, (float *)p.y, (float *)p.rowsum, p.arg,
                        (int)p.rows, p.cols);
     return hipGetLastError();
