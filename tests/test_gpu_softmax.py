@@ -178,7 +178,8 @@ def test_undersized_argument_is_rejected(hip):
 @pytest.mark.parametrize("dt", ["bf16", "f16"])
 @pytest.mark.parametrize("shape", [(1, 1), (5, 10), (64, 252), (33, 256), (9, 1000), (130, 1024), (6, 4092), (5, 4096), (3, 4097),
                                    (2, 16384), (2048, 320),
-                                   (1025, 1024), (1024, 2048), (2050, 4096), (1027, 8192)])  # rows split over the waves of a workgroup
+                                   (1025, 1024), (1024, 2048), (2050, 4096), (1027, 8192),  # rows split over the waves of a workgroup
+                                   (3, 8192), (5, 8184), (2, 12296), (3, 32768), (2, 50264), (2, 65536), (3, 4104)])  # rows in the registers of 8 or 16 waves
 def test_sixteen_bit_storage(hip, oracle, shape, dt):
     """bf16 / f16 rows: elements widen to f32 registers, y is truncated on store, the row sum and the argmax read the stored
     y (zyx/src/codegen/c.rs:456-497, 491-496). Against the oracle's restatement: the device's exp differs from expf in the

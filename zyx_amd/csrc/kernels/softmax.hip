@@ -496,6 +496,105 @@ __global__ __launch_bounds__(W < 4 ? 256 : 64 * W) void softmax_rows_split16_k(c
     }
 }
 
+// 16-bit rows of up to 65536 columns (a multiple of 8): one workgroup per row, W waves holding 512 * NVL columns each
+// in registers, the last part ragged; otherwise as softmax_rows_split16_k. (These rows took the three-pass kernel before.)
+template <int DT, int NVL, int W>
+__global__ __launch_bounds__(64 * W) void softmax_rows_wide16_k(const uint16_t *__restrict__ x, uint16_t *__restrict__ y,
+                                                               uint16_t *__restrict__ rowsum, int32_t *__restrict__ arg, int cols) {
+    typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
+    __shared__ float red[3][16];
+    __shared__ int redi[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row = blockIdx.x;
+    const int nvec = cols >> 3, v0 = wave * (64 * NVL) + lane; // this lane's first 8-element vector of the row
+    const u32x4s *xr = reinterpret_cast<const u32x4s *>(x + row * cols);
+    float v[NVL][8];
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+        if (v0 + 64 * j < nvec) {
+            const u32x4s t = __builtin_nontemporal_load(xr + v0 + 64 * j); // read once
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                v[j][2 * k] = widen<DT>((uint16_t)t[k]);
+                v[j][2 * k + 1] = widen<DT>((uint16_t)(t[k] >> 16));
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) v[j][k] = -FLT_MAX;
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) m = fmaxf(v[j][k], m);
+    }
+    m = wave_allreduce_f32(m, OpMaxF());
+    if (lane == 0) red[0][wave] = m;
+    __syncthreads();
+    m = red[0][0];
+#pragma unroll
+    for (int k = 1; k < W; k++) m = fmaxf(m, red[0][k]);
+
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+        const bool live = v0 + 64 * j < nvec;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float e = DT == DT_BF16 ? __builtin_amdgcn_exp2f((v[j][k] - m) * 1.44269502162933349609375f) : exp_neg(v[j][k] - m);
+            v[j][k] = live ? e : 0.0f;
+        }
+        s += ((v[j][0] + v[j][1]) + (v[j][2] + v[j][3])) + ((v[j][4] + v[j][5]) + (v[j][6] + v[j][7]));
+    }
+    s = wave_allreduce_f32(s, OpAdd());
+    if (lane == 0) red[1][wave] = s;
+    __syncthreads();
+    s = red[1][0];
+#pragma unroll
+    for (int k = 1; k < W; k++) s += red[1][k];
+    const float inv = 1.0f / s;
+    const float ymax = widen<DT>(narrow<DT>(inv)); // the stored y of the row maximum (its exponential is exactly 1)
+
+    float ys = 0.0f;
+    int best = 0;
+    u32x4s *yr = reinterpret_cast<u32x4s *>(y + row * cols);
+#pragma unroll
+    for (int j = 0; j < NVL; j++) {
+        const int i = v0 + 64 * j;
+        if (i >= nvec) continue;
+        const int c0 = i * 8;
+        u32x4s w;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint16_t lo = narrow<DT>(v[j][2 * k] * inv), hi = narrow<DT>(v[j][2 * k + 1] * inv);
+            const float flo = widen<DT>(lo), fhi = widen<DT>(hi);
+            ys += flo + fhi;
+            best = flo == ymax ? max(best, c0 + 2 * k) : best; // largest column among ties
+            best = fhi == ymax ? max(best, c0 + 2 * k + 1) : best;
+            w[k] = (uint32_t)lo | ((uint32_t)hi << 16);
+        }
+        if (y) __builtin_nontemporal_store(w, yr + i);
+    }
+    if (rowsum || arg) {
+        ys = wave_allreduce_f32(ys, OpAdd());
+        best = wave_allreduce_i32(best, OpMaxI());
+        if (lane == 0) {
+            red[2][wave] = ys;
+            redi[wave] = best;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float t = red[2][0];
+            int b = redi[0];
+#pragma unroll
+            for (int k = 1; k < W; k++) {
+                t += red[2][k];
+                b = max(b, redi[k]);
+            }
+            if (rowsum) rowsum[row] = narrow<DT>(t);
+            if (arg) arg[row] = b;
+        }
+    }
+}
+
 template <int DT> static hipError_t softmax_rows16(const SoftmaxRows &p, hipStream_t st) {
     const uint16_t *x = (const uint16_t *)p.x;
     uint16_t *y = (uint16_t *)p.y, *rs = (uint16_t *)p.rowsum;
@@ -536,6 +635,14 @@ template <int DT> static hipError_t softmax_rows16(const SoftmaxRows &p, hipStre
         return hipGetLastError();
     }
     if (p.rows >= (1ll << 31) || p.cols >= (1ll << 31)) return hipErrorInvalidValue;
+    if (al16 && p.cols % 8 == 0 && p.cols > 4096 && p.cols <= 65536) {
+        const dim3 grid((unsigned)p.rows);
+        if (p.cols <= 8192) hipLaunchKernelGGL((softmax_rows_wide16_k<DT, 2, 8>), grid, dim3(512), 0, st, x, y, rs, p.arg, (int)p.cols);
+        else if (p.cols <= 16384) hipLaunchKernelGGL((softmax_rows_wide16_k<DT, 2, 16>), grid, dim3(1024), 0, st, x, y, rs, p.arg, (int)p.cols);
+        else if (p.cols <= 32768) hipLaunchKernelGGL((softmax_rows_wide16_k<DT, 4, 16>), grid, dim3(1024), 0, st, x, y, rs, p.arg, (int)p.cols);
+        else hipLaunchKernelGGL((softmax_rows_wide16_k<DT, 8, 16>), grid, dim3(1024), 0, st, x, y, rs, p.arg, (int)p.cols);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(softmax_rows_generic16_k<DT>, dim3((unsigned)p.rows), dim3(256), 0, st, x, y, rs, p.arg, (int)p.rows, p.cols);
     return hipGetLastError();
 }
