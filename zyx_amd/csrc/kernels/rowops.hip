@@ -259,6 +259,101 @@ __global__ __launch_bounds__(256) void norm_rows_reg_k(const typename RowIO<DT>:
     }
 }
 
+// Rows of any multiple of 4 columns up to 16384: the row is held in the registers of W waves (256 * NV columns per
+// wave, the last part ragged; 4 / W rows per workgroup for W < 4), read from memory once; the two row sums of the W
+// parts meet in LDS in column order. (These widths - 768, 1280, 3072, 5120, 8192 ... - took norm_rows_k before, which
+// reads the row three times: 0.18-0.29 of 8 TB/s at 8192 rows.)
+template <int DT, int MODE, int NV, int W, int VE>
+__global__ __launch_bounds__(W < 4 ? 256 : 64 * W) void norm_rows_wide_k(const typename RowIO<DT>::S *__restrict__ x,
+                                                                      const typename RowIO<DT>::S *__restrict__ w,
+                                                                      const typename RowIO<DT>::S *__restrict__ b,
+                                                                      typename RowIO<DT>::S *__restrict__ y, int64_t rows, int cols,
+                                                                      float eps) {
+    // VE elements per vector: 4, or 8 for 16-bit rows of a multiple of 8 columns (16-byte accesses)
+    typedef RowIO<DT> IO;
+    constexpr int RPB = W < 4 ? 4 / W : 1;
+    __shared__ float red[2][16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, part = wave % W, rw = wave / W;
+    const int64_t row = (int64_t)blockIdx.x * RPB + rw;
+    const bool live_row = row < rows; // every wave reaches every barrier
+    const typename IO::S *xr = x + (live_row ? row : 0) * cols;
+    const int nvec = cols / VE, v0 = part * (64 * NV) + lane;
+    auto load = [&](const typename IO::S *p, int i, float (&t)[VE]) {
+        if constexpr (VE == 8) {
+            float a4[4], b4[4];
+            IO::ld8(p, i * 8, a4, b4);
+#pragma unroll
+            for (int k = 0; k < 4; k++) t[k] = a4[k], t[4 + k] = b4[k];
+        } else {
+            IO::ld4(p, i * 4, t);
+        }
+    };
+    float v[NV][VE];
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        if (v0 + 64 * j < nvec) load(xr, v0 + 64 * j, v[j]);
+        else
+#pragma unroll
+            for (int k = 0; k < VE; k++) v[j][k] = 0.0f;
+#pragma unroll
+        for (int k = 0; k < VE; k += 4) s += (v[j][k] + v[j][k + 1]) + (v[j][k + 2] + v[j][k + 3]);
+    }
+    auto row_total = [&](float t, int slot) { // sum over the row's W parts, in column order, in every wave of the row
+        t = wave_allreduce_f32(t, OpAdd());
+        if (W == 1) return t;
+        if (lane == 0) red[slot][wave] = t;
+        __syncthreads();
+        float r = red[slot][rw * W];
+#pragma unroll
+        for (int k = 1; k < W; k++) r += red[slot][rw * W + k];
+        return r;
+    };
+    float mean = 0.0f, scale;
+    if (MODE == 0) {
+        mean = row_total(s, 0) / (float)cols;
+        float q = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const bool live = v0 + 64 * j < nvec;
+#pragma unroll
+            for (int k = 0; k < VE; k++) q += live ? (v[j][k] - mean) * (v[j][k] - mean) : 0.0f;
+        }
+        scale = 1.0f / sqrtf(row_total(q, 1) / (float)(cols - 1) + eps);
+    } else {
+        float q = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+#pragma unroll
+            for (int k = 0; k < VE; k++) q += v[j][k] * v[j][k]; // dead lanes hold zeros
+        scale = sqrtf(1.0f / (row_total(q, 0) / (float)cols + eps));
+    }
+    if (!live_row) return; // past the last barrier
+    typename IO::S *yr = y + row * cols;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = v0 + 64 * j;
+        if (i >= nvec) continue;
+        float wv[VE], bv[VE], o[VE];
+#pragma unroll
+        for (int k = 0; k < VE; k++) wv[k] = 1.0f, bv[k] = 0.0f;
+        if (w) load(w, i, wv);
+        if (b) load(b, i, bv);
+#pragma unroll
+        for (int k = 0; k < VE; k++) {
+            o[k] = MODE == 0 ? (v[j][k] - mean) * scale : v[j][k] * scale;
+            if (w) o[k] *= wv[k];
+            if (b) o[k] += bv[k];
+        }
+        if constexpr (VE == 8) {
+            const float a4[4] = {o[0], o[1], o[2], o[3]}, b4[4] = {o[4], o[5], o[6], o[7]};
+            IO::st8(yr, i * 8, a4, b4);
+        } else {
+            IO::st4(yr, i * 4, o);
+        }
+    }
+}
+
 // dx for rows of 256*NV columns with x and dy held in registers (one read of each), and the parameter gradients in
 // the same pass: a workgroup of WAVES waves walks rows blockIdx*WAVES + wave, + gridDim*WAVES, ..., every lane keeps
 // running sums of dy*xh and dy for its 4*NV columns, the waves of a workgroup add theirs up through LDS in wave order
@@ -664,7 +759,33 @@ template <int DT, int MODE> hipError_t launch_norm(const NormRows &p, hipStream_
     else if (al16 && p.cols == 2048) ZK_FWD_REG(8);
     else if (al16 && p.cols == 4096) ZK_FWD_REG(16);
 #undef ZK_FWD_REG
-    else if (vec) hipLaunchKernelGGL((norm_rows_k<DT, MODE, true>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.b, (S *)p.y, p.rows, (int)p.cols, p.eps);
+    else if (al16 && p.cols <= 16384) {
+        // VE elements per 16-byte (or, 16-bit rows of an odd multiple of 4 columns, 8-byte) vector; W = waves per row
+        // (4 * 64 * VE columns each at most); NV = 3 or 4 vectors per lane
+        constexpr int VMAX = DT == 1 ? 8 : 4;
+        const bool wide_vec = DT == 1 && p.cols > 1024 /* below, 8-byte vectors fill the lanes better */ && p.cols % 8 == 0 && reinterpret_cast<uintptr_t>(p.x) % 16 == 0 && reinterpret_cast<uintptr_t>(p.y) % 16 == 0 &&
+                              (!p.w || reinterpret_cast<uintptr_t>(p.w) % 16 == 0) && (!p.b || reinterpret_cast<uintptr_t>(p.b) % 16 == 0);
+        const int ve = wide_vec ? 8 : 4, cap = 256 * ve; // columns of a wave at NV = 4
+        const int W = p.cols <= cap ? 1 : p.cols <= 2 * cap ? 2 : p.cols <= 4 * cap ? 4 : p.cols <= 8 * cap ? 8 : 16;
+        const bool three = p.cols <= 3 * 64 * ve * W;
+        const int rpb = W < 4 ? 4 / W : 1;
+        const dim3 wgrid((unsigned)((p.rows + rpb - 1) / rpb)), wblock(W < 4 ? 256 : 64 * W);
+#define ZK_WIDE(NVV, WV, VEV) hipLaunchKernelGGL((norm_rows_wide_k<DT, MODE, NVV, WV, VEV>), wgrid, wblock, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.b, (S *)p.y, p.rows, (int)p.cols, p.eps)
+#define ZK_WIDE2(WV)                                                                                                              \
+    do {                                                                                                                          \
+        if (wide_vec && three) ZK_WIDE(3, WV, VMAX);                                                                              \
+        else if (wide_vec) ZK_WIDE(4, WV, VMAX);                                                                                  \
+        else if (three) ZK_WIDE(3, WV, 4);                                                                                        \
+        else ZK_WIDE(4, WV, 4);                                                                                                   \
+    } while (0)
+        if (W == 1) ZK_WIDE2(1);
+        else if (W == 2) ZK_WIDE2(2);
+        else if (W == 4) ZK_WIDE2(4);
+        else if (W == 8) ZK_WIDE2(8);
+        else ZK_WIDE2(16);
+#undef ZK_WIDE2
+#undef ZK_WIDE
+    } else if (vec) hipLaunchKernelGGL((norm_rows_k<DT, MODE, true>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.b, (S *)p.y, p.rows, (int)p.cols, p.eps);
     else hipLaunchKernelGGL((norm_rows_k<DT, MODE, false>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.b, (S *)p.y, p.rows, (int)p.cols, p.eps);
     return hipGetLastError();
 }
