@@ -88,7 +88,10 @@ def test_cross_entropy(hip, oracle):
 
 # ---- gradients of the norms ---------------------------------------------------------------------------------
 @pytest.mark.parametrize("shape", [(5, 9), (64, 128), (130, 1024), (3, 1000), (2100, 64), (64, 256), (7, 512), (9, 2048),
-                                   (8192, 1024), (4099, 1024), (2051, 512)])  # several rows per wave: rows fetched ahead
+                                   (8192, 1024), (4099, 1024), (2051, 512),  # several rows per wave: rows fetched ahead
+                                   # widths that are not 256 * 2^n, with lanes past the end of the row
+                                   (4100, 768), (2049, 1280), (300, 1536), (37, 1800), (5, 2044), (7, 260), (600, 772), (3, 4),
+                                   (1030, 520), (9, 2052)])
 @pytest.mark.parametrize("rms", [False, True])
 def test_norm_backward_f32(hip, oracle, shape, rms):
     from zyx_amd.kernels import norm_rows_bwd
@@ -108,18 +111,20 @@ def test_norm_backward_f32(hip, oracle, shape, rms):
                 assert np.allclose(g, wv, rtol=1e-5, atol=2e-6 * rows)
 
 
-def test_norm_backward_bf16_config5_rows(hip, oracle):
-    """Rows of 1024 bf16 as in config 5 (8192 rows): f32 arithmetic, one truncating bf16 store."""
+@pytest.mark.parametrize("shape", [(8192, 1024), (4100, 768), (1000, 1288), (300, 2040)])
+def test_norm_backward_bf16_rows(hip, oracle, shape):
+    """Rows of 1024 bf16 as in config 5 (8192 rows), and widths with lanes past the end of the row: f32 arithmetic,
+    one truncating bf16 store."""
     from zyx_amd.kernels import norm_rows_bwd
     from zyx_amd import DType
     dev, pool = hip
     r = oracle.Rng(9)
-    shape = (8192, 1024)
     x, dy, add = [oracle.f32_to_bf16(r.randn(shape)) for _ in range(3)]
-    w = oracle.f32_to_bf16(1.0 + 0.1 * r.randn((1024,)))
+    w = oracle.f32_to_bf16(1.0 + 0.1 * r.randn((shape[1],)))
     got = norm_rows_bwd(dev, pool, x, dy, w, add, dtype=DType.BF16)
     want = oracle.norm_bwd(x, dy, w, add, dtype=oracle.BF16)
-    for g, wv, scale in zip(got, want, (1.0, 90.0, 90.0)):   # column sums of 8192 N(0,1) terms are ~90 in size
+    col = float(np.sqrt(shape[0]))   # column sums of `rows` N(0,1) terms are ~sqrt(rows) in size
+    for g, wv, scale in zip(got, want, (1.0, col, col)):
         gf, wf = oracle.bf16_to_f32(g).astype(np.float64), oracle.bf16_to_f32(wv).astype(np.float64)
         assert np.all(np.abs(gf - wf) <= 2.0 ** -7 * np.abs(wf) + 1e-4 * scale)
 

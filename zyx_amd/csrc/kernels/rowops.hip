@@ -487,6 +487,113 @@ __global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_reg_k(const typename R
     }
 }
 
+// The same pass for rows of any multiple of 4 columns up to 256*NV (768, 1280, 1536 ...): vector lane + 64*j of a
+// row belongs to the lane while it lies inside the row; lanes past the end hold zeros, which every sum but the
+// variance's takes as they are. part rows are cols long.
+template <int DT, int MODE, int NV, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void norm_bwd_dx_ragged_k(const typename RowIO<DT>::S *__restrict__ x,
+                                                                   const typename RowIO<DT>::S *__restrict__ w,
+                                                                   const typename RowIO<DT>::S *__restrict__ dy,
+                                                                   const typename RowIO<DT>::S *__restrict__ add,
+                                                                   typename RowIO<DT>::S *__restrict__ dx, float *__restrict__ part,
+                                                                   int64_t rows, int cols, float eps) {
+    typedef RowIO<DT> IO;
+    constexpr int CAP = 256 * NV;
+    __shared__ float fold[WAVES][2][CAP]; // 128 KiB at most
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nvec = cols >> 2;
+    float pw[NV][4], pb[NV][4];
+#pragma unroll
+    for (int j = 0; j < NV; j++)
+#pragma unroll
+        for (int k = 0; k < 4; k++) pw[j][k] = pb[j][k] = 0.0f;
+    const int64_t stride = (int64_t)gridDim.x * WAVES;
+    for (int64_t row = (int64_t)blockIdx.x * WAVES + wave; row < rows; row += stride) {
+        const int64_t base = row * cols;
+        float xv[NV][4], g[NV][4];
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = lane + 64 * j;
+            if (i < nvec) {
+                IO::ld4(x + base, i * 4, xv[j]);
+                IO::ld4(dy + base, i * 4, g[j]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; k++) xv[j][k] = g[j][k] = 0.0f;
+            }
+        }
+        float mean = 0.0f, rstd;
+        if (MODE == 0) {
+            float s = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NV; j++) s += (xv[j][0] + xv[j][1]) + (xv[j][2] + xv[j][3]);
+            mean = wave_allreduce_f32(s, OpAdd()) / (float)cols;
+            float q = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const bool live = lane + 64 * j < nvec;
+#pragma unroll
+                for (int k = 0; k < 4; k++) q += live ? (xv[j][k] - mean) * (xv[j][k] - mean) : 0.0f;
+            }
+            rstd = 1.0f / sqrtf(wave_allreduce_f32(q, OpAdd()) / (float)(cols - 1) + eps);
+        } else {
+            float q = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NV; j++)
+#pragma unroll
+                for (int k = 0; k < 4; k++) q += xv[j][k] * xv[j][k];
+            rstd = sqrtf(1.0f / (wave_allreduce_f32(q, OpAdd()) / (float)cols + eps));
+        }
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = lane + 64 * j;
+            float wv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+            if (w && i < nvec) IO::ld4(w, i * 4, wv);
+#pragma unroll
+            for (int k = 0; k < 4; k++) { // a lane past the end: g = 0 leaves every sum as it is
+                const float xh = (xv[j][k] - mean) * rstd;
+                pw[j][k] = __builtin_fmaf(g[j][k], xh, pw[j][k]);
+                pb[j][k] += g[j][k];
+                g[j][k] *= wv[k];
+                s1 += g[j][k];
+                s2 += g[j][k] * (MODE == 0 ? xh : xv[j][k]);
+            }
+        }
+        s1 = wave_allreduce_f32(s1, OpAdd());
+        s2 = wave_allreduce_f32(s2, OpAdd());
+        const float k1 = s1 / (float)cols, k2 = MODE == 0 ? s2 / (float)(cols - 1) : rstd * rstd * rstd * s2 / (float)cols;
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = lane + 64 * j;
+            if (i >= nvec) continue;
+            float av[4] = {0.0f, 0.0f, 0.0f, 0.0f}, o[4];
+            if (add) IO::ld4(add + base, i * 4, av);
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                o[k] = (MODE == 0 ? rstd * ((g[j][k] - k1) - ((xv[j][k] - mean) * rstd) * k2) : rstd * g[j][k] - xv[j][k] * k2) + av[k];
+            IO::st4(dx + base, i * 4, o);
+        }
+    }
+    if (!part) return; // uniform over the workgroup
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int c = (lane + 64 * j) * 4;
+        *(f32x4 *)&fold[wave][0][c] = f32x4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]};
+        *(f32x4 *)&fold[wave][1][c] = f32x4{pb[j][0], pb[j][1], pb[j][2], pb[j][3]};
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < cols; c += WAVES * 64) {
+        float a = fold[0][0][c], b = fold[0][1][c];
+#pragma unroll
+        for (int v = 1; v < WAVES; v++) {
+            a += fold[v][0][c];
+            b += fold[v][1][c];
+        }
+        part[((int64_t)blockIdx.x * 2) * cols + c] = a;
+        part[((int64_t)blockIdx.x * 2 + 1) * cols + c] = b;
+    }
+}
+
 // Cross-entropy, one wave per sample. loss[r] = sum_c -(ln_softmax(x)[r,c]) * target[r,c], computed as the reference
 // does: m = x - max; ls = m - ln(sum exp(m)). Targets are class indices (target[r,c] = (c == label[r]); a label outside
 // [0, cols) matches no class: loss 0) or, DENSE, an f32 [rows, cols] tensor of their own (one-hot or soft labels).
@@ -718,6 +825,14 @@ template <int DT, int MODE, int NV> void launch_norm_bwd_reg(const NormRowsBwd &
                        (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, (p.dw || p.db) ? part : nullptr, p.rows, p.eps);
 }
 
+template <int DT, int MODE, int NV> void launch_norm_bwd_ragged(const NormRowsBwd &p, float *part, int &chunks, hipStream_t st) {
+    typedef typename RowIO<DT>::S S;
+    constexpr int WAVES = NV <= 4 ? 16 : 8;
+    chunks = (int)((p.rows + WAVES - 1) / WAVES < kFusedBlocks ? (p.rows + WAVES - 1) / WAVES : kFusedBlocks);
+    hipLaunchKernelGGL((norm_bwd_dx_ragged_k<DT, MODE, NV, WAVES>), dim3((unsigned)chunks), dim3(WAVES * 64), 0, st, (const S *)p.x, (const S *)p.w,
+                       (const S *)p.dy, (const S *)p.add, (S *)p.dx, (p.dw || p.db) ? part : nullptr, p.rows, (int)p.cols, p.eps);
+}
+
 template <int DT, int MODE> hipError_t launch_norm_bwd(const NormRowsBwd &p, hipStream_t st) {
     typedef typename RowIO<DT>::S S;
     const int esz = (int)sizeof(S);
@@ -731,6 +846,13 @@ template <int DT, int MODE> hipError_t launch_norm_bwd(const NormRowsBwd &p, hip
     else if (al16 && p.cols == 512) launch_norm_bwd_reg<DT, MODE, 2>(p, part, chunks, st);
     else if (al16 && p.cols == 1024) launch_norm_bwd_reg<DT, MODE, 4>(p, part, chunks, st);
     else if (al16 && p.cols == 2048) launch_norm_bwd_reg<DT, MODE, 8>(p, part, chunks, st);
+    else if (al16 && p.cols <= 256) launch_norm_bwd_ragged<DT, MODE, 1>(p, part, chunks, st);
+    else if (al16 && p.cols <= 512) launch_norm_bwd_ragged<DT, MODE, 2>(p, part, chunks, st);
+    else if (al16 && p.cols <= 768) launch_norm_bwd_ragged<DT, MODE, 3>(p, part, chunks, st);
+    else if (al16 && p.cols <= 1024) launch_norm_bwd_ragged<DT, MODE, 4>(p, part, chunks, st);
+    else if (al16 && p.cols <= 1280) launch_norm_bwd_ragged<DT, MODE, 5>(p, part, chunks, st);
+    else if (al16 && p.cols <= 1536) launch_norm_bwd_ragged<DT, MODE, 6>(p, part, chunks, st);
+    else if (al16 && p.cols <= 2048) launch_norm_bwd_ragged<DT, MODE, 8>(p, part, chunks, st);
     else if (vec) hipLaunchKernelGGL((norm_bwd_dx_k<DT, MODE, true>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, (int)p.cols, p.eps);
     else hipLaunchKernelGGL((norm_bwd_dx_k<DT, MODE, false>), grid, block, 0, st, (const S *)p.x, (const S *)p.w, (const S *)p.dy, (const S *)p.add, (S *)p.dx, stats, p.rows, (int)p.cols, p.eps);
     if (p.dw || p.db) {
