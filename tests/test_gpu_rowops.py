@@ -86,6 +86,34 @@ def test_cross_entropy(hip, oracle):
     np.testing.assert_allclose(grad.sum(1), [1.0, 1.0], rtol=1e-6)
 
 
+@pytest.mark.parametrize("shape", [(5, 2052), (3, 2049), (9, 4096), (3, 4097), (4, 8192), (2, 8190), (3, 16384), (2, 20000),
+                                   (2, 32768), (2, 40001), (3, 50257), (1, 65536), (2, 65535), (300, 3000)])
+def test_cross_entropy_many_classes(hip, oracle, shape):
+    """Rows of 2049-65536 classes are read once by a workgroup of 4-16 waves (16-byte vectors when the class count is
+    a multiple of 4, single values otherwise); same bar as the one-wave-per-row kernel."""
+    dev, pool = hip
+    rows, cols = shape
+    r = oracle.Rng(cols)
+    x, lab = r.randn(shape, 3.0), r.randint(rows, 0, cols)
+    lab[0] = cols - 1
+    if rows > 1:
+        lab[1] = -1   # matches no class: zero loss, gradient = softmax * scale
+    loss, grad = cross_entropy(dev, pool, x, lab, 1.0 / rows)
+    wl, wg = oracle.cross_entropy(x, lab, 1.0 / rows)
+    # the oracle adds a row's exp terms one after the other in f32: its sum, the divisor of every gradient, carries an
+    # error that grows with the row length (measured 5e-5 at 65536 classes); the kernel's sum is a tree
+    tol = 1e-5 * max(1.0, cols / 4096)
+    np.testing.assert_allclose(loss, wl, rtol=1e-5, atol=tol)
+    np.testing.assert_allclose(grad, wg, rtol=tol, atol=1e-9)
+    s = np.exp(x.astype(np.float64) - x.max(1, keepdims=True))   # against the sum in f64: the usual bar
+    wg64 = (s / s.sum(1, keepdims=True) - (np.arange(cols)[None, :] == lab[:, None])) / rows
+    np.testing.assert_allclose(grad, wg64, rtol=1e-5, atol=1e-9)
+    live = lab >= 0
+    assert np.all(np.abs(grad[live].astype(np.float64).sum(1)) < 1e-6)
+    loss_only, none = cross_entropy(dev, pool, x, lab, None)
+    assert none is None and np.array_equal(loss_only, loss)
+
+
 # ---- gradients of the norms ---------------------------------------------------------------------------------
 @pytest.mark.parametrize("shape", [(5, 9), (64, 128), (130, 1024), (3, 1000), (2100, 64), (64, 256), (7, 512), (9, 2048),
                                    (8192, 1024), (4099, 1024), (2051, 512),  # several rows per wave: rows fetched ahead

@@ -649,6 +649,73 @@ __global__ __launch_bounds__(256) void cross_entropy_k(const float *__restrict__
     cross_entropy_row<DENSE>(x, target, loss, grad, row, cols, gscale, threadIdx.x & 63);
 }
 
+// Class-index targets, rows of 2049-65536 classes: one row per workgroup of W waves, read once and held in registers
+// (NE values per thread; VEC: rows of a multiple of 4 classes in 16-byte vectors, vector t + 64*W*j of the row in
+// thread t, else element t + 64*W*j). The formulas are cross_entropy_row's; exp(x - max) is kept for the gradient.
+// The W waves' maxima and sums meet in LDS and are combined in wave order.
+template <int NE, int W, bool VEC>
+__global__ __launch_bounds__(64 * W) void cross_entropy_wide_k(const float *__restrict__ x, const int32_t *__restrict__ labels,
+                                                               float *__restrict__ loss, float *__restrict__ grad, int cols,
+                                                               float gscale) {
+    constexpr int T = 64 * W, G = VEC ? 4 : 1, NJ = NE / G;
+    __shared__ float red[2][W];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int64_t row = blockIdx.x;
+    const float *xr = x + row * cols;
+    float v[NE];
+    float mx = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+        const int c = (t + T * j) * G;
+        if (c < cols) {
+            if constexpr (VEC) {
+                const f32x4 q = *(const f32x4 *)(xr + c);
+                v[4 * j] = q.x, v[4 * j + 1] = q.y, v[4 * j + 2] = q.z, v[4 * j + 3] = q.w;
+            } else {
+                v[j] = xr[c];
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < G; k++) v[G * j + k] = -INFINITY; // exp(-inf - max) = 0 below
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NE; i++) mx = fmaxf(v[i], mx);
+    mx = wave_allreduce_f32(mx, OpMaxF());
+    if (lane == 0) red[0][wave] = mx;
+    __syncthreads();
+    mx = red[0][0];
+#pragma unroll
+    for (int k = 1; k < W; k++) mx = fmaxf(red[0][k], mx);
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NE; i++) {
+        v[i] = expf(v[i] - mx);
+        s += v[i];
+    }
+    s = wave_allreduce_f32(s, OpAdd());
+    if (lane == 0) red[1][wave] = s;
+    __syncthreads();
+    s = red[1][0];
+#pragma unroll
+    for (int k = 1; k < W; k++) s += red[1][k];
+    const int label = labels[row];
+    if (loss && t == 0) loss[row] = label >= 0 && label < cols ? -((xr[label] - mx) - logf(s)) : 0.0f;
+    if (!grad) return;
+    const float inv = 1.0f / s;
+    float *gr = grad + row * cols;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+        const int c = (t + T * j) * G;
+        if (c >= cols) continue;
+        float o[G];
+#pragma unroll
+        for (int k = 0; k < G; k++) o[k] = (v[G * j + k] * inv - (c + k == label ? 1.0f : 0.0f)) * gscale;
+        if constexpr (VEC) *(f32x4 *)(gr + c) = f32x4{o[0], o[1], o[2], o[3]};
+        else gr[c] = o[0];
+    }
+}
+
 // The whole batch in one workgroup of 16 waves, which also leaves mean[0] = sum(loss) / rows (ReduceOp::Mean): every
 // wave adds its rows' losses in row order, the 16 partial sums are added in wave order.
 template <bool DENSE>
@@ -944,6 +1011,21 @@ hipError_t cross_entropy(const CrossEntropy &p, hipStream_t st) {
         if (p.rows > kCrossEntropyMeanRows) return hipErrorInvalidValue;
         if (p.dense) hipLaunchKernelGGL(cross_entropy_mean_k<true>, dim3(1), dim3(1024), 0, st, p.x, target, p.loss, p.grad, p.mean, p.rows, (int)p.cols, p.gscale);
         else hipLaunchKernelGGL(cross_entropy_mean_k<false>, dim3(1), dim3(1024), 0, st, p.x, target, p.loss, p.grad, p.mean, p.rows, (int)p.cols, p.gscale);
+        return hipGetLastError();
+    }
+    if (!p.dense && p.cols > 2048 && p.cols <= 65536 && p.rows < (1ll << 31)) {
+        const bool vec = p.cols % 4 == 0 && reinterpret_cast<uintptr_t>(p.x) % 16 == 0 && (!p.grad || reinterpret_cast<uintptr_t>(p.grad) % 16 == 0);
+#define ZK_CE(NE, W)                                                                                                              \
+    do {                                                                                                                          \
+        if (vec) hipLaunchKernelGGL((cross_entropy_wide_k<NE, W, true>), dim3((unsigned)p.rows), dim3(64 * W), 0, st, p.x, p.labels, p.loss, p.grad, (int)p.cols, p.gscale); \
+        else hipLaunchKernelGGL((cross_entropy_wide_k<NE, W, false>), dim3((unsigned)p.rows), dim3(64 * W), 0, st, p.x, p.labels, p.loss, p.grad, (int)p.cols, p.gscale); \
+    } while (0)
+        if (p.cols <= 4096) ZK_CE(16, 4);
+        else if (p.cols <= 8192) ZK_CE(16, 8);
+        else if (p.cols <= 16384) ZK_CE(16, 16);
+        else if (p.cols <= 32768) ZK_CE(32, 16);
+        else ZK_CE(64, 16);
+#undef ZK_CE
         return hipGetLastError();
     }
     const dim3 grid((unsigned)((p.rows + 3) / 4));
