@@ -220,6 +220,23 @@ def extra_streaming(dev, pool, kernels, steps=20, warmup=5):
         w, bb = dev_arr(vec, dt), dev_arr(vec, dt)
         timeit(f"layernorm_bwd_{tag}_8192x1024", kernels.norm_rows_bwd_desc(M, D, add=True, dtype=dt),
                lambda: [dev_arr(row, dt), w, dev_arr(row, dt), dev_arr(row, dt), out_arr(M * D, isz), out_arr(D, isz), out_arr(D, isz)], 4 * M * D * isz)
+        # a width that is not 256 * 2^n: rows with lanes past their end
+        D2 = 768
+        row2, vec2 = rng.randn((M, D2)), rng.randn((D2,))
+        w, bb = dev_arr(vec2, dt), dev_arr(vec2, dt)
+        timeit(f"layernorm_{tag}_8192x768", kernels.norm_rows_desc(M, D2, dtype=dt), lambda: [dev_arr(row2, dt), w, bb, out_arr(M * D2, isz)], 2 * M * D2 * isz)
+        w = dev_arr(vec2, dt)
+        timeit(f"layernorm_bwd_{tag}_8192x768", kernels.norm_rows_bwd_desc(M, D2, add=True, dtype=dt),
+               lambda: [dev_arr(row2, dt), w, dev_arr(row2, dt), dev_arr(row2, dt), out_arr(M * D2, isz), out_arr(D2, isz), out_arr(D2, isz)], 4 * M * D2 * isz)
+    # cross-entropy (loss + gradient) over a language model's vocabulary: logits read once, gradient written once
+    R, V = 2048, 32000
+    logits, labels = rng.randn((R, V)), rng.randint((R,), 0, V).astype(np.int32)
+
+    def ce_args():
+        lb, e = kernels.to_device(pool, labels)
+        pool.sync_events([e])
+        return [dev_arr(logits, zyx_amd.DType.F32), lb, out_arr(R, 4), out_arr(R * V, 4)]
+    timeit("cross_entropy_f32_2048x32000", kernels.cross_entropy_desc(R, V, True, True, 1.0 / R), ce_args, 2 * R * V * 4 + R * 8)
     return out
 
 
